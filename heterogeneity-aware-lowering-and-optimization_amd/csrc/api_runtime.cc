@@ -1,0 +1,680 @@
+// ODLA control plane of libodla_hip.so: computations, contexts, binding,
+// execution (hipGraph replay), value introspection, device / memory / logging.
+#include <atomic>
+#include <cstring>
+
+#include "internal.h"
+
+using namespace ohip;
+
+// ---------------------------------------------------------------- logging --
+namespace {
+std::atomic<int> g_log_level{ODLA_LOG_LEVEL_ERROR};
+
+void default_logger(const char* file, int line, const char* func, odla_log_level level, const char* msg) {
+  (void)func;
+  if ((int)level > g_log_level.load()) return;
+  static const char tags[] = {'-', 'F', 'E', 'W', 'I', 'D', 'T'};
+  const char tag = (level >= 0 && level <= ODLA_LOG_LEVEL_TRACE) ? tags[level] : '?';
+  if (file != nullptr && line > 0) fprintf(stderr, "[odla_hip %c] %s:%d %s\n", tag, file, line, msg);
+  else fprintf(stderr, "[odla_hip %c] %s\n", tag, msg);
+}
+std::atomic<odla_logging_func> g_logger{default_logger};
+
+std::mutex g_registry_mu;
+std::vector<_odla_computation*> g_computations;  // live computations, creation order
+thread_local _odla_computation* t_current = nullptr;
+
+const char* kVersion = "odla_hip 0.5.0 (gfx950)";
+}  // namespace
+
+namespace ohip {
+
+void log_msg(const char* file, int line, const char* func, odla_log_level lvl, const char* fmt, ...) {
+  if ((int)lvl > g_log_level.load() && g_logger.load() == default_logger) return;
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  const char* base = file ? strrchr(file, '/') : nullptr;
+  g_logger.load()(base ? base + 1 : file, line, func, lvl, buf);
+}
+
+const char* op_name(OpKind k) {
+  static const char* names[] = {"Conv", "Gemm", "Binary", "Unary", "BatchNorm", "LayerNorm", "Pool",
+                                "Reduce", "Softmax", "Cast", "Concat", "Gather", "Reshape", "Resize",
+                                "Slice", "Transpose", "Quantize", "Dequantize", "NMS"};
+  return names[(int)k];
+}
+
+std::string Shape::str() const {
+  std::string s = "[";
+  for (int i = 0; i < rank; ++i) {
+    if (i) s += ",";
+    s += std::to_string(d[i]);
+  }
+  return s + "]";
+}
+
+Shape shape_from(const odla_value_shape& s) {
+  Shape r;
+  if (s.size <= 0) {  // scalar: rewritten to {1} as the reference does [ref: odla_dnnl.cc:181-190]
+    r.rank = 1;
+    r.d[0] = 1;
+    return r;
+  }
+  r.rank = s.size > ODLA_MAX_DIMENSION ? ODLA_MAX_DIMENSION : s.size;
+  for (int i = 0; i < r.rank; ++i) r.d[i] = s.dims[i];
+  return r;
+}
+
+odla_value_shape shape_to(const Shape& s) {
+  odla_value_shape r;
+  memset(&r, 0, sizeof(r));
+  r.size = s.rank;
+  for (int i = 0; i < s.rank; ++i) r.dims[i] = s.d[i];
+  return r;
+}
+
+bool shape_valid(const odla_value_shape& s) {
+  if (s.size < 1 || s.size > ODLA_MAX_DIMENSION) return false;
+  for (int i = 0; i < s.size; ++i)
+    if (s.dims[i] <= 0 || s.dims[i] > (1ll << 40)) return false;
+  return true;
+}
+
+DType dtype_from_odla(odla_element_type t) {
+  switch (t) {
+    case ODLA_FLOAT32: return DT_F32;
+    case ODLA_FLOAT16: return DT_F16;
+    case ODLA_BFLOAT16: return DT_BF16;
+    case ODLA_INT8: case ODLA_QINT8: return DT_I8;
+    case ODLA_UINT8: case ODLA_QUINT8: return DT_U8;
+    case ODLA_INT32: case ODLA_QINT32: case ODLA_UINT32: return DT_I32;
+    case ODLA_INT64: case ODLA_UINT64: return DT_I64;
+    case ODLA_BOOL: return DT_BOOL;
+    default: return DT_INVALID;
+  }
+}
+
+int odla_type_size(odla_element_type t) { return dtype_size(dtype_from_odla(t)); }
+
+_odla_computation* current_computation() {
+  if (t_current != nullptr) return t_current;
+  std::lock_guard<std::mutex> lk(g_registry_mu);
+  return g_computations.empty() ? nullptr : g_computations.back();
+}
+void set_current_computation(_odla_computation* c) { t_current = c; }
+void forget_computation(_odla_computation* c) {
+  if (t_current == c) t_current = nullptr;
+  std::lock_guard<std::mutex> lk(g_registry_mu);
+  for (size_t i = 0; i < g_computations.size(); ++i)
+    if (g_computations[i] == c) { g_computations.erase(g_computations.begin() + i); break; }
+}
+
+_odla_value* new_value(_odla_computation* c, _odla_value::Kind kind, odla_element_type et,
+                       const Shape& shape, const odla_value_id id) {
+  auto v = std::make_unique<_odla_value>();
+  v->kind = kind;
+  v->etype = et;
+  v->shape = shape;
+  v->comp = c;
+  v->index = (int)c->values.size();
+  if (id != nullptr) {
+    v->name = reinterpret_cast<const char*>(id);
+    if (!v->name.empty()) c->by_name[v->name] = v.get();
+  }
+  _odla_value* raw = v.get();
+  c->values.push_back(std::move(v));
+  return raw;
+}
+
+Plan::~Plan() {
+  if (const_pool != nullptr) (void)hipFree(const_pool);
+}
+
+}  // namespace ohip
+
+namespace {
+
+bool is_live(_odla_computation* c) {
+  std::lock_guard<std::mutex> lk(g_registry_mu);
+  for (auto* p : g_computations)
+    if (p == c) return true;
+  return false;
+}
+
+odla_status ensure_plan(_odla_computation* c) {
+  std::lock_guard<std::mutex> lk(c->mu);
+  if (c->plan) return ODLA_SUCCESS;
+  if (c->plan_failed) return ODLA_FAILURE;
+  std::unique_ptr<Plan> plan;
+  odla_status st = build_plan(c, &plan);
+  if (st != ODLA_SUCCESS) {
+    c->plan_failed = true;
+    return st;
+  }
+  c->plan = std::move(plan);
+  return ODLA_SUCCESS;
+}
+
+void drop_graph(_odla_context* ctx) {
+  if (ctx->graph_exec) { (void)hipGraphExecDestroy(ctx->graph_exec); ctx->graph_exec = nullptr; }
+  if (ctx->graph) { (void)hipGraphDestroy(ctx->graph); ctx->graph = nullptr; }
+}
+
+odla_status run_steps(_odla_context* ctx, const Plan& plan) {
+  ExecEnv env;
+  env.base[SP_ARENA] = ctx->arena;
+  env.base[SP_CONST] = plan.const_pool;
+  for (const Step& s : plan.steps) {
+    hipError_t e = s.fn(env, ctx->stream);
+    if (e != hipSuccess) {
+      OHIP_ERR("step '%s' failed: %s", s.name.c_str(), hipGetErrorString(e));
+      return ODLA_FAILURE;
+    }
+  }
+  return ODLA_SUCCESS;
+}
+
+_odla_value* find_value(_odla_computation* c, const odla_value_id id) {
+  if (c == nullptr || id == nullptr) return nullptr;
+  auto it = c->by_name.find(reinterpret_cast<const char*>(id));
+  return it == c->by_name.end() ? nullptr : it->second;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ------------------------------------------------------------ computation --
+odla_status odla_CreateComputation(odla_computation* computation) {
+  if (computation == nullptr) return ODLA_INVALID_PARAM;
+  auto* c = new (std::nothrow) _odla_computation();
+  if (c == nullptr) return ODLA_MEM_ERROR;
+  {
+    std::lock_guard<std::mutex> lk(g_registry_mu);
+    g_computations.push_back(c);
+  }
+  set_current_computation(c);
+  *computation = c;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_DestroyComputation(odla_computation c) {
+  if (c == nullptr) return ODLA_INVALID_PARAM;
+  if (!is_live(c)) return ODLA_INVALID_PARAM;
+  forget_computation(c);
+  (void)hipDeviceSynchronize();
+  delete c;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_SetComputationItem(odla_computation c, odla_item_type type, odla_item_value value) {
+  if (c == nullptr) return ODLA_INVALID_PARAM;
+  std::lock_guard<std::mutex> lk(c->mu);
+  if (c->plan) {
+    OHIP_WARN("odla_SetComputationItem(%d) after the computation was compiled is ignored", (int)type);
+    return ODLA_FAILURE;
+  }
+  switch ((int)type) {
+    case ODLA_FP16_MODE:
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      c->opts.fp16 = *reinterpret_cast<const bool*>(value);
+      return ODLA_SUCCESS;
+    case ODLA_BF16_MODE:
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      c->opts.bf16 = *reinterpret_cast<const odla_bf16_mode*>(value);
+      return ODLA_SUCCESS;
+    case ODLA_USE_DATA_TYPE: {
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      const odla_element_type t = *reinterpret_cast<const odla_element_type*>(value);
+      if (t == ODLA_INT8 || t == ODLA_QINT8 || t == ODLA_QUINT8 || t == ODLA_UINT8) c->opts.int8 = true;
+      else if (t == ODLA_FLOAT16) c->opts.fp16 = true;
+      else if (t == ODLA_BFLOAT16) c->opts.bf16 = BF16_PERFORMACE_MODE;
+      else if (t == ODLA_FLOAT32) { c->opts.int8 = false; c->opts.fp16 = false; c->opts.bf16 = BF16_DISABLE; }
+      else return ODLA_UNSUPPORTED_DATATYPE;
+      return ODLA_SUCCESS;
+    }
+    case ODLA_QUANT_TABLE:
+      c->opts.qtable = reinterpret_cast<const odla_value_quant_info*>(value);
+      return ODLA_SUCCESS;
+    case ODLA_QUANT_TABLE_SIZE:
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      c->opts.qtable_size = *reinterpret_cast<const int*>(value);
+      return ODLA_SUCCESS;
+    case 1000:  // ODLA_HIP_ITEM_RAW_INT32_ACC
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      c->opts.raw_acc = *reinterpret_cast<const bool*>(value);
+      return ODLA_SUCCESS;
+    default:
+      OHIP_DEBUG("odla_SetComputationItem: item %d accepted and ignored", (int)type);
+      return ODLA_SUCCESS;
+  }
+}
+
+// ---------------------------------------------------------------- context --
+odla_status odla_CreateContext(odla_context* context) {
+  if (context == nullptr) return ODLA_INVALID_PARAM;
+  _odla_computation* c = current_computation();
+  if (c == nullptr) {
+    OHIP_ERR("odla_CreateContext: no computation exists");
+    return ODLA_FAILURE;
+  }
+  odla_status st = ensure_plan(c);
+  if (st != ODLA_SUCCESS) return st;
+  auto ctx = std::make_unique<_odla_context>();
+  ctx->comp = c;
+  if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+    OHIP_ERR("odla_CreateContext: cannot create a HIP stream");
+    return ODLA_FAILURE;
+  }
+  ctx->arena_bytes = c->plan->arena_bytes;
+  if (ctx->arena_bytes > 0) {
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&ctx->arena), ctx->arena_bytes);
+    if (e != hipSuccess) {
+      OHIP_ERR("odla_CreateContext: cannot allocate a %zu-byte device arena: %s", ctx->arena_bytes, hipGetErrorString(e));
+      (void)hipStreamDestroy(ctx->stream);
+      return ODLA_MEM_ERROR;
+    }
+  }
+  *context = ctx.release();
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_DestroyContext(odla_context ctx) {
+  if (ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  drop_graph(ctx);
+  if (ctx->arena) (void)hipFree(ctx->arena);
+  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_SetContextItem(odla_context ctx, odla_item_type type, odla_item_value value) {
+  if (ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (type == ODLA_AGGREGATE_OPS) {
+    if (value == nullptr) return ODLA_INVALID_PARAM;
+    ctx->use_graph = *reinterpret_cast<const bool*>(value);
+    if (!ctx->use_graph) drop_graph(ctx);
+    return ODLA_SUCCESS;
+  }
+  OHIP_DEBUG("odla_SetContextItem: item %d accepted and ignored", (int)type);
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_BindToArgument(odla_value value, const odla_void* data_ptr, odla_context ctx) {
+  if (value == nullptr || data_ptr == nullptr || ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (value->kind != _odla_value::ARG || value->comp != ctx->comp) {
+    OHIP_ERR("odla_BindToArgument: '%s' is not an argument of this computation", value->name.c_str());
+    return ODLA_INVALID_PARAM;
+  }
+  ctx->bound_in[value] = data_ptr;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_BindToArgumentById(const odla_value_id id, const odla_void* data_ptr, odla_context ctx) {
+  if (ctx == nullptr || id == nullptr) return ODLA_INVALID_PARAM;
+  _odla_value* v = find_value(ctx->comp, id);
+  if (v == nullptr) {
+    OHIP_ERR("odla_BindToArgumentById: unknown value id '%s'", reinterpret_cast<const char*>(id));
+    return ODLA_INVALID_PARAM;
+  }
+  return odla_BindToArgument(v, data_ptr, ctx);
+}
+
+odla_status odla_BindToOutput(odla_value value, odla_void* data_ptr, odla_context ctx) {
+  if (value == nullptr || data_ptr == nullptr || ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (!value->is_output || value->comp != ctx->comp) {
+    OHIP_ERR("odla_BindToOutput: '%s' is not an output of this computation", value->name.c_str());
+    return ODLA_INVALID_PARAM;
+  }
+  ctx->bound_out[value] = data_ptr;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_BindToOutputById(const odla_value_id id, odla_void* data_ptr, odla_context ctx) {
+  if (ctx == nullptr || id == nullptr) return ODLA_INVALID_PARAM;
+  _odla_value* v = find_value(ctx->comp, id);
+  if (v == nullptr) {
+    OHIP_ERR("odla_BindToOutputById: unknown value id '%s'", reinterpret_cast<const char*>(id));
+    return ODLA_INVALID_PARAM;
+  }
+  return odla_BindToOutput(v, data_ptr, ctx);
+}
+
+odla_status odla_ExecuteComputation(const odla_computation comp, const odla_context ctx,
+                                    const odla_compute_mode mode, odla_device device) {
+  (void)device;
+  if (ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (comp != nullptr && comp != ctx->comp) {
+    OHIP_ERR("odla_ExecuteComputation: context belongs to another computation");
+    return ODLA_INVALID_PARAM;
+  }
+  if (mode == ODLA_COMPUTE_TRAINING) return ODLA_UNSUPPORTED_OP;
+  _odla_computation* c = ctx->comp;
+  if (!c->plan) return ODLA_FAILURE;
+  const Plan& plan = *c->plan;
+
+  // 1. stage arguments (host -> device across PCIe, or device -> device)
+  for (const Plan::IO& io : plan.inputs) {
+    auto it = ctx->bound_in.find(io.v);
+    if (it == ctx->bound_in.end()) {
+      OHIP_ERR("odla_ExecuteComputation: argument '%s' is not bound", io.v->name.c_str());
+      return ODLA_INVALID_PARAM;
+    }
+    char* dst = ctx->arena + plan.tensors[io.tensor].offset;
+    if (hipMemcpyAsync(dst, it->second, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
+      OHIP_ERR("odla_ExecuteComputation: copy of argument '%s' failed", io.v->name.c_str());
+      return ODLA_FAILURE;
+    }
+  }
+
+  // 2. launch sequence: captured once into a hipGraph, replayed afterwards
+  if (ctx->use_graph && !plan.steps.empty()) {
+    if (ctx->graph_exec == nullptr) {
+      if (hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        OHIP_ERR("odla_ExecuteComputation: hipStreamBeginCapture failed");
+        return ODLA_FAILURE;
+      }
+      odla_status st = run_steps(ctx, plan);
+      hipGraph_t g = nullptr;
+      hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+      if (st != ODLA_SUCCESS || e != hipSuccess || g == nullptr) {
+        if (g) (void)hipGraphDestroy(g);
+        OHIP_ERR("odla_ExecuteComputation: graph capture failed");
+        return ODLA_FAILURE;
+      }
+      ctx->graph = g;
+      if (hipGraphInstantiate(&ctx->graph_exec, g, nullptr, nullptr, 0) != hipSuccess) {
+        drop_graph(ctx);
+        OHIP_ERR("odla_ExecuteComputation: hipGraphInstantiate failed");
+        return ODLA_FAILURE;
+      }
+    }
+    if (hipGraphLaunch(ctx->graph_exec, ctx->stream) != hipSuccess) {
+      OHIP_ERR("odla_ExecuteComputation: hipGraphLaunch failed");
+      return ODLA_FAILURE;
+    }
+  } else {
+    odla_status st = run_steps(ctx, plan);
+    if (st != ODLA_SUCCESS) return st;
+  }
+
+  // 3. results
+  for (const Plan::IO& io : plan.outputs) {
+    auto it = ctx->bound_out.find(io.v);
+    if (it == ctx->bound_out.end()) continue;
+    const PTensor& t = plan.tensors[io.tensor];
+    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset;
+    if (hipMemcpyAsync(it->second, src, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
+      OHIP_ERR("odla_ExecuteComputation: copy of output '%s' failed", io.v->name.c_str());
+      return ODLA_FAILURE;
+    }
+  }
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) {
+    OHIP_ERR("odla_ExecuteComputation: device error: %s", hipGetErrorString(e));
+    return ODLA_FAILURE;
+  }
+  ctx->executed = true;
+  return ODLA_SUCCESS;
+}
+
+// ----------------------------------------------------------- introspection --
+odla_status odla_GetNumOfArgsFromComputation(const odla_computation c, odla_uint32* n) {
+  if (c == nullptr || n == nullptr) return ODLA_INVALID_PARAM;
+  *n = (odla_uint32)c->args.size();
+  return ODLA_SUCCESS;
+}
+odla_status odla_GetArgFromComputationByIdx(const odla_computation c, const odla_uint32 idx, odla_value* v) {
+  if (c == nullptr || v == nullptr) return ODLA_INVALID_PARAM;
+  *v = nullptr;
+  if (idx >= c->args.size()) return ODLA_INVALID_PARAM;
+  *v = c->args[idx];
+  return ODLA_SUCCESS;
+}
+odla_status odla_GetNumOfOutputsFromComputation(const odla_computation c, odla_uint32* n) {
+  if (c == nullptr || n == nullptr) return ODLA_INVALID_PARAM;
+  *n = (odla_uint32)c->outputs.size();
+  return ODLA_SUCCESS;
+}
+odla_status odla_GetOutputFromComputationByIdx(const odla_computation c, const odla_uint32 idx, odla_value* v) {
+  if (c == nullptr || v == nullptr) return ODLA_INVALID_PARAM;
+  *v = nullptr;
+  if (idx >= c->outputs.size()) return ODLA_INVALID_PARAM;
+  *v = c->outputs[idx];
+  return ODLA_SUCCESS;
+}
+odla_status odla_GetRuntimeShape(odla_context ctx, odla_value value, odla_value_shape* shape) {
+  (void)ctx;
+  if (value == nullptr || shape == nullptr) return ODLA_INVALID_PARAM;
+  *shape = shape_to(value->shape);
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_GetValueType(const odla_value value, odla_value_type* type) {
+  if (value == nullptr || type == nullptr) return ODLA_INVALID_PARAM;
+  type->element_type = value->etype;
+  type->shape = shape_to(value->shape);
+  return ODLA_SUCCESS;
+}
+odla_status odla_GetValueId(const odla_value value, odla_value_id* id) {
+  if (value == nullptr || id == nullptr) return ODLA_INVALID_PARAM;
+  *id = reinterpret_cast<odla_value_id>(const_cast<char*>(value->name.c_str()));
+  return ODLA_SUCCESS;
+}
+odla_status odla_FindValueById(const odla_value_id id, odla_value* value) {
+  if (id == nullptr || value == nullptr) return ODLA_INVALID_PARAM;
+  *value = find_value(current_computation(), id);
+  return *value ? ODLA_SUCCESS : ODLA_INVALID_PARAM;
+}
+
+odla_status odla_SetValueAsOutput(odla_value value) {
+  if (value == nullptr || value->comp == nullptr) return ODLA_INVALID_PARAM;
+  _odla_computation* c = value->comp;
+  std::lock_guard<std::mutex> lk(c->mu);
+  if (c->plan) {
+    OHIP_ERR("odla_SetValueAsOutput: computation is already compiled");
+    return ODLA_FAILURE;
+  }
+  if (!value->is_output) {
+    value->is_output = true;
+    c->outputs.push_back(value);
+  }
+  return ODLA_SUCCESS;
+}
+odla_status odla_SetValuesAsOutput(odla_values values) {
+  if (values.size > ODLA_MAX_OUTPUTS) return ODLA_INVALID_PARAM;
+  for (size_t i = 0; i < values.size; ++i) {
+    odla_status st = odla_SetValueAsOutput(values.values[i]);
+    if (st != ODLA_SUCCESS) return st;
+  }
+  return ODLA_SUCCESS;
+}
+odla_status odla_SetValueAsOutputById(const odla_value_id id) {
+  return odla_SetValueAsOutput(find_value(current_computation(), id));
+}
+
+odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr, odla_context ctx) {
+  if (value == nullptr || data_ptr == nullptr || ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (!ctx->executed || !ctx->comp->plan) return ODLA_FAILURE;
+  const Plan& plan = *ctx->comp->plan;
+  for (const Plan::IO& io : plan.outputs) {
+    if (io.v != value) continue;
+    const PTensor& t = plan.tensors[io.tensor];
+    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset;
+    if (hipMemcpy(data_ptr, src, io.bytes, hipMemcpyDefault) != hipSuccess) return ODLA_FAILURE;
+    return ODLA_SUCCESS;
+  }
+  OHIP_ERR("odla_GetValueData: '%s' is not an output; only outputs stay resident after execution", value->name.c_str());
+  return ODLA_INVALID_PARAM;
+}
+odla_status odla_ReleaseValue(odla_value value) { return value ? ODLA_SUCCESS : ODLA_INVALID_PARAM; }
+
+odla_value odla_CreateArgument(const odla_value_type type, const odla_value_id id) {
+  _odla_computation* c = current_computation();
+  if (c == nullptr) { OHIP_ERR("odla_CreateArgument: no current computation"); return nullptr; }
+  if (dtype_from_odla(type.element_type) == DT_INVALID) {
+    OHIP_ERR("odla_CreateArgument: unsupported element type %d", (int)type.element_type);
+    return nullptr;
+  }
+  if (type.shape.size > ODLA_MAX_DIMENSION) { OHIP_ERR("odla_CreateArgument: rank too large"); return nullptr; }
+  Shape s = shape_from(type.shape);
+  for (int i = 0; i < s.rank; ++i)
+    if (s.d[i] <= 0) { OHIP_ERR("odla_CreateArgument: dynamic or empty dimensions are not supported (%s)", s.str().c_str()); return nullptr; }
+  std::lock_guard<std::mutex> lk(c->mu);
+  _odla_value* v = new_value(c, _odla_value::ARG, type.element_type, s, id);
+  c->args.push_back(v);
+  return v;
+}
+
+odla_value odla_CreateConstant(const odla_value_type type, const odla_void* data_ptr, const odla_value_id id) {
+  _odla_computation* c = current_computation();
+  if (c == nullptr) { OHIP_ERR("odla_CreateConstant: no current computation"); return nullptr; }
+  if (data_ptr == nullptr) { OHIP_ERR("odla_CreateConstant: null data"); return nullptr; }
+  if (dtype_from_odla(type.element_type) == DT_INVALID) {
+    OHIP_ERR("odla_CreateConstant: unsupported element type %d", (int)type.element_type);
+    return nullptr;
+  }
+  if (type.shape.size > ODLA_MAX_DIMENSION) { OHIP_ERR("odla_CreateConstant: rank too large"); return nullptr; }
+  Shape s = shape_from(type.shape);
+  for (int i = 0; i < s.rank; ++i)
+    if (s.d[i] <= 0) { OHIP_ERR("odla_CreateConstant: bad shape %s", s.str().c_str()); return nullptr; }
+  std::lock_guard<std::mutex> lk(c->mu);
+  _odla_value* v = new_value(c, _odla_value::CONSTANT, type.element_type, s, id);
+  v->host_data = data_ptr;
+  return v;
+}
+
+// ------------------------------------------------------------------ device --
+odla_status odla_AllocateDevice(odla_vendor vendor, odla_device_name name, odla_int32 idx, odla_device* device) {
+  (void)vendor;
+  if (device == nullptr) return ODLA_INVALID_PARAM;
+  *device = nullptr;
+  if (name != ODLA_DEVICE_DEFAULT) return ODLA_UNSUPPORTED_DEVICE_TYPE;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return ODLA_FAILURE;
+  if (idx < 0 || idx >= count) return ODLA_INVALID_PARAM;
+  auto* d = new (std::nothrow) _odla_device();
+  if (d == nullptr) return ODLA_MEM_ERROR;
+  d->index = idx;
+  *device = d;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_GetDeviceInfo(odla_device device, odla_device_info info, odla_scalar_value* out) {
+  if (device == nullptr || out == nullptr) return ODLA_INVALID_PARAM;
+  static thread_local char text[256];
+  hipDeviceProp_t prop;
+  switch (info) {
+    case ODLA_DEVICE_INFO_ODLA_LIB_VERSION:
+      out->data_type = ODLA_STRING; out->val_str = kVersion; return ODLA_SUCCESS;
+    case ODLA_DEVICE_INFO_DEV_COUNT: {
+      int n = 0;
+      if (hipGetDeviceCount(&n) != hipSuccess) return ODLA_FAILURE;
+      out->data_type = ODLA_INT32; out->val_int32 = n; return ODLA_SUCCESS;
+    }
+    case ODLA_DEVICE_INFO_DEV_INDEX:
+      out->data_type = ODLA_INT32; out->val_int32 = device->index; return ODLA_SUCCESS;
+    case ODLA_DEVICE_INFO_DEV_TYPE:
+      if (hipGetDeviceProperties(&prop, device->index) != hipSuccess) return ODLA_FAILURE;
+      snprintf(text, sizeof(text), "%s (%s)", prop.name, prop.gcnArchName);
+      out->data_type = ODLA_STRING; out->val_str = text; return ODLA_SUCCESS;
+    case ODLA_DEVICE_INFO_DEV_UUID: {
+      hipUUID uuid;
+      if (hipDeviceGetUuid(&uuid, device->index) != hipSuccess) return ODLA_FAILURE;
+      memcpy(text, uuid.bytes, 16); text[16] = 0;
+      out->data_type = ODLA_STRING; out->val_str = text; return ODLA_SUCCESS;
+    }
+    case ODLA_DEVICE_INFO_TOTAL_MEMORY:
+    case ODLA_DEVICE_INFO_USED_MEMORY:
+    case ODLA_DEVICE_INFO_MEMORY_UTIL: {
+      size_t free_b = 0, total_b = 0;
+      int prev = 0;
+      (void)hipGetDevice(&prev);
+      if (hipSetDevice(device->index) != hipSuccess) return ODLA_FAILURE;
+      hipError_t e = hipMemGetInfo(&free_b, &total_b);
+      (void)hipSetDevice(prev);
+      if (e != hipSuccess) return ODLA_FAILURE;
+      if (info == ODLA_DEVICE_INFO_TOTAL_MEMORY) { out->data_type = ODLA_INT64; out->val_int64 = (odla_int64)total_b; }
+      else if (info == ODLA_DEVICE_INFO_USED_MEMORY) { out->data_type = ODLA_INT64; out->val_int64 = (odla_int64)(total_b - free_b); }
+      else { out->data_type = ODLA_FLOAT32; out->val_fp32 = total_b ? (float)(total_b - free_b) / (float)total_b : 0.f; }
+      return ODLA_SUCCESS;
+    }
+    // Utilisation and power need the SMI library; a neutral value is reported
+    // so that generic monitors keep working.
+    case ODLA_DEVICE_INFO_PROCESSOR_UTIL:
+    case ODLA_DEVICE_INFO_POWER_USAGE:
+    case ODLA_DEVICE_INFO_POWER_LIMIT:
+      out->data_type = ODLA_FLOAT32; out->val_fp32 = 0.f; return ODLA_SUCCESS;
+    case ODLA_DEVICE_INFO_DRIVER_VERSION: {
+      int v = 0;
+      if (hipDriverGetVersion(&v) != hipSuccess) return ODLA_FAILURE;
+      snprintf(text, sizeof(text), "%d", v);
+      out->data_type = ODLA_STRING; out->val_str = text; return ODLA_SUCCESS;
+    }
+    case ODLA_DEVICE_INFO_SDK_VERSION: {
+      int v = 0;
+      if (hipRuntimeGetVersion(&v) != hipSuccess) return ODLA_FAILURE;
+      snprintf(text, sizeof(text), "HIP %d", v);
+      out->data_type = ODLA_STRING; out->val_str = text; return ODLA_SUCCESS;
+    }
+  }
+  return ODLA_INVALID_PARAM;
+}
+
+odla_status odla_SetCurrentDevice(odla_device device) {
+  if (device == nullptr) return ODLA_INVALID_PARAM;
+  return hipSetDevice(device->index) == hipSuccess ? ODLA_SUCCESS : ODLA_FAILURE;
+}
+odla_status odla_DestroyDevice(odla_device device) {
+  if (device == nullptr) return ODLA_INVALID_PARAM;
+  delete device;
+  return ODLA_SUCCESS;
+}
+
+// ------------------------------------------------------------------ memory --
+odla_status odla_AllocateDeviceMemory(odla_void** dev_ptr, odla_size_t size) {
+  if (dev_ptr == nullptr || size == 0) return ODLA_INVALID_PARAM;
+  return hipMalloc(dev_ptr, size) == hipSuccess ? ODLA_SUCCESS : ODLA_MEM_ERROR;
+}
+odla_status odla_FreeDeviceMemory(odla_void* ptr) {
+  return hipFree(ptr) == hipSuccess ? ODLA_SUCCESS : ODLA_MEM_ERROR;
+}
+odla_status odla_AllocateHostMemory(odla_void** host_ptr, odla_size_t size) {
+  if (host_ptr == nullptr || size == 0) return ODLA_INVALID_PARAM;
+  return hipHostMalloc(host_ptr, size, hipHostMallocDefault) == hipSuccess ? ODLA_SUCCESS : ODLA_MEM_ERROR;
+}
+odla_status odla_FreeHostMemory(odla_void* ptr) {
+  return hipHostFree(ptr) == hipSuccess ? ODLA_SUCCESS : ODLA_MEM_ERROR;
+}
+odla_status odla_CopyMemory(odla_void* dst, odla_void* src, odla_size_t size, odla_memcpy_type type) {
+  if (dst == nullptr || src == nullptr) return ODLA_INVALID_PARAM;
+  hipMemcpyKind kind;
+  switch (type) {
+    case ODLA_MEMCPY_H2H: kind = hipMemcpyHostToHost; break;
+    case ODLA_MEMCPY_H2D: kind = hipMemcpyHostToDevice; break;
+    case ODLA_MEMCPY_D2H: kind = hipMemcpyDeviceToHost; break;
+    case ODLA_MEMCPY_D2D: kind = hipMemcpyDeviceToDevice; break;
+    default: return ODLA_INVALID_PARAM;
+  }
+  return hipMemcpy(dst, src, size, kind) == hipSuccess ? ODLA_SUCCESS : ODLA_FAILURE;
+}
+
+// ----------------------------------------------------------------- logging --
+odla_status odla_SetLogLevel(odla_log_level level) {
+  g_log_level.store((int)level);
+  return ODLA_SUCCESS;
+}
+odla_status odla_SetLogger(odla_logging_func logger) {
+  g_logger.store(logger ? logger : default_logger);
+  return ODLA_SUCCESS;
+}
+odla_logging_func odla_GetLogger(void) { return g_logger.load(); }
+
+const odla_char* odla_GetVersionString(void) { return kVersion; }
+
+}  // extern "C"

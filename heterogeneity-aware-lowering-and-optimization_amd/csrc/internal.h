@@ -1,0 +1,211 @@
+// Private structures of libodla_hip.so: the recorded graph (values + nodes),
+// the compiled plan (physical tensors + launch steps) and the execution
+// context (device arena, stream, captured hipGraph).
+#ifndef ODLA_HIP_INTERNAL_H_
+#define ODLA_HIP_INTERNAL_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/odla_hip.h"
+#include "kernels/kernels.h"
+
+namespace ohip {
+
+// ---------------------------------------------------------------- logging --
+void log_msg(const char* file, int line, const char* func, odla_log_level lvl, const char* fmt, ...)
+    __attribute__((format(printf, 5, 6)));
+#define OHIP_LOG(lvl, ...) ::ohip::log_msg(__FILE__, __LINE__, __func__, lvl, __VA_ARGS__)
+#define OHIP_ERR(...) OHIP_LOG(ODLA_LOG_LEVEL_ERROR, __VA_ARGS__)
+#define OHIP_WARN(...) OHIP_LOG(ODLA_LOG_LEVEL_WARN, __VA_ARGS__)
+#define OHIP_INFO(...) OHIP_LOG(ODLA_LOG_LEVEL_INFO, __VA_ARGS__)
+#define OHIP_DEBUG(...) OHIP_LOG(ODLA_LOG_LEVEL_DEBUG, __VA_ARGS__)
+
+// ------------------------------------------------------------------ graph --
+enum OpKind : int {
+  OP_CONV, OP_GEMM, OP_BINARY, OP_UNARY, OP_BATCHNORM, OP_LAYERNORM, OP_POOL, OP_REDUCE,
+  OP_SOFTMAX, OP_CAST, OP_CONCAT, OP_GATHER, OP_RESHAPE, OP_RESIZE, OP_SLICE, OP_TRANSPOSE,
+  OP_QUANTIZE, OP_DEQUANTIZE, OP_NMS
+};
+const char* op_name(OpKind k);
+
+struct Shape {
+  int rank = 0;
+  int64_t d[ODLA_MAX_DIMENSION] = {0};
+  int64_t numel() const {
+    int64_t n = 1;
+    for (int i = 0; i < rank; ++i) n *= d[i];
+    return n;
+  }
+  bool operator==(const Shape& o) const {
+    if (rank != o.rank) return false;
+    for (int i = 0; i < rank; ++i)
+      if (d[i] != o.d[i]) return false;
+    return true;
+  }
+  bool operator!=(const Shape& o) const { return !(*this == o); }
+  std::string str() const;
+};
+Shape shape_from(const odla_value_shape& s);    // scalars become {1}
+odla_value_shape shape_to(const Shape& s);
+bool shape_valid(const odla_value_shape& s);     // plausible caller-provided shape?
+
+struct Node;
+
+}  // namespace ohip
+
+struct _odla_computation;
+
+struct _odla_value {
+  enum Kind { ARG, CONSTANT, TEMP };
+  Kind kind = TEMP;
+  std::string name;  // empty for anonymous temporaries
+  odla_element_type etype = ODLA_FLOAT32;
+  ohip::Shape shape;
+  const void* host_data = nullptr;  // CONSTANT: borrowed from the caller
+  int index = -1;                   // position in computation->values
+  int producer = -1;                // node index, -1 for ARG / CONSTANT
+  bool is_output = false;
+  _odla_computation* comp = nullptr;
+};
+
+namespace ohip {
+
+struct Node {
+  OpKind op;
+  std::vector<_odla_value*> in;  // nullptr entries allowed for optional operands
+  _odla_value* out = nullptr;
+  // attributes (meaning depends on op; see api_ops.cc)
+  int64_t i[24] = {0};
+  float f[8] = {0};
+  std::vector<int64_t> iv;
+  bool absorbed = false;  // set by the planner when fused into another node
+};
+
+struct Options {
+  bool fp16 = false;
+  odla_bf16_mode bf16 = BF16_DISABLE;
+  bool int8 = false;
+  bool raw_acc = false;
+  const odla_value_quant_info* qtable = nullptr;
+  int qtable_size = 0;
+};
+
+// ------------------------------------------------------------------- plan --
+enum Layout : int { L_ROWMAJOR = 0, L_NHWC = 1 };
+enum Space : int { SP_ARENA = 0, SP_CONST = 1, SP_INIT = 2, SP_NONE = 3 };
+
+// A physical device tensor.  For L_NHWC the logical shape is N,C,H,W and the
+// memory order N,H,W,cs with cs >= C.
+struct PTensor {
+  DType dt = DT_F32;
+  Layout layout = L_ROWMAJOR;
+  Shape shape;      // logical
+  int cs = 0;       // channel pitch (L_NHWC only)
+  Space space = SP_NONE;
+  size_t offset = 0;
+  size_t bytes = 0;
+  int alias_of = -1;     // shares storage with another tensor (Reshape)
+  int def_step = -1, last_step = -1;
+  bool pinned = false;   // lives for the whole execution (inputs being staged, outputs)
+  bool quant = false;    // 8-bit affine levels stored as q-128
+  float qscale = 1.f;
+  int qzp = 0;
+  int64_t phys_elems() const {
+    if (layout == L_NHWC) return shape.d[0] * shape.d[2] * shape.d[3] * cs;
+    return shape.numel();
+  }
+};
+
+struct ExecEnv {
+  char* base[3] = {nullptr, nullptr, nullptr};  // indexed by Space
+};
+
+struct Step {
+  std::string name;
+  std::function<hipError_t(const ExecEnv&, hipStream_t)> fn;
+};
+
+struct QuantEntry {
+  float scale = 0.f;
+  int zp = 0;
+  float min = 0.f, max = 0.f;
+  std::vector<float> ch_min, ch_max;
+};
+
+struct Plan {
+  std::vector<PTensor> tensors;
+  std::vector<Step> steps;       // replayed on every execution
+  std::vector<Step> init_steps;  // run once when the plan is created
+  size_t arena_bytes = 0;
+  size_t const_bytes = 0;
+  size_t init_bytes = 0;
+  char* const_pool = nullptr;
+  struct IO {
+    _odla_value* v = nullptr;
+    int tensor = -1;  // staging tensor in the arena: row-major, declared element type
+    size_t bytes = 0;
+  };
+  std::vector<IO> inputs, outputs;
+  std::unordered_map<const _odla_value*, int> final_tensor;  // for odla_GetValueData
+  // host blobs copied into the constant pool / init scratch when the plan is built
+  struct Blob { Space space; size_t offset; std::vector<uint8_t> owned; const void* src; size_t bytes; };
+  std::vector<Blob> blobs;
+  ~Plan();
+};
+
+odla_status build_plan(_odla_computation* comp, std::unique_ptr<Plan>* out);
+
+DType dtype_from_odla(odla_element_type t);
+int odla_type_size(odla_element_type t);
+
+}  // namespace ohip
+
+struct _odla_computation {
+  std::vector<std::unique_ptr<_odla_value>> values;
+  std::vector<ohip::Node> nodes;
+  std::vector<_odla_value*> args, outputs;
+  std::unordered_map<std::string, _odla_value*> by_name;
+  // library-created constants (scalars, folded parameters)
+  std::vector<std::unique_ptr<std::vector<uint8_t>>> owned_data;
+  ohip::Options opts;
+  std::mutex mu;
+  std::unique_ptr<ohip::Plan> plan;
+  bool plan_failed = false;
+};
+
+struct _odla_context {
+  _odla_computation* comp = nullptr;
+  hipStream_t stream = nullptr;
+  char* arena = nullptr;
+  size_t arena_bytes = 0;
+  bool use_graph = true;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t graph_exec = nullptr;
+  std::unordered_map<const _odla_value*, const void*> bound_in;
+  std::unordered_map<const _odla_value*, void*> bound_out;
+  bool executed = false;
+};
+
+struct _odla_device {
+  int index = 0;
+};
+
+namespace ohip {
+_odla_computation* current_computation();
+void set_current_computation(_odla_computation* c);
+void forget_computation(_odla_computation* c);
+_odla_value* new_value(_odla_computation* c, _odla_value::Kind kind, odla_element_type et,
+                       const Shape& shape, const odla_value_id id);
+}  // namespace ohip
+
+#endif

@@ -1,0 +1,167 @@
+// Device-side helpers shared by the gfx950 kernels: storage-type traits,
+// 16-byte vector access, activation functions, wavefront reductions.
+#ifndef ODLA_HIP_DEVICE_UTILS_H_
+#define ODLA_HIP_DEVICE_UTILS_H_
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "kernels.h"
+
+namespace ohip {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+// Round to nearest even; NaN stays NaN.
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float f16_to_f32(uint16_t h) {
+  _Float16 v;
+  __builtin_memcpy(&v, &h, 2);
+  return (float)v;
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  _Float16 v = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
+  uint16_t h;
+  __builtin_memcpy(&h, &v, 2);
+  return h;
+}
+
+// Storage traits: load/store one element as float.
+template <typename T> struct Store;
+template <> struct Store<float> {
+  static constexpr DType dt = DT_F32;
+  __device__ static __forceinline__ float ld(const float* p) { return *p; }
+  __device__ static __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct Store<f16_t> {
+  static constexpr DType dt = DT_F16;
+  __device__ static __forceinline__ float ld(const f16_t* p) { return f16_to_f32(p->bits); }
+  __device__ static __forceinline__ void st(f16_t* p, float v) { p->bits = f32_to_f16(v); }
+};
+template <> struct Store<bf16_t> {
+  static constexpr DType dt = DT_BF16;
+  __device__ static __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(p->bits); }
+  __device__ static __forceinline__ void st(bf16_t* p, float v) { p->bits = f32_to_bf16(v); }
+};
+
+// 16-byte vector of T viewed as floats.
+template <typename T> struct Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  uintx4 raw;
+  __device__ __forceinline__ void load(const T* p) { raw = *reinterpret_cast<const uintx4*>(p); }
+  __device__ __forceinline__ void store(T* p) const { *reinterpret_cast<uintx4*>(p) = raw; }
+  __device__ __forceinline__ float get(int i) const {
+    const T* e = reinterpret_cast<const T*>(&raw);
+    return Store<T>::ld(e + i);
+  }
+  __device__ __forceinline__ void set(int i, float v) {
+    T* e = reinterpret_cast<T*>(&raw);
+    Store<T>::st(e + i, v);
+  }
+};
+
+__device__ __forceinline__ float gelu_erf(float x) {
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float k = 0.79788456080286535588f;  // sqrt(2/pi)
+  return 0.5f * x * (1.0f + tanhf(k * (x + 0.044715f * x * x * x)));
+}
+
+__device__ __forceinline__ float apply_act(float v, ActKind act, float a, float b) {
+  switch (act) {
+    case ACT_NONE: return v;
+    case ACT_RELU: return v > 0.f ? v : 0.f;
+    case ACT_LEAKY: return v > 0.f ? v : a * v;
+    case ACT_CLAMP: return fminf(fmaxf(v, a), b);
+    case ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+    case ACT_TANH: return tanhf(v);
+    case ACT_GELU_ERF: return gelu_erf(v);
+    case ACT_GELU_TANH: return gelu_tanh(v);
+    case ACT_EXP: return expf(v);
+    case ACT_LOG: return logf(v);
+    case ACT_SQRT: return sqrtf(v);
+    case ACT_RSQRT: return 1.0f / sqrtf(v);
+    case ACT_ERF: return erff(v);
+    case ACT_ABS: return fabsf(v);
+    case ACT_NEG: return -v;
+    case ACT_ROUND: return rintf(v);
+    case ACT_RECIP: return 1.0f / v;
+  }
+  return v;
+}
+
+// Wavefront (64 lanes) reductions through cross-lane shuffles.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Block-wide reductions for blocks of NT threads (NT multiple of 64, <= 1024).
+// `smem` must hold NT/64 floats; every thread receives the result.
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* smem) {
+  v = wave_sum(v);
+  if (NT == 64) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) smem[w] = v;
+  __syncthreads();
+  float r = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / 64; ++i) r += smem[i];
+  return r;
+}
+template <int NT>
+__device__ __forceinline__ float block_max(float v, float* smem) {
+  v = wave_max(v);
+  if (NT == 64) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) smem[w] = v;
+  __syncthreads();
+  float r = smem[0];
+#pragma unroll
+  for (int i = 1; i < NT / 64; ++i) r = fmaxf(r, smem[i]);
+  return r;
+}
+
+// Quantised 8-bit activations are stored as q-128 (int8); these convert
+// between the stored byte and the unsigned level q in [0,255].
+__device__ __forceinline__ int q_from_stored(int8_t s) { return (int)s + 128; }
+__device__ __forceinline__ int8_t q_to_stored(int q) { return (int8_t)(q - 128); }
+
+inline int grid_for(int64_t work_items, int per_block, int max_blocks = 256 * 32) {
+  int64_t g = (work_items + per_block - 1) / per_block;
+  if (g < 1) g = 1;
+  if (g > max_blocks) g = max_blocks;
+  return (int)g;
+}
+
+}  // namespace ohip
+#endif

@@ -1,0 +1,440 @@
+// Streaming element-wise kernels for gfx950: unary activations, per-channel
+// affine (folded BatchNorm), broadcasting binary ops, casts and affine
+// (de)quantisation.  All are HBM-bound: each thread moves 16-byte vectors,
+// consecutive lanes touch consecutive vectors, and the grid is a grid-stride
+// loop sized to a few workgroups per CU.
+#include "device_utils.h"
+
+namespace ohip {
+
+namespace {
+constexpr int kThreads = 256;
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, ActKind act, float a, float b) {
+  constexpr int V = Vec16<T>::N;
+  const int64_t nvec = n / V;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    Vec16<T> v;
+    v.load(x + i * V);
+#pragma unroll
+    for (int e = 0; e < V; ++e) v.set(e, apply_act(v.get(e), act, a, b));
+    v.store(y + i * V);
+  }
+  // tail
+  const int64_t tail0 = nvec * V;
+  for (int64_t i = tail0 + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
+    Store<T>::st(y + i, apply_act(Store<T>::ld(x + i), act, a, b));
+}
+
+// y = x * scale[c] + shift[c].  INNER1: channel is the innermost index
+// (channels-last), so a vector spans consecutive channels; otherwise the
+// channel is constant across a vector when inner % V == 0.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+channel_affine_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, int64_t inner,
+                      int channels, const float* __restrict__ scale,
+                      const float* __restrict__ shift) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  constexpr int V = Vec16<T>::N;
+  const bool vec_ok = (inner == 1) ? (channels % V == 0) : (inner % V == 0);
+  if (vec_ok) {
+    const int64_t nvec = n / V;
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
+      Vec16<T> v;
+      v.load(x + i * V);
+      const int64_t e0 = i * V;
+      if (inner == 1) {
+        const int c0 = (int)(e0 % channels);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v.set(e, v.get(e) * scale[c0 + e] + shift[c0 + e]);
+      } else {
+        const int c = (int)((e0 / inner) % channels);
+        const float s = scale[c], t = shift[c];
+#pragma unroll
+        for (int e = 0; e < V; ++e) v.set(e, v.get(e) * s + t);
+      }
+      v.store(y + i * V);
+    }
+  } else {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      const int c = (int)((i / inner) % channels);
+      Store<T>::st(y + i, Store<T>::ld(x + i) * scale[c] + shift[c]);
+    }
+  }
+}
+
+__global__ void bn_fold_kernel(const float* mean, const float* var, const float* gamma,
+                               const float* beta, float sgamma, float sbeta, float eps,
+                               int channels, float* scale, float* shift) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const float g = gamma ? gamma[c] : sgamma;
+  const float b = beta ? beta[c] : sbeta;
+  const float m = g / sqrtf(var[c] + eps);
+  scale[c] = m;
+  shift[c] = b - mean[c] * m;
+}
+
+__device__ __forceinline__ float bin_op(float a, float b, BinKind op) {
+  switch (op) {
+    case BIN_ADD: return a + b;
+    case BIN_SUB: return a - b;
+    case BIN_MUL: return a * b;
+    case BIN_DIV: return a / b;
+    case BIN_MAX: return fmaxf(a, b);
+    case BIN_MIN: return fminf(a, b);
+  }
+  return a;
+}
+
+// Same-shape, contiguous operands.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+binary_flat_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, int64_t n,
+                   BinKind op, ActKind act, float aa, float ab) {
+  constexpr int V = Vec16<T>::N;
+  const int64_t nvec = n / V;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    Vec16<T> va, vb;
+    va.load(a + i * V);
+    vb.load(b + i * V);
+#pragma unroll
+    for (int e = 0; e < V; ++e) va.set(e, apply_act(bin_op(va.get(e), vb.get(e), op), act, aa, ab));
+    va.store(y + i * V);
+  }
+  for (int64_t i = nvec * V + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
+    Store<T>::st(y + i, apply_act(bin_op(Store<T>::ld(a + i), Store<T>::ld(b + i), op), act, aa, ab));
+}
+
+// One operand is a vector indexed by the innermost output dim (bias rows,
+// channels-last per-channel constants): b index = i % period.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+binary_rowvec_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y,
+                     int64_t n, int period, bool b_is_lhs, BinKind op, ActKind act, float aa,
+                     float ab) {
+  constexpr int V = Vec16<T>::N;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  if (period % V == 0) {
+    const int64_t nvec = n / V;
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
+      Vec16<T> va, vb;
+      va.load(a + i * V);
+      vb.load(b + (i * V) % period);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float l = b_is_lhs ? vb.get(e) : va.get(e);
+        const float r = b_is_lhs ? va.get(e) : vb.get(e);
+        va.set(e, apply_act(bin_op(l, r, op), act, aa, ab));
+      }
+      va.store(y + i * V);
+    }
+  } else {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+      const float av = Store<T>::ld(a + i), bv = Store<T>::ld(b + i % period);
+      Store<T>::st(y + i, apply_act(b_is_lhs ? bin_op(bv, av, op) : bin_op(av, bv, op), act, aa, ab));
+    }
+  }
+}
+
+// General broadcast: decompose the flat output index over `rank` dims.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+binary_bcast_kernel(BinaryParams p, int64_t n) {
+  const T* a = reinterpret_cast<const T*>(p.a);
+  const T* b = reinterpret_cast<const T*>(p.b);
+  T* y = reinterpret_cast<T*>(p.y);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+    int64_t rem = i, oa = 0, ob = 0;
+#pragma unroll
+    for (int d = 5; d >= 0; --d) {
+      if (d < p.rank) {
+        const int64_t q = rem / p.dims[d];
+        const int64_t idx = rem - q * p.dims[d];
+        rem = q;
+        oa += idx * p.sa[d];
+        ob += idx * p.sb[d];
+      }
+    }
+    Store<T>::st(y + i, apply_act(bin_op(Store<T>::ld(a + oa), Store<T>::ld(b + ob), p.op), p.act,
+                                  p.act_a, p.act_b));
+  }
+}
+
+// Quantised add (8-bit levels stored as q-128), same shape, contiguous:
+// the float sequence dequantise, op, requantise of the unfused graph.
+__global__ void __launch_bounds__(kThreads)
+binary_q8_kernel(BinaryParams p, int64_t n) {
+  const int8_t* a = reinterpret_cast<const int8_t*>(p.a);
+  const int8_t* b = reinterpret_cast<const int8_t*>(p.b);
+  int8_t* y = reinterpret_cast<int8_t*>(p.y);
+  const int64_t nvec = n / 16;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  auto one = [&](int8_t sa, int8_t sb) -> int8_t {
+    const float fa = (float)(q_from_stored(sa) - p.a_zp) * p.a_scale;
+    const float fb = (float)(q_from_stored(sb) - p.b_zp) * p.b_scale;
+    const float f = bin_op(fa, fb, p.op);
+    int q = (int)rintf(f * p.y_inv) + p.y_zp;
+    q = q < p.y_lo ? p.y_lo : q;
+    q = q > 255 ? 255 : q;
+    return q_to_stored(q);
+  };
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    uintx4 va = *reinterpret_cast<const uintx4*>(a + i * 16);
+    uintx4 vb = *reinterpret_cast<const uintx4*>(b + i * 16);
+    const int8_t* ea = reinterpret_cast<const int8_t*>(&va);
+    const int8_t* eb = reinterpret_cast<const int8_t*>(&vb);
+    uintx4 vo;
+    int8_t* eo = reinterpret_cast<int8_t*>(&vo);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) eo[e] = one(ea[e], eb[e]);
+    *reinterpret_cast<uintx4*>(y + i * 16) = vo;
+  }
+  for (int64_t i = nvec * 16 + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
+    y[i] = one(a[i], b[i]);
+}
+
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads)
+cast_kernel(const TS* __restrict__ x, TD* __restrict__ y, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  // 4 elements per thread step keeps loads/stores >= 8 bytes for 16-bit types.
+  const int64_t n4 = n / 4;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += stride) {
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = Store<TS>::ld(x + i * 4 + e);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) Store<TD>::st(y + i * 4 + e, v[e]);
+  }
+  for (int64_t i = n4 * 4 + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
+    Store<TD>::st(y + i, Store<TS>::ld(x + i));
+}
+
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads)
+cast_int_kernel(const TS* __restrict__ x, TD* __restrict__ y, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
+    y[i] = (TD)x[i];
+}
+
+// q = sat(rne(x / scale) + zp)
+template <typename TS>
+__global__ void __launch_bounds__(kThreads)
+quantize_kernel(QuantParams p) {
+  const TS* x = reinterpret_cast<const TS*>(p.src);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < p.n; i += stride) {
+    const int c = (p.channels > 1) ? (int)((i / p.inner) % p.channels) : 0;
+    const float r = rintf(Store<TS>::ld(x + i) / p.scale[c]);
+    const float zf = p.zp ? (float)p.zp[c] : 0.f;
+    const float t = r + zf;  // the reference adds the zero point in float before the saturating cast
+    if (p.dst_signed) {
+      const float s = fminf(fmaxf(t, -128.f), 127.f);
+      reinterpret_cast<int8_t*>(p.dst)[i] = (int8_t)(int)s;
+    } else {
+      const float s = fminf(fmaxf(t, 0.f), 255.f);
+      const int q = (int)s;
+      if (p.dst_dt == DT_I8) reinterpret_cast<int8_t*>(p.dst)[i] = q_to_stored(q);
+      else reinterpret_cast<uint8_t*>(p.dst)[i] = (uint8_t)q;
+    }
+  }
+}
+
+// x = (q - zp) * scale
+template <typename TD>
+__global__ void __launch_bounds__(kThreads)
+dequantize_kernel(QuantParams p) {
+  TD* y = reinterpret_cast<TD*>(p.dst);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < p.n; i += stride) {
+    const int c = (p.channels > 1) ? (int)((i / p.inner) % p.channels) : 0;
+    float q;
+    if (p.src_dt == DT_U8) q = (float)reinterpret_cast<const uint8_t*>(p.src)[i];
+    else if (p.dst_signed) q = (float)reinterpret_cast<const int8_t*>(p.src)[i];
+    else q = (float)q_from_stored(reinterpret_cast<const int8_t*>(p.src)[i]);
+    const float zf = p.zp ? (float)p.zp[c] : 0.f;
+    Store<TD>::st(y + i, (q - zf) * p.scale[c]);
+  }
+}
+
+__global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+}  // namespace
+
+#define FLOAT_DISPATCH(dt, EXPR)                         \
+  switch (dt) {                                          \
+    case DT_F32: { using T = float; EXPR; break; }       \
+    case DT_F16: { using T = f16_t; EXPR; break; }       \
+    case DT_BF16: { using T = bf16_t; EXPR; break; }     \
+    default: return hipErrorInvalidValue;                \
+  }
+
+hipError_t launch_unary(const void* x, void* y, DType dt, int64_t n, ActKind act, float a, float b,
+                        hipStream_t stream) {
+  if (n <= 0) return n == 0 ? hipSuccess : hipErrorInvalidValue;
+  if (!x || !y || !al16(x) || !al16(y)) return hipErrorInvalidValue;
+  const int grid = grid_for(n, kThreads * 8);
+  FLOAT_DISPATCH(dt, hipLaunchKernelGGL(unary_kernel<T>, dim3(grid), dim3(kThreads), 0, stream,
+                                        (const T*)x, (T*)y, n, act, a, b));
+  return hipGetLastError();
+}
+
+hipError_t launch_channel_affine(const void* x, void* y, DType dt, int64_t n, int64_t inner,
+                                 int channels, const float* scale, const float* shift,
+                                 hipStream_t stream) {
+  if (n <= 0) return n == 0 ? hipSuccess : hipErrorInvalidValue;
+  if (!x || !y || !scale || !shift || !al16(x) || !al16(y) || inner <= 0 || channels <= 0)
+    return hipErrorInvalidValue;
+  if (n % (inner * channels) != 0) return hipErrorInvalidValue;
+  const int grid = grid_for(n, kThreads * 8);
+  FLOAT_DISPATCH(dt, hipLaunchKernelGGL(channel_affine_kernel<T>, dim3(grid), dim3(kThreads), 0,
+                                        stream, (const T*)x, (T*)y, n, inner, channels, scale, shift));
+  return hipGetLastError();
+}
+
+hipError_t launch_bn_fold(const float* mean, const float* var, const float* gamma,
+                          const float* beta, float sgamma, float sbeta, float eps, int channels,
+                          float* scale, float* shift, hipStream_t stream) {
+  if (!mean || !var || !scale || !shift || channels <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(bn_fold_kernel, dim3((channels + 255) / 256), dim3(256), 0, stream, mean, var,
+                     gamma, beta, sgamma, sbeta, eps, channels, scale, shift);
+  return hipGetLastError();
+}
+
+hipError_t launch_binary(const BinaryParams& p, hipStream_t stream) {
+  if (!p.a || !p.b || !p.y || p.rank < 1 || p.rank > 6) return hipErrorInvalidValue;
+  int64_t n = 1;
+  for (int d = 0; d < p.rank; ++d) {
+    if (p.dims[d] <= 0) return hipErrorInvalidValue;
+    n *= p.dims[d];
+  }
+  // contiguous strides of the output
+  int64_t cs[6];
+  {
+    int64_t s = 1;
+    for (int d = p.rank - 1; d >= 0; --d) { cs[d] = s; s *= p.dims[d]; }
+  }
+  auto is_full = [&](const int64_t* st) {
+    for (int d = 0; d < p.rank; ++d)
+      if (p.dims[d] != 1 && st[d] != cs[d]) return false;
+    return true;
+  };
+  // operand indexed only by a trailing block of dims (contiguous there), 0 elsewhere
+  auto rowvec_period = [&](const int64_t* st) -> int64_t {
+    int d = p.rank - 1;
+    int64_t period = 1;
+    while (d >= 0 && (p.dims[d] == 1 || st[d] == cs[d])) { period *= p.dims[d]; --d; }
+    for (; d >= 0; --d)
+      if (p.dims[d] != 1 && st[d] != 0) return -1;
+    return period;
+  };
+  const int grid = grid_for(n, kThreads * 8);
+  if (p.dt == DT_I8) {
+    if (!is_full(p.sa) || !is_full(p.sb) || !al16(p.a) || !al16(p.b) || !al16(p.y))
+      return hipErrorInvalidValue;
+    hipLaunchKernelGGL(binary_q8_kernel, dim3(grid_for(n, kThreads * 16)), dim3(kThreads), 0, stream, p, n);
+    return hipGetLastError();
+  }
+  const bool aligned = al16(p.a) && al16(p.b) && al16(p.y);
+  if (aligned && is_full(p.sa) && is_full(p.sb)) {
+    FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL(binary_flat_kernel<T>, dim3(grid), dim3(kThreads), 0, stream,
+                                            (const T*)p.a, (const T*)p.b, (T*)p.y, n, p.op, p.act,
+                                            p.act_a, p.act_b));
+    return hipGetLastError();
+  }
+  if (aligned && is_full(p.sa)) {
+    const int64_t per = rowvec_period(p.sb);
+    if (per > 0 && per < (1ll << 30)) {
+      FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL(binary_rowvec_kernel<T>, dim3(grid), dim3(kThreads), 0,
+                                              stream, (const T*)p.a, (const T*)p.b, (T*)p.y, n, (int)per,
+                                              false, p.op, p.act, p.act_a, p.act_b));
+      return hipGetLastError();
+    }
+  }
+  if (aligned && is_full(p.sb)) {
+    const int64_t per = rowvec_period(p.sa);
+    if (per > 0 && per < (1ll << 30)) {
+      FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL(binary_rowvec_kernel<T>, dim3(grid), dim3(kThreads), 0,
+                                              stream, (const T*)p.b, (const T*)p.a, (T*)p.y, n, (int)per,
+                                              true, p.op, p.act, p.act_a, p.act_b));
+      return hipGetLastError();
+    }
+  }
+  FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL(binary_bcast_kernel<T>, dim3(grid_for(n, kThreads * 2)),
+                                          dim3(kThreads), 0, stream, p, n));
+  return hipGetLastError();
+}
+
+hipError_t launch_cast(const void* src, DType sdt, void* dst, DType ddt, int64_t n, hipStream_t stream) {
+  if (n <= 0) return n == 0 ? hipSuccess : hipErrorInvalidValue;
+  if (!src || !dst) return hipErrorInvalidValue;
+  const int grid = grid_for(n, kThreads * 4);
+#define CAST_CASE(S_, D_, TS_, TD_, K_)                                                   \
+  if (sdt == S_ && ddt == D_) {                                                           \
+    hipLaunchKernelGGL((K_<TS_, TD_>), dim3(grid), dim3(kThreads), 0, stream, (const TS_*)src, \
+                       (TD_*)dst, n);                                                     \
+    return hipGetLastError();                                                             \
+  }
+  CAST_CASE(DT_F32, DT_F16, float, f16_t, cast_kernel)
+  CAST_CASE(DT_F32, DT_BF16, float, bf16_t, cast_kernel)
+  CAST_CASE(DT_F16, DT_F32, f16_t, float, cast_kernel)
+  CAST_CASE(DT_BF16, DT_F32, bf16_t, float, cast_kernel)
+  CAST_CASE(DT_F32, DT_F32, float, float, cast_kernel)
+  CAST_CASE(DT_F16, DT_F16, f16_t, f16_t, cast_kernel)
+  CAST_CASE(DT_BF16, DT_BF16, bf16_t, bf16_t, cast_kernel)
+  CAST_CASE(DT_F16, DT_BF16, f16_t, bf16_t, cast_kernel)
+  CAST_CASE(DT_BF16, DT_F16, bf16_t, f16_t, cast_kernel)
+  CAST_CASE(DT_I64, DT_I32, int64_t, int32_t, cast_int_kernel)
+  CAST_CASE(DT_I32, DT_I64, int32_t, int64_t, cast_int_kernel)
+  CAST_CASE(DT_I32, DT_F32, int32_t, float, cast_int_kernel)
+  CAST_CASE(DT_I64, DT_F32, int64_t, float, cast_int_kernel)
+  CAST_CASE(DT_F32, DT_I32, float, int32_t, cast_int_kernel)
+  CAST_CASE(DT_F32, DT_I64, float, int64_t, cast_int_kernel)
+  CAST_CASE(DT_U8, DT_F32, uint8_t, float, cast_int_kernel)
+  CAST_CASE(DT_I8, DT_F32, int8_t, float, cast_int_kernel)
+  CAST_CASE(DT_BOOL, DT_F32, uint8_t, float, cast_int_kernel)
+  CAST_CASE(DT_I32, DT_I32, int32_t, int32_t, cast_int_kernel)
+  CAST_CASE(DT_I64, DT_I64, int64_t, int64_t, cast_int_kernel)
+  CAST_CASE(DT_U8, DT_U8, uint8_t, uint8_t, cast_int_kernel)
+  CAST_CASE(DT_I8, DT_I8, int8_t, int8_t, cast_int_kernel)
+#undef CAST_CASE
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_quantize(const QuantParams& p, hipStream_t stream) {
+  if (p.n <= 0) return p.n == 0 ? hipSuccess : hipErrorInvalidValue;
+  if (!p.src || !p.dst || !p.scale || p.channels <= 0 || p.inner <= 0) return hipErrorInvalidValue;
+  if (p.dst_dt != DT_U8 && p.dst_dt != DT_I8) return hipErrorInvalidValue;
+  const int grid = grid_for(p.n, kThreads * 4);
+  FLOAT_DISPATCH(p.src_dt, hipLaunchKernelGGL(quantize_kernel<T>, dim3(grid), dim3(kThreads), 0, stream, p));
+  return hipGetLastError();
+}
+
+hipError_t launch_dequantize(const QuantParams& p, hipStream_t stream) {
+  if (p.n <= 0) return p.n == 0 ? hipSuccess : hipErrorInvalidValue;
+  if (!p.src || !p.dst || !p.scale || p.channels <= 0 || p.inner <= 0) return hipErrorInvalidValue;
+  if (p.src_dt != DT_U8 && p.src_dt != DT_I8) return hipErrorInvalidValue;
+  const int grid = grid_for(p.n, kThreads * 4);
+  FLOAT_DISPATCH(p.dst_dt, hipLaunchKernelGGL(dequantize_kernel<T>, dim3(grid), dim3(kThreads), 0, stream, p));
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t stream) {
+  if (n <= 0) return n == 0 ? hipSuccess : hipErrorInvalidValue;
+  if (!p) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(n, 256)), dim3(256), 0, stream, p, n, v);
+  return hipGetLastError();
+}
+
+}  // namespace ohip

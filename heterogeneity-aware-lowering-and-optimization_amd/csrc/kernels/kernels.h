@@ -1,0 +1,231 @@
+// Host-visible launch interface of the gfx950 kernels behind libodla_hip.so.
+//
+// Every launcher validates its operands on the host before enqueueing work on
+// `stream` and returns hipErrorInvalidValue instead of launching a kernel whose
+// indexing assumptions do not hold.  Nothing here allocates memory.
+#ifndef ODLA_HIP_KERNELS_H_
+#define ODLA_HIP_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ohip {
+
+// Storage types of device tensors.
+enum DType : int {
+  DT_F32 = 0,
+  DT_F16 = 1,
+  DT_BF16 = 2,
+  DT_I8 = 3,  // quantised activations are stored as (q - 128) in int8 so that
+              // unsigned 8-bit data feeds the signed MFMA; weights are plain s8
+  DT_U8 = 4,
+  DT_I32 = 5,
+  DT_I64 = 6,
+  DT_BOOL = 7,
+  DT_INVALID = -1
+};
+
+inline int dtype_size(DType t) {
+  switch (t) {
+    case DT_F32: case DT_I32: return 4;
+    case DT_F16: case DT_BF16: return 2;
+    case DT_I8: case DT_U8: case DT_BOOL: return 1;
+    case DT_I64: return 8;
+    default: return 0;
+  }
+}
+inline bool dtype_is_float(DType t) { return t == DT_F32 || t == DT_F16 || t == DT_BF16; }
+
+// Activation applied in a GEMM epilogue or by the unary kernel.
+enum ActKind : int {
+  ACT_NONE = 0, ACT_RELU, ACT_LEAKY, ACT_CLAMP, ACT_SIGMOID, ACT_TANH,
+  ACT_GELU_ERF, ACT_GELU_TANH, ACT_EXP, ACT_LOG, ACT_SQRT, ACT_RSQRT, ACT_ERF,
+  ACT_ABS, ACT_NEG, ACT_ROUND, ACT_RECIP
+};
+
+enum BinKind : int { BIN_ADD = 0, BIN_SUB, BIN_MUL, BIN_DIV, BIN_MAX, BIN_MIN };
+
+// ---------------------------------------------------------------------------
+// Implicit-GEMM convolution / GEMM on MFMA.
+//
+//   y[z][m][n] = epilogue( sum_k A[z][m][k] * Wt[z][n][k] )
+//
+// A is gathered on the fly from a channels-last activation tensor
+// x[z][N][H][W][xcs] (m = (n,ho,wo), k = (r,s,c), c < C); a plain GEMM is the
+// case H = W = R = S = 1.  Wt is a row-major [w_rows][w_rs] matrix whose row n
+// holds output channel n with k ordered (r,s,c); rows >= w_rows and columns
+// >= w_cols are read as zero.  C and w_rs must be multiples of 16 bytes worth
+// of elements, x and w 16-byte aligned.
+struct IgemmParams {
+  const void* x = nullptr;
+  const void* w = nullptr;
+  void* y = nullptr;
+  const void* bias = nullptr;      // float[Kout] (int32[Kout] for int8), or null
+  const void* residual = nullptr;  // same type/geometry as y, or null
+  int N = 1, H = 1, W = 1, C = 0;  // C = reduction channels per tap
+  int xcs = 0;                     // element stride between pixels of x
+  int Ho = 1, Wo = 1, Kout = 0;
+  int R = 1, S = 1, sh = 1, sw = 1, ph = 0, pw = 0, dh = 1, dw = 1;
+  int w_rows = 0, w_cols = 0, w_rs = 0;
+  int ycs = 0;                     // element stride between rows of y
+  int rcs = 0;                     // element stride between rows of residual
+  int batch = 1;                   // grid.z: independent problems (groups, heads)
+  int64_t x_bs = 0, w_bs = 0, y_bs = 0, r_bs = 0, bias_bs = 0;  // per-z element strides
+  DType in_dt = DT_F32;            // type of x and w
+  DType out_dt = DT_F32;           // type of y and residual
+  float alpha = 1.0f;              // scales the accumulator before bias (float types)
+  ActKind act = ACT_NONE;
+  float act_a = 0.0f, act_b = 0.0f;  // leaky slope / clamp lo,hi
+  // int8 only -----------------------------------------------------------
+  // out_dt == DT_I8 : q = clamp(rne(float(acc+bias) * qmul[n]) + q_zp, q_lo, 255)
+  //                   then, if residual: the unfused sequence
+  //                   f = (q - q_zp) * q_scale + (res - r_zp) * r_scale,
+  //                   q = clamp(rne(f * s_inv) + s_zp, s_lo, 255)
+  // out_dt == DT_F32: y = float(acc+bias) * qmul[n]    (dequantised result)
+  // out_dt == DT_I32: y = acc + bias                   (raw accumulators)
+  const float* qmul = nullptr;
+  int a_fill = 0;  // stored byte that represents the real value 0 in x
+  int q_zp = 0, q_lo = 0;
+  float q_scale = 0.f;
+  int r_zp = 0; float r_scale = 0.f;
+  float s_inv = 0.f; int s_zp = 0, s_lo = 0;
+};
+hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream);
+// Name of the kernel variant launch_igemm would pick (for reports).
+const char* igemm_variant_name(const IgemmParams& p);
+
+// Repack a weight tensor into the [G][rows_pad][w_rs] matrix launch_igemm reads.
+// src element (o, i, r, s) lives at o*so + i*si + r*sr + s*ss.
+struct PackWeightsParams {
+  const void* src = nullptr; void* dst = nullptr;
+  DType src_dt = DT_F32, dst_dt = DT_F32;
+  int G = 1, Og = 0, Cg = 0, R = 1, S = 1;  // per-group out / in channels
+  int Cp = 0;                               // padded in-channels per tap (>= Cg)
+  int rows_pad = 0, w_rs = 0;
+  int64_t so = 0, si = 0, sr = 0, ss = 0;
+};
+hipError_t launch_pack_weights(const PackWeightsParams& p, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// Layout conversion between row-major N,C,HW (any float type) and
+// channels-last N,HW,cs with optional channel padding (pad lanes get `fill`).
+struct LayoutParams {
+  const void* src = nullptr; void* dst = nullptr;
+  DType src_dt = DT_F32, dst_dt = DT_F32;
+  int N = 0, C = 0, HW = 0;
+  int cs = 0;          // channel stride of the channels-last side (>= C)
+  // Optional affine quantisation when dst_dt == DT_I8 (to_nhwc) or
+  // dequantisation when src_dt == DT_I8 (to_nchw).
+  float scale = 1.f; int zp = 0;
+};
+hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream);
+hipError_t launch_nhwc_to_nchw(const LayoutParams& p, hipStream_t stream);
+
+// Flat conversions -------------------------------------------------------
+hipError_t launch_cast(const void* src, DType sdt, void* dst, DType ddt, int64_t n,
+                       hipStream_t stream);
+// q = sat(rne(x / scale[c]) + zp[c]); channel c = (i / inner) % channels.
+struct QuantParams {
+  const void* src = nullptr; void* dst = nullptr;
+  DType src_dt = DT_F32, dst_dt = DT_U8;   // DT_I8 here means "stored q-128" of an unsigned q
+  bool dst_signed = false;                 // true: saturate to [-128,127] and store as is
+  const float* scale = nullptr;            // [channels]
+  const int32_t* zp = nullptr;             // [channels] or null
+  int64_t n = 0, inner = 1; int channels = 1;
+};
+hipError_t launch_quantize(const QuantParams& p, hipStream_t stream);
+hipError_t launch_dequantize(const QuantParams& p, hipStream_t stream);  // src int, dst float
+
+// ---------------------------------------------------------------------------
+// Streaming element-wise kernels (flat, 16-byte vectorised).
+hipError_t launch_unary(const void* x, void* y, DType dt, int64_t n, ActKind act,
+                        float a, float b, hipStream_t stream);
+// y = x * scale[c] + shift[c], c = (i / inner) % channels   (folded BatchNorm)
+hipError_t launch_channel_affine(const void* x, void* y, DType dt, int64_t n,
+                                 int64_t inner, int channels, const float* scale,
+                                 const float* shift, hipStream_t stream);
+// scale/shift from BatchNorm statistics, computed on the device for
+// non-constant operands.  Any of gamma/beta may be null (scalars used instead).
+hipError_t launch_bn_fold(const float* mean, const float* var, const float* gamma,
+                          const float* beta, float sgamma, float sbeta, float eps,
+                          int channels, float* scale, float* shift, hipStream_t stream);
+
+// Binary with broadcast.  Output is described by up to 6 physical dims; each
+// operand has one element stride per dim (0 where it broadcasts).
+struct BinaryParams {
+  const void* a = nullptr; const void* b = nullptr; void* y = nullptr;
+  DType dt = DT_F32;        // all three tensors
+  BinKind op = BIN_ADD;
+  int rank = 1;
+  int64_t dims[6] = {1, 1, 1, 1, 1, 1};
+  int64_t sa[6] = {0}, sb[6] = {0};
+  ActKind act = ACT_NONE; float act_a = 0.f, act_b = 0.f;
+  // int8 tensors (dt == DT_I8): f = (a-a_zp)*a_scale op (b-b_zp)*b_scale;
+  // q = clamp(rne(f * y_inv) + y_zp, y_lo, 255)
+  float a_scale = 0.f, b_scale = 0.f, y_inv = 0.f; int a_zp = 0, b_zp = 0, y_zp = 0, y_lo = 0;
+};
+hipError_t launch_binary(const BinaryParams& p, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// Pooling on channels-last tensors x[N][H][W][cs] -> y[N][Ho][Wo][ycs].
+struct PoolParams {
+  const void* x = nullptr; void* y = nullptr;
+  DType dt = DT_F32;
+  int N = 0, H = 0, W = 0, C = 0, cs = 0, Ho = 0, Wo = 0, ycs = 0;
+  int kh = 1, kw = 1, sh = 1, sw = 1, ph = 0, pw = 0;
+  bool is_max = true;
+  bool count_include_pad = false;
+  // int8 average pooling: q = clamp(rne(mean(q_in - zp_in) * mul) + zp_out)
+  float q_mul = 1.f; int zp_in = 0, zp_out = 0;
+};
+hipError_t launch_pool2d(const PoolParams& p, hipStream_t stream);
+
+// Row reductions / normalisations over a contiguous inner axis:
+// x viewed as [outer][len][inner]; one result column per (outer, inner).
+enum ReduceKind : int { RED_MEAN = 0, RED_SUM, RED_MAX };
+hipError_t launch_reduce(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
+                         int64_t len, int64_t inner, ReduceKind kind, hipStream_t stream);
+// Mean over the middle axis of 8-bit levels (stored q-128): fp32 result
+// y = ((sum q - len*zp) / len) * scale.
+hipError_t launch_reduce_q8_mean(const void* x, float* y, int64_t outer, int64_t len, int64_t inner,
+                                 float scale, int zp, hipStream_t stream);
+hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
+                          int64_t len, int64_t inner, bool log_softmax, hipStream_t stream);
+// y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last `len` elements.
+hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int64_t len,
+                            const float* gamma, const float* beta, float eps,
+                            hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// Data movement.
+// Generic strided copy: y (contiguous, `rank` dims) <- x with element strides.
+struct StridedCopyParams {
+  const void* x = nullptr; void* y = nullptr;
+  int elem_size = 4;
+  int rank = 1;
+  int64_t dims[8] = {1, 1, 1, 1, 1, 1, 1, 1};
+  int64_t sx[8] = {0};      // source strides (elements)
+  int64_t sy[8] = {0};      // destination strides (elements)
+  int64_t x_off = 0, y_off = 0;  // element offsets
+};
+hipError_t launch_strided_copy(const StridedCopyParams& p, hipStream_t stream);
+// Nearest-neighbour resize, channels-last: src index = floor(dst * in / out).
+hipError_t launch_resize_nearest_nhwc(const void* x, void* y, int elem_size, int N, int H,
+                                      int W, int cs, int Ho, int Wo, hipStream_t stream);
+// Row gather: y[o][j][:] = x[o][idx[j]][:], rows of row_bytes bytes.
+hipError_t launch_gather_rows(const void* x, const void* idx, DType idx_dt, void* y,
+                              int64_t outer, int64_t n_src_rows, int64_t n_idx,
+                              int64_t row_bytes, hipStream_t stream);
+hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// Batched NMS.  boxes [N][B][4] fp32 corners, scores [N][C][B] fp32.
+// out int32 [N][max_out][3] = {image, class, box}, -1 padded.
+// workspace: at least nms_workspace_bytes(N, B) bytes of device memory.
+size_t nms_workspace_bytes(int N, int B);
+hipError_t launch_nms(const float* boxes, const float* scores, int N, int C, int B,
+                      int max_out, float iou_thr, float score_thr, int32_t* out,
+                      void* workspace, hipStream_t stream);
+
+}  // namespace ohip
+#endif

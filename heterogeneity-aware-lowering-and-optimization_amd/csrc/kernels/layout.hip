@@ -1,0 +1,311 @@
+// Data-movement kernels for gfx950: N,C,HW <-> channels-last conversion with
+// type conversion (LDS-tiled so both sides stay coalesced), generic strided
+// copy (transpose / concat / slice), nearest resize and row gather.
+#include "device_utils.h"
+
+namespace ohip {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int TC = 32;   // channels per tile
+constexpr int THW = 64;  // positions per tile
+
+template <typename T> __device__ __forceinline__ float ld_as_float(const T* p, float, int) {
+  return Store<T>::ld(p);
+}
+// dequantise a stored 8-bit level
+template <> __device__ __forceinline__ float ld_as_float<int8_t>(const int8_t* p, float scale, int zp) {
+  return (float)(q_from_stored(*p) - zp) * scale;
+}
+template <typename T> __device__ __forceinline__ void st_from_float(T* p, float v, float, int) {
+  Store<T>::st(p, v);
+}
+// quantise to a stored 8-bit level: q = clamp(rne(v / scale) + zp, 0, 255)
+template <> __device__ __forceinline__ void st_from_float<int8_t>(int8_t* p, float v, float scale, int zp) {
+  float t = rintf(v / scale) + (float)zp;
+  t = fminf(fmaxf(t, 0.f), 255.f);
+  *p = q_to_stored((int)t);
+}
+
+// src [N][C][HW] -> dst [N][HW][cs]; channels C..cs-1 are written as `fill`.
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads) nchw_to_nhwc_tiled(LayoutParams p, float fill) {
+  __shared__ float tile[TC][THW + 1];
+  const TS* src = reinterpret_cast<const TS*>(p.src);
+  TD* dst = reinterpret_cast<TD*>(p.dst);
+  const int tiles_hw = (p.HW + THW - 1) / THW;
+  const int tiles_c = (p.cs + TC - 1) / TC;
+  const int64_t ntiles = (int64_t)p.N * tiles_hw * tiles_c;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int tc = (int)(t % tiles_c);
+    const int thw = (int)((t / tiles_c) % tiles_hw);
+    const int n = (int)(t / ((int64_t)tiles_c * tiles_hw));
+    const int c0 = tc * TC, hw0 = thw * THW;
+    {
+      const int tx = threadIdx.x % THW, ty = threadIdx.x / THW;
+      for (int cc = ty; cc < TC; cc += kThreads / THW) {
+        const int c = c0 + cc, hw = hw0 + tx;
+        float v = fill;
+        if (c < p.C && hw < p.HW) v = ld_as_float<TS>(src + ((int64_t)n * p.C + c) * p.HW + hw, p.scale, p.zp);
+        tile[cc][tx] = v;
+      }
+    }
+    __syncthreads();
+    {
+      const int tx = threadIdx.x % TC, ty = threadIdx.x / TC;
+      for (int hh = ty; hh < THW; hh += kThreads / TC) {
+        const int c = c0 + tx, hw = hw0 + hh;
+        if (c < p.cs && hw < p.HW)
+          st_from_float<TD>(dst + ((int64_t)n * p.HW + hw) * p.cs + c, tile[tx][hh], p.scale, p.zp);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Few channels (cs <= 16): one thread per pixel, channel planes read
+// coalesced across the wavefront, one contiguous pixel written per thread.
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads) nchw_to_nhwc_smallc(LayoutParams p, float fill) {
+  const TS* src = reinterpret_cast<const TS*>(p.src);
+  TD* dst = reinterpret_cast<TD*>(p.dst);
+  const int64_t total = (int64_t)p.N * p.HW;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t n = i / p.HW, hw = i - n * p.HW;
+    TD out[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      if (c < p.cs) {
+        float v = fill;
+        if (c < p.C) v = ld_as_float<TS>(src + (n * p.C + c) * p.HW + hw, p.scale, p.zp);
+        st_from_float<TD>(&out[c], v, p.scale, p.zp);
+      }
+    }
+    TD* o = dst + i * p.cs;
+    if ((p.cs * sizeof(TD)) % 16 == 0) {
+      const int nv = p.cs * (int)sizeof(TD) / 16;
+      for (int v = 0; v < nv; ++v)
+        reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
+    } else {
+      for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+    }
+  }
+}
+
+// src [N][HW][cs] -> dst [N][C][HW]
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads) nhwc_to_nchw_tiled(LayoutParams p) {
+  __shared__ float tile[TC][THW + 1];
+  const TS* src = reinterpret_cast<const TS*>(p.src);
+  TD* dst = reinterpret_cast<TD*>(p.dst);
+  const int tiles_hw = (p.HW + THW - 1) / THW;
+  const int tiles_c = (p.C + TC - 1) / TC;
+  const int64_t ntiles = (int64_t)p.N * tiles_hw * tiles_c;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int tc = (int)(t % tiles_c);
+    const int thw = (int)((t / tiles_c) % tiles_hw);
+    const int n = (int)(t / ((int64_t)tiles_c * tiles_hw));
+    const int c0 = tc * TC, hw0 = thw * THW;
+    {
+      const int tx = threadIdx.x % TC, ty = threadIdx.x / TC;
+      for (int hh = ty; hh < THW; hh += kThreads / TC) {
+        const int c = c0 + tx, hw = hw0 + hh;
+        float v = 0.f;
+        if (c < p.C && hw < p.HW) v = ld_as_float<TS>(src + ((int64_t)n * p.HW + hw) * p.cs + c, p.scale, p.zp);
+        tile[tx][hh] = v;
+      }
+    }
+    __syncthreads();
+    {
+      const int tx = threadIdx.x % THW, ty = threadIdx.x / THW;
+      for (int cc = ty; cc < TC; cc += kThreads / THW) {
+        const int c = c0 + cc, hw = hw0 + tx;
+        if (c < p.C && hw < p.HW)
+          st_from_float<TD>(dst + ((int64_t)n * p.C + c) * p.HW + hw, tile[cc][tx], p.scale, p.zp);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Generic strided copy of `ES`-byte elements; the innermost dim is walked by
+// consecutive threads.
+template <typename E>
+__global__ void __launch_bounds__(kThreads) strided_copy_kernel(StridedCopyParams p, int64_t n) {
+  const E* x = reinterpret_cast<const E*>(p.x) + p.x_off;
+  E* y = reinterpret_cast<E*>(p.y) + p.y_off;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    int64_t rem = i, ox = 0, oy = 0;
+#pragma unroll
+    for (int d = 7; d >= 0; --d) {
+      if (d < p.rank) {
+        const int64_t q = rem / p.dims[d];
+        const int64_t idx = rem - q * p.dims[d];
+        rem = q;
+        ox += idx * p.sx[d];
+        oy += idx * p.sy[d];
+      }
+    }
+    y[oy] = x[ox];
+  }
+}
+
+template <typename E>
+__global__ void __launch_bounds__(kThreads)
+resize_nearest_kernel(const E* __restrict__ x, E* __restrict__ y, int N, int H, int W, int cv,
+                      int Ho, int Wo) {
+  const int64_t total = (int64_t)N * Ho * Wo * cv;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(i % cv);
+    int64_t t = i / cv;
+    const int wo = (int)(t % Wo); t /= Wo;
+    const int ho = (int)(t % Ho);
+    const int n = (int)(t / Ho);
+    const int hi = (int)(((int64_t)ho * H) / Ho), wi = (int)(((int64_t)wo * W) / Wo);
+    y[i] = x[(((int64_t)n * H + hi) * W + wi) * cv + c];
+  }
+}
+
+template <typename IDX>
+__global__ void __launch_bounds__(kThreads)
+gather_rows_kernel(const unsigned char* __restrict__ x, const IDX* __restrict__ idx,
+                   unsigned char* __restrict__ y, int64_t outer, int64_t n_src, int64_t n_idx,
+                   int64_t row_bytes, int vec) {
+  // vec = bytes moved per thread step (16, 4, 2 or 1; row_bytes % vec == 0)
+  const int64_t per_row = row_bytes / vec;
+  const int64_t total = outer * n_idx * per_row;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t v = i % per_row;
+    const int64_t rj = i / per_row;
+    const int64_t j = rj % n_idx, o = rj / n_idx;
+    int64_t s = (int64_t)idx[j];
+    if (s < 0) s += n_src;
+    s = s < 0 ? 0 : (s >= n_src ? n_src - 1 : s);  // clamp: never read outside the table
+    const unsigned char* src = x + (o * n_src + s) * row_bytes + v * vec;
+    unsigned char* dst = y + rj * row_bytes + v * vec;
+    if (vec == 16) *reinterpret_cast<uintx4*>(dst) = *reinterpret_cast<const uintx4*>(src);
+    else if (vec == 4) *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src);
+    else if (vec == 2) *reinterpret_cast<uint16_t*>(dst) = *reinterpret_cast<const uint16_t*>(src);
+    else *dst = *src;
+  }
+}
+
+struct b16 { uintx4 v; };
+
+}  // namespace
+
+#define LAYOUT_PAIR_DISPATCH(KERNEL, ...)                                                      \
+  do {                                                                                         \
+    if (p.src_dt == DT_F32 && p.dst_dt == DT_F32) { KERNEL(float, float, __VA_ARGS__); }       \
+    else if (p.src_dt == DT_F32 && p.dst_dt == DT_F16) { KERNEL(float, f16_t, __VA_ARGS__); }  \
+    else if (p.src_dt == DT_F32 && p.dst_dt == DT_BF16) { KERNEL(float, bf16_t, __VA_ARGS__); }\
+    else if (p.src_dt == DT_F16 && p.dst_dt == DT_F32) { KERNEL(f16_t, float, __VA_ARGS__); }  \
+    else if (p.src_dt == DT_BF16 && p.dst_dt == DT_F32) { KERNEL(bf16_t, float, __VA_ARGS__); }\
+    else if (p.src_dt == DT_F16 && p.dst_dt == DT_F16) { KERNEL(f16_t, f16_t, __VA_ARGS__); }  \
+    else if (p.src_dt == DT_BF16 && p.dst_dt == DT_BF16) { KERNEL(bf16_t, bf16_t, __VA_ARGS__); }\
+    else if (p.src_dt == DT_F32 && p.dst_dt == DT_I8) { KERNEL(float, int8_t, __VA_ARGS__); }  \
+    else if (p.src_dt == DT_I8 && p.dst_dt == DT_F32) { KERNEL(int8_t, float, __VA_ARGS__); }  \
+    else return hipErrorInvalidValue;                                                          \
+  } while (0)
+
+static bool layout_ok(const LayoutParams& p) {
+  return p.src && p.dst && p.N > 0 && p.C > 0 && p.HW > 0 && p.cs >= p.C;
+}
+
+hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream) {
+  if (!layout_ok(p)) return hipErrorInvalidValue;
+  // padding lanes hold the real value 0 (its quantised level for 8-bit data)
+  const float fill = 0.f;
+  if (p.cs <= 16) {
+    const int grid = grid_for((int64_t)p.N * p.HW, kThreads);
+#define K1(TS, TD, ...) hipLaunchKernelGGL((nchw_to_nhwc_smallc<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p, fill)
+    LAYOUT_PAIR_DISPATCH(K1, 0);
+#undef K1
+  } else {
+    const int64_t ntiles = (int64_t)p.N * ((p.HW + THW - 1) / THW) * ((p.cs + TC - 1) / TC);
+    const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
+#define K2(TS, TD, ...) hipLaunchKernelGGL((nchw_to_nhwc_tiled<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p, fill)
+    LAYOUT_PAIR_DISPATCH(K2, 0);
+#undef K2
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_nhwc_to_nchw(const LayoutParams& p, hipStream_t stream) {
+  if (!layout_ok(p)) return hipErrorInvalidValue;
+  const int64_t ntiles = (int64_t)p.N * ((p.HW + THW - 1) / THW) * ((p.C + TC - 1) / TC);
+  const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
+#define K3(TS, TD, ...) hipLaunchKernelGGL((nhwc_to_nchw_tiled<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p)
+  LAYOUT_PAIR_DISPATCH(K3, 0);
+#undef K3
+  return hipGetLastError();
+}
+
+hipError_t launch_strided_copy(const StridedCopyParams& p, hipStream_t stream) {
+  if (!p.x || !p.y || p.rank < 1 || p.rank > 8) return hipErrorInvalidValue;
+  int64_t n = 1;
+  for (int d = 0; d < p.rank; ++d) {
+    if (p.dims[d] <= 0) return hipErrorInvalidValue;
+    n *= p.dims[d];
+  }
+  const int grid = grid_for(n, kThreads * 2);
+  switch (p.elem_size) {
+    case 1: hipLaunchKernelGGL(strided_copy_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    case 2: hipLaunchKernelGGL(strided_copy_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    case 4: hipLaunchKernelGGL(strided_copy_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    case 8: hipLaunchKernelGGL(strided_copy_kernel<uint64_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    case 16: hipLaunchKernelGGL(strided_copy_kernel<b16>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_resize_nearest_nhwc(const void* x, void* y, int elem_size, int N, int H, int W,
+                                      int cs, int Ho, int Wo, hipStream_t stream) {
+  if (!x || !y || N <= 0 || H <= 0 || W <= 0 || cs <= 0 || Ho <= 0 || Wo <= 0) return hipErrorInvalidValue;
+  const int64_t row_bytes = (int64_t)cs * elem_size;
+  const bool v16 = row_bytes % 16 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+  if (v16) {
+    const int cv = (int)(row_bytes / 16);
+    const int grid = grid_for((int64_t)N * Ho * Wo * cv, kThreads * 2);
+    hipLaunchKernelGGL(resize_nearest_kernel<b16>, dim3(grid), dim3(kThreads), 0, stream,
+                       (const b16*)x, (b16*)y, N, H, W, cv, Ho, Wo);
+  } else {
+    const int grid = grid_for((int64_t)N * Ho * Wo * cs, kThreads * 2);
+    switch (elem_size) {
+      case 1: hipLaunchKernelGGL(resize_nearest_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, (const uint8_t*)x, (uint8_t*)y, N, H, W, cs, Ho, Wo); break;
+      case 2: hipLaunchKernelGGL(resize_nearest_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, (const uint16_t*)x, (uint16_t*)y, N, H, W, cs, Ho, Wo); break;
+      case 4: hipLaunchKernelGGL(resize_nearest_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, (const uint32_t*)x, (uint32_t*)y, N, H, W, cs, Ho, Wo); break;
+      default: return hipErrorInvalidValue;
+    }
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gather_rows(const void* x, const void* idx, DType idx_dt, void* y, int64_t outer,
+                              int64_t n_src_rows, int64_t n_idx, int64_t row_bytes,
+                              hipStream_t stream) {
+  if (!x || !idx || !y || outer <= 0 || n_src_rows <= 0 || n_idx <= 0 || row_bytes <= 0)
+    return hipErrorInvalidValue;
+  const uintptr_t al = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | (uintptr_t)row_bytes;
+  const int vec = (al % 16 == 0) ? 16 : (al % 4 == 0) ? 4 : (al % 2 == 0) ? 2 : 1;
+  const int64_t total = outer * n_idx * (row_bytes / vec);
+  const int grid = grid_for(total, kThreads * 2);
+  if (idx_dt == DT_I32)
+    hipLaunchKernelGGL(gather_rows_kernel<int32_t>, dim3(grid), dim3(kThreads), 0, stream,
+                       (const unsigned char*)x, (const int32_t*)idx, (unsigned char*)y, outer,
+                       n_src_rows, n_idx, row_bytes, vec);
+  else if (idx_dt == DT_I64)
+    hipLaunchKernelGGL(gather_rows_kernel<int64_t>, dim3(grid), dim3(kThreads), 0, stream,
+                       (const unsigned char*)x, (const int64_t*)idx, (unsigned char*)y, outer,
+                       n_src_rows, n_idx, row_bytes, vec);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+}  // namespace ohip

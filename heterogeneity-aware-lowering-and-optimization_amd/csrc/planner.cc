@@ -1,0 +1,1952 @@
+// Graph -> plan compiler of libodla_hip.so.
+//
+// build_plan() walks the recorded nodes once and lowers them to kernel launch
+// steps over physical device tensors:
+//   * storage type: FLOAT32 graph values are kept as fp32, or as fp16 / bf16
+//     when ODLA_FP16_MODE / ODLA_BF16_MODE is set (fp32 accumulate in every
+//     kernel); in the int8 plan values with a quant-table entry are kept as
+//     8-bit levels;
+//   * layout: rank-4 values flowing through Conv / Pool / Resize live
+//     channels-last on the device, everything else row-major; conversions are
+//     inserted where a consumer needs the other form and cached per value;
+//   * fusion: per-channel Add / Mul / BatchNorm after a Conv or Gemm fold into
+//     its weights and bias, a same-shape residual Add and a trailing activation
+//     fold into its epilogue;
+//   * memory: constants are packed once into one device pool; temporaries get
+//     offsets in one arena by liveness (first fit over step intervals).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "internal.h"
+
+namespace ohip {
+namespace {
+
+constexpr size_t kAlign = 256;
+constexpr int kUnset = 1 << 30;  // PTensor::def_step before any step touched the tensor
+size_t align_up(size_t v, size_t a = kAlign) { return (v + a - 1) / a * a; }
+int round_up_i(int v, int a) { return (v + a - 1) / a * a; }
+
+float half_bits_to_float(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1f, man = h & 0x3ffu, u;
+  if (exp == 0) {
+    if (man == 0) u = sign;
+    else {
+      exp = 127 - 15 + 1;
+      while ((man & 0x400u) == 0) { man <<= 1; --exp; }
+      man &= 0x3ffu;
+      u = sign | (exp << 23) | (man << 13);
+    }
+  } else if (exp == 31) u = sign | 0x7f800000u | (man << 13);
+  else u = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+struct PlanError {
+  odla_status status;
+  std::string msg;
+};
+[[noreturn]] void fail(odla_status st, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  throw PlanError{st, buf};
+}
+
+enum Form { FORM_FLOAT = 0, FORM_QUANT = 1 };
+
+struct VState {
+  int slot[2][2] = {{-1, -1}, {-1, -1}};  // [layout][form] -> tensor id
+  int main = -1;
+};
+
+// Epilogue collected while fusing followers into a Conv / Gemm.
+struct Epilogue {
+  std::vector<float> row_scale;  // per output channel multiplier folded into weights
+  std::vector<float> bias;       // per output channel
+  bool has_bias = false;
+  _odla_value* residual = nullptr;
+  ActKind act = ACT_NONE;
+  float act_a = 0.f, act_b = 0.f;
+  _odla_value* pre_residual_value = nullptr;  // value right before the residual Add
+  _odla_value* final_value = nullptr;
+};
+
+class Planner {
+ public:
+  Planner(_odla_computation* c, Plan* p) : comp_(c), plan_(p) {}
+  void run();
+
+ private:
+  _odla_computation* comp_;
+  Plan* plan_;
+  std::vector<VState> vs_;
+  std::vector<std::vector<int>> consumers_;  // value index -> node indices
+  std::unordered_map<std::string, QuantEntry> qmap_;
+  DType cdt_ = DT_F32;
+  bool in_init_ = false;
+
+  // ---------------------------------------------------------------- tensors
+  int new_tensor(DType dt, Layout layout, const Shape& shape, int cs, Space space) {
+    PTensor t;
+    t.dt = dt;
+    t.layout = layout;
+    t.shape = shape;
+    t.cs = cs;
+    t.space = space;
+    t.bytes = (size_t)t.phys_elems() * dtype_size(dt);
+    t.def_step = kUnset;
+    t.last_step = -1;
+    if (space == SP_CONST) { t.offset = plan_->const_bytes; plan_->const_bytes += align_up(t.bytes); }
+    if (space == SP_INIT) { t.offset = plan_->init_bytes; plan_->init_bytes += align_up(t.bytes); }
+    plan_->tensors.push_back(t);
+    return (int)plan_->tensors.size() - 1;
+  }
+  int raw_buffer(size_t bytes, Space space) {
+    Shape s;
+    s.rank = 1;
+    s.d[0] = (int64_t)bytes;
+    return new_tensor(DT_U8, L_ROWMAJOR, s, 0, space);
+  }
+  int alias_tensor(int src, const Shape& shape) {
+    PTensor t = plan_->tensors[src];
+    t.shape = shape;
+    t.layout = L_ROWMAJOR;
+    t.cs = 0;
+    t.alias_of = root(src);
+    plan_->tensors.push_back(t);
+    return (int)plan_->tensors.size() - 1;
+  }
+  int root(int t) const {
+    while (plan_->tensors[t].alias_of >= 0) t = plan_->tensors[t].alias_of;
+    return t;
+  }
+  PTensor& T(int t) { return plan_->tensors[t]; }
+
+  // pointer resolution inside steps
+  struct Ref {
+    const Plan* plan;
+    int t;
+    char* operator()(const ExecEnv& env) const {
+      int r = t;
+      while (plan->tensors[r].alias_of >= 0) r = plan->tensors[r].alias_of;
+      const PTensor& pt = plan->tensors[r];
+      return env.base[pt.space] + pt.offset;
+    }
+  };
+  Ref ref(int t) const { return Ref{plan_, t}; }
+
+  void emit(const std::string& name, std::initializer_list<int> reads, std::initializer_list<int> writes,
+            std::function<hipError_t(const ExecEnv&, hipStream_t)> fn) {
+    if (in_init_) {
+      plan_->init_steps.push_back({name, std::move(fn)});
+      return;
+    }
+    const int idx = (int)plan_->steps.size();
+    auto touch = [&](int t) {
+      if (t < 0) return;
+      PTensor& p = T(root(t));
+      if (p.space != SP_ARENA) return;
+      if (idx < p.def_step) p.def_step = idx;
+      if (idx > p.last_step) p.last_step = idx;
+    };
+    for (int t : reads) touch(t);
+    for (int t : writes) touch(t);
+    plan_->steps.push_back({name, std::move(fn)});
+  }
+
+  // -------------------------------------------------------------- constants
+  size_t add_blob(Space space, size_t offset, const void* src, size_t bytes, std::vector<uint8_t>* owned) {
+    Plan::Blob b;
+    b.space = space;
+    b.offset = offset;
+    b.bytes = bytes;
+    if (owned) { b.owned = std::move(*owned); b.src = nullptr; } else b.src = src;
+    plan_->blobs.push_back(std::move(b));
+    return offset;
+  }
+  // device tensor in the constant pool holding `bytes` of host data
+  int const_from_host(DType dt, const Shape& shape, const void* src, std::vector<uint8_t>* owned) {
+    const int t = new_tensor(dt, L_ROWMAJOR, shape, 0, SP_CONST);
+    add_blob(SP_CONST, T(t).offset, src, T(t).bytes, owned);
+    return t;
+  }
+  template <typename E>
+  int const_vector(DType dt, const std::vector<E>& v) {
+    Shape s;
+    s.rank = 1;
+    s.d[0] = (int64_t)v.size();
+    std::vector<uint8_t> raw(v.size() * sizeof(E));
+    memcpy(raw.data(), v.data(), raw.size());
+    return const_from_host(dt, s, nullptr, &raw);
+  }
+
+  std::vector<float> const_as_float(const _odla_value* v) {
+    if (v->kind != _odla_value::CONSTANT || v->host_data == nullptr) fail(ODLA_INVALID_PARAM, "value '%s' is not a constant", v->name.c_str());
+    const int64_t n = v->shape.numel();
+    std::vector<float> out((size_t)n);
+    switch (dtype_from_odla(v->etype)) {
+      case DT_F32: memcpy(out.data(), v->host_data, (size_t)n * 4); break;
+      case DT_F16: for (int64_t i = 0; i < n; ++i) out[i] = half_bits_to_float(((const uint16_t*)v->host_data)[i]); break;
+      case DT_BF16: for (int64_t i = 0; i < n; ++i) { uint32_t u = (uint32_t)((const uint16_t*)v->host_data)[i] << 16; memcpy(&out[i], &u, 4); } break;
+      case DT_I32: for (int64_t i = 0; i < n; ++i) out[i] = (float)((const int32_t*)v->host_data)[i]; break;
+      case DT_I64: for (int64_t i = 0; i < n; ++i) out[i] = (float)((const int64_t*)v->host_data)[i]; break;
+      case DT_I8: for (int64_t i = 0; i < n; ++i) out[i] = (float)((const int8_t*)v->host_data)[i]; break;
+      case DT_U8: for (int64_t i = 0; i < n; ++i) out[i] = (float)((const uint8_t*)v->host_data)[i]; break;
+      default: fail(ODLA_UNSUPPORTED_DATATYPE, "constant '%s' has an unsupported element type", v->name.c_str());
+    }
+    return out;
+  }
+
+  // ------------------------------------------------------------- dtype rules
+  DType storage_dtype(const _odla_value* v) const {
+    const DType d = dtype_from_odla(v->etype);
+    if (d == DT_F32) return cdt_;
+    return d;
+  }
+  const QuantEntry* qentry(const _odla_value* v) const {
+    if (!comp_->opts.int8 || v == nullptr || v->name.empty()) return nullptr;
+    if (dtype_from_odla(v->etype) != DT_F32) return nullptr;
+    auto it = qmap_.find(v->name);
+    return it == qmap_.end() ? nullptr : &it->second;
+  }
+
+  // --------------------------------------------------- value -> device tensor
+  // Returns a tensor holding `v` in the requested layout and form, inserting
+  // (and caching) a conversion step when the value lives in another one.
+  // `cvec` > 0 asks for a channels-last pitch that is a multiple of cvec.
+  int get(const _odla_value* v, Layout want, Form form = FORM_FLOAT, int cvec = 0) {
+    VState& s = vs_[v->index];
+    if (s.main < 0) materialize_source(v);
+    if (want == L_NHWC && v->shape.rank != 4) fail(ODLA_INTERNAL_LOGIC_ERR, "channels-last form requested for rank-%d value", v->shape.rank);
+    int& slot = s.slot[want][form];
+    if (slot >= 0 && (want != L_NHWC || cvec <= 1 || T(slot).cs % cvec == 0)) return slot;
+    const int have = pick_source(s, want, form);
+    const int made = convert(v, have, want, form, cvec);
+    slot = made;
+    return made;
+  }
+
+  int pick_source(const VState& s, Layout want, Form form) const {
+    // prefer same form, then same layout, then main
+    if (s.slot[want][form] >= 0) return s.slot[want][form];
+    if (s.slot[1 - want][form] >= 0) return s.slot[1 - want][form];
+    if (s.slot[want][1 - form] >= 0) return s.slot[want][1 - form];
+    return s.main;
+  }
+
+  void set_main(const _odla_value* v, int t) {
+    VState& s = vs_[v->index];
+    s.main = t;
+    const PTensor p = T(t);  // by value: the tensor table may grow below
+    s.slot[p.layout][p.quant ? FORM_QUANT : FORM_FLOAT] = t;
+    // a channels-last tensor with one pixel (or one channel) and no padding is
+    // also a valid row-major tensor, and vice versa
+    if (p.shape.rank == 4) {
+      const bool trivial = (p.shape.d[2] * p.shape.d[3] == 1) || (p.shape.d[1] == 1);
+      if (trivial && (p.layout == L_ROWMAJOR || p.cs == p.shape.d[1])) {
+        const int other = 1 - (int)p.layout;
+        if (s.slot[other][p.quant ? FORM_QUANT : FORM_FLOAT] < 0) {
+          PTensor a = p;
+          a.alias_of = root(t);
+          a.layout = (Layout)other;
+          a.cs = other == L_NHWC ? (int)p.shape.d[1] : 0;
+          plan_->tensors.push_back(a);
+          s.slot[other][p.quant ? FORM_QUANT : FORM_FLOAT] = (int)plan_->tensors.size() - 1;
+        }
+      }
+    }
+  }
+
+  // Arguments and constants enter the plan in their declared type, row-major.
+  void materialize_source(const _odla_value* v) {
+    if (v->kind == _odla_value::ARG) {
+      fail(ODLA_INTERNAL_LOGIC_ERR, "argument '%s' was not staged", v->name.c_str());
+    } else if (v->kind == _odla_value::CONSTANT) {
+      const DType src = dtype_from_odla(v->etype);
+      const DType dst = storage_dtype(v);
+      int t;
+      if (src == dst) {
+        t = const_from_host(src, v->shape, v->host_data, nullptr);
+      } else {
+        const int raw = new_tensor(src, L_ROWMAJOR, v->shape, 0, SP_INIT);
+        add_blob(SP_INIT, T(raw).offset, v->host_data, T(raw).bytes, nullptr);
+        t = new_tensor(dst, L_ROWMAJOR, v->shape, 0, SP_CONST);
+        const int64_t n = v->shape.numel();
+        const Ref a = ref(raw), b = ref(t);
+        const bool was_init = in_init_;
+        in_init_ = true;
+        emit("const.cast", {}, {}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), src, b(e), dst, n, st); });
+        in_init_ = was_init;
+      }
+      set_main(v, t);
+    } else {
+      fail(ODLA_INTERNAL_LOGIC_ERR, "value '%s' is used before it is produced", v->name.c_str());
+    }
+  }
+
+  int convert(const _odla_value* v, int have, Layout want, Form form, int cvec) {
+    const PTensor src = T(have);
+    const QuantEntry* q = qentry(v);
+    const bool src_q = src.quant;
+    const bool dst_q = form == FORM_QUANT;
+    if (dst_q && q == nullptr && !src_q) fail(ODLA_INTERNAL_LOGIC_ERR, "quantised form of '%s' requested without a table entry", v->name.c_str());
+    const float scale = src_q ? src.qscale : (q ? q->scale : 1.f);
+    const int zp = src_q ? src.qzp : (q ? q->zp : 0);
+    const DType fdt = dst_q ? DT_I8 : storage_dtype(v);
+    const Space space = SP_ARENA;
+    const Shape& sh = v->shape;
+
+    // Layout change (with optional type / form change fused in) -----------
+    if (src.layout != want || (want == L_NHWC && cvec > 1 && src.cs % cvec != 0)) {
+      if (sh.rank != 4) fail(ODLA_INTERNAL_LOGIC_ERR, "layout conversion of a rank-%d value", sh.rank);
+      int from = have;
+      if (src.layout == L_NHWC && want == L_NHWC) {
+        // repitch: go through row-major
+        from = get(v, L_ROWMAJOR, src_q ? FORM_QUANT : FORM_FLOAT);
+      }
+      const PTensor s2 = T(from);
+      LayoutParams lp;
+      lp.N = (int)sh.d[0]; lp.C = (int)sh.d[1]; lp.HW = (int)(sh.d[2] * sh.d[3]);
+      lp.scale = scale; lp.zp = zp;
+      // the layout kernels convert between float types and to/from 8-bit levels
+      if (s2.quant && dst_q) {
+        // 8-bit to 8-bit relayout: byte-wise strided copy
+        return relayout_bytes(v, from, want, cvec);
+      }
+      lp.src_dt = s2.dt;
+      lp.dst_dt = fdt;
+      if (want == L_NHWC) {
+        const int cs = cvec > 1 ? round_up_i((int)sh.d[1], cvec) : (int)sh.d[1];
+        lp.cs = cs;
+        const int dst = new_tensor(fdt, L_NHWC, sh, cs, space);
+        set_quant(dst, dst_q, scale, zp);
+        const Ref a = ref(from), b = ref(dst);
+        emit("to_nhwc:" + v->name, {from}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+          LayoutParams p = lp; p.src = a(e); p.dst = b(e);
+          return launch_nchw_to_nhwc(p, st);
+        });
+        return dst;
+      } else {
+        lp.cs = s2.cs;
+        const int dst = new_tensor(fdt, L_ROWMAJOR, sh, 0, space);
+        set_quant(dst, dst_q, scale, zp);
+        const Ref a = ref(from), b = ref(dst);
+        emit("to_nchw:" + v->name, {from}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+          LayoutParams p = lp; p.src = a(e); p.dst = b(e);
+          return launch_nhwc_to_nchw(p, st);
+        });
+        return dst;
+      }
+    }
+    // Same layout, form change ----------------------------------------------
+    const int dst = new_tensor(fdt, src.layout, sh, src.cs, space);
+    set_quant(dst, dst_q, scale, zp);
+    const int64_t n = src.phys_elems();
+    const Ref a = ref(have), b = ref(dst);
+    if (src_q && !dst_q) {
+      const int sc = const_vector<float>(DT_F32, {scale});
+      const int zc = const_vector<int32_t>(DT_I32, {zp});
+      const Ref rs = ref(sc), rz = ref(zc);
+      const DType ddt = fdt;
+      emit("dequant:" + v->name, {have}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+        QuantParams p; p.src = a(e); p.dst = b(e); p.src_dt = DT_I8; p.dst_dt = ddt; p.n = n;
+        p.scale = (const float*)rs(e); p.zp = (const int32_t*)rz(e);
+        return launch_dequantize(p, st);
+      });
+    } else if (!src_q && dst_q) {
+      const int sc = const_vector<float>(DT_F32, {scale});
+      const int zc = const_vector<int32_t>(DT_I32, {zp});
+      const Ref rs = ref(sc), rz = ref(zc);
+      const DType sdt = src.dt;
+      emit("quant:" + v->name, {have}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+        QuantParams p; p.src = a(e); p.dst = b(e); p.src_dt = sdt; p.dst_dt = DT_I8; p.n = n;
+        p.scale = (const float*)rs(e); p.zp = (const int32_t*)rz(e);
+        return launch_quantize(p, st);
+      });
+    } else if (src.dt != fdt) {
+      const DType sdt = src.dt, ddt = fdt;
+      emit("cast:" + v->name, {have}, {dst}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), ddt, n, st); });
+    } else {
+      fail(ODLA_INTERNAL_LOGIC_ERR, "no conversion needed for '%s'", v->name.c_str());
+    }
+    return dst;
+  }
+
+  int relayout_bytes(const _odla_value* v, int from, Layout want, int cvec) {
+    const PTensor s = T(from);
+    const Shape& sh = v->shape;
+    const int64_t N = sh.d[0], C = sh.d[1], H = sh.d[2], W = sh.d[3];
+    const int cs = want == L_NHWC ? (cvec > 1 ? round_up_i((int)C, cvec) : (int)C) : 0;
+    if (want == L_NHWC && cs != C) fail(ODLA_UNSUPPORTED_OP, "8-bit relayout with channel padding is not supported ('%s')", v->name.c_str());
+    const int dst = new_tensor(s.dt, want, sh, cs, SP_ARENA);
+    set_quant(dst, s.quant, s.qscale, s.qzp);
+    StridedCopyParams cp;
+    cp.elem_size = dtype_size(s.dt);
+    cp.rank = 4;
+    if (want == L_NHWC) {  // iterate N,H,W,C over the destination
+      cp.dims[0] = N; cp.dims[1] = H; cp.dims[2] = W; cp.dims[3] = C;
+      cp.sy[0] = H * W * cs; cp.sy[1] = W * cs; cp.sy[2] = cs; cp.sy[3] = 1;
+      cp.sx[0] = C * H * W; cp.sx[1] = W; cp.sx[2] = 1; cp.sx[3] = H * W;
+    } else {  // iterate N,C,H,W over the destination
+      cp.dims[0] = N; cp.dims[1] = C; cp.dims[2] = H; cp.dims[3] = W;
+      cp.sy[0] = C * H * W; cp.sy[1] = H * W; cp.sy[2] = W; cp.sy[3] = 1;
+      cp.sx[0] = H * W * s.cs; cp.sx[1] = 1; cp.sx[2] = W * s.cs; cp.sx[3] = s.cs;
+    }
+    const Ref a = ref(from), b = ref(dst);
+    emit("relayout:" + v->name, {from}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+      StridedCopyParams p = cp; p.x = a(e); p.y = b(e);
+      return launch_strided_copy(p, st);
+    });
+    return dst;
+  }
+
+  void set_quant(int t, bool q, float scale, int zp) {
+    T(t).quant = q;
+    T(t).qscale = q ? scale : 1.f;
+    T(t).qzp = q ? zp : 0;
+  }
+
+  // New output tensor of a node in float storage.
+  int out_tensor(const _odla_value* v, Layout layout, int cs = 0, DType dt = DT_INVALID) {
+    if (dt == DT_INVALID) dt = storage_dtype(v);
+    if (layout == L_NHWC && cs == 0) cs = (int)v->shape.d[1];
+    return new_tensor(dt, layout, v->shape, cs, SP_ARENA);
+  }
+
+  int use_count(const _odla_value* v) const { return (int)consumers_[v->index].size() + (v->is_output ? 1 : 0); }
+  bool available(const _odla_value* v) const {
+    return v->kind != _odla_value::TEMP || vs_[v->index].main >= 0;
+  }
+
+  // ------------------------------------------------------------------ nodes
+  void lower(int ni);
+  void lower_conv(int ni);
+  void lower_gemm(int ni);
+  void lower_binary(int ni);
+  void lower_unary(int ni);
+  void lower_batchnorm(int ni);
+  void lower_layernorm(int ni);
+  void lower_pool(int ni);
+  void lower_reduce(int ni);
+  void lower_softmax(int ni);
+  void lower_cast(int ni);
+  void lower_concat(int ni);
+  void lower_gather(int ni);
+  void lower_reshape(int ni);
+  void lower_resize(int ni);
+  void lower_slice(int ni);
+  void lower_transpose(int ni);
+  void lower_qdq(int ni);
+  void lower_nms(int ni);
+
+  void collect_epilogue(int ni, int64_t out_channels, int channel_axis_of_output, Epilogue* ep);
+  bool per_channel_constant(const _odla_value* k, const Shape& aligned, const Shape& out, int ch_axis,
+                            int64_t channels, std::vector<float>* vals);
+  void bn_params_host(const Node& n, int64_t C, std::vector<float>* scale, std::vector<float>* shift);
+  int pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og, int Cg, int R, int S, int Cp,
+                   int64_t so, int64_t si, int64_t sr, int64_t ss, const std::vector<float>& row_scale,
+                   int* w_rs_out, const std::vector<float>* wq_scale);
+  void finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty, const Epilogue& ep,
+                    int64_t Kout_total);
+  int strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp);
+  void assign_arena();
+  void parse_quant_table();
+};
+
+// ============================================================================
+
+void Planner::parse_quant_table() {
+  const Options& o = comp_->opts;
+  if (!o.int8) return;
+  if (o.qtable == nullptr || o.qtable_size <= 0) fail(ODLA_INVALID_PARAM, "int8 data type selected but no ODLA_QUANT_TABLE / ODLA_QUANT_TABLE_SIZE was set");
+  QuantEntry* cur = nullptr;
+  for (int i = 0; i < o.qtable_size; ++i) {
+    const odla_value_quant_info& r = o.qtable[i];
+    if (r.value_id == nullptr) continue;
+    const std::string name(reinterpret_cast<const char*>(r.value_id));
+    if (r.ch_idx < 0) {
+      QuantEntry& e = qmap_[name];
+      e.scale = r.scale;
+      e.zp = (int)std::lrintf(r.offset);
+      e.min = r.min;
+      e.max = r.max;
+      e.ch_min.assign((size_t)(-r.ch_idx), 0.f);
+      e.ch_max.assign((size_t)(-r.ch_idx), 0.f);
+      cur = &e;
+      if (!(e.scale > 0.f) || e.zp < 0 || e.zp > 255) fail(ODLA_INVALID_PARAM, "quant table entry '%s' has scale %g / zero point %d", name.c_str(), e.scale, e.zp);
+    } else {
+      auto it = qmap_.find(name);
+      QuantEntry* e = it != qmap_.end() ? &it->second : cur;
+      if (e == nullptr || (size_t)r.ch_idx >= e->ch_min.size()) fail(ODLA_INVALID_PARAM, "quant table channel record %d of '%s' has no tensor record", r.ch_idx, name.c_str());
+      e->ch_min[r.ch_idx] = r.min;
+      e->ch_max[r.ch_idx] = r.max;
+    }
+  }
+}
+
+void Planner::run() {
+  const Options& o = comp_->opts;
+  if (o.fp16) cdt_ = DT_F16;
+  else if (o.bf16 != BF16_DISABLE) cdt_ = DT_BF16;
+  parse_quant_table();
+
+  vs_.assign(comp_->values.size(), VState());
+  consumers_.assign(comp_->values.size(), {});
+  for (size_t ni = 0; ni < comp_->nodes.size(); ++ni)
+    for (_odla_value* v : comp_->nodes[ni].in)
+      if (v != nullptr) consumers_[v->index].push_back((int)ni);
+
+  // Arguments: one staging tensor each (declared type, row-major), alive from
+  // the start of the execution because the H2D copy precedes every step.
+  for (_odla_value* a : comp_->args) {
+    const DType d = dtype_from_odla(a->etype);
+    const int t = new_tensor(d, L_ROWMAJOR, a->shape, 0, SP_ARENA);
+    T(t).pinned = true;
+    T(t).def_step = -1;
+    Plan::IO io;
+    io.v = a;
+    io.tensor = t;
+    io.bytes = T(t).bytes;
+    plan_->inputs.push_back(io);
+    VState& s = vs_[a->index];
+    s.main = t;
+    if (d == storage_dtype(a)) {
+      set_main(a, t);
+    }
+    // otherwise no slot is filled: consumers convert from the staging tensor
+  }
+
+  for (size_t ni = 0; ni < comp_->nodes.size(); ++ni) {
+    if (comp_->nodes[ni].absorbed) continue;
+    lower((int)ni);
+  }
+
+  // Outputs: row-major, declared element type.
+  for (_odla_value* ov : comp_->outputs) {
+    const DType want = dtype_from_odla(ov->etype);
+    int t = get(ov, L_ROWMAJOR, FORM_FLOAT);
+    if (T(t).dt != want) {
+      const int dst = new_tensor(want, L_ROWMAJOR, ov->shape, 0, SP_ARENA);
+      const int64_t n = ov->shape.numel();
+      const DType sdt = T(t).dt;
+      const Ref a = ref(t), b = ref(dst);
+      emit("out.cast:" + ov->name, {t}, {dst}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), want, n, st); });
+      t = dst;
+    }
+    PTensor& p = T(root(t));
+    if (p.space == SP_ARENA) { p.pinned = true; p.last_step = 1 << 30; }
+    Plan::IO io;
+    io.v = ov;
+    io.tensor = root(t);
+    io.bytes = (size_t)ov->shape.numel() * dtype_size(want);
+    plan_->outputs.push_back(io);
+  }
+  assign_arena();
+}
+
+// Staged arguments whose declared type differs from the storage type have no
+// slot; pick_source() then falls back to `main` (the staging tensor).
+
+void Planner::assign_arena() {
+  struct Item { int t; int a, b; size_t bytes; size_t off; };
+  std::vector<Item> items;
+  for (size_t i = 0; i < plan_->tensors.size(); ++i) {
+    PTensor& p = plan_->tensors[i];
+    if (p.space != SP_ARENA || p.alias_of >= 0) continue;
+    int a = p.def_step, b = p.last_step;
+    if (a == kUnset) { a = 0; if (b < 0) b = 0; }  // never touched by a step: still give it room
+    if (b < a) b = a;
+    items.push_back({(int)i, a, b, align_up(p.bytes ? p.bytes : 1), 0});
+  }
+  std::sort(items.begin(), items.end(), [](const Item& x, const Item& y) {
+    if (x.a != y.a) return x.a < y.a;
+    return x.bytes > y.bytes;
+  });
+  std::vector<Item> placed;
+  size_t total = 0;
+  for (Item& it : items) {
+    std::vector<std::pair<size_t, size_t>> busy;
+    for (const Item& q : placed)
+      if (!(q.b < it.a || it.b < q.a)) busy.push_back({q.off, q.off + q.bytes});
+    std::sort(busy.begin(), busy.end());
+    size_t off = 0;
+    for (auto& r : busy) {
+      if (off + it.bytes <= r.first) break;
+      if (r.second > off) off = r.second;
+    }
+    it.off = off;
+    placed.push_back(it);
+    plan_->tensors[it.t].offset = off;
+    if (off + it.bytes > total) total = off + it.bytes;
+  }
+  plan_->arena_bytes = total;
+}
+
+void Planner::lower(int ni) {
+  const Node& n = comp_->nodes[ni];
+  switch (n.op) {
+    case OP_CONV: lower_conv(ni); break;
+    case OP_GEMM: lower_gemm(ni); break;
+    case OP_BINARY: lower_binary(ni); break;
+    case OP_UNARY: lower_unary(ni); break;
+    case OP_BATCHNORM: lower_batchnorm(ni); break;
+    case OP_LAYERNORM: lower_layernorm(ni); break;
+    case OP_POOL: lower_pool(ni); break;
+    case OP_REDUCE: lower_reduce(ni); break;
+    case OP_SOFTMAX: lower_softmax(ni); break;
+    case OP_CAST: lower_cast(ni); break;
+    case OP_CONCAT: lower_concat(ni); break;
+    case OP_GATHER: lower_gather(ni); break;
+    case OP_RESHAPE: lower_reshape(ni); break;
+    case OP_RESIZE: lower_resize(ni); break;
+    case OP_SLICE: lower_slice(ni); break;
+    case OP_TRANSPOSE: lower_transpose(ni); break;
+    case OP_QUANTIZE: case OP_DEQUANTIZE: lower_qdq(ni); break;
+    case OP_NMS: lower_nms(ni); break;
+  }
+}
+
+// ------------------------------------------------------------------ fusion --
+
+// Is `k` a constant that varies only along `ch_axis` of `out` (or is a scalar)?
+bool Planner::per_channel_constant(const _odla_value* k, const Shape& aligned, const Shape& out,
+                                   int ch_axis, int64_t channels, std::vector<float>* vals) {
+  if (k->kind != _odla_value::CONSTANT) return false;
+  const int64_t n = k->shape.numel();
+  if (n == 1) {
+    const float v = const_as_float(k)[0];
+    vals->assign((size_t)channels, v);
+    return true;
+  }
+  if (n != channels || aligned.rank != out.rank) return false;
+  for (int i = 0; i < aligned.rank; ++i) {
+    if (i == ch_axis) { if (aligned.d[i] != channels) return false; }
+    else if (aligned.d[i] != 1) return false;
+  }
+  *vals = const_as_float(k);
+  return true;
+}
+
+void Planner::bn_params_host(const Node& n, int64_t C, std::vector<float>* scale, std::vector<float>* shift) {
+  const std::vector<float> mean = const_as_float(n.in[1]), var = const_as_float(n.in[2]);
+  std::vector<float> g((size_t)C, n.f[1]), b((size_t)C, n.f[2]);
+  if (n.in[3]) g = const_as_float(n.in[3]);
+  if (n.in[4]) b = const_as_float(n.in[4]);
+  scale->resize((size_t)C);
+  shift->resize((size_t)C);
+  for (int64_t c = 0; c < C; ++c) {
+    const float m = g[c] / std::sqrt(var[c] + n.f[0]);
+    (*scale)[c] = m;
+    (*shift)[c] = b[c] - mean[c] * m;
+  }
+}
+
+// Walk the single-consumer chain behind node `ni` and fold what the igemm
+// epilogue can do.  `ch_axis` is the logical axis of the output that indexes
+// output channels.
+void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* ep) {
+  _odla_value* cur = comp_->nodes[ni].out;
+  ep->final_value = cur;
+  const bool q8 = comp_->opts.int8;
+  while (true) {
+    if (cur->is_output || consumers_[cur->index].size() != 1) break;
+    const int ci = consumers_[cur->index][0];
+    Node& nx = comp_->nodes[ci];
+    if (nx.absorbed) break;
+    bool took = false;
+    if (nx.op == OP_BATCHNORM && nx.in[0] == cur && ep->residual == nullptr && ep->act == ACT_NONE && !q8) {
+      const bool cf = nx.i[0] != ODLA_CHANNELS_LAST;
+      const int bn_axis = cf ? 1 : cur->shape.rank - 1;
+      bool all_const = nx.in[1]->kind == _odla_value::CONSTANT && nx.in[2]->kind == _odla_value::CONSTANT &&
+                       (!nx.in[3] || nx.in[3]->kind == _odla_value::CONSTANT) &&
+                       (!nx.in[4] || nx.in[4]->kind == _odla_value::CONSTANT);
+      if (all_const && bn_axis == ch_axis) {
+        std::vector<float> sc, sh;
+        bn_params_host(nx, channels, &sc, &sh);
+        if (ep->row_scale.empty()) ep->row_scale.assign((size_t)channels, 1.f);
+        if (ep->bias.empty()) ep->bias.assign((size_t)channels, 0.f);
+        for (int64_t c = 0; c < channels; ++c) {
+          ep->row_scale[c] *= sc[c];
+          ep->bias[c] = ep->bias[c] * sc[c] + sh[c];
+        }
+        ep->has_bias = true;
+        took = true;
+      }
+    } else if (nx.op == OP_BINARY && (nx.i[0] == BIN_ADD || nx.i[0] == BIN_MUL || nx.i[0] == BIN_SUB)) {
+      const bool cur_is_lhs = nx.in[0] == cur;
+      _odla_value* other = cur_is_lhs ? nx.in[1] : nx.in[0];
+      if (other != cur && nx.out->shape == cur->shape) {
+        // aligned operand shapes recorded by the builder
+        const int r = (int)nx.iv[0];
+        Shape al;
+        al.rank = r;
+        for (int i = 0; i < r; ++i) al.d[i] = nx.iv[1 + (cur_is_lhs ? r : 0) + i];
+        std::vector<float> vals;
+        if (ep->residual == nullptr && ep->act == ACT_NONE && !q8 &&
+            per_channel_constant(other, al, nx.out->shape, ch_axis, channels, &vals)) {
+          if (ep->bias.empty()) ep->bias.assign((size_t)channels, 0.f);
+          if (nx.i[0] == BIN_ADD) {
+            for (int64_t c = 0; c < channels; ++c) ep->bias[c] += vals[c];
+            ep->has_bias = true;
+            took = true;
+          } else if (nx.i[0] == BIN_SUB && cur_is_lhs) {
+            for (int64_t c = 0; c < channels; ++c) ep->bias[c] -= vals[c];
+            ep->has_bias = true;
+            took = true;
+          } else if (nx.i[0] == BIN_MUL) {
+            if (ep->row_scale.empty()) ep->row_scale.assign((size_t)channels, 1.f);
+            for (int64_t c = 0; c < channels; ++c) { ep->row_scale[c] *= vals[c]; ep->bias[c] *= vals[c]; }
+            took = true;
+          }
+        } else if (nx.i[0] == BIN_ADD && ep->residual == nullptr && ep->act == ACT_NONE &&
+                   other->kind != _odla_value::CONSTANT && other->shape == cur->shape && available(other) &&
+                   storage_dtype(other) == storage_dtype(cur)) {
+          bool ok = true;
+          if (q8) ok = qentry(cur) != nullptr && qentry(other) != nullptr;  // both sides must be 8-bit
+          if (ok) {
+            ep->residual = other;
+            ep->pre_residual_value = cur;
+            took = true;
+          }
+        }
+      }
+    } else if (nx.op == OP_UNARY && ep->act == ACT_NONE) {
+      const ActKind a = (ActKind)nx.i[0];
+      const bool fusable = q8 ? (a == ACT_RELU)
+                              : (a == ACT_RELU || a == ACT_LEAKY || a == ACT_CLAMP || a == ACT_SIGMOID ||
+                                 a == ACT_TANH || a == ACT_GELU_ERF || a == ACT_GELU_TANH);
+      if (fusable) {
+        ep->act = a;
+        ep->act_a = nx.f[0];
+        ep->act_b = nx.f[1];
+        took = true;
+      }
+    }
+    if (!took) break;
+    nx.absorbed = true;
+    cur = nx.out;
+    ep->final_value = cur;
+    if (ep->act != ACT_NONE) break;
+  }
+}
+
+// ------------------------------------------------------------------ weights --
+
+int Planner::pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og, int Cg, int R, int S,
+                          int Cp, int64_t so, int64_t si, int64_t sr, int64_t ss,
+                          const std::vector<float>& row_scale, int* w_rs_out,
+                          const std::vector<float>* wq_scale) {
+  const int es = dtype_size(dst_dt);
+  const int bk = 64 / es;
+  const int w_rs = round_up_i(R * S * Cp, bk);
+  *w_rs_out = w_rs;
+  Shape ws;
+  ws.rank = 3;
+  ws.d[0] = G; ws.d[1] = Og; ws.d[2] = w_rs;
+  PackWeightsParams pp;
+  pp.G = G; pp.Og = Og; pp.Cg = Cg; pp.R = R; pp.S = S; pp.Cp = Cp;
+  pp.rows_pad = Og; pp.w_rs = w_rs;
+  pp.so = so; pp.si = si; pp.sr = sr; pp.ss = ss;
+  pp.dst_dt = dst_dt;
+
+  if (kernel->kind == _odla_value::CONSTANT) {
+    const int64_t n = kernel->shape.numel();
+    const int dst = new_tensor(dst_dt, L_ROWMAJOR, ws, 0, SP_CONST);
+    int raw;
+    if (dst_dt == DT_I8) {
+      // symmetric per-output-channel quantisation on the host:
+      // q = clip(rne(w / s[o]), -127, 127)
+      std::vector<float> w = const_as_float(kernel);
+      std::vector<uint8_t> q((size_t)n);
+      const int64_t O = (int64_t)G * Og;
+      // element (o,i,r,s) at o*so + i*si + r*sr + s*ss
+      for (int64_t o = 0; o < O; ++o) {
+        const float s = (*wq_scale)[o];
+        for (int64_t i = 0; i < Cg; ++i)
+          for (int r = 0; r < R; ++r)
+            for (int t = 0; t < S; ++t) {
+              const int64_t idx = o * so + i * si + r * sr + t * ss;
+              float v = std::nearbyintf(w[idx] / s);
+              v = v < -127.f ? -127.f : (v > 127.f ? 127.f : v);
+              q[idx] = (uint8_t)(int8_t)(int)v;
+            }
+      }
+      raw = new_tensor(DT_I8, L_ROWMAJOR, kernel->shape, 0, SP_INIT);
+      add_blob(SP_INIT, T(raw).offset, nullptr, T(raw).bytes, &q);
+      pp.src_dt = DT_I8;
+    } else if (!row_scale.empty()) {
+      std::vector<float> w = const_as_float(kernel);
+      const int64_t O = (int64_t)G * Og;
+      for (int64_t o = 0; o < O; ++o)
+        for (int64_t i = 0; i < Cg; ++i)
+          for (int r = 0; r < R; ++r)
+            for (int t = 0; t < S; ++t) w[o * so + i * si + r * sr + t * ss] *= row_scale[o];
+      std::vector<uint8_t> bytes((size_t)n * 4);
+      memcpy(bytes.data(), w.data(), bytes.size());
+      raw = new_tensor(DT_F32, L_ROWMAJOR, kernel->shape, 0, SP_INIT);
+      add_blob(SP_INIT, T(raw).offset, nullptr, T(raw).bytes, &bytes);
+      pp.src_dt = DT_F32;
+    } else {
+      const DType sdt = dtype_from_odla(kernel->etype);
+      raw = new_tensor(sdt, L_ROWMAJOR, kernel->shape, 0, SP_INIT);
+      add_blob(SP_INIT, T(raw).offset, kernel->host_data, T(raw).bytes, nullptr);
+      pp.src_dt = sdt;
+    }
+    const Ref a = ref(raw), b = ref(dst);
+    const bool was_init = in_init_;
+    in_init_ = true;
+    emit("pack:" + kernel->name, {}, {}, [=](const ExecEnv& e, hipStream_t st) {
+      PackWeightsParams p = pp; p.src = a(e); p.dst = b(e);
+      return launch_pack_weights(p, st);
+    });
+    in_init_ = was_init;
+    return dst;
+  }
+  // run-time kernel (argument or computed value): repack on every execution
+  if (dst_dt == DT_I8) fail(ODLA_UNSUPPORTED_OP, "int8 convolution needs a constant kernel ('%s')", kernel->name.c_str());
+  if (!row_scale.empty()) fail(ODLA_INTERNAL_LOGIC_ERR, "cannot fold a scale into a run-time kernel");
+  const VState& s = vs_[kernel->index];
+  if (s.main < 0) fail(ODLA_INTERNAL_LOGIC_ERR, "kernel '%s' is not available", kernel->name.c_str());
+  const int src = s.main;  // staging tensor (declared type) or produced tensor, row-major
+  if (T(src).layout != L_ROWMAJOR) fail(ODLA_UNSUPPORTED_OP, "run-time kernel '%s' must be row-major", kernel->name.c_str());
+  pp.src_dt = T(src).dt;
+  const int dst = new_tensor(dst_dt, L_ROWMAJOR, ws, 0, SP_ARENA);
+  const Ref a = ref(src), b = ref(dst);
+  emit("pack:" + kernel->name, {src}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+    PackWeightsParams p = pp; p.src = a(e); p.dst = b(e);
+    return launch_pack_weights(p, st);
+  });
+  return dst;
+}
+
+int Planner::strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp) {
+  const Ref a = ref(src), b = ref(dst);
+  emit(name, {src}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
+    StridedCopyParams p = cp; p.x = a(e); p.y = b(e);
+    return launch_strided_copy(p, st);
+  });
+  return dst;
+}
+
+// Common tail of Conv / Gemm lowering: bias / residual / activation wiring and
+// the launch step.  tx, tw, ty are the operand tensors.
+void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty,
+                           const Epilogue& ep, int64_t Kout_total) {
+  int tb = -1, tr = -1;
+  if (ep.has_bias) {
+    std::vector<float> b = ep.bias;
+    b.resize((size_t)Kout_total, 0.f);
+    tb = const_vector<float>(DT_F32, b);
+  }
+  if (ep.residual != nullptr) {
+    const PTensor yo = T(ty);
+    tr = get(ep.residual, yo.layout, FORM_FLOAT);
+    if (T(tr).dt != yo.dt) fail(ODLA_INTERNAL_LOGIC_ERR, "residual type mismatch");
+    ip.rcs = yo.layout == L_NHWC ? T(tr).cs : ip.ycs;
+  }
+  ip.act = ep.act;
+  ip.act_a = ep.act_a;
+  ip.act_b = ep.act_b;
+  const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty);
+  const Ref rb = ref(tb >= 0 ? tb : tx), rr = ref(tr >= 0 ? tr : tx);
+  const bool hb = tb >= 0, hr = tr >= 0;
+  emit(name, {tx, tw, tr}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    IgemmParams p = ip;
+    p.x = rx(e); p.w = rw(e); p.y = ry(e);
+    p.bias = hb ? rb(e) : nullptr;
+    p.residual = hr ? rr(e) : nullptr;
+    return launch_igemm(p, st);
+  });
+}
+
+// ---------------------------------------------------------------- Conv ----
+void Planner::lower_conv(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const _odla_value* k = n.in[1];
+  const _odla_value* bias = n.in[2];
+  const bool cl = n.i[0] == ODLA_CHANNELS_LAST;
+  const int G = (int)n.i[1];
+  const int kl = (int)n.i[2];
+  const Shape& ks = k->shape;
+  int64_t O, I, R, S, so, si, sr, ss;
+  switch (kl) {
+    case ODLA_SIO: R = ks.d[0]; S = ks.d[1]; I = ks.d[2]; O = ks.d[3]; sr = S * I * O; ss = I * O; si = O; so = 1; break;
+    case ODLA_SOI: R = ks.d[0]; S = ks.d[1]; O = ks.d[2]; I = ks.d[3]; sr = S * O * I; ss = O * I; so = I; si = 1; break;
+    case ODLA_IOS: I = ks.d[0]; O = ks.d[1]; R = ks.d[2]; S = ks.d[3]; si = O * R * S; so = R * S; sr = S; ss = 1; break;
+    default: O = ks.d[0]; I = ks.d[1]; R = ks.d[2]; S = ks.d[3]; so = I * R * S; si = R * S; sr = S; ss = 1; break;
+  }
+  const Shape& xs = x->shape;
+  const Shape& os = n.out->shape;
+  const int64_t N = xs.d[0], C = cl ? xs.d[3] : xs.d[1], H = cl ? xs.d[1] : xs.d[2], W = cl ? xs.d[2] : xs.d[3];
+  const int64_t Ho = cl ? os.d[1] : os.d[2], Wo = cl ? os.d[2] : os.d[3];
+  const int Og = (int)(O / G), Cg = (int)I;
+
+  Epilogue ep;
+  if (bias != nullptr) {
+    if (bias->kind == _odla_value::CONSTANT) { ep.bias = const_as_float(bias); ep.has_bias = true; }
+  }
+  const bool runtime_bias = bias != nullptr && bias->kind != _odla_value::CONSTANT;
+  const bool const_kernel = k->kind == _odla_value::CONSTANT;
+  if (!runtime_bias) {
+    collect_epilogue(ni, O, cl ? 3 : 1, &ep);
+    if (!const_kernel && !ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "scale folding into a run-time kernel");
+  } else {
+    ep.final_value = n.out;
+  }
+  _odla_value* outv = ep.final_value;
+
+  // int8 plan?
+  const QuantEntry* qx = qentry(x);
+  const QuantEntry* qk = qentry(k);
+  const bool q8 = comp_->opts.int8 && qx != nullptr && qk != nullptr && const_kernel && !cl && G == 1 &&
+                  !runtime_bias;
+  if (q8) {
+    // ---- int8 x int8 -> int32 with fused requantisation ----
+    const int vec = 16;
+    const int tx = get(x, L_NHWC, FORM_QUANT, vec);
+    const int Cp = T(tx).cs;
+    if (qk->ch_min.size() != (size_t)O) fail(ODLA_INVALID_PARAM, "quant table entry of kernel '%s' needs %lld channel records", k->name.c_str(), (long long)O);
+    std::vector<float> sw((size_t)O);
+    for (int64_t o = 0; o < O; ++o) {
+      const float m = std::fmax(std::fabs(qk->ch_min[o]), std::fabs(qk->ch_max[o]));
+      sw[o] = m > 0.f ? m / 127.f : 1.f;
+    }
+    int w_rs = 0;
+    const int tw = pack_weights(k, DT_I8, 1, (int)O, Cg, (int)R, (int)S, Cp, so, si, sr, ss, {}, &w_rs, &sw);
+    // int32 bias: rne(b / (s_x * s_w[o])) minus the zero-point correction
+    // (zp_x - 128) * sum_k w_q[o][k]; activations are stored as q - 128.
+    std::vector<float> wf = const_as_float(k);
+    std::vector<int32_t> bi((size_t)O, 0);
+    const float sx = qx->scale;
+    const int zx = qx->zp;
+    for (int64_t o = 0; o < O; ++o) {
+      int64_t wsum = 0;
+      for (int64_t i = 0; i < Cg; ++i)
+        for (int r = 0; r < R; ++r)
+          for (int t = 0; t < S; ++t) {
+            float v = std::nearbyintf(wf[o * so + i * si + r * sr + t * ss] / sw[o]);
+            v = v < -127.f ? -127.f : (v > 127.f ? 127.f : v);
+            wsum += (int64_t)v;
+          }
+      int64_t b = 0;
+      if (ep.has_bias) {
+        const float bs = sx * sw[o];
+        float r = std::nearbyintf(ep.bias[o] / bs);
+        r = r < -2147483648.f ? -2147483648.f : (r > 2147483520.f ? 2147483520.f : r);
+        b = (int64_t)r;
+      }
+      b -= (int64_t)(zx - 128) * wsum;
+      bi[o] = (int32_t)b;
+    }
+    const int tb = const_vector<int32_t>(DT_I32, bi);
+
+    IgemmParams ip;
+    ip.N = (int)N; ip.H = (int)H; ip.W = (int)W; ip.C = Cp; ip.xcs = Cp;
+    ip.Ho = (int)Ho; ip.Wo = (int)Wo; ip.Kout = (int)O;
+    ip.R = (int)R; ip.S = (int)S; ip.sh = (int)n.i[3]; ip.sw = (int)n.i[4];
+    ip.dh = (int)n.i[5]; ip.dw = (int)n.i[6]; ip.ph = (int)n.i[7]; ip.pw = (int)n.i[8];
+    ip.w_rows = (int)O; ip.w_cols = w_rs; ip.w_rs = w_rs;
+    ip.in_dt = DT_I8;
+    ip.a_fill = (zx - 128) & 0xff;
+
+    const _odla_value* qv = ep.residual ? ep.pre_residual_value : outv;
+    const QuantEntry* qo = qentry(qv);
+    const QuantEntry* qf = qentry(outv);
+    std::vector<float> mul((size_t)O);
+    int ty;
+    if (qo != nullptr && qf != nullptr) {
+      for (int64_t o = 0; o < O; ++o) mul[o] = (sx * sw[o]) / qo->scale;
+      ip.out_dt = DT_I8;
+      ip.q_zp = qo->zp;
+      ip.q_scale = qo->scale;
+      const bool relu = ep.act == ACT_RELU;
+      if (ep.residual) {
+        const QuantEntry* qr = qentry(ep.residual);
+        ip.q_lo = 0;
+        ip.r_zp = qr->zp; ip.r_scale = qr->scale;
+        ip.s_inv = 1.0f / qf->scale; ip.s_zp = qf->zp; ip.s_lo = relu ? qf->zp : 0;
+      } else {
+        ip.q_lo = relu ? qo->zp : 0;
+      }
+      ty = new_tensor(DT_I8, L_NHWC, outv->shape, (int)O, SP_ARENA);
+      set_quant(ty, true, qf->scale, qf->zp);
+    } else if (comp_->opts.raw_acc && ep.residual == nullptr && ep.act == ACT_NONE) {
+      ip.out_dt = DT_I32;
+      ty = new_tensor(DT_I32, L_NHWC, outv->shape, (int)O, SP_ARENA);
+    } else {
+      if (ep.residual != nullptr) fail(ODLA_UNSUPPORTED_OP, "int8 residual fusion needs quant entries for '%s'", outv->name.c_str());
+      for (int64_t o = 0; o < O; ++o) mul[o] = sx * sw[o];
+      ip.out_dt = DT_F32;
+      ip.act = ep.act; ip.act_a = ep.act_a; ip.act_b = ep.act_b;
+      ty = new_tensor(DT_F32, L_NHWC, outv->shape, (int)O, SP_ARENA);
+    }
+    ip.ycs = (int)O;
+    const int tm = const_vector<float>(DT_F32, mul);
+    int tr = -1;
+    if (ep.residual) {
+      tr = get(ep.residual, L_NHWC, FORM_QUANT);
+      ip.rcs = T(tr).cs;
+    }
+    const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb), rm = ref(tm), rr = ref(tr >= 0 ? tr : tx);
+    const bool hr = tr >= 0;
+    emit("conv.i8:" + outv->name, {tx, tw, tr}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+      IgemmParams p = ip;
+      p.x = rx(e); p.w = rw(e); p.y = ry(e); p.bias = rb(e);
+      p.qmul = (const float*)rm(e);
+      p.residual = hr ? rr(e) : nullptr;
+      return launch_igemm(p, st);
+    });
+    if (ip.out_dt == DT_I32) {
+      // raw accumulators are exposed through the FLOAT32-typed value as bit patterns
+      T(ty).dt = DT_F32;
+    }
+    if (ip.out_dt == DT_F32 && cdt_ != DT_F32) {
+      const int tc = new_tensor(cdt_, L_NHWC, outv->shape, (int)O, SP_ARENA);
+      const int64_t ne = T(ty).phys_elems();
+      const Ref a = ref(ty), b = ref(tc);
+      const DType ddt = cdt_;
+      emit("cast:" + outv->name, {ty}, {tc}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), DT_F32, b(e), ddt, ne, st); });
+      ty = tc;
+    }
+    set_main(outv, ty);
+    return;
+  }
+
+  // ---- floating-point path ----
+  const DType dt = storage_dtype(x);
+  if (!dtype_is_float(dt)) fail(ODLA_UNSUPPORTED_DATATYPE, "odla_Conv on element type %d", (int)x->etype);
+  const int vec = 16 / dtype_size(dt);
+  int tx;
+  int xcs;
+  if (cl) {
+    tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+    xcs = (int)C;
+  } else {
+    tx = get(x, L_NHWC, FORM_FLOAT, vec);
+    xcs = T(tx).cs;
+  }
+  if (T(tx).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "conv input storage type mismatch");
+  int Cp;
+  if (G == 1) {
+    if (xcs % vec != 0) fail(ODLA_UNSUPPORTED_OP, "channels-last convolution input with %d channels needs a multiple of %d", xcs, vec);
+    Cp = xcs;
+  } else {
+    if (Cg % vec != 0) fail(ODLA_UNSUPPORTED_OP, "grouped convolution with %d channels per group (needs a multiple of %d)", Cg, vec);
+    Cp = Cg;
+  }
+  int w_rs = 0;
+  const int tw = pack_weights(k, dt, G, Og, Cg, (int)R, (int)S, Cp, so, si, sr, ss, ep.row_scale, &w_rs, nullptr);
+
+  IgemmParams ip;
+  ip.N = (int)N; ip.H = (int)H; ip.W = (int)W; ip.C = Cp; ip.xcs = xcs;
+  ip.Ho = (int)Ho; ip.Wo = (int)Wo; ip.Kout = Og;
+  ip.R = (int)R; ip.S = (int)S; ip.sh = (int)n.i[3]; ip.sw = (int)n.i[4];
+  ip.dh = (int)n.i[5]; ip.dw = (int)n.i[6]; ip.ph = (int)n.i[7]; ip.pw = (int)n.i[8];
+  ip.w_rows = Og; ip.w_cols = w_rs; ip.w_rs = w_rs;
+  ip.in_dt = dt; ip.out_dt = dt;
+  ip.batch = G;
+  ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og;
+  ip.ycs = (int)O;
+
+  int ty;
+  if (cl) ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
+  else ty = new_tensor(dt, L_NHWC, outv->shape, (int)O, SP_ARENA);
+
+  if (runtime_bias) {
+    // bias supplied at run time: read it as fp32 from its staging tensor
+    const VState& bs = vs_[bias->index];
+    if (bs.main < 0 || T(bs.main).dt != DT_F32) fail(ODLA_UNSUPPORTED_OP, "run-time conv bias must be FLOAT32");
+    const int tb = bs.main;
+    const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb);
+    emit("conv:" + outv->name, {tx, tw, tb}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+      IgemmParams p = ip;
+      p.x = rx(e); p.w = rw(e); p.y = ry(e); p.bias = rb(e);
+      return launch_igemm(p, st);
+    });
+  } else {
+    finish_igemm("conv:" + outv->name, ip, tx, tw, ty, ep, O);
+  }
+  set_main(outv, ty);
+}
+
+// ---------------------------------------------------------------- Gemm ----
+void Planner::lower_gemm(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* A = n.in[0];
+  const _odla_value* B = n.in[1];
+  const _odla_value* Cv = n.in[2];
+  const bool tA = n.i[0] != 0, tB = n.i[1] != 0;
+  const Shape& as = A->shape;
+  const Shape& bs = B->shape;
+  const Shape& os = n.out->shape;
+  const int64_t M = os.d[os.rank - 2], Nn = os.d[os.rank - 1];
+  const int64_t K = tA ? as.d[as.rank - 2] : as.d[as.rank - 1];
+  int64_t lead = 1;
+  for (int i = 0; i < as.rank - 2; ++i) lead *= as.d[i];
+  const bool shared_b = bs.rank == 2;
+  const DType dt = storage_dtype(A);
+  if (!dtype_is_float(dt)) fail(ODLA_UNSUPPORTED_DATATYPE, "odla_Gemm on element type %d", (int)A->etype);
+  const int vec = 16 / dtype_size(dt);
+
+  Epilogue ep;
+  // bias operand: alpha*(A.B) + beta*C
+  const float alpha = n.f[0], beta = n.f[1];
+  _odla_value* full_c = nullptr;
+  if (Cv != nullptr && beta != 0.f) {
+    const int64_t cn = Cv->shape.numel();
+    if (Cv->kind == _odla_value::CONSTANT && (cn == 1 || cn == Nn)) {
+      std::vector<float> c = const_as_float(Cv);
+      ep.bias.assign((size_t)Nn, 0.f);
+      for (int64_t j = 0; j < Nn; ++j) ep.bias[j] = beta * c[cn == 1 ? 0 : j];
+      ep.has_bias = true;
+    } else if (beta == 1.f && Cv->shape == os && Cv->kind != _odla_value::CONSTANT) {
+      full_c = const_cast<_odla_value*>(Cv);
+    } else {
+      fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: C operand of shape %s with beta %g is not supported", Cv->shape.str().c_str(), beta);
+    }
+  }
+  if (full_c == nullptr) collect_epilogue(ni, Nn, os.rank - 1, &ep);
+  else { ep.residual = full_c; ep.final_value = n.out; }
+  _odla_value* outv = ep.final_value;
+  if (alpha != 1.f && ep.has_bias && !ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: alpha with folded scale");
+
+  // ---- A operand: row-major [lead][M][K], K padded to the vector width ----
+  int ta = get(A, L_ROWMAJOR, FORM_FLOAT);
+  if (T(ta).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "gemm input storage type mismatch");
+  int Kp = round_up_i((int)K, vec);
+  if (tA || Kp != K) {
+    // materialise A^T and/or zero-pad K
+    Shape s2;
+    s2.rank = 3;
+    s2.d[0] = lead; s2.d[1] = M; s2.d[2] = Kp;
+    const int t2 = new_tensor(dt, L_ROWMAJOR, s2, 0, SP_ARENA);
+    if (Kp != K) {
+      const Ref b = ref(t2);
+      const int64_t words = (int64_t)(T(t2).bytes / 4);
+      emit("gemm.zero:" + outv->name, {}, {t2}, [=](const ExecEnv& e, hipStream_t st) { return launch_fill_i32((int32_t*)b(e), words, 0, st); });
+    }
+    StridedCopyParams cp;
+    cp.elem_size = dtype_size(dt);
+    cp.rank = 3;
+    cp.dims[0] = lead; cp.dims[1] = M; cp.dims[2] = K;
+    cp.sy[0] = M * Kp; cp.sy[1] = Kp; cp.sy[2] = 1;
+    cp.sx[0] = M * K; cp.sx[1] = tA ? 1 : K; cp.sx[2] = tA ? M : 1;
+    strided_copy_step("gemm.a:" + outv->name, ta, t2, cp);
+    ta = t2;
+  }
+
+  IgemmParams ip;
+  ip.H = 1; ip.W = 1; ip.Ho = 1; ip.Wo = 1;
+  ip.C = Kp; ip.xcs = Kp;
+  ip.Kout = (int)Nn;
+  ip.in_dt = dt; ip.out_dt = dt;
+  ip.alpha = alpha;
+  ip.ycs = (int)Nn;
+  int tw;
+  if (B->kind == _odla_value::CONSTANT && (shared_b || lead == 1)) {
+    // weights: pack once.  B[k][n] (so=1, si=N) or B^T[n][k] (so=K, si=1)
+    int w_rs = 0;
+    const int64_t so = tB ? K : 1, si = tB ? 1 : Nn;
+    if (alpha != 1.f && !ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: alpha with folded scale");
+    tw = pack_weights(B, dt, 1, (int)Nn, (int)K, 1, 1, Kp, so, si, 0, 0, ep.row_scale, &w_rs, nullptr);
+    ip.w_rows = (int)Nn; ip.w_cols = w_rs; ip.w_rs = w_rs;
+    ip.N = (int)(lead * M);
+    ip.batch = 1;
+  } else {
+    if (!ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: scale folding into a run-time operand");
+    int tb = get(B, L_ROWMAJOR, FORM_FLOAT);
+    if (T(tb).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "gemm operand storage type mismatch");
+    const int64_t blead = shared_b ? 1 : lead;
+    if (!tB || Kp != K) {
+      // need [blead][N][Kp]
+      Shape s2;
+      s2.rank = 3;
+      s2.d[0] = blead; s2.d[1] = Nn; s2.d[2] = Kp;
+      const int t2 = new_tensor(dt, L_ROWMAJOR, s2, 0, SP_ARENA);
+      if (Kp != K) {
+        const Ref b = ref(t2);
+        const int64_t words = (int64_t)(T(t2).bytes / 4);
+        emit("gemm.zero:" + outv->name, {}, {t2}, [=](const ExecEnv& e, hipStream_t st) { return launch_fill_i32((int32_t*)b(e), words, 0, st); });
+      }
+      StridedCopyParams cp;
+      cp.elem_size = dtype_size(dt);
+      cp.rank = 3;
+      cp.dims[0] = blead; cp.dims[1] = Nn; cp.dims[2] = K;
+      cp.sy[0] = Nn * Kp; cp.sy[1] = Kp; cp.sy[2] = 1;
+      cp.sx[0] = K * Nn; cp.sx[1] = tB ? K : 1; cp.sx[2] = tB ? 1 : Nn;
+      strided_copy_step("gemm.b:" + outv->name, tb, t2, cp);
+      tb = t2;
+    }
+    tw = tb;
+    ip.w_rows = (int)Nn; ip.w_cols = Kp; ip.w_rs = Kp;
+    if (shared_b) { ip.N = (int)(lead * M); ip.batch = 1; }
+    else {
+      ip.N = (int)M; ip.batch = (int)lead;
+      ip.x_bs = M * Kp; ip.w_bs = Nn * Kp; ip.y_bs = M * Nn; ip.r_bs = M * Nn; ip.bias_bs = 0;
+    }
+  }
+  const int ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
+  finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
+  set_main(outv, ty);
+}
+
+// -------------------------------------------------------------- Binary ----
+namespace {
+// element stride of each logical dim of a physical tensor
+void logical_strides(const PTensor& t, int64_t* st) {
+  const Shape& s = t.shape;
+  if (t.layout == L_NHWC) {
+    st[0] = s.d[2] * s.d[3] * t.cs;
+    st[1] = 1;
+    st[2] = s.d[3] * t.cs;
+    st[3] = t.cs;
+    return;
+  }
+  int64_t acc = 1;
+  for (int i = s.rank - 1; i >= 0; --i) { st[i] = acc; acc *= s.d[i]; }
+}
+}  // namespace
+
+void Planner::lower_binary(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* a = n.in[0];
+  const _odla_value* b = n.in[1];
+  _odla_value* outv = n.out;
+  const Shape& os = outv->shape;
+  const int r = (int)n.iv[0];
+  Shape sa, sb;
+  sa.rank = sb.rank = r;
+  for (int i = 0; i < r; ++i) { sa.d[i] = n.iv[1 + i]; sb.d[i] = n.iv[1 + r + i]; }
+  const DType dt = storage_dtype(outv);
+
+  // optional trailing activation
+  ActKind act = ACT_NONE;
+  float act_a = 0.f, act_b = 0.f;
+  const QuantEntry* qa = qentry(a);
+  const QuantEntry* qb = qentry(b);
+  const bool q8 = comp_->opts.int8 && qa && qb && a->shape == os && b->shape == os &&
+                  (n.i[0] == BIN_ADD) && a->kind != _odla_value::CONSTANT && b->kind != _odla_value::CONSTANT;
+  if (!outv->is_output && consumers_[outv->index].size() == 1) {
+    Node& nx = comp_->nodes[consumers_[outv->index][0]];
+    if (nx.op == OP_UNARY && !nx.absorbed) {
+      const ActKind k = (ActKind)nx.i[0];
+      if (k == ACT_RELU || (!q8 && (k == ACT_LEAKY || k == ACT_CLAMP))) {
+        if (!q8 || qentry(nx.out) != nullptr) {
+          act = k; act_a = nx.f[0]; act_b = nx.f[1];
+          nx.absorbed = true;
+          outv = nx.out;
+        }
+      }
+    }
+  }
+  const QuantEntry* qo = qentry(outv);
+
+  if (q8 && qo != nullptr) {
+    // both operands 8-bit, same shape: stay in the quantised domain
+    const Layout lay = (os.rank == 4 && vs_[a->index].slot[L_NHWC][FORM_QUANT] >= 0) ? L_NHWC : L_ROWMAJOR;
+    const int ta = get(a, lay, FORM_QUANT);
+    const int tb = get(b, lay, FORM_QUANT);
+    if (lay == L_NHWC && T(ta).cs != T(tb).cs) fail(ODLA_UNSUPPORTED_OP, "quantised add of differently padded tensors");
+    const int ty = new_tensor(DT_I8, lay, os, T(ta).cs, SP_ARENA);
+    set_quant(ty, true, qo->scale, qo->zp);
+    BinaryParams bp;
+    bp.dt = DT_I8;
+    bp.op = BIN_ADD;
+    bp.rank = 1;
+    bp.dims[0] = T(ta).phys_elems();
+    bp.sa[0] = 1; bp.sb[0] = 1;
+    bp.a_scale = T(ta).qscale; bp.a_zp = T(ta).qzp;
+    bp.b_scale = T(tb).qscale; bp.b_zp = T(tb).qzp;
+    bp.y_inv = 1.0f / qo->scale; bp.y_zp = qo->zp; bp.y_lo = act == ACT_RELU ? qo->zp : 0;
+    const Ref ra = ref(ta), rb = ref(tb), ry = ref(ty);
+    emit("add.q8:" + outv->name, {ta, tb}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+      BinaryParams p = bp; p.a = ra(e); p.b = rb(e); p.y = ry(e);
+      return launch_binary(p, st);
+    });
+    set_main(outv, ty);
+    return;
+  }
+
+  if (!dtype_is_float(dt)) fail(ODLA_UNSUPPORTED_DATATYPE, "element-wise arithmetic on non-float values ('%s')", outv->name.c_str());
+  // Output layout: channels-last if either full-size operand already lives that way.
+  Layout lay = L_ROWMAJOR;
+  if (os.rank == 4) {
+    auto nhwc_main = [&](const _odla_value* v) {
+      const VState& s = vs_[v->index];
+      return v->shape == os && s.main >= 0 && T(s.main).layout == L_NHWC;
+    };
+    if (nhwc_main(a) || nhwc_main(b)) lay = L_NHWC;
+  }
+  auto operand = [&](const _odla_value* v, const Shape& aligned) -> int {
+    // full-shape rank-4 operands follow the output layout; broadcast operands stay row-major
+    if (lay == L_NHWC && v->shape == os) return get(v, L_NHWC, FORM_FLOAT);
+    (void)aligned;
+    return get(v, L_ROWMAJOR, FORM_FLOAT);
+  };
+  const int ta = operand(a, sa), tb = operand(b, sb);
+  if (T(ta).dt != dt || T(tb).dt != dt) fail(ODLA_UNSUPPORTED_DATATYPE, "mixed storage types in element-wise op '%s'", outv->name.c_str());
+  int ocs = 0;
+  if (lay == L_NHWC) {
+    ocs = (int)os.d[1];
+    if ((a->shape == os && T(ta).cs != ocs) || (b->shape == os && T(tb).cs != ocs))
+      fail(ODLA_UNSUPPORTED_OP, "element-wise op '%s' on a channel-padded tensor", outv->name.c_str());
+  }
+  const int ty = new_tensor(dt, lay, os, ocs, SP_ARENA);
+
+  // physical iteration order of the output and per-operand strides
+  int order[ODLA_MAX_DIMENSION];
+  int64_t odims[ODLA_MAX_DIMENSION];
+  if (lay == L_NHWC) {
+    order[0] = 0; order[1] = 2; order[2] = 3; order[3] = 1;
+  } else {
+    for (int i = 0; i < r; ++i) order[i] = i;
+  }
+  auto strides_for = [&](int t, const Shape& aligned, int64_t* st_phys) {
+    // strides of the operand's own logical dims, mapped through the aligned shape
+    PTensor pt = T(t);
+    int64_t ls[ODLA_MAX_DIMENSION] = {0};
+    if (pt.layout == L_NHWC) {
+      logical_strides(pt, ls);
+    } else {
+      // the operand is row-major over its aligned shape (alignment only adds 1-dims)
+      int64_t acc = 1;
+      for (int i = r - 1; i >= 0; --i) { ls[i] = acc; acc *= aligned.d[i]; }
+    }
+    for (int i = 0; i < r; ++i) {
+      const int ld = order[i];
+      st_phys[i] = (aligned.d[ld] == 1 && os.d[ld] != 1) ? 0 : ls[ld];
+      if (aligned.d[ld] == 1) st_phys[i] = 0;
+    }
+  };
+  int64_t pa[ODLA_MAX_DIMENSION], pb[ODLA_MAX_DIMENSION];
+  strides_for(ta, sa, pa);
+  strides_for(tb, sb, pb);
+  for (int i = 0; i < r; ++i) odims[i] = os.d[order[i]];
+  // collapse to at most 6 dims by merging adjacent dims that are contiguous in all three
+  BinaryParams bp;
+  bp.dt = dt;
+  bp.op = (BinKind)n.i[0];
+  bp.act = act; bp.act_a = act_a; bp.act_b = act_b;
+  {
+    // output strides in physical order
+    int64_t py[ODLA_MAX_DIMENSION];
+    if (lay == L_NHWC) { py[0] = os.d[2] * os.d[3] * ocs; py[1] = os.d[3] * ocs; py[2] = ocs; py[3] = 1; }
+    else { int64_t acc = 1; for (int i = r - 1; i >= 0; --i) { py[i] = acc; acc *= os.d[i]; } }
+    std::vector<int64_t> d, xa, xb, xy;
+    for (int i = 0; i < r; ++i) {
+      if (odims[i] == 1) continue;
+      if (!d.empty()) {
+        const size_t l = d.size() - 1;
+        const bool merge = xa[l] == pa[i] * odims[i] && xb[l] == pb[i] * odims[i] && xy[l] == py[i] * odims[i];
+        if (merge) { d[l] *= odims[i]; xa[l] = pa[i]; xb[l] = pb[i]; xy[l] = py[i]; continue; }
+      }
+      d.push_back(odims[i]); xa.push_back(pa[i]); xb.push_back(pb[i]); xy.push_back(py[i]);
+    }
+    if (d.empty()) { d.push_back(1); xa.push_back(0); xb.push_back(0); xy.push_back(1); }
+    if (d.size() > 6) fail(ODLA_UNSUPPORTED_OP, "element-wise op '%s' needs more than 6 broadcast dims", outv->name.c_str());
+    // the kernel assumes a contiguous output over dims[]; that holds unless channel padding was dropped
+    int64_t acc = 1;
+    for (int i = (int)d.size() - 1; i >= 0; --i) {
+      if (xy[i] != acc) fail(ODLA_UNSUPPORTED_OP, "element-wise op '%s' on a padded channels-last tensor", outv->name.c_str());
+      acc *= d[i];
+    }
+    bp.rank = (int)d.size();
+    for (size_t i = 0; i < d.size(); ++i) { bp.dims[i] = d[i]; bp.sa[i] = xa[i]; bp.sb[i] = xb[i]; }
+  }
+  const Ref ra = ref(ta), rb = ref(tb), ry = ref(ty);
+  emit("binary:" + outv->name, {ta, tb}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    BinaryParams p = bp; p.a = ra(e); p.b = rb(e); p.y = ry(e);
+    return launch_binary(p, st);
+  });
+  set_main(outv, ty);
+}
+
+// --------------------------------------------------------------- Unary ----
+void Planner::lower_unary(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const VState& s = vs_[x->index];
+  const ActKind act = (ActKind)n.i[0];
+  // 8-bit ReLU keeps the levels: q = max(q, zp), expressed as add-with-zero is
+  // overkill; dequantise instead unless the producer fused it (the common case).
+  Layout lay = L_ROWMAJOR;
+  if (s.main >= 0 && !T(s.main).quant) lay = T(s.main).layout;
+  else if (x->shape.rank == 4 && s.slot[L_NHWC][FORM_FLOAT] >= 0) lay = L_NHWC;
+  else if (s.main >= 0 && T(s.main).quant) lay = T(s.main).layout;
+  const int tx = get(x, lay, FORM_FLOAT);
+  const PTensor px = T(tx);
+  const int ty = new_tensor(px.dt, px.layout, n.out->shape, px.cs, SP_ARENA);
+  const int64_t ne = px.phys_elems();
+  const float fa = n.f[0], fb = n.f[1];
+  const DType dt = px.dt;
+  const Ref a = ref(tx), b = ref(ty);
+  emit(std::string("unary:") + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_unary(a(e), b(e), dt, ne, act, fa, fb, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ----------------------------------------------------------- BatchNorm ----
+void Planner::lower_batchnorm(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const bool cf = n.i[0] != ODLA_CHANNELS_LAST;
+  const Shape& xs = x->shape;
+  const int64_t C = cf ? xs.d[1] : xs.d[xs.rank - 1];
+  const VState& s = vs_[x->index];
+  Layout lay = L_ROWMAJOR;
+  if (cf && xs.rank == 4 && s.main >= 0 && T(s.main).layout == L_NHWC) lay = L_NHWC;
+  const int tx = get(x, lay, FORM_FLOAT);
+  const PTensor px = T(tx);
+  const int ty = new_tensor(px.dt, px.layout, n.out->shape, px.cs, SP_ARENA);
+  int64_t inner;
+  int channels;
+  if (lay == L_NHWC) { inner = 1; channels = px.cs; }
+  else if (cf) { inner = 1; for (int i = 2; i < xs.rank; ++i) inner *= xs.d[i]; channels = (int)C; }
+  else { inner = 1; channels = (int)C; }
+
+  bool all_const = true;
+  for (int i = 1; i <= 4; ++i)
+    if (n.in[i] && n.in[i]->kind != _odla_value::CONSTANT) all_const = false;
+  int tscale, tshift;
+  if (all_const) {
+    std::vector<float> sc, sh;
+    bn_params_host(n, C, &sc, &sh);
+    sc.resize((size_t)channels, 1.f);
+    sh.resize((size_t)channels, 0.f);
+    tscale = const_vector<float>(DT_F32, sc);
+    tshift = const_vector<float>(DT_F32, sh);
+  } else {
+    // statistics arrive at run time (fp32 arguments): fold them on the device
+    if (channels != C) fail(ODLA_UNSUPPORTED_OP, "run-time BatchNorm parameters on a padded tensor");
+    int tp[5] = {-1, -1, -1, -1, -1};
+    for (int i = 1; i <= 4; ++i) {
+      if (!n.in[i]) continue;
+      const _odla_value* pv = n.in[i];
+      if (dtype_from_odla(pv->etype) != DT_F32) fail(ODLA_UNSUPPORTED_DATATYPE, "BatchNorm parameters must be FLOAT32");
+      if (pv->kind == _odla_value::CONSTANT) tp[i] = const_from_host(DT_F32, pv->shape, pv->host_data, nullptr);
+      else {
+        const VState& ps = vs_[pv->index];
+        if (ps.main < 0 || T(ps.main).dt != DT_F32) fail(ODLA_UNSUPPORTED_OP, "BatchNorm parameter '%s' must be a FLOAT32 argument", pv->name.c_str());
+        tp[i] = ps.main;
+      }
+    }
+    Shape cs1;
+    cs1.rank = 1;
+    cs1.d[0] = C;
+    tscale = new_tensor(DT_F32, L_ROWMAJOR, cs1, 0, SP_ARENA);
+    tshift = new_tensor(DT_F32, L_ROWMAJOR, cs1, 0, SP_ARENA);
+    const Ref rm = ref(tp[1]), rv = ref(tp[2]), rg = ref(tp[3] >= 0 ? tp[3] : tp[1]), rb = ref(tp[4] >= 0 ? tp[4] : tp[1]);
+    const bool hg = tp[3] >= 0, hb = tp[4] >= 0;
+    const Ref rs = ref(tscale), rt = ref(tshift);
+    const float sg = n.f[1], sb = n.f[2], eps = n.f[0];
+    const int Ci = (int)C;
+    emit("bn.fold:" + n.out->name, {tp[1], tp[2], tp[3], tp[4]}, {tscale, tshift}, [=](const ExecEnv& e, hipStream_t st) {
+      return launch_bn_fold((const float*)rm(e), (const float*)rv(e), hg ? (const float*)rg(e) : nullptr,
+                            hb ? (const float*)rb(e) : nullptr, sg, sb, eps, Ci, (float*)rs(e), (float*)rt(e), st);
+    });
+  }
+  const int64_t ne = px.phys_elems();
+  const DType dt = px.dt;
+  const Ref a = ref(tx), b = ref(ty), rs = ref(tscale), rt = ref(tshift);
+  emit("bn:" + n.out->name, {tx, tscale, tshift}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_channel_affine(a(e), b(e), dt, ne, inner, channels, (const float*)rs(e), (const float*)rt(e), st);
+  });
+  set_main(n.out, ty);
+}
+
+// ----------------------------------------------------------- LayerNorm ----
+void Planner::lower_layernorm(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const Shape& xs = x->shape;
+  const int na = (int)n.i[0];
+  int64_t len = 1;
+  for (int i = xs.rank - na; i < xs.rank; ++i) len *= xs.d[i];
+  const int64_t rows = xs.numel() / len;
+  int tg = -1, tb = -1;
+  if (n.in[1]) { std::vector<float> g = const_as_float(n.in[1]); tg = const_vector<float>(DT_F32, g); }
+  if (n.in[2]) { std::vector<float> b = const_as_float(n.in[2]); tb = const_vector<float>(DT_F32, b); }
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const Ref a = ref(tx), b = ref(ty), rg = ref(tg >= 0 ? tg : tx), rb = ref(tb >= 0 ? tb : tx);
+  const bool hg = tg >= 0, hb = tb >= 0;
+  const float eps = n.f[0];
+  emit("layernorm:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_layernorm(a(e), b(e), dt, rows, len, hg ? (const float*)rg(e) : nullptr,
+                            hb ? (const float*)rb(e) : nullptr, eps, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ---------------------------------------------------------------- Pool ----
+void Planner::lower_pool(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const bool cl = n.i[0] == ODLA_CHANNELS_LAST;
+  const Shape& xs = x->shape;
+  const Shape& os = n.out->shape;
+  const bool is_max = n.i[1] != 0;
+  // 8-bit max pooling keeps levels (the result inherits the input's scale)
+  const VState& s = vs_[x->index];
+  const bool q8 = is_max && !cl && s.main >= 0 && T(s.main).quant && qentry(n.out) != nullptr && (xs.d[1] % 16 == 0);
+  int tx;
+  if (cl) tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  else tx = get(x, L_NHWC, q8 ? FORM_QUANT : FORM_FLOAT);
+  const PTensor px = T(tx);
+  PoolParams pp;
+  pp.dt = px.dt;
+  pp.N = (int)xs.d[0];
+  pp.H = (int)(cl ? xs.d[1] : xs.d[2]);
+  pp.W = (int)(cl ? xs.d[2] : xs.d[3]);
+  pp.C = (int)(cl ? xs.d[3] : xs.d[1]);
+  pp.cs = cl ? pp.C : px.cs;
+  pp.Ho = (int)(cl ? os.d[1] : os.d[2]);
+  pp.Wo = (int)(cl ? os.d[2] : os.d[3]);
+  pp.ycs = pp.C;
+  pp.kh = (int)n.i[2]; pp.kw = (int)n.i[3]; pp.sh = (int)n.i[4]; pp.sw = (int)n.i[5];
+  pp.ph = (int)n.i[6]; pp.pw = (int)n.i[7];
+  pp.is_max = is_max;
+  pp.count_include_pad = n.i[10] != 0;
+  int ty;
+  if (cl) ty = new_tensor(px.dt, L_ROWMAJOR, os, 0, SP_ARENA);
+  else ty = new_tensor(px.dt, L_NHWC, os, pp.C, SP_ARENA);
+  if (q8) set_quant(ty, true, px.qscale, px.qzp);
+  const Ref a = ref(tx), b = ref(ty);
+  emit(std::string(is_max ? "maxpool:" : "avgpool:") + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    PoolParams p = pp; p.x = a(e); p.y = b(e);
+    return launch_pool2d(p, st);
+  });
+  set_main(n.out, ty);
+}
+
+// -------------------------------------------------------------- Reduce ----
+void Planner::lower_reduce(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const ReduceKind kind = (ReduceKind)n.i[0];
+  const std::vector<int64_t>& axes = n.iv;
+  const VState& s = vs_[x->index];
+  // spatial reduction of a channels-last tensor (global pooling)
+  const bool spatial = xs.rank == 4 && axes.size() == 2 && axes[0] == 2 && axes[1] == 3;
+  if (spatial && s.main >= 0 && T(s.main).layout == L_NHWC) {
+    const PTensor px = T(s.main);
+    const int64_t outer = xs.d[0], len = xs.d[2] * xs.d[3], inner = px.cs;
+    if (px.cs != xs.d[1]) fail(ODLA_UNSUPPORTED_OP, "reduction over a padded channels-last tensor");
+    Shape o4;
+    o4.rank = 4;
+    o4.d[0] = xs.d[0]; o4.d[1] = xs.d[1]; o4.d[2] = 1; o4.d[3] = 1;
+    const Ref a = ref(s.main);
+    int ty;
+    if (px.quant) {
+      if (kind != RED_MEAN) fail(ODLA_UNSUPPORTED_OP, "only ReduceMean is supported on 8-bit tensors");
+      ty = new_tensor(DT_F32, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+      const Ref b = ref(ty);
+      const float sc = px.qscale;
+      const int zp = px.qzp;
+      emit("reduce.q8:" + n.out->name, {s.main}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_reduce_q8_mean(a(e), (float*)b(e), outer, len, inner, sc, zp, st);
+      });
+      if (cdt_ != DT_F32) {
+        const int tc = new_tensor(cdt_, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+        const Ref c = ref(tc);
+        const int64_t ne = n.out->shape.numel();
+        const DType ddt = cdt_;
+        emit("cast:" + n.out->name, {ty}, {tc}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(b(e), DT_F32, c(e), ddt, ne, st); });
+        ty = tc;
+      }
+    } else {
+      ty = new_tensor(px.dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+      const Ref b = ref(ty);
+      const DType dt = px.dt;
+      emit("reduce:" + n.out->name, {s.main}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_reduce(a(e), b(e), dt, dt, outer, len, inner, kind, st);
+      });
+    }
+    set_main(n.out, ty);
+    return;
+  }
+  // general case: the reduced axes must be adjacent in row-major order
+  for (size_t i = 1; i < axes.size(); ++i)
+    if (axes[i] != axes[i - 1] + 1) fail(ODLA_UNSUPPORTED_OP, "reduction over non-adjacent axes");
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  int64_t outer = 1, len = 1, inner = 1;
+  for (int i = 0; i < xs.rank; ++i) {
+    if (i < axes.front()) outer *= xs.d[i];
+    else if (i <= axes.back()) len *= xs.d[i];
+    else inner *= xs.d[i];
+  }
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const Ref a = ref(tx), b = ref(ty);
+  emit("reduce:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_reduce(a(e), b(e), dt, dt, outer, len, inner, kind, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ------------------------------------------------------------- Softmax ----
+void Planner::lower_softmax(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const int axis = (int)n.i[0];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= xs.d[i];
+  for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
+  const int64_t len = xs.d[axis];
+  const DType dt = T(tx).dt;
+  // a graph output is written in fp32 directly
+  const bool to_f32 = n.out->is_output && dtype_from_odla(n.out->etype) == DT_F32 && consumers_[n.out->index].empty();
+  const DType odt = to_f32 ? DT_F32 : dt;
+  const int ty = new_tensor(odt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const bool logsm = n.i[1] != 0;
+  const Ref a = ref(tx), b = ref(ty);
+  emit("softmax:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_softmax(a(e), b(e), dt, odt, outer, len, inner, logsm, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ---------------------------------------------------------------- Cast ----
+void Planner::lower_cast(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const DType sdt = T(tx).dt;
+  const DType ddt = storage_dtype(n.out);
+  if (sdt == ddt) {
+    set_main(n.out, alias_tensor(tx, n.out->shape));
+    return;
+  }
+  const int ty = new_tensor(ddt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const int64_t ne = x->shape.numel();
+  const Ref a = ref(tx), b = ref(ty);
+  emit("cast:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), ddt, ne, st); });
+  set_main(n.out, ty);
+}
+
+// -------------------------------------------------------------- Concat ----
+void Planner::lower_concat(int ni) {
+  Node& n = comp_->nodes[ni];
+  const Shape& os = n.out->shape;
+  const int axis = (int)n.i[0];
+  // channel concat of channels-last tensors stays channels-last
+  bool nhwc = os.rank == 4 && axis == 1;
+  if (nhwc) {
+    bool any = false;
+    for (_odla_value* v : n.in) {
+      const VState& s = vs_[v->index];
+      if (s.main >= 0 && T(s.main).layout == L_NHWC && !T(s.main).quant) any = true;
+    }
+    nhwc = any;
+  }
+  const Layout lay = nhwc ? L_NHWC : L_ROWMAJOR;
+  std::vector<int> tin;
+  for (_odla_value* v : n.in) tin.push_back(get(v, lay, FORM_FLOAT));
+  const DType dt = T(tin[0]).dt;
+  const int es = dtype_size(dt);
+  const int ty = new_tensor(dt, lay, os, nhwc ? (int)os.d[1] : 0, SP_ARENA);
+  int64_t off = 0;
+  for (size_t k = 0; k < n.in.size(); ++k) {
+    const PTensor pi = T(tin[k]);
+    if (pi.dt != dt) fail(ODLA_UNSUPPORTED_DATATYPE, "odla_Concat of mixed storage types");
+    const Shape& is = n.in[k]->shape;
+    StridedCopyParams cp;
+    cp.elem_size = es;
+    if (nhwc) {
+      const int64_t pixels = is.d[0] * is.d[2] * is.d[3];
+      cp.rank = 2;
+      cp.dims[0] = pixels; cp.dims[1] = is.d[1];
+      cp.sx[0] = pi.cs; cp.sx[1] = 1;
+      cp.sy[0] = os.d[1]; cp.sy[1] = 1;
+      cp.y_off = off;
+      off += is.d[1];
+    } else {
+      int64_t outer = 1, inner = 1;
+      for (int i = 0; i < axis; ++i) outer *= is.d[i];
+      for (int i = axis + 1; i < is.rank; ++i) inner *= is.d[i];
+      cp.rank = 2;
+      cp.dims[0] = outer; cp.dims[1] = is.d[axis] * inner;
+      cp.sx[0] = is.d[axis] * inner; cp.sx[1] = 1;
+      cp.sy[0] = os.d[axis] * inner; cp.sy[1] = 1;
+      cp.y_off = off;
+      off += is.d[axis] * inner;
+    }
+    // widen to 16-byte elements when everything is aligned
+    const int w = 16 / es;
+    if (cp.dims[1] % w == 0 && cp.sx[0] % w == 0 && cp.sy[0] % w == 0 && cp.y_off % w == 0) {
+      cp.elem_size = 16;
+      cp.dims[1] /= w; cp.sx[0] /= w; cp.sy[0] /= w; cp.y_off /= w;
+    }
+    strided_copy_step("concat:" + n.out->name, tin[k], ty, cp);
+  }
+  set_main(n.out, ty);
+}
+
+// -------------------------------------------------------------- Gather ----
+void Planner::lower_gather(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const _odla_value* idx = n.in[1];
+  const int axis = (int)n.i[0];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const int ti = get(idx, L_ROWMAJOR, FORM_FLOAT);
+  const Shape& xs = x->shape;
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= xs.d[i];
+  for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
+  const DType dt = T(tx).dt;
+  const DType idt = T(ti).dt;
+  const int64_t n_src = xs.d[axis], n_idx = idx->shape.numel();
+  const int64_t row_bytes = inner * dtype_size(dt);
+  const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const Ref a = ref(tx), ri = ref(ti), b = ref(ty);
+  emit("gather:" + n.out->name, {tx, ti}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_gather_rows(a(e), ri(e), idt, b(e), outer, n_src, n_idx, row_bytes, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ------------------------------------------------------------- Reshape ----
+void Planner::lower_reshape(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const VState& s = vs_[x->index];
+  // keep 8-bit data 8-bit through a reshape when it is already row-major
+  int tx;
+  if (s.main >= 0 && T(s.main).quant && s.slot[L_ROWMAJOR][FORM_QUANT] >= 0 && qentry(n.out) != nullptr)
+    tx = s.slot[L_ROWMAJOR][FORM_QUANT];
+  else
+    tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const int ty = alias_tensor(tx, n.out->shape);
+  set_main(n.out, ty);
+}
+
+// -------------------------------------------------------------- Resize ----
+void Planner::lower_resize(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const int tx = get(x, L_NHWC, FORM_FLOAT);
+  const PTensor px = T(tx);
+  const Shape& xs = x->shape;
+  const Shape& os = n.out->shape;
+  const int ty = new_tensor(px.dt, L_NHWC, os, px.cs, SP_ARENA);
+  const int es = dtype_size(px.dt);
+  const int N = (int)xs.d[0], H = (int)xs.d[2], W = (int)xs.d[3], cs = px.cs, Ho = (int)os.d[2], Wo = (int)os.d[3];
+  const Ref a = ref(tx), b = ref(ty);
+  emit("resize:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_resize_nearest_nhwc(a(e), b(e), es, N, H, W, cs, Ho, Wo, st);
+  });
+  set_main(n.out, ty);
+}
+
+// --------------------------------------------------------------- Slice ----
+void Planner::lower_slice(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const Shape& xs = x->shape;
+  const Shape& os = n.out->shape;
+  const int r = xs.rank;
+  if (r > 8) fail(ODLA_UNSUPPORTED_OP, "odla_Slice of rank > 8");
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, os, 0, SP_ARENA);
+  StridedCopyParams cp;
+  cp.elem_size = dtype_size(dt);
+  cp.rank = r;
+  int64_t sx = 1, sy = 1;
+  for (int i = r - 1; i >= 0; --i) {
+    cp.dims[i] = os.d[i];
+    cp.sx[i] = sx * n.iv[2 * r + i];
+    cp.sy[i] = sy;
+    cp.x_off += n.iv[i] * sx;
+    sx *= xs.d[i];
+    sy *= os.d[i];
+  }
+  strided_copy_step("slice:" + n.out->name, tx, ty, cp);
+  set_main(n.out, ty);
+}
+
+// ----------------------------------------------------------- Transpose ----
+void Planner::lower_transpose(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const Shape& os = n.out->shape;
+  const int r = xs.rank;
+  if (r > 8) fail(ODLA_UNSUPPORTED_OP, "odla_Transpose of rank > 8");
+  // N,C,H,W -> N,H,W,C of a value that already lives channels-last is free
+  const VState& s = vs_[x->index];
+  if (r == 4 && n.iv[0] == 0 && n.iv[1] == 2 && n.iv[2] == 3 && n.iv[3] == 1 && s.main >= 0 &&
+      T(s.main).layout == L_NHWC && !T(s.main).quant && T(s.main).cs == xs.d[1]) {
+    set_main(n.out, alias_tensor(s.main, os));
+    return;
+  }
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, os, 0, SP_ARENA);
+  int64_t xstr[ODLA_MAX_DIMENSION];
+  {
+    int64_t acc = 1;
+    for (int i = r - 1; i >= 0; --i) { xstr[i] = acc; acc *= xs.d[i]; }
+  }
+  StridedCopyParams cp;
+  cp.elem_size = dtype_size(dt);
+  cp.rank = r;
+  int64_t sy = 1;
+  for (int i = r - 1; i >= 0; --i) {
+    cp.dims[i] = os.d[i];
+    cp.sx[i] = xstr[n.iv[i]];
+    cp.sy[i] = sy;
+    sy *= os.d[i];
+  }
+  strided_copy_step("transpose:" + n.out->name, tx, ty, cp);
+  set_main(n.out, ty);
+}
+
+// ------------------------------------------------- Quantize/Dequantize ----
+void Planner::lower_qdq(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const bool quant = n.op == OP_QUANTIZE;
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const Shape& xs = x->shape;
+  const int axis = (int)n.i[0];
+  std::vector<float> sc = const_as_float(n.in[1]);
+  std::vector<int32_t> zp;
+  if (n.in[2]) { std::vector<float> z = const_as_float(n.in[2]); for (float v : z) zp.push_back((int32_t)v); }
+  const int channels = (int)sc.size();
+  int64_t inner = 1;
+  if (channels > 1) for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
+  const int ts = const_vector<float>(DT_F32, sc);
+  const int tz = zp.empty() ? -1 : const_vector<int32_t>(DT_I32, zp);
+  const DType odt = storage_dtype(n.out);
+  const int ty = new_tensor(odt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  QuantParams qp;
+  qp.n = xs.numel(); qp.inner = inner; qp.channels = channels;
+  qp.src_dt = T(tx).dt; qp.dst_dt = odt;
+  qp.dst_signed = quant ? (odt == DT_I8) : (T(tx).dt == DT_I8);
+  const Ref a = ref(tx), b = ref(ty), rs = ref(ts), rz = ref(tz >= 0 ? tz : ts);
+  const bool hz = tz >= 0;
+  emit(std::string(quant ? "quantize:" : "dequantize:") + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    QuantParams p = qp; p.src = a(e); p.dst = b(e); p.scale = (const float*)rs(e); p.zp = hz ? (const int32_t*)rz(e) : nullptr;
+    return quant ? launch_quantize(p, st) : launch_dequantize(p, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ----------------------------------------------------------------- NMS ----
+void Planner::lower_nms(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* boxes = n.in[0];
+  const _odla_value* scores = n.in[1];
+  auto as_f32 = [&](const _odla_value* v) -> int {
+    int t = get(v, L_ROWMAJOR, FORM_FLOAT);
+    if (T(t).dt == DT_F32) return t;
+    const int d = new_tensor(DT_F32, L_ROWMAJOR, v->shape, 0, SP_ARENA);
+    const int64_t ne = v->shape.numel();
+    const DType sdt = T(t).dt;
+    const Ref a = ref(t), b = ref(d);
+    emit("nms.cast:" + v->name, {t}, {d}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), DT_F32, ne, st); });
+    return d;
+  };
+  const int tb = as_f32(boxes), ts = as_f32(scores);
+  const int N = (int)boxes->shape.d[0], B = (int)boxes->shape.d[1], C = (int)scores->shape.d[1];
+  const int max_out = (int)n.i[0];
+  const float iou = n.f[0], thr = n.f[1];
+  const int tw = raw_buffer(nms_workspace_bytes(N, B), SP_ARENA);
+  Shape o32 = n.out->shape;
+  const int ty = new_tensor(DT_I32, L_ROWMAJOR, o32, 0, SP_ARENA);
+  const Ref rb = ref(tb), rs = ref(ts), rw = ref(tw), ry = ref(ty);
+  emit("nms:" + n.out->name, {tb, ts, tw}, {ty, tw}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_nms((const float*)rb(e), (const float*)rs(e), N, C, B, max_out, iou, thr, (int32_t*)ry(e), rw(e), st);
+  });
+  if (dtype_from_odla(n.out->etype) == DT_I64) {
+    const int t64 = new_tensor(DT_I64, L_ROWMAJOR, o32, 0, SP_ARENA);
+    const int64_t ne = o32.numel();
+    const Ref c = ref(t64);
+    emit("nms.i64:" + n.out->name, {ty}, {t64}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(ry(e), DT_I32, c(e), DT_I64, ne, st); });
+    set_main(n.out, t64);
+  } else {
+    set_main(n.out, ty);
+  }
+}
+
+}  // namespace
+
+// ============================================================================
+odla_status build_plan(_odla_computation* comp, std::unique_ptr<Plan>* out) {
+  auto plan = std::make_unique<Plan>();
+  // fusion marks are per-plan
+  for (Node& n : comp->nodes) n.absorbed = false;
+  try {
+    Planner p(comp, plan.get());
+    p.run();
+  } catch (const PlanError& e) {
+    OHIP_ERR("cannot compile computation: %s", e.msg.c_str());
+    return e.status;
+  } catch (const std::exception& e) {
+    OHIP_ERR("cannot compile computation: %s", e.what());
+    return ODLA_FAILURE;
+  }
+
+  // ---- constant pool + one-time initialisation steps ----
+  char* init_tmp = nullptr;
+  auto cleanup = [&]() { if (init_tmp) (void)hipFree(init_tmp); };
+  if (plan->const_bytes > 0 &&
+      hipMalloc(reinterpret_cast<void**>(&plan->const_pool), plan->const_bytes) != hipSuccess) {
+    OHIP_ERR("cannot allocate %zu bytes for constants", plan->const_bytes);
+    return ODLA_MEM_ERROR;
+  }
+  if (plan->init_bytes > 0 && hipMalloc(reinterpret_cast<void**>(&init_tmp), plan->init_bytes) != hipSuccess) {
+    OHIP_ERR("cannot allocate %zu bytes of initialisation scratch", plan->init_bytes);
+    return ODLA_MEM_ERROR;
+  }
+  for (const Plan::Blob& b : plan->blobs) {
+    char* base = b.space == SP_CONST ? plan->const_pool : init_tmp;
+    const void* src = b.src ? b.src : b.owned.data();
+    if (hipMemcpy(base + b.offset, src, b.bytes, hipMemcpyHostToDevice) != hipSuccess) {
+      OHIP_ERR("upload of a constant failed");
+      cleanup();
+      return ODLA_FAILURE;
+    }
+  }
+  ExecEnv env;
+  env.base[SP_CONST] = plan->const_pool;
+  env.base[SP_INIT] = init_tmp;
+  for (const Step& s : plan->init_steps) {
+    hipError_t e = s.fn(env, nullptr);
+    if (e != hipSuccess) {
+      OHIP_ERR("initialisation step '%s' failed: %s", s.name.c_str(), hipGetErrorString(e));
+      cleanup();
+      return ODLA_FAILURE;
+    }
+  }
+  if (hipDeviceSynchronize() != hipSuccess) {
+    OHIP_ERR("device error while preparing constants");
+    cleanup();
+    return ODLA_FAILURE;
+  }
+  cleanup();
+  plan->blobs.clear();
+  plan->blobs.shrink_to_fit();
+  plan->init_steps.clear();
+  OHIP_INFO("plan: %zu steps, arena %.1f MiB, constants %.1f MiB", plan->steps.size(),
+            plan->arena_bytes / 1048576.0, plan->const_bytes / 1048576.0);
+  *out = std::move(plan);
+  return ODLA_SUCCESS;
+}
+
+}  // namespace ohip

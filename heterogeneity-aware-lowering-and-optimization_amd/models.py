@@ -1,0 +1,125 @@
+"""Graph descriptions of the benchmark configurations, written once against the
+builder vocabulary shared by ``HipBuilder`` (GPU, through the ODLA C ABI) and
+the CPU oracle's ``RefBuilder``.
+
+Every ``build_*`` function takes a builder and a dict of weights (numpy) and
+emits the same ODLA call sequence HALO-generated code would emit for the model:
+``odla_CreateArgument`` / ``odla_CreateConstant`` / ``odla_<Op>`` /
+``odla_SetValueAsOutput``.  Weights are synthetic (seeded), shaped like the
+real architectures.
+"""
+import numpy as np
+
+
+# ---------------------------------------------------------------------------
+# C0: softmax regression of the reference's mnist_simple graph
+#     (Gemm + Add + Softmax; docs/mnist_sample.md:22-56 of the reference tree)
+# ---------------------------------------------------------------------------
+def mnist_weights(seed=42):
+    rng = np.random.default_rng(seed)
+    return {"V": (rng.standard_normal((784, 10)) * 0.05).astype(np.float32),
+            "V1": np.zeros((1, 10), np.float32)}
+
+
+def mnist_input(batch=64, seed=1234):
+    rng = np.random.default_rng(seed)
+    return {"x": rng.random((batch, 784), dtype=np.float32)}
+
+
+def build_mnist(b, w, batch=64):
+    x = b.arg("x", (batch, 784))
+    V = b.const("V", w["V"])
+    V1 = b.const("V1", w["V1"])
+    mm = b.gemm(x, V, None, False, False, 1.0, 0.0, name="MatMul")
+    add = b.add(mm, V1, name="add")
+    y = b.softmax(add, -1, name="y")
+    b.output(y, "y")
+
+
+# ---------------------------------------------------------------------------
+# C1 / C2: ResNet-50 v1.5 (stride 2 on the 3x3 of each down-sampling bottleneck),
+# BatchNorm folded into the convolutions (gamma 1, beta 0, mean 0, var 1).
+# ---------------------------------------------------------------------------
+RESNET50_STAGES = [(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)]
+BN_EPS = 1e-5
+
+
+def resnet50_conv_specs(stages=RESNET50_STAGES, stem=64):
+    """[(name, cout, cin, k, stride, pad)] in execution order."""
+    specs = [("stem", stem, 3, 7, 2, 3)]
+    cin = stem
+    for si, (mid, blocks, stride) in enumerate(stages):
+        cout = mid * 4
+        for bi in range(blocks):
+            s = stride if bi == 0 else 1
+            p = "l%db%d" % (si + 1, bi)
+            if bi == 0:
+                specs.append((p + "ds", cout, cin, 1, s, 0))
+            specs.append((p + "c1", mid, cin, 1, 1, 0))
+            specs.append((p + "c2", mid, mid, 3, s, 1))
+            specs.append((p + "c3", cout, mid, 1, 1, 0))
+            cin = cout
+    return specs
+
+
+def resnet50_weights(seed=42, num_classes=1000, stages=RESNET50_STAGES, stem=64):
+    """He-normal conv weights with the identity BatchNorm folded in."""
+    rng = np.random.default_rng(seed)
+    w = {}
+    fold = np.float32(1.0 / np.sqrt(np.float32(1.0) + np.float32(BN_EPS)))
+    for name, cout, cin, k, _, _ in resnet50_conv_specs(stages, stem):
+        std = np.sqrt(2.0 / (cin * k * k))
+        w[name + ".w"] = (rng.standard_normal((cout, cin, k, k)).astype(np.float32) * np.float32(std) * fold)
+        w[name + ".b"] = np.zeros(cout, np.float32)
+    feat = stages[-1][0] * 4
+    w["fc.w"] = (rng.standard_normal((feat, num_classes)) * np.sqrt(1.0 / feat)).astype(np.float32)
+    w["fc.b"] = np.zeros(num_classes, np.float32)
+    return w
+
+
+def resnet50_input(batch, hw=224, seed=1234):
+    rng = np.random.default_rng(seed)
+    return {"input": rng.standard_normal((batch, 3, hw, hw), dtype=np.float32)}
+
+
+def build_resnet50(b, w, batch, hw=224, stages=RESNET50_STAGES, stem=64, num_classes=1000,
+                   with_softmax=True, taps=None):
+    """`taps`: optional list that receives (name, value) of every named
+    activation in execution order (used for calibration / per-layer parity)."""
+    def tap(name, v):
+        if taps is not None:
+            taps.append((name, v))
+        return v
+
+    def conv(x, name, k, stride, pad, relu):
+        y = b.conv(x, b.const(name + ".w", w[name + ".w"]), b.const(name + ".b", w[name + ".b"]),
+                   (stride, stride), (pad, pad, pad, pad), name=name)
+        tap(name, y)
+        if relu:
+            y = tap(name + ".relu", b.relu(y, name=name + ".relu"))
+        return y
+
+    x = tap("input", b.arg("input", (batch, 3, hw, hw)))
+    x = conv(x, "stem", 7, 2, 3, True)
+    x = tap("pool1", b.maxpool(x, (3, 3), (2, 2), (1, 1, 1, 1), name="pool1"))
+    for si, (mid, blocks, stride) in enumerate(stages):
+        for bi in range(blocks):
+            s = stride if bi == 0 else 1
+            p = "l%db%d" % (si + 1, bi)
+            identity = conv(x, p + "ds", 1, s, 0, False) if bi == 0 else x
+            y = conv(x, p + "c1", 1, 1, 0, True)
+            y = conv(y, p + "c2", 3, s, 1, True)
+            y = conv(y, p + "c3", 1, 1, 0, False)
+            y = tap(p + "add", b.add(y, identity, name=p + "add"))
+            x = tap(p + "out", b.relu(y, name=p + "out"))
+    x = tap("gap", b.reduce_mean(x, (2, 3), True, name="gap"))
+    feat = stages[-1][0] * 4
+    x = b.reshape(x, (batch, feat), name="flat")
+    logits = tap("logits", b.gemm(x, b.const("fc.w", w["fc.w"]), b.const("fc.b", w["fc.b"]), False, False, 1.0, 1.0,
+                                  name="logits"))
+    b.output(logits, "logits")
+    if with_softmax:
+        b.output(b.softmax(logits, -1, name="prob"), "prob")
+
+
+RESNET50_GFLOP_PER_IMAGE = 2 * (4087136256 + 2048000) / 1e9   # conv + FC multiply-adds, x2

@@ -1,0 +1,487 @@
+"""ctypes host side of libodla_hip.so.
+
+Mirrors what the reference's Python harness does through ctypes
+(python/halo/odla.py:54-176 of the reference tree): create a computation,
+build the graph by calling the ``odla_<Op>`` builders exactly as HALO-generated
+C code would, create a context, bind numpy buffers, execute.  Enumerator values
+are taken from include/odla_hip.h (the reference harness's own integer
+constants are stale with respect to its headers).
+
+``HipBuilder`` exposes one method per ODLA operator; model descriptions written
+against it can be replayed on the CPU oracle, which offers the same methods.
+The library is required: there is no CPU fallback on this side.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libodla_hip.so")
+
+# ---- enums (include/odla_hip.h) ---------------------------------------------
+(ODLA_INT8, ODLA_INT16, ODLA_INT32, ODLA_INT64, ODLA_UINT8, ODLA_UINT16, ODLA_UINT32, ODLA_UINT64,
+ ODLA_QINT8, ODLA_QINT16, ODLA_QINT32, ODLA_QINT64, ODLA_QUINT8, ODLA_QUINT16, ODLA_QUINT32,
+ ODLA_QUINT64, ODLA_FLOAT16, ODLA_BFLOAT16, ODLA_FLOAT32, ODLA_FLOAT64, ODLA_BOOL, ODLA_STRING) = range(22)
+ODLA_SUCCESS = 0
+ODLA_INVALID_PARAM = 3
+ODLA_COMPUTE_INFERENCE = 1
+(ODLA_DYNAMIC_BATCH, ODLA_MIN_BATCH_SIZE, ODLA_MAX_BATCH_SIZE, ODLA_OPT_BATCH_SIZE, ODLA_RUN_BATCH_SIZE,
+ ODLA_DYNAMIC_SHAPE, ODLA_MIN_SHAPE, ODLA_MAX_SHAPE, ODLA_OPT_SHAPE, ODLA_DYNAMIC_VALUE, ODLA_MIN_VALUE,
+ ODLA_MAX_VALUE, ODLA_OPT_VALUE, ODLA_BF16_MODE, ODLA_FP16_MODE, ODLA_USE_SIM_MODE, ODLA_PROCESSOR_NUM,
+ ODLA_BATCHES_PER_STEP, ODLA_USE_DATA_TYPE, ODLA_LOAD_ENGINE_MODE, ODLA_USE_DLA_CORE, ODLA_QUANT_TABLE,
+ ODLA_QUANT_TABLE_SIZE, ODLA_AGGREGATE_OPS, ODLA_ENABLE_ENGINE_CACHE, ODLA_CACHE_DIR,
+ ODLA_ASYNC_CALLBACK_FUNC, ODLA_ASYNC_CALLBACK_ARG) = range(28)
+ODLA_HIP_ITEM_RAW_INT32_ACC = 1000
+BF16_DISABLE, BF16_ACCURACY_MODE, BF16_PERFORMACE_MODE, BF16_AUTO_MODE = range(4)
+ODLA_CHANNELS_FIRST, ODLA_CHANNELS_LAST, ODLA_SIO, ODLA_SOI, ODLA_OIS, ODLA_IOS = range(6)
+ODLA_NEAREST, ODLA_LINEAR, ODLA_CUBIC = range(3)
+ODLA_ASSYMMETRIC = 0
+ODLA_MEMCPY_H2H, ODLA_MEMCPY_H2D, ODLA_MEMCPY_D2H, ODLA_MEMCPY_D2D = range(4)
+
+ODLA_MAX_DIMENSION = 10
+ODLA_MAX_OUTPUTS = 64
+
+_NP_TO_ODLA = {
+    np.dtype(np.float32): ODLA_FLOAT32, np.dtype(np.float16): ODLA_FLOAT16,
+    np.dtype(np.int32): ODLA_INT32, np.dtype(np.int64): ODLA_INT64,
+    np.dtype(np.int8): ODLA_INT8, np.dtype(np.uint8): ODLA_UINT8, np.dtype(np.bool_): ODLA_BOOL,
+}
+_ODLA_TO_NP = {v: k for k, v in _NP_TO_ODLA.items()}
+
+
+class ValueShape(ctypes.Structure):
+    _fields_ = [("size", ctypes.c_int32), ("dims", ctypes.c_int64 * ODLA_MAX_DIMENSION)]
+
+
+class ValueType(ctypes.Structure):
+    _fields_ = [("element_type", ctypes.c_int32), ("shape", ValueShape)]
+
+
+class Values(ctypes.Structure):
+    _fields_ = [("size", ctypes.c_size_t), ("values", ctypes.c_void_p * ODLA_MAX_OUTPUTS)]
+
+
+class QuantInfo(ctypes.Structure):
+    _fields_ = [("value_id", ctypes.c_char_p), ("ch_idx", ctypes.c_int), ("scale", ctypes.c_float),
+                ("offset", ctypes.c_float), ("min", ctypes.c_float), ("max", ctypes.c_float)]
+
+
+assert ctypes.sizeof(ValueShape) == 88 and ctypes.sizeof(ValueType) == 96
+assert ctypes.sizeof(Values) == 520 and ctypes.sizeof(QuantInfo) == 32
+
+
+def make_shape(dims):
+    s = ValueShape()
+    s.size = len(dims)
+    for i, d in enumerate(dims):
+        s.dims[i] = int(d)
+    return s
+
+
+def undefined_shape():
+    s = ValueShape()
+    s.size = -1
+    return s
+
+
+def make_type(np_dtype, dims):
+    t = ValueType()
+    t.element_type = _NP_TO_ODLA[np.dtype(np_dtype)]
+    t.shape = make_shape(dims)
+    return t
+
+
+_lib = None
+
+
+def load_library(path=None):
+    """Load libodla_hip.so and declare the prototypes of include/odla_hip.h."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    path = path or LIB_PATH
+    if not os.path.exists(path):
+        raise RuntimeError("%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`" % path)
+    L = ctypes.CDLL(path)
+    vp, u32, i32, f32, sz = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int32, ctypes.c_float, ctypes.c_size_t
+    pu32 = ctypes.POINTER(ctypes.c_uint32)
+    pi32 = ctypes.POINTER(ctypes.c_int32)
+    cid = ctypes.c_char_p
+    S, T = ValueShape, ValueType
+
+    def proto(name, res, args):
+        f = getattr(L, name)
+        f.restype = res
+        f.argtypes = args
+
+    proto("odla_CreateComputation", i32, [ctypes.POINTER(vp)])
+    proto("odla_DestroyComputation", i32, [vp])
+    proto("odla_SetComputationItem", i32, [vp, i32, vp])
+    proto("odla_CreateContext", i32, [ctypes.POINTER(vp)])
+    proto("odla_DestroyContext", i32, [vp])
+    proto("odla_SetContextItem", i32, [vp, i32, vp])
+    proto("odla_BindToArgument", i32, [vp, vp, vp])
+    proto("odla_BindToArgumentById", i32, [cid, vp, vp])
+    proto("odla_BindToOutput", i32, [vp, vp, vp])
+    proto("odla_BindToOutputById", i32, [cid, vp, vp])
+    proto("odla_ExecuteComputation", i32, [vp, vp, i32, vp])
+    proto("odla_GetNumOfArgsFromComputation", i32, [vp, pu32])
+    proto("odla_GetArgFromComputationByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
+    proto("odla_GetNumOfOutputsFromComputation", i32, [vp, pu32])
+    proto("odla_GetOutputFromComputationByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
+    proto("odla_GetRuntimeShape", i32, [vp, vp, ctypes.POINTER(S)])
+    proto("odla_GetValueType", i32, [vp, ctypes.POINTER(T)])
+    proto("odla_GetValueId", i32, [vp, ctypes.POINTER(cid)])
+    proto("odla_FindValueById", i32, [cid, ctypes.POINTER(vp)])
+    proto("odla_SetValueAsOutput", i32, [vp])
+    proto("odla_SetValuesAsOutput", i32, [Values])
+    proto("odla_SetValueAsOutputById", i32, [cid])
+    proto("odla_GetValueData", i32, [vp, vp, vp])
+    proto("odla_ReleaseValue", i32, [vp])
+    proto("odla_CreateArgument", vp, [T, cid])
+    proto("odla_CreateConstant", vp, [T, vp, cid])
+    proto("odla_AllocateDevice", i32, [vp, i32, i32, ctypes.POINTER(vp)])
+    proto("odla_GetDeviceInfo", i32, [vp, i32, vp])
+    proto("odla_SetCurrentDevice", i32, [vp])
+    proto("odla_DestroyDevice", i32, [vp])
+    proto("odla_AllocateDeviceMemory", i32, [ctypes.POINTER(vp), sz])
+    proto("odla_FreeDeviceMemory", i32, [vp])
+    proto("odla_AllocateHostMemory", i32, [ctypes.POINTER(vp), sz])
+    proto("odla_FreeHostMemory", i32, [vp])
+    proto("odla_CopyMemory", i32, [vp, vp, sz, i32])
+    proto("odla_SetLogLevel", i32, [i32])
+    proto("odla_SetLogger", i32, [vp])
+    proto("odla_GetLogger", vp, [])
+    proto("odla_GetVersionString", ctypes.c_char_p, [])
+
+    proto("odla_Conv", vp, [vp, i32, u32, vp, i32, pu32, pu32, pu32, pu32, vp, S, cid])
+    proto("odla_Gemm", vp, [vp, u32, vp, u32, f32, f32, vp, S, cid])
+    proto("odla_BatchMatMul", vp, [vp, u32, vp, u32, S, cid])
+    for n in ("Add", "Sub", "Mul", "Div", "Max", "Min"):
+        proto("odla_" + n, vp, [vp, vp, cid])
+    for n in ("Relu", "Sigmoid", "Tanh", "Exp", "Log", "Sqrt", "Rsqrt", "Erf", "Abs", "Neg", "Round"):
+        proto("odla_" + n, vp, [vp, cid])
+    proto("odla_LeakyRelu", vp, [vp, f32, cid])
+    proto("odla_Clamp", vp, [vp, f32, f32, cid])
+    proto("odla_Gelu", vp, [vp, u32, cid])
+    proto("odla_BatchNormalization", vp, [vp, i32, vp, vp, f32, vp, vp, f32, f32, cid])
+    proto("odla_LayerNorm", vp, [vp, sz, pi32, f32, vp, vp, cid])
+    proto("odla_MaxPool", vp, [vp, i32, pu32, pu32, pu32, pu32, S, cid])
+    proto("odla_AveragePool", vp, [vp, i32, pu32, pu32, pu32, pu32, u32, S, cid])
+    for n in ("ReduceMean", "ReduceSum", "ReduceMax"):
+        proto("odla_" + n, vp, [vp, sz, pu32, u32, S, cid])
+    proto("odla_Softmax", vp, [vp, i32, cid])
+    proto("odla_LogSoftmax", vp, [vp, i32, cid])
+    proto("odla_Cast", vp, [vp, i32, cid])
+    proto("odla_Concat", vp, [Values, i32, S, cid])
+    proto("odla_Gather", vp, [vp, vp, i32, S, cid])
+    proto("odla_Reshape", vp, [vp, S, cid])
+    proto("odla_Resize", vp, [vp, i32, i32, u32, S, cid])
+    proto("odla_Slice", vp, [vp, pi32, pi32, pi32, S, cid])
+    proto("odla_Transpose", vp, [vp, S, S, cid])
+    proto("odla_Quantize", vp, [vp, vp, vp, i32, i32, cid])
+    proto("odla_Dequantize", vp, [vp, vp, vp, i32, i32, cid])
+    proto("odla_NMS", vp, [vp, vp, u32, f32, f32, T, cid])
+    if path == LIB_PATH:
+        _lib = L
+    return L
+
+
+def exported_symbols_declared_in_header():
+    """Names of all functions declared in include/odla_hip.h."""
+    import re
+    hdr = os.path.join(os.path.dirname(_HERE), "include", "odla_hip.h")
+    text = open(hdr).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(odla_[A-Z]\w*)\s*\(", text)))
+
+
+def _u32(vals):
+    return (ctypes.c_uint32 * len(vals))(*[int(v) for v in vals])
+
+
+def _i32(vals):
+    return (ctypes.c_int32 * len(vals))(*[int(v) for v in vals])
+
+
+def _cid(name):
+    return name.encode() if name else None
+
+
+class OdlaError(RuntimeError):
+    pass
+
+
+def _check(st, what):
+    if st != ODLA_SUCCESS:
+        raise OdlaError("%s failed with odla_status %d" % (what, st))
+
+
+class HipBuilder:
+    """Builds an ODLA computation on libodla_hip.so; one method per operator."""
+
+    def __init__(self, fp16=False, bf16=False, quant_table=None, raw_acc=False, lib=None):
+        self.L = lib or load_library()
+        self.comp = ctypes.c_void_p()
+        _check(self.L.odla_CreateComputation(ctypes.byref(self.comp)), "odla_CreateComputation")
+        self._keep = []      # numpy arrays / ctypes objects that must outlive the computation
+        self.args = {}       # name -> (handle, shape, dtype)
+        self.outs = {}       # name -> (handle, shape, dtype)
+        self._shapes = {}    # handle value -> tuple shape (for convenience)
+        if fp16:
+            b = ctypes.c_bool(True)
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_FP16_MODE, ctypes.byref(b)), "FP16_MODE")
+        if bf16:
+            m = ctypes.c_int32(BF16_PERFORMACE_MODE)
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_BF16_MODE, ctypes.byref(m)), "BF16_MODE")
+        if quant_table is not None:
+            tbl = (QuantInfo * len(quant_table))(*quant_table)
+            n = ctypes.c_int(len(quant_table))
+            t = ctypes.c_int32(ODLA_INT8)
+            self._keep += [tbl, n, t, quant_table]
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_QUANT_TABLE, ctypes.cast(tbl, ctypes.c_void_p)), "QUANT_TABLE")
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_QUANT_TABLE_SIZE, ctypes.byref(n)), "QUANT_TABLE_SIZE")
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_USE_DATA_TYPE, ctypes.byref(t)), "USE_DATA_TYPE")
+        if raw_acc:
+            b = ctypes.c_bool(True)
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_HIP_ITEM_RAW_INT32_ACC, ctypes.byref(b)), "RAW_ACC")
+
+    # -- helpers --
+    def _ret(self, h, what):
+        if not h:
+            raise OdlaError("%s returned NULL (see the library log)" % what)
+        return h
+
+    def shape_of(self, h):
+        t = ValueType()
+        _check(self.L.odla_GetValueType(h, ctypes.byref(t)), "odla_GetValueType")
+        return tuple(t.shape.dims[i] for i in range(t.shape.size)), _ODLA_TO_NP[t.element_type]
+
+    # -- graph inputs --
+    def arg(self, name, shape, dtype=np.float32):
+        h = self._ret(self.L.odla_CreateArgument(make_type(dtype, shape), _cid(name)), "odla_CreateArgument")
+        self.args[name] = (h, tuple(shape), np.dtype(dtype))
+        return h
+
+    def const(self, name, array):
+        a = np.ascontiguousarray(array)
+        self._keep.append(a)
+        shape = a.shape if a.ndim > 0 else ()
+        return self._ret(self.L.odla_CreateConstant(make_type(a.dtype, shape), a.ctypes.data_as(ctypes.c_void_p),
+                                                    _cid(name)), "odla_CreateConstant")
+
+    def output(self, v, name):
+        _check(self.L.odla_SetValueAsOutput(v), "odla_SetValueAsOutput")
+        shape, dt = self.shape_of(v)
+        self.outs[name] = (v, shape, np.dtype(dt))
+
+    # -- operators --
+    def conv(self, x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), group=1, name=None):
+        return self._ret(self.L.odla_Conv(x, ODLA_CHANNELS_FIRST, group, w, ODLA_OIS, _u32(stride), _u32(dilation),
+                                          _u32(pad[:2]), _u32(pad[2:]), bias, undefined_shape(), _cid(name)), "odla_Conv")
+
+    def gemm(self, a, b, c=None, ta=False, tb=False, alpha=1.0, beta=1.0, name=None):
+        return self._ret(self.L.odla_Gemm(a, int(ta), b, int(tb), alpha, beta, c, undefined_shape(), _cid(name)), "odla_Gemm")
+
+    def _bin(self, fn, a, b, name):
+        return self._ret(getattr(self.L, "odla_" + fn)(a, b, _cid(name)), "odla_" + fn)
+
+    def add(self, a, b, name=None): return self._bin("Add", a, b, name)
+    def sub(self, a, b, name=None): return self._bin("Sub", a, b, name)
+    def mul(self, a, b, name=None): return self._bin("Mul", a, b, name)
+    def div(self, a, b, name=None): return self._bin("Div", a, b, name)
+    def max(self, a, b, name=None): return self._bin("Max", a, b, name)
+    def min(self, a, b, name=None): return self._bin("Min", a, b, name)
+
+    def _un(self, fn, x, name):
+        return self._ret(getattr(self.L, "odla_" + fn)(x, _cid(name)), "odla_" + fn)
+
+    def relu(self, x, name=None): return self._un("Relu", x, name)
+    def sigmoid(self, x, name=None): return self._un("Sigmoid", x, name)
+    def tanh(self, x, name=None): return self._un("Tanh", x, name)
+    def exp(self, x, name=None): return self._un("Exp", x, name)
+    def log(self, x, name=None): return self._un("Log", x, name)
+    def sqrt(self, x, name=None): return self._un("Sqrt", x, name)
+    def rsqrt(self, x, name=None): return self._un("Rsqrt", x, name)
+    def erf(self, x, name=None): return self._un("Erf", x, name)
+    def abs(self, x, name=None): return self._un("Abs", x, name)
+    def neg(self, x, name=None): return self._un("Neg", x, name)
+    def round(self, x, name=None): return self._un("Round", x, name)
+
+    def leaky_relu(self, x, alpha, name=None):
+        return self._ret(self.L.odla_LeakyRelu(x, alpha, _cid(name)), "odla_LeakyRelu")
+
+    def clamp(self, x, lo, hi, name=None):
+        return self._ret(self.L.odla_Clamp(x, lo, hi, _cid(name)), "odla_Clamp")
+
+    def gelu(self, x, approx=False, name=None):
+        return self._ret(self.L.odla_Gelu(x, int(approx), _cid(name)), "odla_Gelu")
+
+    def batchnorm(self, x, mean, var, eps, scale=None, offset=None, scalar_scale=1.0, scalar_offset=0.0, name=None):
+        return self._ret(self.L.odla_BatchNormalization(x, ODLA_CHANNELS_FIRST, mean, var, eps, scale, offset,
+                                                        scalar_scale, scalar_offset, _cid(name)), "odla_BatchNormalization")
+
+    def layernorm(self, x, n_axes, eps, scale=None, offset=None, name=None):
+        axes = _i32([-(i + 1) for i in range(n_axes)][::-1])
+        return self._ret(self.L.odla_LayerNorm(x, n_axes, axes, eps, scale, offset, _cid(name)), "odla_LayerNorm")
+
+    def maxpool(self, x, window, stride, pad, out_hw=None, name=None):
+        od = undefined_shape()
+        if out_hw is not None:
+            s, _ = self.shape_of(x)
+            od = make_shape([s[0], s[1], out_hw[0], out_hw[1]])
+        return self._ret(self.L.odla_MaxPool(x, ODLA_CHANNELS_FIRST, _u32(window), _u32(stride), _u32(pad[:2]),
+                                             _u32(pad[2:]), od, _cid(name)), "odla_MaxPool")
+
+    def avgpool(self, x, window, stride, pad, count_include_pad=False, out_hw=None, name=None):
+        od = undefined_shape()
+        if out_hw is not None:
+            s, _ = self.shape_of(x)
+            od = make_shape([s[0], s[1], out_hw[0], out_hw[1]])
+        return self._ret(self.L.odla_AveragePool(x, ODLA_CHANNELS_FIRST, _u32(window), _u32(stride), _u32(pad[:2]),
+                                                 _u32(pad[2:]), int(count_include_pad), od, _cid(name)), "odla_AveragePool")
+
+    def _reduce(self, fn, x, axes, keep_dims, name):
+        return self._ret(getattr(self.L, "odla_" + fn)(x, len(axes), _u32(axes), int(keep_dims), undefined_shape(),
+                                                       _cid(name)), "odla_" + fn)
+
+    def reduce_mean(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceMean", x, axes, keep_dims, name)
+    def reduce_sum(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceSum", x, axes, keep_dims, name)
+    def reduce_max(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceMax", x, axes, keep_dims, name)
+
+    def softmax(self, x, axis=-1, log=False, name=None):
+        f = self.L.odla_LogSoftmax if log else self.L.odla_Softmax
+        return self._ret(f(x, axis, _cid(name)), "odla_Softmax")
+
+    def cast(self, x, dtype, name=None):
+        return self._ret(self.L.odla_Cast(x, _NP_TO_ODLA[np.dtype(dtype)], _cid(name)), "odla_Cast")
+
+    def concat(self, xs, axis, name=None):
+        vs = Values()
+        vs.size = len(xs)
+        for i, v in enumerate(xs):
+            vs.values[i] = v
+        return self._ret(self.L.odla_Concat(vs, axis, undefined_shape(), _cid(name)), "odla_Concat")
+
+    def gather(self, x, idx, axis=0, name=None):
+        return self._ret(self.L.odla_Gather(x, idx, axis, undefined_shape(), _cid(name)), "odla_Gather")
+
+    def reshape(self, x, shape, name=None):
+        return self._ret(self.L.odla_Reshape(x, make_shape(shape), _cid(name)), "odla_Reshape")
+
+    def transpose(self, x, perm, name=None):
+        return self._ret(self.L.odla_Transpose(x, make_shape(perm), undefined_shape(), _cid(name)), "odla_Transpose")
+
+    def slice(self, x, start, end, stride=None, name=None):
+        stride = stride or [1] * len(start)
+        return self._ret(self.L.odla_Slice(x, _i32(start), _i32(end), _i32(stride), undefined_shape(), _cid(name)), "odla_Slice")
+
+    def resize_nearest(self, x, out_hw, name=None):
+        s, _ = self.shape_of(x)
+        return self._ret(self.L.odla_Resize(x, ODLA_NEAREST, ODLA_ASSYMMETRIC, 0,
+                                            make_shape([s[0], s[1], out_hw[0], out_hw[1]]), _cid(name)), "odla_Resize")
+
+    def quantize(self, x, scale, zp=None, axis=-1, signed=False, name=None):
+        sc = self.const(None, np.asarray(scale, np.float32).reshape(-1))
+        z = None if zp is None else self.const(None, np.asarray(zp, np.int8 if signed else np.uint8).reshape(-1))
+        return self._ret(self.L.odla_Quantize(x, sc, z, axis, ODLA_INT8 if signed else ODLA_UINT8, _cid(name)), "odla_Quantize")
+
+    def dequantize(self, q, scale, zp=None, axis=-1, name=None, zp_dtype=np.uint8):
+        sc = self.const(None, np.asarray(scale, np.float32).reshape(-1))
+        z = None if zp is None else self.const(None, np.asarray(zp, zp_dtype).reshape(-1))
+        return self._ret(self.L.odla_Dequantize(q, sc, z, axis, ODLA_FLOAT32, _cid(name)), "odla_Dequantize")
+
+    def nms(self, boxes, scores, max_out, iou_thr, score_thr, name=None):
+        return self._ret(self.L.odla_NMS(boxes, scores, max_out, iou_thr, score_thr, make_type(np.int32, [1]), _cid(name)), "odla_NMS")
+
+    # -- execution --
+    def session(self, use_graph=True):
+        return Session(self, use_graph)
+
+    def destroy(self):
+        if self.comp:
+            self.L.odla_DestroyComputation(self.comp)
+            self.comp = None
+
+
+class Session:
+    """One odla_context: bind numpy (host) or device buffers, execute."""
+
+    def __init__(self, builder, use_graph=True):
+        self.b = builder
+        self.L = builder.L
+        self.ctx = ctypes.c_void_p()
+        _check(self.L.odla_CreateContext(ctypes.byref(self.ctx)), "odla_CreateContext")
+        if not use_graph:
+            f = ctypes.c_bool(False)
+            _check(self.L.odla_SetContextItem(self.ctx, ODLA_AGGREGATE_OPS, ctypes.byref(f)), "AGGREGATE_OPS")
+        self._dev = []
+
+    def run(self, feeds):
+        """feeds: name -> numpy array.  Returns name -> numpy array."""
+        keep = []
+        for name, (h, shape, dt) in self.b.args.items():
+            a = np.ascontiguousarray(feeds[name], dtype=dt)
+            assert tuple(a.shape) == shape, (name, a.shape, shape)
+            keep.append(a)
+            _check(self.L.odla_BindToArgument(h, a.ctypes.data_as(ctypes.c_void_p), self.ctx), "odla_BindToArgument")
+        outs = {}
+        for name, (h, shape, dt) in self.b.outs.items():
+            o = np.empty(shape, dt)
+            outs[name] = o
+            _check(self.L.odla_BindToOutput(h, o.ctypes.data_as(ctypes.c_void_p), self.ctx), "odla_BindToOutput")
+        _check(self.L.odla_ExecuteComputation(self.b.comp, self.ctx, ODLA_COMPUTE_INFERENCE, None), "odla_ExecuteComputation")
+        return outs
+
+    def bind_device_io(self, feeds):
+        """Copy `feeds` into device memory once and bind device buffers for every
+        argument and output, so that execute() moves no data across PCIe."""
+        self.dev_out = {}
+        for name, (h, shape, dt) in self.b.args.items():
+            a = np.ascontiguousarray(feeds[name], dtype=dt)
+            p = ctypes.c_void_p()
+            _check(self.L.odla_AllocateDeviceMemory(ctypes.byref(p), a.nbytes), "odla_AllocateDeviceMemory")
+            _check(self.L.odla_CopyMemory(p, a.ctypes.data_as(ctypes.c_void_p), a.nbytes, ODLA_MEMCPY_H2D), "odla_CopyMemory")
+            self._dev.append(p)
+            _check(self.L.odla_BindToArgument(h, p, self.ctx), "odla_BindToArgument")
+        for name, (h, shape, dt) in self.b.outs.items():
+            nbytes = int(np.prod(shape)) * dt.itemsize
+            p = ctypes.c_void_p()
+            _check(self.L.odla_AllocateDeviceMemory(ctypes.byref(p), nbytes), "odla_AllocateDeviceMemory")
+            self._dev.append(p)
+            self.dev_out[name] = (p, shape, dt)
+            _check(self.L.odla_BindToOutput(h, p, self.ctx), "odla_BindToOutput")
+
+    def execute(self):
+        _check(self.L.odla_ExecuteComputation(self.b.comp, self.ctx, ODLA_COMPUTE_INFERENCE, None), "odla_ExecuteComputation")
+
+    def fetch_device_outputs(self):
+        outs = {}
+        for name, (p, shape, dt) in self.dev_out.items():
+            o = np.empty(shape, dt)
+            _check(self.L.odla_CopyMemory(o.ctypes.data_as(ctypes.c_void_p), p, o.nbytes, ODLA_MEMCPY_D2H), "odla_CopyMemory")
+            outs[name] = o
+        return outs
+
+    def close(self):
+        for p in self._dev:
+            self.L.odla_FreeDeviceMemory(p)
+        self._dev = []
+        if self.ctx:
+            self.L.odla_DestroyContext(self.ctx)
+            self.ctx = None
+
+
+def quant_table(entries):
+    """entries: list of (name, scale, zero_point, min, max, channel_minmax or None).
+    Emits records in the reference writer's format (utils/halo_pgq.py:308-332):
+    one tensor record with ch_idx = -channels, then one record per channel."""
+    recs = []
+    for name, scale, zp, mn, mx, ch in entries:
+        nch = len(ch) if ch is not None else 1
+        recs.append(QuantInfo(name.encode(), -nch, float(scale), float(zp), float(mn), float(mx)))
+        if ch is not None:
+            for c, (cmn, cmx) in enumerate(ch):
+                recs.append(QuantInfo(name.encode(), c, 0.0, 0.0, float(cmn), float(cmx)))
+    return recs

@@ -1,0 +1,535 @@
+/*
+ * odla_hip.h -- C ABI of libodla_hip.so, an ODLA runtime platform for one AMD
+ * Instinct MI355X (gfx950).
+ *
+ * The library is a drop-in ODLA backend: model code emitted by the HALO
+ * compiler (or any program written against ODLA/include/ODLA/*.h of the
+ * reference tree) links against it in place of libodla_dnnl.so /
+ * libodla_tensorrt.so.  Every type below is binary compatible with the
+ * reference declaration it cites (x86-64 SysV): enumerator order, struct
+ * member order and sizes are part of the ABI and must not change.
+ *
+ * Citations of the form  [ref: <file>:<line>]  name the reference interface a
+ * declaration replaces; paths are relative to the reference tree root.
+ *
+ * All functions are plain C symbols with default visibility.  Control
+ * functions return odla_status (ODLA_SUCCESS == 0); graph builders return an
+ * odla_value handle, or NULL after logging the reason when the request is
+ * malformed or unsupported.  No C++ exception crosses this boundary.
+ */
+#ifndef ODLA_HIP_H_
+#define ODLA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* Scalar and handle types                [ref: ODLA/include/ODLA/odla_common.h:63-137] */
+/* ------------------------------------------------------------------------ */
+typedef int8_t odla_int8;
+typedef int16_t odla_int16;
+typedef int32_t odla_int32;
+typedef int64_t odla_int64;
+typedef uint8_t odla_uint8;
+typedef uint16_t odla_uint16;
+typedef uint32_t odla_uint32;
+typedef uint64_t odla_uint64;
+typedef uint16_t odla_float16;  /* IEEE binary16 bit pattern */
+typedef uint16_t odla_bfloat16; /* bfloat16 bit pattern      */
+typedef float odla_float32;
+typedef double odla_float64;
+typedef const char* odla_string;
+typedef odla_uint32 odla_bool;
+typedef char odla_char;
+typedef size_t odla_size_t;
+typedef void odla_void;
+
+/* Element types.                          [ref: ODLA/include/ODLA/odla_common.h:102-128] */
+typedef enum {
+  ODLA_INT8, ODLA_INT16, ODLA_INT32, ODLA_INT64,
+  ODLA_UINT8, ODLA_UINT16, ODLA_UINT32, ODLA_UINT64,
+  ODLA_QINT8, ODLA_QINT16, ODLA_QINT32, ODLA_QINT64,
+  ODLA_QUINT8, ODLA_QUINT16, ODLA_QUINT32, ODLA_QUINT64,
+  ODLA_FLOAT16, ODLA_BFLOAT16, ODLA_FLOAT32, ODLA_FLOAT64,
+  ODLA_BOOL, ODLA_STRING
+} odla_element_type;
+
+/* Status codes.                           [ref: ODLA/include/ODLA/odla_common.h:140-165] */
+typedef enum {
+  ODLA_SUCCESS,
+  ODLA_DL_ERROR,
+  ODLA_FILE_NOT_EXIST,
+  ODLA_INVALID_PARAM,
+  ODLA_MEM_ERROR,
+  ODLA_UNSUPPORTED_DATATYPE,
+  ODLA_UNSUPPORTED_DEVICE_TYPE,
+  ODLA_UNSUPPORTED_OP,
+  ODLA_TIMEOUT,
+  ODLA_INTERNAL_LOGIC_ERR,
+  ODLA_RECOVERABLE_ERR,
+  ODLA_PARTITION_RESET,
+  ODLA_FULL_RESET,
+  ODLA_UNRECOVERABLE_ERR,
+  ODLA_FAILURE
+} odla_status;
+
+/* Shapes, value types, value lists.       [ref: ODLA/include/ODLA/odla_value.h:32-80] */
+#define ODLA_MAX_DIMENSION 10
+#define ODLA_MAX_OUTPUTS 64
+
+typedef struct {
+  odla_element_type data_type;
+  union {
+    odla_int32 val_int32;
+    odla_uint32 val_uint32;
+    odla_int64 val_int64;
+    odla_uint64 val_uint64;
+    odla_float32 val_fp32;
+    odla_float64 val_fp64;
+    odla_string val_str;
+  };
+} odla_scalar_value;
+
+typedef struct {
+  odla_int32 size; /* rank; 0 = scalar, -1 = undefined */
+  odla_int64 dims[ODLA_MAX_DIMENSION];
+} odla_value_shape; /* 88 bytes */
+
+typedef struct {
+  odla_element_type element_type;
+  odla_value_shape shape;
+} odla_value_type; /* 96 bytes */
+
+typedef struct _odla_value* odla_value;
+typedef struct _odla_value_id* odla_value_id; /* NUL-terminated name, or NULL */
+
+typedef struct {
+  odla_size_t size;
+  odla_value values[ODLA_MAX_OUTPUTS];
+} odla_values; /* 520 bytes */
+
+typedef struct {
+  odla_size_t size;
+  odla_value_id value_ids[ODLA_MAX_OUTPUTS];
+} odla_value_ids;
+
+/* Compute objects.                        [ref: ODLA/include/ODLA/odla_compute.h:34-112] */
+typedef enum {
+  ODLA_COMPUTE_DEFAULT, ODLA_COMPUTE_INFERENCE, ODLA_COMPUTE_TRAINING
+} odla_compute_mode;
+
+typedef enum {
+  ODLA_DYNAMIC_BATCH, ODLA_MIN_BATCH_SIZE, ODLA_MAX_BATCH_SIZE,
+  ODLA_OPT_BATCH_SIZE, ODLA_RUN_BATCH_SIZE, ODLA_DYNAMIC_SHAPE,
+  ODLA_MIN_SHAPE, ODLA_MAX_SHAPE, ODLA_OPT_SHAPE, ODLA_DYNAMIC_VALUE,
+  ODLA_MIN_VALUE, ODLA_MAX_VALUE, ODLA_OPT_VALUE,
+  ODLA_BF16_MODE,        /* value: odla_bf16_mode*                           */
+  ODLA_FP16_MODE,        /* value: bool*; fp16 storage, fp32 accumulate      */
+  ODLA_USE_SIM_MODE, ODLA_PROCESSOR_NUM, ODLA_BATCHES_PER_STEP,
+  ODLA_USE_DATA_TYPE,    /* value: odla_element_type*; ODLA_INT8/QINT8/QUINT8
+                            selects the int8 plan driven by the quant table  */
+  ODLA_LOAD_ENGINE_MODE, ODLA_USE_DLA_CORE,
+  ODLA_QUANT_TABLE,      /* value: const odla_value_quant_info*              */
+  ODLA_QUANT_TABLE_SIZE, /* value: const int*                                */
+  ODLA_AGGREGATE_OPS,    /* context item, value: bool*; hipGraph replay      */
+  ODLA_ENABLE_ENGINE_CACHE, ODLA_CACHE_DIR,
+  ODLA_ASYNC_CALLBACK_FUNC, ODLA_ASYNC_CALLBACK_ARG
+} odla_item_type;
+
+/* Library-private computation item (no counterpart in the reference): when
+ * set to true before the first context is created, every int8 Conv/Gemm whose
+ * result has no quant-table entry writes its raw int32 accumulator (+ int32
+ * bias) bit pattern into the 4-byte elements of its FLOAT32-typed result, so
+ * that tests can compare accumulators bit for bit. */
+#define ODLA_HIP_ITEM_RAW_INT32_ACC ((odla_item_type)1000)
+
+typedef enum {
+  BF16_DISABLE, BF16_ACCURACY_MODE, BF16_PERFORMACE_MODE, BF16_AUTO_MODE
+} odla_bf16_mode;
+
+typedef struct _odla_computation* odla_computation;
+typedef struct _odla_executable* odla_executable;
+typedef struct _odla_context* odla_context;
+typedef struct _odla_item_value* odla_item_value;
+
+/* Device objects.                         [ref: ODLA/include/ODLA/odla_device.h:33-88] */
+typedef enum {
+  ODLA_VENDOR_DEFAULT, ODLA_VENDOR_ALIBABA, ODLA_VENDOR_ARM,
+  ODLA_VENDOR_CAMBRICON, ODLA_VENDOR_GRAPHCORE, ODLA_VENDOR_HABANA,
+  ODLA_VENDOR_INTEL, ODLA_VENDOR_NVIDIA, ODLA_VENDOR_QUALCOMM
+} odla_vendor_name;
+
+typedef enum {
+  ODLA_DEVICE_DEFAULT, ODLA_DEVICE_ALIBABA_HANGUANG, ODLA_DEVICE_ARM_CORTEX_M,
+  ODLA_DEVICE_CAMBRICON_MLU220, ODLA_DEVICE_CAMBRICON_MLU270,
+  ODLA_DEVICE_GRAPHCORE_IPU, ODLA_DEVICE_HABANA_GAUDI, ODLA_DEVICE_HABANA_GOYA,
+  ODLA_DEVICE_INTEL_X86, ODLA_DEVICE_INTEL_DNNL, ODLA_DEVICE_NVIDIA_GPU,
+  ODLA_DEVICE_NVIDIA_TENSORRT, ODLA_DEVICE_QUALCOMM_AIC100
+} odla_device_name;
+
+typedef enum {
+  ODLA_DEVICE_INFO_ODLA_LIB_VERSION, /* string */
+  ODLA_DEVICE_INFO_DEV_COUNT,        /* int32  */
+  ODLA_DEVICE_INFO_DEV_INDEX,        /* int32  */
+  ODLA_DEVICE_INFO_DEV_TYPE,         /* string */
+  ODLA_DEVICE_INFO_DEV_UUID,         /* string */
+  ODLA_DEVICE_INFO_PROCESSOR_UTIL,   /* fp32 in [0,1] */
+  ODLA_DEVICE_INFO_MEMORY_UTIL,      /* fp32 in [0,1] */
+  ODLA_DEVICE_INFO_TOTAL_MEMORY,     /* int64 bytes */
+  ODLA_DEVICE_INFO_USED_MEMORY,      /* int64 bytes */
+  ODLA_DEVICE_INFO_POWER_USAGE,      /* fp32 watt */
+  ODLA_DEVICE_INFO_POWER_LIMIT,      /* fp32 watt */
+  ODLA_DEVICE_INFO_DRIVER_VERSION,   /* string */
+  ODLA_DEVICE_INFO_SDK_VERSION       /* string */
+} odla_device_info;
+
+typedef struct _odla_vendor* odla_vendor;
+typedef struct _odla_device* odla_device;
+
+/* Memory, logging.   [ref: ODLA/include/ODLA/odla_memory.h:33-38, odla_log.h:29-45] */
+typedef enum {
+  ODLA_MEMCPY_H2H, ODLA_MEMCPY_H2D, ODLA_MEMCPY_D2H, ODLA_MEMCPY_D2D
+} odla_memcpy_type;
+
+typedef enum {
+  ODLA_LOG_LEVEL_OFF, ODLA_LOG_LEVEL_FATAL, ODLA_LOG_LEVEL_ERROR,
+  ODLA_LOG_LEVEL_WARN, ODLA_LOG_LEVEL_INFO, ODLA_LOG_LEVEL_DEBUG,
+  ODLA_LOG_LEVEL_TRACE
+} odla_log_level;
+
+typedef void (*odla_logging_func)(const char* file_name, int line,
+                                  const char* func_name, odla_log_level level,
+                                  const char* msg);
+
+/* Operator attribute enums.
+ * [ref: ODLA/include/ODLA/ops/odla_ops_nn.h:35-43, odla_ops_process.h:33-48] */
+typedef enum {
+  ODLA_CHANNELS_FIRST, /* activations N,C,spatial  */
+  ODLA_CHANNELS_LAST,  /* activations N,spatial,C  */
+  ODLA_SIO,            /* kernel spatial,in,out    */
+  ODLA_SOI,            /* kernel spatial,out,in    */
+  ODLA_OIS,            /* kernel out,in,spatial    */
+  ODLA_IOS             /* kernel in,out,spatial    */
+} odla_memory_layout;
+
+typedef enum { ODLA_NEAREST, ODLA_LINEAR, ODLA_CUBIC } odla_interpolation_mode;
+
+typedef enum {
+  ODLA_ASSYMMETRIC, ODLA_HALF_PIXEL, ODLA_HALF_PIXEL_TF, ODLA_ALIGN_CORNERS
+} odla_resize_coordinate_mode;
+
+/* One record of a quantization table.  A tensor is described by one record
+ * with ch_idx = -(number of channels) carrying the per-tensor scale, offset
+ * (zero point) and range, optionally followed by one record per channel
+ * (ch_idx = c) carrying that channel's min/max.
+ * [ref: ODLA/include/ODLA/ops/odla_ops_quantization.h:33-41; writer
+ *  utils/halo_pgq.py:308-332] */
+typedef struct {
+  odla_value_id value_id;
+  int ch_idx;
+  odla_float32 scale;
+  odla_float32 offset;
+  odla_float32 min;
+  odla_float32 max;
+} odla_value_quant_info; /* 32 bytes */
+
+/* ------------------------------------------------------------------------ */
+/* Computation / context / execution                                         */
+/* ------------------------------------------------------------------------ */
+
+/* Create an empty graph and make it the calling thread's current computation.
+ * [ref: ODLA/include/ODLA/odla_compute.h:114-122; dnnl odla_dnnl.cc:98-105] */
+odla_status odla_CreateComputation(odla_computation* computation);
+
+/* Release the graph, its packed weights and every value handle it owns.
+ * [ref: odla_compute.h:223-230; tensorrt odla_tensorrt.cc:104-113] */
+odla_status odla_DestroyComputation(odla_computation computation);
+
+/* Property bag.  Honoured: ODLA_FP16_MODE, ODLA_BF16_MODE, ODLA_USE_DATA_TYPE,
+ * ODLA_QUANT_TABLE, ODLA_QUANT_TABLE_SIZE, ODLA_HIP_ITEM_RAW_INT32_ACC.  Other
+ * items are accepted and ignored (ODLA_SUCCESS) so that harnesses that set
+ * ODLA_USE_SIM_MODE or batch hints keep working.
+ * [ref: odla_compute.h:232-241; dnnl odla_dnnl.cc:84-96; tensorrt :130-199] */
+odla_status odla_SetComputationItem(odla_computation computation,
+                                    odla_item_type type, odla_item_value value);
+
+/* Create an execution context (device arena + stream + captured hipGraph)
+ * for the calling thread's current computation (the most recently created one
+ * when the thread has none).
+ * [ref: odla_compute.h:420-427; dnnl odla_dnnl.cc:122-126; tensorrt :319-329] */
+odla_status odla_CreateContext(odla_context* context);
+odla_status odla_DestroyContext(odla_context context); /* [ref: odla_compute.h:440-446] */
+
+/* Honoured: ODLA_AGGREGATE_OPS (bool*, default true: replay through hipGraph).
+ * [ref: odla_compute.h:429-438; tensorrt odla_tensorrt.cc:284-317] */
+odla_status odla_SetContextItem(odla_context context, odla_item_type type,
+                                odla_item_value value);
+
+/* Attach caller memory to an argument / output for the next execution.  The
+ * pointer may be host memory (copied across PCIe inside Execute) or device
+ * memory obtained from odla_AllocateDeviceMemory (copied on the device).
+ * [ref: odla_compute.h:448-505; dnnl odla_dnnl.cc:246-303,380-407;
+ *  tensorrt odla_tensorrt.cc:422-448] */
+odla_status odla_BindToArgument(odla_value value, const odla_void* data_ptr,
+                                odla_context context);
+odla_status odla_BindToArgumentById(const odla_value_id value_id,
+                                    const odla_void* data_ptr,
+                                    odla_context context);
+odla_status odla_BindToOutput(odla_value value, odla_void* data_ptr,
+                              odla_context context);
+odla_status odla_BindToOutputById(const odla_value_id value_id,
+                                  odla_void* data_ptr, odla_context context);
+
+/* Run the graph once: stage bound arguments, replay the planned launch
+ * sequence, write every bound output, and return after the device is idle.
+ * [ref: odla_compute.h:158-170; dnnl odla_dnnl.cc:133-159;
+ *  tensorrt odla_tensorrt.cc:866-968] */
+odla_status odla_ExecuteComputation(const odla_computation computation,
+                                    const odla_context context,
+                                    const odla_compute_mode mode,
+                                    odla_device device);
+
+/* Introspection used by generic harnesses.
+ * [ref: odla_compute.h:184-221; dnnl odla_dnnl.cc:208-244,363-378] */
+odla_status odla_GetNumOfArgsFromComputation(const odla_computation computation,
+                                             odla_uint32* num_args);
+odla_status odla_GetArgFromComputationByIdx(const odla_computation computation,
+                                            const odla_uint32 arg_idx,
+                                            odla_value* arg_value);
+odla_status odla_GetNumOfOutputsFromComputation(
+    const odla_computation computation, odla_uint32* num_outputs);
+odla_status odla_GetOutputFromComputationByIdx(
+    const odla_computation computation, const odla_uint32 output_idx,
+    odla_value* output_value);
+/* Static shapes only: returns the value's declared shape.
+ * [ref: odla_compute.h:275-284] */
+odla_status odla_GetRuntimeShape(odla_context context, odla_value value,
+                                 odla_value_shape* value_shape_ptr);
+
+/* Values.                      [ref: ODLA/include/ODLA/odla_value.h:82-214] */
+odla_status odla_GetValueType(const odla_value value,
+                              odla_value_type* value_type);
+odla_status odla_GetValueId(const odla_value value, odla_value_id* value_id);
+odla_status odla_FindValueById(const odla_value_id value_id, odla_value* value);
+odla_status odla_SetValueAsOutput(odla_value value);
+odla_status odla_SetValuesAsOutput(odla_values values);
+odla_status odla_SetValueAsOutputById(const odla_value_id value_id);
+/* Copy the device-resident result of `value` from the last execution of
+ * `context` to host memory.  [ref: odla_compute.h:556-565] */
+odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr,
+                              odla_context context);
+odla_status odla_ReleaseValue(odla_value value); /* no-op; values die with the graph */
+
+/* Graph inputs and constants.  A constant's host data must stay valid until
+ * the first context of the computation has been created; it is then resident
+ * on the device.
+ * [ref: ODLA/include/ODLA/ops/odla_ops_basic.h:39-75;
+ *  dnnl odla_dnnl.cc:192-206,305-330] */
+odla_value odla_CreateArgument(const odla_value_type value_type,
+                               const odla_value_id value_id);
+odla_value odla_CreateConstant(const odla_value_type value_type,
+                               const odla_void* data_ptr,
+                               const odla_value_id value_id);
+
+/* ------------------------------------------------------------------------ */
+/* Device, memory, logging, version                                          */
+/* ------------------------------------------------------------------------ */
+/* [ref: odla_device.h:118-174; tensorrt/odla_device.cc:60-200;
+ *  tests/ODLA/device_test.cc:63-89] */
+odla_status odla_AllocateDevice(odla_vendor vendor, odla_device_name device_name,
+                                odla_int32 device_idx, odla_device* device);
+odla_status odla_GetDeviceInfo(odla_device device, odla_device_info info_type,
+                               odla_scalar_value* info_value);
+odla_status odla_SetCurrentDevice(odla_device device);
+odla_status odla_DestroyDevice(odla_device device);
+
+/* [ref: ODLA/include/ODLA/odla_memory.h:47-87] */
+odla_status odla_AllocateDeviceMemory(odla_void** dev_ptr, odla_size_t size);
+odla_status odla_FreeDeviceMemory(odla_void* ptr);
+odla_status odla_AllocateHostMemory(odla_void** host_ptr, odla_size_t size);
+odla_status odla_FreeHostMemory(odla_void* ptr);
+odla_status odla_CopyMemory(odla_void* dst, odla_void* src, odla_size_t size,
+                            odla_memcpy_type type);
+
+/* [ref: ODLA/include/ODLA/odla_log.h:47-68; platforms/common/utils.cc:21-60] */
+odla_status odla_SetLogLevel(odla_log_level level);
+odla_status odla_SetLogger(odla_logging_func logger);
+odla_logging_func odla_GetLogger(void);
+
+/* [ref: ODLA/include/ODLA/odla_version.h:33-43] */
+const odla_char* odla_GetVersionString(void);
+
+/* ------------------------------------------------------------------------ */
+/* Graph builders.  `output_dims` may be left undefined (size <= 0 or          */
+/* garbage): the library infers every result shape itself and only uses a     */
+/* caller-provided shape where inference is ambiguous (Reshape, Resize).      */
+/* ------------------------------------------------------------------------ */
+
+/* 2-D cross-correlation with groups and optional bias.
+ * [ref: ops/odla_ops_nn.h:213-219; dnnl odla_dnnl.cc:1014-1129] */
+odla_value odla_Conv(odla_value input, odla_memory_layout input_layout,
+                     odla_uint32 group, odla_value kernel,
+                     odla_memory_layout kernel_layout,
+                     const odla_uint32* strides, const odla_uint32* dilations,
+                     const odla_uint32* paddings_front,
+                     const odla_uint32* paddings_back, odla_value bias,
+                     odla_value_shape output_dims, const odla_value_id value_id);
+
+/* alpha * op(A) * op(B) + beta * C, rank 2 or batched.
+ * [ref: ops/odla_ops_math.h:361-364; dnnl odla_dnnl.cc:1730-1866] */
+odla_value odla_Gemm(odla_value A, odla_bool A_transpose, odla_value B,
+                     odla_bool B_transpose, odla_float32 alpha,
+                     odla_float32 beta, odla_value C,
+                     odla_value_shape output_dims, const odla_value_id value_id);
+/* [ref: ops/odla_ops_math.h:337-339] */
+odla_value odla_BatchMatMul(odla_value A, odla_bool A_transpose, odla_value B,
+                            odla_bool B_transpose, odla_value_shape output_dims,
+                            const odla_value_id value_id);
+
+/* Element-wise binary with numpy-style broadcast.
+ * [ref: ops/odla_ops_math.h:75,228,601,643,683,968; dnnl odla_dnnl.cc:585-633,
+ *  odla_dnnl.h:301-394] */
+odla_value odla_Add(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Sub(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Mul(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Div(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Max(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Min(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+
+/* Element-wise unary.
+ * [ref: ops/odla_ops_nn.h:431,586,678; ops/odla_ops_math.h:163,253,287,553,
+ *  870,883,941,1009; dnnl odla_dnnl.cc:432-453,635-696,834-837,1868-1904] */
+odla_value odla_Relu(odla_value input, const odla_value_id value_id);
+odla_value odla_LeakyRelu(odla_value input, odla_float32 alpha,
+                          const odla_value_id value_id);
+odla_value odla_Sigmoid(odla_value input, const odla_value_id value_id);
+odla_value odla_Tanh(odla_value input, const odla_value_id value_id);
+odla_value odla_Exp(odla_value input, const odla_value_id value_id);
+odla_value odla_Log(odla_value input, const odla_value_id value_id);
+odla_value odla_Sqrt(odla_value input, const odla_value_id value_id);
+odla_value odla_Rsqrt(odla_value input, const odla_value_id value_id);
+odla_value odla_Erf(odla_value input, const odla_value_id value_id);
+odla_value odla_Abs(odla_value input, const odla_value_id value_id);
+odla_value odla_Neg(odla_value input, const odla_value_id value_id);
+odla_value odla_Round(odla_value input, const odla_value_id value_id);
+odla_value odla_Clamp(odla_value input, odla_float32 lo, odla_float32 hi,
+                      const odla_value_id value_id);
+odla_value odla_Gelu(odla_value input, odla_bool use_approx,
+                     const odla_value_id value_id);
+
+/* Inference batch normalisation with global statistics.
+ * [ref: ops/odla_ops_nn.h:172-176; dnnl odla_dnnl.cc:1448-1524] */
+odla_value odla_BatchNormalization(odla_value input,
+                                   odla_memory_layout input_layout,
+                                   odla_value mean, odla_value var,
+                                   odla_float32 epsilon, odla_value scale,
+                                   odla_value offset, odla_float32 scalar_scale,
+                                   odla_float32 scalar_offset,
+                                   const odla_value_id value_id);
+
+/* Layer normalisation over the trailing axes.  The reference code generator
+ * emits this call but no reference header declares it.
+ * [ref: lib/target/generic_cpp/batchnorm.cc:100-113;
+ *  lib/transforms/fusion.cc:296-313] */
+odla_value odla_LayerNorm(odla_value input, odla_size_t axes_size,
+                          const odla_int32* axes, odla_float32 epsilon,
+                          odla_value scale, odla_value offset,
+                          const odla_value_id value_id);
+
+/* Pooling.  [ref: ops/odla_ops_nn.h:107-112,463-467; dnnl odla_dnnl.cc:1360-1446] */
+odla_value odla_MaxPool(odla_value input, odla_memory_layout input_layout,
+                        const odla_uint32* window_dims,
+                        const odla_uint32* strides,
+                        const odla_uint32* paddings_front,
+                        const odla_uint32* paddings_back,
+                        odla_value_shape output_dims,
+                        const odla_value_id value_id);
+odla_value odla_AveragePool(odla_value input, odla_memory_layout input_layout,
+                            const odla_uint32* window_dims,
+                            const odla_uint32* strides,
+                            const odla_uint32* paddings_front,
+                            const odla_uint32* paddings_back,
+                            odla_bool padding_included,
+                            odla_value_shape output_dims,
+                            const odla_value_id value_id);
+
+/* Reductions.  [ref: ops/odla_ops_math.h:742-820; dnnl odla_dnnl_statistics.cc:20-117] */
+odla_value odla_ReduceMean(odla_value input, odla_size_t num_of_axes,
+                           const odla_uint32* axes, odla_bool keep_dims,
+                           odla_value_shape output_dims,
+                           const odla_value_id value_id);
+odla_value odla_ReduceSum(odla_value input, odla_size_t num_of_axes,
+                          const odla_uint32* axes, odla_bool keep_dims,
+                          odla_value_shape output_dims,
+                          const odla_value_id value_id);
+odla_value odla_ReduceMax(odla_value input, odla_size_t num_of_axes,
+                          const odla_uint32* axes, odla_bool keep_dims,
+                          odla_value_shape output_dims,
+                          const odla_value_id value_id);
+
+/* Softmax along one axis (negative axis = last).
+ * [ref: ops/odla_ops_nn.h:440,691; dnnl odla_dnnl.cc:1628-1669] */
+odla_value odla_Softmax(odla_value input, odla_int32 axis,
+                        const odla_value_id value_id);
+odla_value odla_LogSoftmax(odla_value input, odla_int32 axis,
+                           const odla_value_id value_id);
+
+/* Data movement.
+ * [ref: ops/odla_ops_process.h:80-84,113-116,160-163,253-256,281-284,355-359,
+ *  434-437; dnnl odla_dnnl.cc:455-508,869-898,1331-1358,1526-1551,1906-1990] */
+odla_value odla_Cast(odla_value input, odla_element_type target_type,
+                     const odla_value_id value_id);
+odla_value odla_Concat(odla_values inputs, odla_int32 axis,
+                       odla_value_shape output_shape,
+                       const odla_value_id value_id);
+odla_value odla_Gather(odla_value input, odla_value indices, odla_int32 axis,
+                       odla_value_shape output_dims,
+                       const odla_value_id value_id);
+odla_value odla_Reshape(odla_value input, odla_value_shape output_dims,
+                        const odla_value_id value_id);
+odla_value odla_Resize(odla_value input, odla_interpolation_mode interpolation,
+                       odla_resize_coordinate_mode mode, odla_uint32 axes_mask,
+                       odla_value_shape output_dims,
+                       const odla_value_id value_id);
+odla_value odla_Slice(odla_value input, const odla_int32* start,
+                      const odla_int32* end, const odla_int32* stride,
+                      odla_value_shape output_dims,
+                      const odla_value_id value_id);
+odla_value odla_Transpose(odla_value input, odla_value_shape permutations,
+                          odla_value_shape output_dims,
+                          const odla_value_id value_id);
+
+/* Affine (de)quantisation; scale with more than one element is per-`axis`.
+ * q = saturate(round_half_even(x / scale) + zero_point);  x = (q - zp) * scale.
+ * [ref: ops/odla_ops_quantization.h:55-73; dnnl odla_dnnl_quantization.cc:33-90] */
+odla_value odla_Quantize(odla_value input, odla_value scale,
+                         odla_value zero_point, odla_int32 axis,
+                         odla_element_type target_data_type,
+                         const odla_value_id value_id);
+odla_value odla_Dequantize(odla_value input, odla_value scale,
+                           odla_value zero_point, odla_int32 axis,
+                           odla_element_type target_data_type,
+                           const odla_value_id value_id);
+
+/* Batched non-maximum suppression.  boxes [N,B,4] as (y1,x1,y2,x2) corners,
+ * scores [N,C,B]; result int32 [N*max_num_outputs,3] rows {image, class, box}
+ * in selection order, unused rows filled with -1.  Selection rule per image:
+ * each box competes with its best class score; keep score > score_threshold;
+ * order by (score desc, box index asc); greedily drop a box whose IoU with an
+ * already kept box is >= iou_threshold.
+ * [ref: ops/odla_ops_nn.h:504-507; dnnl odla_dnnl.cc:2113-2181;
+ *  dnnl_utils_avx512.h:977-1079] */
+odla_value odla_NMS(odla_value boxes, odla_value scores,
+                    odla_uint32 max_num_outputs, odla_float32 iou_threshold,
+                    odla_float32 score_threshold,
+                    odla_value_type output_value_type,
+                    const odla_value_id value_id);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* ODLA_HIP_H_ */

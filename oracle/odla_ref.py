@@ -1,0 +1,474 @@
+"""CPU oracle for the ODLA hot path -- TEST INFRASTRUCTURE ONLY.
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module; the shipped library never does.
+
+``RefBuilder`` offers the same builder vocabulary as the GPU-side
+``HipBuilder`` (one method per ``odla_<Op>``) but evaluates every operator
+eagerly on numpy arrays in fp32, restating what the reference CPU backend
+computes.  Each method cites the reference code it follows; paths are relative
+to the reference tree.  Heavy loops live in ``odla_ref.c`` (built to
+``libodla_ref.so`` by ``oracle/Makefile``).
+
+Pin status (what fixes each function independently of this file):
+  conv2d / gemm / pools / softmax / batchnorm   reference-held known-answer
+      vectors (odla_popart/test), the reference's own fp32 kernels built to
+      ``oracle/_ref/libsn_rt.so``, float64 brute force.
+  quantize / dequantize   ONNX QuantizeLinear published example (passes on the
+      reference CPU backend), exhaustive half-integer rounding check.
+  layernorm / gelu / erf / resize / concat / transpose / gather   closed forms
+      and library routines (math.erf, numpy).
+  nms   ONNX NonMaxSuppression published examples, O(n^2) brute force.
+  int8 convolution + requantisation (``qconv`` ...)   PARITY UNPINNED by the
+      reference: it has no int8 convolution of its own.  The int32 accumulators
+      are pinned by int64 brute force; the requantisation formula is this
+      build's definition.
+"""
+import ctypes
+import math
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+def lib():
+    """libodla_ref.so, loaded on first use."""
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "libodla_ref.so")
+        if not os.path.exists(path):
+            raise RuntimeError("oracle/libodla_ref.so is missing: run `make -C oracle`")
+        _LIB = ctypes.CDLL(path)
+        _LIB.odla_ref_num_threads.restype = ctypes.c_int
+    return _LIB
+
+
+def num_threads():
+    return int(lib().odla_ref_num_threads())
+
+
+def _p(a, t):
+    return a.ctypes.data_as(ctypes.POINTER(t))
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+# --------------------------------------------------------------------------
+# Heavy kernels (C)
+# --------------------------------------------------------------------------
+def conv_out_dim(i, k, s, pf, pb, d=1):
+    return (i + pf + pb - ((k - 1) * d + 1)) // s + 1
+
+
+def conv2d(x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), group=1):
+    """NCHW x OIHW cross-correlation.  pad = (top, left, bottom, right).
+    [ref: ODLA/platforms/dnnl/odla_dnnl.cc:1014-1129]"""
+    x, w = _f32(x), _f32(w)
+    N, C, H, W = x.shape
+    O, I, R, S = w.shape
+    assert C == I * group and O % group == 0
+    Ho = conv_out_dim(H, R, stride[0], pad[0], pad[2], dilation[0])
+    Wo = conv_out_dim(W, S, stride[1], pad[1], pad[3], dilation[1])
+    y = np.empty((N, O, Ho, Wo), np.float32)
+    b = None if bias is None else _f32(bias).reshape(-1)
+    lib().odla_ref_conv2d_f32(
+        _p(x, ctypes.c_float), _p(w, ctypes.c_float),
+        _p(b, ctypes.c_float) if b is not None else None, _p(y, ctypes.c_float),
+        N, C, H, W, O, R, S, group, stride[0], stride[1], dilation[0], dilation[1],
+        pad[0], pad[1], Ho, Wo)
+    return y
+
+
+def pool2d(x, window, stride, pad, out_hw=None, is_max=True, count_include_pad=False):
+    """NCHW pooling.  [ref: odla_dnnl.cc:1360-1446]: max pooling ignores padding;
+    average pooling divides by the in-bounds count (oneDNN pooling_avg ==
+    exclude-padding) unless count_include_pad."""
+    x = _f32(x)
+    N, C, H, W = x.shape
+    Ho = conv_out_dim(H, window[0], stride[0], pad[0], pad[2]) if out_hw is None else out_hw[0]
+    Wo = conv_out_dim(W, window[1], stride[1], pad[1], pad[3]) if out_hw is None else out_hw[1]
+    y = np.empty((N, C, Ho, Wo), np.float32)
+    lib().odla_ref_pool2d_f32(_p(x, ctypes.c_float), _p(y, ctypes.c_float), N, C, H, W,
+                              window[0], window[1], stride[0], stride[1], pad[0], pad[1], Ho, Wo,
+                              1 if is_max else 0, 1 if count_include_pad else 0)
+    return y
+
+
+def conv2d_q8_acc(xq, zp_x, wq, bias_i32=None, stride=(1, 1), pad=(0, 0, 0, 0)):
+    """int32 accumulators of a u8 x s8 convolution (see odla_ref.c)."""
+    xq = np.ascontiguousarray(xq, dtype=np.uint8)
+    wq = np.ascontiguousarray(wq, dtype=np.int8)
+    N, C, H, W = xq.shape
+    O, I, R, S = wq.shape
+    assert C == I
+    Ho = conv_out_dim(H, R, stride[0], pad[0], pad[2])
+    Wo = conv_out_dim(W, S, stride[1], pad[1], pad[3])
+    acc = np.empty((N, O, Ho, Wo), np.int32)
+    b = None if bias_i32 is None else np.ascontiguousarray(bias_i32, dtype=np.int32)
+    lib().odla_ref_conv2d_q8(_p(xq, ctypes.c_uint8), int(zp_x), _p(wq, ctypes.c_int8),
+                             _p(b, ctypes.c_int32) if b is not None else None,
+                             _p(acc, ctypes.c_int32), N, C, H, W, O, R, S,
+                             stride[0], stride[1], pad[0], pad[1], Ho, Wo)
+    return acc
+
+
+def requant_q8(acc, mul, zp, lo=0):
+    """q = clamp(rne(float32(acc) * mul[o]) + zp, lo, 255)."""
+    acc = np.ascontiguousarray(acc, dtype=np.int32)
+    N, O = acc.shape[0], acc.shape[1]
+    HW = int(np.prod(acc.shape[2:])) if acc.ndim > 2 else 1
+    mul = _f32(mul).reshape(-1)
+    assert mul.size == O
+    q = np.empty(acc.shape, np.uint8)
+    lib().odla_ref_requant_q8(_p(acc, ctypes.c_int32), _p(mul, ctypes.c_float), int(zp), int(lo),
+                              _p(q, ctypes.c_uint8), N, O, HW)
+    return q
+
+
+# --------------------------------------------------------------------------
+# Quantisation scheme of the int8 plan
+# [ref: utils/halo_pgq.py:283-297 (activations), lib/quantizer/weights_quantizer.cc:35-64,
+#  126-176 (zero-point clamp, bias)]
+# --------------------------------------------------------------------------
+def act_qparams(mn, mx):
+    """Asymmetric u8: scale = (max-min)/255, zp = clip(rne(-min/scale), 0, 255).
+    The range is widened to contain 0 so that 0 is exactly representable."""
+    mn = np.float32(min(float(mn), 0.0))
+    mx = np.float32(max(float(mx), 0.0))
+    scale = np.float32((mx - mn) / np.float32(255.0))
+    if not scale > 0:
+        scale = np.float32(1.0)
+    zp = int(np.clip(np.rint(np.float32(-mn) / scale), 0, 255))
+    return scale, zp
+
+
+def weight_qparams(w):
+    """Symmetric per-output-channel s8: scale[o] = max|w_o| / 127."""
+    w = _f32(w)
+    m = np.abs(w.reshape(w.shape[0], -1)).max(axis=1).astype(np.float32)
+    s = (m / np.float32(127.0)).astype(np.float32)
+    s[m == 0] = np.float32(1.0)
+    return s
+
+
+def quantize_weights(w, s):
+    w = _f32(w)
+    q = np.rint(w / s.reshape((-1,) + (1,) * (w.ndim - 1)).astype(np.float32))
+    return np.clip(q, -127, 127).astype(np.int8)
+
+
+def quantize_bias(b, s_x, s_w):
+    """int32 bias = rne(b / (s_x * s_w[o]))."""
+    bs = (np.float32(s_x) * s_w.astype(np.float32)).astype(np.float32)
+    r = np.rint(_f32(b).reshape(-1) / bs)
+    return np.clip(r, -2147483648.0, 2147483520.0).astype(np.int64).astype(np.int32)
+
+
+def quantize_act(x, scale, zp):
+    """q = clamp(rne(x / scale) + zp, 0, 255)   [ref: odla_dnnl_quantization.cc:61-90]"""
+    t = np.rint(_f32(x) / np.float32(scale)) + np.float32(zp)
+    return np.clip(t, 0, 255).astype(np.uint8)
+
+
+def dequantize_act(q, scale, zp):
+    """x = (q - zp) * scale   [ref: odla_dnnl_quantization.cc:33-59]"""
+    return ((q.astype(np.float32) - np.float32(zp)) * np.float32(scale)).astype(np.float32)
+
+
+def qconv(xq, x_qp, w, bias, out_qp, stride, pad, relu=False):
+    """int8 convolution with fused requantisation, as the int8 plan defines it.
+    Returns (q_out u8, acc int32)."""
+    s_x, zp_x = x_qp
+    s_w = weight_qparams(w)
+    wq = quantize_weights(w, s_w)
+    bi = None if bias is None else quantize_bias(bias, s_x, s_w)
+    acc = conv2d_q8_acc(xq, zp_x, wq, bi, stride, pad)
+    s_y, zp_y = out_qp
+    mul = ((np.float32(s_x) * s_w).astype(np.float32) / np.float32(s_y)).astype(np.float32)
+    q = requant_q8(acc, mul, zp_y, zp_y if relu else 0)
+    return q, acc
+
+
+def qadd(aq, a_qp, bq, b_qp, out_qp, relu=False):
+    """Residual add in the quantised domain: dequantise both, add in fp32,
+    requantise with a multiply by float32(1/s_out)."""
+    fa = dequantize_act(aq, *a_qp)
+    fb = dequantize_act(bq, *b_qp)
+    f = (fa + fb).astype(np.float32)
+    s_y, zp_y = out_qp
+    inv = np.float32(1.0) / np.float32(s_y)
+    q = np.rint(f * inv).astype(np.int64) + int(zp_y)
+    return np.clip(q, zp_y if relu else 0, 255).astype(np.uint8)
+
+
+# --------------------------------------------------------------------------
+# NMS  [ref: ODLA/platforms/dnnl/dnnl_utils_avx512.h:977-1079, selection rule as intended]
+# --------------------------------------------------------------------------
+def _iou_one_to_many(box, others):
+    f = np.float32
+    y1 = np.minimum(box[0], box[2]); x1 = np.minimum(box[1], box[3])
+    y2 = np.maximum(box[0], box[2]); x2 = np.maximum(box[1], box[3])
+    oy1 = np.minimum(others[:, 0], others[:, 2]); ox1 = np.minimum(others[:, 1], others[:, 3])
+    oy2 = np.maximum(others[:, 0], others[:, 2]); ox2 = np.maximum(others[:, 1], others[:, 3])
+    area_i = ((oy2 - oy1) * (ox2 - ox1)).astype(f)
+    area_j = f((y2 - y1) * (x2 - x1))
+    ih = np.maximum(np.minimum(oy2, y2) - np.maximum(oy1, y1), f(0)).astype(f)
+    iw = np.maximum(np.minimum(ox2, x2) - np.maximum(ox1, x1), f(0)).astype(f)
+    inter = (ih * iw).astype(f)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        iou = (inter / ((area_i + area_j).astype(f) - inter).astype(f)).astype(f)
+    iou[(area_i <= 0) | (area_j <= 0)] = 0
+    return iou
+
+
+def nms(boxes, scores, max_out, iou_thr, score_thr):
+    """boxes [N,B,4] (y1,x1,y2,x2), scores [N,C,B] -> int32 [N*max_out,3] rows
+    {image, class, box}, -1 padded."""
+    boxes, scores = _f32(boxes), _f32(scores)
+    N, B, _ = boxes.shape
+    out = np.full((N, max_out, 3), -1, np.int32)
+    for n in range(N):
+        sc = scores[n]                      # [C,B]
+        cls = np.argmax(sc, axis=0)         # first maximum
+        best = sc[cls, np.arange(B)]
+        cand = np.nonzero(best > np.float32(score_thr))[0]
+        if cand.size == 0 or max_out == 0:
+            continue
+        order = cand[np.lexsort((cand, -best[cand].astype(np.float64)))]
+        alive = np.ones(order.size, bool)
+        kept = 0
+        for i in range(order.size):
+            if not alive[i]:
+                continue
+            if kept >= max_out:
+                break
+            bi = order[i]
+            out[n, kept] = (n, cls[bi], bi)
+            kept += 1
+            rest = np.nonzero(alive[i + 1:])[0] + i + 1
+            if rest.size:
+                iou = _iou_one_to_many(boxes[n, bi], boxes[n, order[rest]])
+                alive[rest[iou >= np.float32(iou_thr)]] = False
+    return out.reshape(N * max_out, 3)
+
+
+# --------------------------------------------------------------------------
+# Reference-style broadcast alignment  [ref: ODLA/platforms/dnnl/odla_dnnl.h:301-343]
+# --------------------------------------------------------------------------
+def align_like_reference(src_shape, dst_shape):
+    sn, dn = len(src_shape), len(dst_shape)
+    for j in range(dn - 1, sn - 2, -1):
+        ok = all(dst_shape[j - k] == src_shape[sn - 1 - k] or dst_shape[j - k] == 1 or src_shape[sn - 1 - k] == 1
+                 for k in range(sn))
+        if ok:
+            r = [1] * dn
+            for k in range(sn):
+                r[j - k] = src_shape[sn - 1 - k]
+            return tuple(r)
+    raise ValueError("shapes %s and %s do not broadcast" % (src_shape, dst_shape))
+
+
+_erf = np.vectorize(math.erf, otypes=[np.float64])
+
+
+class RefBuilder:
+    """Eager fp32 evaluation of an ODLA graph on the CPU."""
+
+    def __init__(self, feeds):
+        self.feeds = feeds
+        self.outputs = {}
+        self.values = {}
+
+    def _name(self, name, v):
+        if name:
+            self.values[name] = v
+        return v
+
+    # graph inputs -----------------------------------------------------------
+    def arg(self, name, shape, dtype=np.float32):
+        v = np.ascontiguousarray(self.feeds[name], dtype=dtype)
+        assert tuple(v.shape) == tuple(shape), (name, v.shape, shape)
+        return self._name(name, v)
+
+    def const(self, name, array):
+        return self._name(name, np.ascontiguousarray(array))
+
+    def output(self, v, name):
+        self.outputs[name] = v
+
+    # heavy operators --------------------------------------------------------
+    def conv(self, x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), group=1, name=None):
+        return self._name(name, conv2d(x, w, bias, stride, pad, dilation, group))
+
+    def gemm(self, a, b, c=None, ta=False, tb=False, alpha=1.0, beta=1.0, name=None):
+        """alpha * op(A) op(B) + beta * C; leading dims of A are batch dims.
+        [ref: odla_dnnl.cc:1730-1866]"""
+        a, b = _f32(a), _f32(b)
+        if ta:
+            a = np.swapaxes(a, -1, -2)
+        if tb:
+            b = np.swapaxes(b, -1, -2)
+        y = np.matmul(a.astype(np.float64), b.astype(np.float64))
+        y = y * float(alpha)
+        if c is not None and beta != 0:
+            y = y + float(beta) * _f32(c).astype(np.float64)
+        return self._name(name, y.astype(np.float32))
+
+    def maxpool(self, x, window, stride, pad, out_hw=None, name=None):
+        return self._name(name, pool2d(x, window, stride, pad, out_hw, True))
+
+    def avgpool(self, x, window, stride, pad, count_include_pad=False, out_hw=None, name=None):
+        return self._name(name, pool2d(x, window, stride, pad, out_hw, False, count_include_pad))
+
+    # element-wise -----------------------------------------------------------
+    def _bin(self, f, a, b, name):
+        a, b = np.asarray(a), np.asarray(b)
+        if a.ndim != b.ndim:
+            if a.ndim < b.ndim:
+                a = a.reshape(align_like_reference(a.shape, b.shape))
+            else:
+                b = b.reshape(align_like_reference(b.shape, a.shape))
+        return self._name(name, f(a.astype(np.float32), b.astype(np.float32)).astype(np.float32))
+
+    def add(self, a, b, name=None): return self._bin(np.add, a, b, name)
+    def sub(self, a, b, name=None): return self._bin(np.subtract, a, b, name)
+    def mul(self, a, b, name=None): return self._bin(np.multiply, a, b, name)
+    def div(self, a, b, name=None): return self._bin(np.divide, a, b, name)
+    def max(self, a, b, name=None): return self._bin(np.maximum, a, b, name)
+    def min(self, a, b, name=None): return self._bin(np.minimum, a, b, name)
+
+    def relu(self, x, name=None): return self._name(name, np.maximum(_f32(x), np.float32(0)))
+
+    def leaky_relu(self, x, alpha, name=None):
+        x = _f32(x)
+        return self._name(name, np.where(x > 0, x, np.float32(alpha) * x).astype(np.float32))
+
+    def _unary64(self, f, x, name):
+        return self._name(name, f(_f32(x).astype(np.float64)).astype(np.float32))
+
+    def sigmoid(self, x, name=None): return self._unary64(lambda v: 1.0 / (1.0 + np.exp(-v)), x, name)
+    def tanh(self, x, name=None): return self._unary64(np.tanh, x, name)
+    def exp(self, x, name=None): return self._unary64(np.exp, x, name)
+    def log(self, x, name=None): return self._unary64(np.log, x, name)
+    def sqrt(self, x, name=None): return self._unary64(np.sqrt, x, name)
+    def rsqrt(self, x, name=None): return self._unary64(lambda v: 1.0 / np.sqrt(v), x, name)
+    def erf(self, x, name=None): return self._unary64(_erf, x, name)
+    def abs(self, x, name=None): return self._name(name, np.abs(_f32(x)))
+    def neg(self, x, name=None): return self._name(name, -_f32(x))
+    def round(self, x, name=None): return self._name(name, np.rint(_f32(x)))
+
+    def clamp(self, x, lo, hi, name=None):
+        return self._name(name, np.clip(_f32(x), np.float32(lo), np.float32(hi)))
+
+    def gelu(self, x, approx=False, name=None):
+        """[ref: odla_dnnl.cc:1868-1876]"""
+        if approx:
+            f = lambda v: 0.5 * v * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (v + 0.044715 * v ** 3)))
+        else:
+            f = lambda v: 0.5 * v * (1.0 + _erf(v / math.sqrt(2.0)))
+        return self._unary64(f, x, name)
+
+    # normalisation ----------------------------------------------------------
+    def batchnorm(self, x, mean, var, eps, scale=None, offset=None, scalar_scale=1.0, scalar_offset=0.0,
+                  name=None):
+        """y = scale * (x - mean) / sqrt(var + eps) + offset over channel axis 1.
+        [ref: odla_dnnl.cc:1448-1524]"""
+        x = _f32(x)
+        C = x.shape[1]
+        sh = (1, C) + (1,) * (x.ndim - 2)
+        g = np.full(C, scalar_scale, np.float64) if scale is None else _f32(scale).astype(np.float64)
+        b = np.full(C, scalar_offset, np.float64) if offset is None else _f32(offset).astype(np.float64)
+        m = g / np.sqrt(_f32(var).astype(np.float64) + float(np.float32(eps)))
+        y = x.astype(np.float64) * m.reshape(sh) + (b - _f32(mean).astype(np.float64) * m).reshape(sh)
+        return self._name(name, y.astype(np.float32))
+
+    def layernorm(self, x, n_axes, eps, scale=None, offset=None, name=None):
+        """Biased variance over the trailing n_axes axes, eps inside the root.
+        [ref: lib/transforms/fusion.cc:296-313]"""
+        x64 = _f32(x).astype(np.float64)
+        ax = tuple(range(x64.ndim - n_axes, x64.ndim))
+        mu = x64.mean(axis=ax, keepdims=True)
+        var = ((x64 - mu) ** 2).mean(axis=ax, keepdims=True)
+        y = (x64 - mu) / np.sqrt(var + float(np.float32(eps)))
+        if scale is not None:
+            y = y * _f32(scale).astype(np.float64).reshape(x64.shape[-n_axes:])
+        if offset is not None:
+            y = y + _f32(offset).astype(np.float64).reshape(x64.shape[-n_axes:])
+        return self._name(name, y.astype(np.float32))
+
+    def softmax(self, x, axis=-1, log=False, name=None):
+        """[ref: odla_dnnl.cc:1628-1669]; every negative axis means the last one."""
+        x64 = _f32(x).astype(np.float64)
+        if axis < 0:
+            axis = x64.ndim - 1
+        z = x64 - x64.max(axis=axis, keepdims=True)
+        e = np.exp(z)
+        s = e.sum(axis=axis, keepdims=True)
+        y = z - np.log(s) if log else e / s
+        return self._name(name, y.astype(np.float32))
+
+    def reduce_mean(self, x, axes, keep_dims=True, name=None):
+        """[ref: odla_dnnl_statistics.cc:20-46,111-117]"""
+        y = _f32(x).astype(np.float64).mean(axis=tuple(axes), keepdims=bool(keep_dims))
+        return self._name(name, y.astype(np.float32))
+
+    def reduce_sum(self, x, axes, keep_dims=True, name=None):
+        y = _f32(x).astype(np.float64).sum(axis=tuple(axes), keepdims=bool(keep_dims))
+        return self._name(name, y.astype(np.float32))
+
+    def reduce_max(self, x, axes, keep_dims=True, name=None):
+        return self._name(name, _f32(x).max(axis=tuple(axes), keepdims=bool(keep_dims)))
+
+    # data movement ----------------------------------------------------------
+    def cast(self, x, dtype, name=None): return self._name(name, np.asarray(x).astype(dtype))
+    def concat(self, xs, axis, name=None): return self._name(name, np.concatenate(xs, axis=axis))
+    def gather(self, x, idx, axis=0, name=None): return self._name(name, np.take(x, np.asarray(idx), axis=axis))
+    def reshape(self, x, shape, name=None): return self._name(name, np.reshape(x, shape))
+    def transpose(self, x, perm, name=None): return self._name(name, np.ascontiguousarray(np.transpose(x, perm)))
+
+    def slice(self, x, start, end, stride=None, name=None):
+        stride = stride or [1] * len(start)
+        sl = tuple(slice(s, e, t) for s, e, t in zip(start, end, stride))
+        return self._name(name, np.ascontiguousarray(x[sl]))
+
+    def resize_nearest(self, x, out_hw, name=None):
+        """src index = floor(dst * in / out).  [ref: ODLA/platforms/odla_eigen.cc:602-632]"""
+        x = np.asarray(x)
+        H, W = x.shape[2], x.shape[3]
+        hi = (np.arange(out_hw[0]) * H) // out_hw[0]
+        wi = (np.arange(out_hw[1]) * W) // out_hw[1]
+        return self._name(name, np.ascontiguousarray(x[:, :, hi][:, :, :, wi]))
+
+    # quantisation -----------------------------------------------------------
+    def quantize(self, x, scale, zp=None, axis=-1, signed=False, name=None):
+        """[ref: odla_dnnl_quantization.cc:61-90]"""
+        x = _f32(x)
+        scale = _f32(scale).reshape(-1)
+        sh = [1] * x.ndim
+        if scale.size > 1:
+            sh[axis] = scale.size
+        t = np.rint(x / scale.reshape(sh))
+        if zp is not None:
+            t = t + np.asarray(zp, dtype=np.float32).reshape(sh)
+        lo, hi, dt = (-128, 127, np.int8) if signed else (0, 255, np.uint8)
+        return self._name(name, np.clip(t, lo, hi).astype(dt))
+
+    def dequantize(self, q, scale, zp=None, axis=-1, name=None):
+        """[ref: odla_dnnl_quantization.cc:33-59]"""
+        q = np.asarray(q)
+        scale = _f32(scale).reshape(-1)
+        sh = [1] * q.ndim
+        if scale.size > 1:
+            sh[axis] = scale.size
+        f = q.astype(np.float32)
+        if zp is not None:
+            f = f - np.asarray(zp, dtype=np.float32).reshape(sh)
+        return self._name(name, (f * scale.reshape(sh)).astype(np.float32))
+
+    def nms(self, boxes, scores, max_out, iou_thr, score_thr, name=None):
+        return self._name(name, nms(boxes, scores, max_out, iou_thr, score_thr))

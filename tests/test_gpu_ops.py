@@ -1,0 +1,580 @@
+"""Per-operator parity: libodla_hip.so (through the ODLA C ABI) against the CPU
+oracle on identical seeded inputs, plus the reference-held known-answer
+vectors replayed through the ABI exactly as the reference's doctest suite
+calls it (ODLA/platforms/odla_popart/test/*.cc of the reference tree).
+
+Tolerances: fp32 graphs 1e-4 of the largest expected magnitude; fp16 / bf16
+storage 2e-2 absolute on O(1) data; integer results bit-exact.
+"""
+import numpy as np
+import pytest
+
+from util import announce, max_rel_err, run_both, run_hip
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-4
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# --------------------------------------------------------------------------
+# Known-answer vectors held by the reference's own tests
+# --------------------------------------------------------------------------
+def test_kat_conv_runtime_kernel():
+    """odla_ops_nn_test.cc:147-200: 5x5 ramp * ones 3x3, pad 1; the kernel is an argument."""
+    announce("kat conv")
+
+    def build(b):
+        x = b.arg("input", (1, 1, 5, 5))
+        k = b.arg("kernel", (1, 1, 3, 3))
+        b.output(b.conv(x, k, None, (1, 1), (1, 1, 1, 1), name="Conv"), "Conv")
+
+    feeds = {"input": np.arange(25, dtype=np.float32).reshape(1, 1, 5, 5),
+             "kernel": np.ones((1, 1, 3, 3), np.float32)}
+    got = run_hip(build, feeds)["Conv"].reshape(-1)
+    expected = [12, 21, 27, 33, 24, 33, 54, 63, 72, 51, 63, 99, 108, 117, 81, 93, 144, 153, 162, 111, 72, 111,
+                117, 123, 84]
+    assert got.tolist() == [float(v) for v in expected]
+
+
+def test_kat_pools():
+    """odla_ops_nn_test.cc:38-78 (avg -> 6,7,10,11) and :523-560 (max -> 11,12,15,16)."""
+    announce("kat pools")
+    x = np.arange(1, 17, dtype=np.float32).reshape(1, 1, 4, 4)
+
+    def build(b):
+        v = b.arg("input", (1, 1, 4, 4))
+        b.output(b.avgpool(v, (3, 3), (1, 1), (0, 0, 0, 0), name="avg"), "avg")
+        b.output(b.maxpool(v, (3, 3), (1, 1), (0, 0, 0, 0), name="max"), "max")
+
+    got = run_hip(build, {"input": x})
+    assert np.allclose(got["avg"].reshape(-1), [6, 7, 10, 11], atol=1e-5)
+    assert got["max"].reshape(-1).tolist() == [11, 12, 15, 16]
+
+
+def test_kat_batchnorm_runtime_params():
+    """odla_ops_nn_test.cc:80-145: statistics passed as arguments."""
+    announce("kat batchnorm")
+
+    def build(b):
+        x = b.arg("input", (1, 2, 1, 3))
+        sc = b.arg("scale", (2,))
+        of = b.arg("offset", (2,))
+        mean = b.arg("mean", (2,))
+        var = b.arg("var", (2,))
+        b.output(b.batchnorm(x, mean, var, 1e-5, sc, of, 1.0, 1.0, name="bn"), "bn")
+
+    feeds = {"input": np.array([-1, 0, 1, 2, 3, 4], np.float32).reshape(1, 2, 1, 3),
+             "scale": np.array([1.0, 1.5], np.float32), "offset": np.array([0, 1], np.float32),
+             "mean": np.array([0, 3], np.float32), "var": np.array([1, 1.5], np.float32)}
+    got = run_hip(build, feeds)["bn"].reshape(-1)
+    expected = np.array([-0.999995, 0, 0.999995, -0.224741, 1, 2.22474])
+    assert np.max(np.abs(got - expected)) < 1e-5
+
+
+def test_kat_leakyrelu_relu_gemm():
+    """odla_ops_nn_test.cc:393-422, odla_ops_test.cc:240-267 and :39-79."""
+    announce("kat leakyrelu/relu/gemm")
+
+    def build(b):
+        x = b.arg("x", (1, 3))
+        b.output(b.leaky_relu(x, 0.1, name="lr"), "lr")
+        b.output(b.relu(x, name="r"), "r")
+        a = b.arg("a", (4, 16))
+        w = b.arg("w", (16, 8))
+        b.output(b.gemm(a, w, None, False, False, 1.0, 0.0, name="g"), "g")
+
+    feeds = {"x": np.array([[-1, 0, 1]], np.float32), "a": np.ones((4, 16), np.float32),
+             "w": np.ones((16, 8), np.float32)}
+    got = run_hip(build, feeds)
+    assert np.allclose(got["lr"].reshape(-1), [-0.1, 0, 1], atol=1e-7)
+    assert got["r"].reshape(-1).tolist() == [0, 0, 1]
+    assert np.all(got["g"] == 16.0)
+
+
+def test_kat_executor_scaffold():
+    """tests/compile/test_cxx_gen.cc:46-48 of the reference: (input + w0) * w1 -> 6, 9, 12."""
+    announce("kat executor scaffold")
+
+    def build(b):
+        x = b.arg("input", (3,))
+        w0 = b.const("w0", np.array([1, 1, 1], np.float32))
+        w1 = b.const("w1", np.array([3, 3, 3], np.float32))
+        b.output(b.mul(b.add(x, w0, name="add"), w1, name="mul"), "mul")
+
+    got = run_hip(build, {"input": np.array([1, 2, 3], np.float32)})["mul"]
+    assert got.tolist() == [6, 9, 12]
+
+
+# --------------------------------------------------------------------------
+# Convolution
+# --------------------------------------------------------------------------
+CONV_CASES = [
+    # N, C, H, W, O, k, stride, pad, group, dilation
+    (2, 16, 14, 14, 32, 3, 1, 1, 1, 1),
+    (2, 16, 15, 13, 24, 3, 2, 1, 1, 1),
+    (3, 64, 9, 9, 64, 1, 1, 0, 1, 1),
+    (2, 3, 32, 32, 16, 7, 2, 3, 1, 1),
+    (1, 32, 12, 12, 130, 1, 2, 0, 1, 1),
+    (2, 8, 10, 10, 8, 3, 1, 2, 1, 2),
+    (2, 32, 8, 8, 64, 3, 1, 1, 2, 1),
+    (1, 20, 7, 7, 255, 1, 1, 0, 1, 1),
+    (1, 4, 5, 5, 4, 5, 1, 0, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16"])
+def test_conv_parity(case, mode):
+    N, C, H, W, O, k, s, p, g, d = case
+    announce("conv %s %s" % (mode, case))
+    r = rng(hash(case) % 1000)
+    w = (r.standard_normal((O, C // g, k, k)) * np.sqrt(2.0 / (C // g * k * k))).astype(np.float32)
+    bias = r.standard_normal(O).astype(np.float32)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+
+    def build(b):
+        v = b.arg("x", (N, C, H, W))
+        y = b.conv(v, b.const("w", w), b.const("b", bias), (s, s), (p, p, p, p), (d, d), g, name="y")
+        b.output(y, "y")
+
+    kw = {"fp16": mode == "fp16", "bf16": mode == "bf16"}
+    got, want = run_both(build, {"x": x}, **kw)
+    assert got["y"].shape == want["y"].shape
+    if mode == "fp32":
+        assert max_rel_err(got["y"], want["y"]) <= F32_TOL
+    else:
+        tol = 2e-2 if mode == "fp16" else 6e-2
+        assert np.max(np.abs(got["y"] - want["y"])) <= tol * max(1.0, float(np.max(np.abs(want["y"]))))
+
+
+def test_conv_fused_chain_fp32():
+    """Conv + per-channel Add + BatchNorm + residual Add + ReLU collapses into one
+    launch and must equal the unfused oracle sequence."""
+    announce("conv fused chain")
+    r = rng(5)
+    N, C, H, W, O = 2, 16, 12, 12, 32
+    w = (r.standard_normal((O, C, 3, 3)) * 0.1).astype(np.float32)
+    extra = r.standard_normal((1, O, 1, 1)).astype(np.float32)
+    mean, var = r.standard_normal(O).astype(np.float32), (r.random(O) + 0.5).astype(np.float32)
+    gam, bet = r.standard_normal(O).astype(np.float32), r.standard_normal(O).astype(np.float32)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    res = r.standard_normal((N, O, H, W)).astype(np.float32)
+
+    def build(b):
+        v = b.arg("x", (N, C, H, W))
+        rr = b.arg("res", (N, O, H, W))
+        rr2 = b.relu(rr, name="res_relu")   # a computed residual
+        y = b.conv(v, b.const("w", w), None, (1, 1), (1, 1, 1, 1), name="c")
+        y = b.add(y, b.const("extra", extra), name="a0")
+        y = b.batchnorm(y, b.const("m", mean), b.const("v", var), 1e-5, b.const("g", gam), b.const("be", bet), name="bn")
+        y = b.add(y, rr2, name="a1")
+        y = b.relu(y, name="out")
+        b.output(y, "out")
+
+    got, want = run_both(build, {"x": x, "res": res})
+    assert max_rel_err(got["out"], want["out"]) <= F32_TOL
+
+
+# --------------------------------------------------------------------------
+# Gemm
+# --------------------------------------------------------------------------
+GEMM_CASES = [
+    # M, K, N, tA, tB, alpha, beta, bias kind, const B
+    (64, 784, 10, False, False, 1.0, 0.0, None, True),
+    (33, 40, 17, False, True, 0.5, 2.0, "row", True),
+    (16, 24, 32, True, False, 1.0, 1.0, "scalar", True),
+    (20, 36, 12, False, False, 1.0, 0.0, None, False),
+    (20, 36, 12, False, True, 1.0, 0.0, None, False),
+    (7, 10, 5, False, False, 1.0, 1.0, "row", True),
+]
+
+
+@pytest.mark.parametrize("case", GEMM_CASES)
+def test_gemm_parity(case):
+    M, K, N, tA, tB, alpha, beta, bias, const_b = case
+    announce("gemm %s" % (case,))
+    r = rng(11)
+    A = r.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    Cb = None
+    if bias == "row":
+        Cb = r.standard_normal((N,)).astype(np.float32)
+    elif bias == "scalar":
+        Cb = r.standard_normal((1,)).astype(np.float32)
+
+    def build(b):
+        a = b.arg("A", A.shape)
+        bb = b.const("B", B) if const_b else b.arg("B", B.shape)
+        c = b.const("C", Cb) if Cb is not None else None
+        b.output(b.gemm(a, bb, c, tA, tB, alpha, beta, name="y"), "y")
+
+    feeds = {"A": A}
+    if not const_b:
+        feeds["B"] = B
+    got, want = run_both(build, feeds)
+    assert max_rel_err(got["y"], want["y"]) <= F32_TOL
+
+
+def test_batched_gemm_parity():
+    announce("batched gemm")
+    r = rng(12)
+    q = r.standard_normal((2, 3, 16, 8)).astype(np.float32)
+    k = r.standard_normal((2, 3, 16, 8)).astype(np.float32)
+    v = r.standard_normal((2, 3, 16, 8)).astype(np.float32)
+    wt = r.standard_normal((8, 12)).astype(np.float32)
+
+    def build(b):
+        qq, kk, vv = b.arg("q", q.shape), b.arg("k", k.shape), b.arg("v", v.shape)
+        s = b.gemm(qq, kk, None, False, True, 0.125, 0.0, name="s")        # [2,3,16,16]
+        p = b.softmax(s, -1, name="p")
+        o = b.gemm(p, vv, None, False, False, 1.0, 0.0, name="o")           # [2,3,16,8]
+        z = b.gemm(o, b.const("w", wt), None, False, False, 1.0, 0.0, name="z")  # rank-2 weights
+        b.output(s, "s")
+        b.output(o, "o")
+        b.output(z, "z")
+
+    got, want = run_both(build, {"q": q, "k": k, "v": v})
+    for name in ("s", "o", "z"):
+        assert max_rel_err(got[name], want[name]) <= F32_TOL, name
+
+
+# --------------------------------------------------------------------------
+# Element-wise, normalisation, reductions
+# --------------------------------------------------------------------------
+def test_binary_broadcast_parity():
+    announce("binary broadcast")
+    r = rng(21)
+    x = r.standard_normal((2, 6, 5, 7)).astype(np.float32)
+    y = r.standard_normal((2, 6, 5, 7)).astype(np.float32) + 3.0
+    c1 = r.standard_normal((1, 6, 1, 1)).astype(np.float32)
+    c2 = r.standard_normal((7,)).astype(np.float32)
+    c3 = r.standard_normal((6, 1, 1)).astype(np.float32)
+    c4 = r.standard_normal((1,)).astype(np.float32)
+
+    def build(b):
+        a, bb = b.arg("x", x.shape), b.arg("y", y.shape)
+        b.output(b.add(a, bb, name="o_add"), "o_add")
+        b.output(b.div(a, bb, name="o_div"), "o_div")
+        b.output(b.mul(a, b.const("c1", c1), name="o_c1"), "o_c1")
+        b.output(b.sub(b.const("c2", c2), a, name="o_c2"), "o_c2")
+        b.output(b.max(a, b.const("c3", c3), name="o_c3"), "o_c3")
+        b.output(b.min(a, b.const("c4", c4), name="o_c4"), "o_c4")
+
+    got, want = run_both(build, {"x": x, "y": y})
+    for k in want:
+        assert max_rel_err(got[k], want[k]) <= 1e-6, k
+
+
+def test_reference_alignment_quirk():
+    """[64] against [1,64,128] aligns with dim 1 (odla_dnnl.h:301-343), not with the last dim."""
+    announce("alignment quirk")
+    r = rng(22)
+    x = r.standard_normal((1, 64, 128)).astype(np.float32)
+    c = r.standard_normal((64,)).astype(np.float32)
+
+    def build(b):
+        b.output(b.add(b.arg("x", x.shape), b.const("c", c), name="y"), "y")
+
+    got, want = run_both(build, {"x": x})
+    assert np.array_equal(want["y"], x + c.reshape(1, 64, 1))
+    assert max_rel_err(got["y"], want["y"]) <= 1e-6
+
+
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def test_unary_parity(mode):
+    announce("unary %s" % mode)
+    r = rng(23)
+    x = (r.standard_normal((3, 5, 37)) * 2).astype(np.float32)
+    pos = (r.random((3, 5, 37)) + 0.1).astype(np.float32)
+
+    def build(b):
+        a, p = b.arg("x", x.shape), b.arg("pos", pos.shape)
+        for name in ("relu", "sigmoid", "tanh", "exp", "erf", "abs", "neg"):
+            b.output(getattr(b, name)(a, name=name), name)
+        b.output(b.gelu(a, False, name="gelu"), "gelu")
+        b.output(b.gelu(a, True, name="gelu_tanh"), "gelu_tanh")
+        b.output(b.leaky_relu(a, 0.1, name="leaky"), "leaky")
+        b.output(b.clamp(a, -0.5, 0.75, name="clamp"), "clamp")
+        for name in ("sqrt", "rsqrt", "log"):
+            b.output(getattr(b, name)(p, name=name), name)
+
+    got, want = run_both(build, {"x": x, "pos": pos}, fp16=(mode == "fp16"))
+    for k in want:
+        if mode == "fp32":
+            assert max_rel_err(got[k], want[k]) <= F32_TOL, k
+        else:
+            assert np.max(np.abs(got[k] - want[k])) <= 2e-2 * max(1.0, float(np.max(np.abs(want[k])))), k
+
+
+def test_round_half_even():
+    announce("round")
+    x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, 2.4999, 3.5], np.float32)
+
+    def build(b):
+        b.output(b.round(b.arg("x", x.shape), name="y"), "y")
+
+    got = run_hip(build, {"x": x})["y"]
+    assert got.tolist() == [0, 2, 2, -0, -2, 2, 4]
+
+
+@pytest.mark.parametrize("shape,axis", [((64, 10), -1), ((256, 1000), 1), ((4, 12, 16, 16), 3), ((3, 7, 5), 1),
+                                        ((2, 3000), 1)])
+def test_softmax_parity(shape, axis):
+    announce("softmax %s axis %d" % (shape, axis))
+    x = (rng(31).standard_normal(shape) * 3).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", shape)
+        b.output(b.softmax(a, axis, name="y"), "y")
+        b.output(b.softmax(a, axis, log=True, name="ly"), "ly")
+
+    got, want = run_both(build, {"x": x})
+    assert max_rel_err(got["y"], want["y"]) <= F32_TOL
+    assert np.max(np.abs(got["ly"] - want["ly"])) <= 1e-4
+    ax = len(shape) - 1 if axis < 0 else axis
+    assert np.allclose(got["y"].sum(axis=ax), 1.0, atol=1e-5)
+
+
+def test_softmax_large_numbers():
+    """ONNX softmax_large_number: inputs near 10000 must not overflow."""
+    announce("softmax large")
+    x = np.array([[0, 1, 2, 3], [10000, 10001, 10002, 10003]], np.float32)
+
+    def build(b):
+        b.output(b.softmax(b.arg("x", x.shape), -1, name="y"), "y")
+
+    got = run_hip(build, {"x": x})["y"]
+    expected = np.array([0.032058604, 0.08714432, 0.23688284, 0.6439143], np.float32)
+    assert np.allclose(got[0], expected, atol=1e-6) and np.allclose(got[1], expected, atol=1e-6)
+
+
+@pytest.mark.parametrize("mode", ["fp32", "bf16"])
+def test_layernorm_parity(mode):
+    announce("layernorm %s" % mode)
+    r = rng(41)
+    x = r.standard_normal((4, 9, 768)).astype(np.float32) * 2 + 0.5
+    g = r.standard_normal(768).astype(np.float32)
+    be = r.standard_normal(768).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        b.output(b.layernorm(a, 1, 1e-12, b.const("g", g), b.const("b", be), name="y"), "y")
+
+    got, want = run_both(build, {"x": x}, bf16=(mode == "bf16"))
+    if mode == "fp32":
+        assert max_rel_err(got["y"], want["y"]) <= F32_TOL
+    else:
+        assert np.max(np.abs(got["y"] - want["y"])) <= 6e-2 * float(np.max(np.abs(want["y"])))
+
+
+def test_batchnorm_standalone_parity():
+    announce("batchnorm standalone")
+    r = rng(42)
+    x = r.standard_normal((2, 12, 6, 5)).astype(np.float32)
+    mean, var = r.standard_normal(12).astype(np.float32), (r.random(12) + 0.5).astype(np.float32)
+    g, be = r.standard_normal(12).astype(np.float32), r.standard_normal(12).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        a2 = b.neg(a, name="neg")  # keep the BN from folding into anything
+        b.output(b.batchnorm(a2, b.const("m", mean), b.const("v", var), 1e-3, b.const("g", g), b.const("b", be), name="y"), "y")
+
+    got, want = run_both(build, {"x": x})
+    assert max_rel_err(got["y"], want["y"]) <= F32_TOL
+
+
+POOL_CASES = [
+    # N, C, H, W, k, s, pad(t,l,b,r), include_pad
+    (2, 16, 12, 12, 3, 2, (1, 1, 1, 1), False),
+    (1, 5, 9, 7, 2, 2, (0, 0, 0, 0), False),
+    (2, 8, 7, 7, 7, 1, (0, 0, 0, 0), False),
+    (1, 3, 8, 8, 3, 1, (1, 1, 1, 1), True),
+    (1, 4, 6, 6, 3, 2, (0, 0, 1, 1), False),
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_pool_parity(case):
+    N, C, H, W, k, s, pad, incl = case
+    announce("pool %s" % (case,))
+    x = rng(51).standard_normal((N, C, H, W)).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        b.output(b.maxpool(a, (k, k), (s, s), pad, name="mx"), "mx")
+        b.output(b.avgpool(a, (k, k), (s, s), pad, incl, name="av"), "av")
+
+    got, want = run_both(build, {"x": x})
+    assert np.array_equal(got["mx"], want["mx"])
+    assert max_rel_err(got["av"], want["av"]) <= 1e-6
+
+
+def test_reduce_parity():
+    announce("reduce")
+    x = rng(52).standard_normal((3, 10, 7, 7)).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        b.output(b.reduce_mean(a, (2, 3), True, name="gap"), "gap")
+        b.output(b.reduce_mean(a, (3,), False, name="last"), "last")
+        b.output(b.reduce_sum(a, (1,), True, name="mid"), "mid")
+        b.output(b.reduce_max(a, (1, 2, 3), False, name="mx"), "mx")
+
+    got, want = run_both(build, {"x": x})
+    for k in want:
+        assert got[k].shape == want[k].shape, k
+        assert max_rel_err(got[k], want[k]) <= 1e-5, k
+
+
+# --------------------------------------------------------------------------
+# Data movement
+# --------------------------------------------------------------------------
+def test_movement_parity():
+    announce("movement")
+    r = rng(61)
+    x = r.standard_normal((2, 6, 4, 5)).astype(np.float32)
+    y = r.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    table = r.standard_normal((50, 16)).astype(np.float32)
+    idx = r.integers(0, 50, size=(3, 7)).astype(np.int32)
+    idx64 = r.integers(0, 50, size=(5,)).astype(np.int64)
+
+    def build(b):
+        a, c = b.arg("x", x.shape), b.arg("y", y.shape)
+        b.output(b.concat([a, c], 1, name="cat1"), "cat1")
+        b.output(b.concat([a, a], 3, name="cat3"), "cat3")
+        b.output(b.transpose(a, (0, 2, 3, 1), name="nhwc"), "nhwc")
+        b.output(b.transpose(a, (1, 0, 3, 2), name="t2"), "t2")
+        b.output(b.reshape(a, (2, 6, 20), name="rs"), "rs")
+        b.output(b.slice(a, (0, 1, 0, 2), (2, 5, 4, 5), (1, 2, 1, 1), name="sl"), "sl")
+        b.output(b.resize_nearest(a, (8, 10), name="up2"), "up2")
+        b.output(b.resize_nearest(a, (6, 7), name="upx"), "upx")
+        t = b.const("table", table)
+        b.output(b.gather(t, b.arg("idx", idx.shape, np.int32), 0, name="emb"), "emb")
+        b.output(b.gather(t, b.arg("idx64", idx64.shape, np.int64), 0, name="emb64"), "emb64")
+
+    got, want = run_both(build, {"x": x, "y": y, "idx": idx, "idx64": idx64})
+    for k in want:
+        assert got[k].shape == want[k].shape, k
+        assert np.array_equal(got[k], want[k]), k
+
+
+def test_nhwc_chain_then_concat_resize():
+    """Conv -> LeakyReLU -> nearest 2x -> channel concat stays channels-last on the device."""
+    announce("nhwc chain")
+    r = rng(62)
+    x = r.standard_normal((2, 8, 6, 6)).astype(np.float32)
+    skip = r.standard_normal((2, 16, 12, 12)).astype(np.float32)
+    w1 = (r.standard_normal((8, 8, 3, 3)) * 0.2).astype(np.float32)
+    w2 = (r.standard_normal((16, 16, 1, 1)) * 0.2).astype(np.float32)
+    w3 = (r.standard_normal((255, 24, 1, 1)) * 0.2).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        s = b.arg("skip", skip.shape)
+        y = b.leaky_relu(b.conv(a, b.const("w1", w1), None, (1, 1), (1, 1, 1, 1), name="c1"), 0.1, name="l1")
+        up = b.resize_nearest(y, (12, 12), name="up")
+        s2 = b.leaky_relu(b.conv(s, b.const("w2", w2), None, name="c2"), 0.1, name="l2")
+        cat = b.concat([up, s2], 1, name="cat")
+        head = b.conv(cat, b.const("w3", w3), None, name="head")
+        b.output(head, "head")
+        b.output(b.sigmoid(head, name="sig"), "sig")
+
+    got, want = run_both(build, {"x": x, "skip": skip})
+    assert max_rel_err(got["head"], want["head"]) <= F32_TOL
+    assert max_rel_err(got["sig"], want["sig"]) <= F32_TOL
+
+
+# --------------------------------------------------------------------------
+# Quantize / Dequantize
+# --------------------------------------------------------------------------
+def test_quantize_onnx_example():
+    """ONNX QuantizeLinear example (passes on the reference CPU backend):
+    rounding at 1.5 -> 2 and saturation at both ends."""
+    announce("quantize onnx example")
+    x = np.array([0, 2, 3, 1000, -254, -1000], np.float32)
+
+    def build(b):
+        q = b.quantize(b.arg("x", x.shape), [2.0], [128], name="q")
+        b.output(q, "q")
+        b.output(b.dequantize(q, [2.0], [128], name="dq"), "dq")
+
+    got = run_hip(build, {"x": x})
+    assert got["q"].tolist() == [128, 129, 130, 255, 1, 0]
+    assert got["dq"].tolist() == [0, 2, 4, 254, -254, -256]
+
+
+def test_quantize_parity_per_axis_and_ties():
+    announce("quantize per axis")
+    r = rng(71)
+    x = (r.standard_normal((2, 4, 9)) * 40).astype(np.float32)
+    # exact ties: k + 0.5 multiples of the scale
+    x[0, 0, :] = (np.arange(9, dtype=np.float32) - 4 + 0.5) * 0.25
+    sc = np.array([0.25, 0.5, 1.0, 2.0], np.float32)
+    zp = np.array([0, 10, 128, 200], np.uint8)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        q = b.quantize(a, sc, zp, axis=1, name="q")
+        b.output(q, "q")
+        b.output(b.dequantize(q, sc, zp, axis=1, name="dq"), "dq")
+        b.output(b.quantize(a, [0.5], None, signed=True, name="qs"), "qs")
+
+    got, want = run_both(build, {"x": x})
+    assert np.array_equal(got["q"], want["q"])
+    assert np.array_equal(got["dq"], want["dq"])
+    assert np.array_equal(got["qs"], want["qs"])
+
+
+# --------------------------------------------------------------------------
+# NMS
+# --------------------------------------------------------------------------
+def test_nms_onnx_examples():
+    """Published ONNX NonMaxSuppression cases (single class): suppress by IoU ->
+    [3, 0, 5]; identical boxes -> 1 box; flipped coordinates; score threshold."""
+    announce("nms onnx examples")
+    boxes = np.array([[[0, 0, 1, 1], [0, 0.1, 1, 1.1], [0, -0.1, 1, 0.9], [0, 10, 1, 11], [0, 10.1, 1, 11.1],
+                       [0, 100, 1, 101]]], np.float32)
+    flipped = np.array([[[1, 1, 0, 0], [0, 0.1, 1, 1.1], [0, 0.9, 1, -0.1], [0, 10, 1, 11], [1, 10.1, 0, 11.1],
+                         [1, 101, 0, 100]]], np.float32)
+    scores = np.array([[[0.9, 0.75, 0.6, 0.95, 0.5, 0.3]]], np.float32)
+    same = np.tile(np.array([0, 0, 1, 1], np.float32), (1, 10, 1))
+    same_scores = np.full((1, 1, 10), 0.9, np.float32)
+
+    def build(b):
+        bx, sc = b.arg("boxes", boxes.shape), b.arg("scores", scores.shape)
+        fl = b.arg("flipped", flipped.shape)
+        sm, ss = b.arg("same", same.shape), b.arg("same_scores", same_scores.shape)
+        b.output(b.nms(bx, sc, 3, 0.5, 0.0, name="a"), "a")
+        b.output(b.nms(fl, sc, 3, 0.5, 0.0, name="f"), "f")
+        b.output(b.nms(bx, sc, 3, 0.5, 0.4, name="t"), "t")
+        b.output(b.nms(bx, sc, 2, 0.5, 0.0, name="m2"), "m2")
+        b.output(b.nms(sm, ss, 3, 0.5, 0.0, name="s"), "s")
+
+    got = run_hip(build, {"boxes": boxes, "scores": scores, "flipped": flipped, "same": same,
+                          "same_scores": same_scores})
+    assert got["a"].tolist() == [[0, 0, 3], [0, 0, 0], [0, 0, 5]]
+    assert got["f"].tolist() == [[0, 0, 3], [0, 0, 0], [0, 0, 5]]
+    assert got["t"].tolist() == [[0, 0, 3], [0, 0, 0], [-1, -1, -1]]
+    assert got["m2"].tolist() == [[0, 0, 3], [0, 0, 0]]
+    assert got["s"].tolist() == [[0, 0, 0], [-1, -1, -1], [-1, -1, -1]]
+
+
+@pytest.mark.parametrize("N,B,C,max_out", [(2, 200, 5, 20), (3, 1500, 80, 100), (1, 64, 1, 64)])
+def test_nms_parity_random(N, B, C, max_out):
+    announce("nms random %s" % ((N, B, C, max_out),))
+    r = rng(81 + B)
+    cy, cx = r.random((N, B)) * 10, r.random((N, B)) * 10
+    h, w = r.random((N, B)) * 2 + 0.2, r.random((N, B)) * 2 + 0.2
+    boxes = np.stack([cy - h / 2, cx - w / 2, cy + h / 2, cx + w / 2], axis=-1).astype(np.float32)
+    scores = r.random((N, C, B)).astype(np.float32) ** 4
+    scores[:, :, :5] = 0.77  # ties resolved by box index
+
+    def build(b):
+        b.output(b.nms(b.arg("boxes", boxes.shape), b.arg("scores", scores.shape), max_out, 0.45, 0.3, name="y"), "y")
+
+    got, want = run_both(build, {"boxes": boxes, "scores": scores})
+    assert np.array_equal(got["y"], want["y"])
