@@ -178,6 +178,22 @@ odla_status run_steps(_odla_context* ctx, const Plan& plan) {
   return ODLA_SUCCESS;
 }
 
+odla_status stage_inputs(_odla_context* ctx, const Plan& plan) {
+  for (const Plan::IO& io : plan.inputs) {
+    auto it = ctx->bound_in.find(io.v);
+    if (it == ctx->bound_in.end()) {
+      OHIP_ERR("argument '%s' is not bound", io.v->name.c_str());
+      return ODLA_INVALID_PARAM;
+    }
+    char* dst = ctx->arena + plan.tensors[io.tensor].offset;
+    if (hipMemcpyAsync(dst, it->second, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
+      OHIP_ERR("copy of argument '%s' failed", io.v->name.c_str());
+      return ODLA_FAILURE;
+    }
+  }
+  return ODLA_SUCCESS;
+}
+
 _odla_value* find_value(_odla_computation* c, const odla_value_id id) {
   if (c == nullptr || id == nullptr) return nullptr;
   auto it = c->by_name.find(reinterpret_cast<const char*>(id));
@@ -359,17 +375,9 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
   const Plan& plan = *c->plan;
 
   // 1. stage arguments (host -> device across PCIe, or device -> device)
-  for (const Plan::IO& io : plan.inputs) {
-    auto it = ctx->bound_in.find(io.v);
-    if (it == ctx->bound_in.end()) {
-      OHIP_ERR("odla_ExecuteComputation: argument '%s' is not bound", io.v->name.c_str());
-      return ODLA_INVALID_PARAM;
-    }
-    char* dst = ctx->arena + plan.tensors[io.tensor].offset;
-    if (hipMemcpyAsync(dst, it->second, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
-      OHIP_ERR("odla_ExecuteComputation: copy of argument '%s' failed", io.v->name.c_str());
-      return ODLA_FAILURE;
-    }
+  {
+    odla_status st = stage_inputs(ctx, plan);
+    if (st != ODLA_SUCCESS) return st;
   }
 
   // 2. launch sequence: captured once into a hipGraph, replayed afterwards
@@ -420,6 +428,49 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
     return ODLA_FAILURE;
   }
   ctx->executed = true;
+  return ODLA_SUCCESS;
+}
+
+// Diagnostic: run the launch sequence un-captured `iters` times with a HIP
+// event pair around every step on the context's stream and report the mean
+// duration of each step.  Arguments must be bound.
+odla_status odla_hip_ProfileSteps(odla_context ctx, odla_int32 iters, odla_hip_step_time* out,
+                                  odla_int32 capacity, odla_int32* count) {
+  if (ctx == nullptr || out == nullptr || count == nullptr || iters <= 0) return ODLA_INVALID_PARAM;
+  _odla_computation* c = ctx->comp;
+  if (!c->plan) return ODLA_FAILURE;
+  const Plan& plan = *c->plan;
+  const int n = (int)plan.steps.size();
+  if (n > capacity) return ODLA_INVALID_PARAM;
+  std::vector<hipEvent_t> ev((size_t)n * 2);
+  for (auto& e : ev)
+    if (hipEventCreate(&e) != hipSuccess) return ODLA_FAILURE;
+  std::vector<double> acc((size_t)n, 0.0);
+  ExecEnv env;
+  env.base[SP_ARENA] = ctx->arena;
+  env.base[SP_CONST] = plan.const_pool;
+  odla_status st = ODLA_SUCCESS;
+  for (int it = 0; it < iters && st == ODLA_SUCCESS; ++it) {
+    st = stage_inputs(ctx, plan);
+    for (int i = 0; i < n && st == ODLA_SUCCESS; ++i) {
+      (void)hipEventRecord(ev[2 * i], ctx->stream);
+      if (plan.steps[i].fn(env, ctx->stream) != hipSuccess) st = ODLA_FAILURE;
+      (void)hipEventRecord(ev[2 * i + 1], ctx->stream);
+    }
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess) st = ODLA_FAILURE;
+    for (int i = 0; i < n && st == ODLA_SUCCESS; ++i) {
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) != hipSuccess) st = ODLA_FAILURE;
+      acc[i] += ms;
+    }
+  }
+  for (auto& e : ev) (void)hipEventDestroy(e);
+  if (st != ODLA_SUCCESS) return st;
+  for (int i = 0; i < n; ++i) {
+    snprintf(out[i].name, sizeof(out[i].name), "%s", plan.steps[i].name.c_str());
+    out[i].ms = (float)(acc[i] / iters);
+  }
+  *count = n;
   return ODLA_SUCCESS;
 }
 

@@ -1053,7 +1053,7 @@ void Planner::lower_conv(int ni) {
   ip.w_rows = Og; ip.w_cols = w_rs; ip.w_rs = w_rs;
   ip.in_dt = dt; ip.out_dt = dt;
   ip.batch = G;
-  ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og;
+  if (G > 1) { ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og; }
   ip.ycs = (int)O;
 
   int ty;

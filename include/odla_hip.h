@@ -3,8 +3,8 @@
  * Instinct MI355X (gfx950).
  *
  * The library is a drop-in ODLA backend: model code emitted by the HALO
- * compiler (or any program written against ODLA/include/ODLA/*.h of the
- * reference tree) links against it in place of libodla_dnnl.so /
+ * compiler (or any program written against the headers under ODLA/include/ODLA
+ * of the reference tree) links against it in place of libodla_dnnl.so /
  * libodla_tensorrt.so.  Every type below is binary compatible with the
  * reference declaration it cites (x86-64 SysV): enumerator order, struct
  * member order and sizes are part of the ABI and must not change.
@@ -528,6 +528,22 @@ odla_value odla_NMS(odla_value boxes, odla_value scores,
                     odla_float32 score_threshold,
                     odla_value_type output_value_type,
                     const odla_value_id value_id);
+
+/* ------------------------------------------------------------------------ */
+/* Diagnostics (no counterpart in the reference).                            */
+/* ------------------------------------------------------------------------ */
+typedef struct {
+  char name[64]; /* "<kernel class>:<value id>", e.g. "conv:l1b0c2.relu" */
+  float ms;      /* mean duration of the launch                          */
+} odla_hip_step_time;
+
+/* Runs the compiled launch sequence of `context` un-captured `iters` times,
+ * with a HIP event pair around every launch on the context's stream, and
+ * reports the mean duration of each launch in plan order.  Arguments must be
+ * bound.  Used by the benchmark to price kernels against their roofline. */
+odla_status odla_hip_ProfileSteps(odla_context context, odla_int32 iters,
+                                  odla_hip_step_time* out, odla_int32 capacity,
+                                  odla_int32* count);
 
 #ifdef __cplusplus
 } /* extern "C" */
