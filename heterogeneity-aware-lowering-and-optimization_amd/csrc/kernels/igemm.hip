@@ -54,51 +54,70 @@ template <> struct Mma<int8_t> {
 };
 
 // ---------------------------------------------------------------------------
-// Epilogues.  Each handles four consecutive output channels n..n+3 of one
-// output row; `full` says all four are in range and 16-byte style access is ok.
+// Epilogues.  Each handles eight consecutive output channels n..n+7 of one
+// output row; yrow / rrow / bias already point at channel n.  `vec` says all
+// eight are valid and the row pointers allow one vector access.
+
+// Only the cheap activations are fused (a full transcendental switch inlined
+// per element bloats the epilogue until the compiler stops unrolling it and
+// the accumulators fall out of registers); the planner keeps the others as a
+// separate streaming kernel.
+__device__ __forceinline__ float epi_act(float v, ActKind act, float a, float b) {
+  switch (act) {
+    case ACT_RELU: return v > 0.f ? v : 0.f;
+    case ACT_LEAKY: return v > 0.f ? v : a * v;
+    case ACT_CLAMP: return fminf(fmaxf(v, a), b);
+    default: return v;
+  }
+}
 
 template <typename TOut>
 struct EpiFloat {
   using AccE = float;
-  __device__ static __forceinline__ void run(const IgemmParams& p, const float* acc, int n,
-                                             const float* bias4, void* yrow, const void* rrow,
-                                             bool full) {
-    float v[4];
+  __device__ static __forceinline__ void store8(const IgemmParams& p, const float* acc, int nvalid, bool vec,
+                                                const float* bias, TOut* y, const TOut* r) {
+    float v[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = acc[e] * p.alpha + bias4[e];
-    TOut* y = reinterpret_cast<TOut*>(yrow) + n;
-    const TOut* r = reinterpret_cast<const TOut*>(rrow) + n;
-    if (full) {
-      if (rrow != nullptr) {
+    for (int e = 0; e < 8; ++e) v[e] = acc[e] * p.alpha;
+    if (vec) {
+      if (bias != nullptr) {
+        const floatx4 b0 = *reinterpret_cast<const floatx4*>(bias);
+        const floatx4 b1 = *reinterpret_cast<const floatx4*>(bias + 4);
+        v[0] += b0.x; v[1] += b0.y; v[2] += b0.z; v[3] += b0.w;
+        v[4] += b1.x; v[5] += b1.y; v[6] += b1.z; v[7] += b1.w;
+      }
+      if (r != nullptr) {
         if constexpr (sizeof(TOut) == 4) {
-          floatx4 rv = *reinterpret_cast<const floatx4*>(r);
-          v[0] += rv.x; v[1] += rv.y; v[2] += rv.z; v[3] += rv.w;
+          const floatx4 r0 = *reinterpret_cast<const floatx4*>(r);
+          const floatx4 r1 = *reinterpret_cast<const floatx4*>(r + 4);
+          v[0] += r0.x; v[1] += r0.y; v[2] += r0.z; v[3] += r0.w;
+          v[4] += r1.x; v[5] += r1.y; v[6] += r1.z; v[7] += r1.w;
         } else {
-          uintx2 rv = *reinterpret_cast<const uintx2*>(r);
-          const TOut* re = reinterpret_cast<const TOut*>(&rv);
+          Vec16<TOut> rv;
+          rv.load(r);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] += Store<TOut>::ld(re + e);
+          for (int e = 0; e < 8; ++e) v[e] += rv.get(e);
         }
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = apply_act(v[e], p.act, p.act_a, p.act_b);
+      for (int e = 0; e < 8; ++e) v[e] = epi_act(v[e], p.act, p.act_a, p.act_b);
       if constexpr (sizeof(TOut) == 4) {
-        floatx4 o = {v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<floatx4*>(y) = o;
+        *reinterpret_cast<floatx4*>(y) = (floatx4){v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<floatx4*>(y + 4) = (floatx4){v[4], v[5], v[6], v[7]};
       } else {
-        uintx2 o;
-        TOut* oe = reinterpret_cast<TOut*>(&o);
+        Vec16<TOut> o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) Store<TOut>::st(oe + e, v[e]);
-        *reinterpret_cast<uintx2*>(y) = o;
+        for (int e = 0; e < 8; ++e) o.set(e, v[e]);
+        o.store(y);
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (n + e < p.Kout) {
+      for (int e = 0; e < 8; ++e) {
+        if (e < nvalid) {
           float t = v[e];
-          if (rrow != nullptr) t += Store<TOut>::ld(r + e);
-          Store<TOut>::st(y + e, apply_act(t, p.act, p.act_a, p.act_b));
+          if (bias != nullptr) t += bias[e];
+          if (r != nullptr) t += Store<TOut>::ld(r + e);
+          Store<TOut>::st(y + e, epi_act(t, p.act, p.act_a, p.act_b));
         }
       }
     }
@@ -107,75 +126,121 @@ struct EpiFloat {
 
 // int8 operands, int32 accumulators.  MODE 0: requantised 8-bit output (stored
 // q-128), MODE 1: dequantised fp32 output, MODE 2: raw int32 accumulators.
+template <int MODE> struct QuantOut;
+template <> struct QuantOut<0> { using T = int8_t; };
+template <> struct QuantOut<1> { using T = float; };
+template <> struct QuantOut<2> { using T = int; };
+
 template <int MODE>
 struct EpiQuant {
   using AccE = int;
-  __device__ static __forceinline__ int requant(const IgemmParams& p, int acc, float mul) {
-    float r = (float)acc * mul;          // v_cvt_f32_i32 (RNE) then one v_mul_f32
-    int q = (int)rintf(r) + p.q_zp;      // v_rndne_f32
-    q = q < p.q_lo ? p.q_lo : q;
-    q = q > 255 ? 255 : q;
-    return q;
-  }
-  __device__ static __forceinline__ void run(const IgemmParams& p, const int* acc, int n,
-                                             const int* bias4, void* yrow, const void* rrow,
-                                             bool full) {
+  using TOut = typename QuantOut<MODE>::T;
+  __device__ static __forceinline__ void store8(const IgemmParams& p, const int* acc, int nvalid, bool vec,
+                                                const int* bias, TOut* y, const TOut* r, const float* qmul) {
+    if constexpr (MODE == 0) {
+      int8_t rs[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (r != nullptr) {
+        if (vec) {
+          const uintx2 rv = *reinterpret_cast<const uintx2*>(r);
+          __builtin_memcpy(rs, &rv, 8);
+        } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (!full && n + e >= p.Kout) continue;
-      const int a = acc[e] + bias4[e];
-      if constexpr (MODE == 2) {
-        reinterpret_cast<int*>(yrow)[n + e] = a;
-      } else if constexpr (MODE == 1) {
-        float f = (float)a * p.qmul[n + e];
-        if (rrow != nullptr) f += reinterpret_cast<const float*>(rrow)[n + e];
-        reinterpret_cast<float*>(yrow)[n + e] = apply_act(f, p.act, p.act_a, p.act_b);
-      } else {
-        int q = requant(p, a, p.qmul[n + e]);
-        if (rrow != nullptr) {
-          const int rq = q_from_stored(reinterpret_cast<const int8_t*>(rrow)[n + e]);
-          const float fa = (float)(q - p.q_zp) * p.q_scale;
-          const float fb = (float)(rq - p.r_zp) * p.r_scale;
-          const float f = fa + fb;
-          q = (int)rintf(f * p.s_inv) + p.s_zp;
-          q = q < p.s_lo ? p.s_lo : q;
-          q = q > 255 ? 255 : q;
+          for (int e = 0; e < 8; ++e)
+            if (e < nvalid) rs[e] = r[e];
         }
-        reinterpret_cast<int8_t*>(yrow)[n + e] = q_to_stored(q);
+      }
+      int8_t out[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        int q = 0;
+        if (e < nvalid) {
+          const int a = acc[e] + (bias ? bias[e] : 0);
+          const float f0 = (float)a * qmul[e];  // v_cvt_f32_i32 (RNE), then one v_mul_f32
+          q = (int)rintf(f0) + p.q_zp;           // v_rndne_f32
+          q = q < p.q_lo ? p.q_lo : q;
+          q = q > 255 ? 255 : q;
+          if (r != nullptr) {
+            const float fa = (float)(q - p.q_zp) * p.q_scale;
+            const float fb = (float)(q_from_stored(rs[e]) - p.r_zp) * p.r_scale;
+            const float f = fa + fb;
+            q = (int)rintf(f * p.s_inv) + p.s_zp;
+            q = q < p.s_lo ? p.s_lo : q;
+            q = q > 255 ? 255 : q;
+          }
+        }
+        out[e] = q_to_stored(q);
+      }
+      if (vec) {
+        uintx2 ov;
+        __builtin_memcpy(&ov, out, 8);
+        *reinterpret_cast<uintx2*>(y) = ov;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (e < nvalid) y[e] = out[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (e < nvalid) {
+          const int a = acc[e] + (bias ? bias[e] : 0);
+          if constexpr (MODE == 2) {
+            y[e] = a;
+          } else {
+            float f = (float)a * qmul[e];
+            if (r != nullptr) f += r[e];
+            y[e] = epi_act(f, p.act, p.act_a, p.act_b);
+          }
+        }
       }
     }
   }
 };
 
-template <typename Epi> struct EpiOutSize;
-template <typename T> struct EpiOutSize<EpiFloat<T>> { static constexpr int v = sizeof(T); };
-template <> struct EpiOutSize<EpiQuant<0>> { static constexpr int v = 1; };
-template <> struct EpiOutSize<EpiQuant<1>> { static constexpr int v = 4; };
-template <> struct EpiOutSize<EpiQuant<2>> { static constexpr int v = 4; };
+template <typename Epi> struct EpiTraits;
+template <typename T> struct EpiTraits<EpiFloat<T>> { using TOut = T; static constexpr bool quant = false; };
+template <int M> struct EpiTraits<EpiQuant<M>> { using TOut = typename QuantOut<M>::T; static constexpr bool quant = true; };
 
 // ---------------------------------------------------------------------------
+// Main kernel.
+//
+// K pipeline: per stage the workgroup holds 128 bytes of K per row for both
+// operands in one LDS buffer; the next stage's global loads are issued right
+// after the buffer is published and stay in flight, in registers, while the
+// MFMAs of the current stage run.  Other resident workgroups of the CU cover
+// the two barriers per stage.
+//
+// Epilogue: each wavefront parks one 32-pixel slice of its accumulators in LDS
+// (pixel-major, fp32 / int32), then every lane picks eight consecutive output
+// channels of one pixel, so that global stores and residual loads are 16-byte
+// vectors and consecutive lanes cover contiguous memory.
 template <typename TIn, typename Epi, int BM, int BN, int WM, int WN>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
 igemm_kernel(const IgemmParams p, const int epi_vec) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
   constexpr int ES = sizeof(TIn);
-  constexpr int VEC = 16 / ES;   // elements per 16-byte vector
-  constexpr int BKB = 64;        // bytes of K per row per stage
-  constexpr int BK = BKB / ES;   // elements of K per stage
-  constexpr int ROWB = BKB + 16; // LDS row pitch in bytes
-  constexpr int VPR = BKB / 16;  // vectors per row
-  constexpr int RPP = NT / VPR;  // rows loaded per pass
+  constexpr int VEC = 16 / ES;    // elements per 16-byte vector
+  constexpr int BKB = 128;        // bytes of K per row per stage
+  constexpr int BK = BKB / ES;    // elements of K per stage
+  constexpr int ROWB = BKB + 16;  // LDS row pitch in bytes: 16-byte reads of 16 lanes hit distinct banks
+  constexpr int VPR = BKB / 16;   // vectors per row
+  constexpr int RPP = NT / VPR;   // rows loaded per pass
   constexpr int A_IT = (BM + RPP - 1) / RPP, B_IT = (BN + RPP - 1) / RPP;
   static_assert(BM % RPP == 0 || BM < RPP, "pixel tile must be a multiple of the rows per pass");
   static_assert(BN % RPP == 0 || BN < RPP, "channel tile must be a multiple of the rows per pass");
   constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int EPI_PITCH = WN + 4;  // 4-byte words per staged pixel row
+  constexpr int MAIN_BYTES = (BM + BN) * ROWB;
+  constexpr int EPI_BYTES = NW * 32 * EPI_PITCH * 4;
+  constexpr int SMEM_BYTES = MAIN_BYTES > EPI_BYTES ? MAIN_BYTES : EPI_BYTES;
   using Acc = typename Mma<TIn>::Acc;
   using AccE = typename Epi::AccE;
+  using TOut = typename EpiTraits<Epi>::TOut;
 
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * (BM + BN) * ROWB];
+  __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
   unsigned char* As = smem;
-  unsigned char* Bs = smem + 2 * BM * ROWB;
+  unsigned char* Bs = smem + BM * ROWB;
 
   const int tid = threadIdx.x;
   const int M = p.N * p.Ho * p.Wo;
@@ -262,12 +327,12 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
       if (++ks == p.S) { ks = 0; ++kr; }
     }
   };
-  auto lds_store = [&](int buf) {
-    unsigned char* ab = As + buf * (BM * ROWB) + row0 * ROWB + kv * 16;
+  auto lds_store = [&]() {
+    unsigned char* ab = As + row0 * ROWB + kv * 16;
 #pragma unroll
     for (int i = 0; i < A_IT; ++i)
       if (BM % RPP == 0 || row0 + i * RPP < BM) *reinterpret_cast<uintx4*>(ab + i * RPP * ROWB) = ra[i];
-    unsigned char* bb = Bs + buf * (BN * ROWB) + row0 * ROWB + kv * 16;
+    unsigned char* bb = Bs + row0 * ROWB + kv * 16;
 #pragma unroll
     for (int i = 0; i < B_IT; ++i)
       if (BN % RPP == 0 || row0 + i * RPP < BN) *reinterpret_cast<uintx4*>(bb + i * RPP * ROWB) = rb[i];
@@ -287,15 +352,15 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
 
   const int ktot = p.R * p.S * p.C;
   const int nkt = (ktot + BK - 1) / BK;
+  const unsigned char* ab = As + (wm * WM + l32) * ROWB + lg * 16;
+  const unsigned char* bb = Bs + (wn * WN + l32) * ROWB + lg * 16;
 
   gload();
-  lds_store(0);
-  __syncthreads();
   for (int kt = 0; kt < nkt; ++kt) {
-    const int buf = kt & 1;
+    if (kt > 0) __syncthreads();  // everyone finished reading the previous stage
+    lds_store();
+    __syncthreads();
     if (kt + 1 < nkt) gload();
-    const unsigned char* ab = As + buf * (BM * ROWB) + (wm * WM + l32) * ROWB + lg * 16;
-    const unsigned char* bb = Bs + buf * (BN * ROWB) + (wn * WN + l32) * ROWB + lg * 16;
 #pragma unroll
     for (int kk = 0; kk < BKB / 32; ++kk) {
       uintx4 fa[TM], fb[TN];
@@ -308,42 +373,69 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = Mma<TIn>::run(fb[j], fa[i], acc[i][j]);
     }
-    if (kt + 1 < nkt) lds_store(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue ----
-  constexpr int OES = EpiOutSize<Epi>::v;
-  unsigned char* ybase = reinterpret_cast<unsigned char*>(p.y) + (int64_t)z * p.y_bs * OES;
-  const unsigned char* rbase =
-      p.residual ? reinterpret_cast<const unsigned char*>(p.residual) + (int64_t)z * p.r_bs * OES : nullptr;
+  TOut* ybase = reinterpret_cast<TOut*>(p.y) + (int64_t)z * p.y_bs;
+  const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
   const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
 
+  AccE* stage = reinterpret_cast<AccE*>(smem) + wave * (32 * EPI_PITCH);
+  constexpr int LPP = WN / 8;    // lanes per pixel row in the read-back
+  constexpr int PPP = 64 / LPP;  // pixels per read-back pass
+  const int rp = lane / LPP;     // pixel within a pass
+  const int c8 = (lane % LPP) * 8;
+  const int n = tile_n * BN + wn * WN + c8;
+  int nvalid = p.Kout - n;
+  nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
+  const bool vec = epi_vec && nvalid == 8;
+
+  __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
+  for (int i = 0; i < TM; ++i) {
+    // park: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = tile_n * BN + wn * WN + j * 32 + q * 8 + lg * 4;
-      if (n >= p.Kout) continue;
-      AccE b4[4] = {0, 0, 0, 0};
-      if (bias != nullptr) {
+    for (int j = 0; j < TN; ++j) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < p.Kout) b4[e] = bias[n + e];
-      }
-      const bool full = epi_vec && (n + 3 < p.Kout);
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int m = tile_m * BM + wm * WM + i * 32 + l32;
-        if (m >= M) continue;
-        AccE a4[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) a4[e] = acc[i][j][q * 4 + e];
-        void* yrow = ybase + (int64_t)m * p.ycs * OES;
-        const void* rrow = rbase ? rbase + (int64_t)m * p.rcs * OES : nullptr;
-        Epi::run(p, a4, n, b4, yrow, rrow, full);
+      for (int q = 0; q < 4; ++q) {
+        AccE* dst = stage + l32 * EPI_PITCH + j * 32 + q * 8 + lg * 4;
+        if constexpr (sizeof(AccE) == 4 && !EpiTraits<Epi>::quant) {
+          *reinterpret_cast<floatx4*>(dst) =
+              (floatx4){acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+        } else {
+          *reinterpret_cast<intx4*>(dst) =
+              (intx4){(int)acc[i][j][q * 4 + 0], (int)acc[i][j][q * 4 + 1], (int)acc[i][j][q * 4 + 2], (int)acc[i][j][q * 4 + 3]};
+        }
       }
     }
+    __syncthreads();
+#pragma unroll
+    for (int ps = 0; ps < 32 / PPP; ++ps) {
+      const int pix = ps * PPP + rp;
+      const int m = tile_m * BM + wm * WM + i * 32 + pix;
+      if (m < M && nvalid > 0) {
+        AccE a8[8];
+        const AccE* src = stage + pix * EPI_PITCH + c8;
+        if constexpr (!EpiTraits<Epi>::quant) {
+          const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
+          const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
+          a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
+          a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+        } else {
+          const intx4 v0 = *reinterpret_cast<const intx4*>(src);
+          const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
+          a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
+          a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+        }
+        TOut* yrow = ybase + (int64_t)m * p.ycs + n;
+        const TOut* rrow = rbase ? rbase + (int64_t)m * p.rcs + n : nullptr;
+        if constexpr (EpiTraits<Epi>::quant)
+          Epi::store8(p, a8, nvalid, vec, bias ? bias + n : nullptr, yrow, rrow, p.qmul ? p.qmul + n : nullptr);
+        else
+          Epi::store8(p, a8, nvalid, vec, bias ? bias + n : nullptr, yrow, rrow);
+      }
+    }
+    if (i + 1 < TM) __syncthreads();
   }
 }
 
@@ -401,6 +493,7 @@ hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream) {
   if (!aligned16(p.x) || !aligned16(p.w)) return hipErrorInvalidValue;
   if (p.N <= 0 || p.H <= 0 || p.W <= 0 || p.Ho <= 0 || p.Wo <= 0 || p.Kout <= 0 || p.batch <= 0)
     return hipErrorInvalidValue;
+  if (p.act != ACT_NONE && p.act != ACT_RELU && p.act != ACT_LEAKY && p.act != ACT_CLAMP) return hipErrorInvalidValue;
   if (p.R <= 0 || p.S <= 0 || p.sh <= 0 || p.sw <= 0 || p.dh <= 0 || p.dw <= 0) return hipErrorInvalidValue;
   if (p.xcs < p.C || p.ycs < p.Kout) return hipErrorInvalidValue;
   if ((int64_t)p.H * p.W * p.xcs >= (1ll << 31)) return hipErrorInvalidValue;
@@ -413,12 +506,17 @@ hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream) {
     return hipErrorInvalidValue;
 
   const int oes = dtype_size(p.out_dt);
-  // Four consecutive output elements are accessed as one vector when this holds.
-  int epi_vec = (p.ycs % 4 == 0) && (p.y_bs % 4 == 0) &&
-                ((reinterpret_cast<uintptr_t>(p.y) & (uintptr_t)(4 * oes - 1)) == 0);
-  if (p.residual != nullptr)
-    epi_vec = epi_vec && (p.rcs % 4 == 0) && (p.r_bs % 4 == 0) &&
-              ((reinterpret_cast<uintptr_t>(p.residual) & (uintptr_t)(4 * oes - 1)) == 0);
+  // Eight consecutive output elements are accessed as one vector (16 bytes, or
+  // 8 bytes for 8-bit output, two 16-byte vectors for 4-byte output) when rows
+  // and base pointers are aligned accordingly.
+  const int64_t vbytes = oes == 1 ? 8 : 16;
+  auto rows_ok = [&](const void* ptr, int64_t cs, int64_t bs) {
+    return ((cs * oes) % vbytes == 0) && ((bs * oes) % vbytes == 0) &&
+           ((reinterpret_cast<uintptr_t>(ptr) % (uintptr_t)vbytes) == 0);
+  };
+  int epi_vec = rows_ok(p.y, p.ycs, p.y_bs);
+  if (p.residual != nullptr) epi_vec = epi_vec && rows_ok(p.residual, p.rcs, p.r_bs);
+  if (p.bias != nullptr) epi_vec = epi_vec && ((reinterpret_cast<uintptr_t>(p.bias) % 16) == 0) && (p.bias_bs % 4 == 0);
 
   switch (p.in_dt) {
     case DT_F32:
@@ -435,7 +533,7 @@ hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream) {
     case DT_I8:
       if (p.out_dt == DT_I8) {
         if (p.qmul == nullptr) return hipErrorInvalidValue;
-        return dispatch_tiles<int8_t, EpiQuant<0>>(p, 0, stream);
+        return dispatch_tiles<int8_t, EpiQuant<0>>(p, epi_vec, stream);
       }
       if (p.out_dt == DT_F32) {
         if (p.qmul == nullptr) return hipErrorInvalidValue;
