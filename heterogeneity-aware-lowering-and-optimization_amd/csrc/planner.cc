@@ -420,6 +420,13 @@ class Planner {
     return new_tensor(dt, layout, v->shape, cs, SP_ARENA);
   }
 
+  // Is `v` available as 8-bit levels (already stored so, or quantisable from the table)?
+  bool q8_value(const _odla_value* v) {
+    if (!comp_->opts.int8 || v == nullptr) return false;
+    if (qentry(v) != nullptr) return true;
+    const VState& s = vs_[v->index];
+    return s.main >= 0 && T(s.main).quant;
+  }
   int use_count(const _odla_value* v) const { return (int)consumers_[v->index].size() + (v->is_output ? 1 : 0); }
   bool available(const _odla_value* v) const {
     return v->kind != _odla_value::TEMP || vs_[v->index].main >= 0;
@@ -709,7 +716,9 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
                    other->kind != _odla_value::CONSTANT && other->shape == cur->shape && available(other) &&
                    storage_dtype(other) == storage_dtype(cur)) {
           bool ok = true;
-          if (q8) ok = qentry(cur) != nullptr && qentry(other) != nullptr;  // both sides must be 8-bit
+          if (q8) {  // both sides must be 8-bit
+            ok = qentry(cur) != nullptr && q8_value(other);
+          }
           if (ok) {
             ep->residual = other;
             ep->pre_residual_value = cur;
@@ -903,9 +912,12 @@ void Planner::lower_conv(int ni) {
   _odla_value* outv = ep.final_value;
 
   // int8 plan?
-  const QuantEntry* qx = qentry(x);
   const QuantEntry* qk = qentry(k);
-  const bool q8 = comp_->opts.int8 && qx != nullptr && qk != nullptr && const_kernel && !cl && G == 1 &&
+  // the input is 8-bit if it already lives as levels (e.g. the result of a
+  // quantised producer or of a max-pool that kept its input's scale) or has a
+  // table entry to quantise it with
+  const bool x_q8 = q8_value(x);
+  const bool q8 = comp_->opts.int8 && x_q8 && qk != nullptr && const_kernel && !cl && G == 1 &&
                   !runtime_bias;
   if (q8) {
     // ---- int8 x int8 -> int32 with fused requantisation ----
@@ -924,8 +936,8 @@ void Planner::lower_conv(int ni) {
     // (zp_x - 128) * sum_k w_q[o][k]; activations are stored as q - 128.
     std::vector<float> wf = const_as_float(k);
     std::vector<int32_t> bi((size_t)O, 0);
-    const float sx = qx->scale;
-    const int zx = qx->zp;
+    const float sx = T(tx).qscale;  // parameters of the tensor actually consumed
+    const int zx = T(tx).qzp;
     for (int64_t o = 0; o < O; ++o) {
       int64_t wsum = 0;
       for (int64_t i = 0; i < Cg; ++i)
@@ -968,9 +980,7 @@ void Planner::lower_conv(int ni) {
       ip.q_scale = qo->scale;
       const bool relu = ep.act == ACT_RELU;
       if (ep.residual) {
-        const QuantEntry* qr = qentry(ep.residual);
         ip.q_lo = 0;
-        ip.r_zp = qr->zp; ip.r_scale = qr->scale;
         ip.s_inv = 1.0f / qf->scale; ip.s_zp = qf->zp; ip.s_lo = relu ? qf->zp : 0;
       } else {
         ip.q_lo = relu ? qo->zp : 0;
@@ -993,6 +1003,8 @@ void Planner::lower_conv(int ni) {
     if (ep.residual) {
       tr = get(ep.residual, L_NHWC, FORM_QUANT);
       ip.rcs = T(tr).cs;
+      ip.r_zp = T(tr).qzp;
+      ip.r_scale = T(tr).qscale;
     }
     const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb), rm = ref(tm), rr = ref(tr >= 0 ? tr : tx);
     const bool hr = tr >= 0;
@@ -1229,9 +1241,7 @@ void Planner::lower_binary(int ni) {
   // optional trailing activation
   ActKind act = ACT_NONE;
   float act_a = 0.f, act_b = 0.f;
-  const QuantEntry* qa = qentry(a);
-  const QuantEntry* qb = qentry(b);
-  const bool q8 = comp_->opts.int8 && qa && qb && a->shape == os && b->shape == os &&
+  const bool q8 = comp_->opts.int8 && q8_value(a) && q8_value(b) && a->shape == os && b->shape == os &&
                   (n.i[0] == BIN_ADD) && a->kind != _odla_value::CONSTANT && b->kind != _odla_value::CONSTANT;
   if (!outv->is_output && consumers_[outv->index].size() == 1) {
     Node& nx = comp_->nodes[consumers_[outv->index][0]];
@@ -1497,7 +1507,7 @@ void Planner::lower_pool(int ni) {
   const bool is_max = n.i[1] != 0;
   // 8-bit max pooling keeps levels (the result inherits the input's scale)
   const VState& s = vs_[x->index];
-  const bool q8 = is_max && !cl && s.main >= 0 && T(s.main).quant && qentry(n.out) != nullptr && (xs.d[1] % 16 == 0);
+  const bool q8 = is_max && !cl && s.main >= 0 && T(s.main).quant && (xs.d[1] % 16 == 0);
   int tx;
   if (cl) tx = get(x, L_ROWMAJOR, FORM_FLOAT);
   else tx = get(x, L_NHWC, q8 ? FORM_QUANT : FORM_FLOAT);

@@ -123,3 +123,67 @@ def build_resnet50(b, w, batch, hw=224, stages=RESNET50_STAGES, stem=64, num_cla
 
 
 RESNET50_GFLOP_PER_IMAGE = 2 * (4087136256 + 2048000) / 1e9   # conv + FC multiply-adds, x2
+
+
+# ---------------------------------------------------------------------------
+# C2: post-training quantisation of the same network.
+#
+# The graph stays FLOAT32-typed; an odla_value_quant_info table keyed by value
+# id carries the ranges (this is the channel the reference defines for it:
+# ODLA_QUANT_TABLE / ODLA_QUANT_TABLE_SIZE / ODLA_USE_DATA_TYPE, written by
+# utils/halo_pgq.py:283-332 of the reference tree).
+#   activations  asymmetric u8 per tensor: scale = (max-min)/255,
+#                zp = clip(rne(-min/scale), 0, 255), range widened to contain 0
+#   weights      symmetric s8 per output channel: scale = max|w_c| / 127,
+#                expressed through the per-channel min/max records
+# Values without a table entry stay floating point, which is how the fp32
+# classifier head is expressed.
+# ---------------------------------------------------------------------------
+def act_qparams(mn, mx):
+    mn = np.float32(min(float(mn), 0.0))
+    mx = np.float32(max(float(mx), 0.0))
+    scale = np.float32((mx - mn) / np.float32(255.0))
+    if not scale > 0:
+        scale = np.float32(1.0)
+    zp = int(np.clip(np.rint(np.float32(-mn) / scale), 0, 255))
+    return scale, zp
+
+
+def resnet50_quantized_values(stages=RESNET50_STAGES):
+    """Names of the activations that live as 8-bit levels in the int8 plan."""
+    names = ["input", "stem.relu"]
+    for si, (mid, blocks, stride) in enumerate(stages):
+        for bi in range(blocks):
+            p = "l%db%d" % (si + 1, bi)
+            if bi == 0:
+                names.append(p + "ds")
+            names += [p + "c1.relu", p + "c2.relu", p + "c3", p + "out"]
+    return names
+
+
+def resnet50_quant_entries(w, ranges, stages=RESNET50_STAGES, stem=64):
+    """ranges: name -> (min, max) of the calibrated activations.  Returns the
+    entry list `odla.quant_table` turns into odla_value_quant_info records."""
+    entries = []
+    for name in resnet50_quantized_values(stages):
+        mn, mx = ranges[name]
+        scale, zp = act_qparams(mn, mx)
+        entries.append((name, scale, zp, mn, mx, None))
+    for name, cout, cin, k, _, _ in resnet50_conv_specs(stages, stem):
+        wt = w[name + ".w"].reshape(cout, -1)
+        ch = list(zip(wt.min(axis=1).tolist(), wt.max(axis=1).tolist()))
+        entries.append((name + ".w", 1.0, 0, float(wt.min()), float(wt.max()), ch))
+    return entries
+
+
+def calibrate_ranges(run_taps, batches):
+    """run_taps(feeds) -> {name: array}; min/max over all calibration batches."""
+    ranges = {}
+    for feeds in batches:
+        for name, v in run_taps(feeds).items():
+            mn, mx = float(np.min(v)), float(np.max(v))
+            if name in ranges:
+                ranges[name] = (min(ranges[name][0], mn), max(ranges[name][1], mx))
+            else:
+                ranges[name] = (mn, mx)
+    return ranges

@@ -1,0 +1,177 @@
+"""int8 plan: bit-exact parity with the CPU oracle.
+
+The graph handed to the library is FLOAT32-typed; a quant table
+(ODLA_QUANT_TABLE / ODLA_QUANT_TABLE_SIZE / ODLA_USE_DATA_TYPE) selects the
+int8 kernels.  Checked here:
+  * raw int32 accumulators (+ int32 bias) of single convolutions,
+  * requantised 8-bit outputs of Conv(+ReLU), of the fused Conv+Add+ReLU and of
+    the unfused quantised Add,
+  * every quantised activation and the fp32 logits of a small ResNet.
+All integer comparisons are exact (np.array_equal).
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as entry
+from util import announce, run_hip
+
+pytestmark = pytest.mark.gpu
+
+sys.path.insert(0, os.path.join(entry.ROOT, "oracle"))
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def table_for(odla, acts, weights):
+    """acts: name -> (min, max); weights: name -> array [O, ...]."""
+    models = entry.load().models
+    entries = []
+    for name, (mn, mx) in acts.items():
+        s, z = models.act_qparams(mn, mx)
+        entries.append((name, s, z, mn, mx, None))
+    for name, w in weights.items():
+        wt = w.reshape(w.shape[0], -1)
+        entries.append((name, 1.0, 0, float(wt.min()), float(wt.max()),
+                        list(zip(wt.min(axis=1).tolist(), wt.max(axis=1).tolist()))))
+    return odla.quant_table(entries)
+
+
+Q8_CONV_CASES = [
+    # N, C, H, W, O, k, stride, pad
+    (2, 16, 10, 10, 32, 3, 1, 1),
+    (2, 32, 9, 11, 48, 3, 2, 1),
+    (3, 64, 7, 7, 64, 1, 1, 0),
+    (2, 3, 20, 20, 16, 7, 2, 3),
+    (1, 48, 6, 6, 200, 1, 2, 0),
+    (1, 512, 7, 7, 64, 3, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", Q8_CONV_CASES)
+def test_q8_conv_accumulators_and_requant(case, odla, ref):
+    N, C, H, W, O, k, s, p = case
+    announce("q8 conv %s" % (case,))
+    r = rng(100 + O)
+    x = (r.standard_normal((N, C, H, W)) * 1.5 + 0.3).astype(np.float32)
+    w = (r.standard_normal((O, C, k, k)) * np.sqrt(2.0 / (C * k * k))).astype(np.float32)
+    bias = (r.standard_normal(O) * 0.2).astype(np.float32)
+    x_rng = (float(x.min()), float(x.max()))
+    x_qp = ref.act_qparams(*x_rng)
+    y_rng = (-2.5, 4.0)
+    y_qp = ref.act_qparams(*y_rng)
+
+    def build_acc(b):
+        v = b.arg("x", x.shape)
+        b.output(b.conv(v, b.const("w", w), b.const("b", bias), (s, s), (p, p, p, p), name="y"), "y")
+
+    def build_q(b):
+        v = b.arg("x", x.shape)
+        y = b.conv(v, b.const("w", w), b.const("b", bias), (s, s), (p, p, p, p), name="y")
+        b.output(b.relu(y, name="yr"), "yr")
+
+    # oracle
+    xq = ref.quantize_act(x, *x_qp)
+    q_want, acc_want = ref.qconv(xq, x_qp, w, bias, y_qp, (s, s), (p, p, p, p), relu=True)
+
+    # 1. raw accumulators: the result value has no table entry
+    t = table_for(odla, {"x": x_rng}, {"w": w})
+    got = run_hip(build_acc, {"x": x}, quant_table=t, raw_acc=True)["y"]
+    acc_got = got.view(np.int32)
+    assert acc_got.shape == acc_want.shape
+    assert np.array_equal(acc_got, acc_want)
+
+    # 2. requantised output (ReLU fused as a clamp at the zero point), read back dequantised
+    t = table_for(odla, {"x": x_rng, "yr": y_rng}, {"w": w})
+    got = run_hip(build_q, {"x": x}, quant_table=t)["yr"]
+    want = ref.dequantize_act(q_want, *y_qp)
+    assert np.array_equal(got, want)
+    q_got = np.rint(got / y_qp[0]).astype(np.int64) + y_qp[1]
+    assert np.array_equal(q_got, q_want.astype(np.int64))
+
+
+def test_q8_residual_fused_equals_unfused_equals_oracle(odla, ref):
+    """Conv -> Add(residual) -> ReLU: fused into the conv epilogue, and as separate
+    quantised kernels (the conv result is also a graph output, which blocks fusion)."""
+    announce("q8 residual")
+    r = rng(7)
+    N, C, H, W, O = 2, 32, 8, 8, 64
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    res = (r.standard_normal((N, O, H, W)) * 2).astype(np.float32)
+    w = (r.standard_normal((O, C, 1, 1)) * 0.3).astype(np.float32)
+    bias = r.standard_normal(O).astype(np.float32)
+    ranges = {"x": (float(x.min()), float(x.max())), "res": (float(res.min()), float(res.max())),
+              "c": (-6.0, 6.0), "out": (0.0, 9.0)}
+    qp = {k: ref.act_qparams(*v) for k, v in ranges.items()}
+
+    def build(b, tap_conv):
+        v = b.arg("x", x.shape)
+        rr = b.arg("res", res.shape)
+        c = b.conv(v, b.const("w", w), b.const("b", bias), name="c")
+        if tap_conv:
+            b.output(c, "c")
+        b.output(b.relu(b.add(c, rr, name="add"), name="out"), "out")
+
+    t = table_for(odla, ranges, {"w": w})
+    fused = run_hip(lambda b: build(b, False), {"x": x, "res": res}, quant_table=t)
+    t = table_for(odla, ranges, {"w": w})
+    unfused = run_hip(lambda b: build(b, True), {"x": x, "res": res}, quant_table=t)
+
+    xq = ref.quantize_act(x, *qp["x"])
+    rq = ref.quantize_act(res, *qp["res"])
+    cq, _ = ref.qconv(xq, qp["x"], w, bias, qp["c"], (1, 1), (0, 0, 0, 0), relu=False)
+    oq = ref.qadd(cq, qp["c"], rq, qp["res"], qp["out"], relu=True)
+    want = ref.dequantize_act(oq, *qp["out"])
+    assert np.array_equal(unfused["c"], ref.dequantize_act(cq, *qp["c"]))
+    assert np.array_equal(unfused["out"], want)
+    assert np.array_equal(fused["out"], want)
+
+
+SMALL_STAGES = [(16, 2, 1), (32, 2, 2)]
+
+
+def test_small_resnet_int8_bit_exact(odla, models, ref):
+    """Whole int8 network: every 8-bit activation that ends a fused chain and the fp32 head."""
+    announce("small resnet int8")
+    import resnet_q8_ref
+    batch, hw, stem, classes = 4, 64, 16, 50
+    w = models.resnet50_weights(seed=11, num_classes=classes, stages=SMALL_STAGES, stem=stem)
+    for k in w:  # non-zero biases exercise the int32 bias path
+        if k.endswith(".b") and k != "fc.b":
+            w[k] = (rng(len(k)).standard_normal(w[k].shape) * 0.1).astype(np.float32)
+
+    # calibration: min/max of the fp32 oracle over 4 seeded batches
+    def taps_of(feeds):
+        rb = ref.RefBuilder(feeds)
+        taps = []
+        models.build_resnet50(rb, w, batch, hw, SMALL_STAGES, stem, classes, taps=taps)
+        return dict(taps)
+
+    ranges = models.calibrate_ranges(taps_of, [models.resnet50_input(batch, hw, seed=1000 + i) for i in range(4)])
+    entries = models.resnet50_quant_entries(w, ranges, SMALL_STAGES, stem)
+    qp = {e[0]: (e[1], e[2]) for e in entries if e[5] is None}
+    feeds = models.resnet50_input(batch, hw, seed=1234)
+
+    record = {}
+    want = resnet_q8_ref.run(w, feeds, qp, SMALL_STAGES, stem, batch, hw, record)
+
+    # chain-end activations can be tapped without changing the plan
+    tap_names = [n for n in models.resnet50_quantized_values(SMALL_STAGES) if not n.endswith("c3") and n != "input"]
+
+    def build(b):
+        taps = []
+        models.build_resnet50(b, w, batch, hw, SMALL_STAGES, stem, classes, taps=taps)
+        d = dict(taps)
+        for n in tap_names:
+            b.output(d[n], n)
+
+    got = run_hip(build, feeds, quant_table=odla.quant_table(entries))
+    for n in tap_names:
+        assert np.array_equal(got[n], ref.dequantize_act(record[n], *qp[n])), n
+    # fp32 head behind the 8-bit trunk: same integer input, fp32 Gemm
+    assert np.max(np.abs(got["logits"] - want["logits"])) <= 1e-4 * max(1.0, float(np.max(np.abs(want["logits"]))))
+    assert np.array_equal(np.argmax(got["logits"], 1), np.argmax(want["logits"], 1))
