@@ -46,14 +46,17 @@ def main():
     odla, models = pkg.odla, pkg.models
     L = odla.load_library()
     mode = args.workload.split("_")[1]
-    if mode not in ("fp16", "fp32", "bf16"):
+    if mode not in ("fp16", "fp32", "bf16", "int8"):
         print("unknown workload %s" % args.workload, file=sys.stderr)
         sys.exit(2)
 
     batch = args.batch
     w = models.resnet50_weights()
     feeds = models.resnet50_input(batch)
-    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16=(mode == "bf16"))
+    table = None
+    if mode == "int8":
+        table = odla.quant_table(models.resnet50_quant_entries(w, calibrate_on_gpu(odla, models, w)))
+    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16=(mode == "bf16"), quant_table=table)
     models.build_resnet50(hb, w, batch)
     sess = hb.session(use_graph=True)
     sess.bind_device_io(feeds)
@@ -84,7 +87,7 @@ def main():
         "metric": "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW",
         "value": round(images_per_s, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": {"fp16": "f16", "bf16": "bf16", "fp32": "f32"}[mode],
+        "scaling": "weak", "vs_baseline": None, "dtype": {"fp16": "f16", "bf16": "bf16", "fp32": "f32", "int8": "i8"}[mode],
         "data": "synthetic",
         "config": {"workload": "ResNet-50 v1.5 %s NCHW [%d,3,224,224], folded BN, random He-normal weights, "
                                "softmax head; inputs/outputs resident in HBM" % (mode, batch),
@@ -94,6 +97,30 @@ def main():
     print(json.dumps(line))
     sess.close()
     hb.destroy()
+
+
+def calibrate_on_gpu(odla, models, w, batch=4, n_batches=8):
+    """Activation ranges for the int8 plan: min/max of every named activation of
+    the fp32 graph over 32 seeded N(0,1) images (8 batches of 4), computed by the
+    fp32 plan of the library itself."""
+    hb = odla.HipBuilder()
+    taps = []
+    models.build_resnet50(hb, w, batch, taps=taps, with_softmax=False)
+    wanted = set(models.resnet50_quantized_values())
+    for name, v in taps:
+        if name in wanted and name != "input":
+            hb.output(v, name)
+    sess = hb.session()
+
+    def run_taps(feeds):
+        out = sess.run(feeds)
+        out["input"] = feeds["input"]
+        return out
+
+    ranges = models.calibrate_ranges(run_taps, [models.resnet50_input(batch, seed=1000 + i) for i in range(n_batches)])
+    sess.close()
+    hb.destroy()
+    return ranges
 
 
 def profile_roofline(L, sess, hb, mode, batch, models, dump_path=None):

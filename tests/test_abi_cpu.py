@@ -1,0 +1,190 @@
+"""Host-side checks of the C-ABI boundary that need no GPU: the library loads,
+exports every symbol include/odla_hip.h declares, the by-value structs have the
+reference's sizes, graph builders infer shapes and reject malformed requests,
+and the product path fails loudly (no CPU fallback) when no GPU is present.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as entry
+
+
+def test_library_loads_and_exports_declared_symbols(odla):
+    L = odla.load_library()
+    names = odla.exported_symbols_declared_in_header()
+    assert len(names) >= 80
+    missing = [n for n in names if not hasattr(L, n)]
+    assert missing == []
+    assert L.odla_GetVersionString().startswith(b"odla_hip")
+
+
+def test_struct_layout_matches_reference_abi(odla):
+    assert ctypes.sizeof(odla.ValueShape) == 88
+    assert ctypes.sizeof(odla.ValueType) == 96
+    assert ctypes.sizeof(odla.Values) == 520
+    assert ctypes.sizeof(odla.QuantInfo) == 32
+
+
+REF_INC = "/root/reference/ODLA/include/ODLA"
+
+
+def _enum_names(text, typedef_name):
+    m = re.search(r"typedef\s+enum\s*\{([^{}]*)\}\s*%s\s*;" % typedef_name, text, flags=re.S)
+    assert m, typedef_name
+    body = re.sub(r"/\*.*?\*/", "", m.group(1), flags=re.S)
+    body = re.sub(r"///<.*", "", body)
+    body = re.sub(r"//.*", "", body)
+    return [t.strip().split("=")[0].strip() for t in body.split(",") if t.strip()]
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_INC), reason="reference tree not present on this machine")
+@pytest.mark.parametrize("hdr,enum", [
+    ("odla_common.h", "odla_element_type"), ("odla_common.h", "odla_status"),
+    ("odla_compute.h", "odla_item_type"), ("odla_compute.h", "odla_compute_mode"),
+    ("odla_compute.h", "odla_bf16_mode"), ("odla_device.h", "odla_device_info"),
+    ("odla_device.h", "odla_device_name"), ("odla_memory.h", "odla_memcpy_type"),
+    ("odla_log.h", "odla_log_level"), ("ops/odla_ops_nn.h", "odla_memory_layout"),
+    ("ops/odla_ops_process.h", "odla_interpolation_mode"), ("ops/odla_ops_process.h", "odla_resize_coordinate_mode"),
+])
+def test_enumerators_match_reference_headers(hdr, enum):
+    """Enumerator names and order (= values) are the ABI; compare with the reference headers."""
+    ours = open(os.path.join(entry.ROOT, "include", "odla_hip.h")).read()
+    theirs = open(os.path.join(REF_INC, hdr)).read()
+    assert _enum_names(ours, enum) == _enum_names(theirs, enum)
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_INC), reason="reference tree not present on this machine")
+def test_prototypes_match_reference_headers(odla):
+    """Every function we declare that the reference also declares has the same parameter count."""
+    ours = re.sub(r"/\*.*?\*/", "", open(os.path.join(entry.ROOT, "include", "odla_hip.h")).read(), flags=re.S)
+    theirs = ""
+    for root, _, files in os.walk(REF_INC):
+        for f in files:
+            theirs += open(os.path.join(root, f)).read()
+    theirs = re.sub(r"/\*.*?\*/", "", theirs, flags=re.S)
+    theirs = re.sub(r"//.*", "", theirs)
+
+    def params(text, name):
+        m = re.search(r"\b%s\s*\((.*?)\)\s*;" % name, text, flags=re.S)
+        if not m:
+            return None
+        p = m.group(1).strip()
+        return 0 if p in ("", "void") else p.count(",") + 1
+
+    checked = 0
+    for name in odla.exported_symbols_declared_in_header():
+        n_ref = params(theirs, name)
+        if n_ref is None:
+            continue  # library extensions (odla_LayerNorm, odla_hip_*)
+        assert params(ours, name) == n_ref, name
+        checked += 1
+    assert checked >= 70
+
+
+def test_shape_inference_and_validation(odla):
+    b = odla.HipBuilder()
+    x = b.arg("x", (2, 3, 224, 224))
+    w = b.const("w", np.zeros((64, 3, 7, 7), np.float32))
+    y = b.conv(x, w, None, (2, 2), (3, 3, 3, 3), name="y")
+    assert b.shape_of(y)[0] == (2, 64, 112, 112)
+    p = b.maxpool(y, (3, 3), (2, 2), (1, 1, 1, 1))
+    assert b.shape_of(p)[0] == (2, 64, 56, 56)
+    pc = b.maxpool(y, (3, 3), (2, 2), (0, 0, 0, 0), out_hw=(56, 56))   # ceil mode through output_dims
+    assert b.shape_of(pc)[0] == (2, 64, 56, 56)
+    g = b.reduce_mean(p, (2, 3), True)
+    assert b.shape_of(g)[0] == (2, 64, 1, 1)
+    f = b.reshape(g, (2, 64))
+    fc = b.gemm(f, b.const("fc", np.zeros((64, 10), np.float32)), None)
+    assert b.shape_of(fc)[0] == (2, 10)
+    t = b.transpose(y, (0, 2, 3, 1))
+    assert b.shape_of(t)[0] == (2, 112, 112, 64)
+    c = b.concat([p, p], 1)
+    assert b.shape_of(c)[0] == (2, 128, 56, 56)
+    s = b.slice(p, (0, 0, 0, 0), (2, 32, 56, 28))
+    assert b.shape_of(s)[0] == (2, 32, 56, 28)
+    e = b.gather(b.const("tab", np.zeros((100, 16), np.float32)), b.arg("ids", (4, 5), np.int32), 0)
+    assert b.shape_of(e)[0] == (4, 5, 16)
+    q = b.arg("q", (2, 4, 16, 8))
+    s2 = b.gemm(q, q, None, False, True)
+    assert b.shape_of(s2)[0] == (2, 4, 16, 16)
+    n = b.nms(b.arg("boxes", (2, 50, 4)), b.arg("scores", (2, 3, 50)), 7, 0.5, 0.1)
+    assert b.shape_of(n) == ((14, 3), np.dtype(np.int32))
+    # scalars become shape {1}
+    sc = b.const("s", np.float32(2.0))
+    assert b.shape_of(sc)[0] == (1,)
+    # malformed requests return NULL (raised by the wrapper), they do not crash
+    L = b.L
+    L.odla_SetLogLevel(0)
+    with pytest.raises(odla.OdlaError):
+        b.conv(x, b.const("bad", np.zeros((64, 4, 7, 7), np.float32)))
+    with pytest.raises(odla.OdlaError):
+        b.add(x, b.const("c", np.zeros((5,), np.float32)))
+    with pytest.raises(odla.OdlaError):
+        b.reshape(x, (7, 7))
+    with pytest.raises(odla.OdlaError):
+        b.gemm(f, b.const("fc2", np.zeros((63, 10), np.float32)), None)
+    L.odla_SetLogLevel(2)
+    b.destroy()
+
+
+def test_introspection_and_status_codes(odla):
+    b = odla.HipBuilder()
+    L = b.L
+    x = b.arg("x", (4, 8))
+    y = b.relu(x, name="y")
+    b.output(y, "y")
+    n = ctypes.c_uint32()
+    assert L.odla_GetNumOfArgsFromComputation(b.comp, ctypes.byref(n)) == 0 and n.value == 1
+    assert L.odla_GetNumOfOutputsFromComputation(b.comp, ctypes.byref(n)) == 0 and n.value == 1
+    v = ctypes.c_void_p()
+    assert L.odla_GetArgFromComputationByIdx(b.comp, 0, ctypes.byref(v)) == 0 and v.value == x
+    assert L.odla_GetArgFromComputationByIdx(b.comp, 5, ctypes.byref(v)) == odla.ODLA_INVALID_PARAM
+    vid = ctypes.c_char_p()
+    assert L.odla_GetValueId(y, ctypes.byref(vid)) == 0 and vid.value == b"y"
+    shp = odla.ValueShape()
+    assert L.odla_GetRuntimeShape(None, y, ctypes.byref(shp)) == 0 and shp.size == 2 and shp.dims[1] == 8
+    found = ctypes.c_void_p()
+    assert L.odla_FindValueById(b"y", ctypes.byref(found)) == 0 and found.value == y
+    # unknown property-bag items are accepted (generic harnesses set ODLA_USE_SIM_MODE)
+    t = ctypes.c_bool(True)
+    assert L.odla_SetComputationItem(b.comp, odla.ODLA_USE_SIM_MODE, ctypes.byref(t)) == 0
+    assert L.odla_CreateComputation(None) == odla.ODLA_INVALID_PARAM
+    assert L.odla_BindToArgument(None, None, None) == odla.ODLA_INVALID_PARAM
+    b.destroy()
+
+
+def test_logger_hook(odla):
+    L = odla.load_library()
+    seen = []
+    CB = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p)
+    cb = CB(lambda f, line, fn, lvl, msg: seen.append((lvl, msg)))
+    L.odla_SetLogger(ctypes.cast(cb, ctypes.c_void_p))
+    b = odla.HipBuilder()
+    with pytest.raises(odla.OdlaError):
+        b.reshape(b.arg("x", (3, 3)), (2, 2))
+    L.odla_SetLogger(None)
+    b.destroy()
+    assert seen and seen[0][0] == 2 and b"odla_Reshape" in seen[0][1]
+
+
+def test_no_cpu_fallback_without_gpu(odla, models):
+    """On a machine without a GPU the product path must fail with a status code, not compute on the CPU."""
+    try:
+        import torch
+        has_gpu = torch.cuda.is_available()
+    except Exception:
+        has_gpu = os.path.exists("/dev/kfd")
+    if has_gpu:
+        pytest.skip("a GPU is present")
+    L = odla.load_library()
+    L.odla_SetLogLevel(0)
+    b = odla.HipBuilder()
+    models.build_mnist(b, models.mnist_weights(), 64)
+    with pytest.raises(odla.OdlaError):
+        b.session()
+    L.odla_SetLogLevel(2)
+    b.destroy()

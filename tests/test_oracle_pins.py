@@ -1,0 +1,367 @@
+"""Pins of the CPU oracle (no GPU needed).
+
+Before the oracle is trusted as the checker of the GPU library, each of its
+functions is checked against something that does not come from this
+repository's own formulas: known-answer vectors the reference's tests hold,
+vectors produced by the reference's own fp32 kernels (tests/golden/
+sn_rt_vectors.npz, and live against oracle/_ref/libsn_rt.so when it is built),
+published ONNX operator examples, float64 / int64 brute force, and closed forms
+from the standard library.
+"""
+import math
+import os
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as entry
+
+GOLD = np.load(os.path.join(entry.ROOT, "tests", "golden", "sn_rt_vectors.npz"))
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ------------------------------------------------------------------ conv ----
+def test_conv_kat_from_reference_doctest(ref):
+    """odla_popart/test/odla_ops_nn_test.cc:147-200 of the reference tree."""
+    x = np.arange(25, dtype=np.float32).reshape(1, 1, 5, 5)
+    w = np.ones((1, 1, 3, 3), np.float32)
+    y = ref.conv2d(x, w, None, (1, 1), (1, 1, 1, 1))
+    assert y.reshape(-1).tolist() == [12, 21, 27, 33, 24, 33, 54, 63, 72, 51, 63, 99, 108, 117, 81, 93, 144, 153,
+                                      162, 111, 72, 111, 117, 123, 84]
+
+
+@pytest.mark.parametrize("i", range(5))
+def test_conv_against_reference_kernel_vectors(ref, i):
+    x, w = GOLD["conv%d_x" % i], GOLD["conv%d_w" % i]
+    s, p = (int(v) for v in GOLD["conv%d_attr" % i])
+    y = ref.conv2d(x, w, None, (s, s), (p, p, p, p))
+    want = GOLD["conv%d_y" % i]
+    assert y.shape == want.shape
+    assert np.max(np.abs(y - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+def brute_conv(x, w, b, stride, pad, dil, group):
+    N, C, H, W = x.shape
+    O, I, R, S = w.shape
+    Ho = (H + pad[0] + pad[2] - ((R - 1) * dil[0] + 1)) // stride[0] + 1
+    Wo = (W + pad[1] + pad[3] - ((S - 1) * dil[1] + 1)) // stride[1] + 1
+    y = np.zeros((N, O, Ho, Wo), np.float64)
+    og = O // group
+    for n in range(N):
+        for o in range(O):
+            g = o // og
+            for ho in range(Ho):
+                for wo in range(Wo):
+                    acc = 0.0 if b is None else float(b[o])
+                    for c in range(I):
+                        for r in range(R):
+                            for s in range(S):
+                                hi = ho * stride[0] - pad[0] + r * dil[0]
+                                wi = wo * stride[1] - pad[1] + s * dil[1]
+                                if 0 <= hi < H and 0 <= wi < W:
+                                    acc += float(x[n, g * I + c, hi, wi]) * float(w[o, c, r, s])
+                    y[n, o, ho, wo] = acc
+    return y
+
+
+@pytest.mark.parametrize("case", [
+    (1, 4, 6, 7, 6, 3, (1, 1), (1, 1, 1, 1), (1, 1), 1),
+    (2, 4, 7, 6, 4, 3, (2, 1), (0, 1, 2, 0), (1, 1), 2),   # asymmetric pad, groups, mixed stride
+    (1, 2, 9, 9, 3, 3, (1, 1), (2, 2, 2, 2), (2, 2), 1),   # dilation
+    (1, 3, 8, 8, 2, 5, (2, 2), (2, 2, 2, 2), (1, 1), 1),
+])
+def test_conv_against_float64_brute_force(ref, case):
+    N, C, H, W, O, k, st, pad, dil, g = case
+    r = rng(3)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = r.standard_normal((O, C // g, k, k)).astype(np.float32)
+    b = r.standard_normal(O).astype(np.float32)
+    y = ref.conv2d(x, w, b, st, pad, dil, g)
+    want = brute_conv(x, w, b, st, pad, dil, g)
+    assert y.shape == want.shape
+    assert np.max(np.abs(y - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+def test_conv_identities(ref):
+    """1x1 convolution is a matrix product; a delta kernel is a shifted copy."""
+    r = rng(4)
+    x = r.standard_normal((2, 5, 4, 4)).astype(np.float32)
+    w = r.standard_normal((3, 5, 1, 1)).astype(np.float32)
+    y = ref.conv2d(x, w)
+    want = np.einsum("nchw,oc->nohw", x.astype(np.float64), w[:, :, 0, 0].astype(np.float64))
+    assert np.max(np.abs(y - want)) <= 1e-5
+    d = np.zeros((1, 1, 3, 3), np.float32)
+    d[0, 0, 0, 2] = 1.0  # picks x[h-1, w+1]
+    x1 = r.standard_normal((1, 1, 5, 5)).astype(np.float32)
+    y = ref.conv2d(x1, d, None, (1, 1), (1, 1, 1, 1))
+    want = np.zeros_like(x1)
+    want[0, 0, 1:, :-1] = x1[0, 0, :-1, 1:]
+    assert np.array_equal(y, want)
+
+
+# ---------------------------------------------------------------- pooling ----
+def test_pool_kats_from_reference_doctest(ref):
+    """odla_ops_nn_test.cc:38-78 and :523-560."""
+    x = np.arange(1, 17, dtype=np.float32).reshape(1, 1, 4, 4)
+    assert ref.pool2d(x, (3, 3), (1, 1), (0, 0, 0, 0), None, False).reshape(-1).tolist() == [6, 7, 10, 11]
+    assert ref.pool2d(x, (3, 3), (1, 1), (0, 0, 0, 0), None, True).reshape(-1).tolist() == [11, 12, 15, 16]
+
+
+@pytest.mark.parametrize("i", range(3))
+def test_maxpool_against_reference_kernel_vectors(ref, i):
+    x = GOLD["pool%d_x" % i]
+    k, s, p = (int(v) for v in GOLD["pool%d_attr" % i])
+    y = ref.pool2d(x, (k, k), (s, s), (p, p, p, p), None, True)
+    assert np.array_equal(y, GOLD["pool%d_y" % i])
+
+
+def test_avgpool_padding_rules(ref):
+    """ONNX averagepool_2d_pads (exclude padding, passes on the reference CPU
+    backend) and count_include_pad, on a constant image where both are closed forms."""
+    x = np.ones((1, 1, 4, 4), np.float32)
+    ex = ref.pool2d(x, (3, 3), (1, 1), (1, 1, 1, 1), None, False, False)
+    assert np.allclose(ex, 1.0)
+    inc = ref.pool2d(x, (3, 3), (1, 1), (1, 1, 1, 1), None, False, True)
+    assert np.isclose(inc[0, 0, 0, 0], 4.0 / 9.0) and np.isclose(inc[0, 0, 0, 1], 6.0 / 9.0) and np.isclose(inc[0, 0, 1, 1], 1.0)
+
+
+def test_maxpool_ceil_mode_shape(ref):
+    """odla_dnnl.cc:1411-1429: an output one larger than the floor formula is served by extra back padding."""
+    x = rng(5).standard_normal((1, 1, 6, 6)).astype(np.float32)
+    y = ref.pool2d(x, (3, 3), (2, 2), (0, 0, 0, 0), (3, 3), True)
+    assert y.shape == (1, 1, 3, 3)
+    assert y[0, 0, 2, 2] == x[0, 0, 4:, 4:].max()
+
+
+# ------------------------------------------------------------ gemm/softmax ----
+@pytest.mark.parametrize("i", range(3))
+def test_gemm_against_reference_kernel_vectors(ref, i):
+    a, b, c = GOLD["gemm%d_a" % i], GOLD["gemm%d_b" % i], GOLD["gemm%d_c" % i]
+    ta, tb, alpha, beta = GOLD["gemm%d_attr" % i]
+    rb = ref.RefBuilder({})
+    y = rb.gemm(a, b, c.reshape(1, -1), bool(ta), bool(tb), float(alpha), float(beta))
+    want = GOLD["gemm%d_y" % i]
+    assert np.max(np.abs(y - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+def test_gemm_kat_from_reference_doctest(ref):
+    """odla_ops_test.cc:39-79: ones[4,16] x ones[16,8] = 16."""
+    rb = ref.RefBuilder({})
+    assert np.all(rb.gemm(np.ones((4, 16), np.float32), np.ones((16, 8), np.float32), None, False, False, 1.0, 0.0) == 16.0)
+
+
+@pytest.mark.parametrize("i", range(2))
+def test_softmax_against_reference_kernel_vectors(ref, i):
+    rb = ref.RefBuilder({})
+    y = rb.softmax(GOLD["softmax%d_x" % i], -1)
+    assert np.max(np.abs(y - GOLD["softmax%d_y" % i])) <= 1e-6
+
+
+def test_softmax_large_number_and_sum(ref):
+    rb = ref.RefBuilder({})
+    x = np.array([[0, 1, 2, 3], [10000, 10001, 10002, 10003]], np.float32)
+    y = rb.softmax(x, -1)
+    assert np.allclose(y[0], [0.032058604, 0.08714432, 0.23688284, 0.6439143], atol=1e-7)
+    assert np.allclose(y[0], y[1]) and np.allclose(y.sum(axis=1), 1.0)
+    ly = rb.softmax(x, -1, log=True)
+    assert np.allclose(np.exp(ly), y, atol=1e-6)
+
+
+# ------------------------------------------------------------ normalisation ----
+def test_batchnorm_kat_from_reference_doctest(ref):
+    """odla_ops_nn_test.cc:80-145."""
+    rb = ref.RefBuilder({})
+    x = np.array([-1, 0, 1, 2, 3, 4], np.float32).reshape(1, 2, 1, 3)
+    y = rb.batchnorm(x, np.array([0, 3], np.float32), np.array([1, 1.5], np.float32), 1e-5,
+                     np.array([1.0, 1.5], np.float32), np.array([0, 1], np.float32))
+    assert np.max(np.abs(y.reshape(-1) - [-0.999995, 0, 0.999995, -0.224741, 1, 2.22474])) < 1e-5
+
+
+def test_batchnorm_folding_formula(ref):
+    """lib/transforms/inst_simplify.cc:1408-1415: y = x*m + (b - mean*m), m = s/sqrt(var+eps)."""
+    r = rng(6)
+    x = r.standard_normal((2, 3, 4, 4)).astype(np.float32)
+    mean, var = r.standard_normal(3), r.random(3) + 0.5
+    g, b = r.standard_normal(3), r.standard_normal(3)
+    rb = ref.RefBuilder({})
+    y = rb.batchnorm(x, mean, var, 1e-3, g, b)
+    m = g / np.sqrt(var + 1e-3)
+    want = x * m.reshape(1, 3, 1, 1) + (b - mean * m).reshape(1, 3, 1, 1)
+    assert np.max(np.abs(y - want)) < 1e-5
+
+
+def test_layernorm_invariants(ref):
+    """lib/transforms/fusion.cc:296-313: biased variance; with gamma 1 / beta 0 each row
+    has mean 0 and variance 1; gamma and beta act as an affine map afterwards."""
+    r = rng(7)
+    x = (r.standard_normal((5, 64)) * 3 + 2).astype(np.float32)
+    rb = ref.RefBuilder({})
+    y = rb.layernorm(x, 1, 1e-12)
+    assert np.max(np.abs(y.mean(axis=1))) < 1e-6 and np.max(np.abs(y.var(axis=1) - 1)) < 1e-5
+    g, b = r.standard_normal(64).astype(np.float32), r.standard_normal(64).astype(np.float32)
+    assert np.max(np.abs(rb.layernorm(x, 1, 1e-12, g, b) - (y * g + b))) < 1e-5
+    # translation invariance and scale invariance of the normalised value
+    assert np.max(np.abs(rb.layernorm(x * 4 + 10, 1, 1e-12) - y)) < 1e-4
+
+
+def test_gelu_erf_closed_forms(ref):
+    """odla_dnnl.cc:1868-1876 against math.erf / math.tanh in float64."""
+    rb = ref.RefBuilder({})
+    x = np.linspace(-5, 5, 101).astype(np.float32)
+    want = np.array([0.5 * v * (1 + math.erf(v / math.sqrt(2))) for v in x.astype(np.float64)])
+    assert np.max(np.abs(rb.gelu(x) - want)) < 1e-6
+    want_t = np.array([0.5 * v * (1 + math.tanh(math.sqrt(2 / math.pi) * (v + 0.044715 * v ** 3))) for v in x.astype(np.float64)])
+    assert np.max(np.abs(rb.gelu(x, True) - want_t)) < 1e-6
+    assert np.max(np.abs(rb.erf(x) - np.array([math.erf(v) for v in x.astype(np.float64)]))) < 1e-6
+
+
+# ------------------------------------------------------------- broadcast ----
+def test_reference_alignment_examples(ref):
+    """The three examples in the comment at odla_dnnl.h:303-306."""
+    assert ref.align_like_reference((1, 5), (1, 4, 1)) == (1, 1, 5)
+    assert ref.align_like_reference((64,), (1, 64, 128)) == (1, 64, 1)
+    assert ref.align_like_reference((64,), (1, 64, 64)) == (1, 1, 64)
+    with pytest.raises(ValueError):
+        ref.align_like_reference((7, 31, 64), (2, 31, 64, 64))
+
+
+# ---------------------------------------------------------- quantisation ----
+def test_quantize_onnx_published_example(ref):
+    rb = ref.RefBuilder({})
+    x = np.array([0, 2, 3, 1000, -254, -1000], np.float32)
+    q = rb.quantize(x, [2.0], [128])
+    assert q.tolist() == [128, 129, 130, 255, 1, 0]
+    assert rb.dequantize(q, [2.0], [128]).tolist() == [0, 2, 4, 254, -254, -256]
+
+
+def test_quantize_round_half_even_exhaustive(ref):
+    """Every half-integer in range rounds to the even neighbour."""
+    rb = ref.RefBuilder({})
+    k = np.arange(-300, 300)
+    x = (k + 0.5).astype(np.float32)
+    q = rb.quantize(x, [1.0], [0], signed=True).astype(np.int64)
+    want = np.clip(np.where(k % 2 == 0, k, k + 1), -128, 127)
+    assert np.array_equal(q, want)
+
+
+def test_requant_formula_rounding_and_saturation(ref):
+    acc = np.array([[[[-1000, -3, -1, 0, 1, 3, 5, 1000, 2 ** 24 + 1]]]], np.int32).transpose(0, 3, 1, 2).copy()
+    acc = acc.reshape(1, 9, 1, 1)
+    mul = np.full(9, 0.5, np.float32)
+    q = ref.requant_q8(acc, mul, zp=10, lo=0).reshape(-1)
+    # 0.5*acc: -500,-1.5,-0.5,0,0.5,1.5,2.5,500,2^23 -> rne -> +10 -> clamp
+    assert q.tolist() == [0, 8, 10, 10, 10, 12, 12, 255, 255]
+    assert ref.requant_q8(acc, mul, zp=10, lo=10).reshape(-1).tolist() == [10, 10, 10, 10, 10, 12, 12, 255, 255]
+
+
+def test_q8_accumulators_against_int64_brute_force(ref):
+    r = rng(8)
+    N, C, H, W, O, k = 2, 5, 6, 6, 4, 3
+    xq = r.integers(0, 256, (N, C, H, W)).astype(np.uint8)
+    wq = r.integers(-127, 128, (O, C, k, k)).astype(np.int8)
+    b = r.integers(-1000, 1000, O).astype(np.int32)
+    zp = 131
+    acc = ref.conv2d_q8_acc(xq, zp, wq, b, (2, 2), (1, 1, 1, 1))
+    want = brute_conv(xq.astype(np.float64) - zp, wq.astype(np.float64), b.astype(np.float64), (2, 2), (1, 1, 1, 1), (1, 1), 1)
+    # padding contributes (zp - zp) = 0: brute_conv skips out-of-range taps, same thing
+    assert np.array_equal(acc.astype(np.int64), want.astype(np.int64))
+
+
+def test_weight_and_activation_schemes(ref, models):
+    """utils/halo_pgq.py:283-297 and weights_quantizer.cc:126-176 of the reference:
+    scale=(max-min)/255, zp=round(-min/scale) clamped to [0,255]; symmetric weights max|w|/127.
+    The host-side table writer and the oracle agree."""
+    s, z = ref.act_qparams(-1.0, 3.0)
+    assert np.isclose(s, 4.0 / 255) and z == 64
+    assert ref.act_qparams(0.5, 2.0)[1] == 0            # range widened to contain zero
+    assert models.act_qparams(-1.0, 3.0) == (s, z)
+    w = np.array([[0.5, -1.27], [0.0, 0.0]], np.float32)
+    sw = ref.weight_qparams(w)
+    assert np.isclose(sw[0], 0.01) and sw[1] == 1.0
+    assert ref.quantize_weights(w, sw).tolist() == [[50, -127], [0, 0]]
+    assert ref.quantize_bias(np.array([0.1, 0.0], np.float32), 0.02, sw).tolist() == [500, 0]
+
+
+# -------------------------------------------------------------------- NMS ----
+ONNX_BOXES = np.array([[[0, 0, 1, 1], [0, 0.1, 1, 1.1], [0, -0.1, 1, 0.9], [0, 10, 1, 11], [0, 10.1, 1, 11.1],
+                        [0, 100, 1, 101]]], np.float32)
+ONNX_SCORES = np.array([[[0.9, 0.75, 0.6, 0.95, 0.5, 0.3]]], np.float32)
+
+
+def test_nms_onnx_published_examples(ref):
+    sel = lambda o: [r[2] for r in o.tolist() if r[2] >= 0]
+    assert sel(ref.nms(ONNX_BOXES, ONNX_SCORES, 3, 0.5, 0.0)) == [3, 0, 5]          # suppress_by_IOU
+    assert sel(ref.nms(ONNX_BOXES, ONNX_SCORES, 3, 0.5, 0.4)) == [3, 0]             # ..._and_scores
+    assert sel(ref.nms(ONNX_BOXES, ONNX_SCORES, 2, 0.5, 0.0)) == [3, 0]             # limit_output_size
+    flipped = np.array([[[1, 1, 0, 0], [0, 0.1, 1, 1.1], [0, 0.9, 1, -0.1], [0, 10, 1, 11], [1, 10.1, 0, 11.1],
+                         [1, 101, 0, 100]]], np.float32)
+    assert sel(ref.nms(flipped, ONNX_SCORES, 3, 0.5, 0.0)) == [3, 0, 5]             # flipped_coordinates
+    same = np.tile(np.array([0, 0, 1, 1], np.float32), (1, 10, 1))
+    assert sel(ref.nms(same, np.full((1, 1, 10), 0.9, np.float32), 3, 0.5, 0.0)) == [0]   # identical_boxes
+    two = np.concatenate([ONNX_BOXES, ONNX_BOXES])
+    out = ref.nms(two, np.concatenate([ONNX_SCORES, ONNX_SCORES]), 2, 0.5, 0.0)
+    assert out.tolist() == [[0, 0, 3], [0, 0, 0], [1, 0, 3], [1, 0, 0]]             # two_batches
+
+
+def test_nms_against_brute_force(ref):
+    """Sequential restatement of the reference selection loop (dnnl_utils_avx512.h:1020-1070)
+    in float64-free plain Python on 48 boxes, plus the invariants of the result."""
+    r = rng(9)
+    B, C = 48, 3
+    cy, cx = r.random(B) * 4, r.random(B) * 4
+    boxes = np.stack([cy - 0.5, cx - 0.5, cy + 0.5, cx + 0.5], -1).astype(np.float32)[None]
+    scores = r.random((1, C, B)).astype(np.float32)
+
+    def iou(a, b):
+        f = np.float32
+        ai = f(f(a[2] - a[0]) * f(a[3] - a[1]))
+        aj = f(f(b[2] - b[0]) * f(b[3] - b[1]))
+        if ai <= 0 or aj <= 0:
+            return f(0)
+        ih = max(f(min(a[2], b[2]) - max(a[0], b[0])), f(0))
+        iw = max(f(min(a[3], b[3]) - max(a[1], b[1])), f(0))
+        inter = f(ih * iw)
+        return f(inter / f(f(ai + aj) - inter))
+
+    cand = []
+    for b in range(B):
+        c = int(np.argmax(scores[0, :, b]))
+        if scores[0, c, b] > 0.3:
+            cand.append((-float(scores[0, c, b]), b, c))
+    cand.sort()
+    kept = []
+    for _, b, c in cand:
+        if len(kept) >= 10:
+            break
+        if all(iou(boxes[0, b], boxes[0, kb]) < np.float32(0.45) for kb, _ in kept):
+            kept.append((b, c))
+    out = ref.nms(boxes, scores, 10, 0.45, 0.3)
+    got = [(r_[2], r_[1]) for r_ in out.tolist() if r_[2] >= 0]
+    assert got == kept
+    for i in range(len(got)):
+        for j in range(i):
+            assert iou(boxes[0, got[i][0]], boxes[0, got[j][0]]) < 0.45
+
+
+# -------------------------------------------------------- live reference ----
+def test_live_reference_kernels_if_built(ref):
+    """When oracle/_ref/libsn_rt.so exists (built from the reference tree), one more
+    conv shape is compared live; otherwise the committed vectors above stand in."""
+    import ctypes
+    path = os.path.join(entry.ROOT, "oracle", "_ref", "libsn_rt.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/_ref/libsn_rt.so not built on this machine")
+    L = ctypes.CDLL(path)
+    r = rng(10)
+    x = r.standard_normal((1, 3, 10, 10)).astype(np.float32)
+    w = r.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    y = np.zeros((1, 4, 5, 5), np.float32)
+    f32p, i64 = ctypes.POINTER(ctypes.c_float), ctypes.c_int64
+    L._sn_rt_conv2d_f32_nchw.argtypes = [f32p, f32p, f32p] + [i64] * 15
+    L._sn_rt_conv2d_f32_nchw(y.ctypes.data_as(f32p), x.ctypes.data_as(f32p), w.ctypes.data_as(f32p),
+                             1, 10, 10, 3, 5, 5, 4, 3, 3, 2, 2, 1, 1, 1, 1)
+    got = ref.conv2d(x, w, None, (2, 2), (1, 1, 1, 1))
+    assert np.max(np.abs(got - y)) <= 1e-5 * np.max(np.abs(y))
