@@ -1,15 +1,20 @@
 #!/usr/bin/env python3
 """Throughput benchmark of the ODLA hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50_fp16|resnet50_int8|resnet50_fp32]
-                  [--batch 256] [--cpu-sample N]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--batch B]
+                  [--cpu-sample N] [--dump-steps FILE]
+
+Workloads: resnet50_fp16 (default; the configuration the headline metric is
+quoted on), resnet50_int8, resnet50_bf16, resnet50_fp32, yolov3_fp16, bert_bf16,
+mnist_fp32.
 
 A step is one odla_ExecuteComputation of the whole graph on one batch of
 synthetic input that is already resident in device memory (arguments and
 outputs are bound to buffers from odla_AllocateDeviceMemory).  Prints ONE JSON
-line with images/s, the roofline of the dominant kernel class (the
-implicit-GEMM convolutions, measured live with HIP events around un-captured
-launches on the library's stream) and the CPU oracle timed on a bounded sample.
+line with the throughput, the roofline of the dominant kernel class (the
+implicit-GEMM convolution / GEMM launches, timed live with HIP events around
+un-captured launches on the library's own stream) and the CPU oracle timed on a
+bounded sample of the same workload.
 """
 import argparse
 import ctypes
@@ -18,88 +23,105 @@ import os
 import sys
 import time
 
-import numpy as np
-
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 PEAK = {"fp16": 2500.0, "bf16": 2500.0, "int8": 5000.0, "fp32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
+DTYPE = {"fp16": "f16", "bf16": "bf16", "fp32": "f32", "int8": "i8"}
+METRIC = "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW"
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="resnet50_fp16")
-    ap.add_argument("--batch", type=int, default=256)
-    ap.add_argument("--cpu-sample", type=int, default=4, help="images timed on the CPU oracle (0 = skip)")
-    ap.add_argument("--dump-steps", default=None, help="write the per-launch timing table to this file")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: every box of this build has a single MI355X and the path "
-              "shards by batch without any collective; run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+class Workload:
+    def __init__(self, name, unit, batch, flop_per_step, desc, build, feeds, ref_run, mode, table=None):
+        self.name, self.unit, self.batch, self.flop, self.desc = name, unit, batch, flop_per_step, desc
+        self.build, self.feeds, self.ref_run, self.mode, self.table = build, feeds, ref_run, mode, table
 
-    pkg = entry.load()
+
+def make_workload(name, batch, pkg):
     odla, models = pkg.odla, pkg.models
-    L = odla.load_library()
-    mode = args.workload.split("_")[1]
-    if mode not in ("fp16", "fp32", "bf16", "int8"):
-        print("unknown workload %s" % args.workload, file=sys.stderr)
-        sys.exit(2)
+    family, mode = name.rsplit("_", 1)
+    if family == "resnet50":
+        batch = batch or 256
+        w = models.resnet50_weights()
+        feeds = models.resnet50_input(batch)
+        table = None
+        if mode == "int8":
+            table = odla.quant_table(models.resnet50_quant_entries(w, calibrate_resnet_on_gpu(odla, models, w)))
 
-    batch = args.batch
-    w = models.resnet50_weights()
-    feeds = models.resnet50_input(batch)
-    table = None
-    if mode == "int8":
-        table = odla.quant_table(models.resnet50_quant_entries(w, calibrate_on_gpu(odla, models, w)))
-    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16=(mode == "bf16"), quant_table=table)
-    models.build_resnet50(hb, w, batch)
-    sess = hb.session(use_graph=True)
-    sess.bind_device_io(feeds)
+        def ref_run(ref, n):
+            rb = ref.RefBuilder(models.resnet50_input(n))
+            models.build_resnet50(rb, w, n)
+        return Workload(name, "images/s", batch, models.RESNET50_GFLOP_PER_IMAGE * 1e9 * batch,
+                        "ResNet-50 v1.5 %s NCHW [%d,3,224,224], folded BN, random He-normal weights, softmax head; "
+                        "inputs/outputs resident in HBM" % (mode, batch),
+                        lambda b: models.build_resnet50(b, w, batch), feeds, ref_run, mode, table)
+    if family == "yolov3":
+        my = pkg.models_yolo
+        batch = batch or 16
+        feeds = my.yolov3_input(batch)
+        # head calibration: logits to unit std, bias so that ~1% of the scores pass 0.3
+        w0 = my.yolov3_weights()
+        hb = odla.HipBuilder(fp16=True)
+        my.build_yolov3(hb, w0, 2, postprocess=False)
+        s = hb.session()
+        h = s.run(my.yolov3_input(2))
+        s.close()
+        hb.destroy()
+        scales, bias = my.calibrate_heads([h["head%d" % i] for i in range(3)])
+        w = my.yolov3_weights(head_bias=bias, head_scale=scales)
+        macs = sum(co * ci * k * k * (416 // st) ** 2 for co, ci, k, st in yolo_conv_geometry(my))
 
-    for _ in range(args.warmup):
-        sess.execute()
-    # odla_ExecuteComputation returns after the device is idle, so the wall
-    # clock around K executions is the device-synchronised time of K steps.
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        sess.execute()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    images_per_s = batch / (ms_per_step * 1e-3)
+        def ref_run(ref, n):
+            rb = ref.RefBuilder(my.yolov3_input(n))
+            my.build_yolov3(rb, w, n)
+        return Workload(name, "images/s", batch, 2.0 * macs * batch,
+                        "YOLOv3 %s NCHW [%d,3,416,416], Darknet-53 + FPN + 3 heads, sigmoid decode + batched NMS "
+                        "(IoU 0.45, score 0.3, 80 classes)" % (mode, batch),
+                        lambda b: my.build_yolov3(b, w, batch), feeds, ref_run, mode)
+    if family == "bert":
+        mb = pkg.models_bert
+        batch = batch or 64
+        seq = 128
+        w = mb.bert_weights()
+        feeds = mb.bert_input(batch, seq)
 
-    # Roofline of the convolution kernels: all conv + FC launches of one step,
-    # timed with HIP events on the library's own stream (library entry point
-    # odla_hip_ProfileSteps), algorithmic FLOPs = 2 * MACs of the layers.
-    roof = None
-    if hasattr(L, "odla_hip_ProfileSteps"):
-        roof = profile_roofline(L, sess, hb, mode, batch, models, args.dump_steps)
+        def ref_run(ref, n):
+            rb = ref.RefBuilder(mb.bert_input(n, seq))
+            mb.build_bert(rb, w, n, seq)
+        return Workload(name, "sequences/s", batch, mb.bert_gflop_per_sequence(seq) * 1e9 * batch,
+                        "BERT-base encoder %s, batch %d x seq %d, 12 layers, hidden 768, 12 heads, FFN 3072"
+                        % (mode, batch, seq),
+                        lambda b: mb.build_bert(b, w, batch, seq), feeds, ref_run, mode)
+    if family == "mnist":
+        batch = batch or 64
+        w = models.mnist_weights()
+        feeds = models.mnist_input(batch)
 
-    cpu = None
-    if args.cpu_sample > 0:
-        cpu = cpu_baseline(models, w, args.cpu_sample)
-
-    line = {
-        "metric": "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW",
-        "value": round(images_per_s, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": {"fp16": "f16", "bf16": "bf16", "fp32": "f32", "int8": "i8"}[mode],
-        "data": "synthetic",
-        "config": {"workload": "ResNet-50 v1.5 %s NCHW [%d,3,224,224], folded BN, random He-normal weights, "
-                               "softmax head; inputs/outputs resident in HBM" % (mode, batch),
-                   "batch": batch, "executor": "hipGraph replay through odla_ExecuteComputation"},
-        "roofline": roof, "cpu_baseline": cpu,
-    }
-    print(json.dumps(line))
-    sess.close()
-    hb.destroy()
+        def ref_run(ref, n):
+            rb = ref.RefBuilder(models.mnist_input(n))
+            models.build_mnist(rb, w, n)
+        return Workload(name, "images/s", batch, 2.0 * 784 * 10 * batch,
+                        "mnist_simple softmax regression fp32, Gemm+Add+Softmax, batch %d" % batch,
+                        lambda b: models.build_mnist(b, w, batch), feeds, ref_run, mode)
+    raise SystemExit("unknown workload %s" % name)
 
 
-def calibrate_on_gpu(odla, models, w, batch=4, n_batches=8):
+def yolo_conv_geometry(my):
+    """(cout, cin, k, stride of the OUTPUT grid w.r.t. the input image) per convolution at width 1."""
+    out = []
+    stride = 1
+    for name, cout, cin, k, s, act in my.yolov3_conv_specs():
+        if name.startswith("d"):
+            stride *= s
+            out.append((cout, cin, k, stride))
+        else:
+            hi = int(name[1])
+            out.append((cout, cin, k, {1: 32, 2: 16, 3: 8}[hi] * (2 if name.endswith(".lat") else 1)))
+    return out
+
+
+def calibrate_resnet_on_gpu(odla, models, w, batch=4, n_batches=8):
     """Activation ranges for the int8 plan: min/max of every named activation of
     the fp32 graph over 32 seeded N(0,1) images (8 batches of 4), computed by the
     fp32 plan of the library itself."""
@@ -123,14 +145,77 @@ def calibrate_on_gpu(odla, models, w, batch=4, n_batches=8):
     return ranges
 
 
-def profile_roofline(L, sess, hb, mode, batch, models, dump_path=None):
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="resnet50_fp16")
+    ap.add_argument("--batch", type=int, default=0)
+    ap.add_argument("--cpu-sample", type=int, default=-1,
+                    help="units (images / sequences) timed on the CPU oracle; 0 = skip, -1 = per-workload default")
+    ap.add_argument("--dump-steps", default=None, help="write the per-launch timing table to this file")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has a single MI355X and the path "
+              "shards by batch without any collective; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    pkg = entry.load()
+    odla = pkg.odla
+    L = odla.load_library()
+    wl = make_workload(args.workload, args.batch, pkg)
+    mode = wl.mode
+
+    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16=(mode == "bf16"), quant_table=wl.table)
+    wl.build(hb)
+    sess = hb.session(use_graph=True)
+    sess.bind_device_io(wl.feeds)
+
+    for _ in range(args.warmup):
+        sess.execute()
+    # odla_ExecuteComputation returns after the device is idle, so the wall
+    # clock around K executions is the device-synchronised time of K steps.
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sess.execute()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    per_s = wl.batch / (ms_per_step * 1e-3)
+
+    roof = profile_roofline(L, sess, wl, args.dump_steps)
+
+    cpu = None
+    sample = args.cpu_sample
+    if sample < 0:
+        sample = {"resnet50": 4, "yolov3": 1, "bert": 2, "mnist": 64}[args.workload.rsplit("_", 1)[0]]
+    if sample > 0:
+        cpu = cpu_baseline(wl, sample)
+
+    line = {
+        "metric": METRIC if wl.name.startswith("resnet50") else "%s, %s" % (wl.unit, wl.name),
+        "value": round(per_s, 1), "unit": wl.unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": DTYPE[mode], "data": "synthetic",
+        "config": {"workload": wl.desc, "batch": wl.batch,
+                   "executor": "hipGraph replay through odla_ExecuteComputation"},
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    sess.close()
+    hb.destroy()
+
+
+def profile_roofline(L, sess, wl, dump_path=None):
+    """All conv / gemm launches of one step, each timed with a HIP event pair on
+    the library's stream (odla_hip_ProfileSteps); algorithmic FLOPs = 2 x MACs."""
     class StepTime(ctypes.Structure):
         _fields_ = [("name", ctypes.c_char * 64), ("ms", ctypes.c_float)]
 
     L.odla_hip_ProfileSteps.restype = ctypes.c_int32
     L.odla_hip_ProfileSteps.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(StepTime), ctypes.c_int32,
                                         ctypes.POINTER(ctypes.c_int32)]
-    cap = 1024
+    cap = 4096
     buf = (StepTime * cap)()
     n = ctypes.c_int32(0)
     st = L.odla_hip_ProfileSteps(sess.ctx, 10, buf, cap, ctypes.byref(n))
@@ -140,37 +225,35 @@ def profile_roofline(L, sess, hb, mode, batch, models, dump_path=None):
         with open(dump_path, "w") as f:
             for i in range(n.value):
                 f.write("%-40s %9.4f ms\n" % (buf[i].name.decode(), buf[i].ms))
-    conv_ms = 0.0
-    total_ms = 0.0
+    mm_ms = total_ms = 0.0
     launches = 0
     for i in range(n.value):
         name = buf[i].name.decode()
         total_ms += buf[i].ms
-        if name.startswith("conv") or name.startswith("gemm"):
-            conv_ms += buf[i].ms
+        if name.startswith("conv") or name.startswith("gemm:"):
+            mm_ms += buf[i].ms
             launches += 1
-    flop = models.RESNET50_GFLOP_PER_IMAGE * 1e9 * batch
-    achieved = flop / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
-    peak = PEAK[mode]
+    achieved = wl.flop / (mm_ms * 1e-3) / 1e12 if mm_ms > 0 else 0.0
+    peak = PEAK[wl.mode]
     return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
             "frac": round(achieved / peak, 4), "traffic": None,
-            "kernel": "igemm_kernel (all %d conv/FC launches of one step)" % launches,
-            "conv_ms_per_step": round(conv_ms, 4), "all_kernels_ms_per_step": round(total_ms, 4)}
+            "kernel": "igemm_kernel (all %d conv/gemm launches of one step, avg %.1f us)"
+                      % (launches, 1e3 * mm_ms / max(launches, 1)),
+            "mm_ms_per_step": round(mm_ms, 4), "all_kernels_ms_per_step": round(total_ms, 4),
+            "launches_per_step": n.value}
 
 
-def cpu_baseline(models, w, sample):
-    """The CPU oracle (a port of the reference CPU path's arithmetic) on `sample`
-    images of the same workload, all host cores through OpenMP."""
+def cpu_baseline(wl, sample):
+    """The CPU oracle (a port of the reference CPU path's arithmetic, fp32) on
+    `sample` units of the same workload, all host cores through OpenMP / BLAS."""
     ref = entry.load_oracle()
-    feeds = models.resnet50_input(sample)
-    rb = ref.RefBuilder(feeds)
-    models.build_resnet50(rb, w, sample)      # warm-up (page in weights, spin up threads)
+    wl.ref_run(ref, sample)      # warm-up (page in weights, spin up threads)
     t0 = time.perf_counter()
-    rb = ref.RefBuilder(feeds)
-    models.build_resnet50(rb, w, sample)
+    wl.ref_run(ref, sample)
     dt = time.perf_counter() - t0
-    return {"value": round(sample / dt, 2), "unit": "images/s", "cores": ref.num_threads(), "kind": "port",
-            "sample": "%d images of the same ResNet-50 fp32 graph, one pass after one warm-up pass" % sample}
+    return {"value": round(sample / dt, 2), "unit": wl.unit, "cores": ref.num_threads(), "kind": "port",
+            "sample": "%d %s of the same graph in fp32, one pass after one warm-up pass"
+                      % (sample, wl.unit.split("/")[0])}
 
 
 if __name__ == "__main__":

@@ -1,8 +1,8 @@
 """odla_hip: an ODLA runtime platform for one AMD Instinct MI355X (gfx950).
 
 The product is ``libodla_hip.so`` (built from ``csrc/``); ``odla`` is the ctypes
-host side that drives it through the ODLA C ABI and ``models`` holds the graph
-descriptions of the benchmark configurations.
+host side that drives it through the ODLA C ABI; ``models``, ``models_yolo`` and
+``models_bert`` hold the graph descriptions of the benchmark configurations.
 
 The directory name is not a Python identifier; load the package with
 ``importlib`` under the name ``halo_amd`` (see ``load()`` in the repository's
@@ -10,3 +10,5 @@ The directory name is not a Python identifier; load the package with
 """
 from . import odla  # noqa: F401
 from . import models  # noqa: F401
+from . import models_bert  # noqa: F401
+from . import models_yolo  # noqa: F401

@@ -69,6 +69,7 @@ struct VState {
 // Epilogue collected while fusing followers into a Conv / Gemm.
 struct Epilogue {
   std::vector<float> row_scale;  // per output channel multiplier folded into weights
+  float scalar = 1.f;            // uniform multiplier applied to the accumulator (kernel alpha)
   std::vector<float> bias;       // per output channel
   bool has_bias = false;
   _odla_value* residual = nullptr;
@@ -686,7 +687,7 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
         ep->has_bias = true;
         took = true;
       }
-    } else if (nx.op == OP_BINARY && (nx.i[0] == BIN_ADD || nx.i[0] == BIN_MUL || nx.i[0] == BIN_SUB)) {
+    } else if (nx.op == OP_BINARY && (nx.i[0] == BIN_ADD || nx.i[0] == BIN_MUL || nx.i[0] == BIN_SUB || nx.i[0] == BIN_DIV)) {
       const bool cur_is_lhs = nx.in[0] == cur;
       _odla_value* other = cur_is_lhs ? nx.in[1] : nx.in[0];
       if (other != cur && nx.out->shape == cur->shape) {
@@ -706,6 +707,15 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
           } else if (nx.i[0] == BIN_SUB && cur_is_lhs) {
             for (int64_t c = 0; c < channels; ++c) ep->bias[c] -= vals[c];
             ep->has_bias = true;
+            took = true;
+          } else if (nx.i[0] == BIN_MUL && other->shape.numel() == 1) {
+            ep->scalar *= vals[0];
+            for (int64_t c = 0; c < channels; ++c) ep->bias[c] *= vals[0];
+            took = true;
+          } else if (nx.i[0] == BIN_DIV && cur_is_lhs && other->shape.numel() == 1 && vals[0] != 0.f) {
+            const float inv = 1.0f / vals[0];
+            ep->scalar *= inv;
+            for (int64_t c = 0; c < channels; ++c) ep->bias[c] *= inv;
             took = true;
           } else if (nx.i[0] == BIN_MUL) {
             if (ep->row_scale.empty()) ep->row_scale.assign((size_t)channels, 1.f);
@@ -1064,6 +1074,7 @@ void Planner::lower_conv(int ni) {
   ip.w_rows = Og; ip.w_cols = w_rs; ip.w_rs = w_rs;
   ip.in_dt = dt; ip.out_dt = dt;
   ip.batch = G;
+  ip.alpha = ep.scalar;
   if (G > 1) { ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og; }
   ip.ycs = (int)O;
 
@@ -1127,7 +1138,6 @@ void Planner::lower_gemm(int ni) {
   if (full_c == nullptr) collect_epilogue(ni, Nn, os.rank - 1, &ep);
   else { ep.residual = full_c; ep.final_value = n.out; }
   _odla_value* outv = ep.final_value;
-  if (alpha != 1.f && ep.has_bias && !ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: alpha with folded scale");
 
   // ---- A operand: row-major [lead][M][K], K padded to the vector width ----
   int ta = get(A, L_ROWMAJOR, FORM_FLOAT);
@@ -1159,14 +1169,13 @@ void Planner::lower_gemm(int ni) {
   ip.C = Kp; ip.xcs = Kp;
   ip.Kout = (int)Nn;
   ip.in_dt = dt; ip.out_dt = dt;
-  ip.alpha = alpha;
+  ip.alpha = alpha * ep.scalar;
   ip.ycs = (int)Nn;
   int tw;
   if (B->kind == _odla_value::CONSTANT && (shared_b || lead == 1)) {
     // weights: pack once.  B[k][n] (so=1, si=N) or B^T[n][k] (so=K, si=1)
     int w_rs = 0;
     const int64_t so = tB ? K : 1, si = tB ? 1 : Nn;
-    if (alpha != 1.f && !ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: alpha with folded scale");
     tw = pack_weights(B, dt, 1, (int)Nn, (int)K, 1, 1, Kp, so, si, 0, 0, ep.row_scale, &w_rs, nullptr);
     ip.w_rows = (int)Nn; ip.w_cols = w_rs; ip.w_rs = w_rs;
     ip.N = (int)(lead * M);
