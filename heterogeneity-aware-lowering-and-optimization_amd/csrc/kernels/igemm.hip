@@ -74,18 +74,17 @@ __device__ __forceinline__ float epi_act(float v, ActKind act, float a, float b)
 template <typename TOut>
 struct EpiFloat {
   using AccE = float;
+  using RVec = uintx4;  // eight 2-byte residual elements fetched ahead of use
+  static constexpr bool kPrefetchResidual = sizeof(TOut) == 2;
+  // b8: this lane's eight bias values (zero when absent); rpre: residual vector
+  // fetched ahead (valid when have_rpre), otherwise r points at the residual row.
   __device__ static __forceinline__ void store8(const IgemmParams& p, const float* acc, int nvalid, bool vec,
-                                                const float* bias, TOut* y, const TOut* r) {
+                                                const float* b8, const float*, TOut* y, const TOut* r,
+                                                bool have_rpre, RVec rpre) {
     float v[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = acc[e] * p.alpha;
+    for (int e = 0; e < 8; ++e) v[e] = acc[e] * p.alpha + b8[e];
     if (vec) {
-      if (bias != nullptr) {
-        const floatx4 b0 = *reinterpret_cast<const floatx4*>(bias);
-        const floatx4 b1 = *reinterpret_cast<const floatx4*>(bias + 4);
-        v[0] += b0.x; v[1] += b0.y; v[2] += b0.z; v[3] += b0.w;
-        v[4] += b1.x; v[5] += b1.y; v[6] += b1.z; v[7] += b1.w;
-      }
       if (r != nullptr) {
         if constexpr (sizeof(TOut) == 4) {
           const floatx4 r0 = *reinterpret_cast<const floatx4*>(r);
@@ -94,7 +93,7 @@ struct EpiFloat {
           v[4] += r1.x; v[5] += r1.y; v[6] += r1.z; v[7] += r1.w;
         } else {
           Vec16<TOut> rv;
-          rv.load(r);
+          if (have_rpre) rv.raw = rpre; else rv.load(r);
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] += rv.get(e);
         }
@@ -115,7 +114,6 @@ struct EpiFloat {
       for (int e = 0; e < 8; ++e) {
         if (e < nvalid) {
           float t = v[e];
-          if (bias != nullptr) t += bias[e];
           if (r != nullptr) t += Store<TOut>::ld(r + e);
           Store<TOut>::st(y + e, epi_act(t, p.act, p.act_a, p.act_b));
         }
@@ -135,13 +133,16 @@ template <int MODE>
 struct EpiQuant {
   using AccE = int;
   using TOut = typename QuantOut<MODE>::T;
+  using RVec = uintx2;  // eight 1-byte residual levels fetched ahead of use
+  static constexpr bool kPrefetchResidual = MODE == 0;
   __device__ static __forceinline__ void store8(const IgemmParams& p, const int* acc, int nvalid, bool vec,
-                                                const int* bias, TOut* y, const TOut* r, const float* qmul) {
+                                                const int* b8, const float* m8, TOut* y, const TOut* r,
+                                                bool have_rpre, RVec rpre) {
     if constexpr (MODE == 0) {
       int8_t rs[8] = {0, 0, 0, 0, 0, 0, 0, 0};
       if (r != nullptr) {
         if (vec) {
-          const uintx2 rv = *reinterpret_cast<const uintx2*>(r);
+          const uintx2 rv = have_rpre ? rpre : *reinterpret_cast<const uintx2*>(r);
           __builtin_memcpy(rs, &rv, 8);
         } else {
 #pragma unroll
@@ -152,21 +153,18 @@ struct EpiQuant {
       int8_t out[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        int q = 0;
-        if (e < nvalid) {
-          const int a = acc[e] + (bias ? bias[e] : 0);
-          const float f0 = (float)a * qmul[e];  // v_cvt_f32_i32 (RNE), then one v_mul_f32
-          q = (int)rintf(f0) + p.q_zp;           // v_rndne_f32
-          q = q < p.q_lo ? p.q_lo : q;
+        const int a = acc[e] + b8[e];
+        const float f0 = (float)a * m8[e];   // v_cvt_f32_i32 (RNE), then one v_mul_f32
+        int q = (int)rintf(f0) + p.q_zp;      // v_rndne_f32
+        q = q < p.q_lo ? p.q_lo : q;
+        q = q > 255 ? 255 : q;
+        if (r != nullptr) {
+          const float fa = (float)(q - p.q_zp) * p.q_scale;
+          const float fb = (float)(q_from_stored(rs[e]) - p.r_zp) * p.r_scale;
+          const float f = fa + fb;
+          q = (int)rintf(f * p.s_inv) + p.s_zp;
+          q = q < p.s_lo ? p.s_lo : q;
           q = q > 255 ? 255 : q;
-          if (r != nullptr) {
-            const float fa = (float)(q - p.q_zp) * p.q_scale;
-            const float fb = (float)(q_from_stored(rs[e]) - p.r_zp) * p.r_scale;
-            const float f = fa + fb;
-            q = (int)rintf(f * p.s_inv) + p.s_zp;
-            q = q < p.s_lo ? p.s_lo : q;
-            q = q > 255 ? 255 : q;
-          }
         }
         out[e] = q_to_stored(q);
       }
@@ -183,11 +181,11 @@ struct EpiQuant {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         if (e < nvalid) {
-          const int a = acc[e] + (bias ? bias[e] : 0);
+          const int a = acc[e] + b8[e];
           if constexpr (MODE == 2) {
             y[e] = a;
           } else {
-            float f = (float)a * qmul[e];
+            float f = (float)a * m8[e];
             if (r != nullptr) f += r[e];
             y[e] = epi_act(f, p.act, p.act_a, p.act_b);
           }
@@ -390,6 +388,52 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
   nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
   const bool vec = epi_vec && nvalid == 8;
 
+  // lane-constant epilogue operands: the lane's eight channels are the same in every pass
+  AccE b8[8];
+  float m8[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { b8[e] = 0; m8[e] = 0.f; }
+  if (nvalid > 0) {
+    if (bias != nullptr) {
+      if (vec) {
+        const intx4 t0 = *reinterpret_cast<const intx4*>(bias + n);
+        const intx4 t1 = *reinterpret_cast<const intx4*>(bias + n + 4);
+        __builtin_memcpy(&b8[0], &t0, 16);
+        __builtin_memcpy(&b8[4], &t1, 16);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (e < nvalid) b8[e] = bias[n + e];
+      }
+    }
+    if constexpr (EpiTraits<Epi>::quant) {
+      if (p.qmul != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (e < nvalid) m8[e] = p.qmul[n + e];
+      }
+    }
+  }
+
+  // residual vectors of every pass are requested now so that their latency
+  // overlaps with the staging below instead of serialising the passes
+  constexpr int NPASS = 32 / PPP;
+  using RVec = typename Epi::RVec;
+  RVec rpre[TM][NPASS];
+  const bool have_rpre = Epi::kPrefetchResidual && vec && rbase != nullptr;
+  if constexpr (Epi::kPrefetchResidual) {
+    if (have_rpre) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int ps = 0; ps < NPASS; ++ps) {
+          const int m = tile_m * BM + wm * WM + i * 32 + ps * PPP + rp;
+          const int mc = m < M ? m : M - 1;
+          rpre[i][ps] = *reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n);
+        }
+    }
+  }
+
   __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -408,34 +452,40 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
         }
       }
     }
-    __syncthreads();
+    // Each wavefront only touches its own staging slice and its LDS operations
+    // complete in issue order, so a wavefront-scope fence (no workgroup barrier)
+    // orders the parking writes before the read-back.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-    for (int ps = 0; ps < 32 / PPP; ++ps) {
+    for (int ps = 0; ps < NPASS; ++ps) {
       const int pix = ps * PPP + rp;
       const int m = tile_m * BM + wm * WM + i * 32 + pix;
+      AccE a8[8];
+      const AccE* src = stage + pix * EPI_PITCH + c8;
+      if constexpr (!EpiTraits<Epi>::quant) {
+        const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
+        const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
+        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
+        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+      } else {
+        const intx4 v0 = *reinterpret_cast<const intx4*>(src);
+        const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
+        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
+        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+      }
       if (m < M && nvalid > 0) {
-        AccE a8[8];
-        const AccE* src = stage + pix * EPI_PITCH + c8;
-        if constexpr (!EpiTraits<Epi>::quant) {
-          const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
-          const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
-          a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-          a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-        } else {
-          const intx4 v0 = *reinterpret_cast<const intx4*>(src);
-          const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
-          a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-          a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-        }
         TOut* yrow = ybase + (int64_t)m * p.ycs + n;
         const TOut* rrow = rbase ? rbase + (int64_t)m * p.rcs + n : nullptr;
-        if constexpr (EpiTraits<Epi>::quant)
-          Epi::store8(p, a8, nvalid, vec, bias ? bias + n : nullptr, yrow, rrow, p.qmul ? p.qmul + n : nullptr);
-        else
-          Epi::store8(p, a8, nvalid, vec, bias ? bias + n : nullptr, yrow, rrow);
+        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rpre[i][ps]);
       }
     }
-    if (i + 1 < TM) __syncthreads();
+    if (i + 1 < TM) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
   }
 }
 
