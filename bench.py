@@ -164,6 +164,8 @@ def main():
     pkg = entry.load()
     odla = pkg.odla
     L = odla.load_library()
+    if args.workload.startswith("streaming_"):
+        return streaming_bench(pkg, L, args)
     wl = make_workload(args.workload, args.batch, pkg)
     mode = wl.mode
 
@@ -200,6 +202,76 @@ def main():
         "config": {"workload": wl.desc, "batch": wl.batch,
                    "executor": "hipGraph replay through odla_ExecuteComputation"},
         "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    sess.close()
+    hb.destroy()
+
+
+class StepTime(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 64), ("ms", ctypes.c_float)]
+
+
+def profile_steps(L, sess, iters=10):
+    """[(launch name, mean ms)] of one execution, from odla_hip_ProfileSteps."""
+    L.odla_hip_ProfileSteps.restype = ctypes.c_int32
+    L.odla_hip_ProfileSteps.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(StepTime), ctypes.c_int32,
+                                        ctypes.POINTER(ctypes.c_int32)]
+    cap = 4096
+    buf = (StepTime * cap)()
+    n = ctypes.c_int32(0)
+    if L.odla_hip_ProfileSteps(sess.ctx, iters, buf, cap, ctypes.byref(n)) != 0:
+        return None
+    return [(buf[i].name.decode(), float(buf[i].ms)) for i in range(n.value)]
+
+
+def streaming_bench(pkg, L, args):
+    """HBM roofline of the bandwidth-bound operators (one graph of independent
+    branches at the shapes of the benchmark configurations)."""
+    odla, ms = pkg.odla, pkg.models_streaming
+    mode = args.workload.rsplit("_", 1)[1]
+    es = 4 if mode == "fp32" else 2
+    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16=(mode == "bf16"))
+    ms.build_streaming(hb)
+    sess = hb.session(use_graph=True)
+    sess.bind_device_io(ms.streaming_input())
+    for _ in range(max(args.warmup, 1)):
+        sess.execute()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        sess.execute()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    steps = profile_steps(L, sess, 10) or []
+    by_name = {}
+    for name, t in steps:
+        by_name[name] = by_name.get(name, 0.0) + t
+    rows, tot_b, tot_ms = [], 0.0, 0.0
+    for name, desc, nbytes in ms.streaming_cases(es):
+        t = by_name.get(name)
+        if t is None or t <= 0:
+            continue
+        gbs = nbytes / (t * 1e-3) / 1e9
+        rows.append((name, desc, nbytes, t, gbs))
+        tot_b += nbytes
+        tot_ms += t
+    if args.dump_steps:
+        with open(args.dump_steps, "w") as f:
+            f.write("%-26s %-62s %10s %9s %9s %6s\n" % ("launch", "operator", "MB", "us", "GB/s", "frac"))
+            for name, desc, nbytes, t, gbs in rows:
+                f.write("%-26s %-62s %10.1f %9.1f %9.0f %6.2f\n" % (name, desc, nbytes / 1e6, t * 1e3, gbs, gbs / 8000.0))
+    agg = tot_b / (tot_ms * 1e-3) / 1e9 if tot_ms > 0 else 0.0
+    worst = min(rows, key=lambda r: r[4]) if rows else None
+    line = {
+        "metric": "GB/s, streaming operators (%s)" % mode, "value": round(agg, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": DTYPE[mode], "data": "synthetic",
+        "config": {"workload": "bandwidth-bound ODLA operators at benchmark shapes (%d launches priced)" % len(rows)},
+        "roofline": {"bound": "hbm", "achieved": round(agg, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(agg / 8000.0, 4), "traffic": None,
+                     "kernel": "all streaming launches, algorithmic bytes / summed launch time",
+                     "slowest": None if worst is None else {"launch": worst[0], "GB/s": round(worst[4], 1)},
+                     "per_op_frac": {r[0]: round(r[4] / 8000.0, 3) for r in rows}},
+        "cpu_baseline": None,
     }
     print(json.dumps(line))
     sess.close()

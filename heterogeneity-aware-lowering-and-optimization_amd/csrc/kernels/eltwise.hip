@@ -10,18 +10,38 @@ namespace ohip {
 namespace {
 constexpr int kThreads = 256;
 
+// Streaming loop shape shared by the flat kernels: every thread keeps U 16-byte
+// loads in flight before it touches the data, and results leave with
+// non-temporal stores (they are not re-read by this kernel).
+constexpr int kUnroll = 4;
+
+template <typename T>
+__device__ __forceinline__ void nt_store(Vec16<T>& v, T* p) {
+  v.store(p);
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kThreads)
 unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, ActKind act, float a, float b) {
   constexpr int V = Vec16<T>::N;
   const int64_t nvec = n / V;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
-    Vec16<T> v;
-    v.load(x + i * V);
+  for (int64_t i0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i0 < nvec; i0 += stride * kUnroll) {
+    Vec16<T> v[kUnroll];
 #pragma unroll
-    for (int e = 0; e < V; ++e) v.set(e, apply_act(v.get(e), act, a, b));
-    v.store(y + i * V);
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i < nvec) v[u].load(x + i * V);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[u].set(e, apply_act(v[u].get(e), act, a, b));
+        nt_store(v[u], y + i * V);
+      }
+    }
   }
   // tail
   const int64_t tail0 = nvec * V;
@@ -29,9 +49,12 @@ unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, ActKind act,
     Store<T>::st(y + i, apply_act(Store<T>::ld(x + i), act, a, b));
 }
 
-// y = x * scale[c] + shift[c].  INNER1: channel is the innermost index
-// (channels-last), so a vector spans consecutive channels; otherwise the
-// channel is constant across a vector when inner % V == 0.
+// y = x * scale[c] + shift[c].  inner == 1: channel is the innermost index
+// (channels-last), so a vector spans V consecutive channels; when the grid
+// stride is a multiple of the channel count every thread meets the same V
+// channels in every iteration and keeps their parameters in registers.
+// inner > 1 (row-major N,C,HW): the channel is constant across a vector when
+// inner % V == 0.
 template <typename T>
 __global__ void __launch_bounds__(kThreads)
 channel_affine_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, int64_t inner,
@@ -42,21 +65,41 @@ channel_affine_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, int
   const bool vec_ok = (inner == 1) ? (channels % V == 0) : (inner % V == 0);
   if (vec_ok) {
     const int64_t nvec = n / V;
-    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
-      Vec16<T> v;
-      v.load(x + i * V);
-      const int64_t e0 = i * V;
-      if (inner == 1) {
-        const int c0 = (int)(e0 % channels);
+    const int64_t t0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+    const bool fixed = (inner == 1) && ((stride * V) % channels == 0);
+    float sc[V], sh[V];
+    if (fixed) {
+      const int c0 = (int)((t0 * V) % channels);
 #pragma unroll
-        for (int e = 0; e < V; ++e) v.set(e, v.get(e) * scale[c0 + e] + shift[c0 + e]);
-      } else {
-        const int c = (int)((e0 / inner) % channels);
-        const float s = scale[c], t = shift[c];
+      for (int e = 0; e < V; ++e) { sc[e] = scale[c0 + e]; sh[e] = shift[c0 + e]; }
+    }
+    for (int64_t i0 = t0; i0 < nvec; i0 += stride * kUnroll) {
+      Vec16<T> v[kUnroll];
 #pragma unroll
-        for (int e = 0; e < V; ++e) v.set(e, v.get(e) * s + t);
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = i0 + u * stride;
+        if (i < nvec) v[u].load(x + i * V);
       }
-      v.store(y + i * V);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t i = i0 + u * stride;
+        if (i >= nvec) continue;
+        const int64_t e0 = i * V;
+        if (fixed) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * sc[e] + sh[e]);
+        } else if (inner == 1) {
+          const int c0 = (int)(e0 % channels);
+#pragma unroll
+          for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * scale[c0 + e] + shift[c0 + e]);
+        } else {
+          const int c = (int)((e0 / inner) % channels);
+          const float s = scale[c], t = shift[c];
+#pragma unroll
+          for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * s + t);
+        }
+        nt_store(v[u], y + i * V);
+      }
     }
   } else {
     for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
@@ -96,15 +139,25 @@ __global__ void __launch_bounds__(kThreads)
 binary_flat_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, int64_t n,
                    BinKind op, ActKind act, float aa, float ab) {
   constexpr int V = Vec16<T>::N;
+  constexpr int U = 2;
   const int64_t nvec = n / V;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nvec; i += stride) {
-    Vec16<T> va, vb;
-    va.load(a + i * V);
-    vb.load(b + i * V);
+  for (int64_t i0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i0 < nvec; i0 += stride * U) {
+    Vec16<T> va[U], vb[U];
 #pragma unroll
-    for (int e = 0; e < V; ++e) va.set(e, apply_act(bin_op(va.get(e), vb.get(e), op), act, aa, ab));
-    va.store(y + i * V);
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i < nvec) { va[u].load(a + i * V); vb[u].load(b + i * V); }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = i0 + u * stride;
+      if (i < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) va[u].set(e, apply_act(bin_op(va[u].get(e), vb[u].get(e), op), act, aa, ab));
+        nt_store(va[u], y + i * V);
+      }
+    }
   }
   for (int64_t i = nvec * V + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
     Store<T>::st(y + i, apply_act(bin_op(Store<T>::ld(a + i), Store<T>::ld(b + i), op), act, aa, ab));
@@ -226,24 +279,54 @@ cast_int_kernel(const TS* __restrict__ x, TD* __restrict__ y, int64_t n) {
 
 // q = sat(rne(x / scale) + zp)
 template <typename TS>
+__device__ __forceinline__ int quant_one(float x, float scale, float zf, bool sgn) {
+  const float t = rintf(x / scale) + zf;  // the reference adds the zero point in float before the saturating cast
+  return sgn ? (int)fminf(fmaxf(t, -128.f), 127.f) : (int)fminf(fmaxf(t, 0.f), 255.f);
+}
+
+template <typename TS>
 __global__ void __launch_bounds__(kThreads)
 quantize_kernel(QuantParams p) {
   const TS* x = reinterpret_cast<const TS*>(p.src);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < p.n; i += stride) {
-    const int c = (p.channels > 1) ? (int)((i / p.inner) % p.channels) : 0;
-    const float r = rintf(Store<TS>::ld(x + i) / p.scale[c]);
-    const float zf = p.zp ? (float)p.zp[c] : 0.f;
-    const float t = r + zf;  // the reference adds the zero point in float before the saturating cast
-    if (p.dst_signed) {
-      const float s = fminf(fmaxf(t, -128.f), 127.f);
-      reinterpret_cast<int8_t*>(p.dst)[i] = (int8_t)(int)s;
-    } else {
-      const float s = fminf(fmaxf(t, 0.f), 255.f);
-      const int q = (int)s;
-      if (p.dst_dt == DT_I8) reinterpret_cast<int8_t*>(p.dst)[i] = q_to_stored(q);
-      else reinterpret_cast<uint8_t*>(p.dst)[i] = (uint8_t)q;
+  const int64_t t0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  int64_t done = 0;
+  if (p.channels == 1 && (reinterpret_cast<uintptr_t>(p.src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(p.dst) & 7u) == 0) {
+    // per-tensor parameters: 8 elements per step, one 8-byte store
+    const float sc = p.scale[0], zf = p.zp ? (float)p.zp[0] : 0.f;
+    const int64_t n8 = p.n / 8;
+    for (int64_t i = t0; i < n8; i += stride) {
+      float v[8];
+      if constexpr (sizeof(TS) == 2) {
+        Vec16<TS> t;
+        t.load(x + i * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = t.get(e);
+      } else {
+        Vec16<TS> t0v, t1v;
+        t0v.load(x + i * 8);
+        t1v.load(x + i * 8 + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { v[e] = t0v.get(e); v[e + 4] = t1v.get(e); }
+      }
+      unsigned char o[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int q = quant_one<TS>(v[e], sc, zf, p.dst_signed);
+        o[e] = (unsigned char)((!p.dst_signed && p.dst_dt == DT_I8) ? (q - 128) : q);
+      }
+      uintx2 ov;
+      __builtin_memcpy(&ov, o, 8);
+      *reinterpret_cast<uintx2*>(reinterpret_cast<unsigned char*>(p.dst) + i * 8) = ov;
     }
+    done = n8 * 8;
+  }
+  for (int64_t i = done + t0; i < p.n; i += stride) {
+    const int c = (p.channels > 1) ? (int)((i / p.inner) % p.channels) : 0;
+    const int q = quant_one<TS>(Store<TS>::ld(x + i), p.scale[c], p.zp ? (float)p.zp[c] : 0.f, p.dst_signed);
+    if (p.dst_signed) reinterpret_cast<int8_t*>(p.dst)[i] = (int8_t)q;
+    else if (p.dst_dt == DT_I8) reinterpret_cast<int8_t*>(p.dst)[i] = q_to_stored(q);
+    else reinterpret_cast<uint8_t*>(p.dst)[i] = (uint8_t)q;
   }
 }
 
@@ -253,14 +336,39 @@ __global__ void __launch_bounds__(kThreads)
 dequantize_kernel(QuantParams p) {
   TD* y = reinterpret_cast<TD*>(p.dst);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < p.n; i += stride) {
+  const int64_t t0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  auto level = [&](unsigned char raw) -> float {
+    if (p.src_dt == DT_U8) return (float)raw;
+    if (p.dst_signed) return (float)(int8_t)raw;
+    return (float)q_from_stored((int8_t)raw);
+  };
+  int64_t done = 0;
+  if (p.channels == 1 && (reinterpret_cast<uintptr_t>(p.src) & 7u) == 0 && (reinterpret_cast<uintptr_t>(p.dst) & 15u) == 0) {
+    const float sc = p.scale[0], zf = p.zp ? (float)p.zp[0] : 0.f;
+    const int64_t n8 = p.n / 8;
+    for (int64_t i = t0; i < n8; i += stride) {
+      const uintx2 rv = *reinterpret_cast<const uintx2*>(reinterpret_cast<const unsigned char*>(p.src) + i * 8);
+      unsigned char r[8];
+      __builtin_memcpy(r, &rv, 8);
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (level(r[e]) - zf) * sc;
+      if constexpr (sizeof(TD) == 2) {
+        Vec16<TD> o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o.set(e, v[e]);
+        o.store(y + i * 8);
+      } else {
+        *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(y) + i * 8) = (floatx4){v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(y) + i * 8 + 4) = (floatx4){v[4], v[5], v[6], v[7]};
+      }
+    }
+    done = n8 * 8;
+  }
+  for (int64_t i = done + t0; i < p.n; i += stride) {
     const int c = (p.channels > 1) ? (int)((i / p.inner) % p.channels) : 0;
-    float q;
-    if (p.src_dt == DT_U8) q = (float)reinterpret_cast<const uint8_t*>(p.src)[i];
-    else if (p.dst_signed) q = (float)reinterpret_cast<const int8_t*>(p.src)[i];
-    else q = (float)q_from_stored(reinterpret_cast<const int8_t*>(p.src)[i]);
     const float zf = p.zp ? (float)p.zp[c] : 0.f;
-    Store<TD>::st(y + i, (q - zf) * p.scale[c]);
+    Store<TD>::st(y + i, (level(reinterpret_cast<const unsigned char*>(p.src)[i]) - zf) * p.scale[c]);
   }
 }
 
@@ -416,7 +524,7 @@ hipError_t launch_quantize(const QuantParams& p, hipStream_t stream) {
   if (p.n <= 0) return p.n == 0 ? hipSuccess : hipErrorInvalidValue;
   if (!p.src || !p.dst || !p.scale || p.channels <= 0 || p.inner <= 0) return hipErrorInvalidValue;
   if (p.dst_dt != DT_U8 && p.dst_dt != DT_I8) return hipErrorInvalidValue;
-  const int grid = grid_for(p.n, kThreads * 4);
+  const int grid = grid_for(p.n, kThreads * 16);
   FLOAT_DISPATCH(p.src_dt, hipLaunchKernelGGL(quantize_kernel<T>, dim3(grid), dim3(kThreads), 0, stream, p));
   return hipGetLastError();
 }
@@ -425,7 +533,7 @@ hipError_t launch_dequantize(const QuantParams& p, hipStream_t stream) {
   if (p.n <= 0) return p.n == 0 ? hipSuccess : hipErrorInvalidValue;
   if (!p.src || !p.dst || !p.scale || p.channels <= 0 || p.inner <= 0) return hipErrorInvalidValue;
   if (p.src_dt != DT_U8 && p.src_dt != DT_I8) return hipErrorInvalidValue;
-  const int grid = grid_for(p.n, kThreads * 4);
+  const int grid = grid_for(p.n, kThreads * 16);
   FLOAT_DISPATCH(p.dst_dt, hipLaunchKernelGGL(dequantize_kernel<T>, dim3(grid), dim3(kThreads), 0, stream, p));
   return hipGetLastError();
 }

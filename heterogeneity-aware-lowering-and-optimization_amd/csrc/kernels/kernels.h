@@ -209,6 +209,9 @@ struct StridedCopyParams {
   int64_t x_off = 0, y_off = 0;  // element offsets
 };
 hipError_t launch_strided_copy(const StridedCopyParams& p, hipStream_t stream);
+// Batched 2-D transpose: y[b][c][r] = x[b][r][c], destination row pitch dst_pitch >= rows.
+hipError_t launch_transpose2d(const void* x, void* y, int elem_size, int batch, int rows, int cols,
+                              int dst_pitch, hipStream_t stream);
 // Nearest-neighbour resize, channels-last: src index = floor(dst * in / out).
 hipError_t launch_resize_nearest_nhwc(const void* x, void* y, int elem_size, int N, int H,
                                       int W, int cs, int Ho, int Wo, hipStream_t stream);

@@ -63,32 +63,46 @@ __global__ void __launch_bounds__(kThreads) nchw_to_nhwc_tiled(LayoutParams p, f
   }
 }
 
-// Few channels (cs <= 16): one thread per pixel, channel planes read
-// coalesced across the wavefront, one contiguous pixel written per thread.
-template <typename TS, typename TD>
+// Few channels (cs <= 16): one thread per PX consecutive pixels; each channel
+// plane is read with one PX-wide load per thread (coalesced across the
+// wavefront) and PX contiguous pixels are written per thread.
+template <typename TS, typename TD, int PX>
 __global__ void __launch_bounds__(kThreads) nchw_to_nhwc_smallc(LayoutParams p, float fill) {
   const TS* src = reinterpret_cast<const TS*>(p.src);
   TD* dst = reinterpret_cast<TD*>(p.dst);
-  const int64_t total = (int64_t)p.N * p.HW;
+  const int64_t hwg = p.HW / PX;  // HW % PX == 0 checked by the launcher
+  const int64_t total = (int64_t)p.N * hwg;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t n = i / p.HW, hw = i - n * p.HW;
-    TD out[16];
+    const int64_t n = i / hwg, hw = (i - n * hwg) * PX;
+    float in[16][PX];
 #pragma unroll
     for (int c = 0; c < 16; ++c) {
-      if (c < p.cs) {
-        float v = fill;
-        if (c < p.C) v = ld_as_float<TS>(src + (n * p.C + c) * p.HW + hw, p.scale, p.zp);
-        st_from_float<TD>(&out[c], v, p.scale, p.zp);
+      if (c < p.C) {
+        const TS* s = src + (n * p.C + c) * p.HW + hw;
+        if constexpr (PX == 4 && sizeof(TS) == 4) {
+          const floatx4 t = *reinterpret_cast<const floatx4*>(s);
+          in[c][0] = t.x; in[c][1] = t.y; in[c][2] = t.z; in[c][3] = t.w;
+        } else {
+#pragma unroll
+          for (int k = 0; k < PX; ++k) in[c][k] = ld_as_float<TS>(s + k, p.scale, p.zp);
+        }
       }
     }
-    TD* o = dst + i * p.cs;
-    if ((p.cs * sizeof(TD)) % 16 == 0) {
-      const int nv = p.cs * (int)sizeof(TD) / 16;
-      for (int v = 0; v < nv; ++v)
-        reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
-    } else {
-      for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+#pragma unroll
+    for (int k = 0; k < PX; ++k) {
+      TD out[16];
+#pragma unroll
+      for (int c = 0; c < 16; ++c)
+        if (c < p.cs) st_from_float<TD>(&out[c], c < p.C ? in[c][k] : fill, p.scale, p.zp);
+      TD* o = dst + (n * p.HW + hw + k) * p.cs;
+      if ((p.cs * sizeof(TD)) % 16 == 0) {
+        const int nv = p.cs * (int)sizeof(TD) / 16;
+        for (int v = 0; v < nv; ++v)
+          reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
+      } else {
+        for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+      }
     }
   }
 }
@@ -149,6 +163,35 @@ __global__ void __launch_bounds__(kThreads) strided_copy_kernel(StridedCopyParam
       }
     }
     y[oy] = x[ox];
+  }
+}
+
+// Batched 2-D transpose through an LDS tile: y[b][c][r] = x[b][r][c]; the
+// destination row pitch may exceed `rows` (zero padding is the caller's job).
+template <typename E>
+__global__ void __launch_bounds__(kThreads)
+transpose2d_kernel(const E* __restrict__ x, E* __restrict__ y, int batch, int rows, int cols,
+                   int dst_pitch) {
+  constexpr int TS = 64;
+  __shared__ E tile[TS][TS + 2];
+  const int tr = (rows + TS - 1) / TS, tc = (cols + TS - 1) / TS;
+  const int64_t ntiles = (int64_t)batch * tr * tc;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int ct = (int)(t % tc);
+    const int rt = (int)((t / tc) % tr);
+    const int b = (int)(t / ((int64_t)tc * tr));
+    const int r0 = rt * TS, c0 = ct * TS;
+    const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
+    for (int rr = ty; rr < TS; rr += kThreads / TS) {
+      const int r = r0 + rr, c = c0 + tx;
+      if (r < rows && c < cols) tile[rr][tx] = x[((int64_t)b * rows + r) * cols + c];
+    }
+    __syncthreads();
+    for (int cc = ty; cc < TS; cc += kThreads / TS) {
+      const int c = c0 + cc, r = r0 + tx;
+      if (r < rows && c < cols) y[((int64_t)b * cols + c) * dst_pitch + r] = tile[tx][cc];
+    }
+    __syncthreads();
   }
 }
 
@@ -221,10 +264,18 @@ hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream) {
   // padding lanes hold the real value 0 (its quantised level for 8-bit data)
   const float fill = 0.f;
   if (p.cs <= 16) {
-    const int grid = grid_for((int64_t)p.N * p.HW, kThreads);
-#define K1(TS, TD, ...) hipLaunchKernelGGL((nchw_to_nhwc_smallc<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p, fill)
-    LAYOUT_PAIR_DISPATCH(K1, 0);
+    const bool px4 = p.HW % 4 == 0 && (reinterpret_cast<uintptr_t>(p.src) & 15u) == 0 && p.src_dt == DT_F32;
+    if (px4) {
+      const int grid = grid_for((int64_t)p.N * p.HW / 4, kThreads);
+#define K1(TS, TD, ...) hipLaunchKernelGGL((nchw_to_nhwc_smallc<TS, TD, 4>), dim3(grid), dim3(kThreads), 0, stream, p, fill)
+      LAYOUT_PAIR_DISPATCH(K1, 0);
 #undef K1
+    } else {
+      const int grid = grid_for((int64_t)p.N * p.HW, kThreads);
+#define K1(TS, TD, ...) hipLaunchKernelGGL((nchw_to_nhwc_smallc<TS, TD, 1>), dim3(grid), dim3(kThreads), 0, stream, p, fill)
+      LAYOUT_PAIR_DISPATCH(K1, 0);
+#undef K1
+    }
   } else {
     const int64_t ntiles = (int64_t)p.N * ((p.HW + THW - 1) / THW) * ((p.cs + TC - 1) / TC);
     const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
@@ -259,6 +310,20 @@ hipError_t launch_strided_copy(const StridedCopyParams& p, hipStream_t stream) {
     case 4: hipLaunchKernelGGL(strided_copy_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
     case 8: hipLaunchKernelGGL(strided_copy_kernel<uint64_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
     case 16: hipLaunchKernelGGL(strided_copy_kernel<b16>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_transpose2d(const void* x, void* y, int elem_size, int batch, int rows, int cols,
+                              int dst_pitch, hipStream_t stream) {
+  if (!x || !y || batch <= 0 || rows <= 0 || cols <= 0 || dst_pitch < rows) return hipErrorInvalidValue;
+  const int64_t ntiles = (int64_t)batch * ((rows + 63) / 64) * ((cols + 63) / 64);
+  const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
+  switch (elem_size) {
+    case 1: hipLaunchKernelGGL(transpose2d_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, (const uint8_t*)x, (uint8_t*)y, batch, rows, cols, dst_pitch); break;
+    case 2: hipLaunchKernelGGL(transpose2d_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, (const uint16_t*)x, (uint16_t*)y, batch, rows, cols, dst_pitch); break;
+    case 4: hipLaunchKernelGGL(transpose2d_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, (const uint32_t*)x, (uint32_t*)y, batch, rows, cols, dst_pitch); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();

@@ -9,9 +9,14 @@ namespace {
 
 constexpr int kThreads = 256;
 
+inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 // --------------------------------------------------------------------------
 // Pooling, channels-last.  One thread per (n, ho, wo, channel vector).
-template <typename T, bool IS_MAX>
+// KH, KW > 0: compile-time window; all taps are loaded unconditionally from a
+// clamped (always valid) address so that the loads issue back to back, and
+// out-of-range taps are masked afterwards.  KH == 0: run-time window.
+template <typename T, bool IS_MAX, int KH, int KW>
 __global__ void __launch_bounds__(kThreads) pool2d_vec_kernel(PoolParams p) {
   constexpr int V = Vec16<T>::N;
   const int cv = p.C / V;  // C % V == 0 checked by the launcher
@@ -30,17 +35,40 @@ __global__ void __launch_bounds__(kThreads) pool2d_vec_kernel(PoolParams p) {
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = IS_MAX ? -INFINITY : 0.f;
     int cnt = 0;
-    for (int r = 0; r < p.kh; ++r) {
-      const int hi = h0 + r;
-      if ((unsigned)hi >= (unsigned)p.H) continue;
-      for (int s = 0; s < p.kw; ++s) {
-        const int wi = w0 + s;
-        if ((unsigned)wi >= (unsigned)p.W) continue;
-        Vec16<T> v;
-        v.load(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c);
+    if constexpr (KH > 0) {
+      Vec16<T> v[KH * KW];
+      bool ok[KH * KW];
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc[e] = IS_MAX ? fmaxf(acc[e], v.get(e)) : acc[e] + v.get(e);
-        ++cnt;
+      for (int r = 0; r < KH; ++r)
+#pragma unroll
+        for (int s = 0; s < KW; ++s) {
+          const int hi = h0 + r, wi = w0 + s;
+          ok[r * KW + s] = ((unsigned)hi < (unsigned)p.H) && ((unsigned)wi < (unsigned)p.W);
+          const int hc = hi < 0 ? 0 : (hi >= p.H ? p.H - 1 : hi);
+          const int wc = wi < 0 ? 0 : (wi >= p.W ? p.W - 1 : wi);
+          v[r * KW + s].load(x + (((int64_t)n * p.H + hc) * p.W + wc) * p.cs + c);
+        }
+#pragma unroll
+      for (int k = 0; k < KH * KW; ++k) {
+        if (ok[k]) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) acc[e] = IS_MAX ? fmaxf(acc[e], v[k].get(e)) : acc[e] + v[k].get(e);
+          ++cnt;
+        }
+      }
+    } else {
+      for (int r = 0; r < p.kh; ++r) {
+        const int hi = h0 + r;
+        if ((unsigned)hi >= (unsigned)p.H) continue;
+        for (int s = 0; s < p.kw; ++s) {
+          const int wi = w0 + s;
+          if ((unsigned)wi >= (unsigned)p.W) continue;
+          Vec16<T> v;
+          v.load(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c);
+#pragma unroll
+          for (int e = 0; e < V; ++e) acc[e] = IS_MAX ? fmaxf(acc[e], v.get(e)) : acc[e] + v.get(e);
+          ++cnt;
+        }
       }
     }
     Vec16<T> o;
@@ -52,7 +80,7 @@ __global__ void __launch_bounds__(kThreads) pool2d_vec_kernel(PoolParams p) {
 #pragma unroll
       for (int e = 0; e < V; ++e) o.set(e, acc[e] / div);
     }
-    o.store(y + (((int64_t)n * p.Ho + ho) * p.Wo + wo) * p.ycs + c);
+    __builtin_nontemporal_store(o.raw, reinterpret_cast<uintx4*>(y + (((int64_t)n * p.Ho + ho) * p.Wo + wo) * p.ycs + c));
   }
 }
 
@@ -185,6 +213,46 @@ reduce_cols_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, 
     Store<TO>::st(y + i, acc);
   }
 }
+// inner % V == 0: one thread per (outer, 16-byte group of inner positions); every
+// step over `len` is a coalesced row of vectors.
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(kThreads)
+reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int64_t len,
+                       int64_t inner, ReduceKind kind) {
+  constexpr int V = Vec16<TI>::N;
+  const int64_t iv = inner / V;
+  const int64_t total = outer * iv;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t o = i / iv, in = (i - o * iv) * V;
+    const TI* col = x + o * len * inner + in;
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = kind == RED_MAX ? -INFINITY : 0.f;
+    int64_t k = 0;
+    for (; k + 4 <= len; k += 4) {
+      Vec16<TI> v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u].load(col + (k + u) * inner);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] = kind == RED_MAX ? fmaxf(acc[e], v[u].get(e)) : acc[e] + v[u].get(e);
+    }
+    for (; k < len; ++k) {
+      Vec16<TI> v;
+      v.load(col + k * inner);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = kind == RED_MAX ? fmaxf(acc[e], v.get(e)) : acc[e] + v.get(e);
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      float r = acc[e];
+      if (kind == RED_MEAN) r /= (float)len;
+      Store<TO>::st(y + o * inner + in + e, r);
+    }
+  }
+}
 // Quantised mean over the middle axis: y = ((sum - len*zp) / len) * scale (fp32).
 __global__ void __launch_bounds__(kThreads)
 reduce_cols_q8_kernel(const int8_t* __restrict__ x, float* __restrict__ y, int64_t outer,
@@ -273,6 +341,162 @@ softmax_wave_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, 
     }
   }
 }
+// Rows of 16-byte vectors (len % V == 0, row start 16-byte aligned): LPR lanes
+// share one row, each lane holds PER vectors; several short rows fit in one
+// wavefront.  Reductions are xor-shuffles inside the LPR-lane group.
+template <int LPR>
+__device__ __forceinline__ float group_max(float v) {
+#pragma unroll
+  for (int o = LPR / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+template <int LPR>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = LPR / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <typename TO, int V>
+__device__ __forceinline__ void store_row_vec(TO* dst, const float* v) {
+  if constexpr (sizeof(TO) * V == 16) {
+    Vec16<TO> o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) o.set(e, v[e]);
+    o.store(dst);
+  } else if constexpr (sizeof(TO) == 4 && V % 4 == 0) {
+#pragma unroll
+    for (int e = 0; e < V; e += 4)
+      *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(dst) + e) = (floatx4){v[e], v[e + 1], v[e + 2], v[e + 3]};
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) Store<TO>::st(dst + e, v[e]);
+  }
+}
+
+template <typename TI, typename TO, int LPR, int PER>
+__global__ void __launch_bounds__(kThreads)
+softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, int len, bool logsm) {
+  constexpr int V = Vec16<TI>::N;
+  constexpr int RPW = 64 / LPR;
+  const int lane = threadIdx.x & 63;
+  const int sub = lane % LPR;
+  const int nv = len / V;
+  const int64_t wave = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) >> 6;
+  const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+  for (int64_t r0 = wave * RPW; r0 < rows; r0 += nwaves * RPW) {
+    const int64_t r = r0 + lane / LPR;
+    const bool row_ok = r < rows;
+    const TI* row = x + (row_ok ? r : 0) * (int64_t)len;
+    float v[PER][V];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int vi = sub + k * LPR;
+      if (vi < nv && row_ok) {
+        Vec16<TI> t;
+        t.load(row + vi * V);
+#pragma unroll
+        for (int e = 0; e < V; ++e) { v[k][e] = t.get(e); mx = fmaxf(mx, v[k][e]); }
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[k][e] = -INFINITY;
+      }
+    }
+    mx = group_max<LPR>(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float ex = expf(v[k][e] - mx);   // exp(-inf) = 0 for the padding slots
+        sum += ex;
+        if (!logsm) v[k][e] = ex;
+      }
+    sum = group_sum<LPR>(sum);
+    const float lsum = logf(sum), inv = 1.0f / sum;
+    if (row_ok) {
+      TO* out = y + r * (int64_t)len;
+#pragma unroll
+      for (int k = 0; k < PER; ++k) {
+        const int vi = sub + k * LPR;
+        if (vi < nv) {
+          float o[V];
+#pragma unroll
+          for (int e = 0; e < V; ++e) o[e] = logsm ? (v[k][e] - mx - lsum) : v[k][e] * inv;
+          store_row_vec<TO, V>(out + vi * V, o);
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int LPR, int PER>
+__global__ void __launch_bounds__(kThreads)
+layernorm_vec_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int len,
+                     const float* __restrict__ gamma, const float* __restrict__ beta, float eps) {
+  constexpr int V = Vec16<T>::N;
+  constexpr int RPW = 64 / LPR;
+  const int lane = threadIdx.x & 63;
+  const int sub = lane % LPR;
+  const int nv = len / V;
+  const int64_t wave = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) >> 6;
+  const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+  for (int64_t r0 = wave * RPW; r0 < rows; r0 += nwaves * RPW) {
+    const int64_t r = r0 + lane / LPR;
+    const bool row_ok = r < rows;
+    const T* row = x + (row_ok ? r : 0) * (int64_t)len;
+    float v[PER][V];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int vi = sub + k * LPR;
+      if (vi < nv && row_ok) {
+        Vec16<T> t;
+        t.load(row + vi * V);
+#pragma unroll
+        for (int e = 0; e < V; ++e) { v[k][e] = t.get(e); s += v[k][e]; }
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[k][e] = 0.f;
+      }
+    }
+    const float mean = group_sum<LPR>(s) / (float)len;
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int vi = sub + k * LPR;
+      if (vi < nv) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) { const float d = v[k][e] - mean; q += d * d; }
+      }
+    }
+    const float var = group_sum<LPR>(q) / (float)len;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    if (row_ok) {
+      T* out = y + r * (int64_t)len;
+#pragma unroll
+      for (int k = 0; k < PER; ++k) {
+        const int vi = sub + k * LPR;
+        if (vi < nv) {
+          float o[V], g[V], b[V];
+          // gamma / beta are fp32 vectors, 16-byte aligned (V is a multiple of 4)
+#pragma unroll
+          for (int e = 0; e < V; e += 4) {
+            const floatx4 gv = gamma ? *reinterpret_cast<const floatx4*>(gamma + vi * V + e) : (floatx4){1.f, 1.f, 1.f, 1.f};
+            const floatx4 bv = beta ? *reinterpret_cast<const floatx4*>(beta + vi * V + e) : (floatx4){0.f, 0.f, 0.f, 0.f};
+            g[e] = gv.x; g[e + 1] = gv.y; g[e + 2] = gv.z; g[e + 3] = gv.w;
+            b[e] = bv.x; b[e + 1] = bv.y; b[e + 2] = bv.z; b[e + 3] = bv.w;
+          }
+#pragma unroll
+          for (int e = 0; e < V; ++e) o[e] = (v[k][e] - mean) * rstd * g[e] + b[e];
+          store_row_vec<T, V>(out + vi * V, o);
+        }
+      }
+    }
+  }
+}
+
 // Generic: strided axis or very long rows; three passes over the column.
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(kThreads)
@@ -336,8 +560,6 @@ layernorm_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int l
   }
 }
 
-bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
 }  // namespace
 
 #define FLOAT_DISPATCH(dt, EXPR)                         \
@@ -368,8 +590,13 @@ hipError_t launch_pool2d(const PoolParams& p, hipStream_t stream) {
   if (vec) {
     const int64_t total = (int64_t)p.N * p.Ho * p.Wo * (p.C / V);
     const int grid = grid_for(total, kThreads);
-    if (p.is_max) { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((pool2d_vec_kernel<T, true>), dim3(grid), dim3(kThreads), 0, stream, p)); }
-    else { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((pool2d_vec_kernel<T, false>), dim3(grid), dim3(kThreads), 0, stream, p)); }
+#define POOL_LAUNCH(MAX_, KH_, KW_) \
+  FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((pool2d_vec_kernel<T, MAX_, KH_, KW_>), dim3(grid), dim3(kThreads), 0, stream, p))
+    if (p.kh == 3 && p.kw == 3) { if (p.is_max) { POOL_LAUNCH(true, 3, 3); } else { POOL_LAUNCH(false, 3, 3); } }
+    else if (p.kh == 2 && p.kw == 2) { if (p.is_max) { POOL_LAUNCH(true, 2, 2); } else { POOL_LAUNCH(false, 2, 2); } }
+    else if (p.kh == 1 && p.kw == 1) { if (p.is_max) { POOL_LAUNCH(true, 1, 1); } else { POOL_LAUNCH(false, 1, 1); } }
+    else { if (p.is_max) { POOL_LAUNCH(true, 0, 0); } else { POOL_LAUNCH(false, 0, 0); } }
+#undef POOL_LAUNCH
   } else {
     const int64_t total = (int64_t)p.N * p.Ho * p.Wo * p.C;
     const int grid = grid_for(total, kThreads);
@@ -396,6 +623,10 @@ static hipError_t reduce_out(const void* x, void* y, DType out_dt, int64_t outer
       const int grid = grid_for(outer * 64, kThreads);
       hipLaunchKernelGGL((reduce_rows_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
                          (const TI*)x, (TO*)y, outer, len, kind);
+    } else if (inner % (16 / (int)sizeof(TI)) == 0 && al16(x)) {
+      const int grid = grid_for(outer * (inner / (16 / (int)sizeof(TI))), kThreads);
+      hipLaunchKernelGGL((reduce_cols_vec_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
+                         (const TI*)x, (TO*)y, outer, len, inner, kind);
     } else {
       const int grid = grid_for(outer * inner, kThreads);
       hipLaunchKernelGGL((reduce_cols_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
@@ -423,6 +654,24 @@ hipError_t launch_reduce(const void* x, void* y, DType in_dt, DType out_dt, int6
 template <typename TI, typename TO>
 static hipError_t softmax_typed(const void* x, void* y, int64_t outer, int64_t len, int64_t inner,
                                 bool logsm, hipStream_t stream) {
+  constexpr int V = 16 / (int)sizeof(TI);
+  if (inner == 1 && len % V == 0 && len / V <= 256 && al16(x) && (sizeof(TO) != sizeof(TI) || al16(y))) {
+    const int nv = (int)(len / V);
+    int lpr = 1;
+    while (lpr < nv && lpr < 64) lpr <<= 1;
+    const int per = (nv + lpr - 1) / lpr;
+    const int rpw = 64 / lpr;
+    const int grid = grid_for((outer + rpw - 1) / rpw * 64, kThreads);
+#define SMV(LPR_, PER_) hipLaunchKernelGGL((softmax_vec_kernel<TI, TO, LPR_, PER_>), dim3(grid), dim3(kThreads), 0, stream, (const TI*)x, (TO*)y, outer, (int)len, logsm)
+    if (lpr <= 8) SMV(8, 1);
+    else if (lpr == 16) SMV(16, 1);
+    else if (lpr == 32) SMV(32, 1);
+    else if (per == 1) SMV(64, 1);
+    else if (per == 2) SMV(64, 2);
+    else SMV(64, 4);
+#undef SMV
+    return hipGetLastError();
+  }
   if (inner == 1 && len <= 64 * 4) {
     const int grid = grid_for(outer * 64, kThreads);
     if (len <= 64) hipLaunchKernelGGL((softmax_wave_kernel<TI, TO, 1>), dim3(grid), dim3(kThreads), 0, stream, (const TI*)x, (TO*)y, outer, (int)len, logsm);
@@ -458,6 +707,26 @@ hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int6
                             const float* gamma, const float* beta, float eps, hipStream_t stream) {
   if (!x || !y || rows <= 0 || len <= 0) return hipErrorInvalidValue;
   if (len > 256 * 16) return hipErrorInvalidValue;
+  {
+    const int es = dtype_size(dt);
+    const int V = es ? 16 / es : 1;
+    if (es && len % V == 0 && len / V <= 256 && al16(x) && al16(y) && (!gamma || al16(gamma)) && (!beta || al16(beta))) {
+      const int nv = (int)(len / V);
+      int lpr = 1;
+      while (lpr < nv && lpr < 64) lpr <<= 1;
+      const int per = (nv + lpr - 1) / lpr;
+      const int rpw = 64 / lpr;
+      const int grid = grid_for((rows + rpw - 1) / rpw * 64, kThreads);
+#define LNV(LPR_, PER_) FLOAT_DISPATCH(dt, hipLaunchKernelGGL((layernorm_vec_kernel<T, LPR_, PER_>), dim3(grid), dim3(kThreads), 0, stream, (const T*)x, (T*)y, rows, (int)len, gamma, beta, eps))
+      if (lpr <= 16) { LNV(16, 1); }
+      else if (lpr == 32) { LNV(32, 1); }
+      else if (per == 1) { LNV(64, 1); }
+      else if (per == 2) { LNV(64, 2); }
+      else { LNV(64, 4); }
+#undef LNV
+      return hipGetLastError();
+    }
+  }
   const int grid = (int)(rows < 16384 ? rows : 16384);
   if (len <= 256 * 4) {
     FLOAT_DISPATCH(dt, hipLaunchKernelGGL((layernorm_kernel<T, 256, 4>), dim3(grid), dim3(256), 0, stream,

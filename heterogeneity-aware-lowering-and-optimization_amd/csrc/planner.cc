@@ -463,7 +463,7 @@ class Planner {
                    int* w_rs_out, const std::vector<float>* wq_scale);
   void finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty, const Epilogue& ep,
                     int64_t Kout_total);
-  int strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp);
+  int strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp_in);
   void assign_arena();
   void parse_quant_table();
 };
@@ -844,7 +844,24 @@ int Planner::pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og
   return dst;
 }
 
-int Planner::strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp) {
+int Planner::strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp_in) {
+  StridedCopyParams cp = cp_in;
+  // Move 16-byte elements when the innermost run is contiguous on both sides and
+  // every stride / offset keeps 16-byte alignment (tensor bases are 256-byte aligned).
+  {
+    const int r = cp.rank;
+    const int w = cp.elem_size > 0 && cp.elem_size < 16 ? 16 / cp.elem_size : 0;
+    bool ok = w > 1 && r >= 1 && cp.sx[r - 1] == 1 && cp.sy[r - 1] == 1 && cp.dims[r - 1] % w == 0 &&
+              cp.x_off % w == 0 && cp.y_off % w == 0;
+    for (int d = 0; ok && d < r - 1; ++d) ok = cp.sx[d] % w == 0 && cp.sy[d] % w == 0;
+    if (ok) {
+      cp.elem_size = 16;
+      cp.dims[r - 1] /= w;
+      for (int d = 0; d < r - 1; ++d) { cp.sx[d] /= w; cp.sy[d] /= w; }
+      cp.x_off /= w;
+      cp.y_off /= w;
+    }
+  }
   const Ref a = ref(src), b = ref(dst);
   emit(name, {src}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
     StridedCopyParams p = cp; p.x = a(e); p.y = b(e);
@@ -1196,13 +1213,22 @@ void Planner::lower_gemm(int ni) {
         const int64_t words = (int64_t)(T(t2).bytes / 4);
         emit("gemm.zero:" + outv->name, {}, {t2}, [=](const ExecEnv& e, hipStream_t st) { return launch_fill_i32((int32_t*)b(e), words, 0, st); });
       }
-      StridedCopyParams cp;
-      cp.elem_size = dtype_size(dt);
-      cp.rank = 3;
-      cp.dims[0] = blead; cp.dims[1] = Nn; cp.dims[2] = K;
-      cp.sy[0] = Nn * Kp; cp.sy[1] = Kp; cp.sy[2] = 1;
-      cp.sx[0] = K * Nn; cp.sx[1] = tB ? K : 1; cp.sx[2] = tB ? 1 : Nn;
-      strided_copy_step("gemm.b:" + outv->name, tb, t2, cp);
+      if (!tB) {
+        // [blead][K][N] -> [blead][N][Kp]: LDS-tiled transpose
+        const Ref a2 = ref(tb), b2 = ref(t2);
+        const int es2 = dtype_size(dt), bl = (int)blead, Ki = (int)K, Ni = (int)Nn, Kpi = Kp;
+        emit("gemm.b:" + outv->name, {tb}, {t2}, [=](const ExecEnv& e, hipStream_t st) {
+          return launch_transpose2d(a2(e), b2(e), es2, bl, Ki, Ni, Kpi, st);
+        });
+      } else {
+        StridedCopyParams cp;
+        cp.elem_size = dtype_size(dt);
+        cp.rank = 3;
+        cp.dims[0] = blead; cp.dims[1] = Nn; cp.dims[2] = K;
+        cp.sy[0] = Nn * Kp; cp.sy[1] = Kp; cp.sy[2] = 1;
+        cp.sx[0] = K * Nn; cp.sx[1] = K; cp.sx[2] = 1;
+        strided_copy_step("gemm.b:" + outv->name, tb, t2, cp);
+      }
       tb = t2;
     }
     tw = tb;
