@@ -17,6 +17,10 @@
 // the exact k permutation inside one MFMA is irrelevant to the result.
 #include "device_utils.h"
 
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+
 namespace ohip {
 
 template <typename T> struct Mma;
@@ -200,6 +204,146 @@ template <typename T> struct EpiTraits<EpiFloat<T>> { using TOut = T; static con
 template <int M> struct EpiTraits<EpiQuant<M>> { using TOut = typename QuantOut<M>::T; static constexpr bool quant = true; };
 
 // ---------------------------------------------------------------------------
+// Epilogue shared by the kernels below: each wavefront parks one 32-pixel slice
+// of its accumulators in LDS (pixel-major, fp32 / int32), then every lane picks
+// eight consecutive output channels of one pixel, so that global stores and
+// residual loads are 16-byte vectors and consecutive lanes cover contiguous
+// memory.  `smem` is the K loop's buffer; it is reused once every wavefront of
+// the workgroup has left the loop.
+template <typename TIn, typename Epi, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int epi_vec,
+                                               typename Mma<TIn>::Acc (&acc)[WM / 32][WN / 32],
+                                               unsigned char* smem, const int tile_m, const int tile_n,
+                                               const int z, const int M, const int wave, const int lane) {
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int EPI_PITCH = WN + 4;  // 4-byte words per staged pixel row
+  using AccE = typename Epi::AccE;
+  using TOut = typename EpiTraits<Epi>::TOut;
+  const int wm = wave % (BM / WM), wn = wave / (BM / WM);
+  const int l32 = lane & 31, lg = lane >> 5;
+
+  TOut* ybase = reinterpret_cast<TOut*>(p.y) + (int64_t)z * p.y_bs;
+  const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
+  const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
+
+  AccE* stage = reinterpret_cast<AccE*>(smem) + wave * (32 * EPI_PITCH);
+  constexpr int LPP = WN / 8;    // lanes per pixel row in the read-back
+  constexpr int PPP = 64 / LPP;  // pixels per read-back pass
+  const int rp = lane / LPP;     // pixel within a pass
+  const int c8 = (lane % LPP) * 8;
+  const int n = tile_n * BN + wn * WN + c8;
+  int nvalid = p.Kout - n;
+  nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
+  const bool vec = (epi_vec & 1) && nvalid == 8;
+
+  // lane-constant epilogue operands: the lane's eight channels are the same in every pass
+  AccE b8[8];
+  float m8[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { b8[e] = 0; m8[e] = 0.f; }
+  if (nvalid > 0) {
+    if (bias != nullptr) {
+      if (vec) {
+        const intx4 t0 = *reinterpret_cast<const intx4*>(bias + n);
+        const intx4 t1 = *reinterpret_cast<const intx4*>(bias + n + 4);
+        __builtin_memcpy(&b8[0], &t0, 16);
+        __builtin_memcpy(&b8[4], &t1, 16);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (e < nvalid) b8[e] = bias[n + e];
+      }
+    }
+    if constexpr (EpiTraits<Epi>::quant) {
+      if (p.qmul != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (e < nvalid) m8[e] = p.qmul[n + e];
+      }
+    }
+  }
+
+  // Residual vectors are requested one 32-pixel slice ahead of their use, so
+  // that their latency overlaps with the staging of the previous slice.
+  constexpr int NPASS = 32 / PPP;
+  using RVec = typename Epi::RVec;
+  const bool have_rpre = Epi::kPrefetchResidual && vec && rbase != nullptr;
+  auto rfetch = [&](const int i, RVec (&dst)[NPASS]) {
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int m = tile_m * BM + wm * WM + i * 32 + ps * PPP + rp;
+      const int mc = m < M ? m : M - 1;
+      dst[ps] = *reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n);
+    }
+  };
+  RVec rcur[NPASS], rnxt[NPASS];
+#pragma unroll
+  for (int ps = 0; ps < NPASS; ++ps) { rcur[ps] = RVec{}; rnxt[ps] = RVec{}; }
+  if constexpr (Epi::kPrefetchResidual) {
+    if (have_rpre) rfetch(0, rcur);
+  }
+
+  __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    // park: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        AccE* dst = stage + l32 * EPI_PITCH + j * 32 + q * 8 + lg * 4;
+        if constexpr (sizeof(AccE) == 4 && !EpiTraits<Epi>::quant) {
+          *reinterpret_cast<floatx4*>(dst) =
+              (floatx4){acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+        } else {
+          *reinterpret_cast<intx4*>(dst) =
+              (intx4){(int)acc[i][j][q * 4 + 0], (int)acc[i][j][q * 4 + 1], (int)acc[i][j][q * 4 + 2], (int)acc[i][j][q * 4 + 3]};
+        }
+      }
+    }
+    // Each wavefront only touches its own staging slice and its LDS operations
+    // complete in issue order, so a wavefront-scope fence (no workgroup barrier)
+    // orders the parking writes before the read-back.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if constexpr (Epi::kPrefetchResidual && TM > 1) {
+      if (have_rpre && i + 1 < TM) rfetch(i + 1, rnxt);
+    }
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) {
+      const int pix = ps * PPP + rp;
+      const int m = tile_m * BM + wm * WM + i * 32 + pix;
+      AccE a8[8];
+      const AccE* src = stage + pix * EPI_PITCH + c8;
+      if constexpr (!EpiTraits<Epi>::quant) {
+        const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
+        const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
+        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
+        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+      } else {
+        const intx4 v0 = *reinterpret_cast<const intx4*>(src);
+        const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
+        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
+        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+      }
+      if (m < M && nvalid > 0) {
+        TOut* yrow = ybase + (int64_t)m * p.ycs + n;
+        const TOut* rrow = rbase ? rbase + (int64_t)m * p.rcs + n : nullptr;
+        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rcur[ps]);
+      }
+    }
+#pragma unroll
+    for (int ps = 0; ps < NPASS; ++ps) rcur[ps] = rnxt[ps];
+    if (i + 1 < TM) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Main kernel.
 //
 // K pipeline: per stage the workgroup holds 128 bytes of K per row for both
@@ -373,119 +517,248 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
     }
   }
 
-  // ---- epilogue ----
-  TOut* ybase = reinterpret_cast<TOut*>(p.y) + (int64_t)z * p.y_bs;
-  const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
-  const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
+  igemm_epilogue<TIn, Epi, BM, BN, WM, WN>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
+}
 
-  AccE* stage = reinterpret_cast<AccE*>(smem) + wave * (32 * EPI_PITCH);
-  constexpr int LPP = WN / 8;    // lanes per pixel row in the read-back
-  constexpr int PPP = 64 / LPP;  // pixels per read-back pass
-  const int rp = lane / LPP;     // pixel within a pass
-  const int c8 = (lane % LPP) * 8;
-  const int n = tile_n * BN + wn * WN + c8;
-  int nvalid = p.Kout - n;
-  nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
-  const bool vec = epi_vec && nvalid == 8;
+// ---------------------------------------------------------------------------
+// Variant for constant weights: a deeper pipeline with less LDS traffic.
+//
+// Measured on this part, LDS stores from registers run at a quarter of the LDS
+// load rate, and one K stage of register prefetch does not cover the latency of
+// the gathered pixel loads, so a kernel that stages both operands through
+// registers into LDS is bound by exactly those two things.  Here
+//   - only the 128-pixel tile goes through LDS, written by direct-to-LDS global
+//     loads (no registers, no LDS store instructions) into a ring of three
+//     buffers, two K stages ahead of its use, one barrier per stage;
+//   - the four wavefronts split the 128 output channels; each reads its
+//     32-channel weight fragments straight from global memory into registers,
+//     also two stages ahead.  The fragments were stored at plan time in MFMA
+//     operand order (one contiguous KiB per 32-channel x 32-byte fragment,
+//     lane-major), so every weight byte is fetched by exactly one wavefront
+//     with fully coalesced 16-byte loads.
+//
+// LDS layout of a pixel buffer: row r (128 bytes = eight 16-byte chunks) at
+// r*128, chunk c stored in slot c ^ ((r >> 1) & 7).  A direct-to-LDS load
+// writes lane l of a wavefront at base + 16*l, so lane l fetches, for row
+// base_row + l/8, the chunk that belongs in slot l%8; the fragment reads of 16
+// consecutive rows then fall into 16 distinct 16-byte bank groups.
+//
+// Vector-memory operations retire in issue order, so every load stream has the
+// same depth (two stages) and every load is issued unconditionally (clamped to
+// valid addresses at the ends): the number of operations in flight at each
+// wait is a compile-time constant.  Padding taps and out-of-range rows fetch a
+// 16-byte fill vector stored behind the weight fragments.
+template <typename TIn, typename Epi>
+__global__ void __launch_bounds__(256, 3)  // three wavefronts per SIMD: at most 168 registers
+igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
+  constexpr int BM = 128, BN = 128, WM = 128, WN = 32, NW = 4;
+  constexpr int ES = sizeof(TIn);
+  constexpr int BKB = 128, BK = BKB / ES;
+  constexpr int VEC = 16 / ES, A_IT = 4;
+  constexpr int TM = WM / 32;
+  constexpr int BUF_BYTES = BM * BKB;  // 16 KiB
+  constexpr int NBUF = 3;
+  constexpr int EPI_BYTES = NW * 32 * (WN + 4) * 4;
+  static_assert(NBUF * BUF_BYTES >= EPI_BYTES, "staging area must fit in the pixel buffers");
+  using Acc = typename Mma<TIn>::Acc;
+  // s_waitcnt immediates (vmcnt only; expcnt / lgkmcnt left at their maxima)
+  constexpr int kWaitVm0 = 0x0f70, kWaitVm12 = 0x0f7c;
 
-  // lane-constant epilogue operands: the lane's eight channels are the same in every pass
-  AccE b8[8];
-  float m8[8];
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[NBUF * BUF_BYTES];
+
+  const int tid = threadIdx.x;
+  const int M = p.N * p.Ho * p.Wo;
+  const int tiles_n = (p.Kout + BN - 1) / BN;
+  int bid = blockIdx.x;
+  {
+    const int per = gridDim.x >> 3;
+    if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int tile_n = bid % tiles_n;
+  const int tile_m = bid / tiles_n;
+  const int z = blockIdx.z;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, lg = lane >> 5;
+
+  const TIn* x = reinterpret_cast<const TIn*>(p.x) + (int64_t)z * p.x_bs;
+  // fragment q of this wavefront's 32 channels: wf[q * 64]
+  int wtile = tile_n * (BN / 32) + wave;
+  wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;  // surplus wavefronts compute channels that are never stored
+  const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag) +
+                     ((int64_t)z * p.wf_tiles + wtile) * p.wf_chunks * 64 + lane;
+  const TIn* fill_ptr = reinterpret_cast<const TIn*>(reinterpret_cast<const unsigned char*>(p.w_frag) +
+                                                     (int64_t)p.batch * p.wf_tiles * p.wf_chunks * 1024);
+
+  // ---- gather state: this thread feeds rows row0 + 32*i, slot lane%8 ----
+  const int row0 = tid >> 3;
+  const int kv = (lane & 7) ^ ((row0 >> 1) & 7);  // the chunk that belongs in this lane's slot
+  const TIn* a_ptr[A_IT];
+  int a_hi0[A_IT], a_wi0[A_IT];
+  const int HoWo = p.Ho * p.Wo;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) { b8[e] = 0; m8[e] = 0.f; }
-  if (nvalid > 0) {
-    if (bias != nullptr) {
-      if (vec) {
-        const intx4 t0 = *reinterpret_cast<const intx4*>(bias + n);
-        const intx4 t1 = *reinterpret_cast<const intx4*>(bias + n + 4);
-        __builtin_memcpy(&b8[0], &t0, 16);
-        __builtin_memcpy(&b8[4], &t1, 16);
-      } else {
+  for (int i = 0; i < A_IT; ++i) {
+    const int m = tile_m * BM + row0 + i * 32;
+    const bool ok = m < M;
+    const int mm = ok ? m : 0;
+    const int n_img = mm / HoWo;
+    const int rem = mm - n_img * HoWo;
+    const int ho = rem / p.Wo;
+    const int wo = rem - ho * p.Wo;
+    a_hi0[i] = ok ? ho * p.sh - p.ph : -(1 << 28);  // out-of-range rows never pass the bounds test
+    a_wi0[i] = wo * p.sw - p.pw;
+    a_ptr[i] = x + (int64_t)n_img * p.H * p.W * p.xcs;
+  }
+  int kc = kv * VEC, kr = 0, ks = 0;
+  while (kc >= p.C) {
+    kc -= p.C;
+    if (++ks == p.S) { ks = 0; ++kr; }
+  }
+  using lds_ptr = __attribute__((address_space(3))) void*;
+  // Requests the next K stage of the pixel tile into buffer `buf`.
+  auto dma = [&](const int buf) {
+    const int hoff = kr * p.dh, woff = ks * p.dw;
+    unsigned char* dst = smem + buf * BUF_BYTES + wave * 1024;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) b8[e] = bias[n + e];
-      }
+    for (int i = 0; i < A_IT; ++i) {
+      const int hi = a_hi0[i] + hoff, wi = a_wi0[i] + woff;
+      const bool ok = (kr < p.R) && ((unsigned)hi < (unsigned)p.H) && ((unsigned)wi < (unsigned)p.W);
+      const TIn* src = ok ? a_ptr[i] + ((hi * p.W + wi) * p.xcs + kc) : fill_ptr;
+#if defined(__HIP_DEVICE_COMPILE__)  // (the builtin is unknown to the host pass, which only needs the launch stub)
+      __builtin_amdgcn_global_load_lds(src, (lds_ptr)(dst + i * 4096), 16, 0, 0);
+#else
+      (void)src; (void)dst;
+#endif
     }
-    if constexpr (EpiTraits<Epi>::quant) {
-      if (p.qmul != nullptr) {
+    kc += BK;
+    while (kc >= p.C) {
+      kc -= p.C;
+      if (++ks == p.S) { ks = 0; ++kr; }
+    }
+  };
+
+  Acc acc[TM][1];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) m8[e] = p.qmul[n + e];
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][0][e] = 0;
+
+  const int nkt = p.wf_chunks / 4;
+  // fragment read offsets: row l32 (+32*i), chunk 2*kk + lg, swizzled
+  const int sw = (l32 >> 1) & 7;
+  const int rd_base = l32 * 128 + ((lg ^ (sw & 1)) * 16);
+  const int rd_t = sw >> 1;
+
+  // Weight fragment requests and their waits are issued by hand: next to the
+  // direct-to-LDS loads the compiler would otherwise treat the vector-memory
+  // counter as unordered and wait for everything in flight at each use.
+  // wload: dst <- ptr[off bytes]; wwait<n>: dst is valid once at most n younger
+  // vector-memory operations are still in flight.
+  // (The host pass only needs the kernel's launch stub; it cannot parse the
+  // vector-register constraints.)
+#if defined(__HIP_DEVICE_COMPILE__)
+#define IGEMM_WLOAD(dst, ptr, OFF) \
+  asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "=v"(dst) : "v"(ptr) : "memory")
+#define IGEMM_WWAIT15(dst) asm volatile("s_waitcnt vmcnt(15)" : "+v"(dst) : : "memory")
+#else
+#define IGEMM_WLOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
+#define IGEMM_WWAIT15(dst) (void)(dst)
+#endif
+  uintx4 w0[4], w1[4];
+  {
+    const uintx4* ws = wf + (int64_t)(nkt > 1 ? 1 : 0) * 4 * 64;
+    IGEMM_WLOAD(w0[0], wf, 0);
+    IGEMM_WLOAD(w0[1], wf, 1024);
+    IGEMM_WLOAD(w0[2], wf, 2048);
+    IGEMM_WLOAD(w0[3], wf, 3072);
+    IGEMM_WLOAD(w1[0], ws, 0);
+    IGEMM_WLOAD(w1[1], ws, 1024);
+    IGEMM_WLOAD(w1[2], ws, 2048);
+    IGEMM_WLOAD(w1[3], ws, 3072);
+  }
+  dma(0);
+  dma(1);
+
+  // One K stage.  wc = this stage's weight fragments; each is re-requested for
+  // stage kt+2 right after its use.
+  auto stage = [&](const int kt, const int buf, uintx4 (&wc)[4]) {
+    // the pixel vectors of this stage have landed (mine), and everyone's have
+    // (a bare barrier: the fence of __syncthreads would also wait for the
+    // requests of the stages still in flight)
+    if (kt < 2) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+    else __builtin_amdgcn_s_waitcnt(kWaitVm12);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // every wavefront has also left stage kt-1, whose buffer is (kt+2) % 3
+    dma(buf == 0 ? 2 : buf - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    const unsigned char* ab = smem + buf * BUF_BYTES + rd_base;
+    const int ktn = kt + 2 < nkt ? kt + 2 : nkt - 1;
+    const uintx4* wnext = wf + (int64_t)ktn * 4 * 64;
+    uintx4 fa[2][TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const uintx4*>(ab + ((0 ^ rd_t) * 32) + i * 4096);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      if (kk < 3) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa[(kk + 1) & 1][i] = *reinterpret_cast<const uintx4*>(ab + (((kk + 1) ^ rd_t) * 32) + i * 4096);
       }
+      __builtin_amdgcn_sched_barrier(0);
+      // In flight behind wc[kk] (requested two stages ago at this step): 3-kk
+      // fragments of that stage, 8 operations of the stage between, the 4
+      // pixel requests above and kk fragments of this stage: always 15.
+      IGEMM_WWAIT15(wc[kk]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) acc[i][0] = Mma<TIn>::run(wc[kk], fa[kk & 1][i], acc[i][0]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk == 0) IGEMM_WLOAD(wc[0], wnext, 0);
+      else if (kk == 1) IGEMM_WLOAD(wc[1], wnext, 1024);
+      else if (kk == 2) IGEMM_WLOAD(wc[2], wnext, 2048);
+      else IGEMM_WLOAD(wc[3], wnext, 3072);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  int buf = 0;
+  for (int kt = 0; kt < nkt; kt += 2) {
+    stage(kt, buf, w0);
+    buf = buf == 2 ? 0 : buf + 1;
+    if (kt + 1 < nkt) {
+      stage(kt + 1, buf, w1);
+      buf = buf == 2 ? 0 : buf + 1;
     }
   }
+#undef IGEMM_WLOAD
+#undef IGEMM_WWAIT15
+  // the ring becomes the staging area: no direct-to-LDS write may still be in flight
+  __builtin_amdgcn_s_waitcnt(kWaitVm0);
+  igemm_epilogue<TIn, Epi, BM, BN, WM, WN>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
+}
 
-  // residual vectors of every pass are requested now so that their latency
-  // overlaps with the staging below instead of serialising the passes
-  constexpr int NPASS = 32 / PPP;
-  using RVec = typename Epi::RVec;
-  RVec rpre[TM][NPASS];
-  const bool have_rpre = Epi::kPrefetchResidual && vec && rbase != nullptr;
-  if constexpr (Epi::kPrefetchResidual) {
-    if (have_rpre) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int ps = 0; ps < NPASS; ++ps) {
-          const int m = tile_m * BM + wm * WM + i * 32 + ps * PPP + rp;
-          const int mc = m < M ? m : M - 1;
-          rpre[i][ps] = *reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n);
-        }
-    }
+// Rearranges packed weight rows ([batch][rows][row_bytes], zero padded) into
+// MFMA fragment order, followed by kWfragTailBytes of the fill byte: 16-byte unit ((b * tiles + t) * chunks + q) * 64 + lane
+// holds bytes [q*32 + (lane/32)*16, +16) of row t*32 + lane%32.
+__global__ void __launch_bounds__(256) wfrag_pack_kernel(WfragPackParams p) {
+  const int64_t total = (int64_t)p.batch * p.tiles * p.chunks * 64;
+  const uintx4* src = reinterpret_cast<const uintx4*>(p.src);
+  uintx4* dst = reinterpret_cast<uintx4*>(p.dst);
+  if (blockIdx.x == 0 && threadIdx.x < kWfragTailBytes / 16) {  // the fill vectors behind the fragments
+    const unsigned f = (unsigned)(p.fill & 0xff) * 0x01010101u;
+    dst[total + threadIdx.x] = (uintx4){f, f, f, f};
   }
-
-  __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    // park: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        AccE* dst = stage + l32 * EPI_PITCH + j * 32 + q * 8 + lg * 4;
-        if constexpr (sizeof(AccE) == 4 && !EpiTraits<Epi>::quant) {
-          *reinterpret_cast<floatx4*>(dst) =
-              (floatx4){acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
-        } else {
-          *reinterpret_cast<intx4*>(dst) =
-              (intx4){(int)acc[i][j][q * 4 + 0], (int)acc[i][j][q * 4 + 1], (int)acc[i][j][q * 4 + 2], (int)acc[i][j][q * 4 + 3]};
-        }
-      }
-    }
-    // Each wavefront only touches its own staging slice and its LDS operations
-    // complete in issue order, so a wavefront-scope fence (no workgroup barrier)
-    // orders the parking writes before the read-back.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int ps = 0; ps < NPASS; ++ps) {
-      const int pix = ps * PPP + rp;
-      const int m = tile_m * BM + wm * WM + i * 32 + pix;
-      AccE a8[8];
-      const AccE* src = stage + pix * EPI_PITCH + c8;
-      if constexpr (!EpiTraits<Epi>::quant) {
-        const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
-        const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
-        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-      } else {
-        const intx4 v0 = *reinterpret_cast<const intx4*>(src);
-        const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
-        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-      }
-      if (m < M && nvalid > 0) {
-        TOut* yrow = ybase + (int64_t)m * p.ycs + n;
-        const TOut* rrow = rbase ? rbase + (int64_t)m * p.rcs + n : nullptr;
-        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rpre[i][ps]);
-      }
-    }
-    if (i + 1 < TM) {
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+  for (int64_t u = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; u < total; u += (int64_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(u & 63);
+    int64_t t = u >> 6;
+    const int q = (int)(t % p.chunks);
+    t /= p.chunks;
+    const int tile = (int)(t % p.tiles);
+    const int64_t b = t / p.tiles;
+    const int row = tile * 32 + (lane & 31);
+    const int off = q * 32 + (lane >> 5) * 16;
+    uintx4 v = {0u, 0u, 0u, 0u};
+    if (row < p.rows && off < p.row_bytes) v = src[((b * p.rows + row) * p.row_bytes + off) >> 4];
+    dst[u] = v;
   }
 }
 
@@ -512,6 +785,15 @@ hipError_t launch_variant(const IgemmParams& p, int epi_vec, hipStream_t stream)
 // the launch still covers the 256 CUs.
 Variant choose_variant(const IgemmParams& p) {
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+  if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid: "128x64" etc.
+    int bm = 0, bn = 0;
+    if (sscanf(force, "%dx%d", &bm, &bn) == 2) {
+      if (bm == 128 && bn == 32) return {128, 32, "128x32"};
+      if (bm == 128 && bn == 64) return {128, 64, "128x64"};
+      if (bm == 64 && bn == 128) return {64, 128, "64x128"};
+      if (bm == 128 && bn == 128) return {128, 128, "128x128"};
+    }
+  }
   if (p.Kout <= 32) return {128, 32, "128x32"};
   if (p.Kout <= 64) return {128, 64, "128x64"};
   const int64_t blocks128 = ((M + 127) / 128) * ((p.Kout + 127) / 128) * p.batch;
@@ -530,9 +812,50 @@ hipError_t dispatch_tiles(const IgemmParams& p, int epi_vec, hipStream_t s) {
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+template <typename TIn, typename Epi>
+hipError_t launch_wreg(const IgemmParams& p, int epi_vec, hipStream_t stream) {
+  const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+  const int64_t tiles = ((M + 127) / 128) * ((p.Kout + 127) / 128);
+  if (tiles <= 0 || tiles > 0x7fffffff) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0, stream,
+                     p, epi_vec);
+  return hipGetLastError();
+}
+
+// The weights-in-registers kernel pays off once a layer has enough output
+// channels to give each of the four wavefronts its own 32-channel slice.
+bool wreg_shape(const IgemmParams& p) {
+  if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid
+    if (strcmp(force, "wreg") == 0) return true;
+    if (force[0] != 0) return false;
+  }
+  return p.Kout > 64;
+}
+
+template <typename TIn, typename Epi>
+hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
+  if (p.w_frag != nullptr && wreg_shape(p)) return launch_wreg<TIn, Epi>(p, epi_vec, s);
+  return dispatch_tiles<TIn, Epi>(p, epi_vec, s);
+}
+
 }  // namespace
 
-const char* igemm_variant_name(const IgemmParams& p) { return choose_variant(p).name; }
+bool igemm_wants_wfrag(const IgemmParams& p) { return wreg_shape(p); }
+
+hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
+  if (p.src == nullptr || p.dst == nullptr || p.rows <= 0 || p.row_bytes <= 0 || p.row_bytes % 16 != 0 ||
+      p.tiles * 32 < p.rows || p.chunks * 32 < p.row_bytes || p.chunks % 4 != 0 || p.batch <= 0)
+    return hipErrorInvalidValue;
+  if (!aligned16(p.src) || !aligned16(p.dst)) return hipErrorInvalidValue;
+  const int64_t total = (int64_t)p.batch * p.tiles * p.chunks * 64;
+  hipLaunchKernelGGL(wfrag_pack_kernel, dim3(grid_for(total, 256)), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+const char* igemm_variant_name(const IgemmParams& p) {
+  if (p.w_frag != nullptr && wreg_shape(p)) return "128x128w";
+  return choose_variant(p).name;
+}
 
 hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream) {
   const int es = dtype_size(p.in_dt);
@@ -551,6 +874,12 @@ hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream) {
   if (p.w_rows <= 0 || p.w_cols <= 0 || p.w_cols > p.w_rs) return hipErrorInvalidValue;
   if (p.w_cols % vec != 0) return hipErrorInvalidValue;
   if (p.residual != nullptr && p.rcs < p.Kout) return hipErrorInvalidValue;
+  if (p.w_frag != nullptr) {
+    const int64_t kbytes = (int64_t)p.R * p.S * p.C * es;
+    if (!aligned16(p.w_frag) || p.wf_chunks <= 0 || p.wf_chunks % 4 != 0 || (int64_t)p.wf_chunks * 32 < kbytes ||
+        (int64_t)p.wf_chunks * 32 >= kbytes + 128 || (int64_t)p.wf_tiles * 32 < p.Kout)
+      return hipErrorInvalidValue;
+  }
   // the last output pixel's receptive field must start inside the padded input
   if ((int64_t)(p.Ho - 1) * p.sh - p.ph >= p.H || (int64_t)(p.Wo - 1) * p.sw - p.pw >= p.W)
     return hipErrorInvalidValue;
@@ -571,25 +900,25 @@ hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream) {
   switch (p.in_dt) {
     case DT_F32:
       if (p.out_dt != DT_F32) return hipErrorInvalidValue;
-      return dispatch_tiles<float, EpiFloat<float>>(p, epi_vec, stream);
+      return dispatch<float, EpiFloat<float>>(p, epi_vec, stream);
     case DT_F16:
-      if (p.out_dt == DT_F16) return dispatch_tiles<f16_t, EpiFloat<f16_t>>(p, epi_vec, stream);
-      if (p.out_dt == DT_F32) return dispatch_tiles<f16_t, EpiFloat<float>>(p, epi_vec, stream);
+      if (p.out_dt == DT_F16) return dispatch<f16_t, EpiFloat<f16_t>>(p, epi_vec, stream);
+      if (p.out_dt == DT_F32) return dispatch<f16_t, EpiFloat<float>>(p, epi_vec, stream);
       return hipErrorInvalidValue;
     case DT_BF16:
-      if (p.out_dt == DT_BF16) return dispatch_tiles<bf16_t, EpiFloat<bf16_t>>(p, epi_vec, stream);
-      if (p.out_dt == DT_F32) return dispatch_tiles<bf16_t, EpiFloat<float>>(p, epi_vec, stream);
+      if (p.out_dt == DT_BF16) return dispatch<bf16_t, EpiFloat<bf16_t>>(p, epi_vec, stream);
+      if (p.out_dt == DT_F32) return dispatch<bf16_t, EpiFloat<float>>(p, epi_vec, stream);
       return hipErrorInvalidValue;
     case DT_I8:
       if (p.out_dt == DT_I8) {
         if (p.qmul == nullptr) return hipErrorInvalidValue;
-        return dispatch_tiles<int8_t, EpiQuant<0>>(p, epi_vec, stream);
+        return dispatch<int8_t, EpiQuant<0>>(p, epi_vec, stream);
       }
       if (p.out_dt == DT_F32) {
         if (p.qmul == nullptr) return hipErrorInvalidValue;
-        return dispatch_tiles<int8_t, EpiQuant<1>>(p, 0, stream);
+        return dispatch<int8_t, EpiQuant<1>>(p, 0, stream);
       }
-      if (p.out_dt == DT_I32) return dispatch_tiles<int8_t, EpiQuant<2>>(p, 0, stream);
+      if (p.out_dt == DT_I32) return dispatch<int8_t, EpiQuant<2>>(p, 0, stream);
       return hipErrorInvalidValue;
     default:
       return hipErrorInvalidValue;

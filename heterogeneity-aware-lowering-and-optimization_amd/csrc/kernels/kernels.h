@@ -73,6 +73,12 @@ struct IgemmParams {
   int64_t x_bs = 0, w_bs = 0, y_bs = 0, r_bs = 0, bias_bs = 0;  // per-z element strides
   DType in_dt = DT_F32;            // type of x and w
   DType out_dt = DT_F32;           // type of y and residual
+  // Optional copy of w in MFMA fragment order (see WfragPackParams); when set,
+  // layers with enough output channels read their weights from it directly
+  // into registers.  wf_chunks = 32-byte K chunks per row (a multiple of 4
+  // covering R*S*C), wf_tiles = 32-row tiles per batch entry.
+  const void* w_frag = nullptr;
+  int wf_chunks = 0, wf_tiles = 0;
   float alpha = 1.0f;              // scales the accumulator before bias (float types)
   ActKind act = ACT_NONE;
   float act_a = 0.0f, act_b = 0.0f;  // leaky slope / clamp lo,hi
@@ -93,6 +99,23 @@ struct IgemmParams {
 hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream);
 // Name of the kernel variant launch_igemm would pick (for reports).
 const char* igemm_variant_name(const IgemmParams& p);
+
+// True when launch_igemm would use a fragment-ordered weight copy for this shape.
+bool igemm_wants_wfrag(const IgemmParams& p);
+// [batch][rows][row_bytes] packed weight rows -> fragment order: the 16-byte
+// unit ((b * tiles + t) * chunks + q) * 64 + lane holds bytes
+// [q*32 + (lane/32)*16, +16) of row t*32 + lane%32; rows and bytes beyond the
+// source are zero.
+// The destination holds batch * tiles * chunks KiB of fragments followed by
+// kWfragTailBytes bytes of `fill` (the stored byte that represents the real
+// value 0 of the activation operand; padding taps fetch it).
+constexpr int kWfragTailBytes = 256;
+struct WfragPackParams {
+  const void* src = nullptr; void* dst = nullptr;
+  int batch = 1, rows = 0, row_bytes = 0, tiles = 0, chunks = 0;
+  int fill = 0;
+};
+hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream);
 
 // Repack a weight tensor into the [G][rows_pad][w_rs] matrix launch_igemm reads.
 // src element (o, i, r, s) lives at o*so + i*si + r*sr + s*ss.

@@ -889,6 +889,34 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
   ip.act = ep.act;
   ip.act_a = ep.act_a;
   ip.act_b = ep.act_b;
+  // Constant weights of layers that use the weights-in-registers kernel get a
+  // second copy in MFMA fragment order, built once at initialisation.
+  int tf = -1;
+  if (T(tw).space == SP_CONST && igemm_wants_wfrag(ip)) {
+    const int es = dtype_size(ip.in_dt);
+    WfragPackParams fp;
+    fp.batch = ip.batch;
+    fp.rows = ip.w_rows;
+    fp.row_bytes = ip.w_rs * es;
+    fp.tiles = (ip.w_rows + 31) / 32;
+    fp.chunks = (int)(((int64_t)ip.R * ip.S * ip.C * es + 127) / 128) * 4;
+    if ((int64_t)ip.w_bs == (int64_t)ip.w_rows * ip.w_rs || ip.batch == 1) {
+      fp.fill = ip.a_fill;
+      tf = raw_buffer((size_t)fp.batch * fp.tiles * fp.chunks * 1024 + kWfragTailBytes, SP_CONST);
+      ip.wf_chunks = fp.chunks;
+      ip.wf_tiles = fp.tiles;
+      const Ref a = ref(tw), b = ref(tf);
+      const bool was_init = in_init_;
+      in_init_ = true;
+      emit("wfrag:" + name, {}, {}, [=](const ExecEnv& e, hipStream_t st) {
+        WfragPackParams p = fp; p.src = a(e); p.dst = b(e);
+        return launch_wfrag_pack(p, st);
+      });
+      in_init_ = was_init;
+    }
+  }
+  const bool hf = tf >= 0;
+  const Ref rf = ref(hf ? tf : tx);
   const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty);
   const Ref rb = ref(tb >= 0 ? tb : tx), rr = ref(tr >= 0 ? tr : tx);
   const bool hb = tb >= 0, hr = tr >= 0;
@@ -897,6 +925,7 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
     p.x = rx(e); p.w = rw(e); p.y = ry(e);
     p.bias = hb ? rb(e) : nullptr;
     p.residual = hr ? rr(e) : nullptr;
+    p.w_frag = hf ? rf(e) : nullptr;
     return launch_igemm(p, st);
   });
 }
