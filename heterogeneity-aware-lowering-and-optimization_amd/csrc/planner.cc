@@ -461,6 +461,7 @@ class Planner {
   int pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og, int Cg, int R, int S, int Cp,
                    int64_t so, int64_t si, int64_t sr, int64_t ss, const std::vector<float>& row_scale,
                    int* w_rs_out, const std::vector<float>* wq_scale);
+  int make_wfrag(const std::string& name, IgemmParams* ip, int tw);
   void finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty, const Epilogue& ep,
                     int64_t Kout_total);
   int strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp_in);
@@ -870,6 +871,34 @@ int Planner::strided_copy_step(const std::string& name, int src, int dst, const 
   return dst;
 }
 
+// Constant weights of layers that use the weights-in-registers kernel get a
+// second copy in MFMA fragment order, built once at initialisation.  Returns
+// the tensor (and fills ip->wf_*), or -1 when the layer does not use one.
+int Planner::make_wfrag(const std::string& name, IgemmParams* ip, int tw) {
+  if (T(tw).space != SP_CONST || !igemm_wants_wfrag(*ip)) return -1;
+  if (ip->batch != 1 && (int64_t)ip->w_bs != (int64_t)ip->w_rows * ip->w_rs) return -1;
+  const int es = dtype_size(ip->in_dt);
+  WfragPackParams fp;
+  fp.batch = ip->batch;
+  fp.rows = ip->w_rows;
+  fp.row_bytes = ip->w_rs * es;
+  fp.tiles = (ip->w_rows + 31) / 32;
+  fp.chunks = (int)(((int64_t)ip->R * ip->S * ip->C * es + 127) / 128) * 4;
+  fp.fill = ip->a_fill;
+  const int tf = raw_buffer((size_t)fp.batch * fp.tiles * fp.chunks * 1024 + kWfragTailBytes, SP_CONST);
+  ip->wf_chunks = fp.chunks;
+  ip->wf_tiles = fp.tiles;
+  const Ref a = ref(tw), b = ref(tf);
+  const bool was_init = in_init_;
+  in_init_ = true;
+  emit("wfrag:" + name, {}, {}, [=](const ExecEnv& e, hipStream_t st) {
+    WfragPackParams p = fp; p.src = a(e); p.dst = b(e);
+    return launch_wfrag_pack(p, st);
+  });
+  in_init_ = was_init;
+  return tf;
+}
+
 // Common tail of Conv / Gemm lowering: bias / residual / activation wiring and
 // the launch step.  tx, tw, ty are the operand tensors.
 void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty,
@@ -889,32 +918,7 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
   ip.act = ep.act;
   ip.act_a = ep.act_a;
   ip.act_b = ep.act_b;
-  // Constant weights of layers that use the weights-in-registers kernel get a
-  // second copy in MFMA fragment order, built once at initialisation.
-  int tf = -1;
-  if (T(tw).space == SP_CONST && igemm_wants_wfrag(ip)) {
-    const int es = dtype_size(ip.in_dt);
-    WfragPackParams fp;
-    fp.batch = ip.batch;
-    fp.rows = ip.w_rows;
-    fp.row_bytes = ip.w_rs * es;
-    fp.tiles = (ip.w_rows + 31) / 32;
-    fp.chunks = (int)(((int64_t)ip.R * ip.S * ip.C * es + 127) / 128) * 4;
-    if ((int64_t)ip.w_bs == (int64_t)ip.w_rows * ip.w_rs || ip.batch == 1) {
-      fp.fill = ip.a_fill;
-      tf = raw_buffer((size_t)fp.batch * fp.tiles * fp.chunks * 1024 + kWfragTailBytes, SP_CONST);
-      ip.wf_chunks = fp.chunks;
-      ip.wf_tiles = fp.tiles;
-      const Ref a = ref(tw), b = ref(tf);
-      const bool was_init = in_init_;
-      in_init_ = true;
-      emit("wfrag:" + name, {}, {}, [=](const ExecEnv& e, hipStream_t st) {
-        WfragPackParams p = fp; p.src = a(e); p.dst = b(e);
-        return launch_wfrag_pack(p, st);
-      });
-      in_init_ = was_init;
-    }
-  }
+  const int tf = make_wfrag(name, &ip, tw);
   const bool hf = tf >= 0;
   const Ref rf = ref(hf ? tf : tx);
   const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty);
@@ -1062,6 +1066,9 @@ void Planner::lower_conv(int ni) {
       ip.r_zp = T(tr).qzp;
       ip.r_scale = T(tr).qscale;
     }
+    const int tf = make_wfrag("conv.i8:" + outv->name, &ip, tw);
+    const bool hf = tf >= 0;
+    const Ref rf = ref(hf ? tf : tx);
     const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb), rm = ref(tm), rr = ref(tr >= 0 ? tr : tx);
     const bool hr = tr >= 0;
     emit("conv.i8:" + outv->name, {tx, tw, tr}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
@@ -1069,6 +1076,7 @@ void Planner::lower_conv(int ni) {
       p.x = rx(e); p.w = rw(e); p.y = ry(e); p.bias = rb(e);
       p.qmul = (const float*)rm(e);
       p.residual = hr ? rr(e) : nullptr;
+      p.w_frag = hf ? rf(e) : nullptr;
       return launch_igemm(p, st);
     });
     if (ip.out_dt == DT_I32) {
