@@ -32,10 +32,24 @@ DTYPE = {"fp16": "f16", "bf16": "bf16", "fp32": "f32", "int8": "i8"}
 METRIC = "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW"
 
 
+# HBM bytes per conv/gemm launch (average over the launches of one step) read
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by
+# what the same counters read for a plain elementwise kernel of known size (the
+# ReLU launch of --workload streaming_fp16: 411 MB in, 411 MB out); the
+# summaries the figures come from are the traffic_* files under profiles/.
+# null = not measured.
+MEASURED_TRAFFIC = {
+    # 8.99 GB fetched + 5.69 GB written per step over its 54 conv/gemm launches
+    "resnet50_fp16": 271.8e6,
+}
+
+
 class Workload:
-    def __init__(self, name, unit, batch, flop_per_step, desc, build, feeds, ref_run, mode, table=None):
+    def __init__(self, name, unit, batch, flop_per_step, desc, build, feeds, ref_run, mode, table=None,
+                 conv_elements=None):
         self.name, self.unit, self.batch, self.flop, self.desc = name, unit, batch, flop_per_step, desc
         self.build, self.feeds, self.ref_run, self.mode, self.table = build, feeds, ref_run, mode, table
+        self.conv_elements = conv_elements
 
 
 def make_workload(name, batch, pkg):
@@ -55,7 +69,9 @@ def make_workload(name, batch, pkg):
         return Workload(name, "images/s", batch, models.RESNET50_GFLOP_PER_IMAGE * 1e9 * batch,
                         "ResNet-50 v1.5 %s NCHW [%d,3,224,224], folded BN, random He-normal weights, softmax head; "
                         "inputs/outputs resident in HBM" % (mode, batch),
-                        lambda b: models.build_resnet50(b, w, batch), feeds, ref_run, mode, table)
+                        lambda b: models.build_resnet50(b, w, batch), feeds, ref_run, mode, table,
+                        conv_elements=models.resnet50_conv_elements(batch, cin_stored=16 if mode == "int8" else
+                                                                    (4 if mode == "fp32" else 8)))
     if family == "yolov3":
         my = pkg.models_yolo
         batch = batch or 16
@@ -307,12 +323,42 @@ def profile_roofline(L, sess, wl, dump_path=None):
             launches += 1
     achieved = wl.flop / (mm_ms * 1e-3) / 1e12 if mm_ms > 0 else 0.0
     peak = PEAK[wl.mode]
-    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-            "frac": round(achieved / peak, 4), "traffic": None,
-            "kernel": "igemm_kernel (all %d conv/gemm launches of one step, avg %.1f us)"
-                      % (launches, 1e3 * mm_ms / max(launches, 1)),
+    roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(wl.name),
+            "kernel": "igemm_wreg_kernel / igemm_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
+                      "avg %.2f GFLOP per launch)" % (launches, 1e3 * mm_ms / max(launches, 1),
+                                                     wl.flop / 1e9 / max(launches, 1)),
             "mm_ms_per_step": round(mm_ms, 4), "all_kernels_ms_per_step": round(total_ms, 4),
             "launches_per_step": n.value}
+    if wl.conv_elements is not None:
+        # The same launches priced against both rooflines: per launch the bound is
+        # max(FLOPs / MFMA peak, algorithmic bytes / 8 TB/s); most 1x1 layers of
+        # this network at batch 256 sit on the HBM side.
+        es = {"fp32": 4, "fp16": 2, "bf16": 2, "int8": 1}[wl.mode]
+        t_by = {}
+        for i in range(n.value):
+            name = buf[i].name.decode()
+            if name.startswith("conv"):
+                key = name.split(":", 1)[1].replace(".relu", "").replace("out", "c3")
+                t_by[key] = t_by.get(key, 0.0) + buf[i].ms
+        bound_ms = meas_ms = nbytes = 0.0
+        hbm_bound = 0
+        for key, (fl, act, wt) in wl.conv_elements.items():
+            if key not in t_by:
+                continue
+            by = (act + wt) * es
+            t_m, t_h = fl / (peak * 1e12) * 1e3, by / 8e12 * 1e3
+            hbm_bound += t_h > t_m
+            bound_ms += max(t_m, t_h)
+            meas_ms += t_by[key]
+            nbytes += by
+        if meas_ms > 0:
+            roof["hbm"] = {"algorithmic_GB_per_step": round(nbytes / 1e9, 3),
+                           "achieved_GBps": round(nbytes / (meas_ms * 1e-3) / 1e9, 1), "peak_GBps": 8000.0,
+                           "frac": round(nbytes / (meas_ms * 1e-3) / 8e12, 4),
+                           "launches_hbm_bound": int(hbm_bound), "launches_priced": len(t_by)}
+            roof["frac_of_per_launch_roofline"] = round(bound_ms / meas_ms, 4)
+    return roof
 
 
 def cpu_baseline(wl, sample):
