@@ -49,6 +49,12 @@ Q8_CONV_CASES = [
     (2, 3, 20, 20, 16, 7, 2, 3),
     (1, 48, 6, 6, 200, 1, 2, 0),
     (1, 512, 7, 7, 64, 3, 1, 1),
+    # weights-in-registers kernel (more than 64 output channels, input channels a
+    # multiple of the 128-byte K stage): ragged tiles, stride, several K stages
+    (2, 128, 9, 9, 160, 3, 1, 1),
+    (1, 256, 7, 7, 128, 3, 2, 1),
+    (3, 128, 6, 6, 200, 1, 1, 0),
+    (1, 384, 5, 5, 72, 1, 1, 0),
 ]
 
 
@@ -94,12 +100,14 @@ def test_q8_conv_accumulators_and_requant(case, odla, ref):
     assert np.array_equal(q_got, q_want.astype(np.int64))
 
 
-def test_q8_residual_fused_equals_unfused_equals_oracle(odla, ref):
+@pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (3, 128, 7, 7, 200)])
+def test_q8_residual_fused_equals_unfused_equals_oracle(dims, odla, ref):
     """Conv -> Add(residual) -> ReLU: fused into the conv epilogue, and as separate
-    quantised kernels (the conv result is also a graph output, which blocks fusion)."""
-    announce("q8 residual")
+    quantised kernels (the conv result is also a graph output, which blocks fusion).
+    The second shape takes the weights-in-registers kernel."""
+    announce("q8 residual %s" % (dims,))
     r = rng(7)
-    N, C, H, W, O = 2, 32, 8, 8, 64
+    N, C, H, W, O = dims
     x = r.standard_normal((N, C, H, W)).astype(np.float32)
     res = (r.standard_normal((N, O, H, W)) * 2).astype(np.float32)
     w = (r.standard_normal((O, C, 1, 1)) * 0.3).astype(np.float32)

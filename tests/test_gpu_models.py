@@ -1,7 +1,7 @@
 """End-to-end parity of whole graphs through the ODLA C ABI against the CPU
 oracle: the mnist softmax regression (config 0) and ResNet-50-shaped networks
 (reduced depth/width so the CPU oracle finishes in seconds; the full-size
-network is covered by size-independent checks in test_gpu_resnet50_full.py).
+network is covered by test_gpu_resnet50_full.py).
 """
 import numpy as np
 import pytest

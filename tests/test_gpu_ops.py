@@ -123,6 +123,17 @@ CONV_CASES = [
     (2, 32, 8, 8, 64, 3, 1, 1, 2, 1),
     (1, 20, 7, 7, 255, 1, 1, 0, 1, 1),
     (1, 4, 5, 5, 4, 5, 1, 0, 1, 1),
+    # shapes that take the weights-in-registers kernel (more than 64 output
+    # channels, input channels a multiple of the K stage, at most 32 taps):
+    # ragged pixel and channel tiles, stride, dilation, 1 and many K stages
+    (2, 64, 14, 14, 160, 3, 1, 1, 1, 1),
+    (1, 128, 9, 9, 128, 3, 2, 1, 1, 1),
+    (2, 64, 10, 10, 96, 3, 1, 2, 1, 2),
+    (3, 192, 7, 7, 256, 1, 1, 0, 1, 1),
+    (1, 64, 6, 6, 72, 5, 1, 2, 1, 1),
+    (1, 64, 8, 8, 80, 1, 1, 0, 1, 1),
+    (1, 64, 9, 9, 96, 7, 1, 3, 1, 1),   # 49 taps: stays on the two-operand kernel
+    (5, 64, 12, 12, 300, 1, 1, 0, 1, 1),
 ]
 
 
@@ -177,6 +188,38 @@ def test_conv_fused_chain_fp32():
 
     got, want = run_both(build, {"x": x, "res": res})
     assert max_rel_err(got["out"], want["out"]) <= F32_TOL
+
+
+@pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16"])
+def test_conv_residual_relu_wide(mode):
+    """Bottleneck tail at a width that takes the weights-in-registers kernel:
+    3x3 conv + bias + ReLU, then 1x1 conv + bias + shortcut Add + ReLU, each
+    fused into one launch; 2 x 13 x 13 pixels (338 rows: ragged 128-row tiles)."""
+    announce("conv residual relu wide %s" % mode)
+    r = rng(77)
+    N, C, H, W, O = 2, 64, 13, 13, 192
+    w1 = (r.standard_normal((C, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    b1 = (r.standard_normal(C) * 0.1).astype(np.float32)
+    w2 = (r.standard_normal((O, C, 1, 1)) * np.sqrt(2.0 / C)).astype(np.float32)
+    b2 = (r.standard_normal(O) * 0.1).astype(np.float32)
+    wd = (r.standard_normal((O, C, 1, 1)) * np.sqrt(2.0 / C)).astype(np.float32)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+
+    def build(b):
+        v = b.arg("x", (N, C, H, W))
+        sc = b.conv(v, b.const("wd", wd), None, (1, 1), (0, 0, 0, 0), name="ds")
+        y = b.relu(b.conv(v, b.const("w1", w1), b.const("b1", b1), (1, 1), (1, 1, 1, 1), name="c2"), name="c2r")
+        y = b.conv(y, b.const("w2", w2), b.const("b2", b2), (1, 1), (0, 0, 0, 0), name="c3")
+        y = b.relu(b.add(y, sc, name="sum"), name="out")
+        b.output(y, "out")
+
+    kw = {"fp16": mode == "fp16", "bf16": mode == "bf16"}
+    got, want = run_both(build, {"x": x}, **kw)
+    if mode == "fp32":
+        assert max_rel_err(got["out"], want["out"]) <= F32_TOL
+    else:
+        tol = 2e-2 if mode == "fp16" else 6e-2
+        assert np.max(np.abs(got["out"] - want["out"])) <= tol * max(1.0, float(np.max(np.abs(want["out"]))))
 
 
 # --------------------------------------------------------------------------
