@@ -792,7 +792,9 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   // Requests the next K stage of the pixel tile into buffer `buf`.  Requests
   // past the last tap (the pipeline's run-out) fetch the fill vector.
   auto dma = [&](const int buf) {
-    const bool live = tap < RS;
+    // (1x1 filters may have any channel count: the last stage is then partial
+    // and this thread's chunk may lie beyond C, where the weights are zero)
+    const bool live = tap < RS && kc0 + kv * VEC < p.C;
     const int64_t toff = ((int64_t)(tap_r * p.dh) * p.W + tap_s * p.dw) * p.xcs + kc0;
     unsigned char* dst = smem + buf * BUF_BYTES + wave * 1024;
 #pragma unroll
@@ -806,7 +808,7 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
 #endif
     }
     kc0 += BK;
-    if (kc0 == p.C) {
+    if (kc0 >= p.C) {
       kc0 = 0;
       ++tap;
       if (++tap_s == p.S) { tap_s = 0; ++tap_r; }
@@ -1021,6 +1023,9 @@ bool wreg_shape(const IgemmParams& p) {
     if (force[0] != 0) return false;
   }
   const int bk = 128 / dtype_size(p.in_dt);
+  // A K stage must lie inside one filter tap.  (The kernel also handles 1x1
+  // filters with any channel count, but with less than one full stage of K the
+  // two-operand kernel is faster: measured on the 64 -> 256 int8 layers.)
   return p.Kout > 64 && p.C % bk == 0 && p.R * p.S <= 32;
 }
 
