@@ -177,43 +177,53 @@ struct EpiQuant {
                                                 const int* b8, const float* m8, TOut* y, const TOut* r,
                                                 bool have_rpre, RVec rpre) {
     if constexpr (MODE == 0) {
-      int8_t rs[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      // Levels are carried as floats (small integers are exact): per element
+      //   t  = rne(float(acc + bias) * M)          add, cvt, mul, rndne
+      //   q  = med3(t + zp, lo, 255)               add, med3
+      // and with a fused residual (dequantise, add, requantise, as the unfused
+      // kernels do it)
+      //   f  = (q - zp) * s_q + (r - zp_r) * s_r   sub, mul, cvt_ubyte, sub, mul, add
+      //   q  = med3(rne(f * (1/s_out)) + zp_out, lo_out, 255)
+      // v_cvt_pk_u8_f32 packs a level into its byte; stored bytes are level - 128,
+      // i.e. level ^ 0x80.  Beyond 2^24 the float sums are inexact but far outside
+      // the clamp range on the same side, so the result is the same as in integers.
+      unsigned rw[2] = {0u, 0u};
       if (r != nullptr) {
         if (vec) {
           const uintx2 rv = have_rpre ? rpre : *reinterpret_cast<const uintx2*>(r);
-          __builtin_memcpy(rs, &rv, 8);
+          rw[0] = rv.x;
+          rw[1] = rv.y;
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (e < nvalid) rs[e] = r[e];
+            if (e < nvalid) rw[e >> 2] |= (unsigned)(uint8_t)r[e] << (8 * (e & 3));
         }
+        rw[0] ^= 0x80808080u;  // stored -> levels
+        rw[1] ^= 0x80808080u;
       }
-      int8_t out[8];
+      const float zp = (float)p.q_zp, lo = (float)p.q_lo;
+      const float rzp = (float)p.r_zp, szp = (float)p.s_zp, slo = (float)p.s_lo;
+      unsigned ow[2] = {0u, 0u};
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int a = acc[e] + b8[e];
-        const float f0 = (float)a * m8[e];   // v_cvt_f32_i32 (RNE), then one v_mul_f32
-        int q = (int)rintf(f0) + p.q_zp;      // v_rndne_f32
-        q = q < p.q_lo ? p.q_lo : q;
-        q = q > 255 ? 255 : q;
+        const float t = rintf((float)(acc[e] + b8[e]) * m8[e]);
+        float q = __builtin_amdgcn_fmed3f(t + zp, lo, 255.f);
         if (r != nullptr) {
-          const float fa = (float)(q - p.q_zp) * p.q_scale;
-          const float fb = (float)(q_from_stored(rs[e]) - p.r_zp) * p.r_scale;
+          const float fa = (q - zp) * p.q_scale;
+          const float fb = ((float)((rw[e >> 2] >> (8 * (e & 3))) & 0xffu) - rzp) * p.r_scale;
           const float f = fa + fb;
-          q = (int)rintf(f * p.s_inv) + p.s_zp;
-          q = q < p.s_lo ? p.s_lo : q;
-          q = q > 255 ? 255 : q;
+          q = __builtin_amdgcn_fmed3f(rintf(f * p.s_inv) + szp, slo, 255.f);
         }
-        out[e] = q_to_stored(q);
+        ow[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(q, e & 3, ow[e >> 2]);
       }
+      ow[0] ^= 0x80808080u;  // levels -> stored
+      ow[1] ^= 0x80808080u;
       if (vec) {
-        uintx2 ov;
-        __builtin_memcpy(&ov, out, 8);
-        *reinterpret_cast<uintx2*>(y) = ov;
+        *reinterpret_cast<uintx2*>(y) = (uintx2){ow[0], ow[1]};
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (e < nvalid) y[e] = out[e];
+          if (e < nvalid) y[e] = (int8_t)(ow[e >> 2] >> (8 * (e & 3)));
       }
     } else {
       if constexpr (MODE == 2) {
