@@ -468,7 +468,18 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     if (have_rpre) rfetch(0, rcur);
   }
 
-  __syncthreads();  // the K loop's LDS reads are done; the ring becomes the staging area
+  // Workgroup barrier for LDS traffic only: the fence of __syncthreads would
+  // also wait for the global stores of the slices before, one store round trip
+  // per slice.
+  auto lds_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0), other counters at their maxima
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     AccE* tile = reinterpret_cast<AccE*>(smem) + (i & 1) * TILE_WORDS;
@@ -487,7 +498,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     // One barrier per slice is enough: a wavefront parks slice i+1 into the
     // other tile only after its own read-back of slice i, and nobody passes
     // this barrier before every wavefront has finished reading slice i-1.
-    __syncthreads();
+    lds_barrier();
     if constexpr (Epi::kPrefetchResidual) {
       if (have_rpre && i + 1 < TM) rfetch(i + 1, rnxt);
     }
