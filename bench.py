@@ -323,7 +323,8 @@ def profile_roofline(L, sess, wl, dump_path=None):
             launches += 1
     achieved = wl.flop / (mm_ms * 1e-3) / 1e12 if mm_ms > 0 else 0.0
     peak = PEAK[wl.mode]
-    roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+    roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
+            "unit": "TOP/s" if wl.mode == "int8" else "TFLOP/s",
             "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(wl.name),
             "kernel": "igemm_wreg_kernel / igemm_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
                       "avg %.2f GFLOP per launch)" % (launches, 1e3 * mm_ms / max(launches, 1),
