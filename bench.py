@@ -70,8 +70,9 @@ def make_workload(name, batch, pkg):
                         "ResNet-50 v1.5 %s NCHW [%d,3,224,224], folded BN, random He-normal weights, softmax head; "
                         "inputs/outputs resident in HBM" % (mode, batch),
                         lambda b: models.build_resnet50(b, w, batch), feeds, ref_run, mode, table,
-                        conv_elements=models.resnet50_conv_elements(batch, cin_stored=16 if mode == "int8" else
-                                                                    (4 if mode == "fp32" else 8)))
+                        # the stem reads the space-to-depth copy of the image: 16 stored channels per
+                        # 2x2 block (12 in fp32), i.e. 4 (3) per source pixel
+                        conv_elements=models.resnet50_conv_elements(batch, cin_stored=3 if mode == "fp32" else 4))
     if family == "yolov3":
         my = pkg.models_yolo
         batch = batch or 16

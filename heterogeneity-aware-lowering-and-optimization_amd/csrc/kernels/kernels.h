@@ -145,6 +145,17 @@ struct LayoutParams {
   float scale = 1.f; int zp = 0;
 };
 hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream);
+// NCHW [N][C<=4][H][W] -> channels-last space-to-depth [N][ceil(H/2)][ceil(W/2)][cs],
+// channel (py*2 + px)*C + c = src[n][c][2hh+py][2ww+px]; missing source rows /
+// columns and channels 4C..cs-1 hold the real value 0 (quantised like the rest
+// when dst_dt == DT_I8).
+struct S2dParams {
+  const void* src = nullptr; void* dst = nullptr;
+  DType src_dt = DT_F32, dst_dt = DT_F32;
+  int N = 0, C = 0, H = 0, W = 0, cs = 0;
+  float scale = 1.f; int zp = 0;
+};
+hipError_t launch_nchw_to_s2d(const S2dParams& p, hipStream_t stream);
 hipError_t launch_nhwc_to_nchw(const LayoutParams& p, hipStream_t stream);
 
 // Flat conversions -------------------------------------------------------

@@ -286,6 +286,66 @@ hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// NCHW -> channels-last space-to-depth: dst pixel (hh, ww) of the half-size
+// image holds the 2x2 source block at (2hh, 2ww), channel (py*2 + px)*C + c =
+// src[n][c][2hh+py][2ww+px]; source positions beyond an odd H / W and the
+// channel padding up to cs hold the real value 0.  A stride-2 convolution over
+// the source is a stride-1 convolution over this tensor with a quarter of the
+// filter taps and four times the channels: few-channel network inputs then fill
+// their 16-byte vectors instead of being padded 3 -> 8.
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads) nchw_to_s2d_kernel(S2dParams p) {
+  const TS* src = reinterpret_cast<const TS*>(p.src);
+  TD* dst = reinterpret_cast<TD*>(p.dst);
+  const int Hs = (p.H + 1) >> 1, Ws = (p.W + 1) >> 1;
+  const int64_t total = (int64_t)p.N * Hs * Ws;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int ww = (int)(i % Ws);
+    const int64_t t = i / Ws;
+    const int hh = (int)(t % Hs);
+    const int64_t n = t / Hs;
+    TD out[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) st_from_float<TD>(&out[c], 0.f, p.scale, p.zp);
+#pragma unroll
+    for (int py = 0; py < 2; ++py) {
+      const int h = 2 * hh + py;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (c < p.C && h < p.H) {
+          const TS* row = src + ((n * p.C + c) * p.H + h) * (int64_t)p.W + 2 * ww;
+          const float v0 = ld_as_float<TS>(row, p.scale, p.zp);
+          const float v1 = (2 * ww + 1 < p.W) ? ld_as_float<TS>(row + 1, p.scale, p.zp) : 0.f;
+          // out[(py*2 + px)*C + c]: C is a run-time value, the index is not a constant
+#pragma unroll
+          for (int j = 0; j < 16; ++j) {
+            if (j == (py * 2 + 0) * p.C + c) st_from_float<TD>(&out[j], v0, p.scale, p.zp);
+            if (j == (py * 2 + 1) * p.C + c) st_from_float<TD>(&out[j], v1, p.scale, p.zp);
+          }
+        }
+      }
+    }
+    TD* o = dst + i * p.cs;
+    if ((p.cs * sizeof(TD)) % 16 == 0) {
+      const int nv = p.cs * (int)sizeof(TD) / 16;
+      for (int v = 0; v < nv; ++v) reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
+    } else {
+      for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+    }
+  }
+}
+
+hipError_t launch_nchw_to_s2d(const S2dParams& p, hipStream_t stream) {
+  if (!p.src || !p.dst || p.N <= 0 || p.C <= 0 || p.C > 4 || p.H <= 0 || p.W <= 0 || p.cs < 4 * p.C || p.cs > 16)
+    return hipErrorInvalidValue;
+  const int64_t total = (int64_t)p.N * ((p.H + 1) / 2) * ((p.W + 1) / 2);
+  const int grid = grid_for(total, kThreads);
+#define K4(TS, TD, ...) hipLaunchKernelGGL((nchw_to_s2d_kernel<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p)
+  LAYOUT_PAIR_DISPATCH(K4, 0);
+#undef K4
+  return hipGetLastError();
+}
+
 hipError_t launch_nhwc_to_nchw(const LayoutParams& p, hipStream_t stream) {
   if (!layout_ok(p)) return hipErrorInvalidValue;
   const int64_t ntiles = (int64_t)p.N * ((p.HW + THW - 1) / THW) * ((p.C + TC - 1) / TC);

@@ -953,9 +953,13 @@ void Planner::lower_conv(int ni) {
   }
   const Shape& xs = x->shape;
   const Shape& os = n.out->shape;
-  const int64_t N = xs.d[0], C = cl ? xs.d[3] : xs.d[1], H = cl ? xs.d[1] : xs.d[2], W = cl ? xs.d[2] : xs.d[3];
+  const int64_t N = xs.d[0];
+  int64_t C = cl ? xs.d[3] : xs.d[1], H = cl ? xs.d[1] : xs.d[2], W = cl ? xs.d[2] : xs.d[3];
   const int64_t Ho = cl ? os.d[1] : os.d[2], Wo = cl ? os.d[2] : os.d[3];
-  const int Og = (int)(O / G), Cg = (int)I;
+  const int Og = (int)(O / G);
+  int Cg = (int)I;
+  int str_h = (int)n.i[3], str_w = (int)n.i[4], dil_h = (int)n.i[5], dil_w = (int)n.i[6];
+  int pad_t = (int)n.i[7], pad_l = (int)n.i[8];
 
   Epilogue ep;
   if (bias != nullptr) {
@@ -979,10 +983,83 @@ void Planner::lower_conv(int ni) {
   const bool x_q8 = q8_value(x);
   const bool q8 = comp_->opts.int8 && x_q8 && qk != nullptr && const_kernel && !cl && G == 1 &&
                   !runtime_bias;
+
+  // ---- few-channel stride-2 convolution on an NCHW source (a network stem) ----
+  // Rewritten as a stride-1 convolution over the space-to-depth form of the
+  // input: source row 2*ho - pad + r = 2*(ho + dy) + py with dy = floor((r -
+  // pad) / 2), so the R taps collapse into dy_max - dy_min + 1 taps over four
+  // times the channels, channel (py*2 + px)*C + c.  7x7 / stride 2 / 3 channels
+  // becomes 4x4 / stride 1 / 12 channels: K shrinks from 49 x 8 (channels padded
+  // to one 16-byte vector) to 16 x 16 elements.
+  const _odla_value* kpack = k;  // the kernel tensor that is packed
+  _odla_value k_s2d;
+  int tx_s2d = -1;
+  {
+    const VState& xv = vs_[x->index];
+    const bool src_ok = xv.main >= 0 && T(xv.main).layout == L_ROWMAJOR && !T(xv.main).quant;
+    if (!cl && G == 1 && const_kernel && !runtime_bias && C <= 4 && str_h == 2 && str_w == 2 && dil_h == 1 &&
+        dil_w == 1 && (R > 2 || S > 2) && src_ok) {
+      auto floor2 = [](int e) { return e >= 0 ? e / 2 : -((-e + 1) / 2); };
+      const int dy0 = floor2(-pad_t), dy1 = floor2((int)R - 1 - pad_t);
+      const int dx0 = floor2(-pad_l), dx1 = floor2((int)S - 1 - pad_l);
+      const int R2 = dy1 - dy0 + 1, S2 = dx1 - dx0 + 1, C2 = 4 * (int)C;
+      const std::vector<float> w = const_as_float(k);
+      auto buf = std::make_unique<std::vector<uint8_t>>((size_t)O * C2 * R2 * S2 * 4, (uint8_t)0);
+      float* w2 = reinterpret_cast<float*>(buf->data());
+      for (int64_t o = 0; o < O; ++o)
+        for (int64_t c = 0; c < C; ++c)
+          for (int r = 0; r < R; ++r)
+            for (int t = 0; t < S; ++t) {
+              const int ey = r - pad_t, ex = t - pad_l;
+              const int dy = floor2(ey), dx = floor2(ex);
+              const int py = ey - 2 * dy, px = ex - 2 * dx;
+              const int64_t c2 = (py * 2 + px) * C + c;
+              w2[((o * C2 + c2) * R2 + (dy - dy0)) * S2 + (dx - dx0)] = w[o * so + c * si + r * sr + t * ss];
+            }
+      k_s2d.kind = _odla_value::CONSTANT;
+      k_s2d.name = k->name;
+      k_s2d.etype = ODLA_FLOAT32;
+      k_s2d.shape.rank = 4;
+      k_s2d.shape.d[0] = O; k_s2d.shape.d[1] = C2; k_s2d.shape.d[2] = R2; k_s2d.shape.d[3] = S2;
+      k_s2d.host_data = w2;
+      comp_->owned_data.push_back(std::move(buf));
+      kpack = &k_s2d;
+      so = (int64_t)C2 * R2 * S2; si = (int64_t)R2 * S2; sr = S2; ss = 1;
+
+      // converted input: [N][ceil(H/2)][ceil(W/2)][C2 padded to one vector]
+      const DType fdt = q8 ? DT_I8 : storage_dtype(x);
+      const int vec = 16 / dtype_size(fdt);
+      const int cs = round_up_i(C2, vec);
+      const int64_t H2 = (H + 1) / 2, W2 = (W + 1) / 2;
+      Shape sh2;
+      sh2.rank = 4;
+      sh2.d[0] = N; sh2.d[1] = C2; sh2.d[2] = H2; sh2.d[3] = W2;
+      tx_s2d = new_tensor(fdt, L_NHWC, sh2, cs, SP_ARENA);
+      S2dParams sp;
+      sp.src_dt = T(xv.main).dt; sp.dst_dt = fdt;
+      sp.N = (int)N; sp.C = (int)C; sp.H = (int)H; sp.W = (int)W; sp.cs = cs;
+      if (q8) {
+        const QuantEntry* qx = qentry(x);
+        if (qx == nullptr) fail(ODLA_INTERNAL_LOGIC_ERR, "int8 stem without a table entry for '%s'", x->name.c_str());
+        sp.scale = qx->scale; sp.zp = qx->zp;
+        set_quant(tx_s2d, true, qx->scale, qx->zp);
+      }
+      const int from = xv.main;
+      const Ref a = ref(from), b = ref(tx_s2d);
+      emit("to_s2d:" + x->name, {from}, {tx_s2d}, [=](const ExecEnv& e, hipStream_t st) {
+        S2dParams p = sp; p.src = a(e); p.dst = b(e);
+        return launch_nchw_to_s2d(p, st);
+      });
+      C = C2; Cg = C2; H = H2; W = W2; R = R2; S = S2;
+      str_h = str_w = 1;
+      pad_t = -dy0; pad_l = -dx0;
+    }
+  }
+
   if (q8) {
     // ---- int8 x int8 -> int32 with fused requantisation ----
     const int vec = 16;
-    const int tx = get(x, L_NHWC, FORM_QUANT, vec);
+    const int tx = tx_s2d >= 0 ? tx_s2d : get(x, L_NHWC, FORM_QUANT, vec);
     const int Cp = T(tx).cs;
     if (qk->ch_min.size() != (size_t)O) fail(ODLA_INVALID_PARAM, "quant table entry of kernel '%s' needs %lld channel records", k->name.c_str(), (long long)O);
     std::vector<float> sw((size_t)O);
@@ -991,10 +1068,10 @@ void Planner::lower_conv(int ni) {
       sw[o] = m > 0.f ? m / 127.f : 1.f;
     }
     int w_rs = 0;
-    const int tw = pack_weights(k, DT_I8, 1, (int)O, Cg, (int)R, (int)S, Cp, so, si, sr, ss, {}, &w_rs, &sw);
+    const int tw = pack_weights(kpack, DT_I8, 1, (int)O, Cg, (int)R, (int)S, Cp, so, si, sr, ss, {}, &w_rs, &sw);
     // int32 bias: rne(b / (s_x * s_w[o])) minus the zero-point correction
     // (zp_x - 128) * sum_k w_q[o][k]; activations are stored as q - 128.
-    std::vector<float> wf = const_as_float(k);
+    std::vector<float> wf = const_as_float(kpack);
     std::vector<int32_t> bi((size_t)O, 0);
     const float sx = T(tx).qscale;  // parameters of the tensor actually consumed
     const int zx = T(tx).qzp;
@@ -1022,8 +1099,8 @@ void Planner::lower_conv(int ni) {
     IgemmParams ip;
     ip.N = (int)N; ip.H = (int)H; ip.W = (int)W; ip.C = Cp; ip.xcs = Cp;
     ip.Ho = (int)Ho; ip.Wo = (int)Wo; ip.Kout = (int)O;
-    ip.R = (int)R; ip.S = (int)S; ip.sh = (int)n.i[3]; ip.sw = (int)n.i[4];
-    ip.dh = (int)n.i[5]; ip.dw = (int)n.i[6]; ip.ph = (int)n.i[7]; ip.pw = (int)n.i[8];
+    ip.R = (int)R; ip.S = (int)S; ip.sh = str_h; ip.sw = str_w;
+    ip.dh = dil_h; ip.dw = dil_w; ip.ph = pad_t; ip.pw = pad_l;
     ip.w_rows = (int)O; ip.w_cols = w_rs; ip.w_rs = w_rs;
     ip.in_dt = DT_I8;
     ip.a_fill = (zx - 128) & 0xff;
@@ -1105,7 +1182,7 @@ void Planner::lower_conv(int ni) {
     tx = get(x, L_ROWMAJOR, FORM_FLOAT);
     xcs = (int)C;
   } else {
-    tx = get(x, L_NHWC, FORM_FLOAT, vec);
+    tx = tx_s2d >= 0 ? tx_s2d : get(x, L_NHWC, FORM_FLOAT, vec);
     xcs = T(tx).cs;
   }
   if (T(tx).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "conv input storage type mismatch");
@@ -1118,13 +1195,13 @@ void Planner::lower_conv(int ni) {
     Cp = Cg;
   }
   int w_rs = 0;
-  const int tw = pack_weights(k, dt, G, Og, Cg, (int)R, (int)S, Cp, so, si, sr, ss, ep.row_scale, &w_rs, nullptr);
+  const int tw = pack_weights(kpack, dt, G, Og, Cg, (int)R, (int)S, Cp, so, si, sr, ss, ep.row_scale, &w_rs, nullptr);
 
   IgemmParams ip;
   ip.N = (int)N; ip.H = (int)H; ip.W = (int)W; ip.C = Cp; ip.xcs = xcs;
   ip.Ho = (int)Ho; ip.Wo = (int)Wo; ip.Kout = Og;
-  ip.R = (int)R; ip.S = (int)S; ip.sh = (int)n.i[3]; ip.sw = (int)n.i[4];
-  ip.dh = (int)n.i[5]; ip.dw = (int)n.i[6]; ip.ph = (int)n.i[7]; ip.pw = (int)n.i[8];
+  ip.R = (int)R; ip.S = (int)S; ip.sh = str_h; ip.sw = str_w;
+  ip.dh = dil_h; ip.dw = dil_w; ip.ph = pad_t; ip.pw = pad_l;
   ip.w_rows = Og; ip.w_cols = w_rs; ip.w_rs = w_rs;
   ip.in_dt = dt; ip.out_dt = dt;
   ip.batch = G;

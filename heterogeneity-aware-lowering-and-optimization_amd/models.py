@@ -130,8 +130,8 @@ def resnet50_conv_elements(batch, hw=224, stages=RESNET50_STAGES, stem=64, cin_s
     {name: (flops, activation elements read + written, weight elements)}.
     Each launch reads its input once, its residual once (c3 launches: the
     block's shortcut is fused into them) and writes its output once; the stem
-    reads the channels-last copy of the image, whose 3 channels are stored
-    padded to `cin_stored`."""
+    reads the library's channels-last copy of the image, which stores
+    `cin_stored` channels per source pixel."""
     out = {}
     h = (hw + 2 * 3 - 7) // 2 + 1
     out["stem"] = (2.0 * batch * h * h * stem * 3 * 49, batch * (hw * hw * cin_stored + h * h * stem), stem * 3 * 49)

@@ -55,6 +55,9 @@ Q8_CONV_CASES = [
     (1, 256, 7, 7, 128, 3, 2, 1),
     (3, 128, 6, 6, 200, 1, 1, 0),
     (1, 384, 5, 5, 72, 1, 1, 0),
+    # few-channel stride-2 stems (space-to-depth lowering), odd sizes
+    (2, 3, 15, 17, 8, 3, 2, 1),
+    (1, 2, 11, 9, 6, 5, 2, 2),
 ]
 
 

@@ -134,6 +134,13 @@ CONV_CASES = [
     (1, 64, 8, 8, 80, 1, 1, 0, 1, 1),
     (1, 64, 9, 9, 96, 7, 1, 3, 1, 1),   # 49 taps: stays on the two-operand kernel
     (5, 64, 12, 12, 300, 1, 1, 0, 1, 1),
+    # few input channels, stride 2: lowered through the space-to-depth form of
+    # the input (odd image sizes, even and odd paddings, 1..4 channels)
+    (2, 3, 15, 17, 8, 3, 2, 1, 1, 1),
+    (1, 1, 9, 9, 4, 5, 2, 2, 1, 1),
+    (2, 4, 12, 12, 16, 7, 2, 3, 1, 1),
+    (1, 2, 11, 8, 6, 4, 2, 0, 1, 1),
+    (1, 3, 10, 10, 8, 3, 2, 2, 1, 1),
 ]
 
 
