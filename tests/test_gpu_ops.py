@@ -240,6 +240,11 @@ GEMM_CASES = [
     (20, 36, 12, False, False, 1.0, 0.0, None, False),
     (20, 36, 12, False, True, 1.0, 0.0, None, False),
     (7, 10, 5, False, False, 1.0, 1.0, "row", True),
+    # constant B with more than 64 columns and K a multiple of the K stage:
+    # the weights-in-registers kernel (ragged row / column tiles, both layouts of B, transposed A)
+    (200, 256, 192, False, False, 1.0, 1.0, "row", True),
+    (130, 128, 96, False, True, 0.5, 1.0, "row", True),
+    (70, 64, 300, True, False, 1.0, 0.0, None, True),
 ]
 
 
