@@ -19,6 +19,13 @@
 //   SLICE      iv = start[r] end[r] stride[r];  TRANSPOSE iv = permutation
 //   QUANTIZE / DEQUANTIZE  i0 axis; in = {x, scale, zero_point?}
 //   NMS        i0 max outputs; f0 iou threshold, f1 score threshold
+//   EWISE      i0 EwiseOp; iv = rank, then one aligned shape per operand
+//   ARGEXT     i0 is_max, i1 axis, i2 last index on ties
+//   COPYND     i0 fill first; iv = rank R, dims[R], src strides[R], dst strides[R], src offset,
+//              dst offset (elements; row-major source and result)
+//   TOPK       i0 K, i1 largest, i2 axis; out = values, out2 = indices
+//   LRN        i0 layout, i1 window; f0 alpha, f1 beta, f2 bias
+//   ROWNORM    i0 layout; f0 eps, f1 scalar scale, f2 scalar offset; in = {x, scale?, offset?}
 #include <cmath>
 #include <cstring>
 
@@ -82,8 +89,15 @@ bool expand_like_reference(Shape* src, const Shape& dst) {
   return false;
 }
 
+odla_value ewise_same_type(EwiseOp op, odla_value l, odla_value r, const char* what, const odla_value_id id);
+
 odla_value binary(BinKind kind, odla_value lhs, odla_value rhs, const odla_value_id id) {
   REQUIRE(lhs && rhs, "binary op: null operand");
+  if (!is_float_type(lhs->etype) || !is_float_type(rhs->etype)) {
+    // integer arithmetic [ref: ODLA/platforms/dnnl/odla_dnnl.cc:567-610]
+    static const EwiseOp map[] = {EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_MAX, EW_MIN};
+    return ewise_same_type(map[kind], lhs, rhs, "binary op", id);
+  }
   _odla_computation* c = comp_of(lhs, rhs);
   REQUIRE(c, "binary op: no current computation");
   Shape a = lhs->shape, b = rhs->shape;
@@ -108,6 +122,62 @@ odla_value binary(BinKind kind, odla_value lhs, odla_value rhs, const odla_value
   for (int i = 0; i < a.rank; ++i) n->iv.push_back(a.d[i]);
   for (int i = 0; i < b.rank; ++i) n->iv.push_back(b.d[i]);
   return n->out;
+}
+
+// Typed element-wise node over up to three operands, broadcast like binary():
+// lower-rank operands are aligned against the operand of highest rank.
+odla_value ewise(EwiseOp op, std::vector<odla_value> in, odla_element_type out_type, const char* what,
+                 const odla_value_id id, const Shape* target = nullptr) {
+  for (odla_value v : in) REQUIRE(v, "%s: null operand", what);
+  _odla_computation* c = comp_of(in[0], in.size() > 1 ? in[1] : nullptr);
+  REQUIRE(c, "%s: no current computation", what);
+  Shape hi = target ? *target : in[0]->shape;
+  if (!target)
+    for (odla_value v : in)
+      if (v->shape.rank > hi.rank) hi = v->shape;
+  std::vector<Shape> al;
+  for (odla_value v : in) {
+    Shape s = v->shape;
+    if (s.rank != hi.rank)
+      REQUIRE(s.rank < hi.rank && expand_like_reference(&s, hi), "%s: shapes %s and %s do not broadcast", what,
+              v->shape.str().c_str(), hi.str().c_str());
+    al.push_back(s);
+  }
+  Shape o;
+  o.rank = hi.rank;
+  for (int i = 0; i < o.rank; ++i) {
+    o.d[i] = 1;
+    for (const Shape& s : al)
+      if (s.d[i] > o.d[i]) o.d[i] = s.d[i];
+    for (const Shape& s : al)
+      REQUIRE(s.d[i] == o.d[i] || s.d[i] == 1, "%s: operand shapes do not broadcast in dim %d", what, i);
+  }
+  if (target) REQUIRE(o == *target, "%s: operands do not broadcast to %s", what, target->str().c_str());
+  Node* n = add_node(c, OP_EWISE, in, out_type, o, id);
+  n->i[0] = op;
+  n->iv.push_back(o.rank);
+  for (const Shape& s : al)
+    for (int i = 0; i < o.rank; ++i) n->iv.push_back(s.d[i]);
+  return n->out;
+}
+
+odla_value ewise_same_type(EwiseOp op, odla_value l, odla_value r, const char* what, const odla_value_id id) {
+  REQUIRE(l && r, "%s: null operand", what);
+  REQUIRE(l->etype == r->etype, "%s: operands '%s' and '%s' differ in element type", what, l->name.c_str(),
+          r->name.c_str());
+  REQUIRE(l->etype != ODLA_BOOL, "%s: arithmetic on boolean values", what);
+  return ewise(op, {l, r}, l->etype, what, id);
+}
+odla_value ewise_compare(EwiseOp op, odla_value l, odla_value r, const char* what, const odla_value_id id) {
+  REQUIRE(l && r, "%s: null operand", what);
+  REQUIRE(l->etype == r->etype, "%s: operands '%s' and '%s' differ in element type", what, l->name.c_str(),
+          r->name.c_str());
+  return ewise(op, {l, r}, ODLA_BOOL, what, id);
+}
+odla_value ewise_logic(EwiseOp op, odla_value l, odla_value r, const char* what, const odla_value_id id) {
+  REQUIRE(l && r, "%s: null operand", what);
+  REQUIRE(l->etype == ODLA_BOOL && r->etype == ODLA_BOOL, "%s: operands must be boolean", what);
+  return ewise(op, {l, r}, ODLA_BOOL, what, id);
 }
 
 odla_value unary(ActKind kind, odla_value x, float a, float b, const odla_value_id id) {
@@ -162,7 +232,7 @@ odla_value pool(bool is_max, odla_value input, odla_memory_layout layout, const 
 }
 
 odla_value reduce(ReduceKind kind, odla_value input, odla_size_t num_axes, const odla_uint32* axes,
-                  odla_bool keep_dims, const odla_value_id id) {
+                  odla_bool keep_dims, const odla_value_id id, float eps = 0.f) {
   REQUIRE(input && (axes || num_axes == 0), "reduce: null argument");
   _odla_computation* c = comp_of(input);
   REQUIRE(c, "reduce: no current computation");
@@ -186,8 +256,64 @@ odla_value reduce(ReduceKind kind, odla_value input, odla_size_t num_axes, const
   Node* n = add_node(c, OP_REDUCE, {input}, input->etype, o, id);
   n->i[0] = kind;
   n->i[1] = keep_dims;
+  n->f[0] = eps;
   for (int i = 0; i < r; ++i)
     if (red[i]) n->iv.push_back(i);
+  return n->out;
+}
+
+// Strided gather / scatter copy node over a row-major source and result.
+odla_value copynd(_odla_computation* c, odla_value x, const Shape& out, const std::vector<int64_t>& dims,
+                  const std::vector<int64_t>& sx, const std::vector<int64_t>& sy, int64_t x_off, int64_t y_off,
+                  bool fill, const odla_value_id id) {
+  Node* n = add_node(c, OP_COPYND, {x}, x->etype, out, id);
+  n->i[0] = fill;
+  n->iv.push_back((int64_t)dims.size());
+  n->iv.insert(n->iv.end(), dims.begin(), dims.end());
+  n->iv.insert(n->iv.end(), sx.begin(), sx.end());
+  n->iv.insert(n->iv.end(), sy.begin(), sy.end());
+  n->iv.push_back(x_off);
+  n->iv.push_back(y_off);
+  return n->out;
+}
+odla_value_shape undefined_shape() {
+  odla_value_shape s;
+  memset(&s, 0, sizeof(s));
+  return s;
+}
+std::vector<int64_t> row_major_strides(const Shape& s) {
+  std::vector<int64_t> st(s.rank);
+  int64_t acc = 1;
+  for (int i = s.rank - 1; i >= 0; --i) { st[i] = acc; acc *= s.d[i]; }
+  return st;
+}
+
+// [ref: ODLA/platforms/dnnl/odla_dnnl_statistics.cc:203-300]
+odla_value arg_extreme(bool is_max, odla_value input, odla_int32 axis, odla_bool keep_dims,
+                       odla_bool return_last_index, const odla_value_type& out_type, const odla_value_id id) {
+  REQUIRE(input, "ArgMax/ArgMin: null operand");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "ArgMax/ArgMin: no current computation");
+  REQUIRE(is_float_type(input->etype), "ArgMax/ArgMin: operand must be a float type");
+  const int r = input->shape.rank;
+  if (axis < 0) axis += r;
+  REQUIRE(axis >= 0 && axis < r, "ArgMax/ArgMin: axis out of range for %s", input->shape.str().c_str());
+  const odla_element_type et = out_type.element_type == ODLA_INT64 ? ODLA_INT64 : ODLA_INT32;
+  REQUIRE(out_type.element_type == ODLA_INT64 || out_type.element_type == ODLA_INT32,
+          "ArgMax/ArgMin: the index type must be INT32 or INT64");
+  Shape o;
+  for (int i = 0; i < r; ++i) {
+    if (i == axis) {
+      if (keep_dims) o.d[o.rank++] = 1;
+    } else {
+      o.d[o.rank++] = input->shape.d[i];
+    }
+  }
+  if (o.rank == 0) { o.rank = 1; o.d[0] = 1; }
+  Node* n = add_node(c, OP_ARGEXT, {input}, et, o, id);
+  n->i[0] = is_max;
+  n->i[1] = axis;
+  n->i[2] = return_last_index != 0;
   return n->out;
 }
 
@@ -293,6 +419,71 @@ odla_value odla_Div(odla_value l, odla_value r, const odla_value_id id) { return
 odla_value odla_Max(odla_value l, odla_value r, const odla_value_id id) { return binary(BIN_MAX, l, r, id); }
 odla_value odla_Min(odla_value l, odla_value r, const odla_value_id id) { return binary(BIN_MIN, l, r, id); }
 
+odla_value odla_Pow(odla_value l, odla_value r, const odla_value_id id) { return ewise_same_type(EW_POW, l, r, "odla_Pow", id); }
+odla_value odla_Mod(odla_value l, odla_value r, odla_int64 fmod, const odla_value_id id) {
+  return ewise_same_type(fmod == 1 ? EW_FMOD : EW_MOD, l, r, "odla_Mod", id);
+}
+odla_value odla_SquaredDifference(odla_value l, odla_value r, const odla_value_id id) {
+  return ewise_same_type(EW_SQDIFF, l, r, "odla_SquaredDifference", id);
+}
+odla_value odla_PRelu(odla_value x, odla_value slope, const odla_value_id id) {
+  return ewise_same_type(EW_PRELU, x, slope, "odla_PRelu", id);
+}
+odla_value odla_Equal(odla_value l, odla_value r, const odla_value_id id) { return ewise_compare(EW_EQ, l, r, "odla_Equal", id); }
+odla_value odla_NotEqual(odla_value l, odla_value r, const odla_value_id id) { return ewise_compare(EW_NE, l, r, "odla_NotEqual", id); }
+odla_value odla_Less(odla_value l, odla_value r, const odla_value_id id) { return ewise_compare(EW_LT, l, r, "odla_Less", id); }
+odla_value odla_LessOrEqual(odla_value l, odla_value r, const odla_value_id id) { return ewise_compare(EW_LE, l, r, "odla_LessOrEqual", id); }
+odla_value odla_Greater(odla_value l, odla_value r, const odla_value_id id) { return ewise_compare(EW_GT, l, r, "odla_Greater", id); }
+odla_value odla_GreaterOrEqual(odla_value l, odla_value r, const odla_value_id id) { return ewise_compare(EW_GE, l, r, "odla_GreaterOrEqual", id); }
+odla_value odla_And(odla_value l, odla_value r, const odla_value_id id) { return ewise_logic(EW_AND, l, r, "odla_And", id); }
+odla_value odla_Or(odla_value l, odla_value r, const odla_value_id id) { return ewise_logic(EW_OR, l, r, "odla_Or", id); }
+odla_value odla_Xor(odla_value l, odla_value r, const odla_value_id id) { return ewise_logic(EW_XOR, l, r, "odla_Xor", id); }
+odla_value odla_Not(odla_value x, const odla_value_id id) {
+  REQUIRE(x, "odla_Not: null operand");
+  REQUIRE(x->etype == ODLA_BOOL, "odla_Not: operand must be boolean");
+  return ewise(EW_NOT, {x}, ODLA_BOOL, "odla_Not", id);
+}
+odla_value odla_IsNaN(odla_value x, const odla_value_id id) {
+  REQUIRE(x, "odla_IsNaN: null operand");
+  REQUIRE(is_float_type(x->etype), "odla_IsNaN: operand must be a float type");
+  return ewise(EW_ISNAN, {x}, ODLA_BOOL, "odla_IsNaN", id);
+}
+odla_value odla_IsInf(odla_value x, odla_bool detect_pos, odla_bool detect_neg, const odla_value_id id) {
+  REQUIRE(x, "odla_IsInf: null operand");
+  REQUIRE(is_float_type(x->etype), "odla_IsInf: operand must be a float type");
+  // neither flag set selects the negative test, as in the reference [ref: odla_dnnl_unary.cc:229-238]
+  const EwiseOp op = (detect_pos && detect_neg) ? EW_ISINF : (detect_pos ? EW_ISINF_POS : EW_ISINF_NEG);
+  return ewise(op, {x}, ODLA_BOOL, "odla_IsInf", id);
+}
+odla_value odla_Select(odla_value cond, odla_value a, odla_value b, odla_value_shape output_dims,
+                       const odla_value_id id) {
+  REQUIRE(cond && a && b, "odla_Select: null operand");
+  REQUIRE(cond->etype == ODLA_BOOL, "odla_Select: the condition must be boolean");
+  REQUIRE(a->etype == b->etype, "odla_Select: branches differ in element type");
+  if (shape_valid(output_dims)) {
+    const Shape t = shape_from(output_dims);
+    return ewise(EW_SELECT, {cond, a, b}, a->etype, "odla_Select", id, &t);
+  }
+  return ewise(EW_SELECT, {cond, a, b}, a->etype, "odla_Select", id);
+}
+// Element-wise mean of n same-shaped (or broadcastable) values.
+// [ref: ODLA/platforms/dnnl/odla_dnnl.cc:2432-2441]
+odla_value odla_Mean(odla_values inputs, const odla_value_id id) {
+  REQUIRE(inputs.size >= 1 && inputs.size <= ODLA_MAX_OUTPUTS, "odla_Mean: bad operand count");
+  odla_value acc = inputs.values[0];
+  REQUIRE(acc, "odla_Mean: null operand");
+  REQUIRE(is_float_type(acc->etype), "odla_Mean: operands must be a float type");
+  for (odla_size_t i = 1; i < inputs.size; ++i) {
+    acc = binary(BIN_ADD, acc, inputs.values[i], nullptr);
+    if (acc == nullptr) return nullptr;
+  }
+  _odla_computation* c = comp_of(acc);
+  Node* n = add_node(c, OP_UNARY, {acc}, acc->etype, acc->shape, id);
+  n->i[0] = ACT_DIV_CONST;
+  n->f[0] = (float)inputs.size;
+  return n->out;
+}
+
 odla_value odla_Relu(odla_value x, const odla_value_id id) { return unary(ACT_RELU, x, 0, 0, id); }
 odla_value odla_LeakyRelu(odla_value x, odla_float32 alpha, const odla_value_id id) { return unary(ACT_LEAKY, x, alpha, 0, id); }
 odla_value odla_Sigmoid(odla_value x, const odla_value_id id) { return unary(ACT_SIGMOID, x, 0, 0, id); }
@@ -306,6 +497,43 @@ odla_value odla_Abs(odla_value x, const odla_value_id id) { return unary(ACT_ABS
 odla_value odla_Neg(odla_value x, const odla_value_id id) { return unary(ACT_NEG, x, 0, 0, id); }
 odla_value odla_Round(odla_value x, const odla_value_id id) { return unary(ACT_ROUND, x, 0, 0, id); }
 odla_value odla_Clamp(odla_value x, odla_float32 lo, odla_float32 hi, const odla_value_id id) { return unary(ACT_CLAMP, x, lo, hi, id); }
+odla_value odla_Reciprocal(odla_value x, const odla_value_id id) { return unary(ACT_RECIP, x, 0, 0, id); }
+odla_value odla_Ceil(odla_value x, const odla_value_id id) { return unary(ACT_CEIL, x, 0, 0, id); }
+odla_value odla_Floor(odla_value x, const odla_value_id id) { return unary(ACT_FLOOR, x, 0, 0, id); }
+odla_value odla_Sign(odla_value x, const odla_value_id id) { return unary(ACT_SIGN, x, 0, 0, id); }
+odla_value odla_Sin(odla_value x, const odla_value_id id) { return unary(ACT_SIN, x, 0, 0, id); }
+odla_value odla_Cos(odla_value x, const odla_value_id id) { return unary(ACT_COS, x, 0, 0, id); }
+odla_value odla_Tan(odla_value x, const odla_value_id id) { return unary(ACT_TAN, x, 0, 0, id); }
+odla_value odla_ASin(odla_value x, const odla_value_id id) { return unary(ACT_ASIN, x, 0, 0, id); }
+odla_value odla_ACos(odla_value x, const odla_value_id id) { return unary(ACT_ACOS, x, 0, 0, id); }
+odla_value odla_ATan(odla_value x, const odla_value_id id) { return unary(ACT_ATAN, x, 0, 0, id); }
+odla_value odla_Sinh(odla_value x, const odla_value_id id) { return unary(ACT_SINH, x, 0, 0, id); }
+odla_value odla_Cosh(odla_value x, const odla_value_id id) { return unary(ACT_COSH, x, 0, 0, id); }
+odla_value odla_ASinh(odla_value x, const odla_value_id id) { return unary(ACT_ASINH, x, 0, 0, id); }
+odla_value odla_ACosh(odla_value x, const odla_value_id id) { return unary(ACT_ACOSH, x, 0, 0, id); }
+odla_value odla_ATanh(odla_value x, const odla_value_id id) { return unary(ACT_ATANH, x, 0, 0, id); }
+odla_value odla_Elu(odla_value x, odla_float32 alpha, const odla_value_id id) { return unary(ACT_ELU, x, alpha, 0, id); }
+odla_value odla_Selu(odla_value x, odla_float32 alpha, odla_float32 gamma, const odla_value_id id) {
+  return unary(ACT_SELU, x, alpha, gamma, id);
+}
+odla_value odla_Celu(odla_value x, odla_float32 alpha, const odla_value_id id) {
+  if (alpha == 0.f) {
+    OHIP_ERR("odla_Celu: alpha must not be zero");
+    return nullptr;
+  }
+  return unary(ACT_CELU, x, alpha, 0, id);
+}
+odla_value odla_HardSigmoid(odla_value x, odla_float32 alpha, odla_float32 beta, const odla_value_id id) {
+  return unary(ACT_HARDSIGMOID, x, alpha, beta, id);
+}
+odla_value odla_Softplus(odla_value x, const odla_value_id id) { return unary(ACT_SOFTPLUS, x, 0, 0, id); }
+odla_value odla_Softsign(odla_value x, const odla_value_id id) { return unary(ACT_SOFTSIGN, x, 0, 0, id); }
+odla_value odla_ThresholdedRelu(odla_value x, odla_float32 alpha, const odla_value_id id) {
+  return unary(ACT_THRESHOLDED, x, alpha, 0, id);
+}
+odla_value odla_Shrink(odla_value x, odla_float32 bias, odla_float32 lambd, const odla_value_id id) {
+  return unary(ACT_SHRINK, x, bias, lambd, id);
+}
 odla_value odla_Gelu(odla_value x, odla_bool use_approx, const odla_value_id id) {
   return unary(use_approx ? ACT_GELU_TANH : ACT_GELU_ERF, x, 0, 0, id);
 }
@@ -384,6 +612,63 @@ odla_value odla_ReduceSum(odla_value input, odla_size_t n, const odla_uint32* ax
 odla_value odla_ReduceMax(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
                           odla_value_shape, const odla_value_id id) {
   return reduce(RED_MAX, input, n, axes, keep, id);
+}
+odla_value odla_ReduceMin(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                          odla_value_shape, const odla_value_id id) {
+  return reduce(RED_MIN, input, n, axes, keep, id);
+}
+odla_value odla_ReduceProd(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                           odla_value_shape, const odla_value_id id) {
+  return reduce(RED_PROD, input, n, axes, keep, id);
+}
+odla_value odla_ReduceL1(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                         odla_float32 epsilon, odla_value_shape, const odla_value_id id) {
+  return reduce(RED_L1, input, n, axes, keep, id, epsilon);
+}
+odla_value odla_ReduceL2(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                         odla_float32 epsilon, odla_value_shape, const odla_value_id id) {
+  return reduce(RED_L2, input, n, axes, keep, id, epsilon);
+}
+odla_value odla_ReduceSumSquare(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                                odla_value_shape, const odla_value_id id) {
+  return reduce(RED_SUMSQ, input, n, axes, keep, id);
+}
+odla_value odla_ReduceLogSum(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                             odla_value_shape, const odla_value_id id) {
+  return reduce(RED_LOGSUM, input, n, axes, keep, id);
+}
+// log(sum(exp(x - max))) + max, composed from the existing operators as the
+// reference does.  [ref: ODLA/platforms/dnnl/odla_dnnl_statistics.cc:77-105]
+odla_value odla_ReduceLogSumExp(odla_value input, odla_size_t n, const odla_uint32* axes, odla_bool keep,
+                                odla_value_shape, const odla_value_id id) {
+  odla_value mx = reduce(RED_MAX, input, n, axes, 1, nullptr);
+  if (mx == nullptr) return nullptr;
+  odla_value delta = binary(BIN_SUB, input, mx, nullptr);
+  if (delta == nullptr) return nullptr;
+  odla_value ex = unary(ACT_EXP, delta, 0, 0, nullptr);
+  odla_value ls = reduce(RED_LOGSUM, ex, n, axes, 1, nullptr);
+  if (ls == nullptr) return nullptr;
+  odla_value sum = binary(BIN_ADD, ls, mx, keep ? id : nullptr);
+  if (sum == nullptr || keep) return sum;
+  // drop the reduced dims
+  bool red[ODLA_MAX_DIMENSION] = {false};
+  const int r = input->shape.rank;
+  if (n == 0)
+    for (int i = 0; i < r; ++i) red[i] = true;
+  for (odla_size_t i = 0; i < n; ++i) red[axes[i]] = true;
+  Shape o;
+  for (int i = 0; i < r; ++i)
+    if (!red[i]) o.d[o.rank++] = input->shape.d[i];
+  if (o.rank == 0) { o.rank = 1; o.d[0] = 1; }
+  return odla_Reshape(sum, shape_to(o), id);
+}
+odla_value odla_ArgMax(odla_value input, odla_int32 axis, odla_bool keep_dims, odla_bool return_last_index,
+                       odla_value_type output_value_type, const odla_value_id id) {
+  return arg_extreme(true, input, axis, keep_dims, return_last_index, output_value_type, id);
+}
+odla_value odla_ArgMin(odla_value input, odla_int32 axis, odla_bool keep_dims, odla_bool return_last_index,
+                       odla_value_type output_value_type, const odla_value_id id) {
+  return arg_extreme(false, input, axis, keep_dims, return_last_index, output_value_type, id);
 }
 
 static odla_value softmax_impl(odla_value input, odla_int32 axis, bool logsm, const odla_value_id id) {
@@ -575,6 +860,264 @@ odla_value odla_Quantize(odla_value input, odla_value scale, odla_value zp, odla
 odla_value odla_Dequantize(odla_value input, odla_value scale, odla_value zp, odla_int32 axis,
                            odla_element_type target, const odla_value_id id) {
   return qdq(OP_DEQUANTIZE, input, scale, zp, axis, target, id);
+}
+
+// Zero padding.  [ref: ODLA/include/ODLA/ops/odla_ops_process.h:221-236]
+odla_value odla_Pad(odla_value input, const odla_uint32* padding_front, const odla_uint32* padding_back,
+                    odla_value_shape, const odla_value_id id) {
+  REQUIRE(input && padding_front && padding_back, "odla_Pad: null argument");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_Pad: no current computation");
+  const Shape& xs = input->shape;
+  REQUIRE(xs.rank <= 8, "odla_Pad: rank > 8");
+  Shape o = xs;
+  for (int i = 0; i < xs.rank; ++i) o.d[i] = xs.d[i] + padding_front[i] + padding_back[i];
+  const std::vector<int64_t> sx = row_major_strides(xs), sy = row_major_strides(o);
+  int64_t y_off = 0;
+  for (int i = 0; i < xs.rank; ++i) y_off += (int64_t)padding_front[i] * sy[i];
+  std::vector<int64_t> dims(xs.d, xs.d + xs.rank);
+  return copynd(c, input, o, dims, sx, sy, 0, y_off, true, id);
+}
+
+// Repeats the input `repeat[i]` times along dim i.
+// [ref: ops/odla_ops_process.h:437-451; dnnl odla_dnnl.cc:2183-2254]
+odla_value odla_Tile(odla_value input, const odla_uint32* repeat, odla_value_shape, const odla_value_id id) {
+  REQUIRE(input && repeat, "odla_Tile: null argument");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_Tile: no current computation");
+  const Shape& xs = input->shape;
+  REQUIRE(xs.rank <= 4, "odla_Tile: rank > 4");
+  Shape o = xs;
+  std::vector<int64_t> dims, sx, sy;
+  for (int i = 0; i < xs.rank; ++i) {
+    REQUIRE(repeat[i] >= 1, "odla_Tile: repeat count 0");
+    o.d[i] = xs.d[i] * repeat[i];
+  }
+  const std::vector<int64_t> xst = row_major_strides(xs), yst = row_major_strides(o);
+  for (int i = 0; i < xs.rank; ++i) {
+    dims.push_back(repeat[i]); sx.push_back(0); sy.push_back(yst[i] * xs.d[i]);
+    dims.push_back(xs.d[i]); sx.push_back(xst[i]); sy.push_back(yst[i]);
+  }
+  return copynd(c, input, o, dims, sx, sy, 0, 0, false, id);
+}
+
+// Broadcast to `output_dims`.  [ref: ops/odla_ops_process.h:117-130]
+odla_value odla_ExpandDims(odla_value input, odla_value_shape output_dims, const odla_value_id id) {
+  REQUIRE(input, "odla_ExpandDims: null argument");
+  REQUIRE(shape_valid(output_dims), "odla_ExpandDims: the output shape is required");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_ExpandDims: no current computation");
+  const Shape o = shape_from(output_dims);
+  REQUIRE(o.rank <= 8, "odla_ExpandDims: rank > 8");
+  Shape al = input->shape;
+  if (al.rank != o.rank)
+    REQUIRE(al.rank < o.rank && expand_like_reference(&al, o), "odla_ExpandDims: %s does not broadcast to %s",
+            input->shape.str().c_str(), o.str().c_str());
+  std::vector<int64_t> dims(o.d, o.d + o.rank), sx = row_major_strides(al), sy = row_major_strides(o);
+  for (int i = 0; i < o.rank; ++i) {
+    REQUIRE(al.d[i] == o.d[i] || al.d[i] == 1, "odla_ExpandDims: %s does not broadcast to %s",
+            input->shape.str().c_str(), o.str().c_str());
+    if (al.d[i] == 1) sx[i] = 0;
+  }
+  return copynd(c, input, o, dims, sx, sy, 0, 0, false, id);
+}
+
+// Removes the listed 1-sized dims (all of them when none is listed).
+// [ref: ops/odla_ops_process.h:397-412]
+odla_value odla_Squeeze(odla_value input, odla_size_t num_of_axes, const odla_uint32* axes, odla_value_shape,
+                        const odla_value_id id) {
+  REQUIRE(input && (axes || num_of_axes == 0), "odla_Squeeze: null argument");
+  const Shape& xs = input->shape;
+  bool drop[ODLA_MAX_DIMENSION] = {false};
+  for (odla_size_t i = 0; i < num_of_axes; ++i) {
+    REQUIRE((int)axes[i] < xs.rank && xs.d[axes[i]] == 1, "odla_Squeeze: axis %u of %s is not 1", axes[i], xs.str().c_str());
+    drop[axes[i]] = true;
+  }
+  Shape o;
+  for (int i = 0; i < xs.rank; ++i) {
+    const bool d = num_of_axes == 0 ? xs.d[i] == 1 : drop[i];
+    if (!d) o.d[o.rank++] = xs.d[i];
+  }
+  if (o.rank == 0) { o.rank = 1; o.d[0] = 1; }
+  return odla_Reshape(input, shape_to(o), id);
+}
+
+// Joins same-shaped values along a new axis.  [ref: ops/odla_ops_process.h:414-430]
+odla_value odla_Stack(odla_values inputs, odla_int32 axis, odla_value_shape, const odla_value_id id) {
+  REQUIRE(inputs.size >= 1 && inputs.size <= ODLA_MAX_OUTPUTS && inputs.values[0], "odla_Stack: bad operand list");
+  const Shape& xs = inputs.values[0]->shape;
+  if (axis < 0) axis += xs.rank + 1;
+  REQUIRE(axis >= 0 && axis <= xs.rank && xs.rank < ODLA_MAX_DIMENSION, "odla_Stack: axis out of range");
+  Shape one;
+  one.rank = xs.rank + 1;
+  for (int i = 0, j = 0; i < one.rank; ++i) one.d[i] = i == axis ? 1 : xs.d[j++];
+  odla_values parts;
+  parts.size = inputs.size;
+  for (odla_size_t i = 0; i < inputs.size; ++i) {
+    REQUIRE(inputs.values[i] && inputs.values[i]->shape == xs, "odla_Stack: operands differ in shape");
+    parts.values[i] = odla_Reshape(inputs.values[i], shape_to(one), nullptr);
+    if (parts.values[i] == nullptr) return nullptr;
+  }
+  return odla_Concat(parts, axis, undefined_shape(), id);
+}
+
+// K largest / smallest elements along `axis`, best first, and their indices.
+// [ref: ops/odla_ops_process.h (odla_TopK); dnnl odla_dnnl.cc:2064-2111]
+odla_values odla_TopK(odla_value input, odla_uint32 K, odla_bool largest, odla_bool sorted, odla_uint32 axis,
+                      odla_value_type output_value_type, odla_value_type output_value_index_type,
+                      const odla_value_ids value_ids) {
+  (void)sorted;  // results are always ordered
+  (void)output_value_type;
+  odla_values none;
+  none.size = 0;
+  auto bail = [&](const char* msg) { OHIP_ERR("odla_TopK: %s", msg); return none; };
+  if (input == nullptr) return bail("null operand");
+  _odla_computation* c = comp_of(input);
+  if (c == nullptr) return bail("no current computation");
+  if (!is_float_type(input->etype)) return bail("operand must be a float type");
+  const Shape& xs = input->shape;
+  if ((int)axis >= xs.rank) return bail("axis out of range");
+  if (K < 1 || (int64_t)K > xs.d[axis]) return bail("K out of range");
+  const odla_element_type it = output_value_index_type.element_type == ODLA_INT64 ? ODLA_INT64 : ODLA_INT32;
+  Shape o = xs;
+  o.d[axis] = K;
+  Node* n = add_node(c, OP_TOPK, {input}, input->etype, o, value_ids.size > 0 ? value_ids.value_ids[0] : nullptr);
+  n->out2 = new_value(c, _odla_value::TEMP, it, o, value_ids.size > 1 ? value_ids.value_ids[1] : nullptr);
+  n->out2->producer = n->out->producer;
+  n->i[0] = K;
+  n->i[1] = largest != 0;
+  n->i[2] = axis;
+  odla_values r;
+  r.size = 2;
+  r.values[0] = n->out;
+  r.values[1] = n->out2;
+  return r;
+}
+
+// [ref: ops/odla_ops_nn.h (odla_LRN); dnnl odla_dnnl.cc:1553-1581]
+odla_value odla_LRN(odla_value input, odla_memory_layout layout, odla_int32 window_size, odla_float32 alpha,
+                    odla_float32 beta, odla_float32 bias, const odla_value_id id) {
+  REQUIRE(input, "odla_LRN: null argument");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_LRN: no current computation");
+  REQUIRE(is_float_type(input->etype), "odla_LRN: operand must be a float type");
+  REQUIRE(input->shape.rank >= 3, "odla_LRN: rank < 3");
+  REQUIRE(window_size >= 1 && (window_size & 1), "odla_LRN: the window must be odd");
+  Node* n = add_node(c, OP_LRN, {input}, input->etype, input->shape, id);
+  n->i[0] = layout == ODLA_CHANNELS_LAST ? ODLA_CHANNELS_LAST : ODLA_CHANNELS_FIRST;
+  n->i[1] = window_size;
+  n->f[0] = alpha; n->f[1] = beta; n->f[2] = bias;
+  return n->out;
+}
+
+// Normalisation over the spatial dims of every (sample, channel) pair.
+// [ref: ops/odla_ops_nn.h (odla_InstanceNormalization); dnnl odla_dnnl.cc:1583-1626]
+odla_value odla_InstanceNormalization(odla_value input, odla_memory_layout layout, odla_float32 epsilon,
+                                      odla_value scale, odla_value offset, odla_float32 scalar_scale,
+                                      odla_float32 scalar_offset, const odla_value_id id) {
+  REQUIRE(input, "odla_InstanceNormalization: null argument");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_InstanceNormalization: no current computation");
+  REQUIRE(is_float_type(input->etype), "odla_InstanceNormalization: operand must be a float type");
+  const Shape& xs = input->shape;
+  REQUIRE(xs.rank >= 3, "odla_InstanceNormalization: rank < 3");
+  const bool cl = layout == ODLA_CHANNELS_LAST;
+  const int64_t C = cl ? xs.d[xs.rank - 1] : xs.d[1];
+  if (scale) REQUIRE(scale->kind == _odla_value::CONSTANT && scale->shape.numel() == C,
+                     "odla_InstanceNormalization: scale must be a constant with one element per channel");
+  if (offset) REQUIRE(offset->kind == _odla_value::CONSTANT && offset->shape.numel() == C,
+                      "odla_InstanceNormalization: offset must be a constant with one element per channel");
+  Node* n = add_node(c, OP_ROWNORM, {input, scale, offset}, input->etype, xs, id);
+  n->i[0] = cl ? ODLA_CHANNELS_LAST : ODLA_CHANNELS_FIRST;
+  n->f[0] = epsilon; n->f[1] = scalar_scale; n->f[2] = scalar_offset;
+  return n->out;
+}
+
+// Transposed convolution, rewritten as a stride-1 convolution of the
+// zero-stuffed input with the flipped, in/out-swapped kernel.
+// [ref: ops/odla_ops_nn.h (odla_DeConv); dnnl odla_dnnl.cc:1131-1232]
+odla_value odla_DeConv(odla_value input, odla_memory_layout input_layout, odla_uint32 group, odla_value kernel,
+                       odla_memory_layout kernel_layout, const odla_uint32* strides, const odla_uint32* dilations,
+                       const odla_uint32* paddings_front, const odla_uint32* paddings_back, odla_value bias,
+                       odla_value_shape output_dims, const odla_value_id id) {
+  REQUIRE(input && kernel && strides && dilations && paddings_front && paddings_back, "odla_DeConv: null argument");
+  _odla_computation* c = comp_of(input, kernel);
+  REQUIRE(c, "odla_DeConv: no current computation");
+  REQUIRE(input->shape.rank == 4 && kernel->shape.rank == 4, "odla_DeConv: only 2-D is supported");
+  REQUIRE(input_layout != ODLA_CHANNELS_LAST, "odla_DeConv: channels-last input is not supported");
+  REQUIRE(kernel->kind == _odla_value::CONSTANT && kernel->host_data != nullptr, "odla_DeConv: the kernel must be a constant");
+  REQUIRE(kernel->etype == ODLA_FLOAT32, "odla_DeConv: the kernel must be FLOAT32");
+  REQUIRE(dilations[0] == 1 && dilations[1] == 1, "odla_DeConv: dilation is not supported");
+  REQUIRE(strides[0] >= 1 && strides[1] >= 1, "odla_DeConv: bad stride");
+  if (group == 0) group = 1;
+  const Shape& x = input->shape;
+  const Shape& k = kernel->shape;
+  // element (o_in_group, c, r, s) of the kernel, c = input channel, o = output channel within its group
+  int64_t Cin, Og, R, S, so, sc, sr, ss;
+  switch (kernel_layout) {
+    case ODLA_IOS: Cin = k.d[0]; Og = k.d[1]; R = k.d[2]; S = k.d[3]; sc = Og * R * S; so = R * S; sr = S; ss = 1; break;
+    case ODLA_SIO: R = k.d[0]; S = k.d[1]; Cin = k.d[2]; Og = k.d[3]; sr = S * Cin * Og; ss = Cin * Og; sc = Og; so = 1; break;
+    case ODLA_SOI: R = k.d[0]; S = k.d[1]; Og = k.d[2]; Cin = k.d[3]; sr = S * Cin * Og; ss = Cin * Og; so = Cin; sc = 1; break;
+    default: Og = k.d[0]; Cin = k.d[1]; R = k.d[2]; S = k.d[3]; so = Cin * R * S; sc = R * S; sr = S; ss = 1; break;
+  }
+  const int64_t N = x.d[0], C = x.d[1], H = x.d[2], W = x.d[3];
+  REQUIRE(C == Cin && C % group == 0, "odla_DeConv: input channels %lld do not match the kernel (%lld, group %u)",
+          (long long)C, (long long)Cin, group);
+  const int64_t O = Og * group, Cg = C / group;
+  const int64_t st[2] = {strides[0], strides[1]}, KS[2] = {R, S}, IN[2] = {H, W};
+  int64_t out_hw[2], pf[2], pb[2], up[2];
+  for (int d = 0; d < 2; ++d) {
+    up[d] = (IN[d] - 1) * st[d] + 1;
+    int64_t want = up[d] + KS[d] - 1 - (int64_t)paddings_front[d] - (int64_t)paddings_back[d];
+    if (shape_valid(output_dims) && output_dims.size == 4 && output_dims.dims[2 + d] >= want &&
+        output_dims.dims[2 + d] < want + st[d])
+      want = output_dims.dims[2 + d];  // output padding
+    out_hw[d] = want;
+    pf[d] = KS[d] - 1 - (int64_t)paddings_front[d];
+    pb[d] = want - (up[d] + pf[d] - KS[d] + 1);
+    REQUIRE(pf[d] >= 0 && pb[d] >= 0 && want > 0, "odla_DeConv: padding larger than the kernel is not supported");
+  }
+  if (bias) REQUIRE(bias->shape.numel() == O, "odla_DeConv: bias has %lld elements, expected %lld",
+                    (long long)bias->shape.numel(), (long long)O);
+  // flipped kernel in OIHW order with per-group input channels
+  auto buf = std::make_unique<std::vector<uint8_t>>((size_t)(O * Cg * R * S) * sizeof(float));
+  float* wf = reinterpret_cast<float*>(buf->data());
+  const float* w = static_cast<const float*>(kernel->host_data);
+  for (int64_t g = 0; g < group; ++g)
+    for (int64_t oi = 0; oi < Og; ++oi)
+      for (int64_t ci = 0; ci < Cg; ++ci)
+        for (int64_t r = 0; r < R; ++r)
+          for (int64_t s = 0; s < S; ++s)
+            wf[(((g * Og + oi) * Cg + ci) * R + r) * S + s] =
+                w[oi * so + (g * Cg + ci) * sc + (R - 1 - r) * sr + (S - 1 - s) * ss];
+  Shape ks;
+  ks.rank = 4;
+  ks.d[0] = O; ks.d[1] = Cg; ks.d[2] = R; ks.d[3] = S;
+  odla_value kf = new_value(c, _odla_value::CONSTANT, ODLA_FLOAT32, ks, nullptr);
+  kf->host_data = wf;
+  c->owned_data.push_back(std::move(buf));
+  // zero-stuffed input
+  odla_value xu = input;
+  if (st[0] > 1 || st[1] > 1) {
+    Shape us = x;
+    us.d[2] = up[0]; us.d[3] = up[1];
+    std::vector<int64_t> dims(x.d, x.d + 4), sx = row_major_strides(x), sy = row_major_strides(us);
+    sy[2] *= st[0];
+    sy[3] *= st[1];
+    xu = copynd(c, input, us, dims, sx, sy, 0, 0, true, nullptr);
+  }
+  Shape o;
+  o.rank = 4;
+  o.d[0] = N; o.d[1] = O; o.d[2] = out_hw[0]; o.d[3] = out_hw[1];
+  Node* n = add_node(c, OP_CONV, {xu, kf, bias}, input->etype, o, id);
+  n->i[0] = ODLA_CHANNELS_FIRST;
+  n->i[1] = group;
+  n->i[2] = ODLA_OIS;
+  n->i[3] = 1; n->i[4] = 1;
+  n->i[5] = 1; n->i[6] = 1;
+  n->i[7] = pf[0]; n->i[8] = pf[1];
+  n->i[9] = pb[0]; n->i[10] = pb[1];
+  return n->out;
 }
 
 odla_value odla_NMS(odla_value boxes, odla_value scores, odla_uint32 max_num_outputs,

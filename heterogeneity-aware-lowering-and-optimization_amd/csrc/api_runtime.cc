@@ -44,7 +44,7 @@ void log_msg(const char* file, int line, const char* func, odla_log_level lvl, c
 const char* op_name(OpKind k) {
   static const char* names[] = {"Conv", "Gemm", "Binary", "Unary", "BatchNorm", "LayerNorm", "Pool",
                                 "Reduce", "Softmax", "Cast", "Concat", "Gather", "Reshape", "Resize",
-                                "Slice", "Transpose", "Quantize", "Dequantize", "NMS"};
+                                "Slice", "Transpose", "Quantize", "Dequantize", "NMS", "Elementwise", "ArgExtreme", "CopyND", "TopK", "LRN", "RowNorm"};
   return names[(int)k];
 }
 

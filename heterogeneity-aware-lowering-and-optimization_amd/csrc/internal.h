@@ -34,7 +34,7 @@ void log_msg(const char* file, int line, const char* func, odla_log_level lvl, c
 enum OpKind : int {
   OP_CONV, OP_GEMM, OP_BINARY, OP_UNARY, OP_BATCHNORM, OP_LAYERNORM, OP_POOL, OP_REDUCE,
   OP_SOFTMAX, OP_CAST, OP_CONCAT, OP_GATHER, OP_RESHAPE, OP_RESIZE, OP_SLICE, OP_TRANSPOSE,
-  OP_QUANTIZE, OP_DEQUANTIZE, OP_NMS
+  OP_QUANTIZE, OP_DEQUANTIZE, OP_NMS, OP_EWISE, OP_ARGEXT, OP_COPYND, OP_TOPK, OP_LRN, OP_ROWNORM
 };
 const char* op_name(OpKind k);
 
@@ -84,6 +84,7 @@ struct Node {
   OpKind op;
   std::vector<_odla_value*> in;  // nullptr entries allowed for optional operands
   _odla_value* out = nullptr;
+  _odla_value* out2 = nullptr;  // second result (TopK indices)
   // attributes (meaning depends on op; see api_ops.cc)
   int64_t i[24] = {0};
   float f[8] = {0};

@@ -106,6 +106,29 @@ __device__ __forceinline__ float apply_act(float v, ActKind act, float a, float 
     case ACT_NEG: return -v;
     case ACT_ROUND: return rintf(v);
     case ACT_RECIP: return 1.0f / v;
+    case ACT_CEIL: return ceilf(v);
+    case ACT_FLOOR: return floorf(v);
+    case ACT_SIGN: return v > 0.f ? 1.f : (v < 0.f ? -1.f : v);
+    case ACT_SIN: return sinf(v);
+    case ACT_COS: return cosf(v);
+    case ACT_TAN: return tanf(v);
+    case ACT_ASIN: return asinf(v);
+    case ACT_ACOS: return acosf(v);
+    case ACT_ATAN: return atanf(v);
+    case ACT_SINH: return sinhf(v);
+    case ACT_COSH: return coshf(v);
+    case ACT_ASINH: return asinhf(v);
+    case ACT_ACOSH: return acoshf(v);
+    case ACT_ATANH: return atanhf(v);
+    case ACT_ELU: return v > 0.f ? v : a * expm1f(v);
+    case ACT_SELU: return b * (v > 0.f ? v : a * expm1f(v));
+    case ACT_CELU: return fmaxf(v, 0.f) + fminf(0.f, a * expm1f(v / a));
+    case ACT_HARDSIGMOID: return fminf(fmaxf(a * v + b, 0.f), 1.f);
+    case ACT_SOFTPLUS: return logf(expf(v) + 1.0f);
+    case ACT_SOFTSIGN: return v / (fabsf(v) + 1.0f);
+    case ACT_THRESHOLDED: return v > a ? v : 0.f;
+    case ACT_SHRINK: return v > b ? v - a : (v < -b ? v + a : 0.f);
+    case ACT_DIV_CONST: return v / a;
   }
   return v;
 }

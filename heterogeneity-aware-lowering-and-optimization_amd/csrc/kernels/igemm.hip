@@ -1165,10 +1165,17 @@ __global__ void pack_weights_kernel(PackWeightsParams p) {
     const int c = col - tap * p.Cp;
     TD out;
     __builtin_memset(&out, 0, sizeof(TD));
-    if (o < p.Og && tap < taps && c < p.Cg) {
+    bool live = o < p.Og && tap < taps && c < p.Cg;
+    int cs = c;
+    if (p.dense_groups > 0) {
+      const int cg = p.Cg / p.dense_groups;
+      cs = c - (o / (p.Og / p.dense_groups)) * cg;
+      live = live && cs >= 0 && cs < cg;
+    }
+    if (live) {
       const int r = tap / p.S, s = tap - r * p.S;
       const int64_t og = (int64_t)g * p.Og + o;
-      const TS v = reinterpret_cast<const TS*>(p.src)[og * p.so + c * p.si + r * p.sr + s * p.ss];
+      const TS v = reinterpret_cast<const TS*>(p.src)[og * p.so + cs * p.si + r * p.sr + s * p.ss];
       out = cvt_weight<TS, TD>(v);
     }
     reinterpret_cast<TD*>(p.dst)[i] = out;
@@ -1178,6 +1185,8 @@ __global__ void pack_weights_kernel(PackWeightsParams p) {
 hipError_t launch_pack_weights(const PackWeightsParams& p, hipStream_t stream) {
   if (p.src == nullptr || p.dst == nullptr) return hipErrorInvalidValue;
   if (p.G <= 0 || p.Og <= 0 || p.Cg <= 0 || p.Cp < p.Cg || p.rows_pad < p.Og) return hipErrorInvalidValue;
+  if (p.dense_groups < 0 || (p.dense_groups > 0 && (p.G != 1 || p.Og % p.dense_groups || p.Cg % p.dense_groups)))
+    return hipErrorInvalidValue;
   if ((int64_t)p.R * p.S * p.Cp > p.w_rs) return hipErrorInvalidValue;
   const int64_t total = (int64_t)p.G * p.rows_pad * p.w_rs;
   const int grid = grid_for(total, 256);

@@ -40,7 +40,18 @@ inline bool dtype_is_float(DType t) { return t == DT_F32 || t == DT_F16 || t == 
 enum ActKind : int {
   ACT_NONE = 0, ACT_RELU, ACT_LEAKY, ACT_CLAMP, ACT_SIGMOID, ACT_TANH,
   ACT_GELU_ERF, ACT_GELU_TANH, ACT_EXP, ACT_LOG, ACT_SQRT, ACT_RSQRT, ACT_ERF,
-  ACT_ABS, ACT_NEG, ACT_ROUND, ACT_RECIP
+  ACT_ABS, ACT_NEG, ACT_ROUND, ACT_RECIP,
+  ACT_CEIL, ACT_FLOOR, ACT_SIGN, ACT_SIN, ACT_COS, ACT_TAN, ACT_ASIN, ACT_ACOS, ACT_ATAN,
+  ACT_SINH, ACT_COSH, ACT_ASINH, ACT_ACOSH, ACT_ATANH,
+  ACT_ELU,          // x > 0 ? x : a * (exp(x) - 1)
+  ACT_SELU,         // b * elu(x, a)
+  ACT_CELU,         // max(0, x) + min(0, a * (exp(x / a) - 1))
+  ACT_HARDSIGMOID,  // clamp(a * x + b, 0, 1)
+  ACT_SOFTPLUS,     // log(exp(x) + 1)
+  ACT_SOFTSIGN,     // x / (|x| + 1)
+  ACT_THRESHOLDED,  // x > a ? x : 0
+  ACT_SHRINK,       // x > b ? x - a : (x < -b ? x + a : 0)
+  ACT_DIV_CONST     // x / a
 };
 
 enum BinKind : int { BIN_ADD = 0, BIN_SUB, BIN_MUL, BIN_DIV, BIN_MAX, BIN_MIN };
@@ -127,6 +138,10 @@ struct PackWeightsParams {
   DType src_dt = DT_F32, dst_dt = DT_F32;
   int G = 1, Og = 0, Cg = 0, R = 1, S = 1;  // per-group out / in channels
   int Cp = 0;                               // padded in-channels per tap (>= Cg)
+  // dense_groups > 0 (with G == 1): the source holds that many groups of
+  // Og / dense_groups rows with Cg / dense_groups in-channels each; the result
+  // is the block-diagonal matrix of the equivalent ungrouped convolution.
+  int dense_groups = 0;
   int rows_pad = 0, w_rs = 0;
   int64_t so = 0, si = 0, sr = 0, ss = 0;
 };
@@ -203,6 +218,33 @@ struct BinaryParams {
 };
 hipError_t launch_binary(const BinaryParams& p, hipStream_t stream);
 
+// Typed element-wise operators with broadcast (row-major operands, up to 6
+// collapsed dims, one element stride per dim and operand, 0 where it
+// broadcasts).  EW_ADD .. EW_SQDIFF: y has the operands' type `dt` (float types
+// and integers).  EW_EQ .. EW_GE: operands of type dt, boolean result.
+// EW_AND .. EW_NOT: boolean operands and result.  EW_ISNAN ..: float operand,
+// boolean result.  EW_SELECT: y = a ? b : c with a boolean, b / c / y of type dt.
+enum EwiseOp : int {
+  EW_ADD = 0, EW_SUB, EW_MUL, EW_DIV, EW_MAX, EW_MIN, EW_POW,
+  EW_MOD,    // a - b * floor(a / b)
+  EW_FMOD,   // a - b * trunc(a / b)
+  EW_PRELU,  // a < 0 ? a * b : a
+  EW_SQDIFF, // (a - b)^2
+  EW_SELECT,
+  EW_EQ, EW_NE, EW_LT, EW_LE, EW_GT, EW_GE,
+  EW_AND, EW_OR, EW_XOR, EW_NOT,
+  EW_ISNAN, EW_ISINF, EW_ISINF_POS, EW_ISINF_NEG
+};
+struct EwiseParams {
+  const void* a = nullptr; const void* b = nullptr; const void* c = nullptr; void* y = nullptr;
+  DType dt = DT_F32;
+  EwiseOp op = EW_ADD;
+  int rank = 1;
+  int64_t dims[6] = {1, 1, 1, 1, 1, 1};
+  int64_t sa[6] = {0}, sb[6] = {0}, sc[6] = {0};
+};
+hipError_t launch_ewise(const EwiseParams& p, hipStream_t stream);
+
 // ---------------------------------------------------------------------------
 // Pooling on channels-last tensors x[N][H][W][cs] -> y[N][Ho][Wo][ycs].
 struct PoolParams {
@@ -219,9 +261,17 @@ hipError_t launch_pool2d(const PoolParams& p, hipStream_t stream);
 
 // Row reductions / normalisations over a contiguous inner axis:
 // x viewed as [outer][len][inner]; one result column per (outer, inner).
-enum ReduceKind : int { RED_MEAN = 0, RED_SUM, RED_MAX };
+// RED_L1 = sum |x| + eps, RED_L2 = sqrt(sum x^2 + eps), RED_LOGSUM = log(sum x).
+enum ReduceKind : int {
+  RED_MEAN = 0, RED_SUM, RED_MAX, RED_MIN, RED_PROD, RED_L1, RED_L2, RED_SUMSQ, RED_LOGSUM
+};
 hipError_t launch_reduce(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
-                         int64_t len, int64_t inner, ReduceKind kind, hipStream_t stream);
+                         int64_t len, int64_t inner, ReduceKind kind, hipStream_t stream,
+                         float eps = 0.f);
+// Index (int32 / int64) of the largest or smallest element along the middle
+// axis; ties resolve to the first index, or to the last when `last` is set.
+hipError_t launch_arg_extreme(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
+                              int64_t len, int64_t inner, bool is_max, bool last, hipStream_t stream);
 // Mean over the middle axis of 8-bit levels (stored q-128): fp32 result
 // y = ((sum q - len*zp) / len) * scale.
 hipError_t launch_reduce_q8_mean(const void* x, float* y, int64_t outer, int64_t len, int64_t inner,
@@ -257,6 +307,24 @@ hipError_t launch_gather_rows(const void* x, const void* idx, DType idx_dt, void
                               int64_t outer, int64_t n_src_rows, int64_t n_idx,
                               int64_t row_bytes, hipStream_t stream);
 hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t stream);
+// Fills `bytes` (a multiple of 4) with a repeated 32-bit pattern.
+hipError_t launch_fill_bytes(void* p, size_t bytes, uint32_t pattern, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// TopK along the middle axis of x[outer][len][inner] -> vals / idxs
+// [outer][K][inner], best first, equal values by ascending index.
+hipError_t launch_topk(const void* x, void* vals, void* idxs, DType dt, DType idx_dt, int64_t outer,
+                       int64_t len, int64_t inner, int K, bool largest, hipStream_t stream);
+// LRN across the channels of x[N][C][inner]:
+// y = x / (bias + alpha / (2 half + 1) * sum_{|c'-c| <= half} x[c']^2) ^ beta
+hipError_t launch_lrn(const void* x, void* y, DType dt, int64_t N, int C, int64_t inner, int half, float alpha,
+                      float beta, float bias, hipStream_t stream);
+// Rows of x[rows][len] normalised to zero mean / unit (biased) variance, then
+// scaled by gamma[r % channels] and shifted by beta[r % channels] (scalars
+// sgamma / sbeta where the vectors are null).
+hipError_t launch_rownorm(const void* x, void* y, DType dt, int64_t rows, int64_t len, int channels,
+                          const float* gamma, const float* beta, float sgamma, float sbeta, float eps,
+                          hipStream_t stream);
 
 // ---------------------------------------------------------------------------
 // Batched NMS.  boxes [N][B][4] fp32 corners, scores [N][C][B] fp32.

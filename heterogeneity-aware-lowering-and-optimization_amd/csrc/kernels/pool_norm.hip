@@ -173,24 +173,51 @@ __global__ void __launch_bounds__(kThreads) pool2d_q8_kernel(PoolParams p) {
 
 // --------------------------------------------------------------------------
 // Reduction over the middle axis of [outer][len][inner].
+__device__ __forceinline__ float red_init(ReduceKind k) {
+  return k == RED_MAX ? -INFINITY : (k == RED_MIN ? INFINITY : (k == RED_PROD ? 1.f : 0.f));
+}
+__device__ __forceinline__ float red_step(float acc, float v, ReduceKind k) {
+  switch (k) {
+    case RED_MAX: return fmaxf(acc, v);
+    case RED_MIN: return fminf(acc, v);
+    case RED_PROD: return acc * v;
+    case RED_L1: return acc + fabsf(v);
+    case RED_L2: case RED_SUMSQ: return acc + v * v;
+    default: return acc + v;
+  }
+}
+__device__ __forceinline__ float red_merge(float a, float b, ReduceKind k) {
+  switch (k) {
+    case RED_MAX: return fmaxf(a, b);
+    case RED_MIN: return fminf(a, b);
+    case RED_PROD: return a * b;
+    default: return a + b;
+  }
+}
+__device__ __forceinline__ float red_final(float acc, int64_t len, ReduceKind k, float eps) {
+  switch (k) {
+    case RED_MEAN: return acc / (float)len;
+    case RED_L1: return acc + eps;
+    case RED_L2: return sqrtf(acc + eps);
+    case RED_LOGSUM: return logf(acc);
+    default: return acc;
+  }
+}
 // inner == 1: one wavefront per row, lanes stride the row.
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(kThreads)
 reduce_rows_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, int64_t len,
-                   ReduceKind kind) {
+                   ReduceKind kind, float eps) {
   const int lane = threadIdx.x & 63;
   const int64_t wave = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) >> 6;
   const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
   for (int64_t r = wave; r < rows; r += nwaves) {
     const TI* row = x + r * len;
-    float acc = kind == RED_MAX ? -INFINITY : 0.f;
-    for (int64_t i = lane; i < len; i += 64) {
-      const float v = Store<TI>::ld(row + i);
-      acc = kind == RED_MAX ? fmaxf(acc, v) : acc + v;
-    }
-    acc = kind == RED_MAX ? wave_max(acc) : wave_sum(acc);
-    if (kind == RED_MEAN) acc /= (float)len;
-    if (lane == 0) Store<TO>::st(y + r, acc);
+    float acc = red_init(kind);
+    for (int64_t i = lane; i < len; i += 64) acc = red_step(acc, Store<TI>::ld(row + i), kind);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc = red_merge(acc, __shfl_xor(acc, o, 64), kind);
+    if (lane == 0) Store<TO>::st(y + r, red_final(acc, len, kind, eps));
   }
 }
 // inner > 1: one thread per (outer, inner) column; consecutive threads read
@@ -198,19 +225,15 @@ reduce_rows_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(kThreads)
 reduce_cols_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int64_t len,
-                   int64_t inner, ReduceKind kind) {
+                   int64_t inner, ReduceKind kind, float eps) {
   const int64_t total = outer * inner;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t o = i / inner, in = i - o * inner;
     const TI* col = x + o * len * inner + in;
-    float acc = kind == RED_MAX ? -INFINITY : 0.f;
-    for (int64_t k = 0; k < len; ++k) {
-      const float v = Store<TI>::ld(col + k * inner);
-      acc = kind == RED_MAX ? fmaxf(acc, v) : acc + v;
-    }
-    if (kind == RED_MEAN) acc /= (float)len;
-    Store<TO>::st(y + i, acc);
+    float acc = red_init(kind);
+    for (int64_t k = 0; k < len; ++k) acc = red_step(acc, Store<TI>::ld(col + k * inner), kind);
+    Store<TO>::st(y + i, red_final(acc, len, kind, eps));
   }
 }
 // inner % V == 0: one thread per (outer, 16-byte group of inner positions); every
@@ -218,7 +241,7 @@ reduce_cols_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, 
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(kThreads)
 reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int64_t len,
-                       int64_t inner, ReduceKind kind) {
+                       int64_t inner, ReduceKind kind, float eps) {
   constexpr int V = Vec16<TI>::N;
   const int64_t iv = inner / V;
   const int64_t total = outer * iv;
@@ -228,7 +251,7 @@ reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t out
     const TI* col = x + o * len * inner + in;
     float acc[V];
 #pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = kind == RED_MAX ? -INFINITY : 0.f;
+    for (int e = 0; e < V; ++e) acc[e] = red_init(kind);
     int64_t k = 0;
     for (; k + 4 <= len; k += 4) {
       Vec16<TI> v[4];
@@ -237,20 +260,36 @@ reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t out
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc[e] = kind == RED_MAX ? fmaxf(acc[e], v[u].get(e)) : acc[e] + v[u].get(e);
+        for (int e = 0; e < V; ++e) acc[e] = red_step(acc[e], v[u].get(e), kind);
     }
     for (; k < len; ++k) {
       Vec16<TI> v;
       v.load(col + k * inner);
 #pragma unroll
-      for (int e = 0; e < V; ++e) acc[e] = kind == RED_MAX ? fmaxf(acc[e], v.get(e)) : acc[e] + v.get(e);
+      for (int e = 0; e < V; ++e) acc[e] = red_step(acc[e], v.get(e), kind);
     }
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      float r = acc[e];
-      if (kind == RED_MEAN) r /= (float)len;
-      Store<TO>::st(y + o * inner + in + e, r);
+    for (int e = 0; e < V; ++e) Store<TO>::st(y + o * inner + in + e, red_final(acc[e], len, kind, eps));
+  }
+}
+// Index of the extreme value along the middle axis; one thread per (outer,
+// inner) column.  Ties keep the first index, or the last when `last` is set.
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(kThreads)
+arg_extreme_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int64_t len,
+                   int64_t inner, bool is_max, bool last) {
+  const int64_t total = outer * inner;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t o = i / inner, in = i - o * inner;
+    const TI* col = x + o * len * inner + in;
+    float val = Store<TI>::ld(col);
+    int64_t idx = 0;
+    for (int64_t k = 1; k < len; ++k) {
+      const float cur = Store<TI>::ld(col + k * inner);
+      if ((is_max && cur > val) || (!is_max && cur < val) || (cur == val && last)) { val = cur; idx = k; }
     }
+    y[i] = (TO)idx;
   }
 }
 // Quantised mean over the middle axis: y = ((sum - len*zp) / len) * scale (fp32).
@@ -616,21 +655,21 @@ hipError_t launch_reduce_q8_mean(const void* x, float* y, int64_t outer, int64_t
 
 template <typename TI>
 static hipError_t reduce_out(const void* x, void* y, DType out_dt, int64_t outer, int64_t len,
-                             int64_t inner, ReduceKind kind, hipStream_t stream) {
+                             int64_t inner, ReduceKind kind, float eps, hipStream_t stream) {
   auto go = [&](auto tag) -> hipError_t {
     using TO = decltype(tag);
     if (inner == 1) {
       const int grid = grid_for(outer * 64, kThreads);
       hipLaunchKernelGGL((reduce_rows_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
-                         (const TI*)x, (TO*)y, outer, len, kind);
+                         (const TI*)x, (TO*)y, outer, len, kind, eps);
     } else if (inner % (16 / (int)sizeof(TI)) == 0 && al16(x)) {
       const int grid = grid_for(outer * (inner / (16 / (int)sizeof(TI))), kThreads);
       hipLaunchKernelGGL((reduce_cols_vec_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
-                         (const TI*)x, (TO*)y, outer, len, inner, kind);
+                         (const TI*)x, (TO*)y, outer, len, inner, kind, eps);
     } else {
       const int grid = grid_for(outer * inner, kThreads);
       hipLaunchKernelGGL((reduce_cols_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
-                         (const TI*)x, (TO*)y, outer, len, inner, kind);
+                         (const TI*)x, (TO*)y, outer, len, inner, kind, eps);
     }
     return hipGetLastError();
   };
@@ -641,14 +680,29 @@ static hipError_t reduce_out(const void* x, void* y, DType out_dt, int64_t outer
 }
 
 hipError_t launch_reduce(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
-                         int64_t len, int64_t inner, ReduceKind kind, hipStream_t stream) {
+                         int64_t len, int64_t inner, ReduceKind kind, hipStream_t stream, float eps) {
   if (!x || !y || outer <= 0 || len <= 0 || inner <= 0) return hipErrorInvalidValue;
   switch (in_dt) {
-    case DT_F32: return reduce_out<float>(x, y, out_dt, outer, len, inner, kind, stream);
-    case DT_F16: return reduce_out<f16_t>(x, y, out_dt, outer, len, inner, kind, stream);
-    case DT_BF16: return reduce_out<bf16_t>(x, y, out_dt, outer, len, inner, kind, stream);
+    case DT_F32: return reduce_out<float>(x, y, out_dt, outer, len, inner, kind, eps, stream);
+    case DT_F16: return reduce_out<f16_t>(x, y, out_dt, outer, len, inner, kind, eps, stream);
+    case DT_BF16: return reduce_out<bf16_t>(x, y, out_dt, outer, len, inner, kind, eps, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t launch_arg_extreme(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
+                              int64_t len, int64_t inner, bool is_max, bool last, hipStream_t stream) {
+  if (!x || !y || outer <= 0 || len <= 0 || inner <= 0) return hipErrorInvalidValue;
+  if (out_dt != DT_I32 && out_dt != DT_I64) return hipErrorInvalidValue;
+  const int grid = grid_for(outer * inner, kThreads);
+  if (out_dt == DT_I32) {
+    FLOAT_DISPATCH(in_dt, hipLaunchKernelGGL((arg_extreme_kernel<T, int32_t>), dim3(grid), dim3(kThreads), 0, stream,
+                                             (const T*)x, (int32_t*)y, outer, len, inner, is_max, last));
+  } else {
+    FLOAT_DISPATCH(in_dt, hipLaunchKernelGGL((arg_extreme_kernel<T, int64_t>), dim3(grid), dim3(kThreads), 0, stream,
+                                             (const T*)x, (int64_t*)y, outer, len, inner, is_max, last));
+  }
+  return hipGetLastError();
 }
 
 template <typename TI, typename TO>

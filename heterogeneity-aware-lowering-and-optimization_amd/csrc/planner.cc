@@ -453,14 +453,21 @@ class Planner {
   void lower_transpose(int ni);
   void lower_qdq(int ni);
   void lower_nms(int ni);
+  void lower_ewise(int ni);
+  void lower_argext(int ni);
+  void lower_copynd(int ni);
+  void lower_topk(int ni);
+  void lower_lrn(int ni);
+  void lower_rownorm(int ni);
 
   void collect_epilogue(int ni, int64_t out_channels, int channel_axis_of_output, Epilogue* ep);
   bool per_channel_constant(const _odla_value* k, const Shape& aligned, const Shape& out, int ch_axis,
                             int64_t channels, std::vector<float>* vals);
   void bn_params_host(const Node& n, int64_t C, std::vector<float>* scale, std::vector<float>* shift);
+  // dense_groups > 0: G is 1, Og / Cg are the totals and the kernel holds that many groups
   int pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og, int Cg, int R, int S, int Cp,
                    int64_t so, int64_t si, int64_t sr, int64_t ss, const std::vector<float>& row_scale,
-                   int* w_rs_out, const std::vector<float>* wq_scale);
+                   int* w_rs_out, const std::vector<float>* wq_scale, int dense_groups = 0);
   int make_wfrag(const std::string& name, IgemmParams* ip, int tw);
   void finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty, const Epilogue& ep,
                     int64_t Kout_total);
@@ -619,6 +626,12 @@ void Planner::lower(int ni) {
     case OP_TRANSPOSE: lower_transpose(ni); break;
     case OP_QUANTIZE: case OP_DEQUANTIZE: lower_qdq(ni); break;
     case OP_NMS: lower_nms(ni); break;
+    case OP_EWISE: lower_ewise(ni); break;
+    case OP_ARGEXT: lower_argext(ni); break;
+    case OP_COPYND: lower_copynd(ni); break;
+    case OP_TOPK: lower_topk(ni); break;
+    case OP_LRN: lower_lrn(ni); break;
+    case OP_ROWNORM: lower_rownorm(ni); break;
   }
 }
 
@@ -761,7 +774,7 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
 int Planner::pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og, int Cg, int R, int S,
                           int Cp, int64_t so, int64_t si, int64_t sr, int64_t ss,
                           const std::vector<float>& row_scale, int* w_rs_out,
-                          const std::vector<float>* wq_scale) {
+                          const std::vector<float>* wq_scale, int dense_groups) {
   const int es = dtype_size(dst_dt);
   const int bk = 64 / es;
   const int w_rs = round_up_i(R * S * Cp, bk);
@@ -774,6 +787,8 @@ int Planner::pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og
   pp.rows_pad = Og; pp.w_rs = w_rs;
   pp.so = so; pp.si = si; pp.sr = sr; pp.ss = ss;
   pp.dst_dt = dst_dt;
+  pp.dense_groups = dense_groups;
+  const int64_t Ci = dense_groups > 0 ? Cg / dense_groups : Cg;  // in-channels per output row in the source
 
   if (kernel->kind == _odla_value::CONSTANT) {
     const int64_t n = kernel->shape.numel();
@@ -788,7 +803,7 @@ int Planner::pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og
       // element (o,i,r,s) at o*so + i*si + r*sr + s*ss
       for (int64_t o = 0; o < O; ++o) {
         const float s = (*wq_scale)[o];
-        for (int64_t i = 0; i < Cg; ++i)
+        for (int64_t i = 0; i < Ci; ++i)
           for (int r = 0; r < R; ++r)
             for (int t = 0; t < S; ++t) {
               const int64_t idx = o * so + i * si + r * sr + t * ss;
@@ -804,7 +819,7 @@ int Planner::pack_weights(const _odla_value* kernel, DType dst_dt, int G, int Og
       std::vector<float> w = const_as_float(kernel);
       const int64_t O = (int64_t)G * Og;
       for (int64_t o = 0; o < O; ++o)
-        for (int64_t i = 0; i < Cg; ++i)
+        for (int64_t i = 0; i < Ci; ++i)
           for (int r = 0; r < R; ++r)
             for (int t = 0; t < S; ++t) w[o * so + i * si + r * sr + t * ss] *= row_scale[o];
       std::vector<uint8_t> bytes((size_t)n * 4);
@@ -1186,27 +1201,33 @@ void Planner::lower_conv(int ni) {
     xcs = T(tx).cs;
   }
   if (T(tx).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "conv input storage type mismatch");
+  // Groups with fewer channels than one 16-byte K vector run as one dense
+  // convolution over block-diagonal weights (zero outside each group's block).
+  const bool densify = G > 1 && Cg % vec != 0;
+  const int Ge = densify ? 1 : G, Oge = densify ? (int)O : Og;
   int Cp;
-  if (G == 1) {
+  if (Ge == 1) {
     if (xcs % vec != 0) fail(ODLA_UNSUPPORTED_OP, "channels-last convolution input with %d channels needs a multiple of %d", xcs, vec);
     Cp = xcs;
   } else {
-    if (Cg % vec != 0) fail(ODLA_UNSUPPORTED_OP, "grouped convolution with %d channels per group (needs a multiple of %d)", Cg, vec);
     Cp = Cg;
   }
   int w_rs = 0;
-  const int tw = pack_weights(kpack, dt, G, Og, Cg, (int)R, (int)S, Cp, so, si, sr, ss, ep.row_scale, &w_rs, nullptr);
+  const int tw = densify ? pack_weights(kpack, dt, 1, (int)O, (int)C, (int)R, (int)S, Cp, so, si, sr, ss, ep.row_scale,
+                                        &w_rs, nullptr, G)
+                         : pack_weights(kpack, dt, G, Og, Cg, (int)R, (int)S, Cp, so, si, sr, ss, ep.row_scale, &w_rs,
+                                        nullptr);
 
   IgemmParams ip;
   ip.N = (int)N; ip.H = (int)H; ip.W = (int)W; ip.C = Cp; ip.xcs = xcs;
-  ip.Ho = (int)Ho; ip.Wo = (int)Wo; ip.Kout = Og;
+  ip.Ho = (int)Ho; ip.Wo = (int)Wo; ip.Kout = Oge;
   ip.R = (int)R; ip.S = (int)S; ip.sh = str_h; ip.sw = str_w;
   ip.dh = dil_h; ip.dw = dil_w; ip.ph = pad_t; ip.pw = pad_l;
-  ip.w_rows = Og; ip.w_cols = w_rs; ip.w_rs = w_rs;
+  ip.w_rows = Oge; ip.w_cols = w_rs; ip.w_rs = w_rs;
   ip.in_dt = dt; ip.out_dt = dt;
-  ip.batch = G;
+  ip.batch = Ge;
   ip.alpha = ep.scalar;
-  if (G > 1) { ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og; }
+  if (Ge > 1) { ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og; }
   ip.ycs = (int)O;
 
   int ty;
@@ -1527,6 +1548,75 @@ void Planner::lower_binary(int ni) {
   set_main(outv, ty);
 }
 
+// ------------------------------------------------- typed element-wise ----
+// Integer arithmetic, comparisons, logic, predicates and Select: row-major
+// operands, broadcast through per-dim element strides.
+void Planner::lower_ewise(int ni) {
+  Node& n = comp_->nodes[ni];
+  const Shape& os = n.out->shape;
+  const int r = (int)n.iv[0];
+  const int nin = (int)n.in.size();
+  const EwiseOp op = (EwiseOp)n.i[0];
+  int tin[3] = {-1, -1, -1};
+  int64_t st[3][ODLA_MAX_DIMENSION] = {{0}};
+  for (int k = 0; k < nin; ++k) {
+    tin[k] = get(n.in[k], L_ROWMAJOR, FORM_FLOAT);
+    int64_t acc = 1;
+    for (int i = r - 1; i >= 0; --i) {
+      const int64_t d = n.iv[1 + k * r + i];
+      st[k][i] = d == 1 ? 0 : acc;
+      acc *= d;
+    }
+  }
+  const DType odt = storage_dtype(n.out);
+  // element type of the typed operands (Select: of the two branches)
+  const DType dt = T(tin[op == EW_SELECT ? 1 : 0]).dt;
+  for (int k = (op == EW_SELECT ? 1 : 0); k < nin; ++k)
+    if (T(tin[k]).dt != dt) fail(ODLA_UNSUPPORTED_DATATYPE, "mixed storage types in element-wise op '%s'", n.out->name.c_str());
+  const int ty = new_tensor(odt, L_ROWMAJOR, os, 0, SP_ARENA);
+  EwiseParams ep;
+  ep.dt = dt;
+  ep.op = op;
+  {
+    // merge adjacent dims that are contiguous in every operand
+    std::vector<int64_t> d, x[3];
+    for (int i = 0; i < r; ++i) {
+      if (os.d[i] == 1) continue;
+      if (!d.empty()) {
+        const size_t l = d.size() - 1;
+        bool merge = true;
+        for (int k = 0; k < nin; ++k) merge = merge && x[k][l] == st[k][i] * os.d[i];
+        if (merge) {
+          d[l] *= os.d[i];
+          for (int k = 0; k < nin; ++k) x[k][l] = st[k][i];
+          continue;
+        }
+      }
+      d.push_back(os.d[i]);
+      for (int k = 0; k < nin; ++k) x[k].push_back(st[k][i]);
+    }
+    if (d.empty()) { d.push_back(1); for (int k = 0; k < nin; ++k) x[k].push_back(0); }
+    if (d.size() > 6) fail(ODLA_UNSUPPORTED_OP, "element-wise op '%s' needs more than 6 broadcast dims", n.out->name.c_str());
+    ep.rank = (int)d.size();
+    for (size_t i = 0; i < d.size(); ++i) {
+      ep.dims[i] = d[i];
+      ep.sa[i] = x[0][i];
+      if (nin > 1) ep.sb[i] = x[1][i];
+      if (nin > 2) ep.sc[i] = x[2][i];
+    }
+  }
+  const Ref ra = ref(tin[0]), rb = ref(tin[nin > 1 ? 1 : 0]), rc = ref(tin[nin > 2 ? 2 : 0]), ry = ref(ty);
+  emit("ewise:" + n.out->name, {tin[0], tin[1], tin[2]}, {ty}, [=](const ExecEnv& e, hipStream_t s) {
+    EwiseParams p = ep;
+    p.a = ra(e);
+    if (nin > 1) p.b = rb(e);
+    if (nin > 2) p.c = rc(e);
+    p.y = ry(e);
+    return launch_ewise(p, s);
+  });
+  set_main(n.out, ty);
+}
+
 // --------------------------------------------------------------- Unary ----
 void Planner::lower_unary(int ni) {
   Node& n = comp_->nodes[ni];
@@ -1693,6 +1783,7 @@ void Planner::lower_reduce(int ni) {
   const _odla_value* x = n.in[0];
   const Shape& xs = x->shape;
   const ReduceKind kind = (ReduceKind)n.i[0];
+  const float eps = n.f[0];
   const std::vector<int64_t>& axes = n.iv;
   const VState& s = vs_[x->index];
   // spatial reduction of a channels-last tensor (global pooling)
@@ -1728,7 +1819,7 @@ void Planner::lower_reduce(int ni) {
       const Ref b = ref(ty);
       const DType dt = px.dt;
       emit("reduce:" + n.out->name, {s.main}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
-        return launch_reduce(a(e), b(e), dt, dt, outer, len, inner, kind, st);
+        return launch_reduce(a(e), b(e), dt, dt, outer, len, inner, kind, st, eps);
       });
     }
     set_main(n.out, ty);
@@ -1748,7 +1839,28 @@ void Planner::lower_reduce(int ni) {
   const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
   const Ref a = ref(tx), b = ref(ty);
   emit("reduce:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
-    return launch_reduce(a(e), b(e), dt, dt, outer, len, inner, kind, st);
+    return launch_reduce(a(e), b(e), dt, dt, outer, len, inner, kind, st, eps);
+  });
+  set_main(n.out, ty);
+}
+
+// ---------------------------------------------------- ArgMax / ArgMin ----
+void Planner::lower_argext(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const int axis = (int)n.i[1];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= xs.d[i];
+  for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
+  const int64_t len = xs.d[axis];
+  const DType dt = T(tx).dt, odt = storage_dtype(n.out);
+  const int ty = new_tensor(odt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const bool is_max = n.i[0] != 0, last = n.i[2] != 0;
+  const Ref a = ref(tx), b = ref(ty);
+  emit(std::string(is_max ? "argmax:" : "argmin:") + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_arg_extreme(a(e), b(e), dt, odt, outer, len, inner, is_max, last, st);
   });
   set_main(n.out, ty);
 }
@@ -1934,6 +2046,112 @@ void Planner::lower_slice(int ni) {
     sy *= os.d[i];
   }
   strided_copy_step("slice:" + n.out->name, tx, ty, cp);
+  set_main(n.out, ty);
+}
+
+// ------------------------------------- Pad / Tile / broadcast / stuffing ----
+void Planner::lower_copynd(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const int r = (int)n.iv[0];
+  if (r > 8) fail(ODLA_UNSUPPORTED_OP, "copy of rank > 8 ('%s')", n.out->name.c_str());
+  StridedCopyParams cp;
+  cp.elem_size = dtype_size(dt);
+  cp.rank = r;
+  for (int i = 0; i < r; ++i) {
+    cp.dims[i] = n.iv[1 + i];
+    cp.sx[i] = n.iv[1 + r + i];
+    cp.sy[i] = n.iv[1 + 2 * r + i];
+  }
+  cp.x_off = n.iv[1 + 3 * r];
+  cp.y_off = n.iv[2 + 3 * r];
+  if (n.i[0] != 0) {
+    // the value 0 has an all-zero encoding in every storage type
+    const size_t bytes = (T(ty).bytes + 3) & ~(size_t)3;
+    const Ref b = ref(ty);
+    emit("fill:" + n.out->name, {}, {ty}, [=](const ExecEnv& e, hipStream_t st) { return launch_fill_bytes(b(e), bytes, 0u, st); });
+  }
+  strided_copy_step("copy:" + n.out->name, tx, ty, cp);
+  set_main(n.out, ty);
+}
+
+// ---------------------------------------------------------------- TopK ----
+void Planner::lower_topk(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const int axis = (int)n.i[2], K = (int)n.i[0];
+  const bool largest = n.i[1] != 0;
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= xs.d[i];
+  for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
+  const int64_t len = xs.d[axis];
+  const DType dt = T(tx).dt, idt = storage_dtype(n.out2);
+  const int tv = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const int ti = new_tensor(idt, L_ROWMAJOR, n.out2->shape, 0, SP_ARENA);
+  const Ref a = ref(tx), rv = ref(tv), ri = ref(ti);
+  emit("topk:" + n.out->name, {tx}, {tv, ti}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_topk(a(e), rv(e), ri(e), dt, idt, outer, len, inner, K, largest, st);
+  });
+  set_main(n.out, tv);
+  set_main(n.out2, ti);
+}
+
+// ----------------------------------------------------------------- LRN ----
+void Planner::lower_lrn(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const bool cl = n.i[0] == ODLA_CHANNELS_LAST;
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, xs, 0, SP_ARENA);
+  // row-major [N][C][inner]; channels-last data is the case inner == 1
+  int64_t N, inner;
+  int C;
+  if (cl) {
+    C = (int)xs.d[xs.rank - 1];
+    N = xs.numel() / C;
+    inner = 1;
+  } else {
+    N = xs.d[0];
+    C = (int)xs.d[1];
+    inner = xs.numel() / (N * C);
+  }
+  const int half = ((int)n.i[1] - 1) / 2;
+  const float alpha = n.f[0], beta = n.f[1], bias = n.f[2];
+  const Ref a = ref(tx), b = ref(ty);
+  emit("lrn:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_lrn(a(e), b(e), dt, N, C, inner, half, alpha, beta, bias, st);
+  });
+  set_main(n.out, ty);
+}
+
+// ------------------------------------------------- InstanceNormalization ----
+void Planner::lower_rownorm(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  if (n.i[0] == ODLA_CHANNELS_LAST) fail(ODLA_UNSUPPORTED_OP, "channels-last instance normalisation ('%s')", n.out->name.c_str());
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const DType dt = T(tx).dt;
+  const int ty = new_tensor(dt, L_ROWMAJOR, xs, 0, SP_ARENA);
+  const int C = (int)xs.d[1];
+  const int64_t rows = xs.d[0] * C, len = xs.numel() / rows;
+  int tg = -1, tb = -1;
+  if (n.in[1]) tg = const_vector<float>(DT_F32, const_as_float(n.in[1]));
+  if (n.in[2]) tb = const_vector<float>(DT_F32, const_as_float(n.in[2]));
+  const float eps = n.f[0], sg = n.f[1], sb = n.f[2];
+  const Ref a = ref(tx), b = ref(ty), rg = ref(tg >= 0 ? tg : tx), rb = ref(tb >= 0 ? tb : tx);
+  const bool hg = tg >= 0, hb = tb >= 0;
+  emit("instnorm:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_rownorm(a(e), b(e), dt, rows, len, C, hg ? (const float*)rg(e) : nullptr,
+                          hb ? (const float*)rb(e) : nullptr, sg, sb, eps, st);
+  });
   set_main(n.out, ty);
 }
 

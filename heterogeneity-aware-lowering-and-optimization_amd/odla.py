@@ -62,6 +62,10 @@ class Values(ctypes.Structure):
     _fields_ = [("size", ctypes.c_size_t), ("values", ctypes.c_void_p * ODLA_MAX_OUTPUTS)]
 
 
+class ValueIds(ctypes.Structure):
+    _fields_ = [("size", ctypes.c_size_t), ("value_ids", ctypes.c_char_p * ODLA_MAX_OUTPUTS)]
+
+
 class QuantInfo(ctypes.Structure):
     _fields_ = [("value_id", ctypes.c_char_p), ("ch_idx", ctypes.c_int), ("scale", ctypes.c_float),
                 ("offset", ctypes.c_float), ("min", ctypes.c_float), ("max", ctypes.c_float)]
@@ -183,6 +187,36 @@ def load_library(path=None):
     proto("odla_Quantize", vp, [vp, vp, vp, i32, i32, cid])
     proto("odla_Dequantize", vp, [vp, vp, vp, i32, i32, cid])
     proto("odla_NMS", vp, [vp, vp, u32, f32, f32, T, cid])
+    i64 = ctypes.c_int64
+    for n in ("Reciprocal", "Ceil", "Floor", "Sign", "Sin", "Cos", "Tan", "ASin", "ACos", "ATan", "Sinh", "Cosh",
+              "ASinh", "ACosh", "ATanh", "Softplus", "Softsign", "Not", "IsNaN"):
+        proto("odla_" + n, vp, [vp, cid])
+    for n in ("Elu", "Celu", "ThresholdedRelu"):
+        proto("odla_" + n, vp, [vp, f32, cid])
+    for n in ("Selu", "HardSigmoid", "Shrink"):
+        proto("odla_" + n, vp, [vp, f32, f32, cid])
+    for n in ("Pow", "SquaredDifference", "PRelu", "Equal", "NotEqual", "Less", "LessOrEqual", "Greater",
+              "GreaterOrEqual", "And", "Or", "Xor"):
+        proto("odla_" + n, vp, [vp, vp, cid])
+    proto("odla_Mod", vp, [vp, vp, i64, cid])
+    proto("odla_Mean", vp, [Values, cid])
+    proto("odla_IsInf", vp, [vp, u32, u32, cid])
+    proto("odla_Select", vp, [vp, vp, vp, S, cid])
+    for n in ("ReduceMin", "ReduceProd", "ReduceSumSquare", "ReduceLogSum", "ReduceLogSumExp"):
+        proto("odla_" + n, vp, [vp, sz, pu32, u32, S, cid])
+    for n in ("ReduceL1", "ReduceL2"):
+        proto("odla_" + n, vp, [vp, sz, pu32, u32, f32, S, cid])
+    proto("odla_ArgMax", vp, [vp, i32, u32, u32, T, cid])
+    proto("odla_ArgMin", vp, [vp, i32, u32, u32, T, cid])
+    proto("odla_TopK", Values, [vp, u32, u32, u32, u32, T, T, ValueIds])
+    proto("odla_Pad", vp, [vp, pu32, pu32, S, cid])
+    proto("odla_Tile", vp, [vp, pu32, S, cid])
+    proto("odla_ExpandDims", vp, [vp, S, cid])
+    proto("odla_Squeeze", vp, [vp, sz, pu32, S, cid])
+    proto("odla_Stack", vp, [Values, i32, S, cid])
+    proto("odla_LRN", vp, [vp, i32, i32, f32, f32, f32, cid])
+    proto("odla_InstanceNormalization", vp, [vp, i32, f32, vp, vp, f32, f32, cid])
+    proto("odla_DeConv", vp, [vp, i32, u32, vp, i32, pu32, pu32, pu32, pu32, vp, S, cid])
     if path == LIB_PATH:
         _lib = L
     return L
@@ -394,6 +428,139 @@ class HipBuilder:
 
     def nms(self, boxes, scores, max_out, iou_thr, score_thr, name=None):
         return self._ret(self.L.odla_NMS(boxes, scores, max_out, iou_thr, score_thr, make_type(np.int32, [1]), _cid(name)), "odla_NMS")
+
+    # -- wider operator surface --
+    def _values(self, xs):
+        vs = Values()
+        vs.size = len(xs)
+        for i, v in enumerate(xs):
+            vs.values[i] = v
+        return vs
+
+    def reciprocal(self, x, name=None): return self._un("Reciprocal", x, name)
+    def ceil(self, x, name=None): return self._un("Ceil", x, name)
+    def floor(self, x, name=None): return self._un("Floor", x, name)
+    def sign(self, x, name=None): return self._un("Sign", x, name)
+    def sin(self, x, name=None): return self._un("Sin", x, name)
+    def cos(self, x, name=None): return self._un("Cos", x, name)
+    def tan(self, x, name=None): return self._un("Tan", x, name)
+    def asin(self, x, name=None): return self._un("ASin", x, name)
+    def acos(self, x, name=None): return self._un("ACos", x, name)
+    def atan(self, x, name=None): return self._un("ATan", x, name)
+    def sinh(self, x, name=None): return self._un("Sinh", x, name)
+    def cosh(self, x, name=None): return self._un("Cosh", x, name)
+    def asinh(self, x, name=None): return self._un("ASinh", x, name)
+    def acosh(self, x, name=None): return self._un("ACosh", x, name)
+    def atanh(self, x, name=None): return self._un("ATanh", x, name)
+    def softplus(self, x, name=None): return self._un("Softplus", x, name)
+    def softsign(self, x, name=None): return self._un("Softsign", x, name)
+    def logical_not(self, x, name=None): return self._un("Not", x, name)
+    def isnan(self, x, name=None): return self._un("IsNaN", x, name)
+
+    def isinf(self, x, pos=True, neg=True, name=None):
+        return self._ret(self.L.odla_IsInf(x, int(pos), int(neg), _cid(name)), "odla_IsInf")
+
+    def elu(self, x, alpha, name=None): return self._ret(self.L.odla_Elu(x, alpha, _cid(name)), "odla_Elu")
+    def celu(self, x, alpha, name=None): return self._ret(self.L.odla_Celu(x, alpha, _cid(name)), "odla_Celu")
+
+    def thresholded_relu(self, x, alpha, name=None):
+        return self._ret(self.L.odla_ThresholdedRelu(x, alpha, _cid(name)), "odla_ThresholdedRelu")
+
+    def selu(self, x, alpha, gamma, name=None):
+        return self._ret(self.L.odla_Selu(x, alpha, gamma, _cid(name)), "odla_Selu")
+
+    def hard_sigmoid(self, x, alpha, beta, name=None):
+        return self._ret(self.L.odla_HardSigmoid(x, alpha, beta, _cid(name)), "odla_HardSigmoid")
+
+    def shrink(self, x, bias, lambd, name=None):
+        return self._ret(self.L.odla_Shrink(x, bias, lambd, _cid(name)), "odla_Shrink")
+
+    def pow(self, a, b, name=None): return self._bin("Pow", a, b, name)
+    def squared_difference(self, a, b, name=None): return self._bin("SquaredDifference", a, b, name)
+    def prelu(self, x, slope, name=None): return self._bin("PRelu", x, slope, name)
+    def equal(self, a, b, name=None): return self._bin("Equal", a, b, name)
+    def not_equal(self, a, b, name=None): return self._bin("NotEqual", a, b, name)
+    def less(self, a, b, name=None): return self._bin("Less", a, b, name)
+    def less_equal(self, a, b, name=None): return self._bin("LessOrEqual", a, b, name)
+    def greater(self, a, b, name=None): return self._bin("Greater", a, b, name)
+    def greater_equal(self, a, b, name=None): return self._bin("GreaterOrEqual", a, b, name)
+    def logical_and(self, a, b, name=None): return self._bin("And", a, b, name)
+    def logical_or(self, a, b, name=None): return self._bin("Or", a, b, name)
+    def logical_xor(self, a, b, name=None): return self._bin("Xor", a, b, name)
+
+    def mod(self, a, b, fmod=False, name=None):
+        return self._ret(self.L.odla_Mod(a, b, int(fmod), _cid(name)), "odla_Mod")
+
+    def mean(self, xs, name=None):
+        return self._ret(self.L.odla_Mean(self._values(xs), _cid(name)), "odla_Mean")
+
+    def select(self, cond, a, b, name=None):
+        return self._ret(self.L.odla_Select(cond, a, b, undefined_shape(), _cid(name)), "odla_Select")
+
+    def reduce_min(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceMin", x, axes, keep_dims, name)
+    def reduce_prod(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceProd", x, axes, keep_dims, name)
+    def reduce_sum_square(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceSumSquare", x, axes, keep_dims, name)
+    def reduce_log_sum(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceLogSum", x, axes, keep_dims, name)
+    def reduce_log_sum_exp(self, x, axes, keep_dims=True, name=None): return self._reduce("ReduceLogSumExp", x, axes, keep_dims, name)
+
+    def _reduce_eps(self, fn, x, axes, keep_dims, eps, name):
+        return self._ret(getattr(self.L, "odla_" + fn)(x, len(axes), _u32(axes), int(keep_dims), eps, undefined_shape(),
+                                                       _cid(name)), "odla_" + fn)
+
+    def reduce_l1(self, x, axes, keep_dims=True, eps=0.0, name=None): return self._reduce_eps("ReduceL1", x, axes, keep_dims, eps, name)
+    def reduce_l2(self, x, axes, keep_dims=True, eps=0.0, name=None): return self._reduce_eps("ReduceL2", x, axes, keep_dims, eps, name)
+
+    def _arg(self, fn, x, axis, keep_dims, last, dtype, name):
+        return self._ret(getattr(self.L, "odla_" + fn)(x, axis, int(keep_dims), int(last), make_type(dtype, [1]),
+                                                       _cid(name)), "odla_" + fn)
+
+    def argmax(self, x, axis, keep_dims=True, last=False, dtype=np.int32, name=None):
+        return self._arg("ArgMax", x, axis, keep_dims, last, dtype, name)
+
+    def argmin(self, x, axis, keep_dims=True, last=False, dtype=np.int32, name=None):
+        return self._arg("ArgMin", x, axis, keep_dims, last, dtype, name)
+
+    def topk(self, x, k, axis, largest=True, index_dtype=np.int32, names=(None, None)):
+        ids = ValueIds()
+        ids.size = 2
+        for i, n in enumerate(names):
+            ids.value_ids[i] = _cid(n)
+        r = self.L.odla_TopK(x, k, int(largest), 1, axis, make_type(np.float32, [1]), make_type(index_dtype, [1]), ids)
+        if r.size != 2:
+            raise OdlaError("odla_TopK failed (see the library log)")
+        return r.values[0], r.values[1]
+
+    def pad(self, x, front, back, name=None):
+        return self._ret(self.L.odla_Pad(x, _u32(front), _u32(back), undefined_shape(), _cid(name)), "odla_Pad")
+
+    def tile(self, x, repeat, name=None):
+        return self._ret(self.L.odla_Tile(x, _u32(repeat), undefined_shape(), _cid(name)), "odla_Tile")
+
+    def broadcast_to(self, x, shape, name=None):
+        return self._ret(self.L.odla_ExpandDims(x, make_shape(shape), _cid(name)), "odla_ExpandDims")
+
+    def squeeze(self, x, axes, name=None):
+        return self._ret(self.L.odla_Squeeze(x, len(axes), _u32(axes), undefined_shape(), _cid(name)), "odla_Squeeze")
+
+    def stack(self, xs, axis, name=None):
+        return self._ret(self.L.odla_Stack(self._values(xs), axis, undefined_shape(), _cid(name)), "odla_Stack")
+
+    def lrn(self, x, window, alpha, beta, bias, name=None):
+        return self._ret(self.L.odla_LRN(x, ODLA_CHANNELS_FIRST, window, alpha, beta, bias, _cid(name)), "odla_LRN")
+
+    def instance_norm(self, x, eps, scale=None, offset=None, scalar_scale=1.0, scalar_offset=0.0, name=None):
+        return self._ret(self.L.odla_InstanceNormalization(x, ODLA_CHANNELS_FIRST, eps, scale, offset, scalar_scale,
+                                                           scalar_offset, _cid(name)), "odla_InstanceNormalization")
+
+    def deconv(self, x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), group=1, out_hw=None, name=None):
+        """w in the ONNX ConvTranspose order [C_in, C_out / group, kH, kW]."""
+        od = undefined_shape()
+        if out_hw is not None:
+            s, _ = self.shape_of(x)
+            ws, _ = self.shape_of(w)
+            od = make_shape([s[0], ws[1] * group, out_hw[0], out_hw[1]])
+        return self._ret(self.L.odla_DeConv(x, ODLA_CHANNELS_FIRST, group, w, ODLA_IOS, _u32(stride), _u32((1, 1)),
+                                            _u32(pad[:2]), _u32(pad[2:]), bias, od, _cid(name)), "odla_DeConv")
 
     # -- execution --
     def session(self, use_graph=True):

@@ -530,6 +530,188 @@ odla_value odla_NMS(odla_value boxes, odla_value scores,
                     const odla_value_id value_id);
 
 /* ------------------------------------------------------------------------ */
+/* Wider operator surface (not used by the benchmark graphs).                 */
+/* ------------------------------------------------------------------------ */
+
+/* More element-wise unary operators on float values.
+ * [ref: ops/odla_ops_math.h (ACos .. Tan, Ceil, Floor, Reciprocal, Sign),
+ *  ops/odla_ops_nn.h (Elu, Selu, Celu, HardSigmoid, Softplus, Softsign,
+ *  ThresholdedRelu, Shrink); dnnl odla_dnnl_unary.cc:21-306,
+ *  odla_dnnl.cc:409-430,660-832,1671-1688] */
+odla_value odla_Reciprocal(odla_value input, const odla_value_id value_id);
+odla_value odla_Ceil(odla_value input, const odla_value_id value_id);
+odla_value odla_Floor(odla_value input, const odla_value_id value_id);
+odla_value odla_Sign(odla_value input, const odla_value_id value_id);
+odla_value odla_Sin(odla_value input, const odla_value_id value_id);
+odla_value odla_Cos(odla_value input, const odla_value_id value_id);
+odla_value odla_Tan(odla_value input, const odla_value_id value_id);
+odla_value odla_ASin(odla_value input, const odla_value_id value_id);
+odla_value odla_ACos(odla_value input, const odla_value_id value_id);
+odla_value odla_ATan(odla_value input, const odla_value_id value_id);
+odla_value odla_Sinh(odla_value input, const odla_value_id value_id);
+odla_value odla_Cosh(odla_value input, const odla_value_id value_id);
+odla_value odla_ASinh(odla_value input, const odla_value_id value_id);
+odla_value odla_ACosh(odla_value input, const odla_value_id value_id);
+odla_value odla_ATanh(odla_value input, const odla_value_id value_id);
+/* x > 0 ? x : alpha * (exp(x) - 1) */
+odla_value odla_Elu(odla_value input, odla_float32 alpha,
+                    const odla_value_id value_id);
+/* gamma * elu(x, alpha) */
+odla_value odla_Selu(odla_value input, odla_float32 alpha, odla_float32 gamma,
+                     const odla_value_id value_id);
+/* max(0, x) + min(0, alpha * (exp(x / alpha) - 1)) */
+odla_value odla_Celu(odla_value input, odla_float32 alpha,
+                     const odla_value_id value_id);
+/* clamp(alpha * x + beta, 0, 1) */
+odla_value odla_HardSigmoid(odla_value input, odla_float32 alpha,
+                            odla_float32 beta, const odla_value_id value_id);
+odla_value odla_Softplus(odla_value input, const odla_value_id value_id);
+odla_value odla_Softsign(odla_value input, const odla_value_id value_id);
+/* x > alpha ? x : 0 */
+odla_value odla_ThresholdedRelu(odla_value input, odla_float32 alpha,
+                                const odla_value_id value_id);
+/* x > lambd ? x - bias : (x < -lambd ? x + bias : 0) */
+odla_value odla_Shrink(odla_value input, odla_float32 bias, odla_float32 lambd,
+                       const odla_value_id value_id);
+
+/* Binary operators with broadcast beyond the six above; Add .. Min also accept
+ * integer operands.  Mod: fmod == 1 takes the sign of the dividend (C fmod),
+ * otherwise of the divisor.  PRelu: x < 0 ? x * slope : x.
+ * [ref: ops/odla_ops_math.h (Pow, Mod, SquaredDifference), ops/odla_ops_nn.h
+ *  (PRelu); dnnl odla_dnnl_binary.cc:21-298, odla_dnnl.cc:567-610,698-718] */
+odla_value odla_Pow(odla_value base, odla_value exponent,
+                    const odla_value_id value_id);
+odla_value odla_Mod(odla_value lhs, odla_value rhs, odla_int64 fmod,
+                    const odla_value_id value_id);
+odla_value odla_SquaredDifference(odla_value lhs, odla_value rhs,
+                                  const odla_value_id value_id);
+odla_value odla_PRelu(odla_value input, odla_value slope,
+                      const odla_value_id value_id);
+/* Element-wise mean of the operands.  [ref: dnnl odla_dnnl.cc:2432-2441] */
+odla_value odla_Mean(odla_values inputs, const odla_value_id value_id);
+
+/* Comparisons (operands of one type, BOOL result), logic on BOOL values and
+ * float predicates.
+ * [ref: ops/odla_ops_math.h (Equal .. Xor, IsNaN, IsInf);
+ *  dnnl odla_dnnl_binary.cc:40-90,222-270, odla_dnnl_unary.cc:47-60,140-160,225-238] */
+odla_value odla_Equal(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_NotEqual(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Less(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_LessOrEqual(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Greater(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_GreaterOrEqual(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_And(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Or(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Xor(odla_value lhs, odla_value rhs, const odla_value_id value_id);
+odla_value odla_Not(odla_value input, const odla_value_id value_id);
+odla_value odla_IsNaN(odla_value input, const odla_value_id value_id);
+odla_value odla_IsInf(odla_value input, odla_bool detect_pos,
+                      odla_bool detect_neg, const odla_value_id value_id);
+/* condition ? a : b, all three broadcast to the result shape.
+ * [ref: ops/odla_ops_process.h (odla_Select); dnnl odla_dnnl.cc:2372-2430] */
+odla_value odla_Select(odla_value condition, odla_value a, odla_value b,
+                       odla_value_shape output_dims,
+                       const odla_value_id value_id);
+
+/* More reductions.  L1 = sum|x| + epsilon, L2 = sqrt(sum x^2 + epsilon).
+ * [ref: ops/odla_ops_math.h:657-819; dnnl odla_dnnl_statistics.cc:21-160] */
+odla_value odla_ReduceMin(odla_value input, odla_size_t num_of_axes,
+                          const odla_uint32* axes, odla_bool keep_dims,
+                          odla_value_shape output_dims,
+                          const odla_value_id value_id);
+odla_value odla_ReduceProd(odla_value input, odla_size_t num_of_axes,
+                           const odla_uint32* axes, odla_bool keep_dims,
+                           odla_value_shape output_dims,
+                           const odla_value_id value_id);
+odla_value odla_ReduceL1(odla_value input, odla_size_t num_of_axes,
+                         const odla_uint32* axes, odla_bool keep_dims,
+                         odla_float32 epsilon, odla_value_shape output_dims,
+                         const odla_value_id value_id);
+odla_value odla_ReduceL2(odla_value input, odla_size_t num_of_axes,
+                         const odla_uint32* axes, odla_bool keep_dims,
+                         odla_float32 epsilon, odla_value_shape output_dims,
+                         const odla_value_id value_id);
+odla_value odla_ReduceSumSquare(odla_value input, odla_size_t num_of_axes,
+                                const odla_uint32* axes, odla_bool keep_dims,
+                                odla_value_shape output_dims,
+                                const odla_value_id value_id);
+odla_value odla_ReduceLogSum(odla_value input, odla_size_t num_of_axes,
+                             const odla_uint32* axes, odla_bool keep_dims,
+                             odla_value_shape output_dims,
+                             const odla_value_id value_id);
+odla_value odla_ReduceLogSumExp(odla_value input, odla_size_t num_of_axes,
+                                const odla_uint32* axes, odla_bool keep_dims,
+                                odla_value_shape output_dims,
+                                const odla_value_id value_id);
+/* Index of the extreme element along `axis` (INT32 or INT64); ties keep the
+ * first index, or the last when return_last_index is set.
+ * [ref: ops/odla_ops_math.h (ArgMax, ArgMin);
+ *  dnnl odla_dnnl_statistics.cc:203-300] */
+odla_value odla_ArgMax(odla_value input, odla_int32 axis, odla_bool keep_dims,
+                       odla_bool return_last_index,
+                       odla_value_type output_value_type,
+                       const odla_value_id value_id);
+odla_value odla_ArgMin(odla_value input, odla_int32 axis, odla_bool keep_dims,
+                       odla_bool return_last_index,
+                       odla_value_type output_value_type,
+                       const odla_value_id value_id);
+/* values[0] = the K best elements along `axis`, best first; values[1] =
+ * their indices (INT32 or INT64).  Equal elements are ordered by ascending
+ * index; `sorted` is ignored (the result is always ordered).
+ * [ref: ops/odla_ops_process.h (odla_TopK); dnnl odla_dnnl.cc:2064-2111] */
+odla_values odla_TopK(odla_value input, odla_uint32 K, odla_bool largest,
+                      odla_bool sorted, odla_uint32 axis,
+                      odla_value_type output_value_type,
+                      odla_value_type output_value_index_type,
+                      const odla_value_ids value_ids);
+
+/* Data movement.
+ * [ref: ops/odla_ops_process.h:117-130 (ExpandDims = broadcast), :221-236
+ *  (Pad, zero fill), :397-451 (Squeeze, Stack, Tile); dnnl odla_dnnl.cc:2183-2254] */
+odla_value odla_Pad(odla_value input, const odla_uint32* padding_front,
+                    const odla_uint32* padding_back,
+                    odla_value_shape output_dims, const odla_value_id value_id);
+odla_value odla_Tile(odla_value input, const odla_uint32* repeat,
+                     odla_value_shape output_dims, const odla_value_id value_id);
+odla_value odla_ExpandDims(odla_value input, odla_value_shape output_dims,
+                           const odla_value_id value_id);
+odla_value odla_Squeeze(odla_value input, odla_size_t num_of_axes,
+                        const odla_uint32* axes, odla_value_shape output_dims,
+                        const odla_value_id value_id);
+odla_value odla_Stack(odla_values inputs, odla_int32 axis,
+                      odla_value_shape output_shape,
+                      const odla_value_id value_id);
+
+/* Cross-channel local response normalisation:
+ * y = x / (bias + alpha / window * sum_{window} x^2) ^ beta.
+ * [ref: ops/odla_ops_nn.h (odla_LRN); dnnl odla_dnnl.cc:1553-1581] */
+odla_value odla_LRN(odla_value input, odla_memory_layout input_layout,
+                    odla_int32 window_size, odla_float32 alpha,
+                    odla_float32 beta, odla_float32 bias,
+                    const odla_value_id value_id);
+/* Per (sample, channel) normalisation over the spatial dims (channels-first
+ * input; scale / offset constants with one element per channel, or null to
+ * use the scalars).
+ * [ref: ops/odla_ops_nn.h (odla_InstanceNormalization);
+ *  dnnl odla_dnnl.cc:1583-1626] */
+odla_value odla_InstanceNormalization(
+    odla_value input, odla_memory_layout input_layout, odla_float32 epsilon,
+    odla_value scale, odla_value offset, odla_float32 scalar_scale,
+    odla_float32 scalar_offset, const odla_value_id value_id);
+/* Transposed 2-D convolution (channels-first input, constant FLOAT32 kernel,
+ * dilation 1).  An output shape larger than the minimal one, by less than the
+ * stride, selects the output padding.
+ * [ref: ops/odla_ops_nn.h (odla_DeConv); dnnl odla_dnnl.cc:1131-1232] */
+odla_value odla_DeConv(odla_value input, odla_memory_layout input_layout,
+                       odla_uint32 group, odla_value kernel,
+                       odla_memory_layout kernel_layout,
+                       const odla_uint32* strides, const odla_uint32* dilations,
+                       const odla_uint32* paddings_front,
+                       const odla_uint32* paddings_back, odla_value bias,
+                       odla_value_shape output_dims,
+                       const odla_value_id value_id);
+
+/* ------------------------------------------------------------------------ */
 /* Diagnostics (no counterpart in the reference).                            */
 /* ------------------------------------------------------------------------ */
 typedef struct {

@@ -19,6 +19,13 @@ Pin status (what fixes each function independently of this file):
   layernorm / gelu / erf / resize / concat / transpose / gather   closed forms
       and library routines (math.erf, numpy).
   nms   ONNX NonMaxSuppression published examples, O(n^2) brute force.
+  wider operator surface (trigonometric / hyperbolic functions, Elu family,
+      comparisons, Select, Mod, reductions, ArgMax, TopK, Pad, Tile, LRN,
+      InstanceNormalization, DeConv)   numpy / math library routines and
+      the scatter definition of the transposed convolution (``deconv2d``); cross-checked in
+      tests against torch's CPU operators.  TopK tie order (ascending index) is
+      this build's choice: the reference's portable TopK is not implemented
+      (``dnnl_utils.h:52-56``), so ties are PARITY UNPINNED.
   int8 convolution + requantisation (``qconv`` ...)   PARITY UNPINNED by the
       reference: it has no int8 convolution of its own.  The int32 accumulators
       are pinned by int64 brute force; the requantisation formula is this
@@ -209,6 +216,36 @@ def qadd(aq, a_qp, bq, b_qp, out_qp, relu=False):
 # --------------------------------------------------------------------------
 # NMS  [ref: ODLA/platforms/dnnl/dnnl_utils_avx512.h:977-1079, selection rule as intended]
 # --------------------------------------------------------------------------
+def deconv2d(x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), group=1, out_hw=None):
+    """Transposed convolution by its definition: every input element scatters its
+    kernel-weighted copy into the output, y[n, o, hi*s - p + r, wi*s - p + q] +=
+    x[n, c, hi, wi] * w[c, o_in_group, r, q]  (w in [C_in, C_out/group, kH, kW]
+    order; dnnl deconvolution_direct [ref: odla_dnnl.cc:1131-1232])."""
+    x = _f32(x).astype(np.float64)
+    w = _f32(w).astype(np.float64)
+    N, C, H, W = x.shape
+    Cin, Og, R, S = w.shape
+    assert Cin == C and C % group == 0
+    Cg = C // group
+    Ho = (H - 1) * stride[0] - pad[0] - pad[2] + R
+    Wo = (W - 1) * stride[1] - pad[1] - pad[3] + S
+    if out_hw is not None:
+        Ho, Wo = out_hw
+    full = np.zeros((N, Og * group, (H - 1) * stride[0] + R + stride[0], (W - 1) * stride[1] + S + stride[1]))
+    for g in range(group):
+        xg = x[:, g * Cg:(g + 1) * Cg]
+        wg = w[g * Cg:(g + 1) * Cg]
+        for r in range(R):
+            for q in range(S):
+                contrib = np.einsum("nchw,co->nohw", xg, wg[:, :, r, q])
+                full[:, g * Og:(g + 1) * Og, r:r + (H - 1) * stride[0] + 1:stride[0],
+                     q:q + (W - 1) * stride[1] + 1:stride[1]] += contrib
+    y = full[:, :, pad[0]:pad[0] + Ho, pad[1]:pad[1] + Wo]
+    if bias is not None:
+        y = y + _f32(bias).astype(np.float64).reshape(1, -1, 1, 1)
+    return np.ascontiguousarray(y).astype(np.float32)
+
+
 def _iou_one_to_many(box, others):
     f = np.float32
     y1 = np.minimum(box[0], box[2]); x1 = np.minimum(box[1], box[3])
@@ -333,6 +370,8 @@ class RefBuilder:
                 a = a.reshape(align_like_reference(a.shape, b.shape))
             else:
                 b = b.reshape(align_like_reference(b.shape, a.shape))
+        if a.dtype.kind in "iu" and a.dtype == b.dtype:  # integer arithmetic [ref: odla_dnnl.cc:567-610]
+            return self._name(name, f(a, b).astype(a.dtype))
         return self._name(name, f(a.astype(np.float32), b.astype(np.float32)).astype(np.float32))
 
     def add(self, a, b, name=None): return self._bin(np.add, a, b, name)
@@ -423,6 +462,236 @@ class RefBuilder:
 
     def reduce_max(self, x, axes, keep_dims=True, name=None):
         return self._name(name, _f32(x).max(axis=tuple(axes), keepdims=bool(keep_dims)))
+
+    # wider operator surface ---------------------------------------------------
+    # unary [ref: ODLA/platforms/dnnl/odla_dnnl_unary.cc:61-137; odla_dnnl.cc:409-430]
+    def reciprocal(self, x, name=None): return self._unary64(lambda v: 1.0 / v, x, name)
+    def ceil(self, x, name=None): return self._name(name, np.ceil(_f32(x)))
+    def floor(self, x, name=None): return self._name(name, np.floor(_f32(x)))
+    def sign(self, x, name=None): return self._name(name, np.sign(_f32(x)))
+    def sin(self, x, name=None): return self._unary64(np.sin, x, name)
+    def cos(self, x, name=None): return self._unary64(np.cos, x, name)
+    def tan(self, x, name=None): return self._unary64(np.tan, x, name)
+    def asin(self, x, name=None): return self._unary64(np.arcsin, x, name)
+    def acos(self, x, name=None): return self._unary64(np.arccos, x, name)
+    def atan(self, x, name=None): return self._unary64(np.arctan, x, name)
+    def sinh(self, x, name=None): return self._unary64(np.sinh, x, name)
+    def cosh(self, x, name=None): return self._unary64(np.cosh, x, name)
+    def asinh(self, x, name=None): return self._unary64(np.arcsinh, x, name)
+    def acosh(self, x, name=None): return self._unary64(np.arccosh, x, name)
+    def atanh(self, x, name=None): return self._unary64(np.arctanh, x, name)
+
+    def softplus(self, x, name=None):
+        """log(exp(x) + 1)  [ref: odla_dnnl.cc:1671-1678]"""
+        return self._unary64(lambda v: np.log(np.exp(v) + 1.0), x, name)
+
+    def softsign(self, x, name=None):
+        """x / (|x| + 1)  [ref: odla_dnnl.cc:1680-1687]"""
+        return self._unary64(lambda v: v / (np.abs(v) + 1.0), x, name)
+
+    def elu(self, x, alpha, name=None):
+        """dnnl eltwise_elu: x > 0 ? x : alpha (exp(x) - 1)  [ref: odla_dnnl.cc:720-723]"""
+        return self._unary64(lambda v: np.where(v > 0, v, alpha * np.expm1(v)), x, name)
+
+    def selu(self, x, alpha, gamma, name=None):
+        """gamma * elu(x, alpha)  [ref: odla_dnnl.cc:725-732]"""
+        return self._unary64(lambda v: gamma * np.where(v > 0, v, alpha * np.expm1(v)), x, name)
+
+    def celu(self, x, alpha, name=None):
+        """relu(x) - relu(-elu(x / alpha, alpha))  [ref: odla_dnnl.cc:734-748]"""
+        def f(v):
+            e = np.where(v / alpha > 0, v / alpha, alpha * np.expm1(v / alpha))
+            return np.maximum(v, 0.0) - np.maximum(-e, 0.0)
+        return self._unary64(f, x, name)
+
+    def hard_sigmoid(self, x, alpha, beta, name=None):
+        """clamp(alpha x + beta, 0, 1)  [ref: odla_dnnl.cc:660-686]"""
+        return self._unary64(lambda v: np.clip(alpha * v + beta, 0.0, 1.0), x, name)
+
+    def thresholded_relu(self, x, alpha, name=None):
+        """x > alpha ? x : 0  [ref: odla_dnnl.cc:750-774]"""
+        x = _f32(x)
+        return self._name(name, np.where(x > np.float32(alpha), x, np.float32(0)).astype(np.float32))
+
+    def shrink(self, x, bias, lambd, name=None):
+        """[ref: odla_dnnl.cc:776-789]"""
+        x = _f32(x)
+        b = np.float32(bias)
+        y = np.where(x > lambd, x - b, np.where(x < -lambd, x + b, np.float32(0)))
+        return self._name(name, y.astype(np.float32))
+
+    def isnan(self, x, name=None): return self._name(name, np.isnan(_f32(x)))
+
+    def isinf(self, x, pos=True, neg=True, name=None):
+        """[ref: odla_dnnl_unary.cc:143-155,229-238]: neither flag means the negative test"""
+        x = _f32(x)
+        if pos and neg:
+            return self._name(name, np.isinf(x))
+        return self._name(name, np.isposinf(x) if pos else np.isneginf(x))
+
+    def logical_not(self, x, name=None): return self._name(name, np.logical_not(np.asarray(x, bool)))
+
+    # binary [ref: odla_dnnl_binary.cc:41-141]
+    def _bin_typed(self, f, a, b, name, out_bool=False):
+        a, b = np.asarray(a), np.asarray(b)
+        assert a.dtype == b.dtype
+        if a.ndim != b.ndim:
+            if a.ndim < b.ndim:
+                a = a.reshape(align_like_reference(a.shape, b.shape))
+            else:
+                b = b.reshape(align_like_reference(b.shape, a.shape))
+        r = f(a, b)
+        return self._name(name, r.astype(bool) if out_bool else r.astype(a.dtype))
+
+    def pow(self, a, b, name=None):
+        return self._bin_typed(lambda l, r: np.power(l.astype(np.float64), r.astype(np.float64)) if l.dtype.kind == "f" else np.power(l, r), a, b, name)
+
+    def squared_difference(self, a, b, name=None): return self._bin_typed(lambda l, r: (l - r) * (l - r), a, b, name)
+
+    def prelu(self, x, slope, name=None):
+        """x < 0 ? x * slope : x  [ref: odla_dnnl.cc:698-718]"""
+        return self._bin_typed(lambda l, r: np.where(l < 0, l * r, l), x, slope, name)
+
+    def mod(self, a, b, fmod=False, name=None):
+        """[ref: odla_dnnl_binary.cc:104-127]: quotient from a double division, floor (mod) or
+        truncation through int32 (fmod), then l - r * quo in the operand type."""
+        def f(l, r):
+            t = l.astype(np.float64) / r.astype(np.float64)
+            if fmod:
+                q = np.where(t > 0, np.floor(t), np.ceil(t)).astype(np.int32).astype(l.dtype)
+            else:
+                q = np.floor(t).astype(l.dtype)
+            return l - r * q
+        return self._bin_typed(f, a, b, name)
+
+    def equal(self, a, b, name=None): return self._bin_typed(np.equal, a, b, name, True)
+    def not_equal(self, a, b, name=None): return self._bin_typed(np.not_equal, a, b, name, True)
+    def less(self, a, b, name=None): return self._bin_typed(np.less, a, b, name, True)
+    def less_equal(self, a, b, name=None): return self._bin_typed(np.less_equal, a, b, name, True)
+    def greater(self, a, b, name=None): return self._bin_typed(np.greater, a, b, name, True)
+    def greater_equal(self, a, b, name=None): return self._bin_typed(np.greater_equal, a, b, name, True)
+    def logical_and(self, a, b, name=None): return self._bin_typed(np.logical_and, a, b, name, True)
+    def logical_or(self, a, b, name=None): return self._bin_typed(np.logical_or, a, b, name, True)
+    def logical_xor(self, a, b, name=None): return self._bin_typed(np.logical_xor, a, b, name, True)
+
+    def mean(self, xs, name=None):
+        """((x0 + x1) + x2 ...) / n  [ref: odla_dnnl.cc:2432-2441]"""
+        acc = _f32(xs[0])
+        for v in xs[1:]:
+            acc = (acc + _f32(v)).astype(np.float32)
+        return self._name(name, (acc / np.float32(len(xs))).astype(np.float32))
+
+    def select(self, cond, a, b, name=None):
+        """[ref: odla_dnnl.cc:2372-2430]"""
+        cond, a, b = np.asarray(cond, bool), np.asarray(a), np.asarray(b)
+        hi = max((cond, a, b), key=lambda v: v.ndim).shape
+        al = [v if v.ndim == len(hi) else v.reshape(align_like_reference(v.shape, hi)) for v in (cond, a, b)]
+        return self._name(name, np.where(al[0], al[1], al[2]).astype(a.dtype))
+
+    # reductions [ref: odla_dnnl_statistics.cc:48-160]
+    def _red64(self, f, x, axes, keep_dims, name):
+        return self._name(name, f(_f32(x).astype(np.float64), tuple(axes), bool(keep_dims)).astype(np.float32))
+
+    def reduce_min(self, x, axes, keep_dims=True, name=None):
+        return self._name(name, _f32(x).min(axis=tuple(axes), keepdims=bool(keep_dims)))
+
+    def reduce_prod(self, x, axes, keep_dims=True, name=None):
+        return self._red64(lambda v, a, k: v.prod(axis=a, keepdims=k), x, axes, keep_dims, name)
+
+    def reduce_sum_square(self, x, axes, keep_dims=True, name=None):
+        return self._red64(lambda v, a, k: (v * v).sum(axis=a, keepdims=k), x, axes, keep_dims, name)
+
+    def reduce_l1(self, x, axes, keep_dims=True, eps=0.0, name=None):
+        """dnnl reduction_norm_lp_sum, p = 1: sum |x| + eps"""
+        return self._red64(lambda v, a, k: np.abs(v).sum(axis=a, keepdims=k) + eps, x, axes, keep_dims, name)
+
+    def reduce_l2(self, x, axes, keep_dims=True, eps=0.0, name=None):
+        """dnnl reduction_norm_lp_sum, p = 2: sqrt(sum x^2 + eps)"""
+        return self._red64(lambda v, a, k: np.sqrt((v * v).sum(axis=a, keepdims=k) + eps), x, axes, keep_dims, name)
+
+    def reduce_log_sum(self, x, axes, keep_dims=True, name=None):
+        return self._red64(lambda v, a, k: np.log(v.sum(axis=a, keepdims=k)), x, axes, keep_dims, name)
+
+    def reduce_log_sum_exp(self, x, axes, keep_dims=True, name=None):
+        def f(v, a, k):
+            m = v.max(axis=a, keepdims=True)
+            r = np.log(np.exp(v - m).sum(axis=a, keepdims=True)) + m
+            return r if k else np.squeeze(r, axis=a)
+        return self._red64(f, x, axes, keep_dims, name)
+
+    def _arg(self, is_max, x, axis, keep_dims, last, dtype, name):
+        """[ref: odla_dnnl_statistics.cc:203-232]: strict comparison keeps the first index,
+        ``return_last_index`` also replaces on equality."""
+        x = _f32(x)
+        axis = axis % x.ndim
+        v = x if is_max else -x
+        if last:
+            idx = x.shape[axis] - 1 - np.argmax(np.flip(v, axis=axis), axis=axis)
+        else:
+            idx = np.argmax(v, axis=axis)
+        if keep_dims:
+            idx = np.expand_dims(idx, axis)
+        return self._name(name, idx.astype(dtype))
+
+    def argmax(self, x, axis, keep_dims=True, last=False, dtype=np.int32, name=None):
+        return self._arg(True, x, axis, keep_dims, last, dtype, name)
+
+    def argmin(self, x, axis, keep_dims=True, last=False, dtype=np.int32, name=None):
+        return self._arg(False, x, axis, keep_dims, last, dtype, name)
+
+    def topk(self, x, k, axis, largest=True, index_dtype=np.int32, names=(None, None)):
+        """Ordered, ties by ascending index (a stable sort of the keys)."""
+        x = _f32(x)
+        key = -x if largest else x
+        order = np.argsort(key, axis=axis, kind="stable")
+        idx = np.take(order, np.arange(k), axis=axis)
+        vals = np.take_along_axis(x, idx, axis=axis)
+        return self._name(names[0], vals), self._name(names[1], idx.astype(index_dtype))
+
+    def pad(self, x, front, back, name=None):
+        return self._name(name, np.pad(np.asarray(x), list(zip(front, back))))
+
+    def tile(self, x, repeat, name=None): return self._name(name, np.tile(np.asarray(x), repeat))
+
+    def broadcast_to(self, x, shape, name=None):
+        x = np.asarray(x)
+        if x.ndim != len(shape):
+            x = x.reshape(align_like_reference(x.shape, shape))
+        return self._name(name, np.ascontiguousarray(np.broadcast_to(x, shape)))
+
+    def squeeze(self, x, axes, name=None):
+        return self._name(name, np.squeeze(np.asarray(x), axis=tuple(axes) if len(axes) else None))
+
+    def stack(self, xs, axis, name=None): return self._name(name, np.stack(xs, axis=axis))
+
+    def lrn(self, x, window, alpha, beta, bias, name=None):
+        """dnnl lrn_across_channels: x / (bias + alpha / size * sum_window x^2)^beta
+        [ref: odla_dnnl.cc:1553-1581]"""
+        x64 = _f32(x).astype(np.float64)
+        half = (window - 1) // 2
+        C = x64.shape[1]
+        sq = x64 * x64
+        acc = np.zeros_like(x64)
+        for c in range(C):
+            lo, hi = max(0, c - half), min(C - 1, c + half)
+            acc[:, c] = sq[:, lo:hi + 1].sum(axis=1)
+        y = x64 / np.power(bias + alpha / (2 * half + 1) * acc, beta)
+        return self._name(name, y.astype(np.float32))
+
+    def instance_norm(self, x, eps, scale=None, offset=None, scalar_scale=1.0, scalar_offset=0.0, name=None):
+        """(x - mean) / sqrt(sum((x - mean)^2) / m + eps) * scale + offset over the spatial dims
+        [ref: odla_dnnl.cc:1583-1626]"""
+        x64 = _f32(x).astype(np.float64)
+        ax = tuple(range(2, x64.ndim))
+        d = x64 - x64.mean(axis=ax, keepdims=True)
+        var = (d * d).mean(axis=ax, keepdims=True)
+        shp = (1, -1) + (1,) * (x64.ndim - 2)
+        g = np.asarray(scale, np.float64).reshape(shp) if scale is not None else scalar_scale
+        b = np.asarray(offset, np.float64).reshape(shp) if offset is not None else scalar_offset
+        return self._name(name, (d / np.sqrt(var + eps) * g + b).astype(np.float32))
+
+    def deconv(self, x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), group=1, out_hw=None, name=None):
+        return self._name(name, deconv2d(x, w, bias, stride, pad, group, out_hw))
 
     # data movement ----------------------------------------------------------
     def cast(self, x, dtype, name=None): return self._name(name, np.asarray(x).astype(dtype))
