@@ -156,6 +156,7 @@ odla_status ensure_plan(_odla_computation* c) {
     return st;
   }
   c->plan = std::move(plan);
+  c->planned_nodes = c->nodes.size();
   return ODLA_SUCCESS;
 }
 
@@ -218,11 +219,14 @@ odla_status odla_CreateComputation(odla_computation* computation) {
   return ODLA_SUCCESS;
 }
 
+static void destroy_context(odla_context ctx);
+
 odla_status odla_DestroyComputation(odla_computation c) {
   if (c == nullptr) return ODLA_INVALID_PARAM;
   if (!is_live(c)) return ODLA_INVALID_PARAM;
   forget_computation(c);
   (void)hipDeviceSynchronize();
+  if (c->eager_ctx != nullptr) destroy_context(c->eager_ctx);
   delete c;
   return ODLA_SUCCESS;
 }
@@ -271,6 +275,8 @@ odla_status odla_SetComputationItem(odla_computation c, odla_item_type type, odl
 }
 
 // ---------------------------------------------------------------- context --
+static odla_status create_context_for(_odla_computation* c, odla_context* context);
+
 odla_status odla_CreateContext(odla_context* context) {
   if (context == nullptr) return ODLA_INVALID_PARAM;
   _odla_computation* c = current_computation();
@@ -278,6 +284,15 @@ odla_status odla_CreateContext(odla_context* context) {
     OHIP_ERR("odla_CreateContext: no computation exists");
     return ODLA_FAILURE;
   }
+  odla_status st = create_context_for(c, context);
+  if (st == ODLA_SUCCESS) {
+    std::lock_guard<std::mutex> lk(c->mu);
+    ++c->live_contexts;
+  }
+  return st;
+}
+
+static odla_status create_context_for(_odla_computation* c, odla_context* context) {
   odla_status st = ensure_plan(c);
   if (st != ODLA_SUCCESS) return st;
   auto ctx = std::make_unique<_odla_context>();
@@ -299,13 +314,21 @@ odla_status odla_CreateContext(odla_context* context) {
   return ODLA_SUCCESS;
 }
 
-odla_status odla_DestroyContext(odla_context ctx) {
-  if (ctx == nullptr) return ODLA_INVALID_PARAM;
+static void destroy_context(odla_context ctx) {
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   drop_graph(ctx);
   if (ctx->arena) (void)hipFree(ctx->arena);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
+}
+
+odla_status odla_DestroyContext(odla_context ctx) {
+  if (ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (ctx->comp != nullptr && is_live(ctx->comp)) {
+    std::lock_guard<std::mutex> lk(ctx->comp->mu);
+    if (ctx->comp->live_contexts > 0) --ctx->comp->live_contexts;
+  }
+  destroy_context(ctx);
   return ODLA_SUCCESS;
 }
 
@@ -549,8 +572,81 @@ odla_status odla_SetValueAsOutputById(const odla_value_id id) {
   return odla_SetValueAsOutput(find_value(current_computation(), id));
 }
 
+// Interpret mode: values made by odla_CreateValue carry their own data
+// (odla_SetValueData), operators are recorded as usual, and asking for a
+// value's data with no context compiles what has been recorded so far (again
+// only when the graph has grown or the value was not yet a result), runs it on
+// an internal context and copies the value back.
+// [ref: ODLA/platforms/dnnl/odla_dnnl.cc:161-179,225-230,276-295]
+static odla_status eager_evaluate(_odla_value* value, void* data_ptr) {
+  _odla_computation* c = value->comp;
+  if (c == nullptr || !is_live(c)) return ODLA_INVALID_PARAM;
+  {
+    std::lock_guard<std::mutex> lk(c->mu);
+    const bool stale = !c->plan || c->planned_nodes != c->nodes.size() || !value->is_output;
+    if (stale) {
+      if (c->live_contexts > 0) {
+        OHIP_ERR("odla_GetValueData: '%s' is not a result of the compiled computation and contexts are still alive",
+                 value->name.c_str());
+        return ODLA_FAILURE;
+      }
+      if (c->eager_ctx != nullptr) { destroy_context(c->eager_ctx); c->eager_ctx = nullptr; }
+      if (!value->is_output) { value->is_output = true; c->outputs.push_back(value); }
+      c->plan.reset();
+      c->plan_failed = false;
+      for (Node& n : c->nodes) n.absorbed = false;
+    }
+  }
+  if (c->eager_ctx == nullptr) {
+    odla_status st = create_context_for(c, &c->eager_ctx);
+    if (st != ODLA_SUCCESS) return st;
+    c->eager_ctx->use_graph = false;
+  }
+  _odla_context* ctx = c->eager_ctx;
+  for (_odla_value* a : c->args) {
+    if (!a->eager) continue;
+    if (a->eager_data == nullptr) {
+      OHIP_ERR("odla_GetValueData: value '%s' has no data (odla_SetValueData)", a->name.c_str());
+      return ODLA_INVALID_PARAM;
+    }
+    ctx->bound_in[a] = a->eager_data;
+  }
+  odla_status st = odla_ExecuteComputation(c, ctx, ODLA_COMPUTE_INFERENCE, nullptr);
+  if (st != ODLA_SUCCESS) return st;
+  return odla_GetValueData(value, data_ptr, ctx);
+}
+
+odla_value odla_CreateValue(odla_value_type type, const odla_value_id id) {
+  if (current_computation() == nullptr) {
+    odla_computation c = nullptr;  // the interpreter works on an implicit computation
+    if (odla_CreateComputation(&c) != ODLA_SUCCESS) return nullptr;
+  }
+  odla_value v = odla_CreateArgument(type, id);
+  if (v != nullptr) v->eager = true;
+  return v;
+}
+
+odla_status odla_SetValueData(odla_value value, const odla_void* data_ptr) {
+  if (value == nullptr || data_ptr == nullptr) return ODLA_INVALID_PARAM;
+  if (!value->eager) {
+    OHIP_ERR("odla_SetValueData: '%s' was not made by odla_CreateValue", value->name.c_str());
+    return ODLA_INVALID_PARAM;
+  }
+  value->eager_data = data_ptr;
+  return ODLA_SUCCESS;
+}
+
+odla_status odla_SetValueDataById(const odla_value_id id, const odla_void* data_ptr) {
+  return odla_SetValueData(find_value(current_computation(), id), data_ptr);
+}
+
+odla_status odla_GetValueDataById(const odla_value_id id, odla_void* data_ptr) {
+  return odla_GetValueData(find_value(current_computation(), id), data_ptr, nullptr);
+}
+
 odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr, odla_context ctx) {
-  if (value == nullptr || data_ptr == nullptr || ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (value == nullptr || data_ptr == nullptr) return ODLA_INVALID_PARAM;
+  if (ctx == nullptr) return eager_evaluate(value, data_ptr);
   if (!ctx->executed || !ctx->comp->plan) return ODLA_FAILURE;
   const Plan& plan = *ctx->comp->plan;
   for (const Plan::IO& io : plan.outputs) {

@@ -75,6 +75,8 @@ struct _odla_value {
   int index = -1;                   // position in computation->values
   int producer = -1;                // node index, -1 for ARG / CONSTANT
   bool is_output = false;
+  bool eager = false;               // created by odla_CreateValue: data comes from odla_SetValueData
+  const void* eager_data = nullptr; // borrowed from the caller
   _odla_computation* comp = nullptr;
 };
 
@@ -182,6 +184,9 @@ struct _odla_computation {
   std::mutex mu;
   std::unique_ptr<ohip::Plan> plan;
   bool plan_failed = false;
+  size_t planned_nodes = 0;          // size of `nodes` when the plan was built
+  int live_contexts = 0;             // contexts created by the caller
+  _odla_context* eager_ctx = nullptr;  // context behind odla_GetValueData(value, ptr, NULL)
 };
 
 struct _odla_context {

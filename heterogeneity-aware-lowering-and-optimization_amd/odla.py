@@ -143,6 +143,10 @@ def load_library(path=None):
     proto("odla_SetValueAsOutputById", i32, [cid])
     proto("odla_GetValueData", i32, [vp, vp, vp])
     proto("odla_ReleaseValue", i32, [vp])
+    proto("odla_CreateValue", vp, [T, cid])
+    proto("odla_SetValueData", i32, [vp, vp])
+    proto("odla_SetValueDataById", i32, [cid, vp])
+    proto("odla_GetValueDataById", i32, [cid, vp])
     proto("odla_CreateArgument", vp, [T, cid])
     proto("odla_CreateConstant", vp, [T, vp, cid])
     proto("odla_AllocateDevice", i32, [vp, i32, i32, ctypes.POINTER(vp)])

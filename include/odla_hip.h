@@ -319,9 +319,28 @@ odla_status odla_SetValueAsOutput(odla_value value);
 odla_status odla_SetValuesAsOutput(odla_values values);
 odla_status odla_SetValueAsOutputById(const odla_value_id value_id);
 /* Copy the device-resident result of `value` from the last execution of
- * `context` to host memory.  [ref: odla_compute.h:556-565] */
+ * `context` to host memory.  With a NULL context (interpret mode) the
+ * operators recorded so far are compiled - again only when the graph has
+ * grown or `value` was not yet a result - and run on an internal context with
+ * the data of the odla_CreateValue values; `value` then stays a result of the
+ * computation.  Fails while caller-made contexts of the computation exist and
+ * a recompilation would be needed.
+ * [ref: odla_compute.h:556-565; dnnl odla_dnnl.cc:161-179,286-295] */
 odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr,
                               odla_context context);
+odla_status odla_GetValueDataById(const odla_value_id value_id,
+                                  odla_void* data_ptr);
+/* Interpret mode: a value that carries its own data.  The pointer given to
+ * odla_SetValueData is borrowed (not copied) and read at every evaluation, as
+ * the reference CPU backend does; without a current computation an implicit
+ * one is created.
+ * [ref: ops/odla_ops_basic.h:50-52; odla_value.h:82-120;
+ *  dnnl odla_dnnl.cc:74-82,225-230,276-284] */
+odla_value odla_CreateValue(odla_value_type value_type,
+                            const odla_value_id value_id);
+odla_status odla_SetValueData(odla_value value, const odla_void* data_ptr);
+odla_status odla_SetValueDataById(const odla_value_id value_id,
+                                  const odla_void* data_ptr);
 odla_status odla_ReleaseValue(odla_value value); /* no-op; values die with the graph */
 
 /* Graph inputs and constants.  A constant's host data must stay valid until
