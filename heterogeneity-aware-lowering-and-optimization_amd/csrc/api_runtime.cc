@@ -150,6 +150,7 @@ odla_status ensure_plan(_odla_computation* c) {
   if (c->plan) return ODLA_SUCCESS;
   if (c->plan_failed) return ODLA_FAILURE;
   std::unique_ptr<Plan> plan;
+  profiler_configure(&c->opts);
   odla_status st = build_plan(c, &plan);
   if (st != ODLA_SUCCESS) {
     c->plan_failed = true;
@@ -451,6 +452,7 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
     return ODLA_FAILURE;
   }
   ctx->executed = true;
+  if (!plan.stat_recs.empty()) return profiler_collect(plan, ctx->arena);
   return ODLA_SUCCESS;
 }
 
@@ -583,7 +585,8 @@ static odla_status eager_evaluate(_odla_value* value, void* data_ptr) {
   if (c == nullptr || !is_live(c)) return ODLA_INVALID_PARAM;
   {
     std::lock_guard<std::mutex> lk(c->mu);
-    const bool stale = !c->plan || c->planned_nodes != c->nodes.size() || !value->is_output;
+    const bool stale = !c->plan || c->planned_nodes != c->nodes.size() || !value->is_output ||
+                       c->plan->calibrated != profiler_active();
     if (stale) {
       if (c->live_contexts > 0) {
         OHIP_ERR("odla_GetValueData: '%s' is not a result of the compiled computation and contexts are still alive",

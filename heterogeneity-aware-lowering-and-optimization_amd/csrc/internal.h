@@ -101,6 +101,11 @@ struct Options {
   bool raw_acc = false;
   const odla_value_quant_info* qtable = nullptr;
   int qtable_size = 0;
+  // calibration: fp32, nothing fused, range statistics behind every named fp32 value
+  bool calibrate = false;
+  bool calib_channels = false;   // also per-channel ranges
+  int calib_axis = -1;           // channel axis (negative: from the end)
+  bool calib_skip_weights = false;
 };
 
 // ------------------------------------------------------------------- plan --
@@ -160,6 +165,19 @@ struct Plan {
   };
   std::vector<IO> inputs, outputs;
   std::unordered_map<const _odla_value*, int> final_tensor;  // for odla_GetValueData
+  // calibration plans: one record per profiled value; its partial minima /
+  // maxima live in a pinned arena tensor as [channels][splits][2] floats
+  struct StatRec {
+    std::string name, op_type;
+    Shape shape;
+    int channels = 1;       // partial rows (1 when no per-channel ranges were asked for)
+    bool per_channel = false;
+    int splits = 1;
+    int tensor = -1;
+    std::vector<std::string> inputs;
+  };
+  std::vector<StatRec> stat_recs;
+  bool calibrated = false;
   // host blobs copied into the constant pool / init scratch when the plan is built
   struct Blob { Space space; size_t offset; std::vector<uint8_t> owned; const void* src; size_t bytes; };
   std::vector<Blob> blobs;
@@ -167,6 +185,14 @@ struct Plan {
 };
 
 odla_status build_plan(_odla_computation* comp, std::unique_ptr<Plan>* out);
+
+// Calibration profiler (the control functions StartProfiling .. are exported
+// with the reference profiler's names).
+bool profiler_active();
+void profiler_configure(Options* o);
+// Reads the statistics of one finished execution and appends them to the open run.
+odla_status profiler_collect(const Plan& plan, const char* arena);
+const char* api_op_name(const Node& n);
 
 DType dtype_from_odla(odla_element_type t);
 int odla_type_size(odla_element_type t);

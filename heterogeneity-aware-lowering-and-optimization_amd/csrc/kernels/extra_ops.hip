@@ -117,6 +117,30 @@ rownorm_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t
   }
 }
 
+// --------------------------------------------------------------------------
+// Range statistics for calibration: x fp32 [outer][C][inner] -> partial minima
+// and maxima part[c][s] = {min, max} over the s-th interleaved share of
+// channel c.  grid = (splits, C); the few partials are combined on the host.
+__global__ void __launch_bounds__(kThreads)
+minmax_partial_kernel(const float* __restrict__ x, float* __restrict__ part, int64_t outer, int C, int64_t inner) {
+  __shared__ float red[kThreads / 64];
+  const int c = blockIdx.y, s = blockIdx.x, S = gridDim.x;
+  const int64_t per = outer * inner;
+  float lo = INFINITY, hi = -INFINITY;
+  for (int64_t e = (int64_t)s * kThreads + threadIdx.x; e < per; e += (int64_t)S * kThreads) {
+    const int64_t o = e / inner, i = e - o * inner;
+    const float v = x[(o * C + c) * inner + i];
+    lo = fminf(lo, v);
+    hi = fmaxf(hi, v);
+  }
+  hi = block_max<kThreads>(hi, red);
+  lo = -block_max<kThreads>(-lo, red);
+  if (threadIdx.x == 0) {
+    part[((int64_t)c * S + s) * 2 + 0] = lo;
+    part[((int64_t)c * S + s) * 2 + 1] = hi;
+  }
+}
+
 #define FLOAT_DISPATCH(dt, EXPR)                         \
   switch (dt) {                                          \
     case DT_F32: { using T = float; EXPR; break; }       \
@@ -132,6 +156,13 @@ hipError_t launch_fill_bytes(void* p, size_t bytes, uint32_t pattern, hipStream_
   const int64_t n = (int64_t)(bytes / 4);
   if (n == 0) return hipSuccess;
   hipLaunchKernelGGL(fill_u32_kernel, dim3(grid_for(n, kThreads * 4)), dim3(kThreads), 0, stream, (uint32_t*)p, n, pattern);
+  return hipGetLastError();
+}
+
+hipError_t launch_minmax_partial(const float* x, float* part, int64_t outer, int C, int64_t inner, int splits,
+                                 hipStream_t stream) {
+  if (!x || !part || outer <= 0 || C <= 0 || C > 65535 || inner <= 0 || splits <= 0) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(minmax_partial_kernel, dim3(splits, C), dim3(kThreads), 0, stream, x, part, outer, C, inner);
   return hipGetLastError();
 }
 

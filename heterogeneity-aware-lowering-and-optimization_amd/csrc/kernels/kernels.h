@@ -315,6 +315,10 @@ hipError_t launch_fill_bytes(void* p, size_t bytes, uint32_t pattern, hipStream_
 // [outer][K][inner], best first, equal values by ascending index.
 hipError_t launch_topk(const void* x, void* vals, void* idxs, DType dt, DType idx_dt, int64_t outer,
                        int64_t len, int64_t inner, int K, bool largest, hipStream_t stream);
+// Calibration statistics: part[c][s] = {min, max} of the s-th share of channel
+// c of x[outer][C][inner] (fp32), s < splits, C <= 65535.
+hipError_t launch_minmax_partial(const float* x, float* part, int64_t outer, int C, int64_t inner, int splits,
+                                 hipStream_t stream);
 // LRN across the channels of x[N][C][inner]:
 // y = x / (bias + alpha / (2 half + 1) * sum_{|c'-c| <= half} x[c']^2) ^ beta
 hipError_t launch_lrn(const void* x, void* y, DType dt, int64_t N, int C, int64_t inner, int half, float alpha,

@@ -459,6 +459,8 @@ class Planner {
   void lower_topk(int ni);
   void lower_lrn(int ni);
   void lower_rownorm(int ni);
+  void emit_stats(const _odla_value* v, const char* op_type, int forced_axis, const Node* producer);
+  bool calib_ = false;
 
   void collect_epilogue(int ni, int64_t out_channels, int channel_axis_of_output, Epilogue* ep);
   bool per_channel_constant(const _odla_value* k, const Shape& aligned, const Shape& out, int ch_axis,
@@ -507,11 +509,57 @@ void Planner::parse_quant_table() {
   }
 }
 
+// Calibration: partial minima / maxima of a named fp32 value, kept in a pinned
+// arena tensor until the execution has finished.
+void Planner::emit_stats(const _odla_value* v, const char* op_type, int forced_axis, const Node* producer) {
+  const Options& o = comp_->opts;
+  if (v == nullptr || v->name.empty() || dtype_from_odla(v->etype) != DT_F32) return;
+  const int tx = get(v, L_ROWMAJOR, FORM_FLOAT);
+  if (T(tx).dt != DT_F32) return;
+  const Shape& s = v->shape;
+  Plan::StatRec rec;
+  rec.name = v->name;
+  rec.op_type = op_type;
+  rec.shape = s;
+  int axis = forced_axis >= 0 ? forced_axis : (o.calib_axis < 0 ? s.rank + o.calib_axis : o.calib_axis);
+  int64_t outer = 1, inner = 1, C = 1;
+  if (o.calib_channels && axis >= 0 && axis < s.rank && s.d[axis] <= 65535) {
+    rec.per_channel = true;
+    C = s.d[axis];
+    for (int i = 0; i < axis; ++i) outer *= s.d[i];
+    for (int i = axis + 1; i < s.rank; ++i) inner *= s.d[i];
+  } else {
+    inner = s.numel();
+  }
+  rec.channels = (int)C;
+  const int64_t per = outer * inner;
+  int64_t splits = (per + 8191) / 8192;
+  const int64_t cap = 2048 / C > 1 ? 2048 / C : 1;   // enough workgroups to fill the chip, few partials
+  if (splits > cap) splits = cap;
+  rec.splits = (int)(splits < 1 ? 1 : splits);
+  rec.tensor = raw_buffer((size_t)C * rec.splits * 2 * sizeof(float), SP_ARENA);
+  if (producer != nullptr)
+    for (const _odla_value* in : producer->in)
+      if (in != nullptr && !in->name.empty()) rec.inputs.push_back(in->name);
+  const Ref a = ref(tx), b = ref(rec.tensor);
+  const int Ci = (int)C, sp = rec.splits;
+  emit("stats:" + v->name, {tx}, {rec.tensor}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_minmax_partial((const float*)a(e), (float*)b(e), outer, Ci, inner, sp, st);
+  });
+  PTensor& p = T(rec.tensor);
+  p.pinned = true;
+  p.last_step = 1 << 30;
+  plan_->stat_recs.push_back(std::move(rec));
+}
+
 void Planner::run() {
   const Options& o = comp_->opts;
-  if (o.fp16) cdt_ = DT_F16;
+  calib_ = o.calibrate;
+  plan_->calibrated = calib_;
+  if (calib_) cdt_ = DT_F32;
+  else if (o.fp16) cdt_ = DT_F16;
   else if (o.bf16 != BF16_DISABLE) cdt_ = DT_BF16;
-  parse_quant_table();
+  if (!calib_) parse_quant_table();
 
   vs_.assign(comp_->values.size(), VState());
   consumers_.assign(comp_->values.size(), {});
@@ -539,9 +587,32 @@ void Planner::run() {
     // otherwise no slot is filled: consumers convert from the staging tensor
   }
 
+  if (calib_) {
+    for (_odla_value* a : comp_->args) emit_stats(a, a->eager ? "odla_SetValueData" : "odla_CreateArgument", -1, nullptr);
+    if (!o.calib_skip_weights) {
+      // kernels of convolutions get one range per output channel whatever the channel axis is
+      std::unordered_map<const _odla_value*, int> kernel_axis;
+      for (const Node& n : comp_->nodes)
+        if (n.op == OP_CONV && n.in[1] != nullptr) {
+          const int kl = (int)n.i[2];
+          kernel_axis[n.in[1]] = kl == ODLA_SIO ? 3 : (kl == ODLA_SOI ? 2 : (kl == ODLA_IOS ? 1 : 0));
+        }
+      for (const auto& up : comp_->values) {
+        const _odla_value* v = up.get();
+        if (v->kind != _odla_value::CONSTANT || consumers_[v->index].empty()) continue;
+        auto it = kernel_axis.find(v);
+        emit_stats(v, "odla_CreateConstant", it == kernel_axis.end() ? -1 : it->second, nullptr);
+      }
+    }
+  }
   for (size_t ni = 0; ni < comp_->nodes.size(); ++ni) {
     if (comp_->nodes[ni].absorbed) continue;
     lower((int)ni);
+    if (calib_) {
+      const Node& n = comp_->nodes[ni];
+      emit_stats(n.out, api_op_name(n), -1, &n);
+      if (n.out2 != nullptr) emit_stats(n.out2, api_op_name(n), -1, &n);
+    }
   }
 
   // Outputs: row-major, declared element type.
@@ -676,6 +747,7 @@ void Planner::bn_params_host(const Node& n, int64_t C, std::vector<float>* scale
 void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* ep) {
   _odla_value* cur = comp_->nodes[ni].out;
   ep->final_value = cur;
+  if (calib_) return;  // every value of the graph must exist to be measured
   const bool q8 = comp_->opts.int8;
   while (true) {
     if (cur->is_output || consumers_[cur->index].size() != 1) break;
@@ -1413,7 +1485,7 @@ void Planner::lower_binary(int ni) {
   float act_a = 0.f, act_b = 0.f;
   const bool q8 = comp_->opts.int8 && q8_value(a) && q8_value(b) && a->shape == os && b->shape == os &&
                   (n.i[0] == BIN_ADD) && a->kind != _odla_value::CONSTANT && b->kind != _odla_value::CONSTANT;
-  if (!outv->is_output && consumers_[outv->index].size() == 1) {
+  if (!calib_ && !outv->is_output && consumers_[outv->index].size() == 1) {
     Node& nx = comp_->nodes[consumers_[outv->index][0]];
     if (nx.op == OP_UNARY && !nx.absorbed) {
       const ActKind k = (ActKind)nx.i[0];

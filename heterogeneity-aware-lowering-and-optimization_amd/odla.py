@@ -232,7 +232,9 @@ def exported_symbols_declared_in_header():
     hdr = os.path.join(os.path.dirname(_HERE), "include", "odla_hip.h")
     text = open(hdr).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(odla_[A-Z]\w*)\s*\(", text)))
+    names = set(re.findall(r"\b(odla_[A-Z]\w*)\s*\(", text))
+    names |= set(re.findall(r"^void\s+([A-Z]\w*)\s*\(", text, flags=re.M))  # profiler control functions
+    return sorted(names)
 
 
 def _u32(vals):

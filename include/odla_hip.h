@@ -20,6 +20,7 @@
 #ifndef ODLA_HIP_H_
 #define ODLA_HIP_H_
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -729,6 +730,28 @@ odla_value odla_DeConv(odla_value input, odla_memory_layout input_layout,
                        const odla_uint32* paddings_back, odla_value bias,
                        odla_value_shape output_dims,
                        const odla_value_id value_id);
+
+/* ------------------------------------------------------------------------ */
+/* Calibration profiler.  The control functions keep the names and meaning of */
+/* the reference's profiler library; between StartProfiling and StopProfiling */
+/* computations are compiled in fp32 with nothing fused and range statistics  */
+/* behind every named FLOAT32 value (arguments and constants included), and   */
+/* every execution inside StartOneRun / StopOneRun appends, per value,        */
+/*   "<id>" : {"op_type", "shape", "channels", "min_value", "max_value",     */
+/*             "channels_min", "channels_max"}                                */
+/* to the "ProfilingResults" object of the JSON file; StopProfiling adds the  */
+/* "NetworkInfo" object (the operands of every value).  Kernels of            */
+/* convolutions are always profiled along their output-channel axis.  Start   */
+/* profiling before the computation's first context exists.                   */
+/* [ref: ODLA/platforms/odla_profiler.cc:133-285; utils/halo_pgq.py:205-239] */
+/* ------------------------------------------------------------------------ */
+void StartProfiling(const char* data_path); /* NULL: write to stdout */
+void StartOneRun(const char* tag);
+void StopOneRun(void);
+void StopProfiling(void);
+void EnableChannelWiseProf(void);
+void SetChannelAxis(int axis); /* negative: counted from the last dim */
+void SkipWeightsProfiling(bool skip);
 
 /* ------------------------------------------------------------------------ */
 /* Diagnostics (no counterpart in the reference).                            */
