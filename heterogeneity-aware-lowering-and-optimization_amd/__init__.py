@@ -14,3 +14,4 @@ from . import models_bert  # noqa: F401
 from . import models_yolo  # noqa: F401
 from . import models_streaming  # noqa: F401
 from . import calibration  # noqa: F401
+from . import weights  # noqa: F401

@@ -26,6 +26,23 @@ def test_mnist_softmax_regression_fp32(models):
     assert np.array_equal(np.argmax(got, 1), np.argmax(want, 1))
 
 
+def test_mnist_with_the_reference_weights(pkg, models):
+    """Config 0 with the trained weights of the reference's mnist_simple.pb (tests/golden holds a
+    copy of that data file), read by the GraphDef constant extractor."""
+    announce("mnist fp32, trained weights")
+    import os
+    import __graft_entry__ as entry
+    consts = pkg.weights.read_graphdef_constants(open(os.path.join(entry.ROOT, "tests", "golden", "mnist_simple.pb"), "rb").read())
+    w = {"V": consts["Variable"], "V1": consts["Variable_1"].reshape(1, 10)}
+    feeds = models.mnist_input(64, seed=77)
+    build = lambda b: models.build_mnist(b, w, 64)
+    got = run_hip(build, feeds)["y"]
+    want = run_ref(build, feeds)["y"]
+    assert np.max(np.abs(got - want)) <= 1e-4 * float(np.max(want))
+    assert np.array_equal(np.argmax(got, 1), np.argmax(want, 1))
+    assert np.max(np.abs(got.sum(axis=1) - 1.0)) <= 1e-5
+
+
 def test_small_resnet_fp32(models):
     announce("small resnet fp32")
     w = models.resnet50_weights(seed=3, num_classes=100, stages=SMALL_STAGES, stem=16)
