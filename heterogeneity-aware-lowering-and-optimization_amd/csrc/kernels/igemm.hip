@@ -24,6 +24,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 namespace ohip {
 
@@ -251,11 +252,15 @@ template <int M> struct EpiTraits<EpiQuant<M>> { using TOut = typename QuantOut<
 // residual loads are 16-byte vectors and consecutive lanes cover contiguous
 // memory.  `smem` is the K loop's buffer; it is reused once every wavefront of
 // the workgroup has left the loop.
-template <typename TIn, typename Epi, int BM, int BN, int WM, int WN>
+// kEnterBarrier = false: the caller's wavefronts never shared `smem` before
+// (each only ever touches its own staging slice); n_off shifts the channels
+// this call covers within the tile.
+template <typename TIn, typename Epi, int BM, int BN, int WM, int WN, bool kEnterBarrier = true>
 __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int epi_vec,
                                                typename Mma<TIn>::Acc (&acc)[WM / 32][WN / 32],
                                                unsigned char* smem, const int tile_m, const int tile_n,
-                                               const int z, const int M, const int wave, const int lane) {
+                                               const int z, const int M, const int wave, const int lane,
+                                               const int n_off = 0) {
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int EPI_PITCH = WN + 4;  // 4-byte words per staged pixel row
   using AccE = typename Epi::AccE;
@@ -272,7 +277,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
   constexpr int PPP = 64 / LPP;  // pixels per read-back pass
   const int rp = lane / LPP;     // pixel within a pass
   const int c8 = (lane % LPP) * 8;
-  const int n = tile_n * BN + wn * WN + c8;
+  const int n = tile_n * BN + wn * WN + c8 + n_off;
   int nvalid = p.Kout - n;
   nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
   const bool vec = (epi_vec & 1) && nvalid == 8;
@@ -324,7 +329,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
     if (have_rpre) rfetch(0, rcur);
   }
 
-  __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
+  if constexpr (kEnterBarrier) __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     // park: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
@@ -930,6 +935,93 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
 }
 
+// ---------------------------------------------------------------------------
+// Variant for 1x1 filters over few input channels (K = 64 or 128 bytes per
+// pixel, no padding): such layers are pure streaming - one short burst of
+// matrix instructions between reading 8-16 KiB and writing 16-32 KiB per tile -
+// and with a K loop, operand staging and workgroup barriers their time is the
+// sum of the latencies of those phases.  Here nothing is staged and nothing is
+// shared: every wavefront owns 32 pixels x 128 channels, reads its pixel
+// fragments and the (fragment-ordered, L2-resident) weights straight from
+// global memory into MFMA operand registers, keeps the weights for all the
+// pixel tiles it walks, and requests the pixels of its next tile before it
+// runs the epilogue of the current one.  The epilogue parks 64 channels at a
+// time in the wavefront's private LDS slice (no workgroup barrier anywhere).
+// NKK = 32-byte K steps per pixel; NJ = 32-channel slices per wavefront (the
+// tile is 32 NJ channels wide: 4 slices of 4 K steps do not fit the registers).
+template <typename TIn, typename Epi, int NKK, int NJ>
+__global__ void __launch_bounds__(256, 3)
+igemm_lean_kernel(const IgemmParams p, const int epi_vec, const int tiles_per_wg) {
+  constexpr int BM = 128, BN = 32 * NJ;
+  using Acc = typename Mma<TIn>::Acc;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * 32 * (64 + 4) * 4];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, lg = lane >> 5;
+  const int M = p.N * p.Ho * p.Wo;
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = (p.Kout + BN - 1) / BN;
+  int bid = blockIdx.x;
+  {
+    const int per = gridDim.x >> 3;
+    if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int tile_n = bid % tiles_n;
+  const int tm0 = (bid / tiles_n) * tiles_per_wg;
+  const int tm1 = tm0 + tiles_per_wg < tiles_m ? tm0 + tiles_per_wg : tiles_m;
+
+  const TIn* x = reinterpret_cast<const TIn*>(p.x);
+  const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag) + lane;
+  uintx4 w[NJ][NKK];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    int wtile = tile_n * NJ + j;
+    wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;  // surplus slices compute channels that are never stored
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) w[j][kk] = wf[((int64_t)wtile * p.wf_chunks + kk) * 64];
+  }
+  const int HoWo = p.Ho * p.Wo;
+  // lane (l32, lg) supplies bytes [32 kk + 16 lg, +16) of pixel row l32
+  auto load_a = [&](const int tile_m, uintx4 (&a)[NKK]) {
+    int m = tile_m * BM + wave * 32 + l32;
+    m = m < M ? m : M - 1;
+    const int n_img = fast_div(m, p.howo_magic, p.howo_shift);
+    const int rem = m - n_img * HoWo;
+    const int ho = fast_div(rem, p.wo_magic, p.wo_shift);
+    const int wo = rem - ho * p.Wo;
+    const uintx4* row =
+        reinterpret_cast<const uintx4*>(x + (((int64_t)n_img * p.H + ho * p.sh) * p.W + wo * p.sw) * p.xcs) + lg;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) a[kk] = row[2 * kk];
+  };
+  uintx4 a_cur[NKK], a_nxt[NKK];
+  load_a(tm0, a_cur);
+  for (int tile_m = tm0; tile_m < tm1; ++tile_m) {
+    if (tile_m + 1 < tm1) load_a(tile_m + 1, a_nxt);
+    // 64 channels at a time: half the accumulator registers, half the staging space
+#pragma unroll
+    for (int h = 0; h < NJ / 2; ++h) {
+      Acc acc[1][2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[0][j][e] = 0;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[0][j] = Mma<TIn>::run(w[2 * h + j][kk], a_cur[kk], acc[0][j]);
+      igemm_epilogue<TIn, Epi, BM, BN, 32, 64, false>(p, epi_vec, acc, smem, tile_m, tile_n, 0, M, wave, lane, h * 64);
+      // the same wavefront parks into its slice again next: order it behind the read-back
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) a_cur[kk] = a_nxt[kk];
+  }
+}
+
 // Rearranges packed weight rows ([batch][rows][row_bytes], zero padded) into
 // MFMA fragment order, followed by kWfragTailBytes of the fill byte: 16-byte unit ((b * tiles + t) * chunks + q) * 64 + lane
 // holds bytes [q*32 + (lane/32)*16, +16) of row t*32 + lane%32.
@@ -1016,6 +1108,44 @@ hipError_t launch_wreg(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// 1x1 filters with at most one K stage and no padding: the streaming variant.
+int lean_steps(const IgemmParams& p) {
+  if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid
+    if (strcmp(force, "lean") != 0 && force[0] != 0) return 0;
+  }
+  const int kbytes = p.C * dtype_size(p.in_dt);
+  if (p.R != 1 || p.S != 1 || p.ph != 0 || p.pw != 0 || p.batch != 1 || p.Kout < 64) return 0;
+  // (8-bit layers of this shape are bound by the arithmetic of the requantising
+  // epilogue, not by their staging, and do not gain from it)
+  if (p.in_dt != DT_F16 && p.in_dt != DT_BF16) return 0;
+  if (kbytes != 64 && kbytes != 128) return 0;
+  return kbytes / 32;
+}
+
+template <typename TIn, typename Epi>
+hipError_t launch_lean(const IgemmParams& p, int epi_vec, hipStream_t stream) {
+  const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+  const int steps = lean_steps(p);
+  const int bn = steps == 2 ? 128 : 64;
+  const int64_t tiles_m = (M + 127) / 128, tiles_n = (p.Kout + bn - 1) / bn;
+  // a few pixel tiles per workgroup: the weights are fetched once for all of
+  // them and the next tile's pixels are in flight during each epilogue
+  int tpw = 1;
+  while (tpw < 8 && tiles_m * tiles_n / (tpw * 2) >= 4096) tpw *= 2;
+  if (const char* force = getenv("ODLA_HIP_LEAN_TILES")) {  // test aid: pixel tiles per workgroup
+    const int v = atoi(force);
+    if (v >= 1 && v <= 64) tpw = v;
+  }
+  const int64_t groups = (tiles_m + tpw - 1) / tpw;
+  const int64_t wgs = groups * tiles_n;
+  if (wgs <= 0 || wgs > 0x7fffffff) return hipErrorInvalidValue;
+  if (steps == 2)
+    hipLaunchKernelGGL((igemm_lean_kernel<TIn, Epi, 2, 4>), dim3((unsigned)wgs), dim3(256), 0, stream, p, epi_vec, tpw);
+  else
+    hipLaunchKernelGGL((igemm_lean_kernel<TIn, Epi, 4, 2>), dim3((unsigned)wgs), dim3(256), 0, stream, p, epi_vec, tpw);
+  return hipGetLastError();
+}
+
 // The weights-in-registers kernel pays off once a layer has enough output
 // channels to give each of the four wavefronts its own 32-channel slice.
 bool wreg_shape(const IgemmParams& p) {
@@ -1032,13 +1162,16 @@ bool wreg_shape(const IgemmParams& p) {
 
 template <typename TIn, typename Epi>
 hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
+  if constexpr (!std::is_same<TIn, float>::value) {
+    if (p.w_frag != nullptr && lean_steps(p) > 0) return launch_lean<TIn, Epi>(p, epi_vec, s);
+  }
   if (p.w_frag != nullptr && wreg_shape(p)) return launch_wreg<TIn, Epi>(p, epi_vec, s);
   return dispatch_tiles<TIn, Epi>(p, epi_vec, s);
 }
 
 }  // namespace
 
-bool igemm_wants_wfrag(const IgemmParams& p) { return wreg_shape(p); }
+bool igemm_wants_wfrag(const IgemmParams& p) { return wreg_shape(p) || lean_steps(p) > 0; }
 
 hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
   if (p.src == nullptr || p.dst == nullptr || p.rows <= 0 || p.row_bytes <= 0 || p.row_bytes % 16 != 0 ||
@@ -1051,6 +1184,7 @@ hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
 }
 
 const char* igemm_variant_name(const IgemmParams& p) {
+  if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
   if (p.w_frag != nullptr && wreg_shape(p)) return "128x128w";
   return choose_variant(p).name;
 }

@@ -2,6 +2,8 @@
 // All are HBM-bound streaming kernels: channels-last pooling moves 16-byte
 // channel vectors, row kernels keep the row in registers between the
 // statistics pass and the normalising pass so every element is read once.
+#include <type_traits>
+
 #include "device_utils.h"
 
 namespace ohip {
@@ -173,26 +175,26 @@ __global__ void __launch_bounds__(kThreads) pool2d_q8_kernel(PoolParams p) {
 
 // --------------------------------------------------------------------------
 // Reduction over the middle axis of [outer][len][inner].
-__device__ __forceinline__ float red_init(ReduceKind k) {
-  return k == RED_MAX ? -INFINITY : (k == RED_MIN ? INFINITY : (k == RED_PROD ? 1.f : 0.f));
+// The accumulation rule is a compile-time choice (a run-time switch inside the
+// inner loops costs more than the loads): 0 sum, 1 max, 2 min, 3 product,
+// 4 sum of magnitudes, 5 sum of squares.
+enum { ACC_SUM = 0, ACC_MAX, ACC_MIN, ACC_PROD, ACC_ABS, ACC_SQ };
+template <int A> __device__ __forceinline__ float red_init() {
+  return A == ACC_MAX ? -INFINITY : (A == ACC_MIN ? INFINITY : (A == ACC_PROD ? 1.f : 0.f));
 }
-__device__ __forceinline__ float red_step(float acc, float v, ReduceKind k) {
-  switch (k) {
-    case RED_MAX: return fmaxf(acc, v);
-    case RED_MIN: return fminf(acc, v);
-    case RED_PROD: return acc * v;
-    case RED_L1: return acc + fabsf(v);
-    case RED_L2: case RED_SUMSQ: return acc + v * v;
-    default: return acc + v;
-  }
+template <int A> __device__ __forceinline__ float red_step(float acc, float v) {
+  if (A == ACC_MAX) return fmaxf(acc, v);
+  if (A == ACC_MIN) return fminf(acc, v);
+  if (A == ACC_PROD) return acc * v;
+  if (A == ACC_ABS) return acc + fabsf(v);
+  if (A == ACC_SQ) return acc + v * v;
+  return acc + v;
 }
-__device__ __forceinline__ float red_merge(float a, float b, ReduceKind k) {
-  switch (k) {
-    case RED_MAX: return fmaxf(a, b);
-    case RED_MIN: return fminf(a, b);
-    case RED_PROD: return a * b;
-    default: return a + b;
-  }
+template <int A> __device__ __forceinline__ float red_merge(float a, float b) {
+  if (A == ACC_MAX) return fmaxf(a, b);
+  if (A == ACC_MIN) return fminf(a, b);
+  if (A == ACC_PROD) return a * b;
+  return a + b;
 }
 __device__ __forceinline__ float red_final(float acc, int64_t len, ReduceKind k, float eps) {
   switch (k) {
@@ -204,7 +206,7 @@ __device__ __forceinline__ float red_final(float acc, int64_t len, ReduceKind k,
   }
 }
 // inner == 1: one wavefront per row, lanes stride the row.
-template <typename TI, typename TO>
+template <typename TI, typename TO, int A>
 __global__ void __launch_bounds__(kThreads)
 reduce_rows_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, int64_t len,
                    ReduceKind kind, float eps) {
@@ -213,16 +215,16 @@ reduce_rows_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
   const int64_t nwaves = ((int64_t)gridDim.x * blockDim.x) >> 6;
   for (int64_t r = wave; r < rows; r += nwaves) {
     const TI* row = x + r * len;
-    float acc = red_init(kind);
-    for (int64_t i = lane; i < len; i += 64) acc = red_step(acc, Store<TI>::ld(row + i), kind);
+    float acc = red_init<A>();
+    for (int64_t i = lane; i < len; i += 64) acc = red_step<A>(acc, Store<TI>::ld(row + i));
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) acc = red_merge(acc, __shfl_xor(acc, o, 64), kind);
+    for (int o = 32; o > 0; o >>= 1) acc = red_merge<A>(acc, __shfl_xor(acc, o, 64));
     if (lane == 0) Store<TO>::st(y + r, red_final(acc, len, kind, eps));
   }
 }
 // inner > 1: one thread per (outer, inner) column; consecutive threads read
 // consecutive inner positions, so each step over `len` is a coalesced row.
-template <typename TI, typename TO>
+template <typename TI, typename TO, int A>
 __global__ void __launch_bounds__(kThreads)
 reduce_cols_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int64_t len,
                    int64_t inner, ReduceKind kind, float eps) {
@@ -231,14 +233,14 @@ reduce_cols_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, 
        i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t o = i / inner, in = i - o * inner;
     const TI* col = x + o * len * inner + in;
-    float acc = red_init(kind);
-    for (int64_t k = 0; k < len; ++k) acc = red_step(acc, Store<TI>::ld(col + k * inner), kind);
+    float acc = red_init<A>();
+    for (int64_t k = 0; k < len; ++k) acc = red_step<A>(acc, Store<TI>::ld(col + k * inner));
     Store<TO>::st(y + i, red_final(acc, len, kind, eps));
   }
 }
 // inner % V == 0: one thread per (outer, 16-byte group of inner positions); every
 // step over `len` is a coalesced row of vectors.
-template <typename TI, typename TO>
+template <typename TI, typename TO, int A>
 __global__ void __launch_bounds__(kThreads)
 reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int64_t len,
                        int64_t inner, ReduceKind kind, float eps) {
@@ -251,7 +253,7 @@ reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t out
     const TI* col = x + o * len * inner + in;
     float acc[V];
 #pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = red_init(kind);
+    for (int e = 0; e < V; ++e) acc[e] = red_init<A>();
     int64_t k = 0;
     for (; k + 4 <= len; k += 4) {
       Vec16<TI> v[4];
@@ -260,13 +262,13 @@ reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t out
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
-        for (int e = 0; e < V; ++e) acc[e] = red_step(acc[e], v[u].get(e), kind);
+        for (int e = 0; e < V; ++e) acc[e] = red_step<A>(acc[e], v[u].get(e));
     }
     for (; k < len; ++k) {
       Vec16<TI> v;
       v.load(col + k * inner);
 #pragma unroll
-      for (int e = 0; e < V; ++e) acc[e] = red_step(acc[e], v.get(e), kind);
+      for (int e = 0; e < V; ++e) acc[e] = red_step<A>(acc[e], v.get(e));
     }
 #pragma unroll
     for (int e = 0; e < V; ++e) Store<TO>::st(y + o * inner + in + e, red_final(acc[e], len, kind, eps));
@@ -656,26 +658,37 @@ hipError_t launch_reduce_q8_mean(const void* x, float* y, int64_t outer, int64_t
 template <typename TI>
 static hipError_t reduce_out(const void* x, void* y, DType out_dt, int64_t outer, int64_t len,
                              int64_t inner, ReduceKind kind, float eps, hipStream_t stream) {
-  auto go = [&](auto tag) -> hipError_t {
+  auto go = [&](auto tag, auto rule) -> hipError_t {
     using TO = decltype(tag);
+    constexpr int A = decltype(rule)::value;
     if (inner == 1) {
       const int grid = grid_for(outer * 64, kThreads);
-      hipLaunchKernelGGL((reduce_rows_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
+      hipLaunchKernelGGL((reduce_rows_kernel<TI, TO, A>), dim3(grid), dim3(kThreads), 0, stream,
                          (const TI*)x, (TO*)y, outer, len, kind, eps);
     } else if (inner % (16 / (int)sizeof(TI)) == 0 && al16(x)) {
       const int grid = grid_for(outer * (inner / (16 / (int)sizeof(TI))), kThreads);
-      hipLaunchKernelGGL((reduce_cols_vec_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
+      hipLaunchKernelGGL((reduce_cols_vec_kernel<TI, TO, A>), dim3(grid), dim3(kThreads), 0, stream,
                          (const TI*)x, (TO*)y, outer, len, inner, kind, eps);
     } else {
       const int grid = grid_for(outer * inner, kThreads);
-      hipLaunchKernelGGL((reduce_cols_kernel<TI, TO>), dim3(grid), dim3(kThreads), 0, stream,
+      hipLaunchKernelGGL((reduce_cols_kernel<TI, TO, A>), dim3(grid), dim3(kThreads), 0, stream,
                          (const TI*)x, (TO*)y, outer, len, inner, kind, eps);
     }
     return hipGetLastError();
   };
-  if (out_dt == DT_F32) return go(float{});
-  if (out_dt == DT_F16) return go(f16_t{});
-  if (out_dt == DT_BF16) return go(bf16_t{});
+  auto with_rule = [&](auto tag) -> hipError_t {
+    switch (kind) {
+      case RED_MAX: return go(tag, std::integral_constant<int, ACC_MAX>{});
+      case RED_MIN: return go(tag, std::integral_constant<int, ACC_MIN>{});
+      case RED_PROD: return go(tag, std::integral_constant<int, ACC_PROD>{});
+      case RED_L1: return go(tag, std::integral_constant<int, ACC_ABS>{});
+      case RED_L2: case RED_SUMSQ: return go(tag, std::integral_constant<int, ACC_SQ>{});
+      default: return go(tag, std::integral_constant<int, ACC_SUM>{});
+    }
+  };
+  if (out_dt == DT_F32) return with_rule(float{});
+  if (out_dt == DT_F16) return with_rule(f16_t{});
+  if (out_dt == DT_BF16) return with_rule(bf16_t{});
   return hipErrorInvalidValue;
 }
 

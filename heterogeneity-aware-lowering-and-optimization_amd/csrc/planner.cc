@@ -1404,6 +1404,55 @@ void Planner::lower_gemm(int ni) {
     ip.w_rows = (int)Nn; ip.w_cols = w_rs; ip.w_rs = w_rs;
     ip.N = (int)(lead * M);
     ip.batch = 1;
+    // Few output tiles and a long K (classifier heads): the tiles would walk K
+    // one after the other on a handful of CUs.  Split K into independent
+    // problems (grid.z) that write fp32 partial sums, then add them up.
+    {
+      const int es = dtype_size(dt);
+      const int64_t rows = lead * M;
+      const int64_t tiles = ((rows + 127) / 128) * ((Nn + 127) / 128);
+      const int stage = 128 / es;  // K elements per 128-byte stage
+      int splits = 1;
+      if (!calib_ && ep.residual == nullptr && ep.act == ACT_NONE && tiles <= 64 && (int64_t)Kp * es >= 2048) {
+        while (splits < 16 && Kp % (splits * 2 * stage) == 0 && Kp / (splits * 2) >= 4 * stage && tiles * splits * 2 <= 1024)
+          splits *= 2;
+      }
+      if (splits > 1) {
+        const int Kc = Kp / splits;
+        Shape ps;
+        ps.rank = 3;
+        ps.d[0] = splits; ps.d[1] = rows; ps.d[2] = Nn;
+        const int tp = new_tensor(DT_F32, L_ROWMAJOR, ps, 0, SP_ARENA);
+        int tb = -1;
+        if (ep.has_bias) {  // the first partial carries the bias
+          std::vector<float> b((size_t)splits * Nn, 0.f);
+          for (int64_t i = 0; i < Nn && i < (int64_t)ep.bias.size(); ++i) b[(size_t)i] = ep.bias[(size_t)i];
+          tb = const_vector<float>(DT_F32, b);
+        }
+        IgemmParams sp = ip;
+        sp.C = Kc;
+        sp.w_cols = Kc;
+        sp.batch = splits;
+        sp.x_bs = Kc; sp.w_bs = Kc; sp.y_bs = rows * Nn; sp.bias_bs = Nn;
+        sp.out_dt = DT_F32;
+        const Ref rx = ref(ta), rw = ref(tw), rp = ref(tp), rb = ref(tb >= 0 ? tb : ta);
+        const bool hb = tb >= 0;
+        emit("gemm.splitk:" + outv->name, {ta, tw}, {tp}, [=](const ExecEnv& e, hipStream_t st) {
+          IgemmParams p = sp;
+          p.x = rx(e); p.w = rw(e); p.y = rp(e);
+          p.bias = hb ? rb(e) : nullptr;
+          return launch_igemm(p, st);
+        });
+        const int ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
+        const Ref ry = ref(ty);
+        const int64_t inner = rows * Nn;
+        emit("gemm.sum:" + outv->name, {tp}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+          return launch_reduce(rp(e), ry(e), DT_F32, dt, 1, splits, inner, RED_SUM, st);
+        });
+        set_main(outv, ty);
+        return;
+      }
+    }
   } else {
     if (!ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: scale folding into a run-time operand");
     int tb = get(B, L_ROWMAJOR, FORM_FLOAT);

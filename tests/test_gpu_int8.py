@@ -103,12 +103,17 @@ def test_q8_conv_accumulators_and_requant(case, odla, ref):
     assert np.array_equal(q_got, q_want.astype(np.int64))
 
 
-@pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (3, 128, 7, 7, 200)])
-def test_q8_residual_fused_equals_unfused_equals_oracle(dims, odla, ref):
+@pytest.mark.parametrize("tiles_per_wg", [0, 3])
+@pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (3, 128, 7, 7, 200), (4, 64, 21, 19, 256), (2, 128, 30, 30, 512),
+                                  (3, 256, 9, 9, 136)])
+def test_q8_residual_fused_equals_unfused_equals_oracle(dims, tiles_per_wg, odla, ref, monkeypatch):
     """Conv -> Add(residual) -> ReLU: fused into the conv epilogue, and as separate
     quantised kernels (the conv result is also a graph output, which blocks fusion).
-    The second shape takes the weights-in-registers kernel."""
-    announce("q8 residual %s" % (dims,))
+    64 / 128 input channels take the streaming 1x1 kernel (also with several pixel
+    tiles per workgroup), 256 the weights-in-registers kernel."""
+    announce("q8 residual %s tiles/wg %d" % (dims, tiles_per_wg))
+    if tiles_per_wg:
+        monkeypatch.setenv("ODLA_HIP_LEAN_TILES", str(tiles_per_wg))
     r = rng(7)
     N, C, H, W, O = dims
     x = r.standard_normal((N, C, H, W)).astype(np.float32)

@@ -169,6 +169,44 @@ def test_conv_parity(case, mode):
         assert np.max(np.abs(got["y"] - want["y"])) <= tol * max(1.0, float(np.max(np.abs(want["y"]))))
 
 
+LEAN_CASES = [
+    # 1x1 filters over 64 / 128 bytes of input channels per pixel (the streaming kernel):
+    # N, C, H, W, O, stride, residual
+    (3, 64, 23, 17, 256, 1, True),
+    (2, 64, 20, 20, 200, 2, False),
+    (4, 32, 19, 19, 130, 1, True),
+    (1, 32, 40, 40, 64, 1, False),
+]
+
+
+@pytest.mark.parametrize("tiles_per_wg", [0, 3])
+@pytest.mark.parametrize("case", LEAN_CASES)
+@pytest.mark.parametrize("mode", ["fp16", "bf16"])
+def test_conv_1x1_short_k(case, mode, tiles_per_wg, monkeypatch):
+    N, C, H, W, O, s, with_res = case
+    announce("conv 1x1 short K %s %s tiles/wg %d" % (mode, case, tiles_per_wg))
+    if tiles_per_wg:
+        monkeypatch.setenv("ODLA_HIP_LEAN_TILES", str(tiles_per_wg))
+    r = rng(7 * O + C)
+    w = (r.standard_normal((O, C, 1, 1)) * np.sqrt(2.0 / C)).astype(np.float32)
+    bias = r.standard_normal(O).astype(np.float32)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    Ho, Wo = (H - 1) // s + 1, (W - 1) // s + 1
+    res = r.standard_normal((N, O, Ho, Wo)).astype(np.float32)
+
+    def build(b):
+        v = b.relu(b.arg("x", (N, C, H, W)), name="xr")
+        y = b.conv(v, b.const("w", w), b.const("b", bias), (s, s), (0, 0, 0, 0), name="y")
+        if with_res:
+            y = b.add(y, b.relu(b.arg("res", res.shape), name="rr"), name="sum")
+        b.output(b.relu(y, name="out"), "out")
+
+    feeds = {"x": x, "res": res} if with_res else {"x": x}
+    got, want = run_both(build, feeds, fp16=(mode == "fp16"), bf16=(mode == "bf16"))
+    tol = 2e-2 if mode == "fp16" else 6e-2
+    assert np.max(np.abs(got["out"] - want["out"])) <= tol * max(1.0, float(np.max(np.abs(want["out"]))))
+
+
 def test_conv_fused_chain_fp32():
     """Conv + per-channel Add + BatchNorm + residual Add + ReLU collapses into one
     launch and must equal the unfused oracle sequence."""
@@ -245,6 +283,10 @@ GEMM_CASES = [
     (200, 256, 192, False, False, 1.0, 1.0, "row", True),
     (130, 128, 96, False, True, 0.5, 1.0, "row", True),
     (70, 64, 300, True, False, 1.0, 0.0, None, True),
+    # few output tiles, long K: split along K into partial sums (classifier heads)
+    (64, 2048, 100, False, False, 1.0, 1.0, "row", True),
+    (256, 2048, 1000, False, True, 0.5, 1.0, "row", True),
+    (40, 1536, 130, False, False, 1.0, 0.0, None, True),
 ]
 
 
