@@ -319,15 +319,16 @@ def profile_roofline(L, sess, wl, dump_path=None):
     for i in range(n.value):
         name = buf[i].name.decode()
         total_ms += buf[i].ms
-        if name.startswith("conv") or name.startswith("gemm:"):
+        if name.startswith("conv") or name.startswith("gemm"):
             mm_ms += buf[i].ms
-            launches += 1
+            if not name.startswith("gemm.sum"):   # the reduction behind a split-K GEMM belongs to that GEMM
+                launches += 1
     achieved = wl.flop / (mm_ms * 1e-3) / 1e12 if mm_ms > 0 else 0.0
     peak = PEAK[wl.mode]
     roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
             "unit": "TOP/s" if wl.mode == "int8" else "TFLOP/s",
             "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(wl.name),
-            "kernel": "igemm_wreg_kernel / igemm_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
+            "kernel": "igemm_wreg_kernel / igemm_kernel / igemm_lean_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
                       "avg %.2f GFLOP per launch)" % (launches, 1e3 * mm_ms / max(launches, 1),
                                                      wl.flop / 1e9 / max(launches, 1)),
             "mm_ms_per_step": round(mm_ms, 4), "all_kernels_ms_per_step": round(total_ms, 4),
