@@ -119,6 +119,9 @@ struct EpiFloat {
     float v[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(acc[e], p.alpha, b8[e]);
+    // the activation comes before the residual in networks whose shortcut joins
+    // an already activated branch, behind it in the ResNet order
+    if (p.res_after_act) epi_act8(v, p.act, p.act_a, p.act_b);
     if (vec) {
       if (r != nullptr) {
         if constexpr (sizeof(TOut) == 4) {
@@ -133,7 +136,7 @@ struct EpiFloat {
           for (int e = 0; e < 8; ++e) v[e] += rv.get(e);
         }
       }
-      epi_act8(v, p.act, p.act_a, p.act_b);
+      if (!p.res_after_act) epi_act8(v, p.act, p.act_a, p.act_b);
       if constexpr (sizeof(TOut) == 4) {
         *reinterpret_cast<floatx4*>(y) = (floatx4){v[0], v[1], v[2], v[3]};
         *reinterpret_cast<floatx4*>(y + 4) = (floatx4){v[4], v[5], v[6], v[7]};
@@ -147,7 +150,7 @@ struct EpiFloat {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         if (e < nvalid && r != nullptr) v[e] += Store<TOut>::ld(r + e);
-      epi_act8(v, p.act, p.act_a, p.act_b);
+      if (!p.res_after_act) epi_act8(v, p.act, p.act_a, p.act_b);
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         if (e < nvalid) Store<TOut>::st(y + e, v[e]);

@@ -96,6 +96,7 @@ struct IgemmParams {
   float alpha = 1.0f;              // scales the accumulator before bias (float types)
   ActKind act = ACT_NONE;
   float act_a = 0.0f, act_b = 0.0f;  // leaky slope / clamp lo,hi
+  bool res_after_act = false;        // float types: y = act(..) + residual instead of act(.. + residual)
   // int8 only -----------------------------------------------------------
   // out_dt == DT_I8 : q = clamp(rne(float(acc+bias) * qmul[n]) + q_zp, q_lo, 255)
   //                   then, if residual: the unfused sequence
@@ -276,8 +277,12 @@ hipError_t launch_arg_extreme(const void* x, void* y, DType in_dt, DType out_dt,
 // y = ((sum q - len*zp) / len) * scale.
 hipError_t launch_reduce_q8_mean(const void* x, float* y, int64_t outer, int64_t len, int64_t inner,
                                  float scale, int zp, hipStream_t stream);
+// add (optional, type of x): softmax(x + add) where add holds one row of `len`
+// values per add_div consecutive rows of x (an attention mask); only for
+// inner == 1 and rows of at most 256 16-byte vectors.
 hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
-                          int64_t len, int64_t inner, bool log_softmax, hipStream_t stream);
+                          int64_t len, int64_t inner, bool log_softmax, hipStream_t stream,
+                          const void* add = nullptr, int64_t add_div = 1);
 // y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last `len` elements.
 hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int64_t len,
                             const float* gamma, const float* beta, float eps,

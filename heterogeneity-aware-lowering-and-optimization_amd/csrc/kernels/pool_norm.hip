@@ -417,7 +417,10 @@ __device__ __forceinline__ void store_row_vec(TO* dst, const float* v) {
 
 template <typename TI, typename TO, int LPR, int PER>
 __global__ void __launch_bounds__(kThreads)
-softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, int len, bool logsm) {
+softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, int len, bool logsm,
+                   const TI* __restrict__ add, int64_t add_div) {
+  // add: optional term added to the input first (attention masks), one row of
+  // `len` values shared by add_div consecutive rows of x
   constexpr int V = Vec16<TI>::N;
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63;
@@ -429,6 +432,7 @@ softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
     const int64_t r = r0 + lane / LPR;
     const bool row_ok = r < rows;
     const TI* row = x + (row_ok ? r : 0) * (int64_t)len;
+    const TI* arow = add ? add + ((row_ok ? r : 0) / add_div) * (int64_t)len : nullptr;
     float v[PER][V];
     float mx = -INFINITY;
 #pragma unroll
@@ -437,8 +441,15 @@ softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
       if (vi < nv && row_ok) {
         Vec16<TI> t;
         t.load(row + vi * V);
+        if (arow != nullptr) {
+          Vec16<TI> ta;
+          ta.load(arow + vi * V);
 #pragma unroll
-        for (int e = 0; e < V; ++e) { v[k][e] = t.get(e); mx = fmaxf(mx, v[k][e]); }
+          for (int e = 0; e < V; ++e) { v[k][e] = t.get(e) + ta.get(e); mx = fmaxf(mx, v[k][e]); }
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) { v[k][e] = t.get(e); mx = fmaxf(mx, v[k][e]); }
+        }
       } else {
 #pragma unroll
         for (int e = 0; e < V; ++e) v[k][e] = -INFINITY;
@@ -720,16 +731,18 @@ hipError_t launch_arg_extreme(const void* x, void* y, DType in_dt, DType out_dt,
 
 template <typename TI, typename TO>
 static hipError_t softmax_typed(const void* x, void* y, int64_t outer, int64_t len, int64_t inner,
-                                bool logsm, hipStream_t stream) {
+                                bool logsm, hipStream_t stream, const void* add = nullptr, int64_t add_div = 1) {
   constexpr int V = 16 / (int)sizeof(TI);
-  if (inner == 1 && len % V == 0 && len / V <= 256 && al16(x) && (sizeof(TO) != sizeof(TI) || al16(y))) {
+  const bool vec_ok = inner == 1 && len % V == 0 && len / V <= 256 && al16(x) && (sizeof(TO) != sizeof(TI) || al16(y));
+  if (add != nullptr && (!vec_ok || !al16(add) || add_div <= 0)) return hipErrorInvalidValue;
+  if (vec_ok) {
     const int nv = (int)(len / V);
     int lpr = 1;
     while (lpr < nv && lpr < 64) lpr <<= 1;
     const int per = (nv + lpr - 1) / lpr;
     const int rpw = 64 / lpr;
     const int grid = grid_for((outer + rpw - 1) / rpw * 64, kThreads);
-#define SMV(LPR_, PER_) hipLaunchKernelGGL((softmax_vec_kernel<TI, TO, LPR_, PER_>), dim3(grid), dim3(kThreads), 0, stream, (const TI*)x, (TO*)y, outer, (int)len, logsm)
+#define SMV(LPR_, PER_) hipLaunchKernelGGL((softmax_vec_kernel<TI, TO, LPR_, PER_>), dim3(grid), dim3(kThreads), 0, stream, (const TI*)x, (TO*)y, outer, (int)len, logsm, (const TI*)add, add_div)
     if (lpr <= 8) SMV(8, 1);
     else if (lpr == 16) SMV(16, 1);
     else if (lpr == 32) SMV(32, 1);
@@ -757,10 +770,12 @@ static hipError_t softmax_typed(const void* x, void* y, int64_t outer, int64_t l
 }
 
 hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int64_t outer,
-                          int64_t len, int64_t inner, bool log_softmax, hipStream_t stream) {
+                          int64_t len, int64_t inner, bool log_softmax, hipStream_t stream,
+                          const void* add, int64_t add_div) {
   if (!x || !y || outer <= 0 || len <= 0 || inner <= 0 || len >= (1ll << 31)) return hipErrorInvalidValue;
 #define SM_CASE(I_, O_, TI_, TO_) \
-  if (in_dt == I_ && out_dt == O_) return softmax_typed<TI_, TO_>(x, y, outer, len, inner, log_softmax, stream);
+  if (in_dt == I_ && out_dt == O_)  \
+    return softmax_typed<TI_, TO_>(x, y, outer, len, inner, log_softmax, stream, add, add_div);
   SM_CASE(DT_F32, DT_F32, float, float)
   SM_CASE(DT_F16, DT_F16, f16_t, f16_t)
   SM_CASE(DT_BF16, DT_BF16, bf16_t, bf16_t)

@@ -76,6 +76,7 @@ struct Epilogue {
   ActKind act = ACT_NONE;
   float act_a = 0.f, act_b = 0.f;
   _odla_value* pre_residual_value = nullptr;  // value right before the residual Add
+  bool res_after_act = false;                 // the residual joins behind the activation
   _odla_value* final_value = nullptr;
 };
 
@@ -461,6 +462,8 @@ class Planner {
   void lower_rownorm(int ni);
   void emit_stats(const _odla_value* v, const char* op_type, int forced_axis, const Node* producer);
   bool calib_ = false;
+  struct SoftmaxAdd { const _odla_value* x; const _odla_value* mask; int64_t div; };
+  std::unordered_map<int, SoftmaxAdd> softmax_add_;  // index of a folded Add's result -> its operands
 
   void collect_epilogue(int ni, int64_t out_channels, int channel_axis_of_output, Epilogue* ep);
   bool per_channel_constant(const _odla_value* k, const Shape& aligned, const Shape& out, int ch_axis,
@@ -839,6 +842,21 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
     ep->final_value = cur;
     if (ep->act != ACT_NONE) break;
   }
+  // Shortcut behind the activation (y = act(conv) + x, the Darknet order): one more follower.
+  if (!q8 && ep->act != ACT_NONE && ep->residual == nullptr && !cur->is_output && consumers_[cur->index].size() == 1) {
+    Node& nx = comp_->nodes[consumers_[cur->index][0]];
+    if (!nx.absorbed && nx.op == OP_BINARY && nx.i[0] == BIN_ADD && nx.out->shape == cur->shape) {
+      _odla_value* other = nx.in[0] == cur ? nx.in[1] : nx.in[0];
+      if (other != cur && other->kind != _odla_value::CONSTANT && other->shape == cur->shape && available(other) &&
+          storage_dtype(other) == storage_dtype(cur)) {
+        ep->residual = other;
+        ep->pre_residual_value = cur;
+        ep->res_after_act = true;
+        nx.absorbed = true;
+        ep->final_value = nx.out;
+      }
+    }
+  }
 }
 
 // ------------------------------------------------------------------ weights --
@@ -1005,6 +1023,7 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
   ip.act = ep.act;
   ip.act_a = ep.act_a;
   ip.act_b = ep.act_b;
+  ip.res_after_act = ep.res_after_act;
   const int tf = make_wfrag(name, &ip, tw);
   const bool hf = tf >= 0;
   const Ref rf = ref(hf ? tf : tx);
@@ -1529,6 +1548,32 @@ void Planner::lower_binary(int ni) {
   for (int i = 0; i < r; ++i) { sa.d[i] = n.iv[1 + i]; sb.d[i] = n.iv[1 + r + i]; }
   const DType dt = storage_dtype(outv);
 
+  // x + mask -> Softmax over the last axis (attention): the Softmax launch adds
+  // the mask itself.  The mask must hold whole rows shared by a block of
+  // consecutive rows of x: leading dims equal, then 1s, then the row length.
+  if (!calib_ && n.i[0] == BIN_ADD && dtype_is_float(dt) && !outv->is_output && consumers_[outv->index].size() == 1 && r >= 2) {
+    const Node& nx = comp_->nodes[consumers_[outv->index][0]];
+    const int64_t len = os.d[r - 1];
+    const int vecn = 16 / dtype_size(dt);
+    if (nx.op == OP_SOFTMAX && !nx.absorbed && (int)nx.i[0] == r - 1 && len % vecn == 0 && len / vecn <= 256) {
+      for (int side = 0; side < 2; ++side) {
+        const _odla_value* xv = side == 0 ? a : b;
+        const _odla_value* mv = side == 0 ? b : a;
+        const Shape& sx = side == 0 ? sa : sb;
+        const Shape& sm = side == 0 ? sb : sa;
+        if (!(sx == os) || sm.d[r - 1] != len || storage_dtype(mv) != dt) continue;
+        int p = 0;
+        while (p < r - 1 && sm.d[p] == os.d[p]) ++p;
+        bool ones = true;
+        int64_t div = 1;
+        for (int i = p; i < r - 1; ++i) { ones = ones && sm.d[i] == 1; div *= os.d[i]; }
+        if (!ones) continue;
+        softmax_add_[outv->index] = {xv, mv, div};
+        return;  // nothing to launch here: lower_softmax picks it up
+      }
+    }
+  }
+
   // optional trailing activation
   ActKind act = ACT_NONE;
   float act_a = 0.f, act_b = 0.f;
@@ -1992,20 +2037,32 @@ void Planner::lower_softmax(int ni) {
   const _odla_value* x = n.in[0];
   const Shape& xs = x->shape;
   const int axis = (int)n.i[0];
+  int tadd = -1;
+  int64_t add_div = 1;
+  {
+    auto it = softmax_add_.find(x->index);
+    if (it != softmax_add_.end()) {  // the Add in front was folded into this launch
+      x = it->second.x;
+      tadd = get(it->second.mask, L_ROWMAJOR, FORM_FLOAT);
+      add_div = it->second.div;
+    }
+  }
   const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
   int64_t outer = 1, inner = 1;
   for (int i = 0; i < axis; ++i) outer *= xs.d[i];
   for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
   const int64_t len = xs.d[axis];
   const DType dt = T(tx).dt;
+  if (tadd >= 0 && T(tadd).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "softmax mask storage type mismatch");
   // a graph output is written in fp32 directly
   const bool to_f32 = n.out->is_output && dtype_from_odla(n.out->etype) == DT_F32 && consumers_[n.out->index].empty();
   const DType odt = to_f32 ? DT_F32 : dt;
   const int ty = new_tensor(odt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
   const bool logsm = n.i[1] != 0;
-  const Ref a = ref(tx), b = ref(ty);
-  emit("softmax:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
-    return launch_softmax(a(e), b(e), dt, odt, outer, len, inner, logsm, st);
+  const Ref a = ref(tx), b = ref(ty), m = ref(tadd >= 0 ? tadd : tx);
+  const bool has_add = tadd >= 0;
+  emit("softmax:" + n.out->name, {tx, tadd}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    return launch_softmax(a(e), b(e), dt, odt, outer, len, inner, logsm, st, has_add ? m(e) : nullptr, add_div);
   });
   set_main(n.out, ty);
 }

@@ -207,6 +207,59 @@ def test_conv_1x1_short_k(case, mode, tiles_per_wg, monkeypatch):
     assert np.max(np.abs(got["out"] - want["out"])) <= tol * max(1.0, float(np.max(np.abs(want["out"]))))
 
 
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+@pytest.mark.parametrize("dims", [(2, 16, 13, 13, 32, 3), (1, 64, 12, 12, 128, 1), (2, 128, 9, 9, 160, 3)])
+def test_conv_activation_then_shortcut(dims, mode):
+    """y = LeakyReLU(conv(x)) + shortcut: the residual joins behind the activation (the
+    order of Darknet's shortcut layers); one launch, equal to the unfused oracle sequence."""
+    announce("conv act then shortcut %s %s" % (dims, mode))
+    N, C, H, W, O, k = dims
+    r = rng(31 + O)
+    w = (r.standard_normal((O, C, k, k)) * np.sqrt(2.0 / (C * k * k))).astype(np.float32)
+    bias = r.standard_normal(O).astype(np.float32)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    sc = r.standard_normal((N, O, H, W)).astype(np.float32)
+
+    def build(b):
+        v = b.arg("x", x.shape)
+        s = b.relu(b.arg("sc", sc.shape), name="scr")
+        y = b.conv(v, b.const("w", w), b.const("b", bias), (1, 1), (k // 2,) * 4, name="y")
+        b.output(b.add(b.leaky_relu(y, 0.1, name="act"), s, name="out"), "out")
+
+    got, want = run_both(build, {"x": x, "sc": sc}, fp16=(mode == "fp16"))
+    if mode == "fp32":
+        assert max_rel_err(got["out"], want["out"]) <= F32_TOL
+    else:
+        assert np.max(np.abs(got["out"] - want["out"])) <= 2e-2 * max(1.0, float(np.max(np.abs(want["out"]))))
+
+
+@pytest.mark.parametrize("mode", ["fp32", "bf16"])
+def test_masked_softmax_fused(mode):
+    """softmax(scores + mask) with the attention mask shapes [B,1,1,S] and [1,1,S,S], a
+    full-shape term, and a mask that cannot be folded (broadcast along the row)."""
+    announce("masked softmax %s" % mode)
+    r = rng(37)
+    B, H, S = 3, 4, 64
+    scores = (r.standard_normal((B, H, S, S)) * 2).astype(np.float32)
+    pad = np.where(r.random((B, 1, 1, S)) < 0.25, -10000.0, 0.0).astype(np.float32)
+    causal = np.triu(np.full((S, S), -10000.0, np.float32), 1).reshape(1, 1, S, S)
+    full = r.standard_normal((B, H, S, S)).astype(np.float32)
+    col = r.standard_normal((B, H, S, 1)).astype(np.float32)
+
+    def build(b):
+        s = b.arg("scores", scores.shape)
+        b.output(b.softmax(b.add(s, b.arg("pad", pad.shape), name="a0"), -1, name="p0"), "p0")
+        b.output(b.softmax(b.add(b.const("causal", causal), s, name="a1"), -1, name="p1"), "p1")
+        b.output(b.softmax(b.add(s, b.arg("full", full.shape), name="a2"), -1, name="p2"), "p2")
+        b.output(b.softmax(b.add(s, b.arg("col", col.shape), name="a3"), -1, name="p3"), "p3")
+
+    got, want = run_both(build, {"scores": scores, "pad": pad, "full": full, "col": col}, bf16=(mode == "bf16"))
+    for k in want:
+        tol = 1e-4 if mode == "fp32" else 3e-2
+        assert np.max(np.abs(got[k] - want[k])) <= tol, k
+        assert np.max(np.abs(got[k].sum(-1) - 1.0)) <= (1e-4 if mode == "fp32" else 2e-2), k
+
+
 def test_conv_fused_chain_fp32():
     """Conv + per-channel Add + BatchNorm + residual Add + ReLU collapses into one
     launch and must equal the unfused oracle sequence."""
