@@ -88,7 +88,34 @@ __device__ __forceinline__ float epi_act(float v, ActKind act, float a, float b)
 // Eight values at once: the (wavefront-uniform) switch is taken once, not per
 // element - per element it compiles to a tree of scalar branches that costs
 // more than the arithmetic of the whole epilogue.
+template <bool kRich = false>
 __device__ __forceinline__ void epi_act8(float (&v)[8], ActKind act, float a, float b) {
+  if constexpr (kRich) {
+    // Variant with the transcendental activations (GELU behind a feed-forward
+    // GEMM, Sigmoid / Tanh gates): a separate instantiation, so that the common
+    // epilogue stays small.
+    // (one element after the other: interleaving eight polynomial evaluations
+    // would take the registers the accumulators of the other slices live in)
+    switch (act) {
+      case ACT_GELU_ERF:
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { v[e] = gelu_erf(v[e]); __builtin_amdgcn_sched_barrier(0); }
+        return;
+      case ACT_GELU_TANH:
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { v[e] = gelu_tanh(v[e]); __builtin_amdgcn_sched_barrier(0); }
+        return;
+      case ACT_SIGMOID:
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { v[e] = 1.0f / (1.0f + expf(-v[e])); __builtin_amdgcn_sched_barrier(0); }
+        return;
+      case ACT_TANH:
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { v[e] = tanhf(v[e]); __builtin_amdgcn_sched_barrier(0); }
+        return;
+      default: break;
+    }
+  }
   switch (act) {
     case ACT_RELU:
 #pragma unroll
@@ -106,7 +133,7 @@ __device__ __forceinline__ void epi_act8(float (&v)[8], ActKind act, float a, fl
   }
 }
 
-template <typename TOut>
+template <typename TOut, bool kRich = false>
 struct EpiFloat {
   using AccE = float;
   using RVec = uintx4;  // eight 2-byte residual elements fetched ahead of use
@@ -121,7 +148,7 @@ struct EpiFloat {
     for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(acc[e], p.alpha, b8[e]);
     // the activation comes before the residual in networks whose shortcut joins
     // an already activated branch, behind it in the ResNet order
-    if (p.res_after_act) epi_act8(v, p.act, p.act_a, p.act_b);
+    if (p.res_after_act) epi_act8<kRich>(v, p.act, p.act_a, p.act_b);
     if (vec) {
       if (r != nullptr) {
         if constexpr (sizeof(TOut) == 4) {
@@ -136,7 +163,7 @@ struct EpiFloat {
           for (int e = 0; e < 8; ++e) v[e] += rv.get(e);
         }
       }
-      if (!p.res_after_act) epi_act8(v, p.act, p.act_a, p.act_b);
+      if (!p.res_after_act) epi_act8<kRich>(v, p.act, p.act_a, p.act_b);
       if constexpr (sizeof(TOut) == 4) {
         *reinterpret_cast<floatx4*>(y) = (floatx4){v[0], v[1], v[2], v[3]};
         *reinterpret_cast<floatx4*>(y + 4) = (floatx4){v[4], v[5], v[6], v[7]};
@@ -150,7 +177,7 @@ struct EpiFloat {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         if (e < nvalid && r != nullptr) v[e] += Store<TOut>::ld(r + e);
-      if (!p.res_after_act) epi_act8(v, p.act, p.act_a, p.act_b);
+      if (!p.res_after_act) epi_act8<kRich>(v, p.act, p.act_a, p.act_b);
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         if (e < nvalid) Store<TOut>::st(y + e, v[e]);
@@ -245,8 +272,8 @@ struct EpiQuant {
 };
 
 template <typename Epi> struct EpiTraits;
-template <typename T> struct EpiTraits<EpiFloat<T>> { using TOut = T; static constexpr bool quant = false; };
-template <int M> struct EpiTraits<EpiQuant<M>> { using TOut = typename QuantOut<M>::T; static constexpr bool quant = true; };
+template <typename T, bool R> struct EpiTraits<EpiFloat<T, R>> { using TOut = T; static constexpr bool quant = false; static constexpr bool rich = R; };
+template <int M> struct EpiTraits<EpiQuant<M>> { using TOut = typename QuantOut<M>::T; static constexpr bool quant = true; static constexpr bool rich = false; };
 
 // ---------------------------------------------------------------------------
 // Epilogue shared by the kernels below: each wavefront parks one 32-pixel slice
@@ -482,8 +509,11 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     __builtin_amdgcn_sched_barrier(0);
   };
   lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  // One call per 32-pixel slice with the slice number as a constant: a loop the
+  // optimizer declines to unroll would index the accumulators dynamically and
+  // move them to scratch memory.
+  auto slice = [&](auto slice_no) __attribute__((always_inline)) {
+    constexpr int i = decltype(slice_no)::value;
     AccE* tile = reinterpret_cast<AccE*>(smem) + (i & 1) * TILE_WORDS;
     // park: lane holds, for pixel l32, channels wave*32 + q*8 + lg*4 + (0..3)
 #pragma unroll
@@ -530,7 +560,12 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     }
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps) rcur[ps] = rnxt[ps];
-  }
+  };
+  static_assert(TM == 4, "one call per slice below");
+  slice(std::integral_constant<int, 0>{});
+  slice(std::integral_constant<int, 1>{});
+  slice(std::integral_constant<int, 2>{});
+  slice(std::integral_constant<int, 3>{});
 }
 
 // ---------------------------------------------------------------------------
@@ -739,7 +774,9 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
 // wait is a compile-time constant.  Padding taps and out-of-range rows fetch a
 // 16-byte fill vector stored behind the weight fragments.
 template <typename TIn, typename Epi>
-__global__ void __launch_bounds__(256, 3)  // three wavefronts per SIMD: at most 168 registers
+// three wavefronts per SIMD: at most 168 registers (two with the transcendental
+// activations in the epilogue, which need more)
+__global__ void __launch_bounds__(256, EpiTraits<Epi>::rich ? 2 : 3)
 igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   constexpr int BM = 128, BN = 128, WM = 128, WN = 32, NW = 4;
   constexpr int ES = sizeof(TIn);
@@ -1214,7 +1251,9 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
   if (!aligned16(p.x) || !aligned16(p.w)) return hipErrorInvalidValue;
   if (p.N <= 0 || p.H <= 0 || p.W <= 0 || p.Ho <= 0 || p.Wo <= 0 || p.Kout <= 0 || p.batch <= 0)
     return hipErrorInvalidValue;
-  if (p.act != ACT_NONE && p.act != ACT_RELU && p.act != ACT_LEAKY && p.act != ACT_CLAMP) return hipErrorInvalidValue;
+  const bool rich = p.act == ACT_GELU_ERF || p.act == ACT_GELU_TANH || p.act == ACT_SIGMOID || p.act == ACT_TANH;
+  if (p.act != ACT_NONE && p.act != ACT_RELU && p.act != ACT_LEAKY && p.act != ACT_CLAMP && !rich) return hipErrorInvalidValue;
+  if (rich && (p.in_dt == DT_I8 || p.out_dt != p.in_dt)) return hipErrorInvalidValue;
   if (p.R <= 0 || p.S <= 0 || p.sh <= 0 || p.sw <= 0 || p.dh <= 0 || p.dw <= 0) return hipErrorInvalidValue;
   if (p.xcs < p.C || p.ycs < p.Kout) return hipErrorInvalidValue;
   if ((int64_t)p.H * p.W * p.xcs >= (1ll << 31)) return hipErrorInvalidValue;
@@ -1248,12 +1287,15 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
   switch (p.in_dt) {
     case DT_F32:
       if (p.out_dt != DT_F32) return hipErrorInvalidValue;
+      if (rich) return dispatch<float, EpiFloat<float, true>>(p, epi_vec, stream);
       return dispatch<float, EpiFloat<float>>(p, epi_vec, stream);
     case DT_F16:
+      if (p.out_dt == DT_F16 && rich) return dispatch<f16_t, EpiFloat<f16_t, true>>(p, epi_vec, stream);
       if (p.out_dt == DT_F16) return dispatch<f16_t, EpiFloat<f16_t>>(p, epi_vec, stream);
       if (p.out_dt == DT_F32) return dispatch<f16_t, EpiFloat<float>>(p, epi_vec, stream);
       return hipErrorInvalidValue;
     case DT_BF16:
+      if (p.out_dt == DT_BF16 && rich) return dispatch<bf16_t, EpiFloat<bf16_t, true>>(p, epi_vec, stream);
       if (p.out_dt == DT_BF16) return dispatch<bf16_t, EpiFloat<bf16_t>>(p, epi_vec, stream);
       if (p.out_dt == DT_F32) return dispatch<bf16_t, EpiFloat<float>>(p, epi_vec, stream);
       return hipErrorInvalidValue;

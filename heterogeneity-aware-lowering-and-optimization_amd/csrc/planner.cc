@@ -827,8 +827,11 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
       }
     } else if (nx.op == OP_UNARY && ep->act == ACT_NONE) {
       const ActKind a = (ActKind)nx.i[0];
-      // the igemm epilogue applies the cheap activations only
-      const bool fusable = q8 ? (a == ACT_RELU) : (a == ACT_RELU || a == ACT_LEAKY || a == ACT_CLAMP);
+      // the 8-bit epilogue clamps only; the float ones also have a variant with
+      // the transcendental activations (GELU behind a feed-forward GEMM)
+      const bool fusable = q8 ? (a == ACT_RELU)
+                              : (a == ACT_RELU || a == ACT_LEAKY || a == ACT_CLAMP || a == ACT_GELU_ERF ||
+                                 a == ACT_GELU_TANH || a == ACT_SIGMOID || a == ACT_TANH);
       if (fusable) {
         ep->act = a;
         ep->act_a = nx.f[0];

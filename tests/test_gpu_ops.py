@@ -233,6 +233,42 @@ def test_conv_activation_then_shortcut(dims, mode):
         assert np.max(np.abs(got["out"] - want["out"])) <= 2e-2 * max(1.0, float(np.max(np.abs(want["out"]))))
 
 
+@pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("act", ["gelu", "gelu_tanh", "sigmoid", "tanh"])
+def test_gemm_and_conv_with_fused_transcendental_activation(act, mode):
+    """Feed-forward GEMM + GELU (and the gate activations) in one launch: both the
+    weights-in-registers kernel (wide N) and the two-operand kernel (narrow N), and a conv."""
+    announce("fused %s %s" % (act, mode))
+    r = rng(41)
+    A = r.standard_normal((200, 128)).astype(np.float32)
+    Bw = (r.standard_normal((128, 192)) * 0.1).astype(np.float32)
+    Bn = (r.standard_normal((128, 24)) * 0.1).astype(np.float32)
+    bias_w, bias_n = r.standard_normal(192).astype(np.float32), r.standard_normal(24).astype(np.float32)
+    x = r.standard_normal((2, 64, 10, 10)).astype(np.float32)
+    w = (r.standard_normal((96, 64, 3, 3)) * 0.05).astype(np.float32)
+
+    def apply(b, v, name):
+        if act == "gelu":
+            return b.gelu(v, False, name=name)
+        if act == "gelu_tanh":
+            return b.gelu(v, True, name=name)
+        return getattr(b, act)(v, name=name)
+
+    def build(b):
+        a = b.arg("A", A.shape)
+        b.output(apply(b, b.gemm(a, b.const("Bw", Bw), b.const("bw", bias_w), name="gw"), "yw"), "yw")
+        b.output(apply(b, b.gemm(a, b.const("Bn", Bn), b.const("bn", bias_n), name="gn"), "yn"), "yn")
+        b.output(apply(b, b.conv(b.arg("x", x.shape), b.const("w", w), None, (1, 1), (1, 1, 1, 1), name="c"), "yc"), "yc")
+
+    got, want = run_both(build, {"A": A, "x": x}, fp16=(mode == "fp16"), bf16=(mode == "bf16"))
+    for k in want:
+        if mode == "fp32":
+            assert max_rel_err(got[k], want[k]) <= F32_TOL, k
+        else:
+            tol = 2e-2 if mode == "fp16" else 6e-2
+            assert np.max(np.abs(got[k] - want[k])) <= tol * max(1.0, float(np.max(np.abs(want[k])))), k
+
+
 @pytest.mark.parametrize("mode", ["fp32", "bf16"])
 def test_masked_softmax_fused(mode):
     """softmax(scores + mask) with the attention mask shapes [B,1,1,S] and [1,1,S,S], a
