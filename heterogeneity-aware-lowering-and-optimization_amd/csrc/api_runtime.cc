@@ -161,6 +161,12 @@ odla_status ensure_plan(_odla_computation* c) {
   return ODLA_SUCCESS;
 }
 
+}  // namespace
+namespace ohip {
+odla_status compile_computation(_odla_computation* c) { return ensure_plan(c); }
+}  // namespace ohip
+namespace {
+
 void drop_graph(_odla_context* ctx) {
   if (ctx->graph_exec) { (void)hipGraphExecDestroy(ctx->graph_exec); ctx->graph_exec = nullptr; }
   if (ctx->graph) { (void)hipGraphDestroy(ctx->graph); ctx->graph = nullptr; }

@@ -199,6 +199,11 @@ int odla_type_size(odla_element_type t);
 
 }  // namespace ohip
 
+struct _odla_executable {
+  _odla_computation* comp = nullptr;
+  bool owns = false;  // made by odla_LoadExecutable: destroying it destroys the computation
+};
+
 struct _odla_computation {
   std::vector<std::unique_ptr<_odla_value>> values;
   std::vector<ohip::Node> nodes;
@@ -213,6 +218,10 @@ struct _odla_computation {
   size_t planned_nodes = 0;          // size of `nodes` when the plan was built
   int live_contexts = 0;             // contexts created by the caller
   _odla_context* eager_ctx = nullptr;  // context behind odla_GetValueData(value, ptr, NULL)
+  _odla_executable executable;       // handle given out by odla_CompileComputation / odla_LoadExecutable
+  // quantisation table of a loaded computation (the caller's table is borrowed otherwise)
+  std::vector<odla_value_quant_info> owned_qtable;
+  std::vector<std::string> owned_qnames;
 };
 
 struct _odla_context {
@@ -238,6 +247,7 @@ void set_current_computation(_odla_computation* c);
 void forget_computation(_odla_computation* c);
 _odla_value* new_value(_odla_computation* c, _odla_value::Kind kind, odla_element_type et,
                        const Shape& shape, const odla_value_id id);
+odla_status compile_computation(_odla_computation* c);  // builds the plan if there is none yet
 }  // namespace ohip
 
 #endif

@@ -66,6 +66,24 @@ class ValueIds(ctypes.Structure):
     _fields_ = [("size", ctypes.c_size_t), ("value_ids", ctypes.c_char_p * ODLA_MAX_OUTPUTS)]
 
 
+class ResourceLocation(ctypes.Structure):
+    _fields_ = [("location_type", ctypes.c_int32), ("location", ctypes.c_void_p), ("size", ctypes.c_size_t)]
+
+
+ODLA_LOCATION_PATH, ODLA_LOCATION_MEMORY, ODLA_LOCATION_URI = range(3)
+
+
+def path_location(path):
+    """(location, keep-alive object) for a file path."""
+    buf = ctypes.create_string_buffer(path.encode())
+    return ResourceLocation(ODLA_LOCATION_PATH, ctypes.cast(buf, ctypes.c_void_p), 0), buf
+
+
+def memory_location(data):
+    buf = ctypes.create_string_buffer(bytes(data), len(data))
+    return ResourceLocation(ODLA_LOCATION_MEMORY, ctypes.cast(buf, ctypes.c_void_p), len(data)), buf
+
+
 class QuantInfo(ctypes.Structure):
     _fields_ = [("value_id", ctypes.c_char_p), ("ch_idx", ctypes.c_int), ("scale", ctypes.c_float),
                 ("offset", ctypes.c_float), ("min", ctypes.c_float), ("max", ctypes.c_float)]
@@ -191,6 +209,18 @@ def load_library(path=None):
     proto("odla_Quantize", vp, [vp, vp, vp, i32, i32, cid])
     proto("odla_Dequantize", vp, [vp, vp, vp, i32, i32, cid])
     proto("odla_NMS", vp, [vp, vp, u32, f32, f32, T, cid])
+    RL = ResourceLocation
+    proto("odla_StoreComputation", i32, [RL, vp])
+    proto("odla_LoadComputation", i32, [RL, ctypes.POINTER(vp)])
+    proto("odla_CompileComputation", i32, [vp, vp, ctypes.POINTER(vp)])
+    proto("odla_StoreExecutable", i32, [RL, vp])
+    proto("odla_LoadExecutable", i32, [RL, vp, ctypes.POINTER(vp)])
+    proto("odla_LaunchExecutable", i32, [vp, vp])
+    proto("odla_GetNumOfArgsFromExecutable", i32, [vp, pu32])
+    proto("odla_GetArgFromExecutableByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
+    proto("odla_GetNumOfOutputsFromExecutable", i32, [vp, pu32])
+    proto("odla_GetOutputFromExecutableByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
+    proto("odla_DestroyExecutable", i32, [vp])
     i64 = ctypes.c_int64
     for n in ("Reciprocal", "Ceil", "Floor", "Sign", "Sin", "Cos", "Tan", "ASin", "ACos", "ATan", "Sinh", "Cosh",
               "ASinh", "ACosh", "ATanh", "Softplus", "Softsign", "Not", "IsNaN"):

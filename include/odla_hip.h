@@ -732,6 +732,57 @@ odla_value odla_DeConv(odla_value input, odla_memory_layout input_layout,
                        const odla_value_id value_id);
 
 /* ------------------------------------------------------------------------ */
+/* Stored computations and executables.  What is stored is the recorded       */
+/* computation (values, constants by value, nodes, outputs, precision options */
+/* and quantisation table); compiling it again is a matter of milliseconds.   */
+/* Store while the constants' host data is still valid.  A loaded computation */
+/* becomes the calling thread's current one and owns all its data.            */
+/* ODLA_LOCATION_PATH for both directions, ODLA_LOCATION_MEMORY for loading.  */
+/* [ref: odla_compute.h:80-97,123-156,338-440;                                */
+/*  tensorrt/odla_tensorrt.cc:537-559,561-700,703-811]                        */
+/* ------------------------------------------------------------------------ */
+typedef enum {
+  ODLA_LOCATION_PATH,   /* NUL-terminated file path  */
+  ODLA_LOCATION_MEMORY, /* address + size of a buffer */
+  ODLA_LOCATION_URI     /* not supported             */
+} odla_resource_location_type;
+typedef struct {
+  odla_resource_location_type location_type;
+  const void* location;
+  odla_size_t size;
+} odla_resource_location;
+
+odla_status odla_StoreComputation(odla_resource_location location,
+                                  odla_computation computation);
+odla_status odla_LoadComputation(odla_resource_location location,
+                                 odla_computation* computation);
+/* Compiles (plans) the computation now instead of at the first
+ * odla_CreateContext; the executable is a handle on the computation. */
+odla_status odla_CompileComputation(const odla_computation computation,
+                                    const odla_device device,
+                                    odla_executable* executable);
+odla_status odla_StoreExecutable(odla_resource_location location,
+                                 odla_executable executable);
+odla_status odla_LoadExecutable(odla_resource_location location,
+                                odla_device device, odla_executable* executable);
+/* = odla_ExecuteComputation on the executable's computation */
+odla_status odla_LaunchExecutable(odla_executable executable,
+                                  odla_context context);
+odla_status odla_GetNumOfArgsFromExecutable(const odla_executable executable,
+                                            odla_uint32* num_args);
+odla_status odla_GetArgFromExecutableByIdx(const odla_executable executable,
+                                           const odla_uint32 arg_idx,
+                                           odla_value* arg_value);
+odla_status odla_GetNumOfOutputsFromExecutable(const odla_executable executable,
+                                               odla_uint32* num_outputs);
+odla_status odla_GetOutputFromExecutableByIdx(const odla_executable executable,
+                                              const odla_uint32 output_idx,
+                                              odla_value* output_value);
+/* Destroys the computation behind a loaded executable; a compiled one lives
+ * and dies with the caller's computation. */
+odla_status odla_DestroyExecutable(odla_executable executable);
+
+/* ------------------------------------------------------------------------ */
 /* Calibration profiler.  The control functions keep the names and meaning of */
 /* the reference's profiler library; between StartProfiling and StopProfiling */
 /* computations are compiled in fp32 with nothing fused and range statistics  */
