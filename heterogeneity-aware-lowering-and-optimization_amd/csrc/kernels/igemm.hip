@@ -229,17 +229,25 @@ struct EpiQuant {
       const float zp = (float)p.q_zp, lo = (float)p.q_lo;
       const float rzp = (float)p.r_zp, szp = (float)p.s_zp, slo = (float)p.s_lo;
       unsigned ow[2] = {0u, 0u};
+      if (r != nullptr) {
+        // q - zp = med3(t + zp, lo, 255) - zp = med3(t, lo - zp, 255 - zp): all integers
+        const float ulo = lo - zp, uhi = 255.f - zp;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float t = rintf((float)(acc[e] + b8[e]) * m8[e]);
-        float q = __builtin_amdgcn_fmed3f(t + zp, lo, 255.f);
-        if (r != nullptr) {
-          const float fa = (q - zp) * p.q_scale;
+        for (int e = 0; e < 8; ++e) {
+          const float t = rintf((float)(acc[e] + b8[e]) * m8[e]);
+          const float fa = __builtin_amdgcn_fmed3f(t, ulo, uhi) * p.q_scale;
           const float fb = ((float)((rw[e >> 2] >> (8 * (e & 3))) & 0xffu) - rzp) * p.r_scale;
           const float f = fa + fb;
-          q = __builtin_amdgcn_fmed3f(rintf(f * p.s_inv) + szp, slo, 255.f);
+          const float q = __builtin_amdgcn_fmed3f(rintf(f * p.s_inv) + szp, slo, 255.f);
+          ow[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(q, e & 3, ow[e >> 2]);
         }
-        ow[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(q, e & 3, ow[e >> 2]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float t = rintf((float)(acc[e] + b8[e]) * m8[e]);
+          const float q = __builtin_amdgcn_fmed3f(t + zp, lo, 255.f);
+          ow[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(q, e & 3, ow[e >> 2]);
+        }
       }
       ow[0] ^= 0x80808080u;  // levels -> stored
       ow[1] ^= 0x80808080u;
