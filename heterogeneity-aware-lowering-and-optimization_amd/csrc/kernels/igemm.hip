@@ -464,7 +464,8 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
 #pragma unroll
   for (int e = 0; e < 8; ++e) { b8[e] = 0; m8[e] = 0.f; }
   if (nvalid > 0) {
-    if (bias != nullptr) {
+    // (8-bit layers carry their bias in the accumulators already)
+    if (bias != nullptr && !EpiTraits<Epi>::quant) {
       if (vec) {
         const intx4 t0 = *reinterpret_cast<const intx4*>(bias + n);
         const intx4 t1 = *reinterpret_cast<const intx4*>(bias + n + 4);
@@ -888,6 +889,30 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[i][0][e] = 0;
+  if constexpr (EpiTraits<Epi>::quant) {
+    // 8-bit layers: the int32 bias starts in the accumulators (element q*4 + r of
+    // a lane is channel wave*32 + q*8 + (lane/32)*4 + r), which takes its addition
+    // out of the requantising epilogue, the busiest part of these layers.  The
+    // addresses are wavefront-uniform so that these are scalar loads: a vector
+    // load here would be one more operation in flight than the hand-counted
+    // waits of the K loop allow for.
+    if (p.bias != nullptr) {
+      const int* bias = reinterpret_cast<const int*>(p.bias) + (int64_t)z * p.bias_bs;
+      const int nb = tile_n * BN + __builtin_amdgcn_readfirstlane(wave) * 32;
+      const int last = p.Kout - 1;  // channels past the end are computed but never stored
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int c0 = nb + q * 8 + r, c1 = c0 + 4;
+          const int b0 = bias[c0 < last ? c0 : last], b1 = bias[c1 < last ? c1 : last];
+          const int b = lg ? b1 : b0;
+#pragma unroll
+          for (int i = 0; i < TM; ++i) acc[i][0][q * 4 + r] = b;
+        }
+      }
+    }
+  }
 
   const int nkt = p.wf_chunks / 4;
   // fragment read offsets: row l32 (+32*i), chunk 2*kk + lg, swizzled
@@ -899,16 +924,30 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   // direct-to-LDS loads the compiler would otherwise treat the vector-memory
   // counter as unordered and wait for everything in flight at each use.
   // wload: dst <- ptr[off bytes]; wwait<n>: dst is valid once at most n younger
-  // vector-memory operations are still in flight.
+  // vector-memory operations are still in flight.  A request inside the K loop
+  // names its register as input and output, which ties every request for a
+  // fragment to one physical register, and the wait behind the loop names all
+  // eight: the compiler then sees them occupied on every path out of the loop,
+  // also on those where the last requests are never consumed, and cannot hand
+  // one of them to another value while data is still on its way into it.
   // (The host pass only needs the kernel's launch stub; it cannot parse the
   // vector-register constraints.)
 #if defined(__HIP_DEVICE_COMPILE__)
 #define IGEMM_WLOAD(dst, ptr, OFF) \
   asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "=v"(dst) : "v"(ptr) : "memory")
+#define IGEMM_WRELOAD(dst, ptr, OFF) \
+  asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "+v"(dst) : "v"(ptr) : "memory")
 #define IGEMM_WWAIT15(dst) asm volatile("s_waitcnt vmcnt(15)" : "+v"(dst) : : "memory")
+#define IGEMM_WDRAIN(a, b)                                                                                     \
+  asm volatile("s_waitcnt vmcnt(0)"                                                                            \
+               : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) \
+               :                                                                                               \
+               : "memory")
 #else
 #define IGEMM_WLOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
+#define IGEMM_WRELOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
 #define IGEMM_WWAIT15(dst) (void)(dst)
+#define IGEMM_WDRAIN(a, b) (void)(a), (void)(b)
 #endif
   uintx4 w0[4], w1[4];
   {
@@ -960,10 +999,10 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) acc[i][0] = Mma<TIn>::run(wc[kk], fa[kk & 1][i], acc[i][0]);
       __builtin_amdgcn_sched_barrier(0);
-      if (kk == 0) IGEMM_WLOAD(wc[0], wnext, 0);
-      else if (kk == 1) IGEMM_WLOAD(wc[1], wnext, 1024);
-      else if (kk == 2) IGEMM_WLOAD(wc[2], wnext, 2048);
-      else IGEMM_WLOAD(wc[3], wnext, 3072);
+      if (kk == 0) IGEMM_WRELOAD(wc[0], wnext, 0);
+      else if (kk == 1) IGEMM_WRELOAD(wc[1], wnext, 1024);
+      else if (kk == 2) IGEMM_WRELOAD(wc[2], wnext, 2048);
+      else IGEMM_WRELOAD(wc[3], wnext, 3072);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -976,10 +1015,14 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
       buf = buf == 2 ? 0 : buf + 1;
     }
   }
+  // the ring becomes the staging area: no direct-to-LDS write may still be in
+  // flight, and neither may a weight fragment be
+  IGEMM_WDRAIN(w0, w1);
+  __builtin_amdgcn_sched_barrier(0);
 #undef IGEMM_WLOAD
+#undef IGEMM_WRELOAD
 #undef IGEMM_WWAIT15
-  // the ring becomes the staging area: no direct-to-LDS write may still be in flight
-  __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#undef IGEMM_WDRAIN
   igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
 }
 

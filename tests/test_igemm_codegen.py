@@ -5,10 +5,10 @@ speed rely on and that a compiler change could silently break:
     magnitude);
   * in igemm_wreg_kernel the weight fragments are requested by inline assembly
     into registers the compiler knows nothing about while the request is in
-    flight: between the pipeline fill and the wait that follows the K loop only
-    the MFMAs and those requests themselves may name these registers (a
-    compiler-inserted copy or reuse there would read or clobber data that has
-    not landed yet).
+    flight: each fragment keeps one register quad, and between the pipeline
+    fill and the wait that follows the K loop only the MFMAs and those requests
+    themselves may name these registers, on any path (a compiler-inserted copy
+    or reuse there would read or clobber data that has not landed yet).
 """
 import os
 import re
@@ -66,30 +66,34 @@ def test_weight_fragment_registers_untouched_in_flight(compiled):
     checked = 0
     for name, body in kernel_bodies(asm, "_ZN4ohip17igemm_wreg_kernel"):
         quads = {(int(m.group(1)), int(m.group(2))) for m in map(req.match, body) if m}
-        assert len(quads) >= 8, (name, quads)        # two sets of four fragments (plus those of a peeled first stage)
+        # Two sets of four fragments, each tied to one register quad for the
+        # whole K loop (also in stages the optimizer peels off the loop).
+        assert len(quads) == 8, (name, quads)
+        owned = {x for a, b in quads for x in range(a, b + 1)}
+        assert len(owned) == 32, (name, quads)
         mfma = [i for i, l in enumerate(body) if "v_mfma" in l]
         first = min(i for i, l in enumerate(body) if req.match(l))
         drain = min(i for i, l in enumerate(body) if i > mfma[-1] and l.startswith("s_waitcnt vmcnt(0)"))
-        # Walk the code in layout order.  A quad is "in flight" from its request
-        # until an MFMA consumes it (the kernel waits right before that MFMA);
-        # what is requested at the bottom of the loop body stays in flight up to
-        # the wait behind the loop.
-        in_flight = set()
+        assert first < mfma[0]
+        # From the first request to the wait behind the loop these registers
+        # belong to the requests and to the MFMAs that consume them, whatever
+        # path the control flow takes: any other instruction naming one of them
+        # would read data that may not have landed, or be overwritten by it.
         for i in range(first, drain):
             l = body[i]
-            m = req.match(l)
-            if m:
-                in_flight.add((int(m.group(1)), int(m.group(2))))
-                continue
-            if l.startswith(".LBB"):
+            if req.match(l) or l.startswith(".LBB"):
                 continue
             regs = []
             for r in re.finditer(r"v\[(\d+):(\d+)\]|\bv(\d+)\b", l):
                 regs += list(range(int(r.group(1)), int(r.group(2)) + 1)) if r.group(1) else [int(r.group(3))]
+            hit = [x for x in regs if x in owned]
             if "v_mfma" in l:
-                in_flight = {q for q in in_flight if not any(q[0] <= x <= q[1] for x in regs)}
+                # as the A operand only (v_mfma dst, a, b, c): never as destination or accumulator
+                ops = [o.strip() for o in l.split(None, 1)[1].split(",")]
+                for o in (ops[0], ops[3]):
+                    m = re.match(r"[av]\[(\d+):(\d+)\]", o)
+                    assert not (o.startswith("v") and m and any(x in owned for x in range(int(m.group(1)), int(m.group(2)) + 1))), (name, i, l)
                 continue
-            hit = [x for x in regs if any(a <= x <= b for a, b in in_flight)]
             assert not hit, (name, i, l)
         checked += 1
     assert checked >= 6
