@@ -994,6 +994,59 @@ odla_values odla_TopK(odla_value input, odla_uint32 K, odla_bool largest, odla_b
   return r;
 }
 
+// YOLOv3 post-processing of one image: decode of the 13-, 26- and 52-cell heads
+// and, per class, the boxes that survive the suppression walk.  Results: value
+// "<id>0" [classes, N / 169, 5] rows {y min, x min, y max, x max, score} in
+// source-image pixels, zero padded, and "<id>1" [classes] rows kept (N = boxes
+// of the three heads; the reference leaves the padding undefined and has no
+// bound on the rows of a class - here a class stops at its N / 169 rows).
+// [ref: ops/odla_ops_nn.h:744-759 (odla_PostProcess); popart odla_ops_nn.cc:462-484,
+//  custom_ops/postprocess.cc:67-81 (result shapes), :139-290, codelets_nms.cpp:24-125]
+odla_values odla_PostProcess(odla_value orig_img_w, odla_value orig_img_h, odla_value bb13, odla_value bb26,
+                             odla_value bb52, const odla_value_id value_id) {
+  odla_values none;
+  none.size = 0;
+  auto bail = [&](const char* msg) { OHIP_ERR("odla_PostProcess: %s", msg); return none; };
+  if (!orig_img_w || !orig_img_h || !bb13 || !bb26 || !bb52) return bail("null operand");
+  _odla_computation* c = comp_of(bb13);
+  if (c == nullptr) return bail("no current computation");
+  const odla_value heads[3] = {bb13, bb26, bb52};
+  const odla_value sizes[2] = {orig_img_w, orig_img_h};
+  for (odla_value s : sizes) {
+    if (s->etype != ODLA_UINT32 && s->etype != ODLA_INT32) return bail("the image size must be 32-bit integers");
+    if (s->shape.numel() != 1) return bail("the image size must be scalars");
+  }
+  int64_t total = 0;
+  for (odla_value h : heads) {
+    if (!is_float_type(h->etype)) return bail("the heads must be float tensors");
+    const Shape& s = h->shape;
+    if (s.rank != 4 || s.d[0] != 1) return bail("the heads must be [1, 3 * (5 + classes), dim, dim]");
+    if (s.d[2] != s.d[3] || s.d[2] < 1) return bail("a head is not square");
+    if (s.d[1] != bb13->shape.d[1]) return bail("the heads differ in channels");
+    total += 3 * s.d[2] * s.d[2];
+  }
+  const int64_t ch = bb13->shape.d[1];
+  if (ch % 3 != 0 || ch / 3 < 6) return bail("the channels of a head must be 3 * (5 + classes)");
+  const int64_t classes = ch / 3 - 5, capacity = total / 169;
+  if (capacity < 1) return bail("fewer than 169 boxes");
+  const std::string base = value_id ? std::string(reinterpret_cast<const char*>(value_id)) : std::string();
+  const std::string n0 = base + "0", n1 = base + "1";
+  Shape o0, o1;
+  o0.rank = 3; o0.d[0] = classes; o0.d[1] = capacity; o0.d[2] = 5;
+  o1.rank = 1; o1.d[0] = classes;
+  Node* n = add_node(c, OP_POSTPROCESS, {orig_img_w, orig_img_h, bb13, bb26, bb52}, ODLA_FLOAT32, o0,
+                     value_id ? (const odla_value_id)n0.c_str() : nullptr);
+  n->out2 = new_value(c, _odla_value::TEMP, ODLA_UINT32, o1, value_id ? (const odla_value_id)n1.c_str() : nullptr);
+  n->out2->producer = n->out->producer;
+  n->f[0] = 0.45f;  // IoU above which a box is suppressed
+  n->f[1] = 0.3f;   // lowest score that takes part
+  odla_values r;
+  r.size = 2;
+  r.values[0] = n->out;
+  r.values[1] = n->out2;
+  return r;
+}
+
 // [ref: ops/odla_ops_nn.h (odla_LRN); dnnl odla_dnnl.cc:1553-1581]
 odla_value odla_LRN(odla_value input, odla_memory_layout layout, odla_int32 window_size, odla_float32 alpha,
                     odla_float32 beta, odla_float32 bias, const odla_value_id id) {

@@ -34,7 +34,8 @@ void log_msg(const char* file, int line, const char* func, odla_log_level lvl, c
 enum OpKind : int {
   OP_CONV, OP_GEMM, OP_BINARY, OP_UNARY, OP_BATCHNORM, OP_LAYERNORM, OP_POOL, OP_REDUCE,
   OP_SOFTMAX, OP_CAST, OP_CONCAT, OP_GATHER, OP_RESHAPE, OP_RESIZE, OP_SLICE, OP_TRANSPOSE,
-  OP_QUANTIZE, OP_DEQUANTIZE, OP_NMS, OP_EWISE, OP_ARGEXT, OP_COPYND, OP_TOPK, OP_LRN, OP_ROWNORM
+  OP_QUANTIZE, OP_DEQUANTIZE, OP_NMS, OP_EWISE, OP_ARGEXT, OP_COPYND, OP_TOPK, OP_LRN, OP_ROWNORM,
+  OP_POSTPROCESS
 };
 const char* op_name(OpKind k);
 

@@ -344,5 +344,16 @@ hipError_t launch_nms(const float* boxes, const float* scores, int N, int C, int
                       int max_out, float iou_thr, float score_thr, int32_t* out,
                       void* workspace, hipStream_t stream);
 
+// YOLOv3 post-processing of one image: decode of three heads [3*(5+classes)][dim][dim]
+// (fp32, channels first) into `boxes` [total][4] (y min, x min, y max, x max in
+// source-image pixels) and `scores` [classes][total] (total = 3 * sum dim^2),
+// then per class the reference's suppression walk: `info` [classes][capacity][5]
+// rows {box, score}, zero padded, and `num` [classes] rows kept (at most capacity).
+// anchors[h] = {w0, h0, w1, h1, w2, h2} in pixels of the 416 x 416 network input.
+hipError_t launch_yolo_postprocess(const float* const heads[3], const int dims[3], int classes,
+                                   const int anchors[3][6], const int* img_w, const int* img_h, float iou_thr,
+                                   float score_thr, int capacity, float* boxes, float* scores, float* info,
+                                   int* num, hipStream_t stream);
+
 }  // namespace ohip
 #endif

@@ -460,6 +460,7 @@ class Planner {
   void lower_topk(int ni);
   void lower_lrn(int ni);
   void lower_rownorm(int ni);
+  void lower_postprocess(int ni);
   void emit_stats(const _odla_value* v, const char* op_type, int forced_axis, const Node* producer);
   bool calib_ = false;
   struct SoftmaxAdd { const _odla_value* x; const _odla_value* mask; int64_t div; };
@@ -706,6 +707,7 @@ void Planner::lower(int ni) {
     case OP_TOPK: lower_topk(ni); break;
     case OP_LRN: lower_lrn(ni); break;
     case OP_ROWNORM: lower_rownorm(ni); break;
+    case OP_POSTPROCESS: lower_postprocess(ni); break;
   }
 }
 
@@ -2439,6 +2441,51 @@ void Planner::lower_nms(int ni) {
   } else {
     set_main(n.out, ty);
   }
+}
+
+// -------------------------------------------------------- PostProcess ----
+// [ref: ODLA/platforms/odla_popart/custom_ops/postprocess.cc:139-290: anchors of
+//  the 13-, 26- and 52-cell heads, thresholds 0.45 / 0.3, N / 169 rows per class]
+void Planner::lower_postprocess(int ni) {
+  Node& n = comp_->nodes[ni];
+  auto as_f32 = [&](const _odla_value* v) -> int {
+    int t = get(v, L_ROWMAJOR, FORM_FLOAT);
+    if (T(t).dt == DT_F32) return t;
+    const int d = new_tensor(DT_F32, L_ROWMAJOR, v->shape, 0, SP_ARENA);
+    const int64_t ne = v->shape.numel();
+    const DType sdt = T(t).dt;
+    const Ref a = ref(t), b = ref(d);
+    emit("postprocess.cast:" + v->name, {t}, {d}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), DT_F32, ne, st); });
+    return d;
+  };
+  const int tw = get(n.in[0], L_ROWMAJOR, FORM_FLOAT), th = get(n.in[1], L_ROWMAJOR, FORM_FLOAT);
+  if (T(tw).dt != DT_I32 || T(th).dt != DT_I32) fail(ODLA_UNSUPPORTED_DATATYPE, "odla_PostProcess: the image size must be 32-bit integers");
+  const int t0 = as_f32(n.in[2]), t1 = as_f32(n.in[3]), t2 = as_f32(n.in[4]);
+  struct Args { int dims[3]; int anchors[3][6]; } a;
+  static const int kAnchors[3][6] = {{116, 90, 156, 198, 373, 326}, {30, 61, 62, 45, 59, 119}, {10, 13, 16, 30, 33, 23}};
+  int total = 0;
+  for (int h = 0; h < 3; ++h) {
+    a.dims[h] = (int)n.in[2 + h]->shape.d[2];
+    total += 3 * a.dims[h] * a.dims[h];
+    for (int k = 0; k < 6; ++k) a.anchors[h][k] = kAnchors[h][k];
+  }
+  const int classes = (int)n.out->shape.d[0], capacity = (int)n.out->shape.d[1];
+  Shape bs, ss;
+  bs.rank = 2; bs.d[0] = total; bs.d[1] = 4;
+  ss.rank = 2; ss.d[0] = classes; ss.d[1] = total;
+  const int tb = new_tensor(DT_F32, L_ROWMAJOR, bs, 0, SP_ARENA);
+  const int ts = new_tensor(DT_F32, L_ROWMAJOR, ss, 0, SP_ARENA);
+  const int ti = new_tensor(DT_F32, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const int tn = new_tensor(DT_I32, L_ROWMAJOR, n.out2->shape, 0, SP_ARENA);
+  const float iou = n.f[0], thr = n.f[1];
+  const Ref rw = ref(tw), rh = ref(th), r0 = ref(t0), r1 = ref(t1), r2 = ref(t2), rb = ref(tb), rs = ref(ts), ri = ref(ti), rn = ref(tn);
+  emit("postprocess:" + n.out->name, {tw, th, t0, t1, t2}, {tb, ts, ti, tn}, [=](const ExecEnv& e, hipStream_t st) {
+    const float* heads[3] = {(const float*)r0(e), (const float*)r1(e), (const float*)r2(e)};
+    return launch_yolo_postprocess(heads, a.dims, classes, a.anchors, (const int*)rw(e), (const int*)rh(e), iou, thr,
+                                   capacity, (float*)rb(e), (float*)rs(e), (float*)ri(e), (int*)rn(e), st);
+  });
+  set_main(n.out, ti);
+  set_main(n.out2, tn);
 }
 
 }  // namespace

@@ -155,6 +155,7 @@ const char* api_op_name(const Node& n) {
     case OP_TOPK: return "odla_TopK";
     case OP_LRN: return "odla_LRN";
     case OP_ROWNORM: return "odla_InstanceNormalization";
+    case OP_POSTPROCESS: return "odla_PostProcess";
   }
   return "odla_Op";
 }

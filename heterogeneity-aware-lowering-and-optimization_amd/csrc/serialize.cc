@@ -168,7 +168,7 @@ odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) 
   for (int64_t k = 0; k < nn; ++k) {
     Node n;
     const int64_t op = r.i64();
-    if (op < 0 || op > (int64_t)OP_ROWNORM) return ODLA_INVALID_PARAM;
+    if (op < 0 || op > (int64_t)OP_POSTPROCESS) return ODLA_INVALID_PARAM;
     n.op = (OpKind)op;
     const int64_t nin = r.i64();
     if (!r.ok || nin < 0 || nin > ODLA_MAX_OUTPUTS) return ODLA_INVALID_PARAM;

@@ -46,6 +46,7 @@ _NP_TO_ODLA = {
     np.dtype(np.float32): ODLA_FLOAT32, np.dtype(np.float16): ODLA_FLOAT16,
     np.dtype(np.int32): ODLA_INT32, np.dtype(np.int64): ODLA_INT64,
     np.dtype(np.int8): ODLA_INT8, np.dtype(np.uint8): ODLA_UINT8, np.dtype(np.bool_): ODLA_BOOL,
+    np.dtype(np.uint32): ODLA_UINT32,
 }
 _ODLA_TO_NP = {v: k for k, v in _NP_TO_ODLA.items()}
 
@@ -243,6 +244,7 @@ def load_library(path=None):
     proto("odla_ArgMax", vp, [vp, i32, u32, u32, T, cid])
     proto("odla_ArgMin", vp, [vp, i32, u32, u32, T, cid])
     proto("odla_TopK", Values, [vp, u32, u32, u32, u32, T, T, ValueIds])
+    proto("odla_PostProcess", Values, [vp, vp, vp, vp, vp, cid])
     proto("odla_Pad", vp, [vp, pu32, pu32, S, cid])
     proto("odla_Tile", vp, [vp, pu32, S, cid])
     proto("odla_ExpandDims", vp, [vp, S, cid])
@@ -564,6 +566,13 @@ class HipBuilder:
         r = self.L.odla_TopK(x, k, int(largest), 1, axis, make_type(np.float32, [1]), make_type(index_dtype, [1]), ids)
         if r.size != 2:
             raise OdlaError("odla_TopK failed (see the library log)")
+        return r.values[0], r.values[1]
+
+    def yolo_postprocess(self, img_w, img_h, bb13, bb26, bb52, name=None):
+        """-> (rows [classes, N/169, 5], rows kept [classes]); the values are named name+"0" / name+"1"."""
+        r = self.L.odla_PostProcess(img_w, img_h, bb13, bb26, bb52, _cid(name))
+        if r.size != 2:
+            raise OdlaError("odla_PostProcess failed (see the library log)")
         return r.values[0], r.values[1]
 
     def pad(self, x, front, back, name=None):

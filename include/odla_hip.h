@@ -684,6 +684,20 @@ odla_values odla_TopK(odla_value input, odla_uint32 K, odla_bool largest,
                       odla_value_type output_value_type,
                       odla_value_type output_value_index_type,
                       const odla_value_ids value_ids);
+/* YOLOv3 post-processing of one image (heads [1, 3*(5+classes), dim, dim],
+ * image size as two 32-bit integer scalars bound at run time): values[0] =
+ * "<id>0" FLOAT32 [classes, N/169, 5] rows {y min, x min, y max, x max,
+ * score} in source-image pixels, best first, zero padded; values[1] = "<id>1"
+ * UINT32 [classes] rows kept.  N = boxes of the three heads.  Score threshold
+ * 0.3 (>=), IoU threshold 0.45 (>), a box is compared with the box kept last
+ * only, equal scores are ordered by ascending box index.  The reference leaves
+ * the padding undefined and writes past N/169 rows; here a class stops there.
+ * [ref: ops/odla_ops_nn.h:744-759; popart odla_ops_nn.cc:462-484,
+ *  custom_ops/postprocess.cc:67-81, :139-290, custom_ops/codelets_nms.cpp:24-125;
+ *  models/vision/detection/yolo/yolov3_postproc.cc:34-153 (the host version)] */
+odla_values odla_PostProcess(odla_value orig_img_w, odla_value orig_img_h,
+                             odla_value bb13, odla_value bb26, odla_value bb52,
+                             const odla_value_id value_id);
 
 /* Data movement.
  * [ref: ops/odla_ops_process.h:117-130 (ExpandDims = broadcast), :221-236

@@ -26,6 +26,13 @@ Pin status (what fixes each function independently of this file):
       tests against torch's CPU operators.  TopK tie order (ascending index) is
       this build's choice: the reference's portable TopK is not implemented
       (``dnnl_utils.h:52-56``), so ties are PARITY UNPINNED.
+  yolo_decode / yolo_class_walk / yolo_postprocess   closed forms of the
+      decode (float64 sigmoid / exp), the same boxes from the Sigmoid / Exp
+      graph of the package's YOLOv3 builder, hand-worked walks that separate
+      "compare with the box kept last" from greedy suppression.  The order of
+      equal scores (ascending row) and the stop at N/169 rows per class are
+      this build's choices where the reference leaves the result open
+      (unstable sort; writes past the end): PARITY UNPINNED for those two.
   int8 convolution + requantisation (``qconv`` ...)   PARITY UNPINNED by the
       reference: it has no int8 convolution of its own.  The int32 accumulators
       are pinned by int64 brute force; the requantisation formula is this
@@ -292,6 +299,100 @@ def nms(boxes, scores, max_out, iou_thr, score_thr):
                 iou = _iou_one_to_many(boxes[n, bi], boxes[n, order[rest]])
                 alive[rest[iou >= np.float32(iou_thr)]] = False
     return out.reshape(N * max_out, 3)
+
+
+# --------------------------------------------------------------------------
+# YOLOv3 post-processing of one image
+#   [ref: models/vision/detection/yolo/yolov3_postproc.cc:34-88 (decode), :90-153 (per-class
+#    walk); ODLA/platforms/odla_popart/custom_ops/codelets_nms.cpp:24-125 and
+#    custom_ops/postprocess.cc:139-290 (the same two steps behind odla_PostProcess)]
+# --------------------------------------------------------------------------
+YOLO_ANCHORS = (10, 13, 16, 30, 33, 23, 30, 61, 62, 45, 59, 119, 116, 90, 156, 198, 373, 326)
+YOLO_ANCHOR_MASKS = ((6, 7, 8), (3, 4, 5), (0, 1, 2))   # heads with 13, 26 and 52 cells a side
+
+
+def yolo_decode(img_w, img_h, head, mask):
+    """head [1, 3*(5+C), dim, dim] -> rows [dim*dim*3, 5+C] in the reference's order
+    (cell row, cell column, anchor): {y min, x min, y max, x max, objectness, class scores}.
+    Arithmetic in the reference's mix of float and double: its locals are floats, the
+    literals 416.0 and 2.0 make the sub-expressions around them double."""
+    f32, f64 = np.float32, np.float64
+    head = _f32(head)
+    _, ch, dim, _ = head.shape
+    C = ch // 3 - 5
+    scale = f32(min(416.0 / img_h, 416.0 / img_w))
+    # std::round rounds halves away from zero
+    rnd = lambda v: f32(math.floor(abs(float(v)) + 0.5) * (1 if v >= 0 else -1))
+    new_h, new_w = rnd(f32(img_h) * scale), rnd(f32(img_w) * scale)
+    offset_h = f32(f64(f32(416) - new_h) / 2.0 / 416)
+    offset_w = f32(f64(f32(416) - new_w) / 2.0 / 416)
+    scale_h, scale_w = f32(416) / new_h, f32(416) / new_w
+    t = np.exp(head[0].transpose(1, 2, 0).reshape(dim, dim, 3, 5 + C)).astype(f32)   # channels last, all through exp
+    out = np.empty_like(t)
+    gx = np.arange(dim, dtype=f32).reshape(1, dim, 1)
+    gy = np.arange(dim, dtype=f32).reshape(dim, 1, 1)
+    aw = np.array([YOLO_ANCHORS[2 * m] for m in mask], f32).reshape(1, 1, 3)
+    ah = np.array([YOLO_ANCHORS[2 * m + 1] for m in mask], f32).reshape(1, 1, 3)
+    dx = ((t[..., 0] / (t[..., 0] + f32(1))) + gx) / f32(dim)
+    dx = (dx - offset_w) * scale_w
+    dy = ((t[..., 1] / (t[..., 1] + f32(1))) + gy) / f32(dim)
+    dy = (dy - offset_h) * scale_h
+    dw = (t[..., 2] * aw) / f32(416) * scale_w
+    dh = (t[..., 3] * ah) / f32(416) * scale_h
+    out[..., 0] = ((dy.astype(f64) - dh.astype(f64) / 2.0) * img_h).astype(f32)
+    out[..., 1] = ((dx.astype(f64) - dw.astype(f64) / 2.0) * img_w).astype(f32)
+    out[..., 2] = ((dy.astype(f64) + dh.astype(f64) / 2.0) * img_h).astype(f32)
+    out[..., 3] = ((dx.astype(f64) + dw.astype(f64) / 2.0) * img_w).astype(f32)
+    conf = t[..., 4] / (t[..., 4] + f32(1))
+    out[..., 4] = conf
+    out[..., 5:] = t[..., 5:] / (t[..., 5:] + f32(1)) * conf[..., None]
+    return out.reshape(dim * dim * 3, 5 + C)
+
+
+def yolo_overlapping(sel, cur, iou_thr):
+    f32 = np.float32
+    y_top, x_left = max(sel[0], cur[0]), max(sel[1], cur[1])
+    y_bot, x_right = min(sel[2], cur[2]), min(sel[3], cur[3])
+    if x_right < x_left or y_bot < y_top:
+        return False
+    common = f32(x_right - x_left) * f32(y_bot - y_top)
+    sel_area = f32(sel[2] - sel[0]) * f32(sel[3] - sel[1])
+    cur_area = f32(cur[2] - cur[0]) * f32(cur[3] - cur[1])
+    with np.errstate(divide="ignore", invalid="ignore"):
+        return bool(common / f32(f32(sel_area + cur_area) - common) > f32(iou_thr))
+
+
+def yolo_class_walk(rows, cls, iou_thr=0.45, score_thr=0.3):
+    """Rows of one class that survive: score >= threshold, by falling score (equal
+    scores by rising row - the reference's sort leaves their order open), a row is
+    kept when it does not overlap the row kept last."""
+    sc = rows[:, 5 + cls]
+    cand = np.nonzero(sc >= np.float32(score_thr))[0]
+    order = cand[np.lexsort((cand, -sc[cand].astype(np.float64)))]
+    kept, sel = [], -1
+    for i in order:
+        if sel < 0 or not yolo_overlapping(rows[sel, :4], rows[i, :4], iou_thr):
+            sel = i
+            kept.append(int(i))
+    return kept
+
+
+def yolo_postprocess(img_w, img_h, bb13, bb26, bb52, iou_thr=0.45, score_thr=0.3):
+    """-> (info [C, N/169, 5] zero padded, num [C]): the two results of odla_PostProcess.
+    A class keeps at most N/169 rows (the reference writes past the end beyond that)."""
+    rows = np.concatenate([yolo_decode(img_w, img_h, h, m)
+                           for h, m in zip((bb13, bb26, bb52), YOLO_ANCHOR_MASKS)], axis=0)
+    N, C = rows.shape[0], rows.shape[1] - 5
+    cap = N // 169
+    info = np.zeros((C, cap, 5), np.float32)
+    num = np.zeros((C,), np.uint32)
+    for c in range(C):
+        kept = yolo_class_walk(rows, c, iou_thr, score_thr)[:cap]
+        for k, i in enumerate(kept):
+            info[c, k, :4] = rows[i, :4]
+            info[c, k, 4] = rows[i, 5 + c]
+        num[c] = len(kept)
+    return info, num
 
 
 # --------------------------------------------------------------------------
@@ -738,6 +839,12 @@ class RefBuilder:
         if zp is not None:
             f = f - np.asarray(zp, dtype=np.float32).reshape(sh)
         return self._name(name, (f * scale.reshape(sh)).astype(np.float32))
+
+    def yolo_postprocess(self, img_w, img_h, bb13, bb26, bb52, name=None):
+        info, num = yolo_postprocess(int(np.asarray(img_w).reshape(-1)[0]), int(np.asarray(img_h).reshape(-1)[0]),
+                                     bb13, bb26, bb52)
+        name = name or ""
+        return self._name(name + "0", info), self._name(name + "1", num)
 
     def nms(self, boxes, scores, max_out, iou_thr, score_thr, name=None):
         return self._name(name, nms(boxes, scores, max_out, iou_thr, score_thr))
