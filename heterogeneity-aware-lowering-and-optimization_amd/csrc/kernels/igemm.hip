@@ -1206,6 +1206,8 @@ int lean_steps(const IgemmParams& p) {
   }
   const int kbytes = p.C * dtype_size(p.in_dt);
   if (p.R != 1 || p.S != 1 || p.ph != 0 || p.pw != 0 || p.batch != 1 || p.Kout < 64) return 0;
+  // no padding behind the image either: every output pixel reads a pixel that exists
+  if ((int64_t)(p.Ho - 1) * p.sh >= p.H || (int64_t)(p.Wo - 1) * p.sw >= p.W) return 0;
   // (8-bit layers of this shape are bound by the arithmetic of the requantising
   // epilogue, not by their staging, and do not gain from it)
   if (p.in_dt != DT_F16 && p.in_dt != DT_BF16) return 0;
@@ -1318,8 +1320,10 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
         (int64_t)p.wf_chunks * 32 >= kbytes + 128 || (int64_t)p.wf_tiles * 32 < p.Kout)
       return hipErrorInvalidValue;
   }
-  // the last output pixel's receptive field must start inside the padded input
-  if ((int64_t)(p.Ho - 1) * p.sh - p.ph >= p.H || (int64_t)(p.Wo - 1) * p.sw - p.pw >= p.W)
+  // (An output pixel may lie entirely in the padding: every tap is then masked.)
+  // Source coordinates are computed in 32 bits.
+  if ((int64_t)(p.Ho - 1) * p.sh + (int64_t)(p.R - 1) * p.dh >= (1ll << 30) ||
+      (int64_t)(p.Wo - 1) * p.sw + (int64_t)(p.S - 1) * p.dw >= (1ll << 30) || p.ph >= (1 << 30) || p.pw >= (1 << 30))
     return hipErrorInvalidValue;
 
   const int oes = dtype_size(p.out_dt);
