@@ -399,6 +399,37 @@ odla_value odla_Gemm(odla_value A, odla_bool tA, odla_value B, odla_bool tB, odl
     o.d[a.rank - 2] = M;
     o.d[a.rank - 1] = N;
   }
+  // The GEMM launch itself adds a constant row / scalar (any beta) or a
+  // run-time matrix of the result's shape (beta 1).  Every other C operand - a
+  // constant matrix, a column, a run-time row, another beta - becomes
+  // Gemm -> Add(beta * C), with the reference's broadcasting rules for the Add.
+  bool fused_c = true;
+  if (C != nullptr && beta != 0.f) {
+    const int64_t cn = C->shape.numel();
+    const bool row_const = C->kind == _odla_value::CONSTANT && is_float_type(C->etype) &&
+                           (cn == 1 || (cn == N && C->shape.d[C->shape.rank - 1] == N));
+    const bool full_runtime = C->kind != _odla_value::CONSTANT && C->shape == o && beta == 1.f;
+    fused_c = row_const || full_runtime;
+  }
+  if (!fused_c) {
+    REQUIRE(is_float_type(C->etype), "odla_Gemm: C operand must be a float type");
+    odla_value g = odla_Gemm(A, tA, B, tB, alpha, 0.f, nullptr, output_dims, nullptr);
+    if (g == nullptr) return nullptr;
+    odla_value cs = C;
+    if (beta != 1.f) {
+      auto buf = std::make_unique<std::vector<uint8_t>>(sizeof(float));
+      memcpy(buf->data(), &beta, sizeof(float));
+      Shape one;
+      one.rank = 1;
+      one.d[0] = 1;
+      odla_value k = new_value(c, _odla_value::CONSTANT, ODLA_FLOAT32, one, nullptr);
+      k->host_data = buf->data();
+      c->owned_data.push_back(std::move(buf));
+      cs = binary(BIN_MUL, C, k, nullptr);
+      if (cs == nullptr) return nullptr;
+    }
+    return binary(BIN_ADD, g, cs, id);
+  }
   Node* n = add_node(c, OP_GEMM, {A, B, C}, A->etype, o, id);
   n->i[0] = tA ? 1 : 0;
   n->i[1] = tB ? 1 : 0;

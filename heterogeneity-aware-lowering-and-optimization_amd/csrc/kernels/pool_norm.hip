@@ -612,6 +612,34 @@ layernorm_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int l
   }
 }
 
+// Rows longer than a workgroup can hold in registers: the same three steps, each
+// a strided walk over the row in memory (the second and third walk hit in cache).
+template <typename T, int NT>
+__global__ void __launch_bounds__(NT)
+layernorm_long_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t len,
+                      const float* __restrict__ gamma, const float* __restrict__ beta, float eps) {
+  __shared__ float red[NT / 64];
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const T* row = x + r * len;
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < len; i += NT) s += Store<T>::ld(row + i);
+    const float mean = block_sum<NT>(s, red) / (float)len;
+    float q = 0.f;
+    for (int64_t i = threadIdx.x; i < len; i += NT) {
+      const float d = Store<T>::ld(row + i) - mean;
+      q += d * d;
+    }
+    const float var = block_sum<NT>(q, red) / (float)len;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    T* out = y + r * len;
+    for (int64_t i = threadIdx.x; i < len; i += NT) {
+      const float g = gamma ? gamma[i] : 1.f, b = beta ? beta[i] : 0.f;
+      Store<T>::st(out + i, (Store<T>::ld(row + i) - mean) * rstd * g + b);
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace
 
 #define FLOAT_DISPATCH(dt, EXPR)                         \
@@ -788,7 +816,12 @@ hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int
 hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int64_t len,
                             const float* gamma, const float* beta, float eps, hipStream_t stream) {
   if (!x || !y || rows <= 0 || len <= 0) return hipErrorInvalidValue;
-  if (len > 256 * 16) return hipErrorInvalidValue;
+  if (len > 256 * 16) {
+    const int grid = (int)(rows < 16384 ? rows : 16384);
+    FLOAT_DISPATCH(dt, hipLaunchKernelGGL((layernorm_long_kernel<T, 256>), dim3(grid), dim3(256), 0, stream,
+                                          (const T*)x, (T*)y, rows, len, gamma, beta, eps));
+    return hipGetLastError();
+  }
   {
     const int es = dtype_size(dt);
     const int V = es ? 16 / es : 1;

@@ -1641,14 +1641,20 @@ void Planner::lower_binary(int ni) {
     (void)aligned;
     return get(v, L_ROWMAJOR, FORM_FLOAT);
   };
-  const int ta = operand(a, sa), tb = operand(b, sb);
-  if (T(ta).dt != dt || T(tb).dt != dt) fail(ODLA_UNSUPPORTED_DATATYPE, "mixed storage types in element-wise op '%s'", outv->name.c_str());
+  int ta = operand(a, sa), tb = operand(b, sb);
   int ocs = 0;
   if (lay == L_NHWC) {
     ocs = (int)os.d[1];
-    if ((a->shape == os && T(ta).cs != ocs) || (b->shape == os && T(tb).cs != ocs))
-      fail(ODLA_UNSUPPORTED_OP, "element-wise op '%s' on a channel-padded tensor", outv->name.c_str());
+    if ((a->shape == os && T(ta).cs != ocs) || (b->shape == os && T(tb).cs != ocs)) {
+      // a channels-last operand whose pixels are padded to a vector multiple: the
+      // flat kernels assume dense rows, so this one runs on row-major copies
+      lay = L_ROWMAJOR;
+      ocs = 0;
+      ta = get(a, L_ROWMAJOR, FORM_FLOAT);
+      tb = get(b, L_ROWMAJOR, FORM_FLOAT);
+    }
   }
+  if (T(ta).dt != dt || T(tb).dt != dt) fail(ODLA_UNSUPPORTED_DATATYPE, "mixed storage types in element-wise op '%s'", outv->name.c_str());
   const int ty = new_tensor(dt, lay, os, ocs, SP_ARENA);
 
   // physical iteration order of the output and per-operand strides
@@ -1959,10 +1965,11 @@ void Planner::lower_reduce(int ni) {
   const VState& s = vs_[x->index];
   // spatial reduction of a channels-last tensor (global pooling)
   const bool spatial = xs.rank == 4 && axes.size() == 2 && axes[0] == 2 && axes[1] == 3;
-  if (spatial && s.main >= 0 && T(s.main).layout == L_NHWC) {
+  // (a float tensor whose pixels are padded to a vector multiple takes the general path below)
+  if (spatial && s.main >= 0 && T(s.main).layout == L_NHWC && (T(s.main).cs == xs.d[1] || T(s.main).quant)) {
     const PTensor px = T(s.main);
     const int64_t outer = xs.d[0], len = xs.d[2] * xs.d[3], inner = px.cs;
-    if (px.cs != xs.d[1]) fail(ODLA_UNSUPPORTED_OP, "reduction over a padded channels-last tensor");
+    if (px.cs != xs.d[1]) fail(ODLA_UNSUPPORTED_OP, "reduction over a padded 8-bit channels-last tensor");
     Shape o4;
     o4.rank = 4;
     o4.d[0] = xs.d[0]; o4.d[1] = xs.d[1]; o4.d[2] = 1; o4.d[3] = 1;
@@ -1996,17 +2003,51 @@ void Planner::lower_reduce(int ni) {
     set_main(n.out, ty);
     return;
   }
-  // general case: the reduced axes must be adjacent in row-major order
+  // general case: one launch when the reduced axes are adjacent in row-major
+  // order; otherwise a permuted copy that moves them behind the kept ones first
+  bool adjacent = true;
   for (size_t i = 1; i < axes.size(); ++i)
-    if (axes[i] != axes[i - 1] + 1) fail(ODLA_UNSUPPORTED_OP, "reduction over non-adjacent axes");
-  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
-  int64_t outer = 1, len = 1, inner = 1;
-  for (int i = 0; i < xs.rank; ++i) {
-    if (i < axes.front()) outer *= xs.d[i];
-    else if (i <= axes.back()) len *= xs.d[i];
-    else inner *= xs.d[i];
-  }
+    if (axes[i] != axes[i - 1] + 1) adjacent = false;
+  int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
   const DType dt = T(tx).dt;
+  int64_t outer = 1, len = 1, inner = 1;
+  if (adjacent) {
+    for (int i = 0; i < xs.rank; ++i) {
+      if (i < axes.front()) outer *= xs.d[i];
+      else if (i <= axes.back()) len *= xs.d[i];
+      else inner *= xs.d[i];
+    }
+  } else {
+    const int r = xs.rank;
+    if (r > 8) fail(ODLA_UNSUPPORTED_OP, "reduction over non-adjacent axes of a rank > 8 value");
+    std::vector<int> order;
+    for (int i = 0; i < r; ++i)
+      if (std::find(axes.begin(), axes.end(), (int64_t)i) == axes.end()) order.push_back(i);
+    for (int64_t a : axes) order.push_back((int)a);
+    int64_t xstr[ODLA_MAX_DIMENSION];
+    {
+      int64_t acc = 1;
+      for (int i = r - 1; i >= 0; --i) { xstr[i] = acc; acc *= xs.d[i]; }
+    }
+    Shape ps;
+    ps.rank = r;
+    for (int i = 0; i < r; ++i) ps.d[i] = xs.d[order[i]];
+    const int tp = new_tensor(dt, L_ROWMAJOR, ps, 0, SP_ARENA);
+    StridedCopyParams cp;
+    cp.elem_size = dtype_size(dt);
+    cp.rank = r;
+    int64_t sy = 1;
+    for (int i = r - 1; i >= 0; --i) {
+      cp.dims[i] = ps.d[i];
+      cp.sx[i] = xstr[order[i]];
+      cp.sy[i] = sy;
+      sy *= ps.d[i];
+    }
+    strided_copy_step("reduce.gather:" + n.out->name, tx, tp, cp);
+    tx = tp;
+    for (int64_t a : axes) len *= xs.d[a];
+    outer = xs.numel() / len;
+  }
   const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
   const Ref a = ref(tx), b = ref(ty);
   emit("reduce:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {

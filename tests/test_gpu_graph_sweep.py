@@ -1,0 +1,153 @@
+"""Random operator chains against the oracle: convolutions with per-channel constant
+arithmetic, activations, BatchNorm, shortcuts, pooling, concat, resize and channel
+slices in random order, with random intermediate values marked as outputs (which
+forbids folding them away).  This is aimed at the planner - epilogue fusion, layout
+choices, aliasing and the arena - rather than at any one kernel."""
+import numpy as np
+import pytest
+
+from util import announce, max_rel_err, run_hip, run_ref
+
+pytestmark = pytest.mark.gpu
+
+
+class Chain:
+    """A recorded random program: a list of steps replayed on any builder."""
+
+    def __init__(self, seed):
+        r = np.random.default_rng(seed)
+        self.in_shape = (int(r.integers(1, 4)), int(r.choice([3, 8, 16, 32])), int(r.integers(8, 17)), int(r.integers(8, 17)))
+        self.steps = []
+        shapes = [self.in_shape]          # shape of value k
+        n_steps = int(r.integers(4, 13))
+        for _ in range(n_steps):
+            src = int(r.integers(max(0, len(shapes) - 3), len(shapes)))
+            N, C, H, W = shapes[src]
+            kind = str(r.choice(["conv", "conv", "conv", "chan_arith", "chan_arith", "act", "bn", "shortcut", "pool",
+                                 "concat", "resize", "slice"]))
+            if kind == "conv":
+                k = int(r.choice([1, 1, 3, 3, 5]))
+                s = int(r.choice([1, 1, 1, 2]))
+                p = k // 2 if r.random() < 0.8 else 0
+                O = int(r.choice([8, 16, 24, 64, 72, 136]))
+                if (H + 2 * p - k) // s + 1 < 2 or (W + 2 * p - k) // s + 1 < 2:
+                    continue
+                w = (r.standard_normal((O, C, k, k)) * np.sqrt(1.5 / (C * k * k))).astype(np.float32)
+                b = r.standard_normal(O).astype(np.float32) * 0.3 if r.random() < 0.6 else None
+                self.steps.append(("conv", src, w, b, s, p))
+                shapes.append((N, O, (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1))
+            elif kind == "chan_arith":
+                op = str(r.choice(["add", "mul", "sub", "div"]))
+                form = str(r.choice(["c11", "1c11", "scalar"]))
+                shape = {"c11": (C, 1, 1), "1c11": (1, C, 1, 1), "scalar": (1,)}[form]
+                k = r.standard_normal(shape).astype(np.float32)
+                if op in ("mul", "div"):
+                    k = (np.abs(k) * 0.5 + 0.5).astype(np.float32)
+                self.steps.append(("chan_arith", src, op, k, bool(r.random() < 0.2)))
+                shapes.append((N, C, H, W))
+            elif kind == "act":
+                self.steps.append(("act", src, str(r.choice(["relu", "leaky", "clamp", "sigmoid", "tanh", "gelu"]))))
+                shapes.append((N, C, H, W))
+            elif kind == "bn":
+                self.steps.append(("bn", src, r.standard_normal(C).astype(np.float32) * 0.2,
+                                   (r.random(C) + 0.5).astype(np.float32), (r.random(C) + 0.5).astype(np.float32),
+                                   r.standard_normal(C).astype(np.float32) * 0.2))
+                shapes.append((N, C, H, W))
+            elif kind == "shortcut":
+                same = [i for i, sh in enumerate(shapes) if sh == shapes[src] and i != src]
+                if not same:
+                    continue
+                self.steps.append(("shortcut", src, int(r.choice(same)), bool(r.random() < 0.5)))
+                shapes.append((N, C, H, W))
+            elif kind == "pool":
+                if H < 4 or W < 4:
+                    continue
+                mx = bool(r.random() < 0.5)
+                k, s, p = (3, 2, 1) if r.random() < 0.5 else (2, 2, 0)
+                self.steps.append(("pool", src, mx, k, s, p))
+                shapes.append((N, C, (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1))
+            elif kind == "concat":
+                same = [i for i, sh in enumerate(shapes) if sh[0] == N and sh[2:] == (H, W) and i != src]
+                if not same:
+                    continue
+                other = int(r.choice(same))
+                self.steps.append(("concat", src, other))
+                shapes.append((N, C + shapes[other][1], H, W))
+            elif kind == "resize":
+                if H * W > 400:
+                    continue
+                self.steps.append(("resize", src))
+                shapes.append((N, C, 2 * H, 2 * W))
+            else:
+                if C < 4:
+                    continue
+                c0 = int(r.integers(0, C // 2))
+                c1 = int(r.integers(c0 + 1, C + 1))
+                self.steps.append(("slice", src, c0, c1))
+                shapes.append((N, c1 - c0, H, W))
+        self.shapes = shapes
+        n_vals = len(shapes)
+        marks = set(int(v) for v in r.choice(np.arange(1, n_vals), size=min(n_vals - 1, int(r.integers(1, 4))), replace=False)) if n_vals > 1 else set()
+        marks.add(n_vals - 1)
+        self.outputs = sorted(marks)
+        self.x = r.standard_normal(self.in_shape).astype(np.float32)
+
+    def build(self, b):
+        vals = [b.arg("x", self.in_shape)]
+        for i, st in enumerate(self.steps):
+            name = "v%d" % (i + 1)
+            kind, src = st[0], vals[st[1]]
+            if kind == "conv":
+                _, _, w, bias, s, p = st
+                v = b.conv(src, b.const(name + ".w", w), b.const(name + ".b", bias) if bias is not None else None,
+                           (s, s), (p, p, p, p), name=name)
+            elif kind == "chan_arith":
+                _, _, op, k, swap = st
+                kc = b.const(name + ".k", k)
+                v = getattr(b, op)(kc, src, name=name) if swap and op in ("add", "mul") else getattr(b, op)(src, kc, name=name)
+            elif kind == "act":
+                a = st[2]
+                v = {"relu": lambda: b.relu(src, name=name), "leaky": lambda: b.leaky_relu(src, 0.1, name=name),
+                     "clamp": lambda: b.clamp(src, -1.0, 1.5, name=name), "sigmoid": lambda: b.sigmoid(src, name=name),
+                     "tanh": lambda: b.tanh(src, name=name), "gelu": lambda: b.gelu(src, name=name)}[a]()
+            elif kind == "bn":
+                _, _, mean, var, g, be = st
+                v = b.batchnorm(src, b.const(name + ".m", mean), b.const(name + ".v", var), 1e-5,
+                                b.const(name + ".g", g), b.const(name + ".be", be), name=name)
+            elif kind == "shortcut":
+                v = b.add(src, vals[st[2]], name=name + (".s" if st[3] else ""))
+                if st[3]:
+                    v = b.relu(v, name=name)
+            elif kind == "pool":
+                _, _, mx, k, s, p = st
+                v = (b.maxpool if mx else b.avgpool)(src, (k, k), (s, s), (p, p, p, p), name=name)
+            elif kind == "concat":
+                v = b.concat([src, vals[st[2]]], 1, name=name)
+            elif kind == "resize":
+                sh = self.shapes[st[1]]
+                v = b.resize_nearest(src, (2 * sh[2], 2 * sh[3]), name=name)
+            else:
+                sh = self.shapes[st[1]]
+                v = b.slice(src, (0, st[2], 0, 0), (sh[0], st[3], sh[2], sh[3]), name=name)
+            vals.append(v)
+        for k in self.outputs:
+            b.output(vals[k], "v%d" % k)
+
+
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def test_random_chains(mode):
+    for seed in range(200):
+        ch = Chain(seed)
+        if not ch.steps:
+            continue
+        announce("chain %s seed %d: %s -> outputs %s" % (mode, seed, [s[0] for s in ch.steps], ch.outputs))
+        feeds = {"x": ch.x}
+        want = run_ref(ch.build, feeds)
+        got = run_hip(ch.build, feeds, fp16=(mode == "fp16"), repeats=2)
+        for k, w in want.items():
+            assert got[k].shape == w.shape, (seed, k)
+            if mode == "fp32":
+                assert max_rel_err(got[k], w) <= 5e-4, (seed, k, [s[0] for s in ch.steps])
+            else:
+                scale = max(1.0, float(np.max(np.abs(w))))
+                assert float(np.max(np.abs(got[k] - w))) <= 6e-2 * scale, (seed, k, [s[0] for s in ch.steps])
