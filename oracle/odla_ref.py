@@ -828,7 +828,7 @@ class RefBuilder:
         lo, hi, dt = (-128, 127, np.int8) if signed else (0, 255, np.uint8)
         return self._name(name, np.clip(t, lo, hi).astype(dt))
 
-    def dequantize(self, q, scale, zp=None, axis=-1, name=None):
+    def dequantize(self, q, scale, zp=None, axis=-1, name=None, zp_dtype=None):
         """[ref: odla_dnnl_quantization.cc:33-59]"""
         q = np.asarray(q)
         scale = _f32(scale).reshape(-1)

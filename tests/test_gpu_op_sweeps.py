@@ -11,7 +11,7 @@ from util import announce, max_rel_err, run_hip, run_ref
 pytestmark = pytest.mark.gpu
 
 
-def source(b, name, shape, behind_conv, seed):
+def source(b, name, shape, behind_conv, seed, mix=0.05):
     """A value of `shape`: the argument itself, or a 1x1 convolution of it (identity
     weights plus a little mixing), which the planner stores channels-last.  The
     weights depend on `seed` alone: the oracle and the library build the same graph."""
@@ -20,7 +20,7 @@ def source(b, name, shape, behind_conv, seed):
         return v
     C = shape[1]
     r = np.random.default_rng(seed)
-    w = (np.eye(C, dtype=np.float32) + 0.05 * r.standard_normal((C, C)).astype(np.float32)).reshape(C, C, 1, 1)
+    w = (np.eye(C, dtype=np.float32) + mix * r.standard_normal((C, C)).astype(np.float32)).reshape(C, C, 1, 1)
     return b.conv(v, b.const(name + ".w", w), None, (1, 1), (0, 0, 0, 0), name=name + ".conv")
 
 
@@ -268,3 +268,147 @@ def test_gather_cast_sweep():
         if not const_table:
             feeds["x"] = X
         check(build, feeds, exact=True, tag=tag, modes=("fp32",))
+
+
+UNARY = {
+    # name -> (call, input transform)
+    "relu": (lambda b, x, n: b.relu(x, name=n), None), "sigmoid": (lambda b, x, n: b.sigmoid(x, name=n), None),
+    "tanh": (lambda b, x, n: b.tanh(x, name=n), None), "exp": (lambda b, x, n: b.exp(x, name=n), None),
+    "log": (lambda b, x, n: b.log(x, name=n), "pos"), "sqrt": (lambda b, x, n: b.sqrt(x, name=n), "pos"),
+    "rsqrt": (lambda b, x, n: b.rsqrt(x, name=n), "pos"), "erf": (lambda b, x, n: b.erf(x, name=n), None),
+    "abs": (lambda b, x, n: b.abs(x, name=n), None), "neg": (lambda b, x, n: b.neg(x, name=n), None),
+    "reciprocal": (lambda b, x, n: b.reciprocal(x, name=n), "pos"),
+    "sin": (lambda b, x, n: b.sin(x, name=n), None), "cos": (lambda b, x, n: b.cos(x, name=n), None),
+    "atan": (lambda b, x, n: b.atan(x, name=n), None), "asin": (lambda b, x, n: b.asin(x, name=n), "unit"),
+    "sinh": (lambda b, x, n: b.sinh(x, name=n), None), "asinh": (lambda b, x, n: b.asinh(x, name=n), None),
+    "softplus": (lambda b, x, n: b.softplus(x, name=n), None), "softsign": (lambda b, x, n: b.softsign(x, name=n), None),
+    "gelu": (lambda b, x, n: b.gelu(x, name=n), None), "gelu_tanh": (lambda b, x, n: b.gelu(x, True, name=n), None),
+    "leaky": (lambda b, x, n: b.leaky_relu(x, 0.2, name=n), None), "clamp": (lambda b, x, n: b.clamp(x, -0.3, 0.8, name=n), None),
+    "elu": (lambda b, x, n: b.elu(x, 1.3, name=n), None), "selu": (lambda b, x, n: b.selu(x, 1.67, 1.05, name=n), None),
+    "celu": (lambda b, x, n: b.celu(x, 0.8, name=n), None),
+    "hard_sigmoid": (lambda b, x, n: b.hard_sigmoid(x, 0.2, 0.5, name=n), None),
+    "thresholded_relu": (lambda b, x, n: b.thresholded_relu(x, 0.4, name=n), "grid"),
+    "shrink": (lambda b, x, n: b.shrink(x, 0.1, 0.5, name=n), "grid"),
+    "ceil": (lambda b, x, n: b.ceil(x, name=n), "grid"), "floor": (lambda b, x, n: b.floor(x, name=n), "grid"),
+    "round": (lambda b, x, n: b.round(x, name=n), "grid"), "sign": (lambda b, x, n: b.sign(x, name=n), "grid"),
+}
+
+
+@pytest.mark.parametrize("behind_conv", [False, True])
+def test_unary_sweep(behind_conv):
+    r = np.random.default_rng(81 + behind_conv)
+    for i, (name, (call, dom)) in enumerate(sorted(UNARY.items())):
+        rank = 4 if behind_conv else int(r.integers(1, 5))
+        shape = rand_shape4(r) if rank == 4 else tuple(int(r.integers(1, 40)) for _ in range(rank))
+        tag = "unary %s %s conv=%s" % (name, shape, behind_conv)
+        announce(tag)
+        x = r.standard_normal(shape).astype(np.float32)
+        if dom == "pos":
+            x = np.abs(x) + 0.25
+        elif dom == "unit":
+            x = np.clip(x * 0.4, -0.95, 0.95)
+        elif dom == "grid":
+            # step functions: values a safe distance from every step, exact in fp16
+            x = (np.round(x * 4) / 4 + 0.125).astype(np.float32)
+        x = x.astype(np.float16).astype(np.float32) if dom is not None else x
+
+        def build(b):
+            # restricted domains survive only an identity convolution
+            v = source(b, "x", shape, behind_conv, 4000 + i, mix=0.05 if dom is None else 0.0)
+            b.output(call(b, v, "y"), "y")
+
+        check(build, {"x": x.astype(np.float32)}, tag=tag)
+
+
+def test_compare_select_logic_sweep():
+    r = np.random.default_rng(91)
+    for i in range(30):
+        rank = int(r.integers(1, 5))
+        shape = tuple(int(r.integers(1, 10)) for _ in range(rank))
+        bshape = tuple(d if r.random() < 0.6 else 1 for d in shape)
+        tag = "select #%d %s %s" % (i, shape, bshape)
+        announce(tag)
+        A = (np.round(r.standard_normal(shape) * 2) / 2).astype(np.float32)
+        B = (np.round(r.standard_normal(bshape) * 2) / 2).astype(np.float32)
+        cmp = ["less", "less_equal", "greater", "greater_equal", "equal", "not_equal"][i % 6]
+        logic = ["logical_and", "logical_or", "logical_xor"][i % 3]
+
+        def build(b):
+            a, bb = b.arg("a", shape), b.arg("b", bshape)
+            c1 = getattr(b, cmp)(a, bb, name="c1")
+            c2 = b.greater(a, b.const("z", np.zeros((1,), np.float32)), name="c2")
+            m = getattr(b, logic)(c1, c2, name="m")
+            b.output(c1, "c1")
+            b.output(b.logical_not(m, name="nm"), "nm")
+            b.output(b.select(m, a, b.neg(a, name="na"), name="sel"), "sel")
+
+        check(build, {"a": A, "b": B}, exact=True, tag=tag, modes=("fp32", "fp16"))
+
+
+def test_topk_stack_squeeze_sweep():
+    r = np.random.default_rng(101)
+    for i in range(24):
+        rank = int(r.integers(1, 4))
+        shape = tuple(int(r.integers(2, 30)) for _ in range(rank))
+        axis = int(r.integers(0, rank))
+        k = int(r.integers(1, shape[axis] + 1))
+        largest = bool(i % 2)
+        tag = "topk #%d %s axis %d k %d largest %s" % (i, shape, axis, k, largest)
+        announce(tag)
+        X = r.permutation(int(np.prod(shape))).reshape(shape).astype(np.float32) / 4.0   # distinct, exact in fp16 up to 8k elements
+
+        def build(b):
+            x = b.arg("x", shape)
+            v, idx = b.topk(x, k, axis, largest, np.int64 if i % 3 == 0 else np.int32, names=("v", "i"))
+            b.output(v, "v")
+            b.output(idx, "i")
+            s = b.stack([x, b.neg(x, name="n")], int(r.integers(0, rank + 1)) if False else axis, name="s")
+            b.output(s, "s")
+
+        check(build, {"x": X}, exact=True, tag=tag, modes=("fp32",) if X.size > 2048 else ("fp32", "fp16"))
+
+
+def test_deconv_sweep():
+    r = np.random.default_rng(111)
+    for i in range(16):
+        N, C, O = int(r.integers(1, 3)), int(r.choice([4, 8, 16])), int(r.choice([3, 8, 16]))
+        H, W = int(r.integers(3, 9)), int(r.integers(3, 9))
+        k = int(r.choice([2, 3, 4]))
+        s = int(r.choice([1, 2]))
+        p = int(r.integers(0, min(k - 1, 1) + 1))
+        tag = "deconv #%d N%d C%d O%d %dx%d k%d s%d p%d" % (i, N, C, O, H, W, k, s, p)
+        announce(tag)
+        Wt = (r.standard_normal((C, O, k, k)) * np.sqrt(1.0 / (C * k * k))).astype(np.float32)
+        bias = r.standard_normal(O).astype(np.float32) if i % 2 else None
+        X = r.standard_normal((N, C, H, W)).astype(np.float32)
+
+        def build(b):
+            x = b.arg("x", X.shape)
+            y = b.deconv(x, b.const("w", Wt), b.const("b", bias) if bias is not None else None, (s, s), (p, p, p, p), name="y")
+            b.output(y, "y")
+
+        check(build, {"x": X}, tag=tag)
+
+
+def test_quantize_dequantize_sweep():
+    r = np.random.default_rng(121)
+    for i in range(20):
+        rank = int(r.integers(1, 5))
+        shape = tuple(int(r.integers(1, 12)) for _ in range(rank))
+        axis = int(r.integers(0, rank))
+        per_axis = bool(i % 2)
+        n = shape[axis] if per_axis else 1
+        scale = (r.random(n) * 0.1 + 0.01).astype(np.float32)
+        signed = bool(i % 3 == 0)
+        zp = r.integers(-20, 20, n).astype(np.int8) if signed else r.integers(100, 150, n).astype(np.uint8)
+        tag = "qdq #%d %s axis %d per_axis %s signed %s" % (i, shape, axis, per_axis, signed)
+        announce(tag)
+        X = (r.standard_normal(shape) * 3).astype(np.float32)
+
+        def build(b):
+            x = b.arg("x", shape)
+            q = b.quantize(x, scale, zp, axis, signed, name="q")
+            b.output(q, "q")
+            b.output(b.dequantize(q, scale, zp, axis, name="d", zp_dtype=zp.dtype), "d")
+
+        check(build, {"x": X}, tag=tag, modes=("fp32",))
