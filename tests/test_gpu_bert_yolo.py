@@ -64,3 +64,28 @@ def test_small_yolov3_heads_and_detections():
     ref = entry.load_oracle()
     want_det = ref.nms(pg["boxes"], pg["scores"], 20, 0.45, 0.3)
     assert np.array_equal(pg["detections"], want_det)
+
+
+def test_bert_encoder_random_sizes():
+    """Encoders of random (small) sizes: sequence lengths that are no multiple of any
+    tile, one head, heads of 8 .. 64 features, batch 1 - the masked-softmax fusion, the
+    split-K rule and the batched attention GEMMs have size conditions of their own."""
+    mb = entry.load().models_bert
+    r = np.random.default_rng(17)
+    for i in range(14):
+        heads = int(r.choice([1, 2, 3, 4, 12]))
+        dh = int(r.choice([8, 16, 32, 64]))
+        cfg = dict(layers=int(r.integers(1, 3)), hidden=heads * dh, heads=heads, ffn=heads * dh * int(r.choice([1, 2, 4])),
+                   vocab=int(r.integers(50, 500)), max_pos=160)
+        batch, seq = int(r.integers(1, 5)), int(r.choice([1, 5, 16, 33, 64, 128, 150]))
+        announce("bert #%d %s batch %d seq %d" % (i, cfg, batch, seq))
+        w = mb.bert_weights(cfg, seed=100 + i)
+        feeds = mb.bert_input(batch, seq, cfg, seed=200 + i)
+        if seq > 3:
+            feeds["attention_mask"][0, 0, 0, seq - seq // 3:] = 0.0
+        build = lambda b: mb.build_bert(b, w, batch, seq, cfg)
+        want = run_ref(build, feeds)["hidden"]
+        got = run_hip(build, feeds)["hidden"]
+        assert max_rel_err(got, want) <= 2e-4, (i, cfg, batch, seq)
+        got = run_hip(build, feeds, bf16=True)["hidden"]
+        assert np.max(np.abs(got - want)) <= 3e-2 * max(1.0, float(np.max(np.abs(want)))), (i, cfg, batch, seq)
