@@ -6,7 +6,7 @@ choices, aliasing and the arena - rather than at any one kernel."""
 import numpy as np
 import pytest
 
-from util import announce, max_rel_err, run_hip, run_ref
+from util import announce, max_rel_err, run_hip, run_hip_stored, run_ref
 
 pytestmark = pytest.mark.gpu
 
@@ -135,7 +135,7 @@ class Chain:
 
 
 @pytest.mark.parametrize("mode", ["fp32", "fp16"])
-def test_random_chains(mode):
+def test_random_chains(mode, tmp_path):
     for seed in range(200):
         ch = Chain(seed)
         if not ch.steps:
@@ -144,6 +144,11 @@ def test_random_chains(mode):
         feeds = {"x": ch.x}
         want = run_ref(ch.build, feeds)
         got = run_hip(ch.build, feeds, fp16=(mode == "fp16"), repeats=2)
+        if seed % 4 == 0:
+            # the same program stored to a file and loaded back computes the same bits
+            again = run_hip_stored(ch.build, feeds, str(tmp_path / ("chain%d.odla" % seed)), fp16=(mode == "fp16"))
+            for k in got:
+                assert np.array_equal(again[k], got[k]), (seed, k, "stored")
         for k, w in want.items():
             assert got[k].shape == w.shape, (seed, k)
             if mode == "fp32":

@@ -3,10 +3,14 @@ rank-4 case runs twice: on a graph argument (row-major in the plan) and behind a
 convolution, whose result the plan keeps channels-last - the operator then has to
 honour a layout it did not choose.  fp32 results within 1e-4 of the largest expected
 magnitude, fp16 plans within 2e-2; pure data movement is exact."""
+import os
+import tempfile
+import zlib
+
 import numpy as np
 import pytest
 
-from util import announce, max_rel_err, run_hip, run_ref
+from util import announce, max_rel_err, run_hip, run_hip_stored, run_ref
 
 pytestmark = pytest.mark.gpu
 
@@ -28,6 +32,12 @@ def check(build, feeds, exact=False, modes=("fp32", "fp16"), tag=""):
     want = run_ref(build, feeds)
     for mode in modes:
         got = run_hip(build, feeds, fp16=(mode == "fp16"))
+        if zlib.crc32(tag.encode()) % 4 == 0:
+            # every fourth case also goes through a stored file: same bits expected
+            with tempfile.TemporaryDirectory() as d:
+                again = run_hip_stored(build, feeds, os.path.join(d, "case.odla"), fp16=(mode == "fp16"))
+            for k in got:
+                assert np.array_equal(again[k], got[k], equal_nan=True), (tag, mode, k, "stored")
         for k in want:
             assert got[k].shape == want[k].shape, (tag, mode, k, got[k].shape, want[k].shape)
             if want[k].dtype.kind in "iub":

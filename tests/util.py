@@ -24,6 +24,58 @@ def run_hip(build_fn, feeds, use_graph=True, repeats=1, **builder_kwargs):
         hb.destroy()
 
 
+def run_hip_stored(build_fn, feeds, path, **builder_kwargs):
+    """Record, store the computation to `path`, destroy it, load the file as an
+    executable and run that: name -> numpy array like run_hip."""
+    import ctypes
+    pkg = entry.load()
+    odla = pkg.odla
+    L = odla.load_library()
+    hb = odla.HipBuilder(**builder_kwargs)
+    try:
+        build_fn(hb)
+        outs = {name: (shape, dt) for name, (h, shape, dt) in hb.outs.items()}
+        args = {name: (shape, dt) for name, (h, shape, dt) in hb.args.items()}
+        loc, keep = odla.path_location(path)
+        exe0 = ctypes.c_void_p()
+        assert L.odla_CompileComputation(hb.comp, None, ctypes.byref(exe0)) == 0 and exe0.value
+        assert L.odla_StoreExecutable(loc, exe0) == 0
+    finally:
+        hb.destroy()
+    exe = ctypes.c_void_p()
+    assert L.odla_LoadExecutable(loc, None, ctypes.byref(exe)) == 0
+    ctx = ctypes.c_void_p()
+    assert L.odla_CreateContext(ctypes.byref(ctx)) == 0
+    try:
+        held = []
+        n = ctypes.c_uint32()
+        assert L.odla_GetNumOfArgsFromExecutable(exe, ctypes.byref(n)) == 0 and n.value == len(args)
+        for i in range(n.value):
+            v = ctypes.c_void_p()
+            assert L.odla_GetArgFromExecutableByIdx(exe, i, ctypes.byref(v)) == 0
+            vid = ctypes.c_char_p()
+            assert L.odla_GetValueId(v, ctypes.byref(vid)) == 0
+            name = vid.value.decode()
+            a = np.ascontiguousarray(feeds[name], dtype=args[name][1])
+            held.append(a)
+            assert L.odla_BindToArgument(v, a.ctypes.data_as(ctypes.c_void_p), ctx) == 0
+        assert L.odla_GetNumOfOutputsFromExecutable(exe, ctypes.byref(n)) == 0 and n.value == len(outs)
+        got = {}
+        for i in range(n.value):
+            v = ctypes.c_void_p()
+            assert L.odla_GetOutputFromExecutableByIdx(exe, i, ctypes.byref(v)) == 0
+            vid = ctypes.c_char_p()
+            assert L.odla_GetValueId(v, ctypes.byref(vid)) == 0
+            name = vid.value.decode()
+            got[name] = np.empty(outs[name][0], outs[name][1])
+            assert L.odla_BindToOutput(v, got[name].ctypes.data_as(ctypes.c_void_p), ctx) == 0
+        assert L.odla_LaunchExecutable(exe, ctx) == 0
+        return got
+    finally:
+        L.odla_DestroyContext(ctx)
+        assert L.odla_DestroyExecutable(exe) == 0
+
+
 def run_ref(build_fn, feeds):
     ref = entry.load_oracle()
     rb = ref.RefBuilder(feeds)
