@@ -92,7 +92,7 @@ class Chain:
         self.outputs = sorted(marks)
         self.x = r.standard_normal(self.in_shape).astype(np.float32)
 
-    def build(self, b):
+    def build(self, b, probe=None):
         vals = [b.arg("x", self.in_shape)]
         for i, st in enumerate(self.steps):
             name = "v%d" % (i + 1)
@@ -130,6 +130,8 @@ class Chain:
                 sh = self.shapes[st[1]]
                 v = b.slice(src, (0, st[2], 0, 0), (sh[0], st[3], sh[2], sh[3]), name=name)
             vals.append(v)
+            if probe is not None:
+                probe(len(vals) - 1, v)
         for k in self.outputs:
             b.output(vals[k], "v%d" % k)
 
@@ -156,3 +158,59 @@ def test_random_chains(mode, tmp_path):
             else:
                 scale = max(1.0, float(np.max(np.abs(w))))
                 assert float(np.max(np.abs(got[k] - w))) <= 6e-2 * scale, (seed, k, [s[0] for s in ch.steps])
+
+
+def test_random_chains_in_interpret_mode():
+    """The same programs recorded in interpret mode: the input is a value with data of
+    its own, random values are read back with odla_GetValueData while the graph still
+    grows (each read compiles what exists so far), and again, in another order, once it
+    is complete."""
+    import ctypes
+    import __graft_entry__ as entry
+    odla = entry.load().odla
+
+    class Interp(odla.HipBuilder):
+        def __init__(self, feeds):
+            super().__init__()
+            self.feeds, self.held = feeds, []
+
+        def arg(self, name, shape, dtype=np.float32):
+            a = np.ascontiguousarray(self.feeds[name], dtype=dtype)
+            self.held.append(a)
+            h = self._ret(self.L.odla_CreateValue(odla.make_type(dtype, shape), name.encode()), "odla_CreateValue")
+            assert self.L.odla_SetValueData(h, a.ctypes.data_as(ctypes.c_void_p)) == 0
+            return h
+
+        def output(self, v, name):
+            pass
+
+        def read(self, v):
+            shape, dt = self.shape_of(v)
+            out = np.empty(shape, dt)
+            assert self.L.odla_GetValueData(v, out.ctypes.data_as(ctypes.c_void_p), None) == 0
+            return out
+
+    r = np.random.default_rng(5)
+    for seed in range(0, 200, 5):
+        ch = Chain(seed)
+        if not ch.steps:
+            continue
+        announce("interpret chain seed %d: %s" % (seed, [s[0] for s in ch.steps]))
+        feeds = {"x": ch.x}
+        ref = run_ref(lambda b: ch.build(b, probe=lambda k, v: b.output(v, "p%d" % k)), feeds)
+        ib = Interp(feeds)
+        try:
+            handles = {}
+
+            def probe(k, v):
+                handles[k] = v
+                if r.random() < 0.4:
+                    got = ib.read(v)
+                    assert max_rel_err(got, ref["p%d" % k]) <= 5e-4, (seed, k, "while growing")
+
+            ch.build(ib, probe=probe)
+            for k in r.permutation(sorted(handles)):
+                got = ib.read(handles[int(k)])
+                assert max_rel_err(got, ref["p%d" % int(k)]) <= 5e-4, (seed, int(k), "complete")
+        finally:
+            ib.destroy()
