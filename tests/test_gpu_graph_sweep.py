@@ -214,3 +214,46 @@ def test_random_chains_in_interpret_mode():
                 assert max_rel_err(got, ref["p%d" % int(k)]) <= 5e-4, (seed, int(k), "complete")
         finally:
             ib.destroy()
+
+
+def test_random_chains_under_the_calibration_profiler(tmp_path):
+    """Profiler mode over random programs: the recorded range of every named value -
+    whole tensor and per channel - equals the range of the oracle's value."""
+    import __graft_entry__ as entry
+    pkg = entry.load()
+    cal, odla = pkg.calibration, pkg.odla
+    for seed in range(2, 200, 9):
+        ch = Chain(seed)
+        if not ch.steps:
+            continue
+        announce("profiled chain seed %d: %s" % (seed, [s[0] for s in ch.steps]))
+        feeds = {"x": ch.x}
+        ref = run_ref(lambda b: ch.build(b, probe=lambda k, v: b.output(v, "p%d" % k)), feeds)
+        prof_path = str(tmp_path / ("chain%d.prof" % seed))
+        with cal.Profiler(prof_path, channel_axis=1) as p:
+            hb = odla.HipBuilder()
+            try:
+                ch.build(hb)
+                s = hb.session()
+                try:
+                    with p.run("only"):
+                        s.run(feeds)
+                finally:
+                    s.close()
+            finally:
+                hb.destroy()
+        rec = cal.load_profile(prof_path)["ProfilingResults"]["only"]
+        n_checked = 0
+        for k in range(1, len(ch.steps) + 1):
+            name, want = "v%d" % k, ref["p%d" % k]
+            if name not in rec:
+                continue
+            scale = max(float(np.max(np.abs(want))), 1e-6)
+            assert abs(rec[name]["min_value"] - float(want.min())) <= 5e-4 * scale, (seed, name)
+            assert abs(rec[name]["max_value"] - float(want.max())) <= 5e-4 * scale, (seed, name)
+            assert rec[name]["shape"] == list(want.shape), (seed, name)
+            if "channels_max" in rec[name] and rec[name].get("channels") == want.shape[1]:
+                assert np.allclose(rec[name]["channels_max"], want.max(axis=(0, 2, 3)), rtol=0, atol=5e-4 * scale), (seed, name)
+                assert np.allclose(rec[name]["channels_min"], want.min(axis=(0, 2, 3)), rtol=0, atol=5e-4 * scale), (seed, name)
+            n_checked += 1
+        assert n_checked == len(ch.steps), (seed, sorted(rec))
