@@ -856,31 +856,40 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
       }
     a_mask[i] = mask;
   }
-  int tap = 0, tap_r = 0, tap_s = 0, kc0 = 0;
   using lds_ptr = __attribute__((address_space(3))) void*;
   // Requests the next K stage of the pixel tile into buffer `buf`.  Requests
-  // past the last tap (the pipeline's run-out) fetch the fill vector.
+  // past the last tap (the pipeline's run-out) fetch the fill vector.  All the
+  // bookkeeping is wavefront-uniform and incremental - the element offset of
+  // the stage from tap (0,0), the bit of the tap in the validity masks, the LDS
+  // address - so that a stage costs one select and one request per row.
+  int tap = 0, tap_s = 0, kc0 = 0;
+  int toff = 0;             // offset of (tap, kc0) from tap (0,0), channel 0, in elements
+  unsigned tapbit = 1u;     // 1 << tap, 0 behind the last tap
+  const int step_s = p.dw * p.xcs;                              // to the next tap of the row
+  const int step_r = p.dh * p.W * p.xcs - (p.S - 1) * step_s;   // from the last tap of a row to the first of the next
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const uint64_t fill_u = reinterpret_cast<uint64_t>(fill_ptr);
   auto dma = [&](const int buf) {
-    // (1x1 filters may have any channel count: the last stage is then partial
-    // and this thread's chunk may lie beyond C, where the weights are zero)
-    const bool live = tap < RS && kc0 + kv * VEC < p.C;
-    const int64_t toff = ((int64_t)(tap_r * p.dh) * p.W + tap_s * p.dw) * p.xcs + kc0;
-    unsigned char* dst = smem + buf * BUF_BYTES + wave * 1024;
+    unsigned char* dst = smem + buf * BUF_BYTES + wave_u * 1024;
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) {
-      const bool ok = live && ((a_mask[i] >> (tap & 31)) & 1u);
-      const TIn* src = ok ? a_row[i] + toff : fill_ptr;
+      const uint64_t live = reinterpret_cast<uint64_t>(a_row[i] + toff);
+      const uint64_t src = (a_mask[i] & tapbit) != 0u ? live : fill_u;
 #if defined(__HIP_DEVICE_COMPILE__)  // (the builtin is unknown to the host pass, which only needs the launch stub)
-      __builtin_amdgcn_global_load_lds(src, (lds_ptr)(dst + i * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const TIn*>(src), (lds_ptr)(dst + i * 4096), 16, 0, 0);
 #else
       (void)src; (void)dst;
 #endif
     }
     kc0 += BK;
+    toff += BK;
     if (kc0 >= p.C) {
       kc0 = 0;
+      toff -= p.C;
       ++tap;
-      if (++tap_s == p.S) { tap_s = 0; ++tap_r; }
+      tapbit = tap < RS ? tapbit << 1 : 0u;
+      if (++tap_s == p.S) { tap_s = 0; toff += step_r; }
+      else toff += step_s;
     }
   };
 
@@ -1194,6 +1203,8 @@ hipError_t launch_wreg(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
   const int64_t tiles = ((M + 127) / 128) * ((p.Kout + 127) / 128);
   if (tiles <= 0 || tiles > 0x7fffffff) return hipErrorInvalidValue;
+  // what the kernel's tap walk assumes: whole K stages per tap, one mask bit per tap
+  if (p.C % (128 / (int)sizeof(TIn)) != 0 || p.R * p.S > 32) return hipErrorInvalidValue;
   hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0, stream,
                      p, epi_vec);
   return hipGetLastError();
