@@ -782,23 +782,30 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
 // valid addresses at the ends): the number of operations in flight at each
 // wait is a compile-time constant.  Padding taps and out-of-range rows fetch a
 // 16-byte fill vector stored behind the weight fragments.
-template <typename TIn, typename Epi>
-// three wavefronts per SIMD: at most 168 registers (two with the transcendental
-// activations in the epilogue, which need more)
-__global__ void __launch_bounds__(256, EpiTraits<Epi>::rich ? 2 : 3)
+//
+// NJ = 2: every wavefront owns two 32-channel slices (channels wave*32 and 128 +
+// wave*32 of a 256-channel tile), i.e. twice the MFMA work for the same pixel
+// fragments read from LDS and the same pixel requests; it pays for that with twice
+// the accumulators and weight fragments (two wavefronts per SIMD).
+template <typename TIn, typename Epi, int NJ>
+// NJ = 1: three wavefronts per SIMD: at most 168 registers (two with the
+// transcendental activations in the epilogue, which need more)
+__global__ void __launch_bounds__(256, (EpiTraits<Epi>::rich || NJ == 2) ? 2 : 3)
 igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
-  constexpr int BM = 128, BN = 128, WM = 128, WN = 32, NW = 4;
+  constexpr int BM = 128, BN = 128 * NJ, WM = 128, NW = 4;
+  constexpr int NWF = 4 * NJ;  // weight fragments of a wavefront per K stage
   constexpr int ES = sizeof(TIn);
   constexpr int BKB = 128, BK = BKB / ES;
   constexpr int VEC = 16 / ES, A_IT = 4;
   constexpr int TM = WM / 32;
   constexpr int BUF_BYTES = BM * BKB;  // 16 KiB
   constexpr int NBUF = 3;
-  constexpr int EPI_BYTES = 2 * 32 * (BN + 4) * 4;
+  constexpr int EPI_BYTES = 2 * 32 * (128 + 4) * 4;
   static_assert(NBUF * BUF_BYTES >= EPI_BYTES, "staging area must fit in the pixel buffers");
   using Acc = typename Mma<TIn>::Acc;
-  // s_waitcnt immediates (vmcnt only; expcnt / lgkmcnt left at their maxima)
-  constexpr int kWaitVm0 = 0x0f70, kWaitVm12 = 0x0f7c;
+  // s_waitcnt immediates (vmcnt only; expcnt / lgkmcnt left at their maxima):
+  // vmcnt(0), and vmcnt(2 * NWF + 4) = 12 / 20 for the wait at the top of a stage
+  constexpr int kWaitVm0 = 0x0f70, kWaitVmStage = NJ == 1 ? 0x0f7c : 0x4f74;
 
   __shared__ __attribute__((aligned(1024))) unsigned char smem[NBUF * BUF_BYTES];
 
@@ -817,11 +824,14 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   const int l32 = lane & 31, lg = lane >> 5;
 
   const TIn* x = reinterpret_cast<const TIn*>(p.x) + (int64_t)z * p.x_bs;
-  // fragment q of this wavefront's 32 channels: wf[q * 64]
-  int wtile = tile_n * (BN / 32) + wave;
-  wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;  // surplus wavefronts compute channels that are never stored
-  const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag) +
-                     ((int64_t)z * p.wf_tiles + wtile) * p.wf_chunks * 64 + lane;
+  // fragment q of a 32-channel slice: wf[q * 64]
+  const uintx4* wf[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    int wtile = (tile_n * NJ + j) * 4 + wave;
+    wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;  // surplus slices compute channels that are never stored
+    wf[j] = reinterpret_cast<const uintx4*>(p.w_frag) + ((int64_t)z * p.wf_tiles + wtile) * p.wf_chunks * 64 + lane;
+  }
   const TIn* fill_ptr = reinterpret_cast<const TIn*>(reinterpret_cast<const unsigned char*>(p.w_frag) +
                                                      (int64_t)p.batch * p.wf_tiles * p.wf_chunks * 1024);
 
@@ -893,11 +903,13 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
     }
   };
 
-  Acc acc[TM][1];
+  Acc acc[NJ][TM][1];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int j = 0; j < NJ; ++j)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][0][e] = 0;
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[j][i][0][e] = 0;
   if constexpr (EpiTraits<Epi>::quant) {
     // 8-bit layers: the int32 bias starts in the accumulators (element q*4 + r of
     // a lane is channel wave*32 + q*8 + (lane/32)*4 + r), which takes its addition
@@ -907,17 +919,20 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
     // waits of the K loop allow for.
     if (p.bias != nullptr) {
       const int* bias = reinterpret_cast<const int*>(p.bias) + (int64_t)z * p.bias_bs;
-      const int nb = tile_n * BN + __builtin_amdgcn_readfirstlane(wave) * 32;
       const int last = p.Kout - 1;  // channels past the end are computed but never stored
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int j = 0; j < NJ; ++j) {
+        const int nb = (tile_n * NJ + j) * 128 + wave_u * 32;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int c0 = nb + q * 8 + r, c1 = c0 + 4;
-          const int b0 = bias[c0 < last ? c0 : last], b1 = bias[c1 < last ? c1 : last];
-          const int b = lg ? b1 : b0;
+        for (int q = 0; q < 4; ++q) {
 #pragma unroll
-          for (int i = 0; i < TM; ++i) acc[i][0][q * 4 + r] = b;
+          for (int r = 0; r < 4; ++r) {
+            const int c0 = nb + q * 8 + r, c1 = c0 + 4;
+            const int b0 = bias[c0 < last ? c0 : last], b1 = bias[c1 < last ? c1 : last];
+            const int b = lg ? b1 : b0;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) acc[j][i][0][q * 4 + r] = b;
+          }
         }
       }
     }
@@ -946,8 +961,8 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "=v"(dst) : "v"(ptr) : "memory")
 #define IGEMM_WRELOAD(dst, ptr, OFF) \
   asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "+v"(dst) : "v"(ptr) : "memory")
-#define IGEMM_WWAIT15(dst) asm volatile("s_waitcnt vmcnt(15)" : "+v"(dst) : : "memory")
-#define IGEMM_WDRAIN(a, b)                                                                                     \
+#define IGEMM_WWAIT(N, dst) asm volatile("s_waitcnt vmcnt(" #N ")" : "+v"(dst) : : "memory")
+#define IGEMM_WDRAIN8(a, b)                                                                                    \
   asm volatile("s_waitcnt vmcnt(0)"                                                                            \
                : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) \
                :                                                                                               \
@@ -955,32 +970,46 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
 #else
 #define IGEMM_WLOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
 #define IGEMM_WRELOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
-#define IGEMM_WWAIT15(dst) (void)(dst)
-#define IGEMM_WDRAIN(a, b) (void)(a), (void)(b)
+#define IGEMM_WWAIT(N, dst) (void)(dst)
+#define IGEMM_WDRAIN8(a, b) (void)(a), (void)(b)
 #endif
-  uintx4 w0[4], w1[4];
+  // fragment kk of slice j sits at position kk * NJ + j: the order of use
+  uintx4 w0[NWF], w1[NWF];
+  auto wload = [&](uintx4& dst, const uintx4* ptr, const int kk) __attribute__((always_inline)) {
+    if (kk == 0) IGEMM_WLOAD(dst, ptr, 0);
+    else if (kk == 1) IGEMM_WLOAD(dst, ptr, 1024);
+    else if (kk == 2) IGEMM_WLOAD(dst, ptr, 2048);
+    else IGEMM_WLOAD(dst, ptr, 3072);
+  };
+  auto wreload = [&](uintx4& dst, const uintx4* ptr, const int kk) __attribute__((always_inline)) {
+    if (kk == 0) IGEMM_WRELOAD(dst, ptr, 0);
+    else if (kk == 1) IGEMM_WRELOAD(dst, ptr, 1024);
+    else if (kk == 2) IGEMM_WRELOAD(dst, ptr, 2048);
+    else IGEMM_WRELOAD(dst, ptr, 3072);
+  };
   {
-    const uintx4* ws = wf + (int64_t)(nkt > 1 ? 1 : 0) * 4 * 64;
-    IGEMM_WLOAD(w0[0], wf, 0);
-    IGEMM_WLOAD(w0[1], wf, 1024);
-    IGEMM_WLOAD(w0[2], wf, 2048);
-    IGEMM_WLOAD(w0[3], wf, 3072);
-    IGEMM_WLOAD(w1[0], ws, 0);
-    IGEMM_WLOAD(w1[1], ws, 1024);
-    IGEMM_WLOAD(w1[2], ws, 2048);
-    IGEMM_WLOAD(w1[3], ws, 3072);
+    const int64_t second = (int64_t)(nkt > 1 ? 1 : 0) * 4 * 64;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) wload(w0[kk * NJ + j], wf[j], kk);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) wload(w1[kk * NJ + j], wf[j] + second, kk);
   }
   dma(0);
   dma(1);
 
   // One K stage.  wc = this stage's weight fragments; each is re-requested for
   // stage kt+2 right after its use.
-  auto stage = [&](const int kt, const int buf, uintx4 (&wc)[4]) {
+  auto stage = [&](const int kt, const int buf, uintx4 (&wc)[NWF]) {
     // the pixel vectors of this stage have landed (mine), and everyone's have
     // (a bare barrier: the fence of __syncthreads would also wait for the
-    // requests of the stages still in flight)
+    // requests of the stages still in flight).  Behind them in flight: this
+    // stage's NWF fragments and the 4 + NWF operations of the stage between.
     if (kt < 2) __builtin_amdgcn_s_waitcnt(kWaitVm0);
-    else __builtin_amdgcn_s_waitcnt(kWaitVm12);
+    else __builtin_amdgcn_s_waitcnt(kWaitVmStage);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -989,7 +1018,9 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
     __builtin_amdgcn_sched_barrier(0);
     const unsigned char* ab = smem + buf * BUF_BYTES + rd_base;
     const int ktn = kt + 2 < nkt ? kt + 2 : nkt - 1;
-    const uintx4* wnext = wf + (int64_t)ktn * 4 * 64;
+    const uintx4* wnext[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) wnext[j] = wf[j] + (int64_t)ktn * 4 * 64;
     uintx4 fa[2][TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) fa[0][i] = *reinterpret_cast<const uintx4*>(ab + ((0 ^ rd_t) * 32) + i * 4096);
@@ -1000,18 +1031,21 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
         for (int i = 0; i < TM; ++i)
           fa[(kk + 1) & 1][i] = *reinterpret_cast<const uintx4*>(ab + (((kk + 1) ^ rd_t) * 32) + i * 4096);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      // In flight behind wc[kk] (requested two stages ago at this step): 3-kk
-      // fragments of that stage, 8 operations of the stage between, the 4
-      // pixel requests above and kk fragments of this stage: always 15.
-      IGEMM_WWAIT15(wc[kk]);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) acc[i][0] = Mma<TIn>::run(wc[kk], fa[kk & 1][i], acc[i][0]);
-      __builtin_amdgcn_sched_barrier(0);
-      if (kk == 0) IGEMM_WRELOAD(wc[0], wnext, 0);
-      else if (kk == 1) IGEMM_WRELOAD(wc[1], wnext, 1024);
-      else if (kk == 2) IGEMM_WRELOAD(wc[2], wnext, 2048);
-      else IGEMM_WRELOAD(wc[3], wnext, 3072);
+      for (int j = 0; j < NJ; ++j) {
+        const int k = kk * NJ + j;
+        __builtin_amdgcn_sched_barrier(0);
+        // In flight behind wc[k] (requested two stages ago at this position):
+        // NWF-1-k fragments of that stage, 4 + NWF operations of the stage
+        // between, the 4 pixel requests above and k fragments of this stage:
+        // always 2 * NWF + 7.
+        if constexpr (NJ == 1) IGEMM_WWAIT(15, wc[k]);
+        else IGEMM_WWAIT(23, wc[k]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) acc[j][i][0] = Mma<TIn>::run(wc[k], fa[kk & 1][i], acc[j][i][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        wreload(wc[k], wnext[j], kk);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -1026,13 +1060,32 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   }
   // the ring becomes the staging area: no direct-to-LDS write may still be in
   // flight, and neither may a weight fragment be
-  IGEMM_WDRAIN(w0, w1);
+  if constexpr (NJ == 1) {
+    IGEMM_WDRAIN8(w0, w1);
+  } else {
+    uintx4(&w0a)[4] = reinterpret_cast<uintx4(&)[4]>(w0[0]);
+    uintx4(&w0b)[4] = reinterpret_cast<uintx4(&)[4]>(w0[4]);
+    uintx4(&w1a)[4] = reinterpret_cast<uintx4(&)[4]>(w1[0]);
+    uintx4(&w1b)[4] = reinterpret_cast<uintx4(&)[4]>(w1[4]);
+    // (one wait names all sixteen: with two the compiler could release eight of
+    // them after the first, while their data is still in flight)
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(w0a[0]), "+v"(w0a[1]), "+v"(w0a[2]), "+v"(w0a[3]), "+v"(w0b[0]), "+v"(w0b[1]), "+v"(w0b[2]),
+                   "+v"(w0b[3]), "+v"(w1a[0]), "+v"(w1a[1]), "+v"(w1a[2]), "+v"(w1a[3]), "+v"(w1b[0]), "+v"(w1b[1]),
+                   "+v"(w1b[2]), "+v"(w1b[3])
+                 :
+                 : "memory");
+#endif
+  }
   __builtin_amdgcn_sched_barrier(0);
 #undef IGEMM_WLOAD
 #undef IGEMM_WRELOAD
-#undef IGEMM_WWAIT15
-#undef IGEMM_WDRAIN
-  igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
+#undef IGEMM_WWAIT
+#undef IGEMM_WDRAIN8
+#pragma unroll
+  for (int j = 0; j < NJ; ++j)
+    igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc[j], smem, tile_m, tile_n * NJ + j, z, M, wave, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -1198,15 +1251,41 @@ hipError_t dispatch_tiles(const IgemmParams& p, int epi_vec, hipStream_t s) {
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+// 32-channel slices per wavefront of the weights-in-registers kernel.
+int wreg_slices(const IgemmParams& p) {
+  if (const char* force = getenv("ODLA_HIP_WREG_SLICES")) {  // tuning aid
+    const int v = atoi(force);
+    if (v == 1 || v == 2) return v;
+  }
+  // Two slices halve the workgroups and the LDS reads per MFMA but leave two
+  // wavefronts per SIMD: measured faster only on long K loops whose grid still
+  // covers the chip (ResNet-50 at batch 256: the 3x3 256 -> 256 layers, 784 -> 392
+  // workgroups, 88 -> 76 us, and 1024 -> 256, 48 -> 43 us), slower on short ones.
+  const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+  const int64_t stages = (int64_t)p.R * p.S * p.C * dtype_size(p.in_dt) / 128;
+  const int64_t tiles2 = ((M + 127) / 128) * ((p.Kout + 255) / 256);
+  if (p.Kout % 256 == 0 && stages >= 16 && tiles2 >= 320 && tiles2 <= 512) return 2;
+  return 1;
+}
+
 template <typename TIn, typename Epi>
 hipError_t launch_wreg(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
-  const int64_t tiles = ((M + 127) / 128) * ((p.Kout + 127) / 128);
-  if (tiles <= 0 || tiles > 0x7fffffff) return hipErrorInvalidValue;
   // what the kernel's tap walk assumes: whole K stages per tap, one mask bit per tap
   if (p.C % (128 / (int)sizeof(TIn)) != 0 || p.R * p.S > 32) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0, stream,
-                     p, epi_vec);
+  // (the transcendental epilogues do not fit beside twice the accumulators)
+  const int nj = EpiTraits<Epi>::rich ? 1 : wreg_slices(p);
+  const int64_t tiles = ((M + 127) / 128) * ((p.Kout + 128 * nj - 1) / (128 * nj));
+  if (tiles <= 0 || tiles > 0x7fffffff) return hipErrorInvalidValue;
+  if constexpr (!EpiTraits<Epi>::rich) {
+    if (nj == 2) {
+      hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 2>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0,
+                         stream, p, epi_vec);
+      return hipGetLastError();
+    }
+  }
+  hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 1>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0,
+                     stream, p, epi_vec);
   return hipGetLastError();
 }
 

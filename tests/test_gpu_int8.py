@@ -103,6 +103,13 @@ def test_q8_conv_accumulators_and_requant(case, odla, ref):
     assert np.array_equal(q_got, q_want.astype(np.int64))
 
 
+@pytest.mark.parametrize("case", [c for c in Q8_CONV_CASES if c[4] > 64 and c[1] % 128 == 0])
+def test_q8_conv_two_channel_slices_per_wavefront(case, odla, ref, monkeypatch):
+    """Weights-in-registers kernel with two 32-channel slices per wavefront, 8-bit operands."""
+    monkeypatch.setenv("ODLA_HIP_WREG_SLICES", "2")
+    test_q8_conv_accumulators_and_requant(case, odla, ref)
+
+
 @pytest.mark.parametrize("tiles_per_wg", [0, 3])
 @pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (3, 128, 7, 7, 200), (4, 64, 21, 19, 256), (2, 128, 30, 30, 512),
                                   (3, 256, 9, 9, 136)])

@@ -169,6 +169,15 @@ def test_conv_parity(case, mode):
         assert np.max(np.abs(got["y"] - want["y"])) <= tol * max(1.0, float(np.max(np.abs(want["y"]))))
 
 
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if c[4] > 64 and c[1] % 64 == 0 and c[8] == 1])
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def test_conv_two_channel_slices_per_wavefront(case, mode, monkeypatch):
+    """The weights-in-registers kernel with two 32-channel slices per wavefront (256-channel
+    tiles), which the library picks by itself only for long K loops on large grids."""
+    monkeypatch.setenv("ODLA_HIP_WREG_SLICES", "2")
+    test_conv_parity(case, mode)
+
+
 LEAN_CASES = [
     # 1x1 filters over 64 / 128 bytes of input channels per pixel (the streaming kernel):
     # N, C, H, W, O, stride, residual
