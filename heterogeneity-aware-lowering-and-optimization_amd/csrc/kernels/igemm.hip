@@ -499,11 +499,21 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
       dst[ps] = *reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n);
     }
   };
-  RVec rcur[2], rnxt[2];
+  // The residual vectors of all four slices are requested here, ahead of the
+  // parking and the barriers of the first slice: one memory round trip per tile.
+  // (Fetched a slice ahead instead, each slice would wait for its own request:
+  // behind the stores of the slice before, the compiler waits for every
+  // vector-memory operation in flight.)
+  RVec rall[TM][2];
 #pragma unroll
-  for (int ps = 0; ps < 2; ++ps) { rcur[ps] = RVec{}; rnxt[ps] = RVec{}; }
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) rall[i][ps] = RVec{};
   if constexpr (Epi::kPrefetchResidual) {
-    if (have_rpre) rfetch(0, rcur);
+    if (have_rpre) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) rfetch(i, rall[i]);
+    }
   }
 
   // Workgroup barrier for LDS traffic only: the fence of __syncthreads would
@@ -540,9 +550,6 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     // other tile only after its own read-back of slice i, and nobody passes
     // this barrier before every wavefront has finished reading slice i-1.
     lds_barrier();
-    if constexpr (Epi::kPrefetchResidual) {
-      if (have_rpre && i + 1 < TM) rfetch(i + 1, rnxt);
-    }
 #pragma unroll
     for (int ps = 0; ps < 2; ++ps) {
       const int pix = ps * 16 + rp;
@@ -564,11 +571,9 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
         // thread row pointer + a wavefront-uniform offset
         TOut* yrow = ythr + (int64_t)(i * 32 + ps * 16) * p.ycs;
         const TOut* rrow = rbase ? rthr + (int64_t)(i * 32 + ps * 16) * p.rcs : nullptr;
-        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rcur[ps]);
+        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rall[i][ps]);
       }
     }
-#pragma unroll
-    for (int ps = 0; ps < 2; ++ps) rcur[ps] = rnxt[ps];
   };
   static_assert(TM == 4, "one call per slice below");
   slice(std::integral_constant<int, 0>{});
