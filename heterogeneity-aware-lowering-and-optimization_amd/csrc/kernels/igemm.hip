@@ -840,6 +840,64 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   const TIn* fill_ptr = reinterpret_cast<const TIn*>(reinterpret_cast<const unsigned char*>(p.w_frag) +
                                                      (int64_t)p.batch * p.wf_tiles * p.wf_chunks * 1024);
 
+  const int nkt = p.wf_chunks / 4;
+
+  // Weight fragment requests and their waits are issued by hand: next to the
+  // direct-to-LDS loads the compiler would otherwise treat the vector-memory
+  // counter as unordered and wait for everything in flight at each use.
+  // wload: dst <- ptr[off bytes]; wwait<n>: dst is valid once at most n younger
+  // vector-memory operations are still in flight.  A request inside the K loop
+  // names its register as input and output, which ties every request for a
+  // fragment to one physical register, and the wait behind the loop names all
+  // eight: the compiler then sees them occupied on every path out of the loop,
+  // also on those where the last requests are never consumed, and cannot hand
+  // one of them to another value while data is still on its way into it.
+  // (The host pass only needs the kernel's launch stub; it cannot parse the
+  // vector-register constraints.)
+#if defined(__HIP_DEVICE_COMPILE__)
+#define IGEMM_WLOAD(dst, ptr, OFF) \
+  asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "=v"(dst) : "v"(ptr) : "memory")
+#define IGEMM_WRELOAD(dst, ptr, OFF) \
+  asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "+v"(dst) : "v"(ptr) : "memory")
+#define IGEMM_WWAIT(N, dst) asm volatile("s_waitcnt vmcnt(" #N ")" : "+v"(dst) : : "memory")
+#define IGEMM_WDRAIN8(a, b)                                                                                    \
+  asm volatile("s_waitcnt vmcnt(0)"                                                                            \
+               : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) \
+               :                                                                                               \
+               : "memory")
+#else
+#define IGEMM_WLOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
+#define IGEMM_WRELOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
+#define IGEMM_WWAIT(N, dst) (void)(dst)
+#define IGEMM_WDRAIN8(a, b) (void)(a), (void)(b)
+#endif
+  // fragment kk of slice j sits at position kk * NJ + j: the order of use
+  uintx4 w0[NWF], w1[NWF];
+  auto wload = [&](uintx4& dst, const uintx4* ptr, const int kk) __attribute__((always_inline)) {
+    if (kk == 0) IGEMM_WLOAD(dst, ptr, 0);
+    else if (kk == 1) IGEMM_WLOAD(dst, ptr, 1024);
+    else if (kk == 2) IGEMM_WLOAD(dst, ptr, 2048);
+    else IGEMM_WLOAD(dst, ptr, 3072);
+  };
+  auto wreload = [&](uintx4& dst, const uintx4* ptr, const int kk) __attribute__((always_inline)) {
+    if (kk == 0) IGEMM_WRELOAD(dst, ptr, 0);
+    else if (kk == 1) IGEMM_WRELOAD(dst, ptr, 1024);
+    else if (kk == 2) IGEMM_WRELOAD(dst, ptr, 2048);
+    else IGEMM_WRELOAD(dst, ptr, 3072);
+  };
+  {
+    const int64_t second = (int64_t)(nkt > 1 ? 1 : 0) * 4 * 64;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) wload(w0[kk * NJ + j], wf[j], kk);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) wload(w1[kk * NJ + j], wf[j] + second, kk);
+  }
+  // (requested this early, the fragments travel while the gather state below is computed)
+
   // ---- gather state: this thread feeds rows row0 + 32*i, slot lane%8 ----
   // C is a multiple of the stage depth, so a stage lies inside one filter tap
   // and the tap walk is wavefront-uniform (scalar registers).  Per row the
@@ -943,66 +1001,11 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
     }
   }
 
-  const int nkt = p.wf_chunks / 4;
   // fragment read offsets: row l32 (+32*i), chunk 2*kk + lg, swizzled
   const int sw = (l32 >> 1) & 7;
   const int rd_base = l32 * 128 + ((lg ^ (sw & 1)) * 16);
   const int rd_t = sw >> 1;
 
-  // Weight fragment requests and their waits are issued by hand: next to the
-  // direct-to-LDS loads the compiler would otherwise treat the vector-memory
-  // counter as unordered and wait for everything in flight at each use.
-  // wload: dst <- ptr[off bytes]; wwait<n>: dst is valid once at most n younger
-  // vector-memory operations are still in flight.  A request inside the K loop
-  // names its register as input and output, which ties every request for a
-  // fragment to one physical register, and the wait behind the loop names all
-  // eight: the compiler then sees them occupied on every path out of the loop,
-  // also on those where the last requests are never consumed, and cannot hand
-  // one of them to another value while data is still on its way into it.
-  // (The host pass only needs the kernel's launch stub; it cannot parse the
-  // vector-register constraints.)
-#if defined(__HIP_DEVICE_COMPILE__)
-#define IGEMM_WLOAD(dst, ptr, OFF) \
-  asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "=v"(dst) : "v"(ptr) : "memory")
-#define IGEMM_WRELOAD(dst, ptr, OFF) \
-  asm volatile("global_load_dwordx4 %0, %1, off offset:" #OFF : "+v"(dst) : "v"(ptr) : "memory")
-#define IGEMM_WWAIT(N, dst) asm volatile("s_waitcnt vmcnt(" #N ")" : "+v"(dst) : : "memory")
-#define IGEMM_WDRAIN8(a, b)                                                                                    \
-  asm volatile("s_waitcnt vmcnt(0)"                                                                            \
-               : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) \
-               :                                                                                               \
-               : "memory")
-#else
-#define IGEMM_WLOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
-#define IGEMM_WRELOAD(dst, ptr, OFF) (dst) = (ptr)[(OFF) / 16]
-#define IGEMM_WWAIT(N, dst) (void)(dst)
-#define IGEMM_WDRAIN8(a, b) (void)(a), (void)(b)
-#endif
-  // fragment kk of slice j sits at position kk * NJ + j: the order of use
-  uintx4 w0[NWF], w1[NWF];
-  auto wload = [&](uintx4& dst, const uintx4* ptr, const int kk) __attribute__((always_inline)) {
-    if (kk == 0) IGEMM_WLOAD(dst, ptr, 0);
-    else if (kk == 1) IGEMM_WLOAD(dst, ptr, 1024);
-    else if (kk == 2) IGEMM_WLOAD(dst, ptr, 2048);
-    else IGEMM_WLOAD(dst, ptr, 3072);
-  };
-  auto wreload = [&](uintx4& dst, const uintx4* ptr, const int kk) __attribute__((always_inline)) {
-    if (kk == 0) IGEMM_WRELOAD(dst, ptr, 0);
-    else if (kk == 1) IGEMM_WRELOAD(dst, ptr, 1024);
-    else if (kk == 2) IGEMM_WRELOAD(dst, ptr, 2048);
-    else IGEMM_WRELOAD(dst, ptr, 3072);
-  };
-  {
-    const int64_t second = (int64_t)(nkt > 1 ? 1 : 0) * 4 * 64;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) wload(w0[kk * NJ + j], wf[j], kk);
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) wload(w1[kk * NJ + j], wf[j] + second, kk);
-  }
   dma(0);
   dma(1);
 
