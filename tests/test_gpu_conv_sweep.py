@@ -14,6 +14,9 @@ from util import announce, max_rel_err, run_hip, run_ref
 
 pytestmark = pytest.mark.gpu
 
+# ODLA_SWEEP_SEED=<n> shifts every seed below: other random cases, same code (default 0)
+SEED0 = int(__import__("os").environ.get("ODLA_SWEEP_SEED", "0"))
+
 sys.path.insert(0, os.path.join(entry.ROOT, "oracle"))
 
 CH_IN = [1, 3, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256]
@@ -102,7 +105,7 @@ def cases(seed, count):
 @pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16"])
 def test_random_convolutions(mode):
     kw = {"fp16": mode == "fp16", "bf16": mode == "bf16"}
-    for i, c in enumerate(cases(2024, 60)):
+    for i, c in enumerate(cases(SEED0 + 2024, 60)):
         announce("sweep %s #%d %s" % (mode, i, c))
         x, w, bias, res = tensors_for(c, 500 + i)
         feeds = {"x": x}
@@ -126,7 +129,7 @@ def test_random_convolutions_int8():
     models = entry.load().models
     ref = entry.load_oracle()
     done = 0
-    for i, c in enumerate(cases(777, 140)):
+    for i, c in enumerate(cases(SEED0 + 777, 140)):
         if c["group"] != 1 or c["dh"] != 1 or c["dw"] != 1:
             continue        # the 8-bit plan covers dense, undilated convolutions; the rest stays in float
         if c["pad"][0] != c["pad"][2] or c["pad"][1] != c["pad"][3] or c["kh"] != c["kw"] or c["sh"] != c["sw"]:

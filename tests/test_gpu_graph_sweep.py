@@ -10,6 +10,9 @@ from util import announce, max_rel_err, run_hip, run_hip_stored, run_ref
 
 pytestmark = pytest.mark.gpu
 
+# ODLA_SWEEP_SEED=<n> shifts every seed below: other random cases, same code (default 0)
+SEED0 = int(__import__("os").environ.get("ODLA_SWEEP_SEED", "0"))
+
 
 class Chain:
     """A recorded random program: a list of steps replayed on any builder."""
@@ -139,7 +142,7 @@ class Chain:
 @pytest.mark.parametrize("mode", ["fp32", "fp16"])
 def test_random_chains(mode, tmp_path):
     for seed in range(200):
-        ch = Chain(seed)
+        ch = Chain(SEED0 + seed)
         if not ch.steps:
             continue
         announce("chain %s seed %d: %s -> outputs %s" % (mode, seed, [s[0] for s in ch.steps], ch.outputs))
@@ -190,9 +193,9 @@ def test_random_chains_in_interpret_mode():
             assert self.L.odla_GetValueData(v, out.ctypes.data_as(ctypes.c_void_p), None) == 0
             return out
 
-    r = np.random.default_rng(5)
+    r = np.random.default_rng(SEED0 + 5)
     for seed in range(0, 200, 5):
-        ch = Chain(seed)
+        ch = Chain(SEED0 + seed)
         if not ch.steps:
             continue
         announce("interpret chain seed %d: %s" % (seed, [s[0] for s in ch.steps]))
@@ -223,7 +226,7 @@ def test_random_chains_under_the_calibration_profiler(tmp_path):
     pkg = entry.load()
     cal, odla = pkg.calibration, pkg.odla
     for seed in range(2, 200, 9):
-        ch = Chain(seed)
+        ch = Chain(SEED0 + seed)
         if not ch.steps:
             continue
         announce("profiled chain seed %d: %s" % (seed, [s[0] for s in ch.steps]))

@@ -14,6 +14,9 @@ from util import announce, max_rel_err, run_hip, run_hip_stored, run_ref
 
 pytestmark = pytest.mark.gpu
 
+# ODLA_SWEEP_SEED=<n> shifts every seed below: other random cases, same code (default 0)
+SEED0 = int(__import__("os").environ.get("ODLA_SWEEP_SEED", "0"))
+
 
 def source(b, name, shape, behind_conv, seed, mix=0.05):
     """A value of `shape`: the argument itself, or a 1x1 convolution of it (identity
@@ -58,7 +61,7 @@ def rand_shape4(r):
 
 @pytest.mark.parametrize("behind_conv", [False, True])
 def test_movement_sweep(behind_conv):
-    r = np.random.default_rng(31 + behind_conv)
+    r = np.random.default_rng(SEED0 + 31 + behind_conv)
     for i in range(40):
         shape = rand_shape4(r)
         kind = str(r.choice(["transpose", "slice", "concat", "pad", "tile", "resize", "reshape_transpose", "strided_slice"]))
@@ -106,7 +109,7 @@ def test_movement_sweep(behind_conv):
 
 @pytest.mark.parametrize("behind_conv", [False, True])
 def test_reduction_and_normalisation_sweep(behind_conv):
-    r = np.random.default_rng(41 + behind_conv)
+    r = np.random.default_rng(SEED0 + 41 + behind_conv)
     kinds = ["reduce_mean", "reduce_sum", "reduce_max", "reduce_min", "reduce_sum_square", "reduce_log_sum_exp",
              "softmax", "log_softmax", "layernorm", "batchnorm", "maxpool", "avgpool", "argmax", "instance_norm", "lrn"]
     for i in range(60):
@@ -161,15 +164,16 @@ def test_reduction_and_normalisation_sweep(behind_conv):
         # fp16 plans, representable, so that rounding cannot reorder them)
         modes = ("fp32", "fp16")
         if kind == "argmax":
-            x = (r.permutation(x.size).reshape(shape).astype(np.float32) / 8.0) if x.size < 2048 * 8 else x
-            modes = ("fp32",) if behind_conv else modes
+            x = r.permutation(x.size).reshape(shape).astype(np.float32) / 8.0
+            # k / 8 is exact in fp16 only up to k = 2048: beyond that rounding makes ties
+            modes = ("fp32",) if behind_conv or x.size > 2048 else modes
         if kind in ("reduce_sum", "reduce_sum_square", "reduce_log_sum_exp"):
             modes = ("fp32",) if np.prod([shape[a] for a in axes]) > 512 else modes
         check(build, {"x": x}, tag=tag, modes=modes)
 
 
 def test_gemm_sweep():
-    r = np.random.default_rng(51)
+    r = np.random.default_rng(SEED0 + 51)
     for i in range(50):
         M, K, N = int(r.integers(1, 200)), int(r.choice([1, 7, 16, 64, 100, 256, 777])), int(r.choice([1, 5, 10, 64, 130, 256]))
         ta, tb = bool(r.random() < 0.3), bool(r.random() < 0.4)
@@ -202,7 +206,7 @@ def test_gemm_sweep():
 
 
 def test_binary_broadcast_sweep():
-    r = np.random.default_rng(61)
+    r = np.random.default_rng(SEED0 + 61)
     ops = ["add", "sub", "mul", "div", "max", "min", "pow", "squared_difference", "less", "equal"]
     for i in range(60):
         rank = int(r.integers(1, 5))
@@ -257,7 +261,7 @@ def test_binary_broadcast_sweep():
 
 
 def test_gather_cast_sweep():
-    r = np.random.default_rng(71)
+    r = np.random.default_rng(SEED0 + 71)
     for i in range(20):
         rank = int(r.integers(1, 4))
         shape = tuple(int(r.integers(2, 12)) for _ in range(rank))
@@ -306,7 +310,7 @@ UNARY = {
 
 @pytest.mark.parametrize("behind_conv", [False, True])
 def test_unary_sweep(behind_conv):
-    r = np.random.default_rng(81 + behind_conv)
+    r = np.random.default_rng(SEED0 + 81 + behind_conv)
     for i, (name, (call, dom)) in enumerate(sorted(UNARY.items())):
         rank = 4 if behind_conv else int(r.integers(1, 5))
         shape = rand_shape4(r) if rank == 4 else tuple(int(r.integers(1, 40)) for _ in range(rank))
@@ -331,7 +335,7 @@ def test_unary_sweep(behind_conv):
 
 
 def test_compare_select_logic_sweep():
-    r = np.random.default_rng(91)
+    r = np.random.default_rng(SEED0 + 91)
     for i in range(30):
         rank = int(r.integers(1, 5))
         shape = tuple(int(r.integers(1, 10)) for _ in range(rank))
@@ -356,7 +360,7 @@ def test_compare_select_logic_sweep():
 
 
 def test_topk_stack_squeeze_sweep():
-    r = np.random.default_rng(101)
+    r = np.random.default_rng(SEED0 + 101)
     for i in range(24):
         rank = int(r.integers(1, 4))
         shape = tuple(int(r.integers(2, 30)) for _ in range(rank))
@@ -379,7 +383,7 @@ def test_topk_stack_squeeze_sweep():
 
 
 def test_deconv_sweep():
-    r = np.random.default_rng(111)
+    r = np.random.default_rng(SEED0 + 111)
     for i in range(16):
         N, C, O = int(r.integers(1, 3)), int(r.choice([4, 8, 16])), int(r.choice([3, 8, 16]))
         H, W = int(r.integers(3, 9)), int(r.integers(3, 9))
@@ -401,7 +405,7 @@ def test_deconv_sweep():
 
 
 def test_quantize_dequantize_sweep():
-    r = np.random.default_rng(121)
+    r = np.random.default_rng(SEED0 + 121)
     for i in range(20):
         rank = int(r.integers(1, 5))
         shape = tuple(int(r.integers(1, 12)) for _ in range(rank))
