@@ -446,7 +446,7 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
     auto it = ctx->bound_out.find(io.v);
     if (it == ctx->bound_out.end()) continue;
     const PTensor& t = plan.tensors[io.tensor];
-    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset;
+    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset + io.offset;
     if (hipMemcpyAsync(it->second, src, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
       OHIP_ERR("odla_ExecuteComputation: copy of output '%s' failed", io.v->name.c_str());
       return ODLA_FAILURE;
@@ -661,7 +661,7 @@ odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr, odla_
   for (const Plan::IO& io : plan.outputs) {
     if (io.v != value) continue;
     const PTensor& t = plan.tensors[io.tensor];
-    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset;
+    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset + io.offset;
     if (hipMemcpy(data_ptr, src, io.bytes, hipMemcpyDefault) != hipSuccess) return ODLA_FAILURE;
     return ODLA_SUCCESS;
   }

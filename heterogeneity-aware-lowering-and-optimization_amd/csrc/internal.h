@@ -123,7 +123,8 @@ struct PTensor {
   Space space = SP_NONE;
   size_t offset = 0;
   size_t bytes = 0;
-  int alias_of = -1;     // shares storage with another tensor (Reshape)
+  int alias_of = -1;     // shares storage with another tensor (Reshape, a slice of a merged result)
+  size_t alias_off = 0;  // byte offset of an alias inside the root tensor's storage
   int def_step = -1, last_step = -1;
   bool pinned = false;   // lives for the whole execution (inputs being staged, outputs)
   bool quant = false;    // 8-bit affine levels stored as q-128
@@ -162,6 +163,7 @@ struct Plan {
   struct IO {
     _odla_value* v = nullptr;
     int tensor = -1;  // staging tensor in the arena: row-major, declared element type
+    size_t offset = 0;  // byte offset inside that tensor (results that are slices of a merged launch)
     size_t bytes = 0;
   };
   std::vector<IO> inputs, outputs;

@@ -125,6 +125,18 @@ class Planner {
     plan_->tensors.push_back(t);
     return (int)plan_->tensors.size() - 1;
   }
+  // a dense row-major view of `shape` that starts `byte_off` bytes into `src`
+  int view_tensor(int src, const Shape& shape, size_t byte_off) {
+    PTensor t = plan_->tensors[src];
+    t.shape = shape;
+    t.layout = L_ROWMAJOR;
+    t.cs = 0;
+    t.alias_of = root(src);
+    t.alias_off = plan_->tensors[src].alias_off + byte_off;
+    t.bytes = (size_t)shape.numel() * dtype_size(t.dt);
+    plan_->tensors.push_back(t);
+    return (int)plan_->tensors.size() - 1;
+  }
   int root(int t) const {
     while (plan_->tensors[t].alias_of >= 0) t = plan_->tensors[t].alias_of;
     return t;
@@ -139,7 +151,7 @@ class Planner {
       int r = t;
       while (plan->tensors[r].alias_of >= 0) r = plan->tensors[r].alias_of;
       const PTensor& pt = plan->tensors[r];
-      return env.base[pt.space] + pt.offset;
+      return env.base[pt.space] + pt.offset + plan->tensors[t].alias_off;  // (alias offsets are relative to the root)
     }
   };
   Ref ref(int t) const { return Ref{plan_, t}; }
@@ -461,6 +473,9 @@ class Planner {
   void lower_lrn(int ni);
   void lower_rownorm(int ni);
   void lower_postprocess(int ni);
+  bool gemm_epilogue(int ni, Epilogue* ep);
+  std::unordered_map<int, Epilogue> gemm_ep_ahead_;  // epilogues collected while looking for sibling GEMMs
+  std::vector<char> gemm_merged_;                    // nodes already lowered inside a sibling's launch
   void emit_stats(const _odla_value* v, const char* op_type, int forced_axis, const Node* producer);
   bool calib_ = false;
   struct SoftmaxAdd { const _odla_value* x; const _odla_value* mask; int64_t div; };
@@ -636,6 +651,7 @@ void Planner::run() {
     Plan::IO io;
     io.v = ov;
     io.tensor = root(t);
+    io.offset = T(t).alias_off;
     io.bytes = (size_t)ov->shape.numel() * dtype_size(want);
     plan_->outputs.push_back(io);
   }
@@ -1348,11 +1364,39 @@ void Planner::lower_conv(int ni) {
 }
 
 // ---------------------------------------------------------------- Gemm ----
+// Bias operand of a Gemm node (alpha*(A.B) + beta*C) and the operators folded
+// behind it.  Returns false when C is a run-time matrix (then it rides as the
+// residual and nothing else is folded).
+bool Planner::gemm_epilogue(int ni, Epilogue* ep) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* Cv = n.in[2];
+  const Shape& os = n.out->shape;
+  const int64_t Nn = os.d[os.rank - 1];
+  const float beta = n.f[1];
+  _odla_value* full_c = nullptr;
+  if (Cv != nullptr && beta != 0.f) {
+    const int64_t cn = Cv->shape.numel();
+    if (Cv->kind == _odla_value::CONSTANT && (cn == 1 || cn == Nn)) {
+      std::vector<float> c = const_as_float(Cv);
+      ep->bias.assign((size_t)Nn, 0.f);
+      for (int64_t j = 0; j < Nn; ++j) ep->bias[j] = beta * c[cn == 1 ? 0 : j];
+      ep->has_bias = true;
+    } else if (beta == 1.f && Cv->shape == os && Cv->kind != _odla_value::CONSTANT) {
+      full_c = const_cast<_odla_value*>(Cv);
+    } else {
+      fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: C operand of shape %s with beta %g is not supported", Cv->shape.str().c_str(), beta);
+    }
+  }
+  if (full_c == nullptr) collect_epilogue(ni, Nn, os.rank - 1, ep);
+  else { ep->residual = full_c; ep->final_value = n.out; }
+  return full_c == nullptr;
+}
+
 void Planner::lower_gemm(int ni) {
+  if (ni < (int)gemm_merged_.size() && gemm_merged_[ni]) return;  // computed by an earlier sibling's launch
   Node& n = comp_->nodes[ni];
   const _odla_value* A = n.in[0];
   const _odla_value* B = n.in[1];
-  const _odla_value* Cv = n.in[2];
   const bool tA = n.i[0] != 0, tB = n.i[1] != 0;
   const Shape& as = A->shape;
   const Shape& bs = B->shape;
@@ -1367,25 +1411,53 @@ void Planner::lower_gemm(int ni) {
   const int vec = 16 / dtype_size(dt);
 
   Epilogue ep;
-  // bias operand: alpha*(A.B) + beta*C
-  const float alpha = n.f[0], beta = n.f[1];
-  _odla_value* full_c = nullptr;
-  if (Cv != nullptr && beta != 0.f) {
-    const int64_t cn = Cv->shape.numel();
-    if (Cv->kind == _odla_value::CONSTANT && (cn == 1 || cn == Nn)) {
-      std::vector<float> c = const_as_float(Cv);
-      ep.bias.assign((size_t)Nn, 0.f);
-      for (int64_t j = 0; j < Nn; ++j) ep.bias[j] = beta * c[cn == 1 ? 0 : j];
-      ep.has_bias = true;
-    } else if (beta == 1.f && Cv->shape == os && Cv->kind != _odla_value::CONSTANT) {
-      full_c = const_cast<_odla_value*>(Cv);
-    } else {
-      fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: C operand of shape %s with beta %g is not supported", Cv->shape.str().c_str(), beta);
+  const float alpha = n.f[0];
+  bool plain_c = true;
+  {
+    auto ahead = gemm_ep_ahead_.find(ni);
+    if (ahead != gemm_ep_ahead_.end()) { ep = ahead->second; gemm_ep_ahead_.erase(ahead); }
+    else plain_c = gemm_epilogue(ni, &ep);
+  }
+  _odla_value* outv = ep.final_value;
+
+  // ---- sibling GEMMs: the same left operand against several constant matrices
+  // of one shape (the query / key / value projections of an attention block),
+  // each too small to fill the chip.  They run as ONE batched launch whose
+  // batch stride on the left operand is zero; every result is a slice of the
+  // launch's output.
+  std::vector<int> group;  // node indices, this one first
+  std::vector<Epilogue> group_ep;
+  {
+    const int es0 = dtype_size(dt);
+    const int64_t rows = lead * M;
+    const int64_t tiles = ((rows + 127) / 128) * ((Nn + 127) / 128);
+    auto simple = [&](const Epilogue& e) {
+      return e.residual == nullptr && e.row_scale.empty() && e.final_value != nullptr &&
+             storage_dtype(e.final_value) == dt && !e.final_value->is_output;
+    };
+    if (!calib_ && plain_c && B->kind == _odla_value::CONSTANT && shared_b && !tA && K % vec == 0 && Nn % 32 == 0 &&
+        A->kind != _odla_value::CONSTANT && tiles <= 512 && (int64_t)K * es0 >= 256 && simple(ep)) {
+      group.push_back(ni);
+      group_ep.push_back(ep);
+      for (int mi = ni + 1; mi < (int)comp_->nodes.size() && group.size() < 8; ++mi) {
+        Node& m = comp_->nodes[mi];
+        if (m.op != OP_GEMM || m.absorbed || m.in[0] != A || (m.i[0] != 0) != tA || (m.i[1] != 0) != tB) continue;
+        if (m.f[0] != alpha || m.in[1] == nullptr || m.in[1]->kind != _odla_value::CONSTANT) continue;
+        if (!(m.in[1]->shape == bs) || !(m.out->shape == os) || m.out->etype != n.out->etype) continue;
+        if (gemm_ep_ahead_.count(mi) || (mi < (int)gemm_merged_.size() && gemm_merged_[mi])) continue;
+        Epilogue em;
+        const bool plain = gemm_epilogue(mi, &em);
+        if (plain && simple(em) && em.act == ep.act && em.act_a == ep.act_a && em.act_b == ep.act_b &&
+            em.scalar == ep.scalar && em.res_after_act == ep.res_after_act) {
+          group.push_back(mi);
+          group_ep.push_back(em);
+        } else {
+          gemm_ep_ahead_[mi] = em;  // folded nodes are marked already: keep what was collected for its own turn
+        }
+      }
+      if (group.size() < 2) { group.clear(); group_ep.clear(); }
     }
   }
-  if (full_c == nullptr) collect_epilogue(ni, Nn, os.rank - 1, &ep);
-  else { ep.residual = full_c; ep.final_value = n.out; }
-  _odla_value* outv = ep.final_value;
 
   // ---- A operand: row-major [lead][M][K], K padded to the vector width ----
   int ta = get(A, L_ROWMAJOR, FORM_FLOAT);
@@ -1420,6 +1492,53 @@ void Planner::lower_gemm(int ni) {
   ip.alpha = alpha * ep.scalar;
   ip.ycs = (int)Nn;
   int tw;
+  if (!group.empty()) {
+    const int G = (int)group.size();
+    // one constant [G*N][K] matrix (row n of matrix g = column n of B_g) packed like any other
+    auto buf = std::make_unique<std::vector<uint8_t>>((size_t)G * Nn * K * sizeof(float));
+    float* wcat = reinterpret_cast<float*>(buf->data());
+    std::vector<float> bias_all((size_t)G * Nn, 0.f);
+    bool any_bias = false;
+    for (int g = 0; g < G; ++g) {
+      const std::vector<float> bg = const_as_float(comp_->nodes[group[g]].in[1]);
+      for (int64_t nn = 0; nn < Nn; ++nn)
+        for (int64_t k = 0; k < K; ++k)
+          wcat[((int64_t)g * Nn + nn) * K + k] = tB ? bg[nn * K + k] : bg[k * Nn + nn];
+      if (group_ep[g].has_bias) {
+        any_bias = true;
+        for (int64_t nn = 0; nn < Nn && nn < (int64_t)group_ep[g].bias.size(); ++nn) bias_all[(size_t)(g * Nn + nn)] = group_ep[g].bias[nn];
+      }
+    }
+    _odla_value kcat;
+    kcat.kind = _odla_value::CONSTANT;
+    kcat.name = B->name;
+    kcat.etype = ODLA_FLOAT32;
+    kcat.shape.rank = 2;
+    kcat.shape.d[0] = (int64_t)G * Nn; kcat.shape.d[1] = K;
+    kcat.host_data = wcat;
+    comp_->owned_data.push_back(std::move(buf));
+    int w_rs = 0;
+    const int twc = pack_weights(&kcat, dt, 1, (int)(G * Nn), (int)K, 1, 1, Kp, K, 1, 0, 0, {}, &w_rs, nullptr);
+    ip.w_rows = (int)Nn; ip.w_cols = w_rs; ip.w_rs = w_rs;
+    ip.N = (int)(lead * M);
+    ip.batch = G;
+    ip.x_bs = 0; ip.w_bs = Nn * w_rs; ip.y_bs = lead * M * Nn; ip.bias_bs = Nn;
+    Shape all;
+    all.rank = 3;
+    all.d[0] = G; all.d[1] = lead * M; all.d[2] = Nn;
+    const int tall = new_tensor(dt, L_ROWMAJOR, all, 0, SP_ARENA);
+    Epilogue eall = ep;
+    eall.has_bias = any_bias;
+    eall.bias = bias_all;
+    finish_igemm("gemm.x" + std::to_string(G) + ":" + outv->name, ip, ta, twc, tall, eall, (int64_t)G * Nn);
+    if (gemm_merged_.size() < comp_->nodes.size()) gemm_merged_.resize(comp_->nodes.size(), 0);
+    const size_t slice_bytes = (size_t)(lead * M * Nn) * dtype_size(dt);
+    for (int g = 0; g < G; ++g) {
+      set_main(group_ep[g].final_value, view_tensor(tall, group_ep[g].final_value->shape, (size_t)g * slice_bytes));
+      if (g > 0) gemm_merged_[group[g]] = 1;
+    }
+    return;
+  }
   if (B->kind == _odla_value::CONSTANT && (shared_b || lead == 1)) {
     // weights: pack once.  B[k][n] (so=1, si=N) or B^T[n][k] (so=K, si=1)
     int w_rs = 0;

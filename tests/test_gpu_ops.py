@@ -773,3 +773,43 @@ def test_nms_parity_random(N, B, C, max_out):
 
     got, want = run_both(build, {"boxes": boxes, "scores": scores})
     assert np.array_equal(got["y"], want["y"])
+
+
+@pytest.mark.parametrize("mode", ["fp32", "bf16"])
+def test_sibling_gemms_share_one_launch(mode):
+    """Several GEMMs of one left operand against constant matrices of one shape (attention
+    projections) run as one batched launch; a sibling with another tail (ReLU), one whose
+    result is a graph output, one with another shape and one with a scalar factor stay on
+    their own - all must come out as if computed alone."""
+    announce("sibling gemms %s" % mode)
+    r = rng(77)
+    B_, S_, H_ = 3, 40, 96
+    x = r.standard_normal((B_, S_, H_)).astype(np.float32)
+    ws = [(r.standard_normal((H_, H_)) * 0.1).astype(np.float32) for _ in range(6)]
+    bs = [r.standard_normal((H_,)).astype(np.float32) for _ in range(6)]
+    w_wide = (r.standard_normal((H_, 2 * H_)) * 0.1).astype(np.float32)
+
+    def build(b):
+        v = b.arg("x", x.shape)
+        h = b.tanh(v, name="h")                          # the shared operand is a computed value
+        q = b.add(b.gemm(h, b.const("w0", ws[0]), name="q0"), b.const("b0", bs[0]), name="q")
+        k = b.add(b.gemm(h, b.const("w1", ws[1]), name="k0"), b.const("b1", bs[1]), name="k")
+        vv = b.gemm(h, b.const("w2", ws[2]), name="v")   # no bias
+        rl = b.relu(b.add(b.gemm(h, b.const("w3", ws[3]), name="r0"), b.const("b3", bs[3]), name="r1"), name="rl")
+        out_direct = b.gemm(h, b.const("w4", ws[4]), b.const("b4", bs[4].reshape(1, H_)), name="direct")
+        wide = b.gemm(h, b.const("ww", w_wide), name="wide")
+        half = b.gemm(h, b.const("w5", ws[5]), alpha=0.5, name="half")
+        s = b.add(b.add(q, k, name="qk"), b.add(vv, rl, name="vr"), name="s")
+        b.output(b.add(s, half, name="total"), "total")
+        b.output(out_direct, "direct")
+        b.output(wide, "wide")
+        # head split of one projection, as attention does
+        b.output(b.transpose(b.reshape(k, (B_, S_, 4, H_ // 4), name="kr"), (0, 2, 1, 3), name="kt"), "kt")
+
+    kw = {"bf16": mode == "bf16"}
+    got, want = run_both(build, {"x": x}, **kw)
+    for name in want:
+        if mode == "fp32":
+            assert max_rel_err(got[name], want[name]) <= F32_TOL, name
+        else:
+            assert np.max(np.abs(got[name] - want[name])) <= 6e-2 * max(1.0, float(np.max(np.abs(want[name])))), name
