@@ -1,9 +1,12 @@
-// Batched non-maximum suppression for gfx950, one workgroup per image.
+// Batched non-maximum suppression for gfx950: one launch over all boxes for the
+// class reduction, then one workgroup per image.
 //
 // Phase 1  every box competes with its best class score (first maximum over
 //          the class axis); boxes with score > score_thr become candidates.
 //          scores are [C][B] per image, so for a fixed class consecutive lanes
-//          read consecutive boxes.
+//          read consecutive boxes.  The reduction over the classes reads the
+//          whole score tensor and runs chip-wide (one thread per box); the
+//          per-image workgroup only thresholds and appends.
 // Phase 2  candidates are ordered by (score descending, box index ascending)
 //          with an in-place bitonic sort of 64-bit keys in the workspace.
 // Phase 3  greedy suppression in sorted order: the workgroup walks the list;
@@ -48,16 +51,34 @@ __device__ __forceinline__ float iou_of(const Box4& a, const Box4& b) {
   return inter / (area_a + area_b - inter);
 }
 
+// best[n][b] = max over classes (first maximum), cls[n][b] = its class
+__global__ void __launch_bounds__(256)
+nms_best_class_kernel(const float* __restrict__ scores, int C, int B, float* __restrict__ best_ws,
+                      int32_t* __restrict__ cls_ws) {
+  const int n = blockIdx.y;
+  const int b = blockIdx.x * 256 + threadIdx.x;
+  if (b >= B) return;
+  const float* sc = scores + (int64_t)n * C * B + b;
+  float best = sc[0];
+  int bc = 0;
+  for (int c = 1; c < C; ++c) {
+    const float v = sc[(int64_t)c * B];
+    if (v > best) { best = v; bc = c; }
+  }
+  best_ws[(int64_t)n * B + b] = best;
+  cls_ws[(int64_t)n * B + b] = bc;
+}
+
 __global__ void __launch_bounds__(kNmsThreads)
-nms_kernel(const float* __restrict__ boxes, const float* __restrict__ scores, int C, int B,
+nms_kernel(const float* __restrict__ boxes, const float* __restrict__ best_ws, int B,
            int max_out, float iou_thr, float score_thr, int32_t* __restrict__ out,
-           unsigned long long* keys_ws, int32_t* cls_ws, unsigned char* sup_ws, int64_t bpad) {
+           unsigned long long* keys_ws, const int32_t* cls_ws, unsigned char* sup_ws, int64_t bpad) {
   const int n = blockIdx.x;
   const int tid = threadIdx.x;
   const float* bx = boxes + (int64_t)n * B * 4;
-  const float* sc = scores + (int64_t)n * C * B;
+  const float* bestv = best_ws + (int64_t)n * B;
   unsigned long long* keys = keys_ws + (int64_t)n * bpad;
-  int32_t* cls = cls_ws + (int64_t)n * B;
+  const int32_t* cls = cls_ws + (int64_t)n * B;
   unsigned char* sup = sup_ws + (int64_t)n * bpad;
   int32_t* o = out + (int64_t)n * max_out * 3;
 
@@ -67,20 +88,14 @@ nms_kernel(const float* __restrict__ boxes, const float* __restrict__ scores, in
   for (int i = tid; i < max_out * 3; i += kNmsThreads) o[i] = -1;
   __syncthreads();
 
-  // ---- phase 1: best class per box, threshold, append ----
+  // ---- phase 1 (second half): threshold, append ----
   for (int b = tid; b < B; b += kNmsThreads) {
-    float best = sc[b];
-    int bc = 0;
-    for (int c = 1; c < C; ++c) {
-      const float v = sc[(int64_t)c * B + b];
-      if (v > best) { best = v; bc = c; }
-    }
+    const float best = bestv[b];
     if (best > score_thr) {
       const int slot = atomicAdd(&s_count, 1);
       unsigned u = __float_as_uint(best);
       u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // ascending in u == ascending in value
       keys[slot] = ((unsigned long long)(~u) << 32) | (unsigned)b;  // score desc, then box asc
-      cls[b] = bc;
     }
   }
   __syncthreads();
@@ -137,9 +152,9 @@ nms_kernel(const float* __restrict__ boxes, const float* __restrict__ scores, in
 
 size_t nms_workspace_bytes(int N, int B) {
   const int64_t bpad = next_pow2(B);
-  // keys (8 B) + suppression flags (1 B) per padded slot, class per box (4 B)
+  // keys (8 B) + suppression flags (1 B) per padded slot, class and best score per box (4 B each)
   size_t bytes = (size_t)N * bpad * 8;
-  bytes += (size_t)N * B * 4;
+  bytes += (size_t)N * B * 4 * 2;
   bytes += (size_t)N * bpad;
   return (bytes + 255) & ~(size_t)255;
 }
@@ -154,8 +169,12 @@ hipError_t launch_nms(const float* boxes, const float* scores, int N, int C, int
   if (bpad > (1 << 24)) return hipErrorInvalidValue;
   unsigned long long* keys = reinterpret_cast<unsigned long long*>(workspace);
   int32_t* cls = reinterpret_cast<int32_t*>(keys + (int64_t)N * bpad);
-  unsigned char* sup = reinterpret_cast<unsigned char*>(cls + (int64_t)N * B);
-  hipLaunchKernelGGL(nms_kernel, dim3(N), dim3(kNmsThreads), 0, stream, boxes, scores, C, B, max_out,
+  float* best = reinterpret_cast<float*>(cls + (int64_t)N * B);
+  unsigned char* sup = reinterpret_cast<unsigned char*>(best + (int64_t)N * B);
+  if (N > 65535) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(nms_best_class_kernel, dim3((unsigned)((B + 255) / 256), (unsigned)N), dim3(256), 0, stream,
+                     scores, C, B, best, cls);
+  hipLaunchKernelGGL(nms_kernel, dim3(N), dim3(kNmsThreads), 0, stream, boxes, best, B, max_out,
                      iou_thr, score_thr, out, keys, cls, sup, bpad);
   return hipGetLastError();
 }
