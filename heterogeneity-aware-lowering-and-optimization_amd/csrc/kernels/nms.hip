@@ -72,7 +72,8 @@ nms_best_class_kernel(const float* __restrict__ scores, int C, int B, float* __r
 __global__ void __launch_bounds__(kNmsThreads)
 nms_kernel(const float* __restrict__ boxes, const float* __restrict__ best_ws, int B,
            int max_out, float iou_thr, float score_thr, int32_t* __restrict__ out,
-           unsigned long long* keys_ws, const int32_t* cls_ws, unsigned char* sup_ws, int64_t bpad) {
+           unsigned long long* keys_ws, const int32_t* cls_ws, unsigned char* sup_ws, int64_t bpad,
+           int lds_slots) {
   const int n = blockIdx.x;
   const int tid = threadIdx.x;
   const float* bx = boxes + (int64_t)n * B * 4;
@@ -83,8 +84,7 @@ nms_kernel(const float* __restrict__ boxes, const float* __restrict__ best_ws, i
   int32_t* o = out + (int64_t)n * max_out * 3;
 
   __shared__ int s_count;
-  __shared__ int s_kept;
-  if (tid == 0) { s_count = 0; s_kept = 0; }
+  if (tid == 0) s_count = 0;
   for (int i = tid; i < max_out * 3; i += kNmsThreads) o[i] = -1;
   __syncthreads();
 
@@ -106,25 +106,55 @@ nms_kernel(const float* __restrict__ boxes, const float* __restrict__ best_ws, i
   for (int i = tid; i < M; i += kNmsThreads) sup[i] = 0;
   __syncthreads();
 
-  // ---- phase 2: bitonic sort of keys[0..P) ascending ----
+  // ---- phase 2: bitonic sort of keys[0..P) ascending; in LDS when the list fits ----
+  extern __shared__ unsigned long long lds_keys[];
+  unsigned long long* sk = P <= lds_slots ? lds_keys : keys;
+  if (sk != keys) {
+    for (int i = tid; i < P; i += kNmsThreads) sk[i] = keys[i];
+    __syncthreads();
+  }
   for (int k = 2; k <= P; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
       for (int i = tid; i < P; i += kNmsThreads) {
         const int l = i ^ j;
         if (l > i) {
-          const unsigned long long a = keys[i], b = keys[l];
+          const unsigned long long a = sk[i], b = sk[l];
           const bool up = (i & k) == 0;
-          if ((a > b) == up) { keys[i] = b; keys[l] = a; }
+          if ((a > b) == up) { sk[i] = b; sk[l] = a; }
         }
       }
       __syncthreads();
     }
   }
+  // With the list in LDS the sorted keys go back to memory and the candidates'
+  // boxes and suppression flags take their place: the walk below is a chain of
+  // short rounds, each as long as its slowest read.
+  const bool in_lds = sk != keys;
+  Box4* lbox = reinterpret_cast<Box4*>(lds_keys);
+  unsigned char* lsup = reinterpret_cast<unsigned char*>(lbox + lds_slots);
+  if (in_lds) {
+    for (int i = tid; i < M; i += kNmsThreads) keys[i] = sk[i];
+    __syncthreads();
+    for (int i = tid; i < M; i += kNmsThreads) {
+      lbox[i] = norm_box(bx + (int64_t)(keys[i] & 0xffffffffu) * 4);
+      lsup[i] = 0;
+    }
+    __syncthreads();
+  }
+  unsigned char* const supf = in_lds ? lsup : sup;
 
   // ---- phase 3: greedy suppression ----
+  int kept = 0;  // every thread counts the kept boxes itself: one barrier per kept box
+  const bool flags8 = (reinterpret_cast<uintptr_t>(supf) & 7u) == 0;
   for (int i = 0; i < M; ++i) {
-    if (sup[i]) continue;           // uniform: written before the last barrier
-    const int kept = s_kept;        // uniform
+    // (uniform: the flags were written before the last barrier.)  Runs of
+    // suppressed candidates are skipped eight flags per read: the walk is a chain
+    // of dependent reads, one per step.
+    if (flags8 && (i & 7) == 0) {
+      while (i + 8 <= M && *reinterpret_cast<const unsigned long long*>(supf + i) == 0x0101010101010101ull) i += 8;
+      if (i >= M) break;
+    }
+    if (supf[i]) continue;
     if (kept >= max_out) break;
     const int bi = (int)(keys[i] & 0xffffffffu);
     if (tid == 0) {
@@ -132,18 +162,16 @@ nms_kernel(const float* __restrict__ boxes, const float* __restrict__ best_ws, i
       o[kept * 3 + 1] = cls[bi];
       o[kept * 3 + 2] = bi;
     }
-    const Box4 a = norm_box(bx + (int64_t)bi * 4);
+    const Box4 a = in_lds ? lbox[i] : norm_box(bx + (int64_t)bi * 4);
     for (int j = i + 1 + tid; j < M; j += kNmsThreads) {
-      if (!sup[j]) {
-        const int bj = (int)(keys[j] & 0xffffffffu);
-        const Box4 b = norm_box(bx + (int64_t)bj * 4);
+      if (!supf[j]) {
+        const Box4 b = in_lds ? lbox[j] : norm_box(bx + (int64_t)(keys[j] & 0xffffffffu) * 4);
         // candidate j plays the role of "I", the kept box of "J" in the
         // reference formula; the expression is symmetric in fp32.
-        if (iou_of(b, a) >= iou_thr) sup[j] = 1;
+        if (iou_of(b, a) >= iou_thr) supf[j] = 1;
       }
     }
-    __syncthreads();
-    if (tid == 0) s_kept = kept + 1;
+    ++kept;
     __syncthreads();
   }
 }
@@ -174,8 +202,19 @@ hipError_t launch_nms(const float* boxes, const float* scores, int N, int C, int
   if (N > 65535) return hipErrorInvalidValue;
   hipLaunchKernelGGL(nms_best_class_kernel, dim3((unsigned)((B + 255) / 256), (unsigned)N), dim3(256), 0, stream,
                      scores, C, B, best, cls);
-  hipLaunchKernelGGL(nms_kernel, dim3(N), dim3(kNmsThreads), 0, stream, boxes, best, B, max_out,
-                     iou_thr, score_thr, out, keys, cls, sup, bpad);
+  // candidate list in LDS - first the keys (8 B per slot), then boxes and flags in
+  // their place (16 + 1 B per slot): up to 8192 candidates per image
+  const int lds_slots = (int)(bpad < 8192 ? bpad : 8192);
+  const size_t lds_bytes = (size_t)lds_slots * 17;
+  static bool lds_limit_raised = false;  // (benign if two threads both do it)
+  if (!lds_limit_raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(nms_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            8192 * 17) != hipSuccess)
+      return hipErrorInvalidValue;
+    lds_limit_raised = true;
+  }
+  hipLaunchKernelGGL(nms_kernel, dim3(N), dim3(kNmsThreads), lds_bytes, stream, boxes, best, B, max_out,
+                     iou_thr, score_thr, out, keys, cls, sup, bpad, lds_slots);
   return hipGetLastError();
 }
 
