@@ -11,13 +11,16 @@ to the reference tree.  Heavy loops live in ``odla_ref.c`` (built to
 ``libodla_ref.so`` by ``oracle/Makefile``).
 
 Pin status (what fixes each function independently of this file):
-  conv2d / gemm / pools / softmax / batchnorm   reference-held known-answer
-      vectors (odla_popart/test), the reference's own fp32 kernels built to
-      ``oracle/_ref/libsn_rt.so``, float64 brute force.
+  conv2d / gemm (plain and batched) / pools / softmax / batchnorm
+      reference-held known-answer vectors (odla_popart/test), the reference's
+      own fp32 kernels built to ``oracle/_ref/libsn_rt.so``, float64 brute force.
+  reduce_mean / argmax (first maximum) / slice / gather / transpose / pad /
+      erf / add, sub, mul, div with broadcasting   vectors of the same
+      reference kernels (runtime/generic/*.cc) held in tests/golden.
   quantize / dequantize   ONNX QuantizeLinear published example (passes on the
       reference CPU backend), exhaustive half-integer rounding check.
-  layernorm / gelu / erf / resize / concat / transpose / gather   closed forms
-      and library routines (math.erf, numpy).
+  layernorm / gelu / resize / concat   closed forms and library routines
+      (math.erf, numpy).
   nms   ONNX NonMaxSuppression published examples, O(n^2) brute force.
   wider operator surface (trigonometric / hyperbolic functions, Elu family,
       comparisons, Select, Mod, reductions, ArgMax, TopK, Pad, Tile, LRN,

@@ -64,6 +64,141 @@ def gemm(a, b, c, ta, tb, alpha, beta):
     return y
 
 
+i32p = ctypes.POINTER(ctypes.c_int32)
+i64p = ctypes.POINTER(ctypes.c_int64)
+
+
+def shape64(shape):
+    return (ctypes.c_int64 * len(shape))(*shape)
+
+
+def batchnorm_nchw(x, mean, var, offset, scale, eps):
+    N, C, H, W = x.shape
+    y = np.zeros_like(x)
+    LIB._sn_rt_bn_f32_nchw.argtypes = [f32p] * 6 + [i64] * 4 + [ctypes.c_bool, ctypes.c_bool, ctypes.c_float, ctypes.c_float]
+    LIB._sn_rt_bn_f32_nchw(fp(y), fp(x), fp(mean), fp(var), fp(offset), fp(scale), N, H, W, C, False, False, eps, 1.0)
+    return y
+
+
+def batch_matmul(a, b, ta, tb):
+    batches = a.shape[0]
+    M = a.shape[2] if ta else a.shape[1]
+    N = b.shape[1] if tb else b.shape[2]
+    y = np.zeros((batches, M, N), np.float32)
+    LIB._sn_rt_batch_matmul_f32.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [ctypes.c_bool, ctypes.c_bool]
+    LIB._sn_rt_batch_matmul_f32(fp(y), fp(a), fp(b), batches, a.shape[1], a.shape[2], b.shape[1], b.shape[2], ta, tb)
+    return y
+
+
+def reduce_mean(x, axes):
+    out_shape = [1 if i in axes else d for i, d in enumerate(x.shape)]
+    y = np.zeros(out_shape, np.float32)
+    ax = (ctypes.c_int32 * len(axes))(*axes)
+    LIB._sn_rt_reduce_mean_f32.argtypes = [f32p, f32p, i64p, i32p, i64, ctypes.c_int32, ctypes.c_int32]
+    LIB._sn_rt_reduce_mean_f32(fp(y), fp(x), shape64(x.shape), ax, x.size, x.ndim, len(axes))
+    return y
+
+
+def argmax(x, axis):
+    out_shape = [d for i, d in enumerate(x.shape) if i != axis % x.ndim]
+    y = np.zeros(out_shape, np.int64)
+    ax = (ctypes.c_int32 * 1)(axis)
+    LIB._sn_rt_argmax_f32.argtypes = [i64p, f32p, i64p, i32p, i64, ctypes.c_int32, ctypes.c_int32]
+    LIB._sn_rt_argmax_f32(y.ctypes.data_as(i64p), fp(x), shape64(x.shape), ax, x.size, x.ndim, 1)
+    return y
+
+
+def slice_(x, starts, sizes):
+    y = np.zeros(sizes, np.float32)
+    st = (ctypes.c_int * len(starts))(*starts)
+    sz = (ctypes.c_int * len(sizes))(*sizes)
+    LIB._sn_rt_slice_f32.argtypes = [f32p, f32p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int), i64p, ctypes.c_int]
+    LIB._sn_rt_slice_f32(fp(y), fp(x), st, sz, shape64(x.shape), x.ndim)
+    return y
+
+
+def gather_rows(table, idx):
+    y = np.zeros((idx.size, table.shape[1]), np.float32)
+    ii = np.ascontiguousarray(idx, np.int32)
+    LIB._sn_rt_gather_f32.argtypes = [f32p, f32p, ctypes.POINTER(ctypes.c_int), i64, i64]
+    LIB._sn_rt_gather_f32(fp(y), fp(table), ii.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), table.shape[1], idx.size)
+    return y
+
+
+def transpose(x, perm):
+    y = np.zeros([x.shape[p] for p in perm], np.float32)
+    pm = (ctypes.c_int * len(perm))(*perm)
+    LIB._sn_rt_transpose_f32.argtypes = [f32p, f32p, ctypes.POINTER(ctypes.c_int), i64p, ctypes.c_int]
+    LIB._sn_rt_transpose_f32(fp(y), fp(x), pm, shape64(x.shape), x.ndim)
+    return y
+
+
+def erf(x):
+    y = np.zeros_like(x)
+    LIB._sn_rt_erf_f32.argtypes = [f32p, f32p, i64]
+    LIB._sn_rt_erf_f32(fp(y), fp(x), x.size)
+    return y
+
+
+def binary(name, a, b):
+    """add / sub / mul / div with the reference's broadcast (shapes of equal rank)."""
+    out_shape = tuple(max(p, q) for p, q in zip(a.shape, b.shape))
+    y = np.zeros(out_shape, np.float32)
+    fn = getattr(LIB, "_sn_rt_%s_f32" % name)
+    fn.argtypes = [f32p, f32p, f32p, i64, ctypes.c_bool, i64p, i64p, i64p, ctypes.c_int32]
+    fn(fp(y), fp(a), fp(b), y.size, a.shape != b.shape, shape64(out_shape), shape64(a.shape), shape64(b.shape), len(out_shape))
+    return y
+
+
+def pad_hw_nhwc(x, top, bottom, left, right):
+    N, H, W, C = x.shape
+    y = np.full((N, H + top + bottom, W + left + right, C), np.nan, np.float32)
+    pads = (ctypes.c_int32 * 8)(0, 0, top, bottom, left, right, 0, 0)
+    LIB._sn_rt_pad_f32.argtypes = [f32p, f32p, ctypes.c_int, i64p, i32p]
+    LIB._sn_rt_pad_f32(fp(y), fp(x), 4, shape64(x.shape), pads)
+    return y
+
+
+def more(rng, out):
+    x = rng.standard_normal((2, 5, 4, 3)).astype(np.float32)
+    mean, var = rng.standard_normal(5).astype(np.float32), (rng.random(5) + 0.5).astype(np.float32)
+    offset, scale = rng.standard_normal(5).astype(np.float32), rng.standard_normal(5).astype(np.float32)
+    out["bn_x"], out["bn_mean"], out["bn_var"], out["bn_offset"], out["bn_scale"] = x, mean, var, offset, scale
+    out["bn_y"] = batchnorm_nchw(x, mean, var, offset, scale, 1e-3)
+    for i, (ta, tb) in enumerate([(False, False), (False, True), (True, False)]):
+        a = rng.standard_normal((3, 6, 4) if ta else (3, 4, 6)).astype(np.float32)
+        b = rng.standard_normal((3, 5, 6) if tb else (3, 6, 5)).astype(np.float32)
+        out["bmm%d_a" % i], out["bmm%d_b" % i] = a, b
+        out["bmm%d_attr" % i] = np.array([ta, tb], np.int64)
+        out["bmm%d_y" % i] = batch_matmul(a, b, ta, tb)
+    x = rng.standard_normal((2, 3, 5, 4)).astype(np.float32)
+    out["reduce_x"] = x
+    for i, axes in enumerate([(1,), (3,), (2, 3), (0, 2)]):
+        out["reduce%d_axes" % i] = np.array(axes, np.int64)
+        out["reduce%d_y" % i] = reduce_mean(x, list(axes))
+    for i, axis in enumerate([0, 2, -1]):
+        out["argmax%d_axis" % i] = np.array([axis], np.int64)
+        out["argmax%d_y" % i] = argmax(x, axis)
+    out["slice_starts"], out["slice_sizes"] = np.array([1, 0, 2, 1], np.int64), np.array([1, 2, 3, 2], np.int64)
+    out["slice_y"] = slice_(x, [1, 0, 2, 1], [1, 2, 3, 2])
+    table = rng.standard_normal((9, 6)).astype(np.float32)
+    idx = np.array([[3, 0, 8], [8, 8, 1]], np.int32)
+    out["gather_table"], out["gather_idx"], out["gather_y"] = table, idx, gather_rows(table, idx)
+    for i, perm in enumerate([(0, 2, 3, 1), (3, 1, 0, 2), (1, 0, 2, 3)]):
+        out["transpose%d_perm" % i] = np.array(perm, np.int64)
+        out["transpose%d_y" % i] = transpose(x, perm)
+    e = (rng.standard_normal(64) * 2).astype(np.float32)
+    out["erf_x"], out["erf_y"] = e, erf(e)
+    a = rng.standard_normal((2, 3, 1, 4)).astype(np.float32)
+    b = (rng.standard_normal((1, 3, 5, 1)) + 3).astype(np.float32)
+    out["bin_a"], out["bin_b"] = a, b
+    for name in ("add", "sub", "mul", "div"):
+        out["bin_%s_y" % name] = binary(name, a, b)
+    p = rng.standard_normal((2, 3, 4, 5)).astype(np.float32)     # NHWC
+    out["pad_x"], out["pad_attr"] = p, np.array([1, 2, 0, 3], np.int64)
+    out["pad_y"] = pad_hw_nhwc(p, 1, 2, 0, 3)
+
+
 def main():
     rng = np.random.default_rng(20240)
     out = {}
@@ -95,6 +230,7 @@ def main():
         out["gemm%d_a" % i], out["gemm%d_b" % i], out["gemm%d_c" % i] = a, b, c
         out["gemm%d_attr" % i] = np.array([ta, tb, alpha, beta], np.float64)
         out["gemm%d_y" % i] = gemm(a, b, c, ta, tb, alpha, beta)
+    more(np.random.default_rng(20241), out)
     np.savez(os.path.join(HERE, "sn_rt_vectors.npz"), **out)
     print("wrote %d arrays" % len(out))
 

@@ -347,6 +347,80 @@ def test_nms_against_brute_force(ref):
 
 
 # -------------------------------------------------------- live reference ----
+# ------------------------------------ more of the reference's own fp32 kernels ----
+def test_batchnorm_against_reference_kernel_vectors(ref):
+    rb = ref.RefBuilder({})
+    y = rb.batchnorm(GOLD["bn_x"], GOLD["bn_mean"], GOLD["bn_var"], 1e-3, GOLD["bn_scale"], GOLD["bn_offset"])
+    want = GOLD["bn_y"]
+    assert np.max(np.abs(y - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("i", range(3))
+def test_batched_gemm_against_reference_kernel_vectors(ref, i):
+    ta, tb = GOLD["bmm%d_attr" % i]
+    rb = ref.RefBuilder({})
+    y = rb.gemm(GOLD["bmm%d_a" % i], GOLD["bmm%d_b" % i], None, bool(ta), bool(tb), 1.0, 0.0)
+    want = GOLD["bmm%d_y" % i]
+    assert y.shape == want.shape
+    assert np.max(np.abs(y - want)) <= 1e-5 * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("i", range(4))
+def test_reduce_mean_against_reference_kernel_vectors(ref, i):
+    rb = ref.RefBuilder({})
+    y = rb.reduce_mean(GOLD["reduce_x"], [int(a) for a in GOLD["reduce%d_axes" % i]], keep_dims=True)
+    want = GOLD["reduce%d_y" % i]
+    assert y.shape == want.shape
+    assert np.max(np.abs(y - want)) <= 1e-6
+
+
+@pytest.mark.parametrize("i", range(3))
+def test_argmax_against_reference_kernel_vectors(ref, i):
+    rb = ref.RefBuilder({})
+    x = GOLD["reduce_x"]
+    y = rb.argmax(x, int(GOLD["argmax%d_axis" % i][0]) % x.ndim, keep_dims=False, dtype=np.int64)
+    assert np.array_equal(y, GOLD["argmax%d_y" % i])
+
+
+def test_argmax_first_of_equal_values_like_the_reference_kernel(ref):
+    # runtime/generic/reduction.cc of the reference tree keeps the first maximum
+    # (strict comparison while walking the axis upwards)
+    rb = ref.RefBuilder({})
+    x = np.array([[1, 3, 3, 0], [2, 2, 2, 2]], np.float32)
+    assert rb.argmax(x, 1, keep_dims=False).tolist() == [1, 0]
+    assert rb.argmax(x, 1, keep_dims=False, last=True).tolist() == [2, 3]
+
+
+def test_data_movement_against_reference_kernel_vectors(ref):
+    rb = ref.RefBuilder({})
+    x = GOLD["reduce_x"]
+    st, sz = GOLD["slice_starts"], GOLD["slice_sizes"]
+    assert np.array_equal(rb.slice(x, [int(v) for v in st], [int(a + b) for a, b in zip(st, sz)]), GOLD["slice_y"])
+    idx = GOLD["gather_idx"]
+    got = rb.gather(GOLD["gather_table"], idx, axis=0)
+    assert got.shape == idx.shape + (GOLD["gather_table"].shape[1],)
+    assert np.array_equal(got.reshape(idx.size, -1), GOLD["gather_y"])
+    for i in range(3):
+        assert np.array_equal(rb.transpose(x, [int(p) for p in GOLD["transpose%d_perm" % i]]), GOLD["transpose%d_y" % i])
+    top, bottom, left, right = (int(v) for v in GOLD["pad_attr"])
+    # the reference kernel pads H and W of a channels-last tensor
+    assert np.array_equal(rb.pad(GOLD["pad_x"], [0, top, left, 0], [0, bottom, right, 0]), GOLD["pad_y"])
+
+
+def test_erf_against_reference_kernel_vectors(ref):
+    rb = ref.RefBuilder({})
+    assert np.max(np.abs(rb.erf(GOLD["erf_x"]) - GOLD["erf_y"])) <= 2e-7
+
+
+@pytest.mark.parametrize("name", ["add", "sub", "mul", "div"])
+def test_broadcast_arithmetic_against_reference_kernel_vectors(ref, name):
+    rb = ref.RefBuilder({})
+    y = getattr(rb, name)(GOLD["bin_a"], GOLD["bin_b"])
+    want = GOLD["bin_%s_y" % name]
+    assert y.shape == want.shape == (2, 3, 5, 4)
+    assert np.max(np.abs(y - want)) <= 1e-6 * np.max(np.abs(want))
+
+
 def test_live_reference_kernels_if_built(ref):
     """When oracle/_ref/libsn_rt.so exists (built from the reference tree), one more
     conv shape is compared live; otherwise the committed vectors above stand in."""
