@@ -202,6 +202,53 @@ odla_status stage_inputs(_odla_context* ctx, const Plan& plan) {
   return ODLA_SUCCESS;
 }
 
+odla_status create_context_for(_odla_computation* c, odla_context* context);
+
+// The context that executes `ctx`'s computation at batch `bs`: `ctx` itself at
+// the recorded batch, otherwise a context over a rescaled copy of the recording
+// (made, planned and given an arena on first use).
+odla_status variant_context(_odla_context* ctx, int bs, _odla_context** out) {
+  _odla_computation* c = ctx->comp;
+  const int rec = recorded_batch(*c);
+  if (bs == 0 || bs == rec) { *out = ctx; return ODLA_SUCCESS; }
+  auto have = ctx->variant_ctx.find(bs);
+  if (have != ctx->variant_ctx.end()) { *out = have->second; return ODLA_SUCCESS; }
+  _odla_computation* v = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(c->mu);
+    auto it = c->variants.find(bs);
+    if (it == c->variants.end()) {
+      std::unique_ptr<_odla_computation> copy = clone_for_batch(*c, rec, bs);
+      if (!copy) return ODLA_UNSUPPORTED_OP;
+      it = c->variants.emplace(bs, std::move(copy)).first;
+    }
+    v = it->second.get();
+  }
+  odla_context sub = nullptr;
+  odla_status st = create_context_for(v, &sub);
+  if (st != ODLA_SUCCESS) return st;
+  ctx->variant_ctx[bs] = sub;
+  *out = sub;
+  return ODLA_SUCCESS;
+}
+
+odla_status set_run_batch(_odla_context* ctx, int bs) {
+  const int rec = recorded_batch(*ctx->comp);
+  if (rec == 0) {
+    OHIP_ERR("ODLA_RUN_BATCH_SIZE: the computation was not recorded with ODLA_DYNAMIC_BATCH and ODLA_MAX_BATCH_SIZE");
+    return ODLA_FAILURE;
+  }
+  if (bs < 1 || bs > rec) {
+    OHIP_ERR("ODLA_RUN_BATCH_SIZE: %d is outside 1..%d", bs, rec);
+    return ODLA_FAILURE;
+  }
+  _odla_context* sub = nullptr;
+  odla_status st = variant_context(ctx, bs, &sub);  // compiled here, so that a graph that cannot be rescaled fails early
+  if (st != ODLA_SUCCESS) return st;
+  ctx->run_batch = bs;
+  return ODLA_SUCCESS;
+}
+
 _odla_value* find_value(_odla_computation* c, const odla_value_id id) {
   if (c == nullptr || id == nullptr) return nullptr;
   auto it = c->by_name.find(reinterpret_cast<const char*>(id));
@@ -264,6 +311,23 @@ odla_status odla_SetComputationItem(odla_computation c, odla_item_type type, odl
       else return ODLA_UNSUPPORTED_DATATYPE;
       return ODLA_SUCCESS;
     }
+    case ODLA_DYNAMIC_BATCH:
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      c->dynamic_batch = *reinterpret_cast<const bool*>(value);
+      return ODLA_SUCCESS;
+    case ODLA_MIN_BATCH_SIZE:
+    case ODLA_MAX_BATCH_SIZE:
+    case ODLA_OPT_BATCH_SIZE: {
+      if (value == nullptr) return ODLA_INVALID_PARAM;
+      const int n = *reinterpret_cast<const int*>(value);
+      if (n < 1) return ODLA_INVALID_PARAM;
+      if ((int)type == ODLA_MAX_BATCH_SIZE && !c->args.empty() && n != c->max_batch) {
+        OHIP_ERR("odla_SetComputationItem: the largest batch must be set before the first argument is created");
+        return ODLA_FAILURE;
+      }
+      ((int)type == ODLA_MIN_BATCH_SIZE ? c->min_batch : (int)type == ODLA_MAX_BATCH_SIZE ? c->max_batch : c->opt_batch) = n;
+      return ODLA_SUCCESS;
+    }
     case ODLA_QUANT_TABLE:
       c->opts.qtable = reinterpret_cast<const odla_value_quant_info*>(value);
       return ODLA_SUCCESS;
@@ -282,8 +346,6 @@ odla_status odla_SetComputationItem(odla_computation c, odla_item_type type, odl
 }
 
 // ---------------------------------------------------------------- context --
-static odla_status create_context_for(_odla_computation* c, odla_context* context);
-
 odla_status odla_CreateContext(odla_context* context) {
   if (context == nullptr) return ODLA_INVALID_PARAM;
   _odla_computation* c = current_computation();
@@ -299,7 +361,9 @@ odla_status odla_CreateContext(odla_context* context) {
   return st;
 }
 
-static odla_status create_context_for(_odla_computation* c, odla_context* context) {
+}  // extern "C"
+namespace {
+odla_status create_context_for(_odla_computation* c, odla_context* context) {
   odla_status st = ensure_plan(c);
   if (st != ODLA_SUCCESS) return st;
   auto ctx = std::make_unique<_odla_context>();
@@ -320,8 +384,12 @@ static odla_status create_context_for(_odla_computation* c, odla_context* contex
   *context = ctx.release();
   return ODLA_SUCCESS;
 }
+}  // namespace
+extern "C" {
 
 static void destroy_context(odla_context ctx) {
+  for (auto& kv : ctx->variant_ctx) destroy_context(kv.second);
+  ctx->variant_ctx.clear();
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   drop_graph(ctx);
   if (ctx->arena) (void)hipFree(ctx->arena);
@@ -347,8 +415,45 @@ odla_status odla_SetContextItem(odla_context ctx, odla_item_type type, odla_item
     if (!ctx->use_graph) drop_graph(ctx);
     return ODLA_SUCCESS;
   }
+  if (type == ODLA_RUN_BATCH_SIZE) {
+    if (value == nullptr) return ODLA_INVALID_PARAM;
+    return set_run_batch(ctx, *reinterpret_cast<const int*>(value));
+  }
   OHIP_DEBUG("odla_SetContextItem: item %d accepted and ignored", (int)type);
   return ODLA_SUCCESS;
+}
+
+odla_status odla_SetRuntimeShape(odla_context ctx, odla_value value, odla_value_shape shape) {
+  if (ctx == nullptr || value == nullptr) return ODLA_INVALID_PARAM;
+  // only arguments, as in the reference [ref: odla_tensorrt.cc:251-258]
+  if (value->kind != _odla_value::ARG || value->comp != ctx->comp) return ODLA_FAILURE;
+  const Shape want = shape_from(shape);
+  if (want.rank != value->shape.rank || want.d[0] < 1) return ODLA_INVALID_PARAM;
+  for (int i = 1; i < want.rank; ++i) {
+    if (want.d[i] != value->shape.d[i]) {
+      OHIP_ERR("odla_SetRuntimeShape: only the leading extent of '%s' %s may change at run time (asked for %s)",
+               value->name.c_str(), value->shape.str().c_str(), want.str().c_str());
+      return ODLA_UNSUPPORTED_OP;
+    }
+  }
+  const int rec = recorded_batch(*ctx->comp);
+  if (rec == 0 || value->shape.d[0] != rec) {
+    if (want.d[0] == value->shape.d[0]) return ODLA_SUCCESS;
+    OHIP_ERR("odla_SetRuntimeShape: '%s' was not recorded with a dynamic batch", value->name.c_str());
+    return ODLA_UNSUPPORTED_OP;
+  }
+  return set_run_batch(ctx, (int)want.d[0]);
+}
+
+odla_status odla_SetRuntimeValueType(odla_context ctx, odla_value value, odla_value_type type) {
+  if (value != nullptr && type.element_type != value->etype) return ODLA_UNSUPPORTED_DATATYPE;
+  return odla_SetRuntimeShape(ctx, value, type.shape);
+}
+
+odla_status odla_GetRuntimeValueType(odla_context ctx, odla_value value, odla_value_type* type) {
+  if (value == nullptr || type == nullptr) return ODLA_INVALID_PARAM;
+  type->element_type = value->etype;
+  return odla_GetRuntimeShape(ctx, value, &type->shape);
 }
 
 odla_status odla_BindToArgument(odla_value value, const odla_void* data_ptr, odla_context ctx) {
@@ -401,6 +506,23 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
   }
   if (mode == ODLA_COMPUTE_TRAINING) return ODLA_UNSUPPORTED_OP;
   _odla_computation* c = ctx->comp;
+  if (ctx->run_batch > 0 && ctx->run_batch != recorded_batch(*c)) {
+    // another batch than the recorded one: the same bindings, on the copy planned for that batch
+    _odla_context* sub = nullptr;
+    odla_status st = variant_context(ctx, ctx->run_batch, &sub);
+    if (st != ODLA_SUCCESS) return st;
+    if (sub->use_graph != ctx->use_graph) {
+      sub->use_graph = ctx->use_graph;
+      if (!sub->use_graph) drop_graph(sub);
+    }
+    sub->bound_in.clear();
+    sub->bound_out.clear();
+    for (const auto& kv : ctx->bound_in) sub->bound_in[sub->comp->values[kv.first->index].get()] = kv.second;
+    for (const auto& kv : ctx->bound_out) sub->bound_out[sub->comp->values[kv.first->index].get()] = kv.second;
+    st = odla_ExecuteComputation(sub->comp, sub, mode, device);
+    ctx->executed = st == ODLA_SUCCESS;
+    return st;
+  }
   if (!c->plan) return ODLA_FAILURE;
   const Plan& plan = *c->plan;
 
@@ -531,9 +653,13 @@ odla_status odla_GetOutputFromComputationByIdx(const odla_computation c, const o
   return ODLA_SUCCESS;
 }
 odla_status odla_GetRuntimeShape(odla_context ctx, odla_value value, odla_value_shape* shape) {
-  (void)ctx;
   if (value == nullptr || shape == nullptr) return ODLA_INVALID_PARAM;
   *shape = shape_to(value->shape);
+  if (ctx != nullptr && value->comp == ctx->comp && ctx->run_batch > 0) {
+    // the value's shape at the batch this context runs at
+    auto it = ctx->variant_ctx.find(ctx->run_batch);
+    if (it != ctx->variant_ctx.end()) *shape = shape_to(it->second->comp->values[value->index]->shape);
+  }
   return ODLA_SUCCESS;
 }
 
@@ -656,6 +782,11 @@ odla_status odla_GetValueDataById(const odla_value_id id, odla_void* data_ptr) {
 odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr, odla_context ctx) {
   if (value == nullptr || data_ptr == nullptr) return ODLA_INVALID_PARAM;
   if (ctx == nullptr) return eager_evaluate(value, data_ptr);
+  if (ctx->run_batch > 0 && value->comp == ctx->comp) {
+    auto it = ctx->variant_ctx.find(ctx->run_batch);
+    if (it != ctx->variant_ctx.end())
+      return odla_GetValueData(it->second->comp->values[value->index].get(), data_ptr, it->second);
+  }
   if (!ctx->executed || !ctx->comp->plan) return ODLA_FAILURE;
   const Plan& plan = *ctx->comp->plan;
   for (const Plan::IO& io : plan.outputs) {
@@ -679,10 +810,21 @@ odla_value odla_CreateArgument(const odla_value_type type, const odla_value_id i
   }
   if (type.shape.size > ODLA_MAX_DIMENSION) { OHIP_ERR("odla_CreateArgument: rank too large"); return nullptr; }
   Shape s = shape_from(type.shape);
+  bool dyn = false;
+  if (s.d[0] < 0) {
+    // the batch of a computation recorded with ODLA_DYNAMIC_BATCH: planned at the largest batch
+    if (recorded_batch(*c) == 0) {
+      OHIP_ERR("odla_CreateArgument: a negative leading extent needs ODLA_DYNAMIC_BATCH and ODLA_MAX_BATCH_SIZE set before");
+      return nullptr;
+    }
+    s.d[0] = recorded_batch(*c);
+    dyn = true;
+  }
   for (int i = 0; i < s.rank; ++i)
-    if (s.d[i] <= 0) { OHIP_ERR("odla_CreateArgument: dynamic or empty dimensions are not supported (%s)", s.str().c_str()); return nullptr; }
+    if (s.d[i] <= 0) { OHIP_ERR("odla_CreateArgument: only the leading extent may be dynamic (%s)", s.str().c_str()); return nullptr; }
   std::lock_guard<std::mutex> lk(c->mu);
   _odla_value* v = new_value(c, _odla_value::ARG, type.element_type, s, id);
+  v->dyn_batch = dyn;
   c->args.push_back(v);
   return v;
 }

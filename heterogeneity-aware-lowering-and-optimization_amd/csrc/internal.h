@@ -10,6 +10,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <functional>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -76,6 +77,7 @@ struct _odla_value {
   int index = -1;                   // position in computation->values
   int producer = -1;                // node index, -1 for ARG / CONSTANT
   bool is_output = false;
+  bool dyn_batch = false;           // ARG declared with a negative leading extent (the run-time batch)
   bool eager = false;               // created by odla_CreateValue: data comes from odla_SetValueData
   const void* eager_data = nullptr; // borrowed from the caller
   _odla_computation* comp = nullptr;
@@ -222,6 +224,12 @@ struct _odla_computation {
   int live_contexts = 0;             // contexts created by the caller
   _odla_context* eager_ctx = nullptr;  // context behind odla_GetValueData(value, ptr, NULL)
   _odla_executable executable;       // handle given out by odla_CompileComputation / odla_LoadExecutable
+  // dynamic batch [ref: ODLA/platforms/tensorrt/odla_tensorrt.cc:138-179]: arguments are
+  // recorded with max_batch as their leading extent; a context that asks for
+  // another batch runs a copy of the recording whose shapes were rescaled
+  bool dynamic_batch = false;
+  int min_batch = 0, max_batch = 0, opt_batch = 0;
+  std::map<int, std::unique_ptr<_odla_computation>> variants;  // by run-time batch
   // quantisation table of a loaded computation (the caller's table is borrowed otherwise)
   std::vector<odla_value_quant_info> owned_qtable;
   std::vector<std::string> owned_qnames;
@@ -238,6 +246,8 @@ struct _odla_context {
   std::unordered_map<const _odla_value*, const void*> bound_in;
   std::unordered_map<const _odla_value*, void*> bound_out;
   bool executed = false;
+  int run_batch = 0;                              // 0: the recorded shapes
+  std::map<int, _odla_context*> variant_ctx;      // contexts over comp->variants, by batch
 };
 
 struct _odla_device {
@@ -251,6 +261,12 @@ void forget_computation(_odla_computation* c);
 _odla_value* new_value(_odla_computation* c, _odla_value::Kind kind, odla_element_type et,
                        const Shape& shape, const odla_value_id id);
 odla_status compile_computation(_odla_computation* c);  // builds the plan if there is none yet
+// Leading extent the dynamic-batch arguments of `c` were recorded with (0: none).
+int recorded_batch(const _odla_computation& c);
+// A copy of the recording of `c` in which every value that depends on an
+// argument has its leading extent rescaled from `from` to `to`; nullptr (and a
+// log line) when the graph moves the batch out of the leading position.
+std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, int64_t from, int64_t to);
 }  // namespace ohip
 
 #endif

@@ -22,7 +22,7 @@ using namespace ohip;
 
 namespace {
 
-const char kMagic[8] = {'O', 'D', 'L', 'A', 'H', 'I', 'P', '1'};
+const char kMagic[8] = {'O', 'D', 'L', 'A', 'H', 'I', 'P', '2'};
 
 struct Writer {
   std::vector<uint8_t> buf;
@@ -59,6 +59,7 @@ odla_status serialize(_odla_computation* c, std::vector<uint8_t>* out) {
   w.raw(kMagic, 8);
   const Options& o = c->opts;
   w.i64(o.fp16); w.i64((int64_t)o.bf16); w.i64(o.int8); w.i64(o.raw_acc);
+  w.i64(c->dynamic_batch); w.i64(c->min_batch); w.i64(c->max_batch); w.i64(c->opt_batch);
   w.i64(o.qtable != nullptr ? o.qtable_size : 0);
   for (int i = 0; o.qtable != nullptr && i < o.qtable_size; ++i) {
     const odla_value_quant_info& q = o.qtable[i];
@@ -71,7 +72,7 @@ odla_status serialize(_odla_computation* c, std::vector<uint8_t>* out) {
     w.i64((int64_t)v.kind); w.i64((int64_t)v.etype); w.i64(v.shape.rank);
     for (int i = 0; i < v.shape.rank; ++i) w.i64(v.shape.d[i]);
     w.str(v.name);
-    w.i64(v.is_output); w.i64(v.eager); w.i64(v.producer);
+    w.i64(v.is_output); w.i64(v.eager); w.i64(v.producer); w.i64(v.dyn_batch);
     if (v.kind == _odla_value::CONSTANT) {
       const size_t bytes = (size_t)v.shape.numel() * (size_t)odla_type_size(v.etype);
       if (v.host_data == nullptr || bytes == 0) {
@@ -113,6 +114,9 @@ odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) 
   }
   Options& o = c->opts;
   o.fp16 = r.i64() != 0; o.bf16 = (odla_bf16_mode)r.i64(); o.int8 = r.i64() != 0; o.raw_acc = r.i64() != 0;
+  c->dynamic_batch = r.i64() != 0;
+  c->min_batch = (int)r.i64(); c->max_batch = (int)r.i64(); c->opt_batch = (int)r.i64();
+  if (!r.ok || c->min_batch < 0 || c->max_batch < 0 || c->opt_batch < 0) return ODLA_INVALID_PARAM;
   const int64_t nq = r.i64();
   if (!r.ok || nq < 0 || nq > (1 << 24)) return ODLA_INVALID_PARAM;
   c->owned_qnames.reserve((size_t)nq);
@@ -141,6 +145,7 @@ odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) 
     v->is_output = r.i64() != 0;
     v->eager = r.i64() != 0;
     v->producer = (int)r.i64();
+    v->dyn_batch = r.i64() != 0;
     if (v->kind == _odla_value::CONSTANT) {
       const int64_t bytes = r.i64();
       if (!r.ok || bytes <= 0 || (size_t)bytes > r.n - r.pos ||

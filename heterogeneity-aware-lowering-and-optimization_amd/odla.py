@@ -154,6 +154,9 @@ def load_library(path=None):
     proto("odla_GetNumOfOutputsFromComputation", i32, [vp, pu32])
     proto("odla_GetOutputFromComputationByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
     proto("odla_GetRuntimeShape", i32, [vp, vp, ctypes.POINTER(S)])
+    proto("odla_SetRuntimeShape", i32, [vp, vp, S])
+    proto("odla_SetRuntimeValueType", i32, [vp, vp, T])
+    proto("odla_GetRuntimeValueType", i32, [vp, vp, ctypes.POINTER(T)])
     proto("odla_GetValueType", i32, [vp, ctypes.POINTER(T)])
     proto("odla_GetValueId", i32, [vp, ctypes.POINTER(cid)])
     proto("odla_FindValueById", i32, [cid, ctypes.POINTER(vp)])
@@ -293,10 +296,21 @@ def _check(st, what):
 class HipBuilder:
     """Builds an ODLA computation on libodla_hip.so; one method per operator."""
 
-    def __init__(self, fp16=False, bf16=False, quant_table=None, raw_acc=False, lib=None):
+    def __init__(self, fp16=False, bf16=False, quant_table=None, raw_acc=False, lib=None, max_batch=0):
+        """max_batch > 0 records a dynamic-batch computation: arguments declared with a
+        leading extent of -1 are planned at max_batch and a Session may run any
+        batch 1..max_batch (Session.set_batch)."""
         self.L = lib or load_library()
         self.comp = ctypes.c_void_p()
         _check(self.L.odla_CreateComputation(ctypes.byref(self.comp)), "odla_CreateComputation")
+        self.max_batch = int(max_batch)
+        if self.max_batch > 0:
+            t = ctypes.c_bool(True)
+            _check(self.L.odla_SetComputationItem(self.comp, ODLA_DYNAMIC_BATCH, ctypes.byref(t)), "DYNAMIC_BATCH")
+            for item, n in ((ODLA_MIN_BATCH_SIZE, 1), (ODLA_MAX_BATCH_SIZE, self.max_batch),
+                            (ODLA_OPT_BATCH_SIZE, self.max_batch)):
+                v = ctypes.c_int(n)
+                _check(self.L.odla_SetComputationItem(self.comp, item, ctypes.byref(v)), "BATCH_SIZE item")
         self._keep = []      # numpy arrays / ctypes objects that must outlive the computation
         self.args = {}       # name -> (handle, shape, dtype)
         self.outs = {}       # name -> (handle, shape, dtype)
@@ -333,6 +347,8 @@ class HipBuilder:
     # -- graph inputs --
     def arg(self, name, shape, dtype=np.float32):
         h = self._ret(self.L.odla_CreateArgument(make_type(dtype, shape), _cid(name)), "odla_CreateArgument")
+        if shape and shape[0] < 0:          # the dynamic batch: recorded at the largest one
+            shape = (self.max_batch,) + tuple(shape[1:])
         self.args[name] = (h, tuple(shape), np.dtype(dtype))
         return h
 
@@ -630,17 +646,28 @@ class Session:
             _check(self.L.odla_SetContextItem(self.ctx, ODLA_AGGREGATE_OPS, ctypes.byref(f)), "AGGREGATE_OPS")
         self._dev = []
 
+    def set_batch(self, batch):
+        """Run the following executions at `batch` (dynamic-batch computations)."""
+        v = ctypes.c_int(int(batch))
+        _check(self.L.odla_SetContextItem(self.ctx, ODLA_RUN_BATCH_SIZE, ctypes.byref(v)), "RUN_BATCH_SIZE")
+
+    def runtime_shape(self, h):
+        """Shape of a value at the batch this session runs at."""
+        s = ValueShape()
+        _check(self.L.odla_GetRuntimeShape(self.ctx, h, ctypes.byref(s)), "odla_GetRuntimeShape")
+        return tuple(s.dims[i] for i in range(s.size))
+
     def run(self, feeds):
         """feeds: name -> numpy array.  Returns name -> numpy array."""
         keep = []
         for name, (h, shape, dt) in self.b.args.items():
             a = np.ascontiguousarray(feeds[name], dtype=dt)
-            assert tuple(a.shape) == shape, (name, a.shape, shape)
+            assert tuple(a.shape) == self.runtime_shape(h), (name, a.shape, self.runtime_shape(h))
             keep.append(a)
             _check(self.L.odla_BindToArgument(h, a.ctypes.data_as(ctypes.c_void_p), self.ctx), "odla_BindToArgument")
         outs = {}
         for name, (h, shape, dt) in self.b.outs.items():
-            o = np.empty(shape, dt)
+            o = np.empty(self.runtime_shape(h), dt)
             outs[name] = o
             _check(self.L.odla_BindToOutput(h, o.ctypes.data_as(ctypes.c_void_p), self.ctx), "odla_BindToOutput")
         _check(self.L.odla_ExecuteComputation(self.b.comp, self.ctx, ODLA_COMPUTE_INFERENCE, None), "odla_ExecuteComputation")

@@ -306,10 +306,30 @@ odla_status odla_GetNumOfOutputsFromComputation(
 odla_status odla_GetOutputFromComputationByIdx(
     const odla_computation computation, const odla_uint32 output_idx,
     odla_value* output_value);
-/* Static shapes only: returns the value's declared shape.
- * [ref: odla_compute.h:275-284] */
+/* Dynamic batch.  A computation recorded after
+ *   odla_SetComputationItem(comp, ODLA_DYNAMIC_BATCH, &true) and
+ *   odla_SetComputationItem(comp, ODLA_MAX_BATCH_SIZE, &n)
+ * declares its batch as a leading extent of -1 (odla_CreateArgument; -1 in the
+ * output dims of odla_Reshape is inferred) and is planned at batch n.  A context
+ * runs it at any batch 1..n chosen with
+ *   odla_SetContextItem(ctx, ODLA_RUN_BATCH_SIZE, &bs)   or
+ *   odla_SetRuntimeShape(ctx, argument, shape with the leading extent bs);
+ * bound buffers then hold bs rows.  Each batch is planned on first use from a
+ * copy of the recording with rescaled shapes (its own kernels, arena and
+ * hipGraph); graphs that move the batch out of the leading extent (a transpose
+ * of it, a reduction, slice or softmax along it) are refused with
+ * ODLA_UNSUPPORTED_OP.  Only the leading extent may change at run time.
+ * odla_GetRuntimeShape returns a value's shape at the context's batch.
+ * [ref: ODLA/include/ODLA/odla_compute.h:275-299,532-545;
+ *  ODLA/platforms/tensorrt/odla_tensorrt.cc:138-179,251-296] */
+odla_status odla_SetRuntimeShape(odla_context context, odla_value value,
+                                 odla_value_shape value_shape);
 odla_status odla_GetRuntimeShape(odla_context context, odla_value value,
                                  odla_value_shape* value_shape_ptr);
+odla_status odla_SetRuntimeValueType(odla_context context, odla_value value,
+                                     odla_value_type value_type);
+odla_status odla_GetRuntimeValueType(odla_context context, odla_value value,
+                                     odla_value_type* value_type_ptr);
 
 /* Values.                      [ref: ODLA/include/ODLA/odla_value.h:82-214] */
 odla_status odla_GetValueType(const odla_value value,

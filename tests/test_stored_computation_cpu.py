@@ -39,7 +39,7 @@ def test_store_load_store_is_identical(odla, tmp_path, with_table):
     loc1, k1 = odla.path_location(p1)
     assert L.odla_StoreComputation(loc1, hb.comp) == 0
     blob = open(p1, "rb").read()
-    assert blob[:8] == b"ODLAHIP1" and len(blob) > 8 * 3 * 3 * 3 * 4
+    assert blob[:8] == b"ODLAHIP2" and len(blob) > 8 * 3 * 3 * 3 * 4
 
     comp2 = ctypes.c_void_p()
     assert L.odla_LoadComputation(loc1, ctypes.byref(comp2)) == 0
