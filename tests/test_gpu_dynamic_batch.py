@@ -308,3 +308,67 @@ def test_stored_executable_keeps_the_dynamic_batch(tmp_path):
     finally:
         L.odla_DestroyContext(ctx)
         assert L.odla_DestroyExecutable(exe) == 0
+
+
+SMALL_STAGES = [(16, 2, 1), (32, 2, 2), (64, 1, 2)]
+
+
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def test_resnet_builder_recorded_with_a_dynamic_batch(mode):
+    """The package's ResNet-50 builder (stem with its space-to-depth copy, bottleneck
+    blocks with projection shortcuts, pooling, classifier) recorded once at batch -1."""
+    pkg = entry.load()
+    odla, models = pkg.odla, pkg.models
+    w = models.resnet50_weights(seed=3, num_classes=100, stages=SMALL_STAGES, stem=16)
+    MAXB = 6
+    hb = odla.HipBuilder(fp16=(mode == "fp16"), max_batch=MAXB)
+    try:
+        models.build_resnet50(hb, w, -1, 64, SMALL_STAGES, 16, 100)
+        s = hb.session(True)
+        try:
+            for bs in (1, MAXB, 4, 1):
+                announce("dynamic batch resnet builder %s batch %d" % (mode, bs))
+                feeds = models.resnet50_input(bs, 64, seed=40 + bs)
+                s.set_batch(bs)
+                got = s.run(feeds)
+                want = run_ref(lambda b: models.build_resnet50(b, w, bs, 64, SMALL_STAGES, 16, 100), feeds)
+                assert got["logits"].shape == (bs, 100)
+                scale = max(1.0, float(np.max(np.abs(want["logits"]))))
+                tol = 1e-4 if mode == "fp32" else 2e-2
+                assert np.max(np.abs(got["logits"] - want["logits"])) <= tol * scale, bs
+                if mode == "fp16":
+                    assert np.array_equal(np.argmax(got["logits"], 1), np.argmax(want["logits"], 1))
+        finally:
+            s.close()
+    finally:
+        hb.destroy()
+
+
+def test_bert_builder_recorded_with_a_dynamic_batch():
+    pkg = entry.load()
+    odla, mb = pkg.odla, pkg.models_bert
+    cfg = dict(layers=2, hidden=96, heads=3, ffn=192, vocab=120, max_pos=64)
+    w = mb.bert_weights(cfg, seed=31)
+    MAXB, seq = 5, 33
+    for mode in ("fp32", "bf16"):
+        hb = odla.HipBuilder(bf16=(mode == "bf16"), max_batch=MAXB)
+        try:
+            mb.build_bert(hb, w, -1, seq, cfg)
+            s = hb.session(True)
+            try:
+                for bs in (2, MAXB, 1):
+                    announce("dynamic batch bert builder %s batch %d" % (mode, bs))
+                    feeds = mb.bert_input(bs, seq, cfg, seed=50 + bs)
+                    feeds["attention_mask"][0, 0, 0, seq - 9:] = 0.0
+                    s.set_batch(bs)
+                    got = s.run(feeds)["hidden"]
+                    want = run_ref(lambda b: mb.build_bert(b, w, bs, seq, cfg), feeds)["hidden"]
+                    assert got.shape == want.shape
+                    if mode == "fp32":
+                        assert max_rel_err(got, want) <= 2e-4, bs
+                    else:
+                        assert np.max(np.abs(got - want)) <= 3e-2 * max(1.0, float(np.max(np.abs(want)))), bs
+            finally:
+                s.close()
+        finally:
+            hb.destroy()
