@@ -95,8 +95,11 @@ class Chain:
         self.outputs = sorted(marks)
         self.x = r.standard_normal(self.in_shape).astype(np.float32)
 
-    def build(self, b, probe=None):
-        vals = [b.arg("x", self.in_shape)]
+    def build(self, b, probe=None, batch=None, rows=None):
+        """batch: leading extent given to the argument (-1 records a dynamic batch);
+        rows: the batch the slices span (the largest batch of a dynamic recording)."""
+        vals = [b.arg("x", self.in_shape if batch is None else (batch,) + self.in_shape[1:])]
+        rows = rows or (self.in_shape[0] if batch is None else batch)
         for i, st in enumerate(self.steps):
             name = "v%d" % (i + 1)
             kind, src = st[0], vals[st[1]]
@@ -131,7 +134,7 @@ class Chain:
                 v = b.resize_nearest(src, (2 * sh[2], 2 * sh[3]), name=name)
             else:
                 sh = self.shapes[st[1]]
-                v = b.slice(src, (0, st[2], 0, 0), (sh[0], st[3], sh[2], sh[3]), name=name)
+                v = b.slice(src, (0, st[2], 0, 0), (rows, st[3], sh[2], sh[3]), name=name)
             vals.append(v)
             if probe is not None:
                 probe(len(vals) - 1, v)
@@ -161,6 +164,44 @@ def test_random_chains(mode, tmp_path):
             else:
                 scale = max(1.0, float(np.max(np.abs(w))))
                 assert float(np.max(np.abs(got[k] - w))) <= 6e-2 * scale, (seed, k, [s[0] for s in ch.steps])
+
+
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def test_random_chains_recorded_with_a_dynamic_batch(mode):
+    """The same programs recorded once with a batch of -1 and a largest batch above
+    the chain's own, run at the chain's batch, at the largest one and at the chain's
+    batch again: every batch is planned from a rescaled copy of the recording."""
+    import __graft_entry__ as entry
+    odla = entry.load().odla
+    for seed in range(1, 200, 3):
+        ch = Chain(SEED0 + seed)
+        if not ch.steps:
+            continue
+        n = ch.in_shape[0]
+        big = n + 1 + seed % 3
+        announce("dynamic-batch chain %s seed %d: %s, batch %d of %d" % (mode, seed, [s[0] for s in ch.steps], n, big))
+        r = np.random.default_rng(SEED0 + 9000 + seed)
+        xs = {n: ch.x, big: r.standard_normal((big,) + ch.in_shape[1:]).astype(np.float32)}
+        want = {k: run_ref(lambda b: ch.build(b, batch=k), {"x": x}) for k, x in xs.items()}
+        hb = odla.HipBuilder(fp16=(mode == "fp16"), max_batch=big)
+        try:
+            ch.build(hb, batch=-1, rows=big)
+            sess = hb.session(True)
+            try:
+                for k in (n, big, n):
+                    sess.set_batch(k)
+                    got = sess.run({"x": xs[k]})
+                    for name, w in want[k].items():
+                        assert got[name].shape == w.shape, (seed, k, name)
+                        if mode == "fp32":
+                            assert max_rel_err(got[name], w) <= 5e-4, (seed, k, name)
+                        else:
+                            scale = max(1.0, float(np.max(np.abs(w))))
+                            assert float(np.max(np.abs(got[name] - w))) <= 6e-2 * scale, (seed, k, name)
+            finally:
+                sess.close()
+        finally:
+            hb.destroy()
 
 
 def test_random_chains_in_interpret_mode():
