@@ -171,7 +171,15 @@ struct EpiFloat {
         Vec16<TOut> o;
 #pragma unroll
         for (int e = 0; e < 8; ++e) o.set(e, v[e]);
-        o.store(y);
+        if (p.stream_out) {
+          // The pointer passes through an empty asm so that the optimizer cannot
+          // fold this store and the plain one below into one plain store.
+          uintx4* yv = reinterpret_cast<uintx4*>(y);
+          asm volatile("" : "+v"(yv));
+          __builtin_nontemporal_store(o.raw, (__attribute__((address_space(1))) uintx4*)yv);
+        } else {
+          o.store(y);
+        }
       }
     } else {
 #pragma unroll
@@ -252,7 +260,13 @@ struct EpiQuant {
       ow[0] ^= 0x80808080u;  // levels -> stored
       ow[1] ^= 0x80808080u;
       if (vec) {
-        *reinterpret_cast<uintx2*>(y) = (uintx2){ow[0], ow[1]};
+        if (p.stream_out) {
+          uintx2* yv = reinterpret_cast<uintx2*>(y);
+          asm volatile("" : "+v"(yv));  // see EpiFloat::store8
+          __builtin_nontemporal_store((uintx2){ow[0], ow[1]}, (__attribute__((address_space(1))) uintx2*)yv);
+        } else {
+          *reinterpret_cast<uintx2*>(y) = (uintx2){ow[0], ow[1]};
+        }
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e)

@@ -97,6 +97,7 @@ struct IgemmParams {
   ActKind act = ACT_NONE;
   float act_a = 0.0f, act_b = 0.0f;  // leaky slope / clamp lo,hi
   bool res_after_act = false;        // float types: y = act(..) + residual instead of act(.. + residual)
+  bool stream_out = false;           // 2-byte results leave with non-temporal stores (results far larger than the last-level cache)
   // int8 only -----------------------------------------------------------
   // out_dt == DT_I8 : q = clamp(rne(float(acc+bias) * qmul[n]) + q_zp, q_lo, 255)
   //                   then, if residual: the unfused sequence

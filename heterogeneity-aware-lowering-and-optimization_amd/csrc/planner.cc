@@ -25,6 +25,15 @@ namespace {
 
 constexpr size_t kAlign = 256;
 constexpr int kUnset = 1 << 30;  // PTensor::def_step before any step touched the tensor
+// Convolution results of at least this size are written with non-temporal stores
+// (the chip's last-level cache holds 256 MiB); ODLA_HIP_STREAM_OUT_MB overrides it.
+size_t stream_out_bytes() {
+  static const size_t v = [] {
+    const char* e = getenv("ODLA_HIP_STREAM_OUT_MB");
+    return (size_t)(e != nullptr ? atol(e) : 150) << 20;
+  }();
+  return v;
+}
 size_t align_up(size_t v, size_t a = kAlign) { return (v + a - 1) / a * a; }
 int round_up_i(int v, int a) { return (v + a - 1) / a * a; }
 
@@ -1045,6 +1054,9 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
   ip.act_a = ep.act_a;
   ip.act_b = ep.act_b;
   ip.res_after_act = ep.res_after_act;
+  // A result much larger than the last-level cache cannot be kept there for its
+  // consumer; written around the cache it leaves the lines of smaller tensors alone.
+  ip.stream_out = T(ty).bytes >= stream_out_bytes();
   const int tf = make_wfrag(name, &ip, tw);
   const bool hf = tf >= 0;
   const Ref rf = ref(hf ? tf : tx);
@@ -1270,6 +1282,7 @@ void Planner::lower_conv(int ni) {
       ip.r_zp = T(tr).qzp;
       ip.r_scale = T(tr).qscale;
     }
+    ip.stream_out = T(ty).bytes >= stream_out_bytes();
     const int tf = make_wfrag("conv.i8:" + outv->name, &ip, tw);
     const bool hf = tf >= 0;
     const Ref rf = ref(hf ? tf : tx);
