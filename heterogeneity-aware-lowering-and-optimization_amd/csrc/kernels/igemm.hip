@@ -371,7 +371,8 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
     for (int ps = 0; ps < NPASS; ++ps) {
       const int m = tile_m * BM + wm * WM + i * 32 + ps * PPP + rp;
       const int mc = m < M ? m : M - 1;
-      dst[ps] = *reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n);
+      // read once by the whole launch: a non-temporal load leaves the cache lines to the operands that are re-read
+      dst[ps] = __builtin_nontemporal_load(reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n));
     }
   };
   RVec rcur[NPASS], rnxt[NPASS];
@@ -510,7 +511,8 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     for (int ps = 0; ps < 2; ++ps) {
       const int m = tile_m * BM + i * 32 + ps * 16 + rp;
       const int mc = m < M ? m : M - 1;
-      dst[ps] = *reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n);
+      // read once by the whole launch: a non-temporal load leaves the cache lines to the operands that are re-read
+      dst[ps] = __builtin_nontemporal_load(reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n));
     }
   };
   // The residual vectors of all four slices are requested here, ahead of the
