@@ -171,7 +171,8 @@ struct EpiFloat {
         Vec16<TOut> o;
 #pragma unroll
         for (int e = 0; e < 8; ++e) o.set(e, v[e]);
-        if (p.stream_out) {
+        // (not in the instantiations with the wider activation set: they have no registers to spare)
+        if (!kRich && p.stream_out) {
           // The pointer passes through an empty asm so that the optimizer cannot
           // fold this store and the plain one below into one plain store.
           uintx4* yv = reinterpret_cast<uintx4*>(y);
