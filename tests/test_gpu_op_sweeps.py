@@ -234,7 +234,8 @@ def test_binary_broadcast_sweep():
             B = np.where(r.random(sb) < 0.5, np.broadcast_to(A, np.broadcast_shapes(sa, sb))[tuple(slice(0, d) for d in sb)] if False else B, B)
 
         def build(b):
-            x = source(b, "a", sa, behind, wr)
+            # pow needs a positive base: no mixing in the convolution in front of it
+            x = source(b, "a", sa, behind, wr, mix=0.0 if op == "pow" else 0.05)
             y = b.const("b", B) if const_rhs else b.arg("b", sb)
             b.output(getattr(b, op)(x, y, name="y"), "y")
 
