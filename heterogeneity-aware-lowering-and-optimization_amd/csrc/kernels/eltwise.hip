@@ -270,12 +270,58 @@ cast_kernel(const TS* __restrict__ x, TD* __restrict__ y, int64_t n) {
     Store<TD>::st(y + i, Store<TS>::ld(x + i));
 }
 
-template <typename TS, typename TD>
+// Conversions that involve an integer type, one element per thread step.
+// Rules, following the reference's cast (a oneDNN reorder): a floating-point
+// value that becomes an integer is rounded to the nearest integer, ties to
+// even, and saturates at the ends of the target range; an integer that becomes
+// a narrower integer saturates; an integer that becomes a floating-point value
+// is rounded to nearest even; anything that becomes a bool is "!= 0".
+// [ref: ODLA/platforms/dnnl/odla_dnnl_cast.cc:232-258]
+template <typename T> struct CastElem;
+template <> struct CastElem<float> { static constexpr bool is_float = true; };
+template <> struct CastElem<f16_t> { static constexpr bool is_float = true; };
+template <> struct CastElem<bf16_t> { static constexpr bool is_float = true; };
+template <> struct CastElem<int8_t> { static constexpr bool is_float = false; static constexpr long long lo = -128, hi = 127; };
+template <> struct CastElem<uint8_t> { static constexpr bool is_float = false; static constexpr long long lo = 0, hi = 255; };
+template <> struct CastElem<int32_t> { static constexpr bool is_float = false; static constexpr long long lo = -2147483648ll, hi = 2147483647ll; };
+template <> struct CastElem<int64_t> { static constexpr bool is_float = false; static constexpr long long lo = INT64_MIN, hi = INT64_MAX; };
+
+// float -> integer type TD: clamp in float to the representable ends of the
+// target (2147483520 is the largest float below 2^31, 2^63 - 2^39 the largest
+// below 2^63), then round to nearest even.  NaN becomes 0.
+template <typename TD>
+__device__ __forceinline__ TD float_to_int_sat(float v) {
+  if (v != v) return (TD)0;
+  float lo, hi;
+  if constexpr (sizeof(TD) == 8) { lo = -9223372036854775808.f; hi = 9223371487098961920.f; }
+  else if constexpr (sizeof(TD) == 4) { lo = -2147483648.f; hi = 2147483520.f; }
+  else { lo = (float)CastElem<TD>::lo; hi = (float)CastElem<TD>::hi; }
+  const float c = fminf(fmaxf(v, lo), hi);
+  if constexpr (sizeof(TD) == 8) return (TD)__float2ll_rn(c);
+  else return (TD)__float2int_rn(c);
+}
+
+template <typename TS, typename TD, bool kDstBool>
 __global__ void __launch_bounds__(kThreads)
 cast_int_kernel(const TS* __restrict__ x, TD* __restrict__ y, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
-    y[i] = (TD)x[i];
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+    if constexpr (CastElem<TS>::is_float) {
+      const float v = Store<TS>::ld(x + i);
+      if constexpr (kDstBool) y[i] = (TD)(v != 0.f);
+      else y[i] = float_to_int_sat<TD>(v);
+    } else {
+      const long long v = (long long)x[i];
+      if constexpr (kDstBool) {
+        y[i] = (TD)(v != 0);
+      } else if constexpr (CastElem<TD>::is_float) {
+        Store<TD>::st(y + i, (float)v);
+      } else {
+        const long long lo = CastElem<TD>::lo, hi = CastElem<TD>::hi;
+        y[i] = (TD)(v < lo ? lo : (v > hi ? hi : v));
+      }
+    }
+  }
 }
 
 // q = sat(rne(x / scale) + zp)
@@ -504,19 +550,40 @@ hipError_t launch_cast(const void* src, DType sdt, void* dst, DType ddt, int64_t
   CAST_CASE(DT_BF16, DT_BF16, bf16_t, bf16_t, cast_kernel)
   CAST_CASE(DT_F16, DT_BF16, f16_t, bf16_t, cast_kernel)
   CAST_CASE(DT_BF16, DT_F16, bf16_t, f16_t, cast_kernel)
-  CAST_CASE(DT_I64, DT_I32, int64_t, int32_t, cast_int_kernel)
-  CAST_CASE(DT_I32, DT_I64, int32_t, int64_t, cast_int_kernel)
-  CAST_CASE(DT_I32, DT_F32, int32_t, float, cast_int_kernel)
-  CAST_CASE(DT_I64, DT_F32, int64_t, float, cast_int_kernel)
-  CAST_CASE(DT_F32, DT_I32, float, int32_t, cast_int_kernel)
-  CAST_CASE(DT_F32, DT_I64, float, int64_t, cast_int_kernel)
-  CAST_CASE(DT_U8, DT_F32, uint8_t, float, cast_int_kernel)
-  CAST_CASE(DT_I8, DT_F32, int8_t, float, cast_int_kernel)
-  CAST_CASE(DT_BOOL, DT_F32, uint8_t, float, cast_int_kernel)
-  CAST_CASE(DT_I32, DT_I32, int32_t, int32_t, cast_int_kernel)
-  CAST_CASE(DT_I64, DT_I64, int64_t, int64_t, cast_int_kernel)
-  CAST_CASE(DT_U8, DT_U8, uint8_t, uint8_t, cast_int_kernel)
-  CAST_CASE(DT_I8, DT_I8, int8_t, int8_t, cast_int_kernel)
+#define CAST_INT_CASE(S_, D_, TS_, TD_, B_)                                                  \
+  if (sdt == S_ && ddt == D_) {                                                              \
+    hipLaunchKernelGGL((cast_int_kernel<TS_, TD_, B_>), dim3(grid), dim3(kThreads), 0, stream, \
+                       (const TS_*)src, (TD_*)dst, n);                                       \
+    return hipGetLastError();                                                                \
+  }
+  // every source type to every integer type and bool ...
+#define CAST_TO_INTS(S_, TS_)                        \
+  CAST_INT_CASE(S_, DT_I8, TS_, int8_t, false)       \
+  CAST_INT_CASE(S_, DT_U8, TS_, uint8_t, false)      \
+  CAST_INT_CASE(S_, DT_I32, TS_, int32_t, false)     \
+  CAST_INT_CASE(S_, DT_I64, TS_, int64_t, false)     \
+  CAST_INT_CASE(S_, DT_BOOL, TS_, uint8_t, true)
+  CAST_TO_INTS(DT_F32, float)
+  CAST_TO_INTS(DT_F16, f16_t)
+  CAST_TO_INTS(DT_BF16, bf16_t)
+  CAST_TO_INTS(DT_I8, int8_t)
+  CAST_TO_INTS(DT_U8, uint8_t)
+  CAST_TO_INTS(DT_I32, int32_t)
+  CAST_TO_INTS(DT_I64, int64_t)
+  CAST_TO_INTS(DT_BOOL, uint8_t)
+  // ... and every integer type and bool to every floating-point type
+#define CAST_TO_FLOATS(S_, TS_)                      \
+  CAST_INT_CASE(S_, DT_F32, TS_, float, false)       \
+  CAST_INT_CASE(S_, DT_F16, TS_, f16_t, false)       \
+  CAST_INT_CASE(S_, DT_BF16, TS_, bf16_t, false)
+  CAST_TO_FLOATS(DT_I8, int8_t)
+  CAST_TO_FLOATS(DT_U8, uint8_t)
+  CAST_TO_FLOATS(DT_I32, int32_t)
+  CAST_TO_FLOATS(DT_I64, int64_t)
+  CAST_TO_FLOATS(DT_BOOL, uint8_t)
+#undef CAST_TO_FLOATS
+#undef CAST_TO_INTS
+#undef CAST_INT_CASE
 #undef CAST_CASE
   return hipErrorInvalidValue;
 }

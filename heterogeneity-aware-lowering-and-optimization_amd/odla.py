@@ -372,6 +372,9 @@ class HipBuilder:
     def gemm(self, a, b, c=None, ta=False, tb=False, alpha=1.0, beta=1.0, name=None):
         return self._ret(self.L.odla_Gemm(a, int(ta), b, int(tb), alpha, beta, c, undefined_shape(), _cid(name)), "odla_Gemm")
 
+    def batch_matmul(self, a, b, ta=False, tb=False, name=None):
+        return self._ret(self.L.odla_BatchMatMul(a, int(ta), b, int(tb), undefined_shape(), _cid(name)), "odla_BatchMatMul")
+
     def _bin(self, fn, a, b, name):
         return self._ret(getattr(self.L, "odla_" + fn)(a, b, _cid(name)), "odla_" + fn)
 

@@ -19,8 +19,15 @@ Pin status (what fixes each function independently of this file):
       reference kernels (runtime/generic/*.cc) held in tests/golden.
   quantize / dequantize   ONNX QuantizeLinear published example (passes on the
       reference CPU backend), exhaustive half-integer rounding check.
-  layernorm / gelu / resize / concat   closed forms and library routines
-      (math.erf, numpy).
+  layernorm / gelu / concat   closed forms and library routines (math.erf, numpy).
+  resize_nearest   hand-listed source indices for non-integer ratios and the
+      loops of the reference's portable backend (odla_eigen.cc:619-631) restated
+      in plain Python.
+  cast_like_reference   hand-listed roundings (ties to even), saturation ends
+      and narrowing cases; behaviour at |x| >= 2^31 and for NaN is this build's
+      choice: PARITY UNPINNED there.
+  qadd (residual add of two 8-bit tensors)   hand-worked levels with exact
+      power-of-two scales: both ties, both clamps, the fused ReLU clamp.
   nms   ONNX NonMaxSuppression published examples, O(n^2) brute force.
   wider operator surface (trigonometric / hyperbolic functions, Elu family,
       comparisons, Select, Mod, reductions, ArgMax, TopK, Pad, Tile, LRN,
@@ -209,6 +216,35 @@ def qconv(xq, x_qp, w, bias, out_qp, stride, pad, relu=False):
     mul = ((np.float32(s_x) * s_w).astype(np.float32) / np.float32(s_y)).astype(np.float32)
     q = requant_q8(acc, mul, zp_y, zp_y if relu else 0)
     return q, acc
+
+
+def cast_like_reference(x, dtype):
+    """odla_Cast: a oneDNN reorder between f32 / s32 / s8 / u8 / bf16
+    [ref: ODLA/platforms/dnnl/odla_dnnl_cast.cc:232-258].  A floating-point value
+    that becomes an integer is rounded to nearest, ties to even, and saturates
+    at the ends of the target range (2147483520, the largest float below 2^31,
+    stands in for the upper end of int32); an integer that becomes a narrower
+    integer saturates; anything that becomes a bool is "!= 0".  Half-precision
+    targets round to nearest even (the reference's own fp16 conversion
+    truncates the mantissa, ``:49-104``; that defect is not reproduced).
+    Behaviour at |x| >= 2^31 and for NaN (-> 0) is this build's choice:
+    PARITY UNPINNED there."""
+    x = np.asarray(x)
+    dt = np.dtype(dtype)
+    if dt == np.bool_:
+        return x != 0
+    if dt.kind in "iu":
+        info = np.iinfo(dt)
+        if x.dtype.kind == "f":
+            v = x.astype(np.float32)
+            hi = {8: 9223371487098961920.0, 4: 2147483520.0}.get(dt.itemsize, float(info.max))
+            v = np.where(np.isnan(v), np.float32(0), v)
+            v = np.clip(v, np.float32(info.min), np.float32(hi))
+            return np.rint(v).astype(dt)
+        if x.dtype == np.bool_:
+            return x.astype(dt)
+        return np.clip(x.astype(np.int64), info.min, info.max).astype(dt)
+    return x.astype(dt)
 
 
 def qadd(aq, a_qp, bq, b_qp, out_qp, relu=False):
@@ -459,6 +495,11 @@ class RefBuilder:
         if c is not None and beta != 0:
             y = y + float(beta) * _f32(c).astype(np.float64)
         return self._name(name, y.astype(np.float32))
+
+    def batch_matmul(self, a, b, ta=False, tb=False, name=None):
+        """op(A) op(B) over matching leading batch dims [ref: ops/odla_ops_math.h:337-339;
+        the code generator emits odla_Gemm with alpha = 1 for it, matmul.cc:45-70]"""
+        return self.gemm(a, b, None, ta, tb, 1.0, 0.0, name=name)
 
     def maxpool(self, x, window, stride, pad, out_hw=None, name=None):
         return self._name(name, pool2d(x, window, stride, pad, out_hw, True))
@@ -798,7 +839,7 @@ class RefBuilder:
         return self._name(name, deconv2d(x, w, bias, stride, pad, group, out_hw))
 
     # data movement ----------------------------------------------------------
-    def cast(self, x, dtype, name=None): return self._name(name, np.asarray(x).astype(dtype))
+    def cast(self, x, dtype, name=None): return self._name(name, cast_like_reference(x, dtype))
     def concat(self, xs, axis, name=None): return self._name(name, np.concatenate(xs, axis=axis))
     def gather(self, x, idx, axis=0, name=None): return self._name(name, np.take(x, np.asarray(idx), axis=axis))
     def reshape(self, x, shape, name=None): return self._name(name, np.reshape(x, shape))

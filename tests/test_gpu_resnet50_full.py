@@ -1,14 +1,14 @@
-"""Full-size ResNet-50 v1.5 at the benchmark batch (256 x 3 x 224 x 224), where
-the CPU oracle cannot follow in test time.  The whole batch is checked through
-properties that do not depend on its size, and a few images of it against the
-oracle:
+"""Full-size ResNet-50 v1.5 at the benchmark batch (256 x 3 x 224 x 224).
 
   * fp16: probabilities are finite and sum to 1; the images of the batch do not
     influence each other (reversing the batch reverses the outputs bit for bit);
-    the first images agree with the fp32 oracle within the fp16 tolerance (2e-2
-    of the largest logit) with the same top-1 class.
+    EVERY image of the batch is compared with the fp32 oracle: largest absolute
+    difference of the logits at most 2e-2 and the same top-1 class on all 256
+    (the measured error and the logit scale are printed).
   * int8: the first images of the batch-256 run equal, bit for bit, the same
     images run at batch 4, and those equal the integer oracle's activations.
+    Activation ranges come from 32 seeded N(0,1) batches (seeds 1000 .. 1031,
+    one image each) run through the fp32 oracle.
 """
 import os
 import sys
@@ -24,7 +24,8 @@ pytestmark = pytest.mark.gpu
 sys.path.insert(0, os.path.join(entry.ROOT, "oracle"))
 
 BATCH = 256
-N_ORACLE = 2
+ORACLE_CHUNK = 32    # images per oracle pass (bounds the oracle's memory)
+FP16_ABS_TOL = 2e-2  # on the logits, absolute
 
 
 def test_resnet50_fp16_batch256(models):
@@ -43,12 +44,20 @@ def test_resnet50_fp16_batch256(models):
     rev = run_hip(build, {"input": np.ascontiguousarray(feeds["input"][::-1])}, fp16=True)
     assert np.array_equal(rev["logits"][::-1], logits)
 
-    announce("resnet50 fp32 oracle, %d images" % N_ORACLE)
-    sub = {"input": np.ascontiguousarray(feeds["input"][:N_ORACLE])}
-    want = run_ref(lambda b: models.build_resnet50(b, w, N_ORACLE), sub)
-    scale = max(1.0, float(np.max(np.abs(want["logits"]))))
-    assert np.max(np.abs(logits[:N_ORACLE] - want["logits"])) <= 2e-2 * scale
-    assert np.array_equal(np.argmax(logits[:N_ORACLE], 1), np.argmax(want["logits"], 1))
+    want = np.empty_like(logits)
+    for i0 in range(0, BATCH, ORACLE_CHUNK):
+        announce("resnet50 fp32 oracle, images %d .. %d" % (i0, i0 + ORACLE_CHUNK - 1))
+        sub = {"input": np.ascontiguousarray(feeds["input"][i0:i0 + ORACLE_CHUNK])}
+        want[i0:i0 + ORACLE_CHUNK] = run_ref(lambda b: models.build_resnet50(b, w, ORACLE_CHUNK), sub)["logits"]
+    err = np.max(np.abs(logits - want), axis=1)
+    top_ok = np.argmax(logits, 1) == np.argmax(want, 1)
+    srt = np.sort(want, axis=1)
+    announce("resnet50 fp16 vs fp32 oracle over %d images: max |d logits| = %.3e (mean of per-image maxima %.3e), "
+             "largest |logit| = %.3f, top-1 equal on %d / %d, smallest top-1 margin of the oracle = %.3e"
+             % (BATCH, err.max(), err.mean(), np.max(np.abs(want)), int(top_ok.sum()), BATCH,
+                float(np.min(srt[:, -1] - srt[:, -2]))))
+    assert err.max() <= FP16_ABS_TOL
+    assert np.all(top_ok)
 
 
 def test_resnet50_int8_batch256(models, odla, ref):
@@ -60,10 +69,10 @@ def test_resnet50_int8_batch256(models, odla, ref):
     def taps_of(feeds):
         rb = ref.RefBuilder(feeds)
         taps = []
-        models.build_resnet50(rb, w, 2, taps=taps)
+        models.build_resnet50(rb, w, 1, taps=taps)
         return dict(taps)
 
-    ranges = models.calibrate_ranges(taps_of, [models.resnet50_input(2, seed=2000 + i) for i in range(2)])
+    ranges = models.calibrate_ranges(taps_of, [models.resnet50_input(1, seed=1000 + i) for i in range(32)])
     entries = models.resnet50_quant_entries(w, ranges)
     qp = {e[0]: (e[1], e[2]) for e in entries if e[5] is None}
     qp["pool1"] = qp["stem.relu"]   # max pooling works on levels and keeps its input's scale / zero point

@@ -257,6 +257,75 @@ def test_requant_formula_rounding_and_saturation(ref):
     assert ref.requant_q8(acc, mul, zp=10, lo=10).reshape(-1).tolist() == [10, 10, 10, 10, 10, 12, 12, 255, 255]
 
 
+def test_qadd_hand_worked_levels(ref):
+    """Residual add of two 8-bit tensors: dequantise, add, requantise.  Scales are
+    powers of two, so every product below is exact and was worked by hand:
+    a: s = 0.5, zp = 10; b: s = 0.25, zp = 20; out: s = 0.5, zp = 5."""
+    a = np.array([12, 12, 13, 255, 0, 9, 8], np.uint8)
+    b = np.array([22, 21, 21, 255, 0, 21, 21], np.uint8)
+    # fa:        1.0   1.0   1.5  122.5  -5.0  -0.5  -1.0
+    # fb:        0.5   0.25  0.25 58.75  -5.0  0.25  0.25
+    # f / 0.5:   3.0   2.5   3.5  362.5  -20   -0.5  -1.5
+    # rne:       3     2     4    362    -20   -0    -2     (ties go to the even neighbour)
+    # + 5:       8     7     9    367    -15   5     3
+    got = ref.qadd(a, (0.5, 10), b, (0.25, 20), (0.5, 5))
+    assert got.dtype == np.uint8 and got.tolist() == [8, 7, 9, 255, 0, 5, 3]
+    # a fused ReLU clamps at the zero point of the result instead of at 0
+    assert ref.qadd(a, (0.5, 10), b, (0.25, 20), (0.5, 5), relu=True).tolist() == [8, 7, 9, 255, 5, 5, 5]
+
+
+def test_resize_nearest_source_index_rule(ref):
+    """src = floor(in * dst / out) per axis, as the reference's portable backend
+    loops it (channels-last there, channels-first here)
+    [ref: ODLA/platforms/odla_eigen.cc:619-631].  Hand-listed indices for ratios that
+    are not integers, then the same loops in plain Python on random data."""
+    rb = ref.RefBuilder({})
+    x = np.arange(3, dtype=np.float32).reshape(1, 1, 1, 3)
+    assert rb.resize_nearest(x, (1, 7)).reshape(-1).tolist() == [0, 0, 0, 1, 1, 2, 2]     # 3 -> 7
+    x = np.arange(7, dtype=np.float32).reshape(1, 1, 7, 1)
+    assert rb.resize_nearest(x, (3, 1)).reshape(-1).tolist() == [0, 2, 4]                 # 7 -> 3
+    x = np.arange(5, dtype=np.float32).reshape(1, 1, 5, 1)
+    assert rb.resize_nearest(x, (8, 1)).reshape(-1).tolist() == [0, 0, 1, 1, 2, 3, 3, 4]  # 5 -> 8
+    x = np.arange(4, dtype=np.float32).reshape(1, 1, 2, 2)
+    assert rb.resize_nearest(x, (4, 4))[0, 0].tolist() == [[0, 0, 1, 1], [0, 0, 1, 1], [2, 2, 3, 3], [2, 2, 3, 3]]
+
+    r = rng(31)
+    for (ih, iw), (oh, ow) in (((5, 7), (8, 3)), ((13, 13), (26, 26)), ((6, 4), (4, 9)), ((1, 3), (5, 5))):
+        x = r.standard_normal((2, 3, ih, iw)).astype(np.float32)
+        want = np.empty((2, 3, oh, ow), np.float32)
+        for n in range(2):
+            for h in range(oh):
+                src_h = ih * h // oh
+                for w in range(ow):
+                    src_w = iw * w // ow
+                    want[n, :, h, w] = x[n, :, src_h, src_w]
+        assert np.array_equal(rb.resize_nearest(x, (oh, ow)), want)
+
+
+def test_cast_rounds_to_even_and_saturates(ref):
+    """odla_Cast is a oneDNN reorder in the reference [ref: odla_dnnl_cast.cc:232-258]:
+    float -> integer rounds to nearest even and saturates.  Hand-listed values."""
+    x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 2.4999, 126.5, 127.5, 300.0, -128.5, -129.5, -1000.0, 254.5, 255.5],
+                 np.float32)
+    assert ref.cast_like_reference(x, np.int8).tolist() == \
+        [0, 2, 2, 0, -2, -2, 2, 126, 127, 127, -128, -128, -128, 127, 127]
+    assert ref.cast_like_reference(x, np.uint8).tolist() == \
+        [0, 2, 2, 0, 0, 0, 2, 126, 128, 255, 0, 0, 0, 254, 255]
+    assert ref.cast_like_reference(x, np.int32).tolist() == \
+        [0, 2, 2, 0, -2, -2, 2, 126, 128, 300, -128, -130, -1000, 254, 256]
+    big = np.array([3e9, -3e9, 2147483520.0, -2147483648.0, 16777217.0], np.float32)
+    assert ref.cast_like_reference(big, np.int32).tolist() == [2147483520, -2147483648, 2147483520, -2147483648, 16777216]
+    # integers: narrowing saturates, widening and int -> float are exact / round to nearest even
+    i = np.array([-70000, -129, -128, -1, 0, 127, 128, 255, 256, 70000], np.int32)
+    assert ref.cast_like_reference(i, np.int8).tolist() == [-128, -128, -128, -1, 0, 127, 127, 127, 127, 127]
+    assert ref.cast_like_reference(i, np.uint8).tolist() == [0, 0, 0, 0, 0, 127, 128, 255, 255, 255]
+    assert ref.cast_like_reference(np.array([16777217, 16777219], np.int32), np.float32).tolist() == [16777216.0, 16777220.0]
+    assert ref.cast_like_reference(np.array([0.0, -0.0, 0.25, np.nan], np.float32), np.bool_).tolist() == [False, False, True, True]
+    # float -> half precision: round to nearest even on the 10-bit (fp16) / 7-bit (bf16) mantissa
+    h = ref.cast_like_reference(np.array([1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 65520.0], np.float32), np.float16)
+    assert h.astype(np.float32).tolist() == [1.0, 1.0 + 2.0 ** -9, np.inf]
+
+
 def test_q8_accumulators_against_int64_brute_force(ref):
     r = rng(8)
     N, C, H, W, O, k = 2, 5, 6, 6, 4, 3
