@@ -2,9 +2,14 @@
 
   * fp16: probabilities are finite and sum to 1; the images of the batch do not
     influence each other (reversing the batch reverses the outputs bit for bit);
-    EVERY image of the batch is compared with the fp32 oracle: largest absolute
-    difference of the logits at most 2e-2 and the same top-1 class on all 256
-    (the measured error and the logit scale are printed).
+    EVERY image of the batch is compared with the fp32 oracle: same top-1 class
+    on all 256, and the largest difference of the logits within 1e-3 of the
+    largest logit.  The stated bound, 2e-2 absolute, presumes logits of the
+    usual magnitude (about 20, where it is the same 1e-3): the random He-normal
+    weights of this configuration, with identity batch norms, give logits up to
+    3.7e3, where neighbouring fp16 numbers are 2.0 apart, so an absolute 2e-2
+    cannot hold for fp16 storage; measured 3.0 = 8e-4 of the scale.  The
+    measured error, the logit scale and the top-1 margin are printed.
   * int8: the first images of the batch-256 run equal, bit for bit, the same
     images run at batch 4, and those equal the integer oracle's activations.
     Activation ranges come from 32 seeded N(0,1) batches (seeds 1000 .. 1031,
@@ -25,7 +30,8 @@ sys.path.insert(0, os.path.join(entry.ROOT, "oracle"))
 
 BATCH = 256
 ORACLE_CHUNK = 32    # images per oracle pass (bounds the oracle's memory)
-FP16_ABS_TOL = 2e-2  # on the logits, absolute
+FP16_ABS_TOL = 2e-2  # on the logits, absolute, for logits of magnitude up to 20
+FP16_REL_TOL = 1e-3  # ... and this fraction of the largest logit beyond
 
 
 def test_resnet50_fp16_batch256(models):
@@ -56,7 +62,7 @@ def test_resnet50_fp16_batch256(models):
              "largest |logit| = %.3f, top-1 equal on %d / %d, smallest top-1 margin of the oracle = %.3e"
              % (BATCH, err.max(), err.mean(), np.max(np.abs(want)), int(top_ok.sum()), BATCH,
                 float(np.min(srt[:, -1] - srt[:, -2]))))
-    assert err.max() <= FP16_ABS_TOL
+    assert err.max() <= max(FP16_ABS_TOL, FP16_REL_TOL * float(np.max(np.abs(want))))
     assert np.all(top_ok)
 
 
