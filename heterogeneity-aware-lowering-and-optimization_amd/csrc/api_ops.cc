@@ -41,8 +41,24 @@ _odla_computation* comp_of(odla_value a, odla_value b = nullptr) {
   return current_computation();
 }
 
+// Appends a node and its result value.  Returns nullptr (and logs) when the
+// computation no longer takes operators - it has been compiled and a caller's
+// context runs its plan - or when an operand belongs to another computation.
+// One thread records into a computation at a time; the lock only orders the
+// append against a compilation running on another thread.
 Node* add_node(_odla_computation* c, OpKind op, std::vector<odla_value> in, odla_element_type et,
                const Shape& shape, const odla_value_id id) {
+  for (const odla_value v : in) {
+    if (v != nullptr && v->comp != c) {
+      OHIP_ERR("odla_%s: operand '%s' belongs to another computation", op_name(op), v->name.c_str());
+      return nullptr;
+    }
+  }
+  std::lock_guard<std::mutex> lk(c->mu);
+  if (c->plan && c->live_contexts > 0) {
+    OHIP_ERR("odla_%s: the computation is compiled and has contexts; operators recorded now would not run", op_name(op));
+    return nullptr;
+  }
   odla_value out = new_value(c, _odla_value::TEMP, et, shape, id);
   c->nodes.emplace_back();
   Node& n = c->nodes.back();
@@ -52,6 +68,8 @@ Node* add_node(_odla_computation* c, OpKind op, std::vector<odla_value> in, odla
   out->producer = (int)c->nodes.size() - 1;
   return &n;
 }
+
+#define ADD_NODE_FAILED {}
 
 bool is_float_type(odla_element_type t) {
   return t == ODLA_FLOAT32 || t == ODLA_FLOAT16 || t == ODLA_BFLOAT16;
@@ -115,6 +133,7 @@ odla_value binary(BinKind kind, odla_value lhs, odla_value rhs, const odla_value
     o.d[i] = a.d[i] > b.d[i] ? a.d[i] : b.d[i];
   }
   Node* n = add_node(c, OP_BINARY, {lhs, rhs}, lhs->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = kind;
   // remember the aligned operand shapes for the planner
   n->iv.clear();
@@ -154,6 +173,7 @@ odla_value ewise(EwiseOp op, std::vector<odla_value> in, odla_element_type out_t
   }
   if (target) REQUIRE(o == *target, "%s: operands do not broadcast to %s", what, target->str().c_str());
   Node* n = add_node(c, OP_EWISE, in, out_type, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = op;
   n->iv.push_back(o.rank);
   for (const Shape& s : al)
@@ -186,6 +206,7 @@ odla_value unary(ActKind kind, odla_value x, float a, float b, const odla_value_
   REQUIRE(c, "unary op: no current computation");
   REQUIRE(is_float_type(x->etype), "unary op on non-float value '%s'", x->name.c_str());
   Node* n = add_node(c, OP_UNARY, {x}, x->etype, x->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = kind;
   n->f[0] = a;
   n->f[1] = b;
@@ -221,6 +242,7 @@ odla_value pool(bool is_max, odla_value input, odla_memory_layout layout, const 
   }
   REQUIRE(o.d[hd] > 0 && o.d[wd] > 0, "pool: empty output");
   Node* n = add_node(c, OP_POOL, {input}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = layout;
   n->i[1] = is_max;
   n->i[2] = window[0]; n->i[3] = window[1];
@@ -254,6 +276,7 @@ odla_value reduce(ReduceKind kind, odla_value input, odla_size_t num_axes, const
   }
   if (o.rank == 0) { o.rank = 1; o.d[0] = 1; }
   Node* n = add_node(c, OP_REDUCE, {input}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = kind;
   n->i[1] = keep_dims;
   n->f[0] = eps;
@@ -267,6 +290,7 @@ odla_value copynd(_odla_computation* c, odla_value x, const Shape& out, const st
                   const std::vector<int64_t>& sx, const std::vector<int64_t>& sy, int64_t x_off, int64_t y_off,
                   bool fill, const odla_value_id id) {
   Node* n = add_node(c, OP_COPYND, {x}, x->etype, out, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = fill;
   n->iv.push_back((int64_t)dims.size());
   n->iv.insert(n->iv.end(), dims.begin(), dims.end());
@@ -311,6 +335,7 @@ odla_value arg_extreme(bool is_max, odla_value input, odla_int32 axis, odla_bool
   }
   if (o.rank == 0) { o.rank = 1; o.d[0] = 1; }
   Node* n = add_node(c, OP_ARGEXT, {input}, et, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = is_max;
   n->i[1] = axis;
   n->i[2] = return_last_index != 0;
@@ -361,6 +386,7 @@ odla_value odla_Conv(odla_value input, odla_memory_layout input_layout, odla_uin
   o.d[0] = N;
   if (cl) { o.d[1] = Ho; o.d[2] = Wo; o.d[3] = O; } else { o.d[1] = O; o.d[2] = Ho; o.d[3] = Wo; }
   Node* n = add_node(c, OP_CONV, {input, kernel, bias}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = input_layout;
   n->i[1] = group;
   n->i[2] = kernel_layout;
@@ -431,6 +457,7 @@ odla_value odla_Gemm(odla_value A, odla_bool tA, odla_value B, odla_bool tB, odl
     return binary(BIN_ADD, g, cs, id);
   }
   Node* n = add_node(c, OP_GEMM, {A, B, C}, A->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = tA ? 1 : 0;
   n->i[1] = tB ? 1 : 0;
   n->f[0] = alpha;
@@ -510,6 +537,7 @@ odla_value odla_Mean(odla_values inputs, const odla_value_id id) {
   }
   _odla_computation* c = comp_of(acc);
   Node* n = add_node(c, OP_UNARY, {acc}, acc->etype, acc->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = ACT_DIV_CONST;
   n->f[0] = (float)inputs.size;
   return n->out;
@@ -583,6 +611,7 @@ odla_value odla_BatchNormalization(odla_value input, odla_memory_layout layout, 
   if (scale) REQUIRE(scale->shape.numel() == C, "odla_BatchNormalization: scale size");
   if (offset) REQUIRE(offset->shape.numel() == C, "odla_BatchNormalization: offset size");
   Node* n = add_node(c, OP_BATCHNORM, {input, mean, var, scale, offset}, input->etype, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = layout;
   n->f[0] = epsilon;
   n->f[1] = scalar_scale;
@@ -615,6 +644,7 @@ odla_value odla_LayerNorm(odla_value input, odla_size_t axes_size, const odla_in
   if (scale) REQUIRE(scale->shape.numel() == len, "odla_LayerNorm: scale must have %lld elements", (long long)len);
   if (offset) REQUIRE(offset->shape.numel() == len, "odla_LayerNorm: offset must have %lld elements", (long long)len);
   Node* n = add_node(c, OP_LAYERNORM, {input, scale, offset}, input->etype, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = n_axes;
   n->f[0] = epsilon;
   return n->out;
@@ -711,6 +741,7 @@ static odla_value softmax_impl(odla_value input, odla_int32 axis, bool logsm, co
   if (axis < 0) axis = r - 1;
   REQUIRE(axis < r, "softmax: axis %d out of range for %s", axis, input->shape.str().c_str());
   Node* n = add_node(c, OP_SOFTMAX, {input}, input->etype, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = axis;
   n->i[1] = logsm;
   return n->out;
@@ -724,6 +755,7 @@ odla_value odla_Cast(odla_value input, odla_element_type target, const odla_valu
   REQUIRE(c, "odla_Cast: no current computation");
   REQUIRE(dtype_from_odla(target) != DT_INVALID, "odla_Cast: unsupported target type %d", (int)target);
   Node* n = add_node(c, OP_CAST, {input}, target, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   return n->out;
 }
 
@@ -748,6 +780,7 @@ odla_value odla_Concat(odla_values inputs, odla_int32 axis, odla_value_shape, co
     in.push_back(v);
   }
   Node* n = add_node(c, OP_CONCAT, in, first->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = axis;
   return n->out;
 }
@@ -767,6 +800,7 @@ odla_value odla_Gather(odla_value input, odla_value indices, odla_int32 axis, od
   for (int i = axis + 1; i < r; ++i) o.d[o.rank++] = input->shape.d[i];
   REQUIRE(o.rank <= ODLA_MAX_DIMENSION, "odla_Gather: result rank too large");
   Node* n = add_node(c, OP_GATHER, {input, indices}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = axis;
   return n->out;
 }
@@ -791,6 +825,7 @@ odla_value odla_Reshape(odla_value input, odla_value_shape output_dims, const od
   REQUIRE(o.numel() == input->shape.numel(), "odla_Reshape: %s -> %s changes the element count",
           input->shape.str().c_str(), o.str().c_str());
   Node* n = add_node(c, OP_RESHAPE, {input}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   return n->out;
 }
 
@@ -807,6 +842,7 @@ odla_value odla_Resize(odla_value input, odla_interpolation_mode interpolation,
   REQUIRE(o.d[0] == input->shape.d[0] && o.d[1] == input->shape.d[1] && o.d[2] > 0 && o.d[3] > 0,
           "odla_Resize: output %s must keep batch and channels of %s", o.str().c_str(), input->shape.str().c_str());
   Node* n = add_node(c, OP_RESIZE, {input}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = interpolation;
   n->i[1] = mode;
   return n->out;
@@ -834,6 +870,7 @@ odla_value odla_Slice(odla_value input, const odla_int32* start, const odla_int3
     iv[i] = s; iv[r + i] = e; iv[2 * r + i] = stride[i];
   }
   Node* n = add_node(c, OP_SLICE, {input}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->iv = iv;
   return n->out;
 }
@@ -857,6 +894,7 @@ odla_value odla_Transpose(odla_value input, odla_value_shape permutations, odla_
     o.d[i] = input->shape.d[p];
   }
   Node* n = add_node(c, OP_TRANSPOSE, {input}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->iv = perm;
   return n->out;
 }
@@ -881,6 +919,7 @@ static odla_value qdq(OpKind op, odla_value input, odla_value scale, odla_value 
     REQUIRE(target == ODLA_FLOAT32, "odla_Dequantize: target must be FLOAT32");
   }
   Node* n = add_node(c, op, {input, scale, zp}, target, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = axis;
   return n->out;
 }
@@ -1013,6 +1052,7 @@ odla_values odla_TopK(odla_value input, odla_uint32 K, odla_bool largest, odla_b
   Shape o = xs;
   o.d[axis] = K;
   Node* n = add_node(c, OP_TOPK, {input}, input->etype, o, value_ids.size > 0 ? value_ids.value_ids[0] : nullptr);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->out2 = new_value(c, _odla_value::TEMP, it, o, value_ids.size > 1 ? value_ids.value_ids[1] : nullptr);
   n->out2->producer = n->out->producer;
   n->i[0] = K;
@@ -1067,6 +1107,7 @@ odla_values odla_PostProcess(odla_value orig_img_w, odla_value orig_img_h, odla_
   o1.rank = 1; o1.d[0] = classes;
   Node* n = add_node(c, OP_POSTPROCESS, {orig_img_w, orig_img_h, bb13, bb26, bb52}, ODLA_FLOAT32, o0,
                      value_id ? (const odla_value_id)n0.c_str() : nullptr);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->out2 = new_value(c, _odla_value::TEMP, ODLA_UINT32, o1, value_id ? (const odla_value_id)n1.c_str() : nullptr);
   n->out2->producer = n->out->producer;
   n->f[0] = 0.45f;  // IoU above which a box is suppressed
@@ -1088,6 +1129,7 @@ odla_value odla_LRN(odla_value input, odla_memory_layout layout, odla_int32 wind
   REQUIRE(input->shape.rank >= 3, "odla_LRN: rank < 3");
   REQUIRE(window_size >= 1 && (window_size & 1), "odla_LRN: the window must be odd");
   Node* n = add_node(c, OP_LRN, {input}, input->etype, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = layout == ODLA_CHANNELS_LAST ? ODLA_CHANNELS_LAST : ODLA_CHANNELS_FIRST;
   n->i[1] = window_size;
   n->f[0] = alpha; n->f[1] = beta; n->f[2] = bias;
@@ -1112,6 +1154,7 @@ odla_value odla_InstanceNormalization(odla_value input, odla_memory_layout layou
   if (offset) REQUIRE(offset->kind == _odla_value::CONSTANT && offset->shape.numel() == C,
                       "odla_InstanceNormalization: offset must be a constant with one element per channel");
   Node* n = add_node(c, OP_ROWNORM, {input, scale, offset}, input->etype, xs, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = cl ? ODLA_CHANNELS_LAST : ODLA_CHANNELS_FIRST;
   n->f[0] = epsilon; n->f[1] = scalar_scale; n->f[2] = scalar_offset;
   return n->out;
@@ -1194,6 +1237,7 @@ odla_value odla_DeConv(odla_value input, odla_memory_layout input_layout, odla_u
   o.rank = 4;
   o.d[0] = N; o.d[1] = O; o.d[2] = out_hw[0]; o.d[3] = out_hw[1];
   Node* n = add_node(c, OP_CONV, {xu, kf, bias}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = ODLA_CHANNELS_FIRST;
   n->i[1] = group;
   n->i[2] = ODLA_OIS;
@@ -1220,6 +1264,7 @@ odla_value odla_NMS(odla_value boxes, odla_value scores, odla_uint32 max_num_out
   o.d[1] = 3;
   REQUIRE(o.d[0] > 0, "odla_NMS: max_num_outputs must be positive");
   Node* n = add_node(c, OP_NMS, {boxes, scores}, et, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = max_num_outputs;
   n->f[0] = iou_threshold;
   n->f[1] = score_threshold;

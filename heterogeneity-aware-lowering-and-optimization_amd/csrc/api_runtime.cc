@@ -1,6 +1,7 @@
 // ODLA control plane of libodla_hip.so: computations, contexts, binding,
 // execution (hipGraph replay), value introspection, device / memory / logging.
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 
 #include "internal.h"
@@ -44,7 +45,10 @@ void log_msg(const char* file, int line, const char* func, odla_log_level lvl, c
 const char* op_name(OpKind k) {
   static const char* names[] = {"Conv", "Gemm", "Binary", "Unary", "BatchNorm", "LayerNorm", "Pool",
                                 "Reduce", "Softmax", "Cast", "Concat", "Gather", "Reshape", "Resize",
-                                "Slice", "Transpose", "Quantize", "Dequantize", "NMS", "Elementwise", "ArgExtreme", "CopyND", "TopK", "LRN", "RowNorm"};
+                                "Slice", "Transpose", "Quantize", "Dequantize", "NMS", "Elementwise", "ArgExtreme",
+                                "CopyND", "TopK", "LRN", "RowNorm", "PostProcess"};
+  static_assert(sizeof(names) / sizeof(names[0]) == (size_t)OP_POSTPROCESS + 1, "one name per OpKind");
+  if ((int)k < 0 || (int)k > (int)OP_POSTPROCESS) return "?";
   return names[(int)k];
 }
 
@@ -207,27 +211,64 @@ odla_status create_context_for(_odla_computation* c, odla_context* context);
 // The context that executes `ctx`'s computation at batch `bs`: `ctx` itself at
 // the recorded batch, otherwise a context over a rescaled copy of the recording
 // (made, planned and given an arena on first use).
+// Destroys a context and the contexts it holds over batch variants.
+void destroy_context_tree(_odla_context* ctx) {
+  for (auto& kv : ctx->variant_ctx) destroy_context_tree(kv.second.ctx);
+  ctx->variant_ctx.clear();
+  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  drop_graph(ctx);
+  if (ctx->arena) (void)hipFree(ctx->arena);
+  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+}
+
+// Batches (other than the recorded one) a context keeps planned at a time.
+int max_batch_variants() {
+  static const int n = [] {
+    const char* e = getenv("ODLA_HIP_MAX_BATCH_VARIANTS");
+    const int v = e ? atoi(e) : 0;
+    return v >= 1 ? v : 4;
+  }();
+  return n;
+}
+
 odla_status variant_context(_odla_context* ctx, int bs, _odla_context** out) {
   _odla_computation* c = ctx->comp;
   const int rec = recorded_batch(*c);
   if (bs == 0 || bs == rec) { *out = ctx; return ODLA_SUCCESS; }
   auto have = ctx->variant_ctx.find(bs);
-  if (have != ctx->variant_ctx.end()) { *out = have->second; return ODLA_SUCCESS; }
-  _odla_computation* v = nullptr;
+  if (have != ctx->variant_ctx.end()) {
+    have->second.last_use = ++ctx->variant_clock;
+    *out = have->second.ctx;
+    return ODLA_SUCCESS;
+  }
+  // make room first, so that the peak stays within the bound
+  while ((int)ctx->variant_ctx.size() >= max_batch_variants()) {
+    auto lru = ctx->variant_ctx.begin();
+    for (auto it = ctx->variant_ctx.begin(); it != ctx->variant_ctx.end(); ++it)
+      if (it->second.last_use < lru->second.last_use) lru = it;
+    destroy_context_tree(lru->second.ctx);
+    ctx->variant_ctx.erase(lru);  // drops this context's share of the variant: the last share frees its plan
+  }
+  std::shared_ptr<_odla_computation> v;
   {
     std::lock_guard<std::mutex> lk(c->mu);
     auto it = c->variants.find(bs);
-    if (it == c->variants.end()) {
+    if (it != c->variants.end()) v = it->second.lock();
+    if (!v) {
       std::unique_ptr<_odla_computation> copy = clone_for_batch(*c, rec, bs);
       if (!copy) return ODLA_UNSUPPORTED_OP;
-      it = c->variants.emplace(bs, std::move(copy)).first;
+      v = std::move(copy);
+      c->variants[bs] = v;
     }
-    v = it->second.get();
   }
   odla_context sub = nullptr;
-  odla_status st = create_context_for(v, &sub);
+  odla_status st = create_context_for(v.get(), &sub);
   if (st != ODLA_SUCCESS) return st;
-  ctx->variant_ctx[bs] = sub;
+  _odla_context::Variant& slot = ctx->variant_ctx[bs];
+  slot.comp = std::move(v);
+  slot.ctx = sub;
+  slot.last_use = ++ctx->variant_clock;
   *out = sub;
   return ODLA_SUCCESS;
 }
@@ -238,8 +279,9 @@ odla_status set_run_batch(_odla_context* ctx, int bs) {
     OHIP_ERR("ODLA_RUN_BATCH_SIZE: the computation was not recorded with ODLA_DYNAMIC_BATCH and ODLA_MAX_BATCH_SIZE");
     return ODLA_FAILURE;
   }
-  if (bs < 1 || bs > rec) {
-    OHIP_ERR("ODLA_RUN_BATCH_SIZE: %d is outside 1..%d", bs, rec);
+  const int lo = ctx->comp->min_batch > 0 ? ctx->comp->min_batch : 1;
+  if (bs < lo || bs > rec) {
+    OHIP_ERR("ODLA_RUN_BATCH_SIZE: %d is outside %d..%d (ODLA_MIN_BATCH_SIZE .. ODLA_MAX_BATCH_SIZE)", bs, lo, rec);
     return ODLA_FAILURE;
   }
   _odla_context* sub = nullptr;
@@ -387,15 +429,7 @@ odla_status create_context_for(_odla_computation* c, odla_context* context) {
 }  // namespace
 extern "C" {
 
-static void destroy_context(odla_context ctx) {
-  for (auto& kv : ctx->variant_ctx) destroy_context(kv.second);
-  ctx->variant_ctx.clear();
-  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-  drop_graph(ctx);
-  if (ctx->arena) (void)hipFree(ctx->arena);
-  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
-  delete ctx;
-}
+static void destroy_context(odla_context ctx) { destroy_context_tree(ctx); }
 
 odla_status odla_DestroyContext(odla_context ctx) {
   if (ctx == nullptr) return ODLA_INVALID_PARAM;
@@ -658,7 +692,7 @@ odla_status odla_GetRuntimeShape(odla_context ctx, odla_value value, odla_value_
   if (ctx != nullptr && value->comp == ctx->comp && ctx->run_batch > 0) {
     // the value's shape at the batch this context runs at
     auto it = ctx->variant_ctx.find(ctx->run_batch);
-    if (it != ctx->variant_ctx.end()) *shape = shape_to(it->second->comp->values[value->index]->shape);
+    if (it != ctx->variant_ctx.end()) *shape = shape_to(it->second.comp->values[value->index]->shape);
   }
   return ODLA_SUCCESS;
 }
@@ -785,7 +819,7 @@ odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr, odla_
   if (ctx->run_batch > 0 && value->comp == ctx->comp) {
     auto it = ctx->variant_ctx.find(ctx->run_batch);
     if (it != ctx->variant_ctx.end())
-      return odla_GetValueData(it->second->comp->values[value->index].get(), data_ptr, it->second);
+      return odla_GetValueData(it->second.comp->values[value->index].get(), data_ptr, it->second.ctx);
   }
   if (!ctx->executed || !ctx->comp->plan) return ODLA_FAILURE;
   const Plan& plan = *ctx->comp->plan;

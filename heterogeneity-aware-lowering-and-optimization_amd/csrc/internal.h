@@ -229,7 +229,9 @@ struct _odla_computation {
   // another batch runs a copy of the recording whose shapes were rescaled
   bool dynamic_batch = false;
   int min_batch = 0, max_batch = 0, opt_batch = 0;
-  std::map<int, std::unique_ptr<_odla_computation>> variants;  // by run-time batch
+  // by run-time batch; owned by the contexts that run them (see _odla_context::variant_ctx):
+  // a variant, its plan and its packed constants go away with its last user
+  std::map<int, std::weak_ptr<_odla_computation>> variants;
   // quantisation table of a loaded computation (the caller's table is borrowed otherwise)
   std::vector<odla_value_quant_info> owned_qtable;
   std::vector<std::string> owned_qnames;
@@ -247,7 +249,17 @@ struct _odla_context {
   std::unordered_map<const _odla_value*, void*> bound_out;
   bool executed = false;
   int run_batch = 0;                              // 0: the recorded shapes
-  std::map<int, _odla_context*> variant_ctx;      // contexts over comp->variants, by batch
+  // Contexts over comp->variants, by batch.  Every batch a context has run keeps a
+  // planned copy of the recording alive (packed constants, arena, stream, graph),
+  // so the map is bounded: beyond kMaxBatchVariants (ODLA_HIP_MAX_BATCH_VARIANTS)
+  // entries the one used longest ago is destroyed and rebuilt if it is asked for again.
+  struct Variant {
+    std::shared_ptr<_odla_computation> comp;
+    _odla_context* ctx = nullptr;
+    uint64_t last_use = 0;
+  };
+  std::map<int, Variant> variant_ctx;
+  uint64_t variant_clock = 0;
 };
 
 struct _odla_device {

@@ -8,8 +8,13 @@
 // their attributes, outputs, precision options and the quantisation table.  A
 // loaded computation owns everything it needs and compiles like a recorded one.
 //
-// File layout (little endian): "ODLAHIP1", then the sections written by
-// Writer below; every variable-length item is preceded by its 64-bit length.
+// File layout (little endian): "ODLAHIP3", then the sections written by
+// Writer below; every variable-length item is preceded by its 64-bit length;
+// the last eight bytes are the FNV-1a hash of everything before them, so a
+// truncated or damaged file is refused before any of it is interpreted.  What
+// passes the hash is still checked record by record (validate_loaded): shapes,
+// element types and, per operator, the operands and attributes the planner
+// will index.
 #include <cstdio>
 #include <cstring>
 #include <memory>
@@ -22,7 +27,13 @@ using namespace ohip;
 
 namespace {
 
-const char kMagic[8] = {'O', 'D', 'L', 'A', 'H', 'I', 'P', '2'};
+const char kMagic[8] = {'O', 'D', 'L', 'A', 'H', 'I', 'P', '3'};
+
+uint64_t fnv1a(const uint8_t* p, size_t n) {
+  uint64_t h = 1469598103934665603ull;
+  for (size_t i = 0; i < n; ++i) { h ^= p[i]; h *= 1099511628211ull; }
+  return h;
+}
 
 struct Writer {
   std::vector<uint8_t> buf;
@@ -101,17 +112,223 @@ odla_status serialize(_odla_computation* c, std::vector<uint8_t>* out) {
     w.i64((int64_t)n.iv.size());
     for (int64_t v : n.iv) w.i64(v);
   }
+  const uint64_t h = fnv1a(w.buf.data(), w.buf.size());
+  w.raw(&h, 8);
   *out = std::move(w.buf);
   return ODLA_SUCCESS;
 }
 
+// ---------------------------------------------------------------------------
+// What a node of each operator must look like for the planner to index it
+// safely: operand slots (count and which may be empty), second result, the
+// length of the integer list, attribute ranges.  Mirrors what the builders in
+// api_ops.cc record.
+struct OpRule {
+  int min_in, max_in;   // operand slots
+  unsigned required;    // bit k: slot k must hold a value
+  bool out2;
+};
+
+bool op_rule(OpKind op, OpRule* r) {
+  switch (op) {
+    case OP_CONV: *r = {3, 3, 0x3, false}; return true;
+    case OP_GEMM: *r = {3, 3, 0x3, false}; return true;
+    case OP_BINARY: *r = {2, 2, 0x3, false}; return true;
+    case OP_UNARY: *r = {1, 1, 0x1, false}; return true;
+    case OP_BATCHNORM: *r = {5, 5, 0x7, false}; return true;
+    case OP_LAYERNORM: *r = {3, 3, 0x1, false}; return true;
+    case OP_POOL: *r = {1, 1, 0x1, false}; return true;
+    case OP_REDUCE: *r = {1, 1, 0x1, false}; return true;
+    case OP_SOFTMAX: *r = {1, 1, 0x1, false}; return true;
+    case OP_CAST: *r = {1, 1, 0x1, false}; return true;
+    case OP_CONCAT: *r = {1, ODLA_MAX_OUTPUTS, ~0u, false}; return true;
+    case OP_GATHER: *r = {2, 2, 0x3, false}; return true;
+    case OP_RESHAPE: *r = {1, 1, 0x1, false}; return true;
+    case OP_RESIZE: *r = {1, 1, 0x1, false}; return true;
+    case OP_SLICE: *r = {1, 1, 0x1, false}; return true;
+    case OP_TRANSPOSE: *r = {1, 1, 0x1, false}; return true;
+    case OP_QUANTIZE: case OP_DEQUANTIZE: *r = {3, 3, 0x3, false}; return true;
+    case OP_NMS: *r = {2, 2, 0x3, false}; return true;
+    case OP_EWISE: *r = {1, 3, ~0u, false}; return true;
+    case OP_ARGEXT: *r = {1, 1, 0x1, false}; return true;
+    case OP_COPYND: *r = {1, 1, 0x1, false}; return true;
+    case OP_TOPK: *r = {1, 1, 0x1, true}; return true;
+    case OP_LRN: *r = {1, 1, 0x1, false}; return true;
+    case OP_ROWNORM: *r = {3, 3, 0x1, false}; return true;
+    case OP_POSTPROCESS: *r = {5, 5, 0x1f, true}; return true;
+  }
+  return false;
+}
+
+#define LOADED_REQUIRE(cond, ...)                                   \
+  do {                                                              \
+    if (!(cond)) {                                                  \
+      OHIP_ERR("stored computation rejected: " __VA_ARGS__);        \
+      return ODLA_INVALID_PARAM;                                    \
+    }                                                               \
+  } while (0)
+
+odla_status validate_loaded(const _odla_computation* c) {
+  const int64_t nn = (int64_t)c->nodes.size();
+  for (const auto& up : c->values) {
+    const _odla_value& v = *up;
+    LOADED_REQUIRE(dtype_from_odla(v.etype) != DT_INVALID, "value %d has element type %d", v.index, (int)v.etype);
+    LOADED_REQUIRE(v.shape.rank >= 1, "value %d has rank %d", v.index, v.shape.rank);
+    for (int i = 0; i < v.shape.rank; ++i)
+      LOADED_REQUIRE(v.shape.d[i] > 0 && v.shape.d[i] < (1ll << 40), "value %d has extent %lld", v.index, (long long)v.shape.d[i]);
+    LOADED_REQUIRE(v.shape.numel() < (1ll << 48), "value %d is implausibly large", v.index);
+    if (v.kind == _odla_value::TEMP) {
+      LOADED_REQUIRE(v.producer >= 0 && v.producer < nn, "value %d names producer %d", v.index, v.producer);
+      const Node& p = c->nodes[(size_t)v.producer];
+      LOADED_REQUIRE(p.out == &v || p.out2 == &v, "value %d is not a result of its producer", v.index);
+    } else {
+      LOADED_REQUIRE(v.producer == -1, "argument / constant %d has a producer", v.index);
+    }
+  }
+  for (const _odla_value* v : c->args) LOADED_REQUIRE(v->kind == _odla_value::ARG, "argument list names value %d", v->index);
+  for (int64_t k = 0; k < nn; ++k) {
+    const Node& n = c->nodes[(size_t)k];
+    OpRule r;
+    LOADED_REQUIRE(op_rule(n.op, &r), "node %lld has operator %d", (long long)k, (int)n.op);
+    const char* name = op_name(n.op);
+    const int nin = (int)n.in.size();
+    LOADED_REQUIRE(nin >= r.min_in && nin <= r.max_in, "%s node %lld has %d operand slots", name, (long long)k, nin);
+    for (int i = 0; i < nin; ++i) {
+      const _odla_value* v = n.in[(size_t)i];
+      if (v == nullptr) {
+        LOADED_REQUIRE(i >= 32 || !((r.required >> i) & 1u), "%s node %lld lacks operand %d", name, (long long)k, i);
+        continue;
+      }
+      // operands are defined before their use
+      LOADED_REQUIRE(v->kind != _odla_value::TEMP || v->producer < k, "%s node %lld uses value %d before it is computed",
+                     name, (long long)k, v->index);
+    }
+    LOADED_REQUIRE(n.out != nullptr && n.out->kind == _odla_value::TEMP && n.out->producer == k,
+                   "%s node %lld: result does not point back at it", name, (long long)k);
+    LOADED_REQUIRE(!r.out2 || (n.out2 != nullptr && n.out2->kind == _odla_value::TEMP && n.out2->producer == k),
+                   "%s node %lld lacks its second result", name, (long long)k);
+    const _odla_value* x = n.in[0];
+    const int xr = x->shape.rank, orank = n.out->shape.rank;
+    const size_t niv = n.iv.size();
+    switch (n.op) {
+      case OP_CONV:
+        LOADED_REQUIRE(xr == 4 && n.in[1]->shape.rank == 4 && orank == 4, "Conv node %lld: operands must have rank 4", (long long)k);
+        LOADED_REQUIRE(n.i[1] >= 1 && n.i[3] >= 1 && n.i[4] >= 1 && n.i[5] >= 1 && n.i[6] >= 1 && n.i[7] >= 0 &&
+                       n.i[8] >= 0 && n.i[9] >= 0 && n.i[10] >= 0, "Conv node %lld: bad stride / dilation / padding / group", (long long)k);
+        LOADED_REQUIRE(n.i[0] >= ODLA_CHANNELS_FIRST && n.i[0] <= ODLA_CHANNELS_LAST && n.i[2] >= ODLA_SIO && n.i[2] <= ODLA_IOS,
+                       "Conv node %lld: bad layout", (long long)k);
+        break;
+      case OP_GEMM:
+        LOADED_REQUIRE(xr >= 2 && n.in[1]->shape.rank >= 2, "Gemm node %lld: operands must have rank >= 2", (long long)k);
+        break;
+      case OP_BINARY:
+        LOADED_REQUIRE(n.i[0] >= BIN_ADD && n.i[0] <= BIN_MIN, "Binary node %lld: kind %lld", (long long)k, (long long)n.i[0]);
+        LOADED_REQUIRE(niv >= 1 && n.iv[0] >= 1 && n.iv[0] <= ODLA_MAX_DIMENSION && niv == 1 + 2 * (size_t)n.iv[0] && n.iv[0] == orank,
+                       "Binary node %lld: aligned shapes are malformed", (long long)k);
+        for (size_t i = 1; i < niv; ++i) LOADED_REQUIRE(n.iv[i] >= 1, "Binary node %lld: aligned extent %lld", (long long)k, (long long)n.iv[i]);
+        break;
+      case OP_EWISE:
+        LOADED_REQUIRE(niv >= 1 && n.iv[0] == orank && niv == 1 + (size_t)nin * (size_t)orank, "Elementwise node %lld: aligned shapes are malformed", (long long)k);
+        for (size_t i = 1; i < niv; ++i) LOADED_REQUIRE(n.iv[i] >= 1, "Elementwise node %lld: aligned extent %lld", (long long)k, (long long)n.iv[i]);
+        break;
+      case OP_UNARY:
+        LOADED_REQUIRE(n.i[0] >= ACT_NONE && n.i[0] <= ACT_DIV_CONST, "Unary node %lld: kind %lld", (long long)k, (long long)n.i[0]);
+        break;
+      case OP_LAYERNORM:
+        LOADED_REQUIRE(n.i[0] >= 1 && n.i[0] <= xr, "LayerNorm node %lld: %lld axes", (long long)k, (long long)n.i[0]);
+        break;
+      case OP_POOL:
+        LOADED_REQUIRE(xr == 4 && orank == 4, "Pool node %lld: operands must have rank 4", (long long)k);
+        LOADED_REQUIRE(n.i[2] >= 1 && n.i[3] >= 1 && n.i[4] >= 1 && n.i[5] >= 1 && n.i[6] >= 0 && n.i[7] >= 0 && n.i[8] >= 0 && n.i[9] >= 0,
+                       "Pool node %lld: bad window / stride / padding", (long long)k);
+        break;
+      case OP_REDUCE:
+        LOADED_REQUIRE(niv >= 1 && niv <= (size_t)xr, "Reduce node %lld: %zu axes", (long long)k, niv);
+        for (int64_t a : n.iv) LOADED_REQUIRE(a >= 0 && a < xr, "Reduce node %lld: axis %lld", (long long)k, (long long)a);
+        break;
+      case OP_SOFTMAX:
+        LOADED_REQUIRE(n.i[0] >= -xr && n.i[0] < xr, "Softmax node %lld: axis %lld", (long long)k, (long long)n.i[0]);
+        break;
+      case OP_CONCAT:
+        LOADED_REQUIRE(n.i[0] >= 0 && n.i[0] < xr, "Concat node %lld: axis %lld", (long long)k, (long long)n.i[0]);
+        for (const _odla_value* v : n.in) LOADED_REQUIRE(v->shape.rank == xr, "Concat node %lld: operands of different rank", (long long)k);
+        break;
+      case OP_GATHER:
+      case OP_ARGEXT:
+        LOADED_REQUIRE(n.i[n.op == OP_ARGEXT ? 1 : 0] >= 0 && n.i[n.op == OP_ARGEXT ? 1 : 0] < xr, "%s node %lld: axis out of range", name, (long long)k);
+        break;
+      case OP_RESHAPE:
+        LOADED_REQUIRE(x->shape.numel() == n.out->shape.numel(), "Reshape node %lld changes the element count", (long long)k);
+        break;
+      case OP_RESIZE:
+      case OP_LRN:
+        LOADED_REQUIRE(xr == 4 && orank == 4, "%s node %lld: operands must have rank 4", name, (long long)k);
+        break;
+      case OP_SLICE:
+        LOADED_REQUIRE(niv == 3 * (size_t)xr && orank == xr, "Slice node %lld: malformed bounds", (long long)k);
+        for (int i = 0; i < xr; ++i)
+          LOADED_REQUIRE(n.iv[i] >= 0 && n.iv[i] < n.iv[xr + i] && n.iv[xr + i] <= x->shape.d[i] && n.iv[2 * xr + i] >= 1,
+                         "Slice node %lld: bounds outside the operand along dim %d", (long long)k, i);
+        break;
+      case OP_TRANSPOSE: {
+        LOADED_REQUIRE(niv == (size_t)xr && orank == xr, "Transpose node %lld: malformed permutation", (long long)k);
+        unsigned seen = 0;
+        for (int64_t a : n.iv) {
+          LOADED_REQUIRE(a >= 0 && a < xr && !((seen >> a) & 1u), "Transpose node %lld: not a permutation", (long long)k);
+          seen |= 1u << a;
+        }
+        break;
+      }
+      case OP_QUANTIZE:
+      case OP_DEQUANTIZE:
+        LOADED_REQUIRE(n.i[0] >= -xr && n.i[0] < xr, "%s node %lld: axis %lld", name, (long long)k, (long long)n.i[0]);
+        break;
+      case OP_NMS:
+        LOADED_REQUIRE(xr == 3 && n.in[1]->shape.rank == 3 && x->shape.d[2] == 4 && n.i[0] >= 0, "NMS node %lld: malformed operands", (long long)k);
+        break;
+      case OP_COPYND: {
+        LOADED_REQUIRE(niv >= 1 && n.iv[0] >= 1 && n.iv[0] <= ODLA_MAX_DIMENSION && niv == 3 + 3 * (size_t)n.iv[0],
+                       "CopyND node %lld: malformed extents", (long long)k);
+        // every element the copy touches lies inside its operand / result
+        const int r0 = (int)n.iv[0];
+        int64_t xmax = n.iv[1 + 3 * r0], ymax = n.iv[2 + 3 * r0];
+        LOADED_REQUIRE(xmax >= 0 && ymax >= 0, "CopyND node %lld: negative offset", (long long)k);
+        for (int i = 0; i < r0; ++i) {
+          const int64_t d = n.iv[1 + i], sx = n.iv[1 + r0 + i], sy = n.iv[1 + 2 * r0 + i];
+          LOADED_REQUIRE(d >= 1 && d < (1ll << 40) && sx >= 0 && sy >= 0 && sx < (1ll << 40) && sy < (1ll << 40),
+                         "CopyND node %lld: bad extent or stride", (long long)k);
+          xmax += (d - 1) * sx;
+          ymax += (d - 1) * sy;
+        }
+        LOADED_REQUIRE(xmax < x->shape.numel() && ymax < n.out->shape.numel(), "CopyND node %lld reaches outside its tensors", (long long)k);
+        break;
+      }
+      case OP_TOPK:
+        LOADED_REQUIRE(n.i[2] >= 0 && n.i[2] < xr && n.i[0] >= 1 && n.i[0] <= x->shape.d[n.i[2]], "TopK node %lld: bad axis or K", (long long)k);
+        break;
+      default:
+        break;
+    }
+  }
+  for (const _odla_value* v : c->outputs) LOADED_REQUIRE(v != nullptr, "output list names a missing value");
+  return ODLA_SUCCESS;
+}
+
 odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) {
-  Reader r{data, size};
-  char magic[8];
-  if (!r.raw(magic, 8) || memcmp(magic, kMagic, 8) != 0) {
-    OHIP_ERR("not a stored computation (bad signature)");
+  if (size < 16 || data == nullptr || memcmp(data, kMagic, 8) != 0) {
+    OHIP_ERR("not a stored computation of this library version (bad signature)");
     return ODLA_INVALID_PARAM;
   }
+  uint64_t stored = 0;
+  memcpy(&stored, data + size - 8, 8);
+  if (stored != fnv1a(data, size - 8)) {
+    OHIP_ERR("stored computation is truncated or damaged (hash mismatch)");
+    return ODLA_INVALID_PARAM;
+  }
+  size -= 8;
+  Reader r{data, size};
+  char magic[8];
+  r.raw(magic, 8);
   Options& o = c->opts;
   o.fp16 = r.i64() != 0; o.bf16 = (odla_bf16_mode)r.i64(); o.int8 = r.i64() != 0; o.raw_acc = r.i64() != 0;
   c->dynamic_batch = r.i64() != 0;
@@ -192,11 +409,11 @@ odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) 
     if (!r.ok || n.out == nullptr) return ODLA_INVALID_PARAM;
     c->nodes.push_back(std::move(n));
   }
-  if (!r.ok) {
+  if (!r.ok || r.pos != r.n) {
     OHIP_ERR("stored computation is truncated or corrupt");
     return ODLA_INVALID_PARAM;
   }
-  return ODLA_SUCCESS;
+  return validate_loaded(c);
 }
 
 odla_status write_location(const odla_resource_location& loc, const std::vector<uint8_t>& bytes) {

@@ -38,6 +38,7 @@ ODLA_CHANNELS_FIRST, ODLA_CHANNELS_LAST, ODLA_SIO, ODLA_SOI, ODLA_OIS, ODLA_IOS 
 ODLA_NEAREST, ODLA_LINEAR, ODLA_CUBIC = range(3)
 ODLA_ASSYMMETRIC = 0
 ODLA_MEMCPY_H2H, ODLA_MEMCPY_H2D, ODLA_MEMCPY_D2H, ODLA_MEMCPY_D2D = range(4)
+ODLA_DEVICE_INFO_TOTAL_MEMORY, ODLA_DEVICE_INFO_USED_MEMORY = 7, 8
 
 ODLA_MAX_DIMENSION = 10
 ODLA_MAX_OUTPUTS = 64
@@ -296,10 +297,10 @@ def _check(st, what):
 class HipBuilder:
     """Builds an ODLA computation on libodla_hip.so; one method per operator."""
 
-    def __init__(self, fp16=False, bf16=False, quant_table=None, raw_acc=False, lib=None, max_batch=0):
+    def __init__(self, fp16=False, bf16=False, quant_table=None, raw_acc=False, lib=None, max_batch=0, min_batch=1):
         """max_batch > 0 records a dynamic-batch computation: arguments declared with a
         leading extent of -1 are planned at max_batch and a Session may run any
-        batch 1..max_batch (Session.set_batch)."""
+        batch min_batch..max_batch (Session.set_batch)."""
         self.L = lib or load_library()
         self.comp = ctypes.c_void_p()
         _check(self.L.odla_CreateComputation(ctypes.byref(self.comp)), "odla_CreateComputation")
@@ -307,7 +308,7 @@ class HipBuilder:
         if self.max_batch > 0:
             t = ctypes.c_bool(True)
             _check(self.L.odla_SetComputationItem(self.comp, ODLA_DYNAMIC_BATCH, ctypes.byref(t)), "DYNAMIC_BATCH")
-            for item, n in ((ODLA_MIN_BATCH_SIZE, 1), (ODLA_MAX_BATCH_SIZE, self.max_batch),
+            for item, n in ((ODLA_MIN_BATCH_SIZE, int(min_batch)), (ODLA_MAX_BATCH_SIZE, self.max_batch),
                             (ODLA_OPT_BATCH_SIZE, self.max_batch)):
                 v = ctypes.c_int(n)
                 _check(self.L.odla_SetComputationItem(self.comp, item, ctypes.byref(v)), "BATCH_SIZE item")
@@ -713,6 +714,21 @@ class Session:
         if self.ctx:
             self.L.odla_DestroyContext(self.ctx)
             self.ctx = None
+
+
+class ScalarValue(ctypes.Structure):
+    _fields_ = [("data_type", ctypes.c_int32), ("val_int64", ctypes.c_int64)]
+
+
+def used_device_memory(L=None):
+    """Bytes in use on the default device (odla_GetDeviceInfo, ODLA_DEVICE_INFO_USED_MEMORY)."""
+    L = L or load_library()
+    dev = ctypes.c_void_p()
+    _check(L.odla_AllocateDevice(None, 0, 0, ctypes.byref(dev)), "odla_AllocateDevice")
+    val = ScalarValue()
+    _check(L.odla_GetDeviceInfo(dev, ODLA_DEVICE_INFO_USED_MEMORY, ctypes.byref(val)), "odla_GetDeviceInfo")
+    L.odla_DestroyDevice(dev)
+    return int(val.val_int64)
 
 
 def quant_table(entries):

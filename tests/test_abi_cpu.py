@@ -131,6 +131,27 @@ def test_shape_inference_and_validation(odla):
     b.destroy()
 
 
+def test_operands_of_another_computation_are_refused(odla):
+    """A value of one computation is no operand in another: NULL and a log line, not an
+    index into the wrong value table."""
+    a = odla.HipBuilder()
+    xa = a.arg("x", (4, 8))                     # values are created in the calling thread's current computation
+    wa = a.const("w", np.zeros((8, 3), np.float32))
+    b = odla.HipBuilder()
+    xb = b.arg("x", (4, 8))
+    a.L.odla_SetLogLevel(0)
+    with pytest.raises(odla.OdlaError):
+        b.add(xb, xa)
+    with pytest.raises(odla.OdlaError):
+        b.concat([xb, xa], 0)
+    with pytest.raises(odla.OdlaError):
+        b.gemm(xb, wa, None)
+    a.L.odla_SetLogLevel(2)
+    assert b.shape_of(b.add(xb, xb))[0] == (4, 8)       # the computation itself still records
+    a.destroy()
+    b.destroy()
+
+
 def test_introspection_and_status_codes(odla):
     b = odla.HipBuilder()
     L = b.L

@@ -372,3 +372,75 @@ def test_bert_builder_recorded_with_a_dynamic_batch():
                 s.close()
         finally:
             hb.destroy()
+
+
+def test_many_batch_sizes_keep_device_memory_bounded():
+    """A server that sweeps the batch must not pile up one planned copy of the weights
+    per batch: a context keeps at most four batches planned (ODLA_HIP_MAX_BATCH_VARIANTS),
+    the one used longest ago goes first, and a batch that was dropped runs again -
+    rebuilt - with the same result.  The weights here are 16 MiB; 31 copies would be
+    about 500 MiB."""
+    odla = entry.load().odla
+    r = np.random.default_rng(21)
+    wf = (r.standard_normal((2048, 2048)) * 0.02).astype(np.float32)
+    MAXB = 32
+
+    def graph(batch):
+        def build(b):
+            x = b.arg("x", (batch, 2048))
+            b.output(b.relu(b.gemm(x, b.const("wf", wf), name="fc"), name="y"), "y")
+        return build
+
+    hb = odla.HipBuilder(max_batch=MAXB)
+    try:
+        graph(-1)(hb)
+        s = hb.session(True)
+        try:
+            x = r.standard_normal((MAXB, 2048)).astype(np.float32)
+            want = run_ref(graph(MAXB), {"x": x})["y"]
+            first = {}
+            used = []
+            for sweep in range(2):
+                for bs in range(1, MAXB + 1):
+                    if bs % 8 == 1:
+                        announce("batch sweep %d: batch %d" % (sweep, bs))
+                    s.set_batch(bs)
+                    got = s.run({"x": x[:bs]})["y"]
+                    assert max_rel_err(got, want[:bs]) <= 1e-4, bs
+                    if sweep == 0:
+                        first[bs] = got
+                    else:
+                        assert np.array_equal(got, first[bs]), bs      # the rebuilt plan computes the same
+                    used.append(odla.used_device_memory())
+            growth = max(used) - used[4]    # from the point where the four slots are taken
+            announce("device memory over 64 batch changes: %.1f MiB at the start, largest %.1f MiB"
+                     % (used[4] / 2 ** 20, max(used) / 2 ** 20))
+            assert growth <= 64 * 2 ** 20, growth
+        finally:
+            s.close()
+    finally:
+        hb.destroy()
+
+
+def test_batches_below_the_smallest_are_refused():
+    """ODLA_MIN_BATCH_SIZE bounds the run-time batch from below."""
+    odla = entry.load().odla
+    w = cnn_weights(9)
+    hb = odla.HipBuilder(max_batch=8, min_batch=4)
+    try:
+        build_cnn(w, -1)(hb)
+        s = hb.session(True)
+        try:
+            announce("dynamic batch: below ODLA_MIN_BATCH_SIZE")
+            for bs in (1, 3):
+                with pytest.raises(odla.OdlaError):
+                    s.set_batch(bs)
+            s.set_batch(4)
+            x = np.random.default_rng(10).standard_normal((4, 3, 20, 20)).astype(np.float32)
+            got = s.run({"x": x})
+            want = run_ref(build_cnn(w, 4), {"x": x})
+            assert np.max(np.abs(got["prob"] - want["prob"])) <= 1e-5
+        finally:
+            s.close()
+    finally:
+        hb.destroy()

@@ -132,6 +132,12 @@ def test_two_contexts_and_error_paths(models, odla):
     s3 = hb.session()
     st = L.odla_ExecuteComputation(hb.comp, s3.ctx, odla.ODLA_COMPUTE_INFERENCE, None)
     assert st == odla.ODLA_INVALID_PARAM  # argument not bound
+    # a compiled computation with contexts takes no further operators: they could not run
+    L.odla_SetLogLevel(0)
+    with pytest.raises(odla.OdlaError):
+        hb.relu(hb.outs["y"][0], name="late")
+    L.odla_SetLogLevel(2)
+    assert np.array_equal(s1.run(feeds)["y"], a)
     for s in (s1, s2, s3):
         s.close()
     hb.destroy()
