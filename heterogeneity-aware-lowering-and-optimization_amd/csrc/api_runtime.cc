@@ -176,9 +176,9 @@ void drop_graph(_odla_context* ctx) {
   if (ctx->graph) { (void)hipGraphDestroy(ctx->graph); ctx->graph = nullptr; }
 }
 
-odla_status run_steps(_odla_context* ctx, const Plan& plan) {
+odla_status run_steps(_odla_context* ctx, const Plan& plan, char* arena) {
   ExecEnv env;
-  env.base[SP_ARENA] = ctx->arena;
+  env.base[SP_ARENA] = arena;
   env.base[SP_CONST] = plan.const_pool;
   for (const Step& s : plan.steps) {
     hipError_t e = s.fn(env, ctx->stream);
@@ -190,18 +190,38 @@ odla_status run_steps(_odla_context* ctx, const Plan& plan) {
   return ODLA_SUCCESS;
 }
 
-odla_status stage_inputs(_odla_context* ctx, const Plan& plan) {
+odla_status stage_inputs(_odla_context* ctx, const Plan& plan, char* arena) {
   for (const Plan::IO& io : plan.inputs) {
     auto it = ctx->bound_in.find(io.v);
     if (it == ctx->bound_in.end()) {
       OHIP_ERR("argument '%s' is not bound", io.v->name.c_str());
       return ODLA_INVALID_PARAM;
     }
-    char* dst = ctx->arena + plan.tensors[io.tensor].offset;
+    char* dst = arena + plan.tensors[io.tensor].offset;
     if (hipMemcpyAsync(dst, it->second, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
       OHIP_ERR("copy of argument '%s' failed", io.v->name.c_str());
       return ODLA_FAILURE;
     }
+  }
+  return ODLA_SUCCESS;
+}
+
+// Copies the bound results out of `arena` (or the constant pool) and waits for the stream.
+odla_status fetch_outputs(_odla_context* ctx, const Plan& plan, const char* arena) {
+  for (const Plan::IO& io : plan.outputs) {
+    auto it = ctx->bound_out.find(io.v);
+    if (it == ctx->bound_out.end()) continue;
+    const PTensor& t = plan.tensors[io.tensor];
+    const char* src = (t.space == SP_CONST ? plan.const_pool : arena) + t.offset + io.offset;
+    if (hipMemcpyAsync(it->second, src, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
+      OHIP_ERR("copy of output '%s' failed", io.v->name.c_str());
+      return ODLA_FAILURE;
+    }
+  }
+  hipError_t e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) {
+    OHIP_ERR("device error: %s", hipGetErrorString(e));
+    return ODLA_FAILURE;
   }
   return ODLA_SUCCESS;
 }
@@ -423,6 +443,12 @@ odla_status create_context_for(_odla_computation* c, odla_context* context) {
       return ODLA_MEM_ERROR;
     }
   }
+  // set-up for odla_hip_ExecuteComputationStatic: resolve this device's copy of the static
+  // scratch now, so that the entry point itself only reads the cached address
+  {
+    void* base = nullptr;
+    if (static_arena(&base, nullptr) != hipSuccess) OHIP_WARN("odla_CreateContext: the static scratch could not be resolved");
+  }
   *context = ctx.release();
   return ODLA_SUCCESS;
 }
@@ -562,7 +588,7 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
 
   // 1. stage arguments (host -> device across PCIe, or device -> device)
   {
-    odla_status st = stage_inputs(ctx, plan);
+    odla_status st = stage_inputs(ctx, plan, ctx->arena);
     if (st != ODLA_SUCCESS) return st;
   }
 
@@ -573,7 +599,7 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
         OHIP_ERR("odla_ExecuteComputation: hipStreamBeginCapture failed");
         return ODLA_FAILURE;
       }
-      odla_status st = run_steps(ctx, plan);
+      odla_status st = run_steps(ctx, plan, ctx->arena);
       hipGraph_t g = nullptr;
       hipError_t e = hipStreamEndCapture(ctx->stream, &g);
       if (st != ODLA_SUCCESS || e != hipSuccess || g == nullptr) {
@@ -593,29 +619,64 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
       return ODLA_FAILURE;
     }
   } else {
-    odla_status st = run_steps(ctx, plan);
+    odla_status st = run_steps(ctx, plan, ctx->arena);
     if (st != ODLA_SUCCESS) return st;
   }
 
   // 3. results
-  for (const Plan::IO& io : plan.outputs) {
-    auto it = ctx->bound_out.find(io.v);
-    if (it == ctx->bound_out.end()) continue;
-    const PTensor& t = plan.tensors[io.tensor];
-    const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset + io.offset;
-    if (hipMemcpyAsync(it->second, src, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
-      OHIP_ERR("odla_ExecuteComputation: copy of output '%s' failed", io.v->name.c_str());
-      return ODLA_FAILURE;
-    }
-  }
-  hipError_t e = hipStreamSynchronize(ctx->stream);
-  if (e != hipSuccess) {
-    OHIP_ERR("odla_ExecuteComputation: device error: %s", hipGetErrorString(e));
-    return ODLA_FAILURE;
-  }
+  odla_status st = fetch_outputs(ctx, plan, ctx->arena);
+  if (st != ODLA_SUCCESS) return st;
   ctx->executed = true;
   if (!plan.stat_recs.empty()) return profiler_collect(plan, ctx->arena);
   return ODLA_SUCCESS;
+}
+
+static_assert(kStaticArenaBytes == ODLA_HIP_STATIC_SCRATCH_BYTES, "the header states the size of the static scratch");
+
+// odla_ExecuteComputation for callers that must not allocate device memory.
+// The plan's temporaries live in the library's static device scratch instead
+// of the context's arena, and the launch sequence runs un-captured (building a
+// hipGraph allocates), so the call performs no hipMalloc / hipFree.  The
+// context supplies the stream and the bindings; its own arena is not touched.
+odla_status odla_hip_ExecuteComputationStatic(odla_computation comp, odla_context ctx,
+                                              const odla_compute_mode mode, odla_device device) {
+  (void)device;
+  if (ctx == nullptr) return ODLA_INVALID_PARAM;
+  if (comp != nullptr && comp != ctx->comp) {
+    OHIP_ERR("odla_hip_ExecuteComputationStatic: context belongs to another computation");
+    return ODLA_INVALID_PARAM;
+  }
+  if (mode == ODLA_COMPUTE_TRAINING) return ODLA_UNSUPPORTED_OP;
+  _odla_computation* c = ctx->comp;
+  if (ctx->run_batch > 0 && ctx->run_batch != recorded_batch(*c)) {
+    // another batch runs a copy of the recording that is planned on first use: that allocates
+    OHIP_ERR("odla_hip_ExecuteComputationStatic: runs the recorded batch only (context is set to batch %d)", ctx->run_batch);
+    return ODLA_UNSUPPORTED_OP;
+  }
+  if (!c->plan) return ODLA_FAILURE;
+  const Plan& plan = *c->plan;
+  if (!plan.stat_recs.empty()) {
+    OHIP_ERR("odla_hip_ExecuteComputationStatic: calibration plans are not supported");
+    return ODLA_UNSUPPORTED_OP;
+  }
+  void* base = nullptr;
+  size_t cap = 0;
+  hipError_t e = static_arena(&base, &cap);
+  if (e != hipSuccess) {
+    OHIP_ERR("odla_hip_ExecuteComputationStatic: static scratch unavailable: %s", hipGetErrorString(e));
+    return ODLA_FAILURE;
+  }
+  if (plan.arena_bytes > cap) {
+    OHIP_ERR("odla_hip_ExecuteComputationStatic: the plan needs %zu bytes of temporaries, the static scratch holds %zu; "
+             "use odla_ExecuteComputation", plan.arena_bytes, cap);
+    return ODLA_MEM_ERROR;
+  }
+  char* arena = static_cast<char*>(base);
+  odla_status st = stage_inputs(ctx, plan, arena);
+  if (st != ODLA_SUCCESS) return st;
+  st = run_steps(ctx, plan, arena);
+  if (st != ODLA_SUCCESS) return st;
+  return fetch_outputs(ctx, plan, arena);
 }
 
 // Diagnostic: run the launch sequence un-captured `iters` times with a HIP
@@ -638,7 +699,7 @@ odla_status odla_hip_ProfileSteps(odla_context ctx, odla_int32 iters, odla_hip_s
   env.base[SP_CONST] = plan.const_pool;
   odla_status st = ODLA_SUCCESS;
   for (int it = 0; it < iters && st == ODLA_SUCCESS; ++it) {
-    st = stage_inputs(ctx, plan);
+    st = stage_inputs(ctx, plan, ctx->arena);
     for (int i = 0; i < n && st == ODLA_SUCCESS; ++i) {
       (void)hipEventRecord(ev[2 * i], ctx->stream);
       if (plan.steps[i].fn(env, ctx->stream) != hipSuccess) st = ODLA_FAILURE;

@@ -11,6 +11,14 @@
 
 namespace ohip {
 
+// Size of the statically allocated device scratch behind
+// odla_hip_ExecuteComputationStatic (kernels/static_arena.hip): plans whose
+// temporaries need more are refused by that entry point.
+constexpr size_t kStaticArenaBytes = 64u << 20;
+// Address (on the calling thread's current device) and size of that scratch.
+// Allocates nothing; the first call on a device resolves the symbol.
+hipError_t static_arena(void** ptr, size_t* bytes);
+
 // Storage types of device tensors.
 enum DType : int {
   DT_F32 = 0,

@@ -150,6 +150,7 @@ def load_library(path=None):
     proto("odla_BindToOutput", i32, [vp, vp, vp])
     proto("odla_BindToOutputById", i32, [cid, vp, vp])
     proto("odla_ExecuteComputation", i32, [vp, vp, i32, vp])
+    proto("odla_hip_ExecuteComputationStatic", i32, [vp, vp, i32, vp])
     proto("odla_GetNumOfArgsFromComputation", i32, [vp, pu32])
     proto("odla_GetArgFromComputationByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
     proto("odla_GetNumOfOutputsFromComputation", i32, [vp, pu32])
@@ -698,6 +699,11 @@ class Session:
 
     def execute(self):
         _check(self.L.odla_ExecuteComputation(self.b.comp, self.ctx, ODLA_COMPUTE_INFERENCE, None), "odla_ExecuteComputation")
+
+    def execute_static(self):
+        """The same step through the entry point that allocates nothing (temporaries in the
+        library's static device scratch); returns the status code."""
+        return self.L.odla_hip_ExecuteComputationStatic(self.b.comp, self.ctx, ODLA_COMPUTE_INFERENCE, None)
 
     def fetch_device_outputs(self):
         outs = {}

@@ -854,6 +854,35 @@ odla_status odla_hip_ProfileSteps(odla_context context, odla_int32 iters,
                                   odla_hip_step_time* out, odla_int32 capacity,
                                   odla_int32* count);
 
+/* ------------------------------------------------------------------------ */
+/* Execution without device-memory allocation.                               */
+/* No counterpart in the reference.  For callers that cannot allocate device */
+/* memory while they run: code under HIP graph capture, tight serving loops, */
+/* harnesses that forbid hipMalloc.                                          */
+/* ------------------------------------------------------------------------ */
+/* Temporaries larger than this are refused (ODLA_MEM_ERROR). */
+#define ODLA_HIP_STATIC_SCRATCH_BYTES (64u << 20)
+
+/* odla_ExecuteComputation with the plan's temporaries placed in a statically
+ * allocated device buffer of ODLA_HIP_STATIC_SCRATCH_BYTES (one per GPU, held
+ * from the library's load to the end of the process) instead of the context's
+ * arena, and the launch sequence issued directly on the context's stream (no
+ * hipGraph is built).  The call performs no hipMalloc / hipFree and calls no
+ * allocating library routine; bind device pointers for arguments and outputs
+ * so that the copies in and out are device-to-device.  `context` comes from
+ * odla_CreateContext as usual (created ahead of time; it supplies the stream
+ * and the bindings) and must run the recorded batch.  Results are delivered
+ * through bound outputs only (odla_GetValueData reads a context's own arena).
+ * Returns ODLA_MEM_ERROR when the plan's temporaries exceed the buffer,
+ * ODLA_UNSUPPORTED_OP for another run-time batch or a calibration plan.
+ * All calls on one GPU share that GPU's buffer, which keeps the previous
+ * call's contents (no launch relies on them): calls that overlap in time on
+ * one GPU race and must be serialised by the caller. */
+odla_status odla_hip_ExecuteComputationStatic(odla_computation computation,
+                                              odla_context context,
+                                              odla_compute_mode mode,
+                                              odla_device device);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif
