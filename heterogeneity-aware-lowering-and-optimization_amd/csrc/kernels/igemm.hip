@@ -19,7 +19,7 @@
 // of four consecutive output channels, which is what a channels-last store
 // wants.  Both operands use the same k -> (lane group, element) assignment, so
 // the exact k permutation inside one MFMA is irrelevant to the result.
-#include "device_utils.h"
+#include "igemm_common.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -28,419 +28,91 @@
 
 namespace ohip {
 
-// n / d for 0 <= n < 2^31 with the divisor's magic pair (see div_magic on the
-// host side): three instructions instead of the ~35 of a 32-bit division.
-__device__ __forceinline__ int fast_div(int n, unsigned magic, int shift) {
-  return (int)(__umulhi((unsigned)n << 1, magic) >> shift);
-}
-
-template <typename T> struct Mma;
-template <> struct Mma<float> {
-  using Acc = floatx16;
-  __device__ static __forceinline__ Acc run(uintx4 a, uintx4 b, Acc c) {
-    // 16 bytes = 4 k values per lane; 32x32x2 consumes one per lane group.
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
-    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
-    return c;
-  }
-};
-template <> struct Mma<f16_t> {
-  using Acc = floatx16;
-  __device__ static __forceinline__ Acc run(uintx4 a, uintx4 b, Acc c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a),
-                                                  __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma<bf16_t> {
-  using Acc = floatx16;
-  __device__ static __forceinline__ Acc run(uintx4 a, uintx4 b, Acc c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma<int8_t> {
-  using Acc = intx16;
-  __device__ static __forceinline__ Acc run(uintx4 a, uintx4 b, Acc c) {
-    return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a),
-                                                 __builtin_bit_cast(intx4, b), c, 0, 0, 0);
-  }
-};
-
 // ---------------------------------------------------------------------------
-// Epilogues.  Each handles eight consecutive output channels n..n+7 of one
-// output row; yrow / rrow / bias already point at channel n.  `vec` says all
-// eight are valid and the row pointers allow one vector access.
-
-// Only the cheap activations are fused (a full transcendental switch inlined
-// per element bloats the epilogue until the compiler stops unrolling it and
-// the accumulators fall out of registers); the planner keeps the others as a
-// separate streaming kernel.
-__device__ __forceinline__ float epi_act(float v, ActKind act, float a, float b) {
-  switch (act) {
-    case ACT_RELU: return v > 0.f ? v : 0.f;
-    case ACT_LEAKY: return v > 0.f ? v : a * v;
-    case ACT_CLAMP: return fminf(fmaxf(v, a), b);
-    default: return v;
-  }
-}
-// Eight values at once: the (wavefront-uniform) switch is taken once, not per
-// element - per element it compiles to a tree of scalar branches that costs
-// more than the arithmetic of the whole epilogue.
-template <bool kRich = false>
-__device__ __forceinline__ void epi_act8(float (&v)[8], ActKind act, float a, float b) {
-  if constexpr (kRich) {
-    // Variant with the transcendental activations (GELU behind a feed-forward
-    // GEMM, Sigmoid / Tanh gates): a separate instantiation, so that the common
-    // epilogue stays small.
-    // (one element after the other: interleaving eight polynomial evaluations
-    // would take the registers the accumulators of the other slices live in)
-    switch (act) {
-      case ACT_GELU_ERF:
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { v[e] = gelu_erf(v[e]); __builtin_amdgcn_sched_barrier(0); }
-        return;
-      case ACT_GELU_TANH:
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { v[e] = gelu_tanh(v[e]); __builtin_amdgcn_sched_barrier(0); }
-        return;
-      case ACT_SIGMOID:
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { v[e] = 1.0f / (1.0f + expf(-v[e])); __builtin_amdgcn_sched_barrier(0); }
-        return;
-      case ACT_TANH:
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { v[e] = tanhf(v[e]); __builtin_amdgcn_sched_barrier(0); }
-        return;
-      default: break;
-    }
-  }
-  switch (act) {
-    case ACT_RELU:
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = v[e] > 0.f ? v[e] : 0.f;
-      break;
-    case ACT_LEAKY:
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = v[e] > 0.f ? v[e] : a * v[e];
-      break;
-    case ACT_CLAMP:
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = fminf(fmaxf(v[e], a), b);
-      break;
-    default: break;
-  }
-}
-
-template <typename TOut, bool kRich = false>
-struct EpiFloat {
-  using AccE = float;
-  using RVec = uintx4;  // eight 2-byte residual elements fetched ahead of use
-  static constexpr bool kPrefetchResidual = sizeof(TOut) == 2;
-  // b8: this lane's eight bias values (zero when absent); rpre: residual vector
-  // fetched ahead (valid when have_rpre), otherwise r points at the residual row.
-  __device__ static __forceinline__ void store8(const IgemmParams& p, const float* acc, int nvalid, bool vec,
-                                                const float* b8, const float*, TOut* y, const TOut* r,
-                                                bool have_rpre, RVec rpre) {
-    float v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(acc[e], p.alpha, b8[e]);
-    // the activation comes before the residual in networks whose shortcut joins
-    // an already activated branch, behind it in the ResNet order
-    if (p.res_after_act) epi_act8<kRich>(v, p.act, p.act_a, p.act_b);
-    if (vec) {
-      if (r != nullptr) {
-        if constexpr (sizeof(TOut) == 4) {
-          const floatx4 r0 = *reinterpret_cast<const floatx4*>(r);
-          const floatx4 r1 = *reinterpret_cast<const floatx4*>(r + 4);
-          v[0] += r0.x; v[1] += r0.y; v[2] += r0.z; v[3] += r0.w;
-          v[4] += r1.x; v[5] += r1.y; v[6] += r1.z; v[7] += r1.w;
-        } else {
-          Vec16<TOut> rv;
-          if (have_rpre) rv.raw = rpre; else rv.load(r);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] += rv.get(e);
-        }
-      }
-      if (!p.res_after_act) epi_act8<kRich>(v, p.act, p.act_a, p.act_b);
-      if constexpr (sizeof(TOut) == 4) {
-        *reinterpret_cast<floatx4*>(y) = (floatx4){v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<floatx4*>(y + 4) = (floatx4){v[4], v[5], v[6], v[7]};
-      } else {
-        Vec16<TOut> o;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o.set(e, v[e]);
-        // (not in the instantiations with the wider activation set: they have no registers to spare)
-        if (!kRich && p.stream_out) {
-          // The pointer passes through an empty asm so that the optimizer cannot
-          // fold this store and the plain one below into one plain store.
-          uintx4* yv = reinterpret_cast<uintx4*>(y);
-          asm volatile("" : "+v"(yv));
-          __builtin_nontemporal_store(o.raw, (__attribute__((address_space(1))) uintx4*)yv);
-        } else {
-          o.store(y);
-        }
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (e < nvalid && r != nullptr) v[e] += Store<TOut>::ld(r + e);
-      if (!p.res_after_act) epi_act8<kRich>(v, p.act, p.act_a, p.act_b);
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (e < nvalid) Store<TOut>::st(y + e, v[e]);
-    }
-  }
-};
-
-// int8 operands, int32 accumulators.  MODE 0: requantised 8-bit output (stored
-// q-128), MODE 1: dequantised fp32 output, MODE 2: raw int32 accumulators.
-template <int MODE> struct QuantOut;
-template <> struct QuantOut<0> { using T = int8_t; };
-template <> struct QuantOut<1> { using T = float; };
-template <> struct QuantOut<2> { using T = int; };
-
-template <int MODE>
-struct EpiQuant {
-  using AccE = int;
-  using TOut = typename QuantOut<MODE>::T;
-  using RVec = uintx2;  // eight 1-byte residual levels fetched ahead of use
-  static constexpr bool kPrefetchResidual = MODE == 0;
-  __device__ static __forceinline__ void store8(const IgemmParams& p, const int* acc, int nvalid, bool vec,
-                                                const int* b8, const float* m8, TOut* y, const TOut* r,
-                                                bool have_rpre, RVec rpre) {
-    if constexpr (MODE == 0) {
-      // Levels are carried as floats (small integers are exact): per element
-      //   t  = rne(float(acc + bias) * M)          add, cvt, mul, rndne
-      //   q  = med3(t + zp, lo, 255)               add, med3
-      // and with a fused residual (dequantise, add, requantise, as the unfused
-      // kernels do it)
-      //   f  = (q - zp) * s_q + (r - zp_r) * s_r   sub, mul, cvt_ubyte, sub, mul, add
-      //   q  = med3(rne(f * (1/s_out)) + zp_out, lo_out, 255)
-      // v_cvt_pk_u8_f32 packs a level into its byte; stored bytes are level - 128,
-      // i.e. level ^ 0x80.  Beyond 2^24 the float sums are inexact but far outside
-      // the clamp range on the same side, so the result is the same as in integers.
-      unsigned rw[2] = {0u, 0u};
-      if (r != nullptr) {
-        if (vec) {
-          const uintx2 rv = have_rpre ? rpre : *reinterpret_cast<const uintx2*>(r);
-          rw[0] = rv.x;
-          rw[1] = rv.y;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (e < nvalid) rw[e >> 2] |= (unsigned)(uint8_t)r[e] << (8 * (e & 3));
-        }
-        rw[0] ^= 0x80808080u;  // stored -> levels
-        rw[1] ^= 0x80808080u;
-      }
-      const float zp = (float)p.q_zp, lo = (float)p.q_lo;
-      const float rzp = (float)p.r_zp, szp = (float)p.s_zp, slo = (float)p.s_lo;
-      unsigned ow[2] = {0u, 0u};
-      if (r != nullptr) {
-        // q - zp = med3(t + zp, lo, 255) - zp = med3(t, lo - zp, 255 - zp): all integers
-        const float ulo = lo - zp, uhi = 255.f - zp;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float t = rintf((float)(acc[e] + b8[e]) * m8[e]);
-          const float fa = __builtin_amdgcn_fmed3f(t, ulo, uhi) * p.q_scale;
-          const float fb = ((float)((rw[e >> 2] >> (8 * (e & 3))) & 0xffu) - rzp) * p.r_scale;
-          const float f = fa + fb;
-          const float q = __builtin_amdgcn_fmed3f(rintf(f * p.s_inv) + szp, slo, 255.f);
-          ow[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(q, e & 3, ow[e >> 2]);
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float t = rintf((float)(acc[e] + b8[e]) * m8[e]);
-          const float q = __builtin_amdgcn_fmed3f(t + zp, lo, 255.f);
-          ow[e >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(q, e & 3, ow[e >> 2]);
-        }
-      }
-      ow[0] ^= 0x80808080u;  // levels -> stored
-      ow[1] ^= 0x80808080u;
-      if (vec) {
-        if (p.stream_out) {
-          uintx2* yv = reinterpret_cast<uintx2*>(y);
-          asm volatile("" : "+v"(yv));  // see EpiFloat::store8
-          __builtin_nontemporal_store((uintx2){ow[0], ow[1]}, (__attribute__((address_space(1))) uintx2*)yv);
-        } else {
-          *reinterpret_cast<uintx2*>(y) = (uintx2){ow[0], ow[1]};
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) y[e] = (int8_t)(ow[e >> 2] >> (8 * (e & 3)));
-      }
-    } else {
-      if constexpr (MODE == 2) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) y[e] = acc[e] + b8[e];
-      } else {
-        float f[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          f[e] = (float)(acc[e] + b8[e]) * m8[e];
-          if (e < nvalid && r != nullptr) f[e] += r[e];
-        }
-        epi_act8(f, p.act, p.act_a, p.act_b);
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) y[e] = f[e];
-      }
-    }
-  }
-};
-
-template <typename Epi> struct EpiTraits;
-template <typename T, bool R> struct EpiTraits<EpiFloat<T, R>> { using TOut = T; static constexpr bool quant = false; static constexpr bool rich = R; };
-template <int M> struct EpiTraits<EpiQuant<M>> { using TOut = typename QuantOut<M>::T; static constexpr bool quant = true; static constexpr bool rich = false; };
-
-// ---------------------------------------------------------------------------
-// Epilogue shared by the kernels below: each wavefront parks one 32-pixel slice
-// of its accumulators in LDS (pixel-major, fp32 / int32), then every lane picks
-// eight consecutive output channels of one pixel, so that global stores and
-// residual loads are 16-byte vectors and consecutive lanes cover contiguous
-// memory.  `smem` is the K loop's buffer; it is reused once every wavefront of
-// the workgroup has left the loop.
-// kEnterBarrier = false: the caller's wavefronts never shared `smem` before
-// (each only ever touches its own staging slice); n_off shifts the channels
-// this call covers within the tile.
-template <typename TIn, typename Epi, int BM, int BN, int WM, int WN, bool kEnterBarrier = true>
-__device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int epi_vec,
-                                               typename Mma<TIn>::Acc (&acc)[WM / 32][WN / 32],
-                                               unsigned char* smem, const int tile_m, const int tile_n,
-                                               const int z, const int M, const int wave, const int lane,
-                                               const int n_off = 0) {
-  constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int EPI_PITCH = WN + 4;  // 4-byte words per staged pixel row
-  using AccE = typename Epi::AccE;
-  using TOut = typename EpiTraits<Epi>::TOut;
-  const int wm = wave % (BM / WM), wn = wave / (BM / WM);
+// The 8-bit form of the epilogue below (four wavefronts, each with all 128 pixels
+// of the tile and a 32-channel slice): every wavefront requantises its slice in
+// the accumulator layout and writes the dwords of its 32 channels into one
+// [32 pixels][128 channels] BYTE tile, side by side with the others; then each
+// of the 256 threads moves 16 consecutive channels of one pixel, i.e. one pass
+// covers the 32 x 128 tile with full 128-byte rows.  The residual tile takes the
+// same road in the other direction.  Two tile pairs alternate, so that a slice
+// needs one barrier between its phases and one before its tiles are reused.
+__device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[4][1],
+                                                          unsigned char* smem, const int tile_m, const int tile_n,
+                                                          const int z, const int M, const int wave, const int lane) {
+  constexpr int BM = 128, BN = 128, TM = 4;
+  constexpr int PITCH = BN + 16;  // bytes per staged pixel row
+  constexpr int TILE = 32 * PITCH;
+  const int tid = wave * 64 + lane;
   const int l32 = lane & 31, lg = lane >> 5;
+  const int n0 = tile_n * BN;
 
-  TOut* ybase = reinterpret_cast<TOut*>(p.y) + (int64_t)z * p.y_bs;
-  const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
-  const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
+  int8_t* ybase = reinterpret_cast<int8_t*>(p.y) + (int64_t)z * p.y_bs;
+  const int8_t* rbase = p.residual ? reinterpret_cast<const int8_t*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
+  const bool has_res = rbase != nullptr;
 
-  AccE* stage = reinterpret_cast<AccE*>(smem) + wave * (32 * EPI_PITCH);
-  constexpr int LPP = WN / 8;    // lanes per pixel row in the read-back
-  constexpr int PPP = 64 / LPP;  // pixels per read-back pass
-  const int rp = lane / LPP;     // pixel within a pass
-  const int c8 = (lane % LPP) * 8;
-  const int n = tile_n * BN + wn * WN + c8 + n_off;
-  int nvalid = p.Kout - n;
-  nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
-  const bool vec = (epi_vec & 1) && nvalid == 8;
+  const int rp = tid >> 3;         // pixel of the slice this thread moves
+  const int c16 = (tid & 7) * 16;  // ... and its 16 channels
+  int nvalid = p.Kout - (n0 + c16);
+  nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
+  const bool vec = (epi_vec & 2) && nvalid == 16;
 
-  // lane-constant epilogue operands: the lane's eight channels are the same in every pass
-  AccE b8[8];
-  float m8[8];
+  floatx4 mq[4];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) { b8[e] = 0; m8[e] = 0.f; }
-  if (nvalid > 0) {
-    if (bias != nullptr) {
-      if (vec) {
-        const intx4 t0 = *reinterpret_cast<const intx4*>(bias + n);
-        const intx4 t1 = *reinterpret_cast<const intx4*>(bias + n + 4);
-        __builtin_memcpy(&b8[0], &t0, 16);
-        __builtin_memcpy(&b8[4], &t1, 16);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) b8[e] = bias[n + e];
-      }
-    }
-    if constexpr (EpiTraits<Epi>::quant) {
-      if (p.qmul != nullptr) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) m8[e] = p.qmul[n + e];
-      }
-    }
-  }
+  for (int q = 0; q < 4; ++q) mq[q] = load_qmul4(p.qmul, n0 + wave * 32 + q * 8 + lg * 4, p.Kout);
 
-  // Residual vectors are requested one 32-pixel slice ahead of their use, so
-  // that their latency overlaps with the staging of the previous slice.
-  constexpr int NPASS = 32 / PPP;
-  using RVec = typename Epi::RVec;
-  const bool have_rpre = Epi::kPrefetchResidual && vec && rbase != nullptr;
-  auto rfetch = [&](const int i, RVec (&dst)[NPASS]) {
-#pragma unroll
-    for (int ps = 0; ps < NPASS; ++ps) {
-      const int m = tile_m * BM + wm * WM + i * 32 + ps * PPP + rp;
-      const int mc = m < M ? m : M - 1;
-      // read once by the whole launch: a non-temporal load leaves the cache lines to the operands that are re-read
-      dst[ps] = __builtin_nontemporal_load(reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n));
-    }
-  };
-  RVec rcur[NPASS], rnxt[NPASS];
-#pragma unroll
-  for (int ps = 0; ps < NPASS; ++ps) { rcur[ps] = RVec{}; rnxt[ps] = RVec{}; }
-  if constexpr (Epi::kPrefetchResidual) {
-    if (have_rpre) rfetch(0, rcur);
-  }
-
-  if constexpr (kEnterBarrier) __syncthreads();  // the K loop's LDS reads are done; the buffer becomes the staging area
+  // The residual rows of all four slices are requested ahead of the first barrier:
+  // one memory round trip per tile.
+  uintx4 rall[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    // park: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        AccE* dst = stage + l32 * EPI_PITCH + j * 32 + q * 8 + lg * 4;
-        if constexpr (sizeof(AccE) == 4 && !EpiTraits<Epi>::quant) {
-          *reinterpret_cast<floatx4*>(dst) =
-              (floatx4){acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
-        } else {
-          *reinterpret_cast<intx4*>(dst) =
-              (intx4){(int)acc[i][j][q * 4 + 0], (int)acc[i][j][q * 4 + 1], (int)acc[i][j][q * 4 + 2], (int)acc[i][j][q * 4 + 3]};
-        }
-      }
-    }
-    // Each wavefront only touches its own staging slice and its LDS operations
-    // complete in issue order, so a wavefront-scope fence (no workgroup barrier)
-    // orders the parking writes before the read-back.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if constexpr (Epi::kPrefetchResidual && TM > 1) {
-      if (have_rpre && i + 1 < TM) rfetch(i + 1, rnxt);
-    }
-#pragma unroll
-    for (int ps = 0; ps < NPASS; ++ps) {
-      const int pix = ps * PPP + rp;
-      const int m = tile_m * BM + wm * WM + i * 32 + pix;
-      AccE a8[8];
-      const AccE* src = stage + pix * EPI_PITCH + c8;
-      if constexpr (!EpiTraits<Epi>::quant) {
-        const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
-        const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
-        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-      } else {
-        const intx4 v0 = *reinterpret_cast<const intx4*>(src);
-        const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
-        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-      }
-      if (m < M && nvalid > 0) {
-        TOut* yrow = ybase + (int64_t)m * p.ycs + n;
-        const TOut* rrow = rbase ? rbase + (int64_t)m * p.rcs + n : nullptr;
-        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rcur[ps]);
-      }
-    }
-#pragma unroll
-    for (int ps = 0; ps < NPASS; ++ps) rcur[ps] = rnxt[ps];
-    if (i + 1 < TM) {
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    rall[i] = uintx4{0u, 0u, 0u, 0u};
+    if (has_res && nvalid > 0) {
+      const int m = tile_m * BM + i * 32 + rp;
+      const int mc = m < M ? m : M - 1;
+      rall[i] = load_row16(rbase + (int64_t)mc * p.rcs + n0 + c16, vec, nvalid);
     }
   }
+
+  // Workgroup barrier for LDS traffic only: the fence of __syncthreads would
+  // also wait for the global stores of the slices before.
+  auto lds_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0), other counters at their maxima
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
+  auto slice = [&](auto slice_no) __attribute__((always_inline)) {
+    constexpr int i = decltype(slice_no)::value;
+    unsigned char* otile = smem + (i & 1) * (2 * TILE);
+    unsigned char* rtile = otile + TILE;
+    if (has_res) {
+      *reinterpret_cast<uintx4*>(rtile + rp * PITCH + c16) = rall[i];
+      lds_barrier();
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int off = l32 * PITCH + wave * 32 + q * 8 + lg * 4;
+      const unsigned rs = has_res ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
+      const unsigned w = requant4(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3],
+                                  mq[q], has_res, rs, p);
+      *reinterpret_cast<unsigned*>(otile + off) = w;
+    }
+    // Nobody passes this barrier before every wavefront has written slice i; a wavefront
+    // writes slice i+1 into the other tile pair, and slice i+2 into this one only after
+    // the barrier(s) of slice i+1, which every wavefront reaches after its reads here.
+    lds_barrier();
+    const int m = tile_m * BM + i * 32 + rp;
+    const uintx4 v = *reinterpret_cast<const uintx4*>(otile + rp * PITCH + c16);
+    if (m < M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
+  };
+  slice(std::integral_constant<int, 0>{});
+  slice(std::integral_constant<int, 1>{});
+  slice(std::integral_constant<int, 2>{});
+  slice(std::integral_constant<int, 3>{});
 }
 
 // ---------------------------------------------------------------------------
@@ -456,6 +128,10 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
                                                        typename Mma<TIn>::Acc (&acc)[4][1], unsigned char* smem,
                                                        const int tile_m, const int tile_n, const int z, const int M,
                                                        const int wave, const int lane) {
+  if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
+    igemm_epilogue_rows128_q8(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
+    return;
+  }
   constexpr int BM = 128, BN = 128, TM = 4;
   constexpr int PITCH = BN + 4;  // 4-byte words per staged pixel row
   constexpr int TILE_WORDS = 32 * PITCH;
@@ -613,7 +289,8 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
 // channels of one pixel, so that global stores and residual loads are 16-byte
 // vectors and consecutive lanes cover contiguous memory.
 template <typename TIn, typename Epi, int BM, int BN, int WM, int WN>
-__global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64)
+// (the 128 x 128 tile is held to three wavefronts per SIMD: 168 registers)
+__global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, (BM == 128 && BN == 128) ? 3 : 1)
 igemm_kernel(const IgemmParams p, const int epi_vec) {
   constexpr int NW = (BM / WM) * (BN / WN);
   constexpr int NT = NW * 64;
@@ -747,6 +424,9 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  if constexpr (EpiTraits<Epi>::quant)
+    acc_init_bias<TM, TN>(p, z, tile_n * BN + __builtin_amdgcn_readfirstlane(wn) * WN, lg, acc);
 
   const int ktot = p.R * p.S * p.C;
   const int nkt = (ktot + BK - 1) / BK;
@@ -1370,7 +1050,8 @@ bool wreg_shape(const IgemmParams& p) {
 
 template <typename TIn, typename Epi>
 hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
-  if constexpr (!std::is_same<TIn, float>::value) {
+  // (the streaming kernel serves the 2-byte types only: no instantiation for the others)
+  if constexpr (std::is_same<TIn, f16_t>::value || std::is_same<TIn, bf16_t>::value) {
     if (p.w_frag != nullptr && lean_steps(p) > 0) return launch_lean<TIn, Epi>(p, epi_vec, s);
   }
   if (p.w_frag != nullptr && wreg_shape(p)) return launch_wreg<TIn, Epi>(p, epi_vec, s);
@@ -1392,6 +1073,12 @@ hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
 }
 
 const char* igemm_variant_name(const IgemmParams& p) {
+  switch (igemm_big_variant(p)) {
+    case 1: return "256x256";
+    case 2: return "256x128";
+    case 3: return "128x256";
+    default: break;
+  }
   if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
   if (p.w_frag != nullptr && wreg_shape(p)) return "128x128w";
   return choose_variant(p).name;
@@ -1453,6 +1140,17 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
   int epi_vec = rows_ok(p.y, p.ycs, p.y_bs);
   if (p.residual != nullptr) epi_vec = epi_vec && rows_ok(p.residual, p.rcs, p.r_bs);
   if (p.bias != nullptr) epi_vec = epi_vec && ((reinterpret_cast<uintptr_t>(p.bias) % 16) == 0) && (p.bias_bs % 4 == 0);
+  if (oes == 1) {
+    // bit 2: 8-bit rows allow 16-byte accesses (the requantising epilogue moves 16 channels per lane)
+    auto rows16 = [&](const void* ptr, int64_t cs, int64_t bs) {
+      return cs % 16 == 0 && bs % 16 == 0 && (reinterpret_cast<uintptr_t>(ptr) % 16u) == 0;
+    };
+    bool ok16 = rows16(p.y, p.ycs, p.y_bs);
+    if (p.residual != nullptr) ok16 = ok16 && rows16(p.residual, p.rcs, p.r_bs);
+    if (ok16) epi_vec |= 2;
+  }
+
+  if (const int big = igemm_big_variant(p)) return launch_igemm_big(p, epi_vec, big, stream);
 
   switch (p.in_dt) {
     case DT_F32:

@@ -107,22 +107,30 @@ struct IgemmParams {
   bool res_after_act = false;        // float types: y = act(..) + residual instead of act(.. + residual)
   bool stream_out = false;           // 2-byte results leave with non-temporal stores (results far larger than the last-level cache)
   // int8 only -----------------------------------------------------------
-  // out_dt == DT_I8 : q = clamp(rne(float(acc+bias) * qmul[n]) + q_zp, q_lo, 255)
-  //                   then, if residual: the unfused sequence
-  //                   f = (q - q_zp) * q_scale + (res - r_zp) * r_scale,
-  //                   q = clamp(rne(f * s_inv) + s_zp, s_lo, 255)
-  // out_dt == DT_F32: y = float(acc+bias) * qmul[n]    (dequantised result)
-  // out_dt == DT_I32: y = acc + bias                   (raw accumulators)
+  // acc = int32 accumulator + int32 bias; fma = one fused multiply-add in fp32
+  // (a single rounding); sat8 = round to nearest even and saturate to [0, 255].
+  // out_dt == DT_I8 : q = sat8(max(fma(float(acc), qmul[n], q_add), q_lo))
+  //                   with q_add = the zero point of the result, or, with a
+  //                   residual r (levels of an 8-bit tensor):
+  //                   q = sat8(max(fma(float(acc), qmul[n], fma(float(r), r_mul, r_add)), q_lo))
+  //                   qmul[n] = s_x s_w[n] / s_y, r_mul = s_r / s_y,
+  //                   r_add = zp_y - zp_r * r_mul: convolution, residual add and
+  //                   ReLU (q_lo = zp_y) are requantised ONCE.
+  // out_dt == DT_F32: y = float(acc) * qmul[n]    (dequantised result)
+  // out_dt == DT_I32: y = acc                     (raw accumulators)
   const float* qmul = nullptr;
   int a_fill = 0;  // stored byte that represents the real value 0 in x
-  int q_zp = 0, q_lo = 0;
-  float q_scale = 0.f;
-  int r_zp = 0; float r_scale = 0.f;
-  float s_inv = 0.f; int s_zp = 0, s_lo = 0;
+  float q_add = 0.f, q_lo = 0.f;
+  float r_mul = 0.f, r_add = 0.f;
 };
 hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream);
 // Name of the kernel variant launch_igemm would pick (for reports).
 const char* igemm_variant_name(const IgemmParams& p);
+
+// Large-tile kernels (igemm_big.hip) for matrix-core-bound layers: the variant
+// launch_igemm uses for this shape (0: none), and the launch itself.
+int igemm_big_variant(const IgemmParams& p);
+hipError_t launch_igemm_big(const IgemmParams& p, int epi_vec, int variant, hipStream_t stream);
 
 // True when launch_igemm would use a fragment-ordered weight copy for this shape.
 bool igemm_wants_wfrag(const IgemmParams& p);

@@ -1244,23 +1244,17 @@ void Planner::lower_conv(int ni) {
     ip.in_dt = DT_I8;
     ip.a_fill = (zx - 128) & 0xff;
 
-    const _odla_value* qv = ep.residual ? ep.pre_residual_value : outv;
-    const QuantEntry* qo = qentry(qv);
     const QuantEntry* qf = qentry(outv);
     std::vector<float> mul((size_t)O);
     int ty;
-    if (qo != nullptr && qf != nullptr) {
-      for (int64_t o = 0; o < O; ++o) mul[o] = (sx * sw[o]) / qo->scale;
+    if (qf != nullptr) {
+      // One requantisation per convolution, whatever is fused behind it: the result
+      // (after the residual add and the ReLU, if any) takes the scale and zero point
+      // of the last fused value.
+      for (int64_t o = 0; o < O; ++o) mul[o] = (sx * sw[o]) / qf->scale;
       ip.out_dt = DT_I8;
-      ip.q_zp = qo->zp;
-      ip.q_scale = qo->scale;
-      const bool relu = ep.act == ACT_RELU;
-      if (ep.residual) {
-        ip.q_lo = 0;
-        ip.s_inv = 1.0f / qf->scale; ip.s_zp = qf->zp; ip.s_lo = relu ? qf->zp : 0;
-      } else {
-        ip.q_lo = relu ? qo->zp : 0;
-      }
+      ip.q_add = (float)qf->zp;
+      ip.q_lo = ep.act == ACT_RELU ? (float)qf->zp : 0.f;
       ty = new_tensor(DT_I8, L_NHWC, outv->shape, (int)O, SP_ARENA);
       set_quant(ty, true, qf->scale, qf->zp);
     } else if (comp_->opts.raw_acc && ep.residual == nullptr && ep.act == ACT_NONE) {
@@ -1279,8 +1273,10 @@ void Planner::lower_conv(int ni) {
     if (ep.residual) {
       tr = get(ep.residual, L_NHWC, FORM_QUANT);
       ip.rcs = T(tr).cs;
-      ip.r_zp = T(tr).qzp;
-      ip.r_scale = T(tr).qscale;
+      // the residual's levels enter as fma(float(r), r_mul, r_add), r_add carrying both zero points
+      const QuantEntry* qy = qentry(outv);
+      ip.r_mul = T(tr).qscale / qy->scale;
+      ip.r_add = (float)qy->zp - (float)T(tr).qzp * ip.r_mul;
     }
     ip.stream_out = T(ty).bytes >= stream_out_bytes();
     const int tf = make_wfrag("conv.i8:" + outv->name, &ip, tw);

@@ -19,9 +19,9 @@
  *       convolution of its own; oneDNN would supply it).  Defines the int8
  *       plan: u8 activations with zero point, s8 weights, exact int32
  *       accumulation of (x - zp_x) * w, plus int32 bias.
- *   odla_ref_requant_q8   the requantisation sequence: fp32 multiply of the
- *       int32 accumulator by a per-channel multiplier, round-half-even, add
- *       zero point, clamp to [lo, 255].
+ *   odla_ref_requant_q8   the requantisation: one fused multiply-add of the
+ *       int32 accumulator with a per-channel multiplier and the zero point (or
+ *       the rescaled residual), lower clamp, round-half-even, saturate.
  */
 #include <math.h>
 #include <stddef.h>
@@ -150,20 +150,27 @@ void odla_ref_conv2d_q8(const uint8_t* x, int zp_x, const int8_t* w, const int32
   }
 }
 
-/* q = clamp(rne((float)acc * mul[o]) + zp, lo, 255) per channel o; acc is [N][O][HW]. */
-void odla_ref_requant_q8(const int32_t* acc, const float* mul, int zp, int lo, uint8_t* q, int N, int O,
-                         int HW) {
+/* Requantisation of the int8 plan, per channel o; acc (int32 accumulator plus
+ * int32 bias) is [N][O][HW]:
+ *   q = sat8(max(fma((float)acc, mul[o], add), lo))
+ * where `add` is the zero point of the result, or, with a residual r (levels of
+ * an 8-bit tensor of the same shape), add = fma((float)r, r_mul, r_add) per
+ * element.  fma is ONE fused multiply-add in binary32 (a single rounding: fmaf);
+ * sat8 rounds to the nearest integer, ties to even, and saturates to [0, 255]. */
+void odla_ref_requant_q8(const int32_t* acc, const float* mul, float add, float lo, const uint8_t* res,
+                         float r_mul, float r_add, uint8_t* q, int N, int O, int HW) {
 #pragma omp parallel for collapse(2) schedule(static)
   for (int n = 0; n < N; ++n) {
     for (int o = 0; o < O; ++o) {
       const size_t base = ((size_t)n * O + o) * HW;
       const float m = mul[o];
       for (int i = 0; i < HW; ++i) {
-        const float r = (float)acc[base + i] * m;
-        int v = (int)nearbyintf(r) + zp;
-        v = v < lo ? lo : v;
-        v = v > 255 ? 255 : v;
-        q[base + i] = (uint8_t)v;
+        const float a = res ? fmaf((float)res[base + i], r_mul, r_add) : add;
+        float f = fmaf((float)acc[base + i], m, a);
+        f = f > lo ? f : lo;
+        float r = nearbyintf(f);
+        r = r < 0.f ? 0.f : (r > 255.f ? 255.f : r);
+        q[base + i] = (uint8_t)r;
       }
     }
   }

@@ -141,16 +141,29 @@ def conv2d_q8_acc(xq, zp_x, wq, bias_i32=None, stride=(1, 1), pad=(0, 0, 0, 0)):
     return acc
 
 
-def requant_q8(acc, mul, zp, lo=0):
-    """q = clamp(rne(float32(acc) * mul[o]) + zp, lo, 255)."""
+def requant_q8(acc, mul, zp, lo=0, res=None, r_mul=0.0, r_add=0.0):
+    """q = sat8(max(fma(float32(acc), mul[o], add), lo)) with add = zp, or, with a
+    residual `res` (uint8 levels shaped like acc), add = fma(float32(res), r_mul, r_add).
+    fma = one fused multiply-add in float32 (C fmaf); sat8 = round half to even,
+    saturate to [0, 255].  This is the int8 plan's own definition (PARITY UNPINNED by
+    the reference, which has no int8 convolution)."""
     acc = np.ascontiguousarray(acc, dtype=np.int32)
     N, O = acc.shape[0], acc.shape[1]
     HW = int(np.prod(acc.shape[2:])) if acc.ndim > 2 else 1
     mul = _f32(mul).reshape(-1)
     assert mul.size == O
     q = np.empty(acc.shape, np.uint8)
-    lib().odla_ref_requant_q8(_p(acc, ctypes.c_int32), _p(mul, ctypes.c_float), int(zp), int(lo),
-                              _p(q, ctypes.c_uint8), N, O, HW)
+    f = lib().odla_ref_requant_q8
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_float, ctypes.c_void_p, ctypes.c_float,
+                  ctypes.c_float, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    f.restype = None
+    rp = None
+    if res is not None:
+        res = np.ascontiguousarray(res, dtype=np.uint8)
+        assert res.shape == acc.shape
+        rp = res.ctypes.data
+    f(acc.ctypes.data, mul.ctypes.data, float(np.float32(zp)), float(np.float32(lo)), rp, float(np.float32(r_mul)),
+      float(np.float32(r_add)), q.ctypes.data, N, O, HW)
     return q
 
 
@@ -204,8 +217,12 @@ def dequantize_act(q, scale, zp):
     return ((q.astype(np.float32) - np.float32(zp)) * np.float32(scale)).astype(np.float32)
 
 
-def qconv(xq, x_qp, w, bias, out_qp, stride, pad, relu=False):
-    """int8 convolution with fused requantisation, as the int8 plan defines it.
+def qconv(xq, x_qp, w, bias, out_qp, stride, pad, relu=False, residual=None):
+    """int8 convolution with fused requantisation, as the int8 plan defines it:
+    ONE requantisation to out_qp behind everything fused into the convolution - the
+    ReLU (a lower clamp at the zero point) and, when `residual` = (levels, (scale,
+    zp)) is given, the residual add: its levels enter the fused multiply-add as
+    fma(float(r), s_r / s_y, zp_y - zp_r * (s_r / s_y)).
     Returns (q_out u8, acc int32)."""
     s_x, zp_x = x_qp
     s_w = weight_qparams(w)
@@ -214,8 +231,13 @@ def qconv(xq, x_qp, w, bias, out_qp, stride, pad, relu=False):
     acc = conv2d_q8_acc(xq, zp_x, wq, bi, stride, pad)
     s_y, zp_y = out_qp
     mul = ((np.float32(s_x) * s_w).astype(np.float32) / np.float32(s_y)).astype(np.float32)
-    q = requant_q8(acc, mul, zp_y, zp_y if relu else 0)
-    return q, acc
+    lo = zp_y if relu else 0
+    if residual is None:
+        return requant_q8(acc, mul, zp_y, lo), acc
+    rq, (s_r, zp_r) = residual
+    r_mul = np.float32(s_r) / np.float32(s_y)
+    r_add = np.float32(zp_y) - np.float32(zp_r) * r_mul
+    return requant_q8(acc, mul, zp_y, lo, rq, r_mul, r_add), acc
 
 
 def cast_like_reference(x, dtype):

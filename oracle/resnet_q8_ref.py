@@ -4,8 +4,9 @@ Evaluates the post-training-quantised ResNet-50-shaped network with explicit
 integer arithmetic (u8 activations, s8 weights, int32 accumulators) following
 the fusion rules of the int8 plan:
   conv (+ ReLU)          -> requantise to the table entry of the last fused value
-  conv + residual + ReLU -> requantise to the conv's own entry, then the
-                            dequantise / add / requantise sequence
+  conv + residual + ReLU -> likewise, ONE requantisation: the residual's levels
+                            enter the fused multiply-add of the requantisation
+                            (ref.qconv with `residual`)
   max-pool               -> keeps levels and its input's scale
   global average pool    -> fp32 (the head has no table entries)
 PARITY UNPINNED by the reference for the requantisation formula (the reference
@@ -28,9 +29,9 @@ def run(w, feeds, qp, stages, stem, batch, hw, record=None):
     cur_qp = qp["input"]
     rec("input", x)
 
-    def conv(xq, x_qp, name, stride, pad, out_name, relu):
+    def conv(xq, x_qp, name, stride, pad, out_name, relu, residual=None):
         q, acc = ref.qconv(xq, x_qp, w[name + ".w"], w[name + ".b"], qp[out_name], (stride, stride),
-                           (pad, pad, pad, pad), relu)
+                           (pad, pad, pad, pad), relu, residual)
         rec(out_name, q, acc)
         return q
 
@@ -50,9 +51,7 @@ def run(w, feeds, qp, stages, stem, batch, hw, record=None):
                 ident, ident_qp = x, cur_qp
             y = conv(x, cur_qp, p + "c1", 1, 0, p + "c1.relu", True)
             y = conv(y, qp[p + "c1.relu"], p + "c2", s, 1, p + "c2.relu", True)
-            y = conv(y, qp[p + "c2.relu"], p + "c3", 1, 0, p + "c3", False)
-            x = ref.qadd(y, qp[p + "c3"], ident, ident_qp, qp[p + "out"], relu=True)
-            rec(p + "out", x)
+            x = conv(y, qp[p + "c2.relu"], p + "c3", 1, 0, p + "out", True, (ident, ident_qp))
             cur_qp = qp[p + "out"]
     # global average pool -> fp32: ((sum q - n*zp) / n) * scale
     n = x.shape[2] * x.shape[3]

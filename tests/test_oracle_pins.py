@@ -248,13 +248,79 @@ def test_quantize_round_half_even_exhaustive(ref):
 
 
 def test_requant_formula_rounding_and_saturation(ref):
-    acc = np.array([[[[-1000, -3, -1, 0, 1, 3, 5, 1000, 2 ** 24 + 1]]]], np.int32).transpose(0, 3, 1, 2).copy()
-    acc = acc.reshape(1, 9, 1, 1)
+    """q = sat8(max(fma(float(acc), mul, zp), lo)): hand-worked, mul = 0.5 (exact products)."""
+    acc = np.array([-1000, -3, -1, 0, 1, 3, 5, 1000, 2 ** 24 + 1], np.int32).reshape(1, 9, 1, 1)
     mul = np.full(9, 0.5, np.float32)
-    q = ref.requant_q8(acc, mul, zp=10, lo=0).reshape(-1)
-    # 0.5*acc: -500,-1.5,-0.5,0,0.5,1.5,2.5,500,2^23 -> rne -> +10 -> clamp
-    assert q.tolist() == [0, 8, 10, 10, 10, 12, 12, 255, 255]
+    # 0.5*acc + 10: -490, 8.5, 9.5, 10, 10.5, 11.5, 12.5, 510, 2^23 + 10 -> ties to even, saturate
+    assert ref.requant_q8(acc, mul, zp=10, lo=0).reshape(-1).tolist() == [0, 8, 10, 10, 10, 12, 12, 255, 255]
     assert ref.requant_q8(acc, mul, zp=10, lo=10).reshape(-1).tolist() == [10, 10, 10, 10, 10, 12, 12, 255, 255]
+    # the zero point is inside the rounding: with an odd one the ties fall the other way
+    # 0.5*acc + 11: -489, 9.5, 10.5, 11, 11.5, 12.5, 13.5, 511, ...
+    assert ref.requant_q8(acc, mul, zp=11, lo=0).reshape(-1).tolist() == [0, 10, 10, 11, 12, 12, 14, 255, 255]
+    # with a residual: add = fma(r, r_mul, r_add); r_mul = 0.25, r_add = 5 - 20 * 0.25 = 0
+    res = np.array([0, 20, 22, 21, 23, 255, 255, 0, 0], np.uint8).reshape(1, 9, 1, 1)
+    # 0.5*acc:   -500  -1.5  -0.5  0     0.5   1.5    2.5    500  2^23
+    # 0.25*r:    0     5     5.5   5.25  5.75  63.75  63.75  0    0
+    # sum:       -500  3.5   5.0   5.25  6.25  65.25  66.25  500  2^23
+    assert ref.requant_q8(acc, mul, 5, 0, res, 0.25, 0.0).reshape(-1).tolist() == [0, 4, 5, 5, 6, 65, 66, 255, 255]
+    assert ref.requant_q8(acc, mul, 5, 5, res, 0.25, 0.0).reshape(-1).tolist() == [5, 5, 5, 5, 6, 65, 66, 255, 255]
+
+
+def _round_to_f32(fr):
+    """Nearest binary32 value (ties to even) of an exact rational, as a Fraction."""
+    from fractions import Fraction
+    if fr == 0:
+        return Fraction(0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = 0
+    while a >= 2 ** 24:
+        a /= 2
+        e += 1
+    while a < 2 ** 23:
+        a *= 2
+        e -= 1
+    n = round(a)          # Python rounds exact halves to the even integer
+    return sign * Fraction(n) * Fraction(2) ** e
+
+
+def test_requant_is_one_fused_multiply_add_against_exact_rationals(ref):
+    """The requantisation rounds acc * mul + add ONCE to binary32 (a fused multiply-add),
+    then to the nearest integer (ties to even), then saturates: checked against exact
+    rational arithmetic, so that neither a separate multiply and add (two roundings)
+    nor a double-precision detour would pass."""
+    from fractions import Fraction
+    r = rng(91)
+    n = 4000
+    acc = r.integers(-70000, 70000, n).astype(np.int32)
+    acc[:8] = [1, 3, -3, 5, 2 ** 24 + 1, -(2 ** 24) - 3, 2 ** 31 - 1, -(2 ** 31)]
+    mul = (r.random(n, dtype=np.float32) * np.float32(0.01)).astype(np.float32)
+    mul[:4] = np.float32(0.5) + np.float32(2.0 ** -24)     # products just beside a tie
+    # cases found by search in which rounding the product before the zero point is added
+    # (two roundings) lands on the other side of a tie: one fused multiply-add gives 5, 5, 27, 17
+    acc[8:12] = [-38736, -50321, -52629, -25444]
+    mul[8:12] = [float.fromhex(h) for h in ("0x1.a7cfc8p-8", "0x1.44f044p-8", "0x1.1c89dap-8", "0x1.31dd26p-7")]
+    zp = 255.0
+    resq = r.integers(0, 256, n).astype(np.uint8)
+    r_mul, r_add = np.float32(0.3713), np.float32(-11.625)
+    got = ref.requant_q8(acc.reshape(1, n, 1, 1), mul, zp, 3).reshape(-1)
+    got_r = ref.requant_q8(acc.reshape(1, n, 1, 1), mul, zp, 3, resq.reshape(1, n, 1, 1), r_mul, r_add).reshape(-1)
+
+    def sat8(fr):
+        fr = max(fr, Fraction(3))
+        return int(min(max(round(fr), 0), 255))
+
+    two_roundings_differ = 0
+    for i in range(n):
+        a = _round_to_f32(Fraction(int(acc[i])))                      # int32 -> float32
+        m = Fraction(float(mul[i]))
+        want = sat8(_round_to_f32(a * m + Fraction(zp)))
+        assert int(got[i]) == want, (i, int(acc[i]), float(mul[i]))
+        add = _round_to_f32(Fraction(int(resq[i])) * Fraction(float(r_mul)) + Fraction(float(r_add)))
+        assert int(got_r[i]) == sat8(_round_to_f32(a * m + add)), i
+        two_roundings_differ += sat8(_round_to_f32(_round_to_f32(a * m) + Fraction(zp))) != want
+    assert got[8:12].tolist() == [5, 5, 27, 17]
+    assert two_roundings_differ >= 4       # the sample does tell the two formulations apart
 
 
 def test_qadd_hand_worked_levels(ref):
