@@ -133,6 +133,12 @@ __device__ __forceinline__ float apply_act(float v, ActKind act, float a, float 
   return v;
 }
 
+// n / d for 0 <= n < 2^31 with the divisor's magic pair (div_magic on the host
+// side): three instructions instead of the ~35 of a 32-bit division.
+__device__ __forceinline__ int fast_div(int n, unsigned magic, int shift) {
+  return (int)(__umulhi((unsigned)n << 1, magic) >> shift);
+}
+
 // Wavefront (64 lanes) reductions through cross-lane shuffles.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

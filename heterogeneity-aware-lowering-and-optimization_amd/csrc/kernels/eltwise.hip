@@ -21,33 +21,39 @@ __device__ __forceinline__ void out_store(Vec16<T>& v, T* p) {
   v.store(p);
 }
 
-template <typename T>
+// A workgroup owns one contiguous tile of kThreads * U 16-byte vectors: load u of
+// a thread is vector tile * kThreads * U + u * kThreads + thread, so that every
+// load instruction of a wavefront covers one contiguous KiB and a workgroup's U
+// loads cover one contiguous U * 4 KiB, all in flight before the first use.
+// KIND >= 0 fixes the activation at compile time (the switch folds away; per
+// element it would cost more than the arithmetic); KIND < 0 takes it from `act`.
+template <typename T, int KIND, int U>
 __global__ void __launch_bounds__(kThreads)
 unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, ActKind act, float a, float b) {
   constexpr int V = Vec16<T>::N;
+  const ActKind kind = KIND >= 0 ? (ActKind)KIND : act;
   const int64_t nvec = n / V;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i0 < nvec; i0 += stride * kUnroll) {
-    Vec16<T> v[kUnroll];
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  Vec16<T> v[U];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t i = i0 + u * stride;
-      if (i < nvec) v[u].load(x + i * V);
-    }
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * kThreads;
+    if (i < nvec) v[u].raw = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(x + i * V));
+  }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int64_t i = i0 + u * stride;
-      if (i < nvec) {
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * kThreads;
+    if (i < nvec) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) v[u].set(e, apply_act(v[u].get(e), act, a, b));
-        out_store(v[u], y + i * V);
-      }
+      for (int e = 0; e < V; ++e) v[u].set(e, apply_act(v[u].get(e), kind, a, b));
+      out_store(v[u], y + i * V);
     }
   }
-  // tail
-  const int64_t tail0 = nvec * V;
-  for (int64_t i = tail0 + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
-    Store<T>::st(y + i, apply_act(Store<T>::ld(x + i), act, a, b));
+  // tail (fewer than V elements), by the first workgroup
+  if (blockIdx.x == 0) {
+    for (int64_t i = nvec * V + threadIdx.x; i < n; i += kThreads)
+      Store<T>::st(y + i, apply_act(Store<T>::ld(x + i), kind, a, b));
+  }
 }
 
 // y = x * scale[c] + shift[c].  inner == 1: channel is the innermost index
@@ -56,54 +62,55 @@ unary_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, ActKind act,
 // channels in every iteration and keeps their parameters in registers.
 // inner > 1 (row-major N,C,HW): the channel is constant across a vector when
 // inner % V == 0.
-template <typename T>
+template <typename T, int U>
 __global__ void __launch_bounds__(kThreads)
 channel_affine_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, int64_t inner,
                       int channels, const float* __restrict__ scale,
                       const float* __restrict__ shift) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   constexpr int V = Vec16<T>::N;
   const bool vec_ok = (inner == 1) ? (channels % V == 0) : (inner % V == 0);
   if (vec_ok) {
+    // tiled like unary_kernel: a workgroup owns kThreads * U consecutive vectors
     const int64_t nvec = n / V;
-    const int64_t t0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-    const bool fixed = (inner == 1) && ((stride * V) % channels == 0);
-    float sc[V], sh[V];
-    if (fixed) {
-      const int c0 = (int)((t0 * V) % channels);
+    const int64_t tile0 = (int64_t)blockIdx.x * (kThreads * U);
+    const int64_t base = tile0 + threadIdx.x;
+    // channel of the tile's first element (wavefront-uniform), then 32-bit arithmetic per vector
+    const unsigned c_tile = inner == 1 ? (unsigned)((tile0 * V) % channels) : 0u;
+    Vec16<T> v[U];
 #pragma unroll
-      for (int e = 0; e < V; ++e) { sc[e] = scale[c0 + e]; sh[e] = shift[c0 + e]; }
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i < nvec) v[u].raw = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(x + i * V));
     }
-    for (int64_t i0 = t0; i0 < nvec; i0 += stride * kUnroll) {
-      Vec16<T> v[kUnroll];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int64_t i = i0 + u * stride;
-        if (i < nvec) v[u].load(x + i * V);
-      }
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int64_t i = i0 + u * stride;
-        if (i >= nvec) continue;
-        const int64_t e0 = i * V;
-        if (fixed) {
-#pragma unroll
-          for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * sc[e] + sh[e]);
-        } else if (inner == 1) {
-          const int c0 = (int)(e0 % channels);
-#pragma unroll
-          for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * scale[c0 + e] + shift[c0 + e]);
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * kThreads;
+      if (i >= nvec) continue;
+      if (inner == 1) {
+        const unsigned c0 = (c_tile + (unsigned)(u * kThreads + threadIdx.x) * V) % (unsigned)channels;
+        float sc[V], sh[V];
+        if constexpr (V == 8) {
+          const floatx4 s0 = *reinterpret_cast<const floatx4*>(scale + c0), s1 = *reinterpret_cast<const floatx4*>(scale + c0 + 4);
+          const floatx4 t0 = *reinterpret_cast<const floatx4*>(shift + c0), t1 = *reinterpret_cast<const floatx4*>(shift + c0 + 4);
+          sc[0] = s0.x; sc[1] = s0.y; sc[2] = s0.z; sc[3] = s0.w; sc[4] = s1.x; sc[5] = s1.y; sc[6] = s1.z; sc[7] = s1.w;
+          sh[0] = t0.x; sh[1] = t0.y; sh[2] = t0.z; sh[3] = t0.w; sh[4] = t1.x; sh[5] = t1.y; sh[6] = t1.z; sh[7] = t1.w;
         } else {
-          const int c = (int)((e0 / inner) % channels);
-          const float s = scale[c], t = shift[c];
 #pragma unroll
-          for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * s + t);
+          for (int e = 0; e < V; ++e) { sc[e] = scale[c0 + e]; sh[e] = shift[c0 + e]; }
         }
-        out_store(v[u], y + i * V);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * sc[e] + sh[e]);
+      } else {
+        const int c = (int)(((i * V) / inner) % channels);
+        const float sc = scale[c], sh = shift[c];
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[u].set(e, v[u].get(e) * sc + sh);
       }
+      out_store(v[u], y + i * V);
     }
   } else {
-    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x * U;
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride / U) {
       const int c = (int)((i / inner) % channels);
       Store<T>::st(y + i, Store<T>::ld(x + i) * scale[c] + shift[c]);
     }
@@ -134,34 +141,39 @@ __device__ __forceinline__ float bin_op(float a, float b, BinKind op) {
   return a;
 }
 
-// Same-shape, contiguous operands.
-template <typename T>
+// Same-shape, contiguous operands; tiled like unary_kernel.  OP / KIND >= 0 fix the
+// operator / the fused activation at compile time.
+template <typename T, int OP, int KIND, int U>
 __global__ void __launch_bounds__(kThreads)
 binary_flat_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ y, int64_t n,
-                   BinKind op, ActKind act, float aa, float ab) {
+                   BinKind op_rt, ActKind act, float aa, float ab) {
   constexpr int V = Vec16<T>::N;
-  constexpr int U = 2;
+  const BinKind op = OP >= 0 ? (BinKind)OP : op_rt;
+  const ActKind kind = KIND >= 0 ? (ActKind)KIND : act;
   const int64_t nvec = n / V;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i0 < nvec; i0 += stride * U) {
-    Vec16<T> va[U], vb[U];
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * U) + threadIdx.x;
+  Vec16<T> va[U], vb[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int64_t i = i0 + u * stride;
-      if (i < nvec) { va[u].load(a + i * V); vb[u].load(b + i * V); }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int64_t i = i0 + u * stride;
-      if (i < nvec) {
-#pragma unroll
-        for (int e = 0; e < V; ++e) va[u].set(e, apply_act(bin_op(va[u].get(e), vb[u].get(e), op), act, aa, ab));
-        out_store(va[u], y + i * V);
-      }
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * kThreads;
+    if (i < nvec) {
+      va[u].raw = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(a + i * V));
+      vb[u].raw = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(b + i * V));
     }
   }
-  for (int64_t i = nvec * V + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride)
-    Store<T>::st(y + i, apply_act(bin_op(Store<T>::ld(a + i), Store<T>::ld(b + i), op), act, aa, ab));
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * kThreads;
+    if (i < nvec) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) va[u].set(e, apply_act(bin_op(va[u].get(e), vb[u].get(e), op), kind, aa, ab));
+      out_store(va[u], y + i * V);
+    }
+  }
+  if (blockIdx.x == 0) {
+    for (int64_t i = nvec * V + threadIdx.x; i < n; i += kThreads)
+      Store<T>::st(y + i, apply_act(bin_op(Store<T>::ld(a + i), Store<T>::ld(b + i), op), kind, aa, ab));
+  }
 }
 
 // One operand is a vector indexed by the innermost output dim (bias rows,
@@ -439,9 +451,30 @@ hipError_t launch_unary(const void* x, void* y, DType dt, int64_t n, ActKind act
                         hipStream_t stream) {
   if (n <= 0) return n == 0 ? hipSuccess : hipErrorInvalidValue;
   if (!x || !y || !al16(x) || !al16(y)) return hipErrorInvalidValue;
-  const int grid = grid_for(n, kThreads * 8);
-  FLOAT_DISPATCH(dt, hipLaunchKernelGGL(unary_kernel<T>, dim3(grid), dim3(kThreads), 0, stream,
-                                        (const T*)x, (T*)y, n, act, a, b));
+  constexpr int U = 4;
+  const int64_t tiles = (n / (16 / dtype_size(dt)) + kThreads * U - 1) / (kThreads * U);
+  if (tiles > 0x7fffffff) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(tiles > 0 ? tiles : 1));
+#define UNARY_CASE(K_)                                                                                  \
+  case K_:                                                                                              \
+    FLOAT_DISPATCH(dt, hipLaunchKernelGGL((unary_kernel<T, (int)K_, U>), grid, dim3(kThreads), 0, stream, \
+                                          (const T*)x, (T*)y, n, act, a, b));                           \
+    break;
+  switch (act) {
+    UNARY_CASE(ACT_RELU)
+    UNARY_CASE(ACT_LEAKY)
+    UNARY_CASE(ACT_CLAMP)
+    UNARY_CASE(ACT_NEG)
+    UNARY_CASE(ACT_SIGMOID)
+    UNARY_CASE(ACT_TANH)
+    UNARY_CASE(ACT_GELU_ERF)
+    UNARY_CASE(ACT_GELU_TANH)
+    UNARY_CASE(ACT_EXP)
+    default:
+      FLOAT_DISPATCH(dt, hipLaunchKernelGGL((unary_kernel<T, -1, U>), grid, dim3(kThreads), 0, stream, (const T*)x,
+                                            (T*)y, n, act, a, b));
+  }
+#undef UNARY_CASE
   return hipGetLastError();
 }
 
@@ -452,8 +485,11 @@ hipError_t launch_channel_affine(const void* x, void* y, DType dt, int64_t n, in
   if (!x || !y || !scale || !shift || !al16(x) || !al16(y) || inner <= 0 || channels <= 0)
     return hipErrorInvalidValue;
   if (n % (inner * channels) != 0) return hipErrorInvalidValue;
-  const int grid = grid_for(n, kThreads * 8);
-  FLOAT_DISPATCH(dt, hipLaunchKernelGGL(channel_affine_kernel<T>, dim3(grid), dim3(kThreads), 0,
+  constexpr int U = 4;
+  const int64_t tiles = (n / (16 / dtype_size(dt)) + kThreads * U - 1) / (kThreads * U);
+  if (tiles > 0x7fffffff) return hipErrorInvalidValue;
+  const unsigned grid = (unsigned)(tiles > 0 ? tiles : 1);
+  FLOAT_DISPATCH(dt, hipLaunchKernelGGL((channel_affine_kernel<T, U>), dim3(grid), dim3(kThreads), 0,
                                         stream, (const T*)x, (T*)y, n, inner, channels, scale, shift));
   return hipGetLastError();
 }
@@ -503,9 +539,19 @@ hipError_t launch_binary(const BinaryParams& p, hipStream_t stream) {
   }
   const bool aligned = al16(p.a) && al16(p.b) && al16(p.y);
   if (aligned && is_full(p.sa) && is_full(p.sb)) {
-    FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL(binary_flat_kernel<T>, dim3(grid), dim3(kThreads), 0, stream,
-                                            (const T*)p.a, (const T*)p.b, (T*)p.y, n, p.op, p.act,
-                                            p.act_a, p.act_b));
+    constexpr int U = 4;
+    const int64_t tiles = (n / (16 / dtype_size(p.dt)) + kThreads * U - 1) / (kThreads * U);
+    if (tiles > 0x7fffffff) return hipErrorInvalidValue;
+    const dim3 fgrid((unsigned)(tiles > 0 ? tiles : 1));
+#define BIN_FLAT(OP_, K_)                                                                                           \
+  FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((binary_flat_kernel<T, OP_, K_, U>), fgrid, dim3(kThreads), 0, stream,     \
+                                          (const T*)p.a, (const T*)p.b, (T*)p.y, n, p.op, p.act, p.act_a, p.act_b))
+    if (p.op == BIN_ADD && p.act == ACT_NONE) { BIN_FLAT((int)BIN_ADD, (int)ACT_NONE); }
+    else if (p.op == BIN_ADD && p.act == ACT_RELU) { BIN_FLAT((int)BIN_ADD, (int)ACT_RELU); }
+    else if (p.op == BIN_MUL && p.act == ACT_NONE) { BIN_FLAT((int)BIN_MUL, (int)ACT_NONE); }
+    else if (p.op == BIN_SUB && p.act == ACT_NONE) { BIN_FLAT((int)BIN_SUB, (int)ACT_NONE); }
+    else { BIN_FLAT(-1, -1); }
+#undef BIN_FLAT
     return hipGetLastError();
   }
   if (aligned && is_full(p.sa)) {

@@ -1084,14 +1084,6 @@ const char* igemm_variant_name(const IgemmParams& p) {
   return choose_variant(p).name;
 }
 
-// magic pair for fast_div: shift = ceil(log2 d), magic = ceil(2^(31+shift) / d)
-static void div_magic(int d, unsigned* magic, int* shift) {
-  int s = 0;
-  while ((1ll << s) < d) ++s;
-  *shift = s;
-  *magic = (unsigned)((((unsigned long long)1 << (31 + s)) + (unsigned long long)d - 1) / (unsigned long long)d);
-}
-
 hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
   IgemmParams p = p_in;
   if (p.Ho > 0 && p.Wo > 0) {

@@ -10,12 +10,6 @@
 
 namespace ohip {
 
-// n / d for 0 <= n < 2^31 with the divisor's magic pair (see div_magic on the
-// host side): three instructions instead of the ~35 of a 32-bit division.
-__device__ __forceinline__ int fast_div(int n, unsigned magic, int shift) {
-  return (int)(__umulhi((unsigned)n << 1, magic) >> shift);
-}
-
 template <typename T> struct Mma;
 template <> struct Mma<float> {
   using Acc = floatx16;

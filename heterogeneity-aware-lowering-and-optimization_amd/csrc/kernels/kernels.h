@@ -44,6 +44,15 @@ inline int dtype_size(DType t) {
 }
 inline bool dtype_is_float(DType t) { return t == DT_F32 || t == DT_F16 || t == DT_BF16; }
 
+// Magic pair for the kernels' fast_div(n, magic, shift) = n / d, 0 <= n < 2^31, 1 <= d < 2^31:
+// shift = ceil(log2 d), magic = ceil(2^(31+shift) / d).
+inline void div_magic(int d, unsigned* magic, int* shift) {
+  int s = 0;
+  while ((1ll << s) < d) ++s;
+  *shift = s;
+  *magic = (unsigned)((((unsigned long long)1 << (31 + s)) + (unsigned long long)d - 1) / (unsigned long long)d);
+}
+
 // Activation applied in a GEMM epilogue or by the unary kernel.
 enum ActKind : int {
   ACT_NONE = 0, ACT_RELU, ACT_LEAKY, ACT_CLAMP, ACT_SIGMOID, ACT_TANH,
@@ -274,6 +283,9 @@ struct PoolParams {
   bool count_include_pad = false;
   // int8 average pooling: q = clamp(rne(mean(q_in - zp_in) * mul) + zp_out)
   float q_mul = 1.f; int zp_in = 0, zp_out = 0;
+  // filled in by launch_pool2d: magic pairs for the divisions by Wo * (C / vector) and C / vector
+  unsigned row_magic = 0, cv_magic = 0;
+  int row_shift = 0, cv_shift = 0;
 };
 hipError_t launch_pool2d(const PoolParams& p, hipStream_t stream);
 

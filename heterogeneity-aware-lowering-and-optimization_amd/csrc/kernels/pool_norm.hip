@@ -22,16 +22,19 @@ template <typename T, bool IS_MAX, int KH, int KW>
 __global__ void __launch_bounds__(kThreads) pool2d_vec_kernel(PoolParams p) {
   constexpr int V = Vec16<T>::N;
   const int cv = p.C / V;  // C % V == 0 checked by the launcher
-  const int64_t total = (int64_t)p.N * p.Ho * p.Wo * cv;
   const T* x = reinterpret_cast<const T*>(p.x);
   T* y = reinterpret_cast<T*>(p.y);
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const int c = (int)(i % cv) * V;
-    int64_t t = i / cv;
-    const int wo = (int)(t % p.Wo); t /= p.Wo;
-    const int ho = (int)(t % p.Ho);
-    const int n = (int)(t / p.Ho);
+  // blockIdx.x walks the (ho, wo, channel vector) positions of one image, blockIdx.y the
+  // images: 32-bit index arithmetic with magic divisions (a 64-bit division per thread
+  // costs as much as the thread's memory traffic)
+  const int per_image = p.Ho * p.Wo * cv, row = p.Wo * cv;
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= per_image) return;
+  const int ho = fast_div(i, p.row_magic, p.row_shift);
+  const int rem = i - ho * row;
+  const int wo = fast_div(rem, p.cv_magic, p.cv_shift);
+  const int c = (rem - wo * cv) * V;
+  for (int n = blockIdx.y; n < p.N; n += gridDim.y) {
     const int h0 = ho * p.sh - p.ph, w0 = wo * p.sw - p.pw;
     float acc[V];
 #pragma unroll
@@ -123,53 +126,76 @@ __global__ void __launch_bounds__(kThreads) pool2d_scalar_kernel(PoolParams p) {
 template <bool IS_MAX>
 __global__ void __launch_bounds__(kThreads) pool2d_q8_kernel(PoolParams p) {
   const int cv = p.C / 16;
-  const int64_t total = (int64_t)p.N * p.Ho * p.Wo * cv;
   const int8_t* x = reinterpret_cast<const int8_t*>(p.x);
   int8_t* y = reinterpret_cast<int8_t*>(p.y);
-  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const int c = (int)(i % cv) * 16;
-    int64_t t = i / cv;
-    const int wo = (int)(t % p.Wo); t /= p.Wo;
-    const int ho = (int)(t % p.Ho);
-    const int n = (int)(t / p.Ho);
+  const int per_image = p.Ho * p.Wo * cv, row = p.Wo * cv;
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= per_image) return;
+  const int ho = fast_div(i, p.row_magic, p.row_shift);
+  const int rem = i - ho * row;
+  const int wo = fast_div(rem, p.cv_magic, p.cv_shift);
+  const int c = (rem - wo * cv) * 16;
+  for (int n = blockIdx.y; n < p.N; n += gridDim.y) {
     const int h0 = ho * p.sh - p.ph, w0 = wo * p.sw - p.pw;
-    int acc[16];
+    if constexpr (IS_MAX) {
+      // Levels as unsigned bytes (stored ^ 0x80); even and odd bytes of a dword are two
+      // 16-bit lanes each, so one packed 16-bit maximum handles two levels.
+      typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
+      unsigned ev[4] = {0u, 0u, 0u, 0u}, od[4] = {0u, 0u, 0u, 0u};
+      for (int r = 0; r < p.kh; ++r) {
+        const int hi = h0 + r;
+        if ((unsigned)hi >= (unsigned)p.H) continue;
+        for (int s = 0; s < p.kw; ++s) {
+          const int wi = w0 + s;
+          if ((unsigned)wi >= (unsigned)p.W) continue;
+          const uintx4 v = *reinterpret_cast<const uintx4*>(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c);
+          const unsigned w[4] = {v.x ^ 0x80808080u, v.y ^ 0x80808080u, v.z ^ 0x80808080u, v.w ^ 0x80808080u};
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = IS_MAX ? -1000 : 0;
-    int cnt = 0;
-    for (int r = 0; r < p.kh; ++r) {
-      const int hi = h0 + r;
-      if ((unsigned)hi >= (unsigned)p.H) continue;
-      for (int s = 0; s < p.kw; ++s) {
-        const int wi = w0 + s;
-        if ((unsigned)wi >= (unsigned)p.W) continue;
-        const uintx4 v = *reinterpret_cast<const uintx4*>(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c);
-        const int8_t* ev = reinterpret_cast<const int8_t*>(&v);
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int q = q_from_stored(ev[e]);
-          acc[e] = IS_MAX ? (q > acc[e] ? q : acc[e]) : acc[e] + q;
+          for (int k = 0; k < 4; ++k) {
+            const ushortx2 a0 = __builtin_bit_cast(ushortx2, ev[k]), b0 = __builtin_bit_cast(ushortx2, w[k] & 0x00ff00ffu);
+            const ushortx2 a1 = __builtin_bit_cast(ushortx2, od[k]), b1 = __builtin_bit_cast(ushortx2, (w[k] >> 8) & 0x00ff00ffu);
+            ev[k] = __builtin_bit_cast(unsigned, __builtin_elementwise_max(a0, b0));
+            od[k] = __builtin_bit_cast(unsigned, __builtin_elementwise_max(a1, b1));
+          }
         }
-        ++cnt;
       }
-    }
-    uintx4 o;
-    int8_t* eo = reinterpret_cast<int8_t*>(&o);
-    const int div = p.count_include_pad ? p.kh * p.kw : (cnt > 0 ? cnt : 1);
+      uintx4 o;
+      o.x = (ev[0] | (od[0] << 8)) ^ 0x80808080u;
+      o.y = (ev[1] | (od[1] << 8)) ^ 0x80808080u;
+      o.z = (ev[2] | (od[2] << 8)) ^ 0x80808080u;
+      o.w = (ev[3] | (od[3] << 8)) ^ 0x80808080u;
+      // (a window without a valid tap cannot occur: the planner derives Ho, Wo from the padding)
+      *reinterpret_cast<uintx4*>(y + (((int64_t)n * p.Ho + ho) * p.Wo + wo) * p.ycs + c) = o;
+    } else {
+      int acc[16];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      int q;
-      if (IS_MAX) {
-        q = acc[e];
-      } else {
-        const float f = (float)(acc[e] - cnt * p.zp_in) / (float)div;
-        q = (int)rintf(f * p.q_mul) + p.zp_out;
-        q = q < 0 ? 0 : (q > 255 ? 255 : q);
+      for (int e = 0; e < 16; ++e) acc[e] = 0;
+      int cnt = 0;
+      for (int r = 0; r < p.kh; ++r) {
+        const int hi = h0 + r;
+        if ((unsigned)hi >= (unsigned)p.H) continue;
+        for (int s = 0; s < p.kw; ++s) {
+          const int wi = w0 + s;
+          if ((unsigned)wi >= (unsigned)p.W) continue;
+          const uintx4 v = *reinterpret_cast<const uintx4*>(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c);
+          const int8_t* ev = reinterpret_cast<const int8_t*>(&v);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[e] += q_from_stored(ev[e]);
+          ++cnt;
+        }
       }
-      eo[e] = q_to_stored(q);
+      uintx4 o;
+      int8_t* eo = reinterpret_cast<int8_t*>(&o);
+      const int div = p.count_include_pad ? p.kh * p.kw : (cnt > 0 ? cnt : 1);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float f = (float)(acc[e] - cnt * p.zp_in) / (float)div;
+        int q = (int)rintf(f * p.q_mul) + p.zp_out;
+        q = q < 0 ? 0 : (q > 255 ? 255 : q);
+        eo[e] = q_to_stored(q);
+      }
+      *reinterpret_cast<uintx4*>(y + (((int64_t)n * p.Ho + ho) * p.Wo + wo) * p.ycs + c) = o;
     }
-    *reinterpret_cast<uintx4*>(y + (((int64_t)n * p.Ho + ho) * p.Wo + wo) * p.ycs + c) = o;
   }
 }
 
@@ -650,7 +676,8 @@ layernorm_long_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, 
     default: return hipErrorInvalidValue;                \
   }
 
-hipError_t launch_pool2d(const PoolParams& p, hipStream_t stream) {
+hipError_t launch_pool2d(const PoolParams& p_in, hipStream_t stream) {
+  PoolParams p = p_in;
   if (!p.x || !p.y || p.N <= 0 || p.H <= 0 || p.W <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0)
     return hipErrorInvalidValue;
   if (p.cs < p.C || p.ycs < p.C || p.kh <= 0 || p.kw <= 0 || p.sh <= 0 || p.sw <= 0)
@@ -659,19 +686,22 @@ hipError_t launch_pool2d(const PoolParams& p, hipStream_t stream) {
   if (es == 0) return hipErrorInvalidValue;
   const int V = 16 / es;
   const bool vec = (p.C % V == 0) && (p.cs % V == 0) && (p.ycs % V == 0) && al16(p.x) && al16(p.y);
-  if (p.dt == DT_I8) {
-    if (!vec) return hipErrorInvalidValue;
-    const int64_t total = (int64_t)p.N * p.Ho * p.Wo * (p.C / 16);
-    const int grid = grid_for(total, kThreads);
-    if (p.is_max) hipLaunchKernelGGL(pool2d_q8_kernel<true>, dim3(grid), dim3(kThreads), 0, stream, p);
-    else hipLaunchKernelGGL(pool2d_q8_kernel<false>, dim3(grid), dim3(kThreads), 0, stream, p);
-    return hipGetLastError();
-  }
+  if (p.dt == DT_I8 && !vec) return hipErrorInvalidValue;
   if (vec) {
-    const int64_t total = (int64_t)p.N * p.Ho * p.Wo * (p.C / V);
-    const int grid = grid_for(total, kThreads);
+    // one image per blockIdx.y (folded beyond the grid limit), positions of an image along x
+    const int cv = p.C / V;
+    const int64_t per_image = (int64_t)p.Ho * p.Wo * cv;
+    if (per_image >= (1ll << 31)) return hipErrorInvalidValue;
+    div_magic(p.Wo * cv, &p.row_magic, &p.row_shift);
+    div_magic(cv, &p.cv_magic, &p.cv_shift);
+    const dim3 grid((unsigned)((per_image + kThreads - 1) / kThreads), (unsigned)(p.N < 65535 ? p.N : 65535));
+    if (p.dt == DT_I8) {
+      if (p.is_max) hipLaunchKernelGGL(pool2d_q8_kernel<true>, grid, dim3(kThreads), 0, stream, p);
+      else hipLaunchKernelGGL(pool2d_q8_kernel<false>, grid, dim3(kThreads), 0, stream, p);
+      return hipGetLastError();
+    }
 #define POOL_LAUNCH(MAX_, KH_, KW_) \
-  FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((pool2d_vec_kernel<T, MAX_, KH_, KW_>), dim3(grid), dim3(kThreads), 0, stream, p))
+  FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((pool2d_vec_kernel<T, MAX_, KH_, KW_>), grid, dim3(kThreads), 0, stream, p))
     if (p.kh == 3 && p.kw == 3) { if (p.is_max) { POOL_LAUNCH(true, 3, 3); } else { POOL_LAUNCH(false, 3, 3); } }
     else if (p.kh == 2 && p.kw == 2) { if (p.is_max) { POOL_LAUNCH(true, 2, 2); } else { POOL_LAUNCH(false, 2, 2); } }
     else if (p.kh == 1 && p.kw == 1) { if (p.is_max) { POOL_LAUNCH(true, 1, 1); } else { POOL_LAUNCH(false, 1, 1); } }
