@@ -140,7 +140,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
   const int tid = wave * 64 + lane;
   const int l32 = lane & 31, lg = lane >> 5;
 
-  TOut* ybase = reinterpret_cast<TOut*>(p.y) + (int64_t)z * p.y_bs;
+  TOut* ybase = reinterpret_cast<TOut*>(p.y) + y_batch_off(p, z);
   const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
   const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
 
@@ -178,7 +178,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     }
   }
 
-  TOut* const ythr = ybase + (int64_t)(tile_m * BM + rp) * p.ycs + n;
+  TOut* const ythr = ybase + y_col_off(p, n);  // + the row's offset
   const TOut* const rthr = rbase ? rbase + (int64_t)(tile_m * BM + rp) * p.rcs + n : nullptr;
 
   using RVec = typename Epi::RVec;
@@ -262,7 +262,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
       }
       if (m < M && nvalid > 0) {
         // thread row pointer + a wavefront-uniform offset
-        TOut* yrow = ythr + (int64_t)(i * 32 + ps * 16) * p.ycs;
+        TOut* yrow = ythr + y_row_off(p, m);
         const TOut* rrow = rbase ? rthr + (int64_t)(i * 32 + ps * 16) * p.rcs : nullptr;
         Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rall[i][ps]);
       }
@@ -1108,6 +1108,11 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
   if (p.w_rows <= 0 || p.w_cols <= 0 || p.w_cols > p.w_rs) return hipErrorInvalidValue;
   if (p.w_cols % vec != 0) return hipErrorInvalidValue;
   if (p.residual != nullptr && p.rcs < p.Kout) return hipErrorInvalidValue;
+  if (p.y_rdiv > 0 || p.y_zdiv > 0) {
+    // remapped result addressing: float results without residual; eight consecutive columns stay together
+    if (!dtype_is_float(p.out_dt) || p.residual != nullptr) return hipErrorInvalidValue;
+    if (p.y_rdiv > 0 && (p.y_cdiv <= 0 || p.y_cdiv % 8 != 0 || p.Kout % p.y_cdiv != 0 || p.y_rlo < p.y_cdiv)) return hipErrorInvalidValue;
+  }
   if (p.w_frag != nullptr) {
     const int64_t kbytes = (int64_t)p.R * p.S * p.C * es;
     if (!aligned16(p.w_frag) || p.wf_chunks <= 0 || p.wf_chunks % 4 != 0 || (int64_t)p.wf_chunks * 32 < kbytes ||
@@ -1130,6 +1135,8 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
            ((reinterpret_cast<uintptr_t>(ptr) % (uintptr_t)vbytes) == 0);
   };
   int epi_vec = rows_ok(p.y, p.ycs, p.y_bs);
+  if (p.y_rdiv > 0) epi_vec = epi_vec && rows_ok(p.y, p.y_rlo, p.y_rhi) && rows_ok(p.y, p.y_chi, p.y_chi);
+  if (p.y_zdiv > 0) epi_vec = epi_vec && rows_ok(p.y, p.ycs, p.y_bs_hi);
   if (p.residual != nullptr) epi_vec = epi_vec && rows_ok(p.residual, p.rcs, p.r_bs);
   if (p.bias != nullptr) epi_vec = epi_vec && ((reinterpret_cast<uintptr_t>(p.bias) % 16) == 0) && (p.bias_bs % 4 == 0);
   if (oes == 1) {

@@ -10,6 +10,20 @@
 
 namespace ohip {
 
+// Element offset of result row m / column n / problem z (see IgemmParams::y_rdiv, y_zdiv).
+__device__ __forceinline__ int64_t y_row_off(const IgemmParams& p, const int m) {
+  if (p.y_rdiv > 0) return (int64_t)((unsigned)m / (unsigned)p.y_rdiv) * p.y_rhi + (int64_t)((unsigned)m % (unsigned)p.y_rdiv) * p.y_rlo;
+  return (int64_t)m * p.ycs;
+}
+__device__ __forceinline__ int64_t y_col_off(const IgemmParams& p, const int n) {
+  if (p.y_rdiv > 0) return (int64_t)((unsigned)n / (unsigned)p.y_cdiv) * p.y_chi + (int64_t)((unsigned)n % (unsigned)p.y_cdiv);
+  return n;
+}
+__device__ __forceinline__ int64_t y_batch_off(const IgemmParams& p, const int z) {
+  if (p.y_zdiv > 0) return (int64_t)(z / p.y_zdiv) * p.y_bs_hi + (int64_t)(z % p.y_zdiv) * p.y_bs;
+  return (int64_t)z * p.y_bs;
+}
+
 template <typename T> struct Mma;
 template <> struct Mma<float> {
   using Acc = floatx16;
@@ -426,7 +440,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
   const int wm = wave % (BM / WM), wn = wave / (BM / WM);
   const int l32 = lane & 31, lg = lane >> 5;
 
-  TOut* ybase = reinterpret_cast<TOut*>(p.y) + (int64_t)z * p.y_bs;
+  TOut* ybase = reinterpret_cast<TOut*>(p.y) + y_batch_off(p, z);
   const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
   const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
 
@@ -439,6 +453,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
   int nvalid = p.Kout - n;
   nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
   const bool vec = (epi_vec & 1) && nvalid == 8;
+  const int64_t ycol = y_col_off(p, n);
 
   // lane-constant epilogue operands: the lane's eight channels are the same in every pass
   AccE b8[8];
@@ -534,7 +549,7 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
         a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
       }
       if (m < M && nvalid > 0) {
-        TOut* yrow = ybase + (int64_t)m * p.ycs + n;
+        TOut* yrow = ybase + y_row_off(p, m) + ycol;
         const TOut* rrow = rbase ? rbase + (int64_t)m * p.rcs + n : nullptr;
         Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rcur[ps]);
       }

@@ -99,6 +99,15 @@ struct IgemmParams {
   int rcs = 0;                     // element stride between rows of residual
   int batch = 1;                   // grid.z: independent problems (groups, heads)
   int64_t x_bs = 0, w_bs = 0, y_bs = 0, r_bs = 0, bias_bs = 0;  // per-z element strides
+  // Result addressing beyond "row m at m * ycs" (float types, no residual), so that a
+  // transposition behind the GEMM costs nothing:
+  //   y_rdiv > 0: row m = (a, b) with b = m % y_rdiv lies at a * y_rhi + b * y_rlo, and
+  //               column n = (c, d) with d = n % y_cdiv at c * y_chi + d - a [B*S, heads*d]
+  //               result stored as [B, heads, S, d];
+  //   y_zdiv > 0: problem z = (u, v) with v = z % y_zdiv starts at u * y_bs_hi + v * y_bs -
+  //               a [B*heads] batch of [S, d] results stored as [B, S, heads, d] (ycs = heads*d).
+  int y_rdiv = 0, y_cdiv = 1, y_zdiv = 0;
+  int64_t y_rhi = 0, y_rlo = 0, y_chi = 0, y_bs_hi = 0;
   DType in_dt = DT_F32;            // type of x and w
   DType out_dt = DT_F32;           // type of y and residual
   // Optional copy of w in MFMA fragment order (see WfragPackParams); when set,

@@ -499,6 +499,12 @@ class Planner {
                    int64_t so, int64_t si, int64_t sr, int64_t ss, const std::vector<float>& row_scale,
                    int* w_rs_out, const std::vector<float>* wq_scale, int dense_groups = 0);
   int make_wfrag(const std::string& name, IgemmParams* ip, int tw);
+  // A value whose only use is Reshape -> [B, S, heads, d] -> Transpose (0, 2, 1, 3): the
+  // GEMM that computes it can store [B, heads, S, d] directly (IgemmParams::y_rdiv).
+  struct HeadSplit { int reshape = -1, transpose = -1; int64_t B = 0, S = 0, heads = 0, d = 0; _odla_value* out = nullptr; };
+  bool head_split_behind(const _odla_value* v, int64_t rows, int64_t cols, HeadSplit* hs) const;
+  // The Transpose (0, 2, 1, 3) that is the only use of a rank-4 value, or -1.
+  int head_merge_behind(const _odla_value* v) const;
   void finish_igemm(const std::string& name, IgemmParams ip, int tx, int tw, int ty, const Epilogue& ep,
                     int64_t Kout_total);
   int strided_copy_step(const std::string& name, int src, int dst, const StridedCopyParams& cp_in);
@@ -1401,6 +1407,33 @@ bool Planner::gemm_epilogue(int ni, Epilogue* ep) {
   return full_c == nullptr;
 }
 
+bool Planner::head_split_behind(const _odla_value* v, int64_t rows, int64_t cols, HeadSplit* hs) const {
+  if (calib_ || v == nullptr || v->is_output || consumers_[v->index].size() != 1) return false;
+  const int ri = consumers_[v->index][0];
+  const Node& r = comp_->nodes[ri];
+  if (r.op != OP_RESHAPE || r.absorbed || r.out->is_output || r.out->shape.rank != 4) return false;
+  const Shape& s4 = r.out->shape;
+  if (s4.d[0] * s4.d[1] != rows || s4.d[2] * s4.d[3] != cols || s4.d[3] % 8 != 0) return false;
+  if (consumers_[r.out->index].size() != 1) return false;
+  const int ti = consumers_[r.out->index][0];
+  const Node& t = comp_->nodes[ti];
+  if (t.op != OP_TRANSPOSE || t.absorbed || t.out->is_output || t.iv.size() != 4) return false;
+  if (t.iv[0] != 0 || t.iv[1] != 2 || t.iv[2] != 1 || t.iv[3] != 3) return false;
+  hs->reshape = ri; hs->transpose = ti;
+  hs->B = s4.d[0]; hs->S = s4.d[1]; hs->heads = s4.d[2]; hs->d = s4.d[3];
+  hs->out = t.out;
+  return true;
+}
+
+int Planner::head_merge_behind(const _odla_value* v) const {
+  if (calib_ || v == nullptr || v->is_output || v->shape.rank != 4 || consumers_[v->index].size() != 1) return -1;
+  const int ti = consumers_[v->index][0];
+  const Node& t = comp_->nodes[ti];
+  if (t.op != OP_TRANSPOSE || t.absorbed || t.iv.size() != 4) return -1;
+  if (t.iv[0] != 0 || t.iv[1] != 2 || t.iv[2] != 1 || t.iv[3] != 3) return -1;
+  return ti;
+}
+
 void Planner::lower_gemm(int ni) {
   if (ni < (int)gemm_merged_.size() && gemm_merged_[ni]) return;  // computed by an earlier sibling's launch
   Node& n = comp_->nodes[ni];
@@ -1539,11 +1572,29 @@ void Planner::lower_gemm(int ni) {
     Epilogue eall = ep;
     eall.has_bias = any_bias;
     eall.bias = bias_all;
+    // Every member feeds Reshape -> Transpose into [B, heads, S, d] (the head split of an
+    // attention block): the launch stores that order itself and the transposes vanish.
+    std::vector<HeadSplit> hs((size_t)G);
+    bool split = true;
+    for (int g = 0; g < G && split; ++g) {
+      split = head_split_behind(group_ep[g].final_value, lead * M, Nn, &hs[g]);
+      if (split && g > 0) split = hs[g].S == hs[0].S && hs[g].d == hs[0].d && hs[g].heads == hs[0].heads;
+    }
+    if (split) {
+      ip.y_rdiv = (int)hs[0].S; ip.y_rlo = hs[0].d; ip.y_rhi = hs[0].heads * hs[0].S * hs[0].d;
+      ip.y_cdiv = (int)hs[0].d; ip.y_chi = hs[0].S * hs[0].d;
+    }
     finish_igemm("gemm.x" + std::to_string(G) + ":" + outv->name, ip, ta, twc, tall, eall, (int64_t)G * Nn);
     if (gemm_merged_.size() < comp_->nodes.size()) gemm_merged_.resize(comp_->nodes.size(), 0);
     const size_t slice_bytes = (size_t)(lead * M * Nn) * dtype_size(dt);
     for (int g = 0; g < G; ++g) {
-      set_main(group_ep[g].final_value, view_tensor(tall, group_ep[g].final_value->shape, (size_t)g * slice_bytes));
+      if (split) {
+        set_main(hs[g].out, view_tensor(tall, hs[g].out->shape, (size_t)g * slice_bytes));
+        comp_->nodes[hs[g].reshape].absorbed = true;
+        comp_->nodes[hs[g].transpose].absorbed = true;
+      } else {
+        set_main(group_ep[g].final_value, view_tensor(tall, group_ep[g].final_value->shape, (size_t)g * slice_bytes));
+      }
       if (g > 0) gemm_merged_[group[g]] = 1;
     }
     return;
@@ -1645,6 +1696,33 @@ void Planner::lower_gemm(int ni) {
     else {
       ip.N = (int)M; ip.batch = (int)lead;
       ip.x_bs = M * Kp; ip.w_bs = Nn * Kp; ip.y_bs = M * Nn; ip.r_bs = M * Nn; ip.bias_bs = 0;
+    }
+  }
+  if (ep.residual == nullptr) {
+    HeadSplit hs;
+    if (ip.batch == 1 && head_split_behind(outv, lead * M, Nn, &hs)) {
+      // [B*S, heads*d] stored as [B, heads, S, d]: the Reshape -> Transpose behind it costs nothing
+      ip.y_rdiv = (int)hs.S; ip.y_rlo = hs.d; ip.y_rhi = hs.heads * hs.S * hs.d;
+      ip.y_cdiv = (int)hs.d; ip.y_chi = hs.S * hs.d;
+      const int ty = new_tensor(dt, L_ROWMAJOR, hs.out->shape, 0, SP_ARENA);
+      finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
+      set_main(hs.out, ty);
+      comp_->nodes[hs.reshape].absorbed = true;
+      comp_->nodes[hs.transpose].absorbed = true;
+      return;
+    }
+    const int ti = ip.batch > 1 && os.rank == 4 && outv->shape == os ? head_merge_behind(outv) : -1;
+    if (ti >= 0) {
+      // a [B*heads] batch of [S, d] results stored as [B, S, heads, d]: the head merge behind
+      // an attention block's context product
+      Node& t = comp_->nodes[ti];
+      const int64_t heads = os.d[1], S = os.d[2], d = os.d[3];
+      ip.y_zdiv = (int)heads; ip.y_bs_hi = S * heads * d; ip.y_bs = d; ip.ycs = (int)(heads * d);
+      const int ty = new_tensor(dt, L_ROWMAJOR, t.out->shape, 0, SP_ARENA);
+      finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
+      set_main(t.out, ty);
+      t.absorbed = true;
+      return;
     }
   }
   const int ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
