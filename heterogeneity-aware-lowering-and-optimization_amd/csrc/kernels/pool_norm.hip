@@ -300,6 +300,89 @@ reduce_cols_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t out
     for (int e = 0; e < V; ++e) Store<TO>::st(y + o * inner + in + e, red_final(acc[e], len, kind, eps));
   }
 }
+// Few columns and many rows (a global pool over a large image, a mean over a
+// long sequence): one thread per column leaves most of the chip idle.  Here a
+// workgroup owns `cl` 16-byte column groups of one outer index, its NT / cl
+// thread rows stride the reduced axis, and the partial results meet in LDS.
+template <typename TI, typename TO, int A, int NT>
+__global__ void __launch_bounds__(NT)
+reduce_cols_split_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t len, int64_t inner,
+                         int cl, ReduceKind kind, float eps) {
+  constexpr int V = Vec16<TI>::N;
+  __shared__ float part[NT * V];
+  const int c = threadIdx.x % cl, s = threadIdx.x / cl, S = NT / cl;
+  const int64_t iv = inner / V;
+  const int64_t cv = blockIdx.x * (int64_t)cl + c;
+  const int64_t o = blockIdx.y;
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = red_init<A>();
+  if (cv < iv) {
+    const TI* col = x + o * len * inner + cv * V;
+    int64_t k = s;
+    for (; k + 3 * (int64_t)S < len; k += 4 * (int64_t)S) {
+      Vec16<TI> v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u].load(col + (k + u * (int64_t)S) * inner);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] = red_step<A>(acc[e], v[u].get(e));
+    }
+    for (; k < len; k += S) {
+      Vec16<TI> v;
+      v.load(col + k * inner);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = red_step<A>(acc[e], v.get(e));
+    }
+  }
+  const int width = cl * V;
+#pragma unroll
+  for (int e = 0; e < V; ++e) part[s * width + c * V + e] = acc[e];
+  __syncthreads();
+  for (int j = threadIdx.x; j < width; j += NT) {
+    const int64_t col = blockIdx.x * (int64_t)width + j;
+    if (col >= inner) break;
+    float r = part[j];
+    for (int t = 1; t < S; ++t) r = red_merge<A>(r, part[t * width + j]);
+    Store<TO>::st(y + o * inner + col, red_final(r, len, kind, eps));
+  }
+}
+// Few long rows (inner == 1): a workgroup per row, 16-byte loads.
+template <typename TI, typename TO, int A>
+__global__ void __launch_bounds__(kThreads)
+reduce_row_block_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t len, ReduceKind kind, float eps) {
+  constexpr int V = Vec16<TI>::N;
+  __shared__ float part[kThreads / 64];
+  const TI* row = x + blockIdx.x * len;
+  const int64_t nv = len / V;
+  float acc = red_init<A>();
+  int64_t i = threadIdx.x;
+  for (; i + 3 * kThreads < nv; i += 4 * kThreads) {
+    Vec16<TI> v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u].load(row + (i + u * kThreads) * V);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc = red_step<A>(acc, v[u].get(e));
+  }
+  for (; i < nv; i += kThreads) {
+    Vec16<TI> v;
+    v.load(row + i * V);
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc = red_step<A>(acc, v.get(e));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc = red_merge<A>(acc, __shfl_xor(acc, o, 64));
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float r = part[0];
+    for (int w = 1; w < kThreads / 64; ++w) r = red_merge<A>(r, part[w]);
+    Store<TO>::st(y + blockIdx.x, red_final(r, len, kind, eps));
+  }
+}
 // Index of the extreme value along the middle axis; one thread per (outer,
 // inner) column.  Ties keep the first index, or the last when `last` is set.
 template <typename TI, typename TO>
@@ -332,6 +415,41 @@ reduce_cols_q8_kernel(const int8_t* __restrict__ x, float* __restrict__ y, int64
     int acc = 0;
     for (int64_t k = 0; k < len; ++k) acc += q_from_stored(col[k * inner]);
     y[i] = ((float)(acc - (int)len * zp) / (float)len) * scale;
+  }
+}
+
+// The same with 16 columns per thread and the rows of one outer index split
+// over the workgroup (the global pool behind a quantised backbone: 49 rows).
+__global__ void __launch_bounds__(kThreads)
+reduce_cols_q8_split_kernel(const int8_t* __restrict__ x, float* __restrict__ y, int64_t len,
+                            int64_t inner, int cl, float scale, int zp) {
+  __shared__ int part[kThreads * 16];
+  const int c = threadIdx.x % cl, s = threadIdx.x / cl, S = kThreads / cl;
+  const int64_t iv = inner / 16;
+  const int64_t cv = blockIdx.x * (int64_t)cl + c;
+  const int64_t o = blockIdx.y;
+  int acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+  if (cv < iv) {
+    const int8_t* col = x + o * len * inner + cv * 16;
+    for (int64_t k = s; k < len; k += S) {
+      const uintx4 v = *reinterpret_cast<const uintx4*>(col + k * inner);
+      const int8_t* b = reinterpret_cast<const int8_t*>(&v);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[e] += q_from_stored(b[e]);
+    }
+  }
+  const int width = cl * 16;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) part[s * width + c * 16 + e] = acc[e];
+  __syncthreads();
+  for (int j = threadIdx.x; j < width; j += kThreads) {
+    const int64_t col = blockIdx.x * (int64_t)width + j;
+    if (col >= inner) break;
+    int r = part[j];
+    for (int t = 1; t < S; ++t) r += part[t * width + j];
+    y[o * inner + col] = ((float)(r - (int)len * zp) / (float)len) * scale;
   }
 }
 
@@ -716,9 +834,24 @@ hipError_t launch_pool2d(const PoolParams& p_in, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Below this many column threads (half the chip's resident threads at 512 per
+// CU) the reductions split the reduced axis over the workgroup as well.
+static constexpr int64_t kSplitBelow = 256 * 512;
+static int split_columns(int64_t groups) {
+  int cl = 64;
+  while (cl > 1 && cl > groups) cl >>= 1;
+  return cl;
+}
+
 hipError_t launch_reduce_q8_mean(const void* x, float* y, int64_t outer, int64_t len, int64_t inner,
                                  float scale, int zp, hipStream_t stream) {
   if (!x || !y || outer <= 0 || len <= 0 || inner <= 0 || len > (1 << 23)) return hipErrorInvalidValue;
+  if (inner % 16 == 0 && al16(x) && outer * (inner / 16) < kSplitBelow && len >= 8 && outer <= 65535) {
+    const int cl = split_columns(inner / 16);
+    hipLaunchKernelGGL(reduce_cols_q8_split_kernel, dim3((unsigned)((inner / 16 + cl - 1) / cl), (unsigned)outer),
+                       dim3(kThreads), 0, stream, (const int8_t*)x, y, len, inner, cl, scale, zp);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(reduce_cols_q8_kernel, dim3(grid_for(outer * inner, kThreads)), dim3(kThreads), 0,
                      stream, (const int8_t*)x, y, outer, len, inner, scale, zp);
   return hipGetLastError();
@@ -730,7 +863,21 @@ static hipError_t reduce_out(const void* x, void* y, DType out_dt, int64_t outer
   auto go = [&](auto tag, auto rule) -> hipError_t {
     using TO = decltype(tag);
     constexpr int A = decltype(rule)::value;
-    if (inner == 1) {
+    constexpr int V = 16 / (int)sizeof(TI);
+    if (inner == 1 && outer <= 2048 && len >= 16384 && len % V == 0 && al16(x)) {
+      hipLaunchKernelGGL((reduce_row_block_kernel<TI, TO, A>), dim3((unsigned)outer), dim3(kThreads), 0, stream,
+                         (const TI*)x, (TO*)y, len, kind, eps);
+    } else if (inner > 1 && inner % V == 0 && al16(x) && outer * (inner / V) < kSplitBelow && len >= 32 &&
+               outer <= 65535) {
+      const int cl = split_columns(inner / V);
+      const dim3 grid((unsigned)((inner / V + cl - 1) / cl), (unsigned)outer);
+      if (len >= 1024)
+        hipLaunchKernelGGL((reduce_cols_split_kernel<TI, TO, A, 1024>), grid, dim3(1024), 0, stream,
+                           (const TI*)x, (TO*)y, len, inner, cl, kind, eps);
+      else
+        hipLaunchKernelGGL((reduce_cols_split_kernel<TI, TO, A, kThreads>), grid, dim3(kThreads), 0, stream,
+                           (const TI*)x, (TO*)y, len, inner, cl, kind, eps);
+    } else if (inner == 1) {
       const int grid = grid_for(outer * 64, kThreads);
       hipLaunchKernelGGL((reduce_rows_kernel<TI, TO, A>), dim3(grid), dim3(kThreads), 0, stream,
                          (const TI*)x, (TO*)y, outer, len, kind, eps);

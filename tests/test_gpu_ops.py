@@ -625,6 +625,38 @@ def test_reduce_parity():
         assert max_rel_err(got[k], want[k]) <= 1e-5, k
 
 
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def test_reduce_few_columns_parity(mode):
+    """Reductions with too few columns to give every thread one: the rows of the
+    reduced axis are split over the workgroup (long and short axes, a ragged
+    column count, rows of a plain matrix)."""
+    announce("reduce, split rows (%s)" % mode)
+    r = rng(53)
+    x1 = r.standard_normal((2, 64, 40, 40)).astype(np.float32)
+    x2 = r.standard_normal((4, 256, 7, 7)).astype(np.float32)
+    x3 = r.standard_normal((2, 48, 6, 6)).astype(np.float32)
+    x4 = r.standard_normal((3, 40000)).astype(np.float32)
+
+    def build(b):
+        for name, x in (("a", x1), ("b", x2), ("c", x3)):
+            a = b.arg(name, x.shape)
+            cl = b.maxpool(a, (1, 1), (1, 1), (0, 0, 0, 0), name=name + "_cl")   # channels-last on the device
+            b.output(b.reduce_mean(cl, (2, 3), True, name=name + "_mean"), name + "_mean")
+            b.output(b.reduce_max(cl, (2, 3), False, name=name + "_max"), name + "_max")
+            b.output(b.reduce_sum(a, (2, 3), False, name=name + "_sum"), name + "_sum")
+        d = b.arg("d", x4.shape)
+        b.output(b.reduce_max(d, (1,), False, name="d_max"), "d_max")
+        b.output(b.reduce_mean(d, (1,), True, name="d_mean"), "d_mean")
+
+    got, want = run_both(build, {"a": x1, "b": x2, "c": x3, "d": x4}, fp16=(mode == "fp16"))
+    for k in want:
+        assert got[k].shape == want[k].shape, k
+        if mode == "fp32":
+            assert np.max(np.abs(got[k] - want[k])) <= 1e-5 * max(1.0, float(np.max(np.abs(want[k])))), k
+        else:   # inputs and results rounded to fp16, sums kept in fp32
+            assert np.max(np.abs(got[k] - want[k])) <= 2e-3 * max(1.0, float(np.max(np.abs(want[k])))), k
+
+
 # --------------------------------------------------------------------------
 # Data movement
 # --------------------------------------------------------------------------
