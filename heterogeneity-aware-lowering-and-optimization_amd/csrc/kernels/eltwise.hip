@@ -437,6 +437,70 @@ __global__ void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
 }
 
 bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// One launch for a group of unary / binary operators (see FusedParams).  The
+// registers of the program live in LDS, one column per thread, because the
+// program addresses them at run time.  A thread runs every instruction for E
+// consecutive points of its walk at once (register q, point e at
+// regs[(q * E + e) * kThreads + thread]): the E loads of an instruction are in
+// flight together and the decoding of the instruction is shared.
+template <typename T, int E>
+__global__ void __launch_bounds__(kThreads) fused_eltwise_kernel(const FusedParams p) {
+  extern __shared__ float fused_regs[];
+  float* r = fused_regs + threadIdx.x;
+  const int64_t d1 = p.dims[1], d2 = p.dims[2], d3 = p.dims[3];
+  const int64_t walk = p.walk > 0 ? p.walk : d2;
+  const int64_t pieces = (d2 + walk - 1) / walk;
+  const int64_t total = p.dims[0] * d1 * pieces * d3;
+  for (int64_t t = blockIdx.x * (int64_t)kThreads + threadIdx.x; t < total; t += (int64_t)gridDim.x * kThreads) {
+    const int64_t i3 = t % d3;
+    int64_t q = t / d3;
+    const int64_t piece = q % pieces;
+    q /= pieces;
+    const int64_t i1 = q % d1, i0 = q / d1;
+    const int64_t i2_end = piece * walk + walk < d2 ? piece * walk + walk : d2;
+    for (int64_t i2 = piece * walk; i2 < i2_end; i2 += E) {
+      const int live = i2_end - i2 < E ? (int)(i2_end - i2) : E;
+      for (int k = 0; k < p.n_instr; ++k) {
+        const FusedInstr& in = p.prog[k];
+        switch (in.op) {
+          case FOP_LOAD: {
+            const FusedView& v = p.view[in.a];
+            const T* src = reinterpret_cast<const T*>(v.base) + v.off + i0 * v.st[0] + i1 * v.st[1] + i2 * v.st[2] + i3 * v.st[3];
+            float val[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) val[e] = e < live ? Store<T>::ld(src + e * v.st[2]) : 0.f;
+#pragma unroll
+            for (int e = 0; e < E; ++e) r[(in.dst * E + e) * kThreads] = val[e];
+            break;
+          }
+          case FOP_UNARY:
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+              r[(in.dst * E + e) * kThreads] = apply_act(r[(in.a * E + e) * kThreads], (ActKind)in.kind, in.fa, in.fb);
+            break;
+          case FOP_BINARY:   // a negative register number selects the immediate
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+              const float lhs = in.a < 0 ? in.fa : r[(in.a * E + e) * kThreads];
+              const float rhs = in.b < 0 ? in.fa : r[(in.b * E + e) * kThreads];
+              r[(in.dst * E + e) * kThreads] = bin_op(lhs, rhs, (BinKind)in.kind);
+            }
+            break;
+          default: {
+            const FusedView& v = p.view[in.dst];
+            T* dst = const_cast<T*>(reinterpret_cast<const T*>(v.base)) + v.off + i0 * v.st[0] + i1 * v.st[1] + i2 * v.st[2] + i3 * v.st[3];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+              if (e < live) Store<T>::st(dst + e * v.st[2], r[(in.a * E + e) * kThreads]);
+            break;
+          }
+        }
+      }
+    }
+  }
+}
+
 }  // namespace
 
 #define FLOAT_DISPATCH(dt, EXPR)                         \
@@ -656,6 +720,40 @@ hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t stream)
   if (n <= 0) return n == 0 ? hipSuccess : hipErrorInvalidValue;
   if (!p) return hipErrorInvalidValue;
   hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(n, 256)), dim3(256), 0, stream, p, n, v);
+  return hipGetLastError();
+}
+
+hipError_t launch_fused_eltwise(const FusedParams& p, hipStream_t stream) {
+  if (p.n_instr <= 0 || p.n_instr > kFusedMaxInstr) return hipErrorInvalidValue;
+  int64_t threads = 1;
+  for (int i = 0; i < 4; ++i) {
+    if (p.dims[i] <= 0) return hipErrorInvalidValue;
+    if (i != 2) threads *= p.dims[i];
+  }
+  if (p.walk < 0) return hipErrorInvalidValue;
+  const int64_t walk = p.walk > 0 ? p.walk : p.dims[2];
+  threads *= (p.dims[2] + walk - 1) / walk;
+  for (int k = 0; k < p.n_instr; ++k) {
+    const FusedInstr& in = p.prog[k];
+    const bool is_store = in.op == FOP_STORE, is_load = in.op == FOP_LOAD;
+    const int view = is_store ? in.dst : in.a;
+    if ((is_store || is_load) && (view < 0 || view >= kFusedMaxViews || p.view[view].base == nullptr)) return hipErrorInvalidValue;
+    if (!is_store && (in.dst < 0 || in.dst >= kFusedMaxRegs)) return hipErrorInvalidValue;
+    const bool is_bin = in.op == FOP_BINARY;
+    if (!is_load && (in.a >= kFusedMaxRegs || (in.a < 0 && !is_bin))) return hipErrorInvalidValue;
+    if (is_bin && (in.b >= kFusedMaxRegs || (in.a < 0 && in.b < 0))) return hipErrorInvalidValue;
+    if (in.op < FOP_LOAD || in.op > FOP_STORE) return hipErrorInvalidValue;
+  }
+  int n_regs = 1;
+  for (int k = 0; k < p.n_instr; ++k)
+    if (p.prog[k].op != FOP_STORE && p.prog[k].dst + 1 > n_regs) n_regs = p.prog[k].dst + 1;
+  // points of the walk per instruction: as many as 32 KiB of LDS registers allow
+  const int e = (walk >= 4 && n_regs * 4 <= 32) ? 4 : ((walk >= 2 && n_regs * 2 <= 32) ? 2 : 1);
+  const size_t lds = (size_t)n_regs * e * kThreads * sizeof(float);
+  const int grid = grid_for(threads, kThreads);
+  if (e == 4) { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, 4>), dim3(grid), dim3(kThreads), lds, stream, p)); }
+  else if (e == 2) { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, 2>), dim3(grid), dim3(kThreads), lds, stream, p)); }
+  else { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, 1>), dim3(grid), dim3(kThreads), lds, stream, p)); }
   return hipGetLastError();
 }
 

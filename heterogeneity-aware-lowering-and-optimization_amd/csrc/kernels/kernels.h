@@ -254,6 +254,39 @@ struct BinaryParams {
 };
 hipError_t launch_binary(const BinaryParams& p, hipStream_t stream);
 
+// A connected group of float unary / binary operators run as one launch.
+// Every thread evaluates the whole group for one point of the iteration space
+// dims[0..3]: threads enumerate (dims[0], dims[1], pieces of dims[2], dims[3])
+// with dims[3] fastest and walk their piece of dims[2] themselves, so that the
+// planner can give stores a unit stride across threads and loads a unit stride
+// along a thread's walk.
+// The group is a short program over per-thread registers: loads and stores go
+// through views (base pointer, element offset, one element stride per dim; a
+// stride of 0 broadcasts), all of storage type `dt`; arithmetic is fp32.
+enum FusedOp : int { FOP_LOAD = 0, FOP_UNARY, FOP_BINARY, FOP_STORE };
+struct FusedView {
+  const void* base = nullptr;   // stores cast the const away
+  int64_t off = 0;
+  int64_t st[4] = {0, 0, 0, 0};
+};
+struct FusedInstr {
+  int op = FOP_LOAD;   // FusedOp
+  int dst = 0;         // register written (FOP_STORE: view index)
+  int a = 0, b = 0;    // registers read (FOP_LOAD: a = view index; FOP_BINARY: -1 = the immediate fa)
+  int kind = 0;        // ActKind / BinKind
+  float fa = 0.f, fb = 0.f;   // FOP_UNARY: the activation's parameters
+};
+constexpr int kFusedMaxRegs = 32, kFusedMaxViews = 24, kFusedMaxInstr = 64;
+struct FusedParams {
+  DType dt = DT_F32;
+  int n_instr = 0;
+  int64_t dims[4] = {1, 1, 1, 1};
+  int64_t walk = 0;    // points of dims[2] per thread (0: all of them); short walks give more threads
+  FusedView view[kFusedMaxViews];
+  FusedInstr prog[kFusedMaxInstr];
+};
+hipError_t launch_fused_eltwise(const FusedParams& p, hipStream_t stream);
+
 // Typed element-wise operators with broadcast (row-major operands, up to 6
 // collapsed dims, one element stride per dim and operand, 0 where it
 // broadcasts).  EW_ADD .. EW_SQDIFF: y has the operands' type `dt` (float types

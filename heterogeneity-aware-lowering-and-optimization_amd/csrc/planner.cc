@@ -167,6 +167,10 @@ class Planner {
 
   void emit(const std::string& name, std::initializer_list<int> reads, std::initializer_list<int> writes,
             std::function<hipError_t(const ExecEnv&, hipStream_t)> fn) {
+    emit_lists(name, std::vector<int>(reads), std::vector<int>(writes), std::move(fn));
+  }
+  void emit_lists(const std::string& name, const std::vector<int>& reads, const std::vector<int>& writes,
+                  std::function<hipError_t(const ExecEnv&, hipStream_t)> fn) {
     if (in_init_) {
       plan_->init_steps.push_back({name, std::move(fn)});
       return;
@@ -482,9 +486,13 @@ class Planner {
   void lower_lrn(int ni);
   void lower_rownorm(int ni);
   void lower_postprocess(int ni);
+  bool lower_fused_group(int seed, int from);
+  bool fuse_slice_seed(int ni) const;
+  bool fuse_candidate(int ni) const;
   bool gemm_epilogue(int ni, Epilogue* ep);
   std::unordered_map<int, Epilogue> gemm_ep_ahead_;  // epilogues collected while looking for sibling GEMMs
   std::vector<char> gemm_merged_;                    // nodes already lowered inside a sibling's launch
+  std::vector<char> no_fuse_;                        // nodes of an element-wise group that was given up
   void emit_stats(const _odla_value* v, const char* op_type, int forced_axis, const Node* producer);
   bool calib_ = false;
   struct SoftmaxAdd { const _odla_value* x; const _odla_value* mask; int64_t div; };
@@ -641,6 +649,12 @@ void Planner::run() {
   }
   for (size_t ni = 0; ni < comp_->nodes.size(); ++ni) {
     if (comp_->nodes[ni].absorbed) continue;
+    if (!calib_ && !o.int8) {
+      if (fuse_candidate((int)ni) && lower_fused_group((int)ni, (int)ni)) continue;
+      if (fuse_slice_seed((int)ni) && lower_fused_group(consumers_[comp_->nodes[ni].out->index][0], (int)ni) &&
+          comp_->nodes[ni].absorbed)
+        continue;
+    }
     lower((int)ni);
     if (calib_) {
       const Node& n = comp_->nodes[ni];
@@ -2023,6 +2037,407 @@ void Planner::lower_unary(int ni) {
     return launch_unary(a(e), b(e), dt, ne, act, fa, fb, st);
   });
   set_main(n.out, ty);
+}
+
+// ------------------------------------------- element-wise group fusion ----
+// Float unary / binary operators on values of rank <= 3 (rank-4 values belong
+// to the convolution epilogues and may live channels-last) that feed each other
+// run as one launch: launch_fused_eltwise evaluates the whole group per element.
+// Slices of available tensors become strided loads; a Concat of group results
+// or a Transpose of one becomes a strided store.  The group is emitted at its
+// first operator, so every outside operand must already be available there;
+// whatever does not fit is left to the ordinary one-launch-per-operator path.
+bool Planner::fuse_candidate(int ni) const {
+  const Node& n = comp_->nodes[ni];
+  if (n.absorbed || (!no_fuse_.empty() && no_fuse_[ni])) return false;
+  if (n.op != OP_UNARY && n.op != OP_BINARY) return false;
+  const Shape& os = n.out->shape;
+  if (os.rank < 1 || os.rank > 3) return false;
+  const DType dt = storage_dtype(n.out);
+  if (!dtype_is_float(dt)) return false;
+  for (const _odla_value* v : n.in)
+    if (v == nullptr || storage_dtype(v) != dt || v->shape.rank > 3) return false;
+  return true;
+}
+
+// A Slice met before the operators that read it: the first of them seeds the group.
+bool Planner::fuse_slice_seed(int ni) const {
+  const Node& n = comp_->nodes[ni];
+  if (n.op != OP_SLICE || n.absorbed || n.out->is_output || consumers_[n.out->index].empty()) return false;
+  if (n.out->shape.rank > 3 || !dtype_is_float(storage_dtype(n.out))) return false;
+  return fuse_candidate(consumers_[n.out->index][0]);
+}
+
+// `seed`: the operator the group grows from; `from` <= seed: the node being
+// lowered, where the group's launch is emitted.
+bool Planner::lower_fused_group(int seed, int from) {
+  const int n_nodes = (int)comp_->nodes.size();
+  if (no_fuse_.empty()) no_fuse_.assign((size_t)n_nodes, 0);
+  const int scan_end = std::min(n_nodes, seed + 512);
+  const DType dt = storage_dtype(comp_->nodes[seed].out);
+
+  // ---- operators and slices that could run at the seed's position
+  std::unordered_map<const _odla_value*, int> member_of, slice_of;
+  for (int j = from; j < scan_end; ++j) {
+    const Node& n = comp_->nodes[j];
+    if (n.absorbed) continue;
+    if (n.op == OP_SLICE && n.out->shape.rank <= 3 && !n.out->is_output && storage_dtype(n.out) == dt &&
+        dtype_is_float(dt) && available(n.in[0]) && !consumers_[n.out->index].empty()) {
+      bool ok = true;
+      for (int c : consumers_[n.out->index]) ok = ok && (comp_->nodes[c].op == OP_UNARY || comp_->nodes[c].op == OP_BINARY);
+      if (ok) slice_of[n.out] = j;
+      continue;
+    }
+    if (!fuse_candidate(j) || storage_dtype(n.out) != dt) continue;
+    bool ok = true;
+    for (const _odla_value* v : n.in) ok = ok && (member_of.count(v) || slice_of.count(v) || available(v));
+    if (ok) member_of[n.out] = j;
+  }
+  {
+    auto m = member_of.find(comp_->nodes[seed].out);
+    if (m == member_of.end() || m->second != seed) return false;   // an operand of the seed is not ready here
+  }
+  // ---- the connected part that holds the seed
+  std::vector<int> members;
+  std::vector<int> slices;
+  {
+    std::vector<char> seen((size_t)n_nodes, 0);
+    std::vector<int> todo{seed};
+    seen[seed] = 1;
+    auto push = [&](int j) { if (!seen[j]) { seen[j] = 1; todo.push_back(j); } };
+    while (!todo.empty()) {
+      const int j = todo.back();
+      todo.pop_back();
+      const Node& n = comp_->nodes[j];
+      if (n.op == OP_SLICE) {
+        slices.push_back(j);
+        for (int c : consumers_[n.out->index]) if (member_of.count(comp_->nodes[c].out) && member_of[comp_->nodes[c].out] == c) push(c);
+        continue;
+      }
+      members.push_back(j);
+      for (const _odla_value* v : n.in) {
+        auto m = member_of.find(v);
+        if (m != member_of.end()) push(m->second);
+        auto sl = slice_of.find(v);
+        if (sl != slice_of.end()) push(sl->second);
+      }
+      for (int c : consumers_[n.out->index]) {
+        const Node& cn = comp_->nodes[c];
+        auto m = member_of.find(cn.out);
+        if (m != member_of.end() && m->second == c) push(c);
+        if (cn.op == OP_CONCAT && !cn.absorbed) {   // the parts of a Concat belong together
+          bool all = true;
+          for (const _odla_value* ci : cn.in) all = all && member_of.count(ci);
+          if (all) for (const _odla_value* ci : cn.in) push(member_of[ci]);
+        }
+      }
+    }
+  }
+  std::sort(members.begin(), members.end());
+  auto give_up = [&]() { for (int j : members) no_fuse_[j] = 1; return false; };
+  if (members.size() < 2) return give_up();
+  std::unordered_map<const _odla_value*, int> in_group;   // value -> member node
+  for (int j : members) in_group[comp_->nodes[j].out] = j;
+  for (int j : slices)
+    for (int c : consumers_[comp_->nodes[j].out->index])
+      if (!in_group.count(comp_->nodes[c].out) || in_group[comp_->nodes[c].out] != c) return give_up();
+
+  // ---- iteration space: every member's shape, right-aligned, is 1 or S per dim
+  int R = 1;
+  for (int j : members) R = std::max(R, comp_->nodes[j].out->shape.rank);
+  auto padded = [&](const Shape& sh) {
+    Shape o;
+    o.rank = R;
+    for (int i = 0; i < R; ++i) o.d[i] = 1;
+    for (int i = 0; i < sh.rank; ++i) o.d[R - sh.rank + i] = sh.d[i];
+    return o;
+  };
+  Shape S = padded(comp_->nodes[members[0]].out->shape);
+  for (int j : members) {
+    const Shape p = padded(comp_->nodes[j].out->shape);
+    for (int i = 0; i < R; ++i) S.d[i] = std::max(S.d[i], p.d[i]);
+  }
+  for (int j : members) {
+    const Shape p = padded(comp_->nodes[j].out->shape);
+    for (int i = 0; i < R; ++i) if (p.d[i] != 1 && p.d[i] != S.d[i]) return give_up();
+  }
+  // operand shape as the consuming operator aligns it
+  auto aligned_operand = [&](const Node& n, int k) {
+    if (n.op == OP_UNARY) return n.in[0]->shape;
+    const int r = (int)n.iv[0];
+    Shape a;
+    a.rank = r;
+    for (int i = 0; i < r; ++i) a.d[i] = n.iv[1 + k * r + i];
+    return a;
+  };
+
+  // ---- program over virtual registers
+  struct View { int tensor = -1; const _odla_value* value = nullptr; int64_t off = 0; int64_t st[3] = {0, 0, 0}; bool store = false; };
+  std::vector<View> views;
+  struct VI { int op, dst, a, b, kind; float fa, fb; };
+  std::vector<VI> prog;
+  std::unordered_map<const _odla_value*, int> reg_of;   // member result or loaded operand -> virtual register
+  int n_vregs = 0;
+  struct PendingLoad { const _odla_value* v; Shape aligned; int reg; };
+  std::vector<PendingLoad> loads;
+  for (int j : members) {
+    const Node& n = comp_->nodes[j];
+    int src[2] = {-1, -1};
+    float imm[2] = {0.f, 0.f};
+    const int n_in = n.op == OP_UNARY ? 1 : 2;
+    for (int k = 0; k < n_in; ++k) {
+      const _odla_value* v = n.in[k];
+      const Shape al = aligned_operand(n, k);
+      if (al.rank > R) return give_up();
+      if (in_group.count(v)) {
+        if (!(padded(al) == padded(v->shape))) return give_up();
+        src[k] = reg_of.at(v);
+        continue;
+      }
+      if (n.op == OP_BINARY && v->kind == _odla_value::CONSTANT && v->shape.numel() == 1 && v->host_data != nullptr) {
+        imm[k] = const_as_float(v)[0];
+        continue;   // src stays -1: immediate operand
+      }
+      auto it = reg_of.find(v);
+      if (it != reg_of.end()) {
+        // the same outside value twice: both uses must see it with the same alignment
+        bool same = false;
+        for (const PendingLoad& l : loads) if (l.v == v) same = padded(l.aligned) == padded(al);
+        if (!same) return give_up();
+        src[k] = it->second;
+        continue;
+      }
+      const Shape pal = padded(al);
+      for (int i = 0; i < R; ++i) if (pal.d[i] != 1 && pal.d[i] != S.d[i]) return give_up();
+      if (al.numel() != v->shape.numel()) return give_up();
+      const int reg = n_vregs++;
+      reg_of[v] = reg;
+      loads.push_back({v, al, reg});
+      prog.push_back({FOP_LOAD, reg, (int)loads.size() - 1, 0, 0, 0.f, 0.f});   // a = load index for now
+      src[k] = reg;
+    }
+    const int dst = n_vregs++;
+    reg_of[n.out] = dst;
+    if (n.op == OP_UNARY) {
+      prog.push_back({FOP_UNARY, dst, src[0], 0, (int)n.i[0], n.f[0], n.f[1]});
+    } else {
+      if (src[0] < 0 && src[1] < 0) return give_up();
+      prog.push_back({FOP_BINARY, dst, src[0], src[1], (int)n.i[0], src[0] < 0 ? imm[0] : imm[1], 0.f});
+    }
+  }
+  // ---- results that leave the group: plain, through a Concat, through a Transpose
+  struct Sink { int node; const _odla_value* src; int kind; /* 0 plain, 1 concat part, 2 transpose */ int part; };
+  std::vector<Sink> sinks;
+  std::vector<int> sink_nodes;
+  for (int j : members) {
+    const Node& n = comp_->nodes[j];
+    const _odla_value* v = n.out;
+    bool plain = v->is_output;
+    for (int c : consumers_[v->index]) {
+      const Node& cn = comp_->nodes[c];
+      if (in_group.count(cn.out) && in_group[cn.out] == c) continue;
+      const bool full = v->shape.rank == R && v->shape == S;
+      if (cn.op == OP_CONCAT && !cn.absorbed && full && storage_dtype(cn.out) == dt && cn.out->shape.rank == R) {
+        bool all = true;
+        for (const _odla_value* ci : cn.in) all = all && in_group.count(ci) && ci->shape.rank == R;
+        if (all) {
+          const int axis = (int)cn.i[0];
+          for (const _odla_value* ci : cn.in)
+            for (int i = 0; i < R; ++i) if (i != axis && ci->shape.d[i] != S.d[i]) all = false;
+          for (const _odla_value* ci : cn.in) if (!(ci->shape == S)) all = false;
+        }
+        if (all) {
+          if (std::find(sink_nodes.begin(), sink_nodes.end(), c) == sink_nodes.end()) {
+            sink_nodes.push_back(c);
+            for (size_t k = 0; k < cn.in.size(); ++k) sinks.push_back({c, cn.in[k], 1, (int)k});
+          }
+          continue;
+        }
+      }
+      if (cn.op == OP_TRANSPOSE && !cn.absorbed && full && storage_dtype(cn.out) == dt && (int)cn.iv.size() == R) {
+        if (std::find(sink_nodes.begin(), sink_nodes.end(), c) == sink_nodes.end()) {
+          sink_nodes.push_back(c);
+          sinks.push_back({c, v, 2, 0});
+        }
+        continue;
+      }
+      plain = true;
+    }
+    if (plain) {
+      if (!(padded(v->shape) == S)) return give_up();
+      sinks.push_back({j, v, 0, 0});
+    }
+  }
+  if (sinks.empty()) return give_up();
+  if ((int)(loads.size() + sinks.size()) > kFusedMaxViews || (int)(prog.size() + sinks.size()) > kFusedMaxInstr) return give_up();
+
+  // ---- physical registers: a register is free again after its last reader
+  std::vector<int> last_use((size_t)n_vregs, -1);
+  for (size_t k = 0; k < prog.size(); ++k) {
+    if (prog[k].op != FOP_LOAD && prog[k].a >= 0) last_use[prog[k].a] = (int)k;
+    if (prog[k].op == FOP_BINARY && prog[k].b >= 0) last_use[prog[k].b] = (int)k;
+  }
+  for (const Sink& sk : sinks) last_use[reg_of.at(sk.src)] = (int)prog.size();   // stores come last
+  std::vector<int> phys((size_t)n_vregs, -1);
+  {
+    std::vector<int> free_regs;
+    for (int i = kFusedMaxRegs - 1; i >= 0; --i) free_regs.push_back(i);
+    for (size_t k = 0; k < prog.size(); ++k) {
+      VI& in = prog[k];
+      const int va = in.op != FOP_LOAD ? in.a : -1, vb = in.op == FOP_BINARY ? in.b : -1;
+      // operands read before the result is written: a register freed here may take the result
+      if (va >= 0 && last_use[va] == (int)k) free_regs.push_back(phys[va]);
+      if (vb >= 0 && vb != va && last_use[vb] == (int)k) free_regs.push_back(phys[vb]);
+      if (free_regs.empty()) return give_up();
+      phys[in.dst] = free_regs.back();
+      free_regs.pop_back();
+      if (last_use[in.dst] < 0) free_regs.push_back(phys[in.dst]);   // never read: reusable at once
+    }
+  }
+
+  // ---- from here on the plan changes: nothing below gives up
+  // outside operands (conversion steps, if any, are emitted here, before the group)
+  FusedParams fp;
+  fp.dt = dt;
+  std::vector<int> read_tensors, write_tensors;
+  std::vector<int64_t> in_main_stride;   // per load: used to pick the iteration order
+  for (const PendingLoad& l : loads) {
+    View vw;
+    auto sl = slice_of.find(l.v);
+    const Shape pal = padded(l.aligned);
+    if (sl != slice_of.end() && std::find(slices.begin(), slices.end(), sl->second) != slices.end()) {
+      const Node& sn = comp_->nodes[sl->second];
+      const _odla_value* x = sn.in[0];
+      const int r = x->shape.rank;
+      vw.tensor = get(x, L_ROWMAJOR, FORM_FLOAT);
+      // strides of the slice's own dims, then mapped through the aligned shape (which only adds 1-dims)
+      std::vector<int64_t> own_st((size_t)r);
+      int64_t acc = 1;
+      for (int i = r - 1; i >= 0; --i) {
+        own_st[i] = acc * sn.iv[2 * r + i];
+        vw.off += sn.iv[i] * acc;
+        acc *= x->shape.d[i];
+      }
+      // walk the non-1 dims of the slice result and of the aligned shape together
+      int oi = 0;
+      for (int i = 0; i < R; ++i) {
+        if (pal.d[i] == 1) continue;
+        while (oi < r && sn.out->shape.d[oi] == 1) ++oi;
+        vw.st[i] = own_st[oi++];
+      }
+    } else {
+      vw.tensor = get(l.v, L_ROWMAJOR, FORM_FLOAT);
+      int64_t acc = 1;
+      for (int i = R - 1; i >= 0; --i) { vw.st[i] = pal.d[i] == 1 ? 0 : acc; acc *= pal.d[i]; }
+    }
+    if (T(vw.tensor).dt != dt) fail(ODLA_UNSUPPORTED_DATATYPE, "mixed storage types in the element-wise group at '%s'", comp_->nodes[seed].out->name.c_str());
+    vw.value = l.v;
+    views.push_back(vw);
+    read_tensors.push_back(vw.tensor);
+  }
+  const size_t n_loads = views.size();
+  std::unordered_map<int, int> sink_tensor;   // sink node -> its result tensor
+  std::vector<std::pair<_odla_value*, int>> results;
+  auto row_major = [&](const Shape& sh, int64_t* st) { int64_t acc = 1; for (int i = sh.rank - 1; i >= 0; --i) { st[i] = acc; acc *= sh.d[i]; } };
+  for (const Sink& sk : sinks) {
+    const Node& sn = comp_->nodes[sk.node];
+    View vw;
+    vw.store = true;
+    vw.value = sk.src;
+    int64_t st[ODLA_MAX_DIMENSION] = {0};
+    if (sk.kind == 0) {
+      vw.tensor = new_tensor(dt, L_ROWMAJOR, sk.src->shape, 0, SP_ARENA);
+      results.push_back({sn.out, vw.tensor});
+      row_major(S, st);
+      for (int i = 0; i < R; ++i) vw.st[i] = st[i];
+    } else {
+      auto it = sink_tensor.find(sk.node);
+      if (it == sink_tensor.end()) {
+        const int t = new_tensor(dt, L_ROWMAJOR, sn.out->shape, 0, SP_ARENA);
+        it = sink_tensor.emplace(sk.node, t).first;
+        results.push_back({sn.out, t});
+      }
+      vw.tensor = it->second;
+      row_major(sn.out->shape, st);
+      if (sk.kind == 1) {
+        const int axis = (int)sn.i[0];
+        int64_t before = 0;
+        for (int k = 0; k < sk.part; ++k) before += sn.in[k]->shape.d[axis];
+        vw.off = before * st[axis];
+        for (int i = 0; i < R; ++i) vw.st[i] = st[i];
+      } else {
+        for (int i = 0; i < R; ++i) vw.st[(int)sn.iv[i]] = st[i];   // result dim i walks source dim perm[i]
+      }
+    }
+    views.push_back(vw);
+    if (std::find(write_tensors.begin(), write_tensors.end(), vw.tensor) == write_tensors.end()) write_tensors.push_back(vw.tensor);
+  }
+
+  // ---- iteration order: stores contiguous across threads, loads along a thread's walk
+  int d3 = R - 1, d2 = -1;
+  {
+    const View& mo = views[n_loads];
+    int64_t best = 0;
+    for (int i = 0; i < R; ++i)
+      if (S.d[i] > 1 && mo.st[i] > 0 && (best == 0 || mo.st[i] < best)) { best = mo.st[i]; d3 = i; }
+    int64_t most = -1;
+    const View* mi = nullptr;
+    for (size_t k = 0; k < n_loads; ++k) {
+      int64_t elems = 1;
+      for (int i = 0; i < R; ++i) if (views[k].st[i] != 0) elems *= S.d[i];
+      if (elems > most) { most = elems; mi = &views[k]; }
+    }
+    if (mi != nullptr && mi->st[d3] != 1)
+      for (int i = 0; i < R; ++i) if (i != d3 && S.d[i] > 1 && mi->st[i] == 1) d2 = i;
+  }
+  int order[4] = {-1, -1, d2, d3};
+  {
+    int slot = 1;
+    for (int i = R - 1; i >= 0; --i) if (i != d2 && i != d3) order[slot--] = i;
+  }
+  for (int k = 0; k < 4; ++k) fp.dims[k] = order[k] < 0 ? 1 : S.d[order[k]];
+  {
+    // every step of a walk waits for its loads: keep walks short until the chip has
+    // a few resident threads per lane (256 CUs x 2048 threads x 2)
+    const int64_t base = fp.dims[0] * fp.dims[1] * fp.dims[3];
+    const int64_t want = 256 * 2048 * 2;
+    int64_t w = fp.dims[2] * base / want;
+    fp.walk = std::min<int64_t>(fp.dims[2], std::max<int64_t>(4, w));
+  }
+  for (size_t k = 0; k < views.size(); ++k) {
+    fp.view[k].off = views[k].off;
+    for (int q = 0; q < 4; ++q) fp.view[k].st[q] = order[q] < 0 ? 0 : views[k].st[order[q]];
+  }
+  int ni = 0;
+  for (const VI& in : prog) {
+    FusedInstr& o = fp.prog[ni++];
+    o.op = in.op; o.kind = in.kind; o.fa = in.fa; o.fb = in.fb;
+    o.dst = phys[in.dst];
+    o.a = in.op == FOP_LOAD ? in.a : (in.a < 0 ? -1 : phys[in.a]);
+    o.b = in.op == FOP_BINARY ? (in.b < 0 ? -1 : phys[in.b]) : 0;
+  }
+  for (size_t k = 0; k < sinks.size(); ++k) {
+    FusedInstr& o = fp.prog[ni++];
+    o.op = FOP_STORE;
+    o.dst = (int)(n_loads + k);
+    o.a = phys[reg_of.at(sinks[k].src)];
+  }
+  fp.n_instr = ni;
+
+  std::vector<Ref> refs;
+  for (const View& vw : views) refs.push_back(ref(vw.tensor));
+  std::vector<int64_t> elem_off;
+  const std::string name = "fused:" + comp_->nodes[members.back()].out->name + "(" + std::to_string(members.size()) + ")";
+  emit_lists(name, read_tensors, write_tensors, [=](const ExecEnv& e, hipStream_t st) {
+    FusedParams p = fp;
+    for (size_t k = 0; k < refs.size(); ++k) p.view[k].base = refs[k](e);
+    return launch_fused_eltwise(p, st);
+  });
+  for (int j : members) comp_->nodes[j].absorbed = true;
+  for (int j : slices) comp_->nodes[j].absorbed = true;
+  for (int j : sink_nodes) comp_->nodes[j].absorbed = true;
+  for (auto& rv : results) set_main(rv.first, rv.second);
+  return true;
 }
 
 // ----------------------------------------------------------- BatchNorm ----
