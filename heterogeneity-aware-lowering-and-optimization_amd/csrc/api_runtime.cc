@@ -682,6 +682,25 @@ odla_status odla_hip_ExecuteComputationStatic(odla_computation comp, odla_contex
 // Diagnostic: run the launch sequence un-captured `iters` times with a HIP
 // event pair around every step on the context's stream and report the mean
 // duration of each step.  Arguments must be bound.
+odla_status odla_hip_PlanSummary(odla_computation c, odla_hip_plan_summary* summary) {
+  if (c == nullptr || summary == nullptr || !is_live(c)) return ODLA_INVALID_PARAM;
+  std::lock_guard<std::mutex> lk(c->mu);
+  if (c->plan && c->live_contexts > 0) {
+    OHIP_ERR("odla_hip_PlanSummary: the computation is compiled and has live contexts");
+    return ODLA_FAILURE;   // the fusion marks of the nodes belong to the live plan
+  }
+  int launches = 0, init_launches = 0;
+  size_t arena = 0, consts = 0;
+  profiler_configure(&c->opts);
+  const odla_status st = plan_summary(c, &launches, &init_launches, &arena, &consts);
+  if (st != ODLA_SUCCESS) return st;
+  summary->launches = launches;
+  summary->init_launches = init_launches;
+  summary->arena_bytes = arena;
+  summary->constant_bytes = consts;
+  return ODLA_SUCCESS;
+}
+
 odla_status odla_hip_ProfileSteps(odla_context ctx, odla_int32 iters, odla_hip_step_time* out,
                                   odla_int32 capacity, odla_int32* count) {
   if (ctx == nullptr || out == nullptr || count == nullptr || iters <= 0) return ODLA_INVALID_PARAM;

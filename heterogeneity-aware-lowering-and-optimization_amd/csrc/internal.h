@@ -190,6 +190,9 @@ struct Plan {
 };
 
 odla_status build_plan(_odla_computation* comp, std::unique_ptr<Plan>* out);
+// Host-only lowering: the plan is built, measured and dropped (no device call).
+odla_status plan_summary(_odla_computation* comp, int* launches, int* init_launches, size_t* arena_bytes,
+                         size_t* const_bytes);
 
 // Calibration profiler (the control functions StartProfiling .. are exported
 // with the reference profiler's names).

@@ -3153,6 +3153,30 @@ void Planner::lower_postprocess(int ni) {
 }  // namespace
 
 // ============================================================================
+odla_status plan_summary(_odla_computation* comp, int* launches, int* init_launches, size_t* arena_bytes,
+                         size_t* const_bytes) {
+  auto plan = std::make_unique<Plan>();
+  for (Node& n : comp->nodes) n.absorbed = false;
+  odla_status st = ODLA_SUCCESS;
+  try {
+    Planner p(comp, plan.get());
+    p.run();
+  } catch (const PlanError& e) {
+    OHIP_ERR("cannot compile computation: %s", e.msg.c_str());
+    st = e.status;
+  } catch (const std::exception& e) {
+    OHIP_ERR("cannot compile computation: %s", e.what());
+    st = ODLA_FAILURE;
+  }
+  for (Node& n : comp->nodes) n.absorbed = false;
+  if (st != ODLA_SUCCESS) return st;
+  *launches = (int)plan->steps.size();
+  *init_launches = (int)plan->init_steps.size();
+  *arena_bytes = plan->arena_bytes;
+  *const_bytes = plan->const_bytes;
+  return ODLA_SUCCESS;
+}
+
 odla_status build_plan(_odla_computation* comp, std::unique_ptr<Plan>* out) {
   auto plan = std::make_unique<Plan>();
   // fusion marks are per-plan

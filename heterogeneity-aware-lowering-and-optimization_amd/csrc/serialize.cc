@@ -353,6 +353,10 @@ odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) 
   for (int64_t k = 0; k < nv; ++k) {
     const int64_t kind = r.i64(), et = r.i64(), rank = r.i64();
     if (!r.ok || rank < 0 || rank > ODLA_MAX_DIMENSION || kind < 0 || kind > 2) return ODLA_INVALID_PARAM;
+    if (et < 0 || et > (int64_t)ODLA_STRING) {   // checked before the number becomes an enumerator
+      OHIP_ERR("stored computation rejected: value %lld has element type %lld", (long long)k, (long long)et);
+      return ODLA_INVALID_PARAM;
+    }
     Shape s;
     s.rank = (int)rank;
     for (int i = 0; i < s.rank; ++i) s.d[i] = r.i64();

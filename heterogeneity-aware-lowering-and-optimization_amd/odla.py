@@ -17,7 +17,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libodla_hip.so")
+# ODLA_HIP_LIBRARY names another build of the library (the sanitizer build of the host code)
+LIB_PATH = os.environ.get("ODLA_HIP_LIBRARY") or os.path.join(_HERE, "libodla_hip.so")
 
 # ---- enums (include/odla_hip.h) ---------------------------------------------
 (ODLA_INT8, ODLA_INT16, ODLA_INT32, ODLA_INT64, ODLA_UINT8, ODLA_UINT16, ODLA_UINT32, ODLA_UINT64,
@@ -86,6 +87,12 @@ def memory_location(data):
     return ResourceLocation(ODLA_LOCATION_MEMORY, ctypes.cast(buf, ctypes.c_void_p), len(data)), buf
 
 
+class PlanSummary(ctypes.Structure):
+    """odla_hip_plan_summary."""
+    _fields_ = [("launches", ctypes.c_int32), ("init_launches", ctypes.c_int32),
+                ("arena_bytes", ctypes.c_uint64), ("constant_bytes", ctypes.c_uint64)]
+
+
 class QuantInfo(ctypes.Structure):
     _fields_ = [("value_id", ctypes.c_char_p), ("ch_idx", ctypes.c_int), ("scale", ctypes.c_float),
                 ("offset", ctypes.c_float), ("min", ctypes.c_float), ("max", ctypes.c_float)]
@@ -151,6 +158,7 @@ def load_library(path=None):
     proto("odla_BindToOutputById", i32, [cid, vp, vp])
     proto("odla_ExecuteComputation", i32, [vp, vp, i32, vp])
     proto("odla_hip_ExecuteComputationStatic", i32, [vp, vp, i32, vp])
+    proto("odla_hip_PlanSummary", i32, [vp, ctypes.POINTER(PlanSummary)])
     proto("odla_GetNumOfArgsFromComputation", i32, [vp, pu32])
     proto("odla_GetArgFromComputationByIdx", i32, [vp, u32, ctypes.POINTER(vp)])
     proto("odla_GetNumOfOutputsFromComputation", i32, [vp, pu32])
@@ -631,6 +639,14 @@ class HipBuilder:
     # -- execution --
     def session(self, use_graph=True):
         return Session(self, use_graph)
+
+    def plan_summary(self):
+        """odla_hip_PlanSummary: lowers the recorded graph on the host (no device
+        needed) and returns its launch count and device-memory needs."""
+        ps = PlanSummary()
+        _check(self.L.odla_hip_PlanSummary(self.comp, ctypes.byref(ps)), "odla_hip_PlanSummary")
+        return {"launches": ps.launches, "init_launches": ps.init_launches, "arena_bytes": ps.arena_bytes,
+                "constant_bytes": ps.constant_bytes}
 
     def destroy(self):
         if self.comp:

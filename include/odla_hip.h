@@ -854,6 +854,22 @@ odla_status odla_hip_ProfileSteps(odla_context context, odla_int32 iters,
                                   odla_hip_step_time* out, odla_int32 capacity,
                                   odla_int32* count);
 
+typedef struct {
+  odla_int32 launches;        /* kernel launches of one execution              */
+  odla_int32 init_launches;   /* one-time launches that prepare the constants  */
+  odla_uint64 arena_bytes;    /* temporaries of one context                    */
+  odla_uint64 constant_bytes; /* packed constants, shared by all contexts      */
+} odla_hip_plan_summary;
+
+/* Lowers what has been recorded in `computation` to its launch sequence on the
+ * host, reports its size and discards it.  No device is touched: a build
+ * machine without a GPU can check that a model compiles (unsupported operators
+ * and shapes are reported exactly as odla_CreateContext would report them) and
+ * how much device memory it will need.  The computation itself is unchanged
+ * and can be compiled, extended or stored afterwards.  No counterpart in the
+ * reference. */
+odla_status odla_hip_PlanSummary(odla_computation computation, odla_hip_plan_summary* summary);
+
 /* ------------------------------------------------------------------------ */
 /* Execution without device-memory allocation.                               */
 /* No counterpart in the reference.  For callers that cannot allocate device */
