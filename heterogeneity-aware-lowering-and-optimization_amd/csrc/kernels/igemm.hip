@@ -90,12 +90,12 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
     unsigned char* otile = smem + (i & 1) * (2 * TILE);
     unsigned char* rtile = otile + TILE;
     if (has_res) {
-      *reinterpret_cast<uintx4*>(rtile + rp * PITCH + c16) = rall[i];
+      *reinterpret_cast<uintx4*>(rtile + rp * PITCH + c16) = q8_swz_chunk(rall[i], rp);
       lds_barrier();
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int off = l32 * PITCH + wave * 32 + q * 8 + lg * 4;
+      const int off = (l32 * PITCH + wave * 32 + q * 8 + lg * 4) ^ q8_swz(l32);
       const unsigned rs = has_res ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
       const unsigned w = requant4(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3],
                                   mq[q], has_res, rs, p);
@@ -106,7 +106,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
     // the barrier(s) of slice i+1, which every wavefront reaches after its reads here.
     lds_barrier();
     const int m = tile_m * BM + i * 32 + rp;
-    const uintx4 v = *reinterpret_cast<const uintx4*>(otile + rp * PITCH + c16);
+    const uintx4 v = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + rp * PITCH + c16), rp);
     if (m < M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
   };
   slice(std::integral_constant<int, 0>{});

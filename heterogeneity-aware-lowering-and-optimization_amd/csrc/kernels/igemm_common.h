@@ -313,6 +313,18 @@ __device__ __forceinline__ void store_row16(int8_t* row, const uintx4 v, const b
   for (int e = 0; e < nvalid; ++e) row[e] = (int8_t)(w[e >> 2] >> (8 * (e & 3)));
 }
 
+// Bank swizzle of the staged byte tiles.  Row pitches are a multiple of 16 bytes
+// (the 16-byte row accesses need that), i.e. 4 banks modulo 8, so the dword that
+// 32 lanes hold for 32 pixel rows would land in 8 banks, four rows each.  Dword d
+// of row r therefore lives at d ^ ((r >> 3) & 3): the four rows that share a bank
+// group take its four banks.  A 16-byte chunk stays a chunk; its dwords are
+// exchanged on the way in and out (the exchange is its own inverse).
+__device__ __forceinline__ int q8_swz(const int row) { return ((row >> 3) & 3) << 2; }
+__device__ __forceinline__ uintx4 q8_swz_chunk(const uintx4 v, const int row) {
+  const uintx4 t = (row & 8) ? uintx4{v.y, v.x, v.w, v.z} : v;
+  return (row & 16) ? uintx4{t.z, t.w, t.x, t.y} : t;
+}
+
 // ---------------------------------------------------------------------------
 // Epilogue of the 8-bit layers, per wavefront.  The requantisation runs in the
 // accumulator layout (a lane's four consecutive channels become one dword), so
@@ -321,8 +333,8 @@ __device__ __forceinline__ void store_row16(int8_t* row, const uintx4 v, const b
 // per element is cvt, fma, max, cvt_pk.  A residual tile takes the same road in
 // the other direction: 16-byte row loads, through LDS, read back as the dword of
 // the lane's four channels.
-// LDS per wavefront: two [32 pixels][WN + 16] byte tiles (result, residual) and
-// the WN multipliers of its channels.
+// LDS per wavefront: two [32 pixels][WN + 16] byte tiles (result, residual; dwords
+// swizzled by q8_swz) and the WN multipliers of its channels.
 template <int BM, int BN, int WM, int WN, bool kEnterBarrier = true>
 __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[WM / 32][WN / 32],
                                                   unsigned char* smem, const int tile_m, const int tile_n, const int z,
@@ -385,7 +397,7 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
     if (has_res) {
 #pragma unroll
       for (int ps = 0; ps < NPASS; ++ps)
-        *reinterpret_cast<uintx4*>(rtile + (ps * PPP + rp) * PITCH + c16) = rcur[ps];
+        *reinterpret_cast<uintx4*>(rtile + (ps * PPP + rp) * PITCH + c16) = q8_swz_chunk(rcur[ps], ps * PPP + rp);
     }
     wave_fence();
     if (has_res && i + 1 < TM) rfetch(i + 1);
@@ -395,7 +407,7 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int ch = j * 32 + q * 8 + lg * 4;
-        const int off = l32 * PITCH + ch;
+        const int off = (l32 * PITCH + ch) ^ q8_swz(l32);
         const floatx4 m = *reinterpret_cast<const floatx4*>(mtile + ch);
         const unsigned rs = has_res ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
         const unsigned w = requant4(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3],
@@ -407,7 +419,7 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
     for (int ps = 0; ps < NPASS; ++ps) {
       const int pix = ps * PPP + rp;
       const int m = tile_m * BM + wm * WM + i * 32 + pix;
-      const uintx4 v = *reinterpret_cast<const uintx4*>(otile + pix * PITCH + c16);
+      const uintx4 v = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + pix * PITCH + c16), pix);
       if (m < M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
     }
   }
