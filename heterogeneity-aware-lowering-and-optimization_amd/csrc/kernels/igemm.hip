@@ -1090,6 +1090,10 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
     div_magic(p.Ho * p.Wo, &p.howo_magic, &p.howo_shift);
     div_magic(p.Wo, &p.wo_magic, &p.wo_shift);
   }
+  if (p.y_rdiv > 0 && p.y_cdiv > 0) {
+    div_magic(p.y_rdiv, &p.yr_magic, &p.yr_shift);
+    div_magic(p.y_cdiv, &p.yc_magic, &p.yc_shift);
+  }
   const int es = dtype_size(p.in_dt);
   if (es == 0 || p.x == nullptr || p.w == nullptr || p.y == nullptr) return hipErrorInvalidValue;
   const int vec = 16 / es;

@@ -12,11 +12,17 @@ namespace ohip {
 
 // Element offset of result row m / column n / problem z (see IgemmParams::y_rdiv, y_zdiv).
 __device__ __forceinline__ int64_t y_row_off(const IgemmParams& p, const int m) {
-  if (p.y_rdiv > 0) return (int64_t)((unsigned)m / (unsigned)p.y_rdiv) * p.y_rhi + (int64_t)((unsigned)m % (unsigned)p.y_rdiv) * p.y_rlo;
+  if (p.y_rdiv > 0) {
+    const int a = fast_div(m, p.yr_magic, p.yr_shift);
+    return (int64_t)a * p.y_rhi + (int64_t)(m - a * p.y_rdiv) * p.y_rlo;
+  }
   return (int64_t)m * p.ycs;
 }
 __device__ __forceinline__ int64_t y_col_off(const IgemmParams& p, const int n) {
-  if (p.y_rdiv > 0) return (int64_t)((unsigned)n / (unsigned)p.y_cdiv) * p.y_chi + (int64_t)((unsigned)n % (unsigned)p.y_cdiv);
+  if (p.y_rdiv > 0) {
+    const int c = fast_div(n, p.yc_magic, p.yc_shift);
+    return (int64_t)c * p.y_chi + (int64_t)(n - c * p.y_cdiv);
+  }
   return n;
 }
 __device__ __forceinline__ int64_t y_batch_off(const IgemmParams& p, const int z) {

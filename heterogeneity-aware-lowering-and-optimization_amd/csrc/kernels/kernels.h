@@ -116,9 +116,9 @@ struct IgemmParams {
   // covering R*S*C), wf_tiles = 32-row tiles per batch entry.
   const void* w_frag = nullptr;
   int wf_chunks = 0, wf_tiles = 0;
-  // filled in by launch_igemm: magic pairs for the divisions by Ho*Wo and Wo
-  unsigned howo_magic = 0, wo_magic = 0;
-  int howo_shift = 0, wo_shift = 0;
+  // filled in by launch_igemm: magic pairs for the divisions by Ho*Wo, Wo, y_rdiv and y_cdiv
+  unsigned howo_magic = 0, wo_magic = 0, yr_magic = 0, yc_magic = 0;
+  int howo_shift = 0, wo_shift = 0, yr_shift = 0, yc_shift = 0;
   float alpha = 1.0f;              // scales the accumulator before bias (float types)
   ActKind act = ACT_NONE;
   float act_a = 0.0f, act_b = 0.0f;  // leaky slope / clamp lo,hi
