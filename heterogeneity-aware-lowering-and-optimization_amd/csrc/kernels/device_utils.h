@@ -139,16 +139,41 @@ __device__ __forceinline__ int fast_div(int n, unsigned magic, int shift) {
   return (int)(__umulhi((unsigned)n << 1, magic) >> shift);
 }
 
-// Wavefront (64 lanes) reductions through cross-lane shuffles.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// Cross-lane reductions.  Inside a row of 16 lanes the partner values arrive
+// through DPP operands of the arithmetic instruction itself (quad permutes,
+// then the half-row and row mirrors: once a quad / half row is uniform, its
+// mirror image is the other quad / half row), which costs no LDS crossbar trip
+// like ds_bpermute does; the four row totals are then read as scalars.
+// Every lane of a group of LPR lanes (a power of two, groups aligned) receives
+// op over the group.  Call from wavefront-uniform control flow only: DPP and
+// v_readlane read lanes whatever their EXEC bit.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(const float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int LPR, typename Op>
+__device__ __forceinline__ float group_allreduce(float v, Op op) {
+  static_assert(LPR >= 1 && LPR <= 64 && (LPR & (LPR - 1)) == 0, "groups are powers of two up to the wavefront");
+  if constexpr (LPR >= 2) v = op(v, dpp_move<0xB1>(v));    // quad_perm:[1,0,3,2]
+  if constexpr (LPR >= 4) v = op(v, dpp_move<0x4E>(v));    // quad_perm:[2,3,0,1]
+  if constexpr (LPR >= 8) v = op(v, dpp_move<0x141>(v));   // row_half_mirror
+  if constexpr (LPR >= 16) v = op(v, dpp_move<0x140>(v));  // row_mirror
+  if constexpr (LPR >= 32) {
+    const int bits = __builtin_bit_cast(int, v);
+    const float t0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+    const float t1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+    const float t2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+    const float t3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+    if constexpr (LPR == 64) v = op(op(t0, t1), op(t2, t3));
+    else v = (threadIdx.x & 32) ? op(t2, t3) : op(t0, t1);
+  }
   return v;
 }
+__device__ __forceinline__ float wave_sum(float v) {
+  return group_allreduce<64>(v, [](float a, float b) { return a + b; });
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  return group_allreduce<64>(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
 // Block-wide reductions for blocks of NT threads (NT multiple of 64, <= 1024).

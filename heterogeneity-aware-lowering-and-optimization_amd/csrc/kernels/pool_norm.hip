@@ -243,8 +243,7 @@ reduce_rows_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
     const TI* row = x + r * len;
     float acc = red_init<A>();
     for (int64_t i = lane; i < len; i += 64) acc = red_step<A>(acc, Store<TI>::ld(row + i));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) acc = red_merge<A>(acc, __shfl_xor(acc, o, 64));
+    acc = group_allreduce<64>(acc, [](float a, float b) { return red_merge<A>(a, b); });
     if (lane == 0) Store<TO>::st(y + r, red_final(acc, len, kind, eps));
   }
 }
@@ -373,8 +372,7 @@ reduce_row_block_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t le
 #pragma unroll
     for (int e = 0; e < V; ++e) acc = red_step<A>(acc, v.get(e));
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) acc = red_merge<A>(acc, __shfl_xor(acc, o, 64));
+  acc = group_allreduce<64>(acc, [](float a, float b) { return red_merge<A>(a, b); });
   if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -528,18 +526,14 @@ softmax_wave_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, 
 }
 // Rows of 16-byte vectors (len % V == 0, row start 16-byte aligned): LPR lanes
 // share one row, each lane holds PER vectors; several short rows fit in one
-// wavefront.  Reductions are xor-shuffles inside the LPR-lane group.
+// wavefront.  Reductions stay inside the LPR-lane group (group_allreduce).
 template <int LPR>
 __device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-  for (int o = LPR / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  return group_allreduce<LPR>(v, [](float a, float b) { return fmaxf(a, b); });
 }
 template <int LPR>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int o = LPR / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  return group_allreduce<LPR>(v, [](float a, float b) { return a + b; });
 }
 
 template <typename TO, int V>
