@@ -837,7 +837,10 @@ odla_value odla_Resize(odla_value input, odla_interpolation_mode interpolation,
   _odla_computation* c = comp_of(input);
   REQUIRE(c, "odla_Resize: no current computation");
   REQUIRE(input->shape.rank == 4 && output_dims.size == 4, "odla_Resize: rank-4 tensors only");
-  REQUIRE(interpolation == ODLA_NEAREST, "odla_Resize: only nearest interpolation is supported");
+  REQUIRE(interpolation == ODLA_NEAREST || interpolation == ODLA_LINEAR, "odla_Resize: nearest and linear interpolation are supported");
+  REQUIRE(interpolation == ODLA_NEAREST || input->etype == ODLA_FLOAT32 || input->etype == ODLA_FLOAT16 ||
+              input->etype == ODLA_BFLOAT16,
+          "odla_Resize: linear interpolation needs a float input");
   Shape o = shape_from(output_dims);
   REQUIRE(o.d[0] == input->shape.d[0] && o.d[1] == input->shape.d[1] && o.d[2] > 0 && o.d[3] > 0,
           "odla_Resize: output %s must keep batch and channels of %s", o.str().c_str(), input->shape.str().c_str());

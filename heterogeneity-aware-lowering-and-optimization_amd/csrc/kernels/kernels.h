@@ -378,6 +378,9 @@ hipError_t launch_transpose2d(const void* x, void* y, int elem_size, int batch, 
 // Nearest-neighbour resize, channels-last: src index = floor(dst * in / out).
 hipError_t launch_resize_nearest_nhwc(const void* x, void* y, int elem_size, int N, int H,
                                       int W, int cs, int Ho, int Wo, hipStream_t stream);
+// Bilinear resize, channels-last, float types: half-pixel centres, edges clamped.
+hipError_t launch_resize_linear_nhwc(const void* x, void* y, DType dt, int N, int H, int W, int cs,
+                                     int Ho, int Wo, hipStream_t stream);
 // Row gather: y[o][j][:] = x[o][idx[j]][:], rows of row_bytes bytes.
 hipError_t launch_gather_rows(const void* x, const void* idx, DType idx_dt, void* y,
                               int64_t outer, int64_t n_src_rows, int64_t n_idx,

@@ -212,6 +212,52 @@ resize_nearest_kernel(const E* __restrict__ x, E* __restrict__ y, int N, int H, 
   }
 }
 
+// Bilinear resize, channels-last, pixel centres at half-integers and edge
+// clamping: source coordinate s = (o + 0.5) * in / out - 0.5, neighbours
+// floor(s) and floor(s) + 1 clamped into the image, weights 1 - frac and frac
+// (oneDNN's resampling_linear, which is what the reference calls for
+// ODLA_LINEAR whatever coordinate mode is passed).  One thread per group of V
+// channels of one output pixel.
+template <typename T, int V>
+__global__ void __launch_bounds__(kThreads)
+resize_linear_kernel(const T* __restrict__ x, T* __restrict__ y, int N, int H, int W, int cs,
+                     int Ho, int Wo, float fh, float fw) {
+  const int cv = cs / V;
+  const int64_t total = (int64_t)N * Ho * Wo * cv;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int c = (int)(i % cv) * V;
+    int64_t t = i / cv;
+    const int wo = (int)(t % Wo); t /= Wo;
+    const int ho = (int)(t % Ho);
+    const int n = (int)(t / Ho);
+    float sh = ((float)ho + 0.5f) * fh - 0.5f, sw = ((float)wo + 0.5f) * fw - 0.5f;
+    sh = sh < 0.f ? 0.f : sh;
+    sw = sw < 0.f ? 0.f : sw;
+    int h0 = (int)sh, w0 = (int)sw;
+    h0 = h0 > H - 1 ? H - 1 : h0;
+    w0 = w0 > W - 1 ? W - 1 : w0;
+    const int h1 = h0 < H - 1 ? h0 + 1 : h0, w1 = w0 < W - 1 ? w0 + 1 : w0;
+    const float ah = sh - (float)h0, aw = sw - (float)w0;
+    const float k00 = (1.f - ah) * (1.f - aw), k01 = (1.f - ah) * aw, k10 = ah * (1.f - aw), k11 = ah * aw;
+    const T* base = x + (int64_t)n * H * W * cs + c;
+    const T* p00 = base + ((int64_t)h0 * W + w0) * cs;
+    const T* p01 = base + ((int64_t)h0 * W + w1) * cs;
+    const T* p10 = base + ((int64_t)h1 * W + w0) * cs;
+    const T* p11 = base + ((int64_t)h1 * W + w1) * cs;
+    T* out = y + (((int64_t)n * Ho + ho) * Wo + wo) * cs + c;
+    if constexpr (V > 1) {
+      Vec16<T> a, b, d, e, o;
+      a.load(p00); b.load(p01); d.load(p10); e.load(p11);
+#pragma unroll
+      for (int k = 0; k < V; ++k) o.set(k, k00 * a.get(k) + k01 * b.get(k) + k10 * d.get(k) + k11 * e.get(k));
+      o.store(out);
+    } else {
+      Store<T>::st(out, k00 * Store<T>::ld(p00) + k01 * Store<T>::ld(p01) + k10 * Store<T>::ld(p10) + k11 * Store<T>::ld(p11));
+    }
+  }
+}
+
 template <typename IDX>
 __global__ void __launch_bounds__(kThreads)
 gather_rows_kernel(const unsigned char* __restrict__ x, const IDX* __restrict__ idx,
@@ -408,6 +454,34 @@ hipError_t launch_resize_nearest_nhwc(const void* x, void* y, int elem_size, int
       default: return hipErrorInvalidValue;
     }
   }
+  return hipGetLastError();
+}
+
+hipError_t launch_resize_linear_nhwc(const void* x, void* y, DType dt, int N, int H, int W, int cs,
+                                     int Ho, int Wo, hipStream_t stream) {
+  if (!x || !y || N <= 0 || H <= 0 || W <= 0 || cs <= 0 || Ho <= 0 || Wo <= 0) return hipErrorInvalidValue;
+  const float fh = (float)H / (float)Ho, fw = (float)W / (float)Wo;
+  const int es = dtype_size(dt);
+  if (es == 0) return hipErrorInvalidValue;
+  const int v = 16 / es;
+  const bool vec = cs % v == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
+  const int grid = grid_for((int64_t)N * Ho * Wo * (vec ? cs / v : cs), kThreads);
+#define RESIZE_LINEAR(T_)                                                                                          \
+  do {                                                                                                             \
+    if (vec)                                                                                                       \
+      hipLaunchKernelGGL((resize_linear_kernel<T_, 16 / (int)sizeof(T_)>), dim3(grid), dim3(kThreads), 0, stream,  \
+                         (const T_*)x, (T_*)y, N, H, W, cs, Ho, Wo, fh, fw);                                      \
+    else                                                                                                           \
+      hipLaunchKernelGGL((resize_linear_kernel<T_, 1>), dim3(grid), dim3(kThreads), 0, stream, (const T_*)x,       \
+                         (T_*)y, N, H, W, cs, Ho, Wo, fh, fw);                                                     \
+  } while (0)
+  switch (dt) {
+    case DT_F32: RESIZE_LINEAR(float); break;
+    case DT_F16: RESIZE_LINEAR(f16_t); break;
+    case DT_BF16: RESIZE_LINEAR(bf16_t); break;
+    default: return hipErrorInvalidValue;
+  }
+#undef RESIZE_LINEAR
   return hipGetLastError();
 }
 

@@ -2861,9 +2861,17 @@ void Planner::lower_resize(int ni) {
   const int es = dtype_size(px.dt);
   const int N = (int)xs.d[0], H = (int)xs.d[2], W = (int)xs.d[3], cs = px.cs, Ho = (int)os.d[2], Wo = (int)os.d[3];
   const Ref a = ref(tx), b = ref(ty);
-  emit("resize:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
-    return launch_resize_nearest_nhwc(a(e), b(e), es, N, H, W, cs, Ho, Wo, st);
-  });
+  if (n.i[0] == ODLA_LINEAR) {
+    const DType dt = px.dt;
+    if (!dtype_is_float(dt)) fail(ODLA_UNSUPPORTED_DATATYPE, "linear odla_Resize of a non-float value ('%s')", n.out->name.c_str());
+    emit("resize.linear:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+      return launch_resize_linear_nhwc(a(e), b(e), dt, N, H, W, cs, Ho, Wo, st);
+    });
+  } else {
+    emit("resize:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+      return launch_resize_nearest_nhwc(a(e), b(e), es, N, H, W, cs, Ho, Wo, st);
+    });
+  }
   set_main(n.out, ty);
 }
 

@@ -261,6 +261,8 @@ odla_status validate_loaded(const _odla_computation* c) {
         LOADED_REQUIRE(x->shape.numel() == n.out->shape.numel(), "Reshape node %lld changes the element count", (long long)k);
         break;
       case OP_RESIZE:
+        LOADED_REQUIRE(n.i[0] == ODLA_NEAREST || n.i[0] == ODLA_LINEAR, "Resize node %lld: interpolation %lld", (long long)k, (long long)n.i[0]);
+        [[fallthrough]];
       case OP_LRN:
         LOADED_REQUIRE(xr == 4 && orank == 4, "%s node %lld: operands must have rank 4", name, (long long)k);
         break;

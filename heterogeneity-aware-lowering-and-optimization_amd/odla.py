@@ -37,7 +37,7 @@ ODLA_HIP_ITEM_RAW_INT32_ACC = 1000
 BF16_DISABLE, BF16_ACCURACY_MODE, BF16_PERFORMACE_MODE, BF16_AUTO_MODE = range(4)
 ODLA_CHANNELS_FIRST, ODLA_CHANNELS_LAST, ODLA_SIO, ODLA_SOI, ODLA_OIS, ODLA_IOS = range(6)
 ODLA_NEAREST, ODLA_LINEAR, ODLA_CUBIC = range(3)
-ODLA_ASSYMMETRIC = 0
+ODLA_ASSYMMETRIC, ODLA_HALF_PIXEL, ODLA_HALF_PIXEL_TF, ODLA_ALIGN_CORNERS = range(4)
 ODLA_MEMCPY_H2H, ODLA_MEMCPY_H2D, ODLA_MEMCPY_D2H, ODLA_MEMCPY_D2D = range(4)
 ODLA_DEVICE_INFO_TOTAL_MEMORY, ODLA_DEVICE_INFO_USED_MEMORY = 7, 8
 
@@ -481,6 +481,11 @@ class HipBuilder:
     def resize_nearest(self, x, out_hw, name=None):
         s, _ = self.shape_of(x)
         return self._ret(self.L.odla_Resize(x, ODLA_NEAREST, ODLA_ASSYMMETRIC, 0,
+                                            make_shape([s[0], s[1], out_hw[0], out_hw[1]]), _cid(name)), "odla_Resize")
+
+    def resize_linear(self, x, out_hw, name=None):
+        s, _ = self.shape_of(x)
+        return self._ret(self.L.odla_Resize(x, ODLA_LINEAR, ODLA_HALF_PIXEL, 0,
                                             make_shape([s[0], s[1], out_hw[0], out_hw[1]]), _cid(name)), "odla_Resize")
 
     def quantize(self, x, scale, zp=None, axis=-1, signed=False, name=None):

@@ -518,9 +518,13 @@ odla_value odla_Softmax(odla_value input, odla_int32 axis,
 odla_value odla_LogSoftmax(odla_value input, odla_int32 axis,
                            const odla_value_id value_id);
 
-/* Data movement.
+/* Data movement.  odla_Resize: rank-4 channels-first values; ODLA_NEAREST takes
+ * source index floor(dst * in / out), ODLA_LINEAR is bilinear with pixel
+ * centres at half-integers and clamped edges (the coordinate mode is ignored,
+ * as in the reference's oneDNN backend); ODLA_CUBIC is refused.
  * [ref: ops/odla_ops_process.h:80-84,113-116,160-163,253-256,281-284,355-359,
- *  434-437; dnnl odla_dnnl.cc:455-508,869-898,1331-1358,1526-1551,1906-1990] */
+ *  434-437; dnnl odla_dnnl.cc:455-508,869-898,1331-1358,1526-1551,1906-1990;
+ *  odla_eigen.cc:602-632] */
 odla_value odla_Cast(odla_value input, odla_element_type target_type,
                      const odla_value_id value_id);
 odla_value odla_Concat(odla_values inputs, odla_int32 axis,

@@ -880,6 +880,31 @@ class RefBuilder:
         wi = (np.arange(out_hw[1]) * W) // out_hw[1]
         return self._name(name, np.ascontiguousarray(x[:, :, hi][:, :, :, wi]))
 
+    def resize_linear(self, x, out_hw, name=None):
+        """Bilinear, pixel centres at half-integers, edges clamped: source coordinate
+        s = (o + 0.5) * in / out - 0.5, neighbours floor(s) and floor(s) + 1 clamped
+        into the image, weights 1 - frac and frac.  The reference calls oneDNN's
+        resampling_linear for ODLA_LINEAR whatever coordinate mode is passed
+        [ref: ODLA/platforms/dnnl/odla_dnnl.cc:1526-1551]; oneDNN (1.x / 2.x, not in
+        the reference tree) documents exactly this formula for its linear algorithm."""
+        x = np.asarray(x, np.float64)
+        H, W = x.shape[2], x.shape[3]
+
+        def taps(o_n, i_n):
+            s = (np.arange(o_n, dtype=np.float64) + 0.5) * (i_n / o_n) - 0.5
+            s = np.maximum(s, 0.0)
+            i0 = np.minimum(np.floor(s).astype(np.int64), i_n - 1)
+            i1 = np.minimum(i0 + 1, i_n - 1)
+            return i0, i1, s - i0
+
+        h0, h1, ah = taps(out_hw[0], H)
+        w0, w1, aw = taps(out_hw[1], W)
+        ah = ah.reshape(1, 1, -1, 1)
+        aw = aw.reshape(1, 1, 1, -1)
+        top = x[:, :, h0][:, :, :, w0] * (1 - aw) + x[:, :, h0][:, :, :, w1] * aw
+        bot = x[:, :, h1][:, :, :, w0] * (1 - aw) + x[:, :, h1][:, :, :, w1] * aw
+        return self._name(name, np.ascontiguousarray((top * (1 - ah) + bot * ah).astype(np.float32)))
+
     # quantisation -----------------------------------------------------------
     def quantize(self, x, scale, zp=None, axis=-1, signed=False, name=None):
         """[ref: odla_dnnl_quantization.cc:61-90]"""

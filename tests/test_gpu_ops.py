@@ -625,6 +625,35 @@ def test_reduce_parity():
         assert max_rel_err(got[k], want[k]) <= 1e-5, k
 
 
+@pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16"])
+def test_resize_linear_parity(mode):
+    """Bilinear odla_Resize (up, down, mixed, non-integer ratios, a single row) on a
+    graph argument and on the channels-last result of a convolution."""
+    announce("resize linear (%s)" % mode)
+    r = rng(62)
+    x = r.standard_normal((2, 6, 5, 7)).astype(np.float32)
+    w = (r.standard_normal((8, 6, 1, 1)) * 0.3).astype(np.float32)
+    row = r.standard_normal((1, 3, 1, 9)).astype(np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        b.output(b.resize_linear(a, (10, 14), name="up2"), "up2")
+        b.output(b.resize_linear(a, (8, 3), name="mixed"), "mixed")
+        b.output(b.resize_linear(a, (3, 4), name="down"), "down")
+        c = b.conv(a, b.const("w", w), None, name="c")
+        b.output(b.resize_linear(c, (9, 16), name="after_conv"), "after_conv")
+        b.output(b.resize_linear(b.arg("row", row.shape), (4, 23), name="row_up"), "row_up")
+
+    got, want = run_both(build, {"x": x, "row": row}, fp16=(mode == "fp16"), bf16=(mode == "bf16"))
+    for k in want:
+        assert got[k].shape == want[k].shape, k
+        err = float(np.max(np.abs(got[k] - want[k])))
+        if mode == "fp32":
+            assert err <= F32_TOL * max(1.0, float(np.max(np.abs(want[k])))), k
+        else:
+            assert err <= (2e-2 if mode == "fp16" else 6e-2), k
+
+
 @pytest.mark.parametrize("mode", ["fp32", "fp16"])
 def test_reduce_few_columns_parity(mode):
     """Reductions with too few columns to give every thread one: the rows of the

@@ -368,6 +368,45 @@ def test_resize_nearest_source_index_rule(ref):
         assert np.array_equal(rb.resize_nearest(x, (oh, ow)), want)
 
 
+def test_resize_linear_half_pixel_rule(ref):
+    """ODLA_LINEAR is oneDNN's resampling_linear in the reference
+    [ref: ODLA/platforms/dnnl/odla_dnnl.cc:1526-1551]; that library (1.x / 2.x) is
+    not part of the reference tree, so the oracle restates its published rule
+    (source coordinate (o + 0.5) * in / out - 0.5, two neighbours, edges clamped)
+    and is pinned by what fixes that rule: hand-worked 2x weights, exactness on
+    ramps in the interior, constancy, and two independent library routines that
+    implement the same rule (torch bilinear without corner alignment; scipy's
+    zoom in grid mode with edge replication)."""
+    rb = ref.RefBuilder({})
+    # 2 -> 4: sources at -0.25, 0.25, 0.75, 1.25 -> clamp, 3:1, 1:3, clamp
+    x = np.array([10.0, 20.0], np.float32).reshape(1, 1, 1, 2)
+    assert rb.resize_linear(x, (1, 4)).reshape(-1).tolist() == [10.0, 12.5, 17.5, 20.0]
+    # 4 -> 2: sources at 0.5 and 2.5 -> plain means of neighbours
+    x = np.array([1.0, 3.0, 5.0, 9.0], np.float32).reshape(1, 1, 4, 1)
+    assert rb.resize_linear(x, (2, 1)).reshape(-1).tolist() == [2.0, 7.0]
+    # 3 -> 5 (ratio 0.6): sources -0.2, 0.4, 1.0, 1.6, 2.2
+    x = np.array([0.0, 10.0, 40.0], np.float32).reshape(1, 1, 1, 3)
+    assert np.allclose(rb.resize_linear(x, (1, 5)).reshape(-1), [0.0, 4.0, 10.0, 28.0, 40.0], atol=1e-5)
+    # a ramp is reproduced wherever both neighbours exist; a constant everywhere
+    ramp = (3.0 * np.arange(9, dtype=np.float32) + 2.0).reshape(1, 1, 1, 9)
+    got = rb.resize_linear(ramp, (1, 23)).reshape(-1)
+    src = (np.arange(23) + 0.5) * 9 / 23 - 0.5
+    inside = (src >= 0) & (src <= 8)
+    assert np.allclose(got[inside], 3.0 * src[inside] + 2.0, atol=1e-4)
+    assert np.array_equal(rb.resize_linear(np.full((2, 3, 5, 4), 7.5, np.float32), (9, 11)), np.full((2, 3, 9, 11), 7.5, np.float32))
+
+    torch = pytest.importorskip("torch")
+    from scipy import ndimage
+    r = rng(32)
+    for (ih, iw), (oh, ow) in (((5, 7), (8, 3)), ((13, 13), (26, 26)), ((6, 4), (4, 9)), ((1, 3), (5, 5)), ((7, 5), (7, 12))):
+        x = r.standard_normal((2, 3, ih, iw)).astype(np.float32)
+        got = rb.resize_linear(x, (oh, ow))
+        want = torch.nn.functional.interpolate(torch.from_numpy(x), size=(oh, ow), mode="bilinear", align_corners=False).numpy()
+        assert np.max(np.abs(got - want)) <= 1e-5
+        zoomed = ndimage.zoom(x.astype(np.float64), (1, 1, oh / ih, ow / iw), order=1, mode="nearest", grid_mode=True)
+        assert zoomed.shape == got.shape and np.max(np.abs(got - zoomed)) <= 1e-5
+
+
 def test_cast_rounds_to_even_and_saturates(ref):
     """odla_Cast is a oneDNN reorder in the reference [ref: odla_dnnl_cast.cc:232-258]:
     float -> integer rounds to nearest even and saturates.  Hand-listed values."""
