@@ -339,38 +339,51 @@ hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream) {
 // the source is a stride-1 convolution over this tensor with a quarter of the
 // filter taps and four times the channels: few-channel network inputs then fill
 // their 16-byte vectors instead of being padded 3 -> 8.
-template <typename TS, typename TD>
+// CC = number of source channels (a template parameter so that the channel
+// index of every value is a constant and `out` stays in registers).
+template <typename TS, typename TD, int CC>
 __global__ void __launch_bounds__(kThreads) nchw_to_s2d_kernel(S2dParams p) {
   const TS* src = reinterpret_cast<const TS*>(p.src);
   TD* dst = reinterpret_cast<TD*>(p.dst);
   const int Hs = (p.H + 1) >> 1, Ws = (p.W + 1) >> 1;
   const int64_t total = (int64_t)p.N * Hs * Ws;
+  // an even row length keeps every 2-pixel pair of a float source 8-byte aligned
+  const bool pairs = std::is_same<TS, float>::value && (p.W & 1) == 0 && (reinterpret_cast<uintptr_t>(src) & 7u) == 0;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int ww = (int)(i % Ws);
     const int64_t t = i / Ws;
     const int hh = (int)(t % Hs);
     const int64_t n = t / Hs;
-    TD out[16];
-#pragma unroll
-    for (int c = 0; c < 16; ++c) st_from_float<TD>(&out[c], 0.f, p.scale, p.zp);
+    float in[2][CC][2];
 #pragma unroll
     for (int py = 0; py < 2; ++py) {
       const int h = 2 * hh + py;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if (c < p.C && h < p.H) {
-          const TS* row = src + ((n * p.C + c) * p.H + h) * (int64_t)p.W + 2 * ww;
-          const float v0 = ld_as_float<TS>(row, p.scale, p.zp);
-          const float v1 = (2 * ww + 1 < p.W) ? ld_as_float<TS>(row + 1, p.scale, p.zp) : 0.f;
-          // out[(py*2 + px)*C + c]: C is a run-time value, the index is not a constant
-#pragma unroll
-          for (int j = 0; j < 16; ++j) {
-            if (j == (py * 2 + 0) * p.C + c) st_from_float<TD>(&out[j], v0, p.scale, p.zp);
-            if (j == (py * 2 + 1) * p.C + c) st_from_float<TD>(&out[j], v1, p.scale, p.zp);
+      for (int c = 0; c < CC; ++c) {
+        in[py][c][0] = in[py][c][1] = 0.f;
+        if (h < p.H) {
+          const TS* row = src + ((n * CC + c) * p.H + h) * (int64_t)p.W + 2 * ww;
+          if (pairs) {
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+            const floatx2 v = __builtin_nontemporal_load(reinterpret_cast<const floatx2*>(row));
+            in[py][c][0] = v.x;
+            in[py][c][1] = v.y;
+          } else {
+            in[py][c][0] = ld_as_float<TS>(row, p.scale, p.zp);
+            if (2 * ww + 1 < p.W) in[py][c][1] = ld_as_float<TS>(row + 1, p.scale, p.zp);
           }
         }
       }
     }
+    TD out[16];
+#pragma unroll
+    for (int c = 4 * CC; c < 16; ++c) st_from_float<TD>(&out[c], 0.f, p.scale, p.zp);
+#pragma unroll
+    for (int py = 0; py < 2; ++py)
+#pragma unroll
+      for (int px = 0; px < 2; ++px)
+#pragma unroll
+        for (int c = 0; c < CC; ++c) st_from_float<TD>(&out[(py * 2 + px) * CC + c], in[py][c][px], p.scale, p.zp);
     TD* o = dst + i * p.cs;
     if ((p.cs * sizeof(TD)) % 16 == 0) {
       const int nv = p.cs * (int)sizeof(TD) / 16;
@@ -386,8 +399,13 @@ hipError_t launch_nchw_to_s2d(const S2dParams& p, hipStream_t stream) {
     return hipErrorInvalidValue;
   const int64_t total = (int64_t)p.N * ((p.H + 1) / 2) * ((p.W + 1) / 2);
   const int grid = grid_for(total, kThreads);
-#define K4(TS, TD, ...) hipLaunchKernelGGL((nchw_to_s2d_kernel<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p)
-  LAYOUT_PAIR_DISPATCH(K4, 0);
+#define K4(TS, TD, CC_) hipLaunchKernelGGL((nchw_to_s2d_kernel<TS, TD, CC_>), dim3(grid), dim3(kThreads), 0, stream, p)
+  switch (p.C) {
+    case 1: LAYOUT_PAIR_DISPATCH(K4, 1); break;
+    case 2: LAYOUT_PAIR_DISPATCH(K4, 2); break;
+    case 3: LAYOUT_PAIR_DISPATCH(K4, 3); break;
+    default: LAYOUT_PAIR_DISPATCH(K4, 4); break;
+  }
 #undef K4
   return hipGetLastError();
 }
