@@ -507,6 +507,14 @@ class Planner {
                    int64_t so, int64_t si, int64_t sr, int64_t ss, const std::vector<float>& row_scale,
                    int* w_rs_out, const std::vector<float>* wq_scale, int dense_groups = 0);
   int make_wfrag(const std::string& name, IgemmParams* ip, int tw);
+  // Debug-level log line "<launch>: kernel <variant>" (the device pointers that the
+  // choice looks at are replaced by stand-ins: only their presence matters).
+  void log_igemm_choice(const std::string& name, IgemmParams ip, bool has_wfrag, bool has_residual) {
+    static int dummy;
+    ip.w_frag = has_wfrag ? &dummy : nullptr;
+    ip.residual = has_residual ? &dummy : nullptr;
+    OHIP_DEBUG("%s: kernel %s", name.c_str(), igemm_variant_name(ip));
+  }
   // A value whose only use is Reshape -> [B, S, heads, d] -> Transpose (0, 2, 1, 3): the
   // GEMM that computes it can store [B, heads, S, d] directly (IgemmParams::y_rdiv).
   struct HeadSplit { int reshape = -1, transpose = -1; int64_t B = 0, S = 0, heads = 0, d = 0; _odla_value* out = nullptr; };
@@ -1079,6 +1087,7 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
   ip.stream_out = T(ty).bytes >= stream_out_bytes();
   const int tf = make_wfrag(name, &ip, tw);
   const bool hf = tf >= 0;
+  log_igemm_choice(name, ip, hf, tr >= 0);
   const Ref rf = ref(hf ? tf : tx);
   const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty);
   const Ref rb = ref(tb >= 0 ? tb : tx), rr = ref(tr >= 0 ? tr : tx);
@@ -1301,6 +1310,7 @@ void Planner::lower_conv(int ni) {
     ip.stream_out = T(ty).bytes >= stream_out_bytes();
     const int tf = make_wfrag("conv.i8:" + outv->name, &ip, tw);
     const bool hf = tf >= 0;
+    log_igemm_choice("conv.i8:" + outv->name, ip, hf, tr >= 0);
     const Ref rf = ref(hf ? tf : tx);
     const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb), rm = ref(tm), rr = ref(tr >= 0 ? tr : tx);
     const bool hr = tr >= 0;

@@ -41,10 +41,27 @@ def test_int8_requantisation_cases(tile, monkeypatch, odla, ref):
 
 
 @pytest.mark.parametrize("tile", TILES)
-def test_gemm_with_gelu_bf16(tile, monkeypatch):
-    """[600, 256] x [256, 520] + bias -> GELU: ragged in both tile directions."""
+def test_gemm_with_gelu_bf16(tile, monkeypatch, odla):
+    """[600, 256] x [256, 520] + bias -> GELU: ragged in both tile directions.  The
+    planner's debug log names the kernel it chose for the launch."""
+    import ctypes
     monkeypatch.setenv("ODLA_HIP_IGEMM_TILE", tile)
     announce("big tile gemm %s" % tile)
+    L = odla.load_library()
+    seen = []
+    CB = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p)
+    cb = CB(lambda f, line, fn, lvl, msg: seen.append(msg.decode()))
+    L.odla_SetLogger(ctypes.cast(cb, ctypes.c_void_p))
+    L.odla_SetLogLevel(5)   # ODLA_LOG_LEVEL_DEBUG
+    try:
+        _gemm_with_gelu_bf16()
+    finally:
+        L.odla_SetLogLevel(2)
+        L.odla_SetLogger(None)
+    assert any(m.endswith("kernel " + tile[3:]) for m in seen), seen
+
+
+def _gemm_with_gelu_bf16():
     r = np.random.default_rng(31)
     x = r.standard_normal((600, 256)).astype(np.float32)
     w = (r.standard_normal((256, 520)) * 0.06).astype(np.float32)
