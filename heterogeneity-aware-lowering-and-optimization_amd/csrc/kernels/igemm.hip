@@ -96,9 +96,13 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int off = (l32 * PITCH + wave * 32 + q * 8 + lg * 4) ^ q8_swz(l32);
-      const unsigned rs = has_res ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
-      const unsigned w = requant4(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3],
-                                  mq[q], has_res, rs, p);
+      unsigned w;
+      if (has_res)   // wavefront-uniform
+        w = requant4<true>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q],
+                           *reinterpret_cast<const unsigned*>(rtile + off), p);
+      else
+        w = requant4<false>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q],
+                            0u, p);
       *reinterpret_cast<unsigned*>(otile + off) = w;
     }
     // Nobody passes this barrier before every wavefront has written slice i; a wavefront
@@ -354,7 +358,11 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
     const int wo = rem - ho * p.Wo;
     a_hi0[i] = ok ? ho * p.sh - p.ph : -(1 << 28);  // out-of-range rows never pass the bounds test
     a_wi0[i] = wo * p.sw - p.pw;
-    a_ptr[i] = x + (int64_t)n_img * p.H * p.W * p.xcs;
+    // address of tap (0, 0), channel 0 of this row - possibly outside the image, and only
+    // dereferenced behind the bounds test: a stage then adds one per-thread tap offset
+    // instead of multiplying out (hi * W + wi) * xcs per row (integer multiplies run at a
+    // quarter of the VALU rate)
+    a_ptr[i] = x + ((int64_t)n_img * p.H * p.W + (int64_t)(ok ? ho * p.sh - p.ph : 0) * p.W + a_wi0[i]) * p.xcs;
   }
   // ---- per-thread state for its B (weight) rows ----
   const TIn* b_ptr[B_IT];
@@ -383,11 +391,12 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
   uintx4 ra[A_IT], rb[B_IT];
   auto gload = [&]() {
     const int hoff = kr * p.dh, woff = ks * p.dw;
+    const int toff = (hoff * p.W + woff) * p.xcs + kc;   // from tap (0, 0), channel 0
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) {
       const int hi = a_hi0[i] + hoff, wi = a_wi0[i] + woff;
       const bool ok = (kr < p.R) && ((unsigned)hi < (unsigned)p.H) && ((unsigned)wi < (unsigned)p.W);
-      ra[i] = ok ? *reinterpret_cast<const uintx4*>(a_ptr[i] + ((hi * p.W + wi) * p.xcs + kc)) : fillv;
+      ra[i] = ok ? *reinterpret_cast<const uintx4*>(a_ptr[i] + toff) : fillv;
     }
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) {
@@ -426,7 +435,7 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   if constexpr (EpiTraits<Epi>::quant)
-    acc_init_bias<TM, TN>(p, z, tile_n * BN + __builtin_amdgcn_readfirstlane(wn) * WN, lg, acc);
+    acc_init_bias_vec<TM, TN>(p, z, tile_n * BN + __builtin_amdgcn_readfirstlane(wn) * WN, lg, acc);
 
   const int ktot = p.R * p.S * p.C;
   const int nkt = (ktot + BK - 1) / BK;

@@ -256,15 +256,49 @@ __device__ __forceinline__ void acc_init_bias(const IgemmParams& p, const int z,
       }
 }
 
+// The same through 16-byte vector loads (a lane's four channels of a block are
+// consecutive): for kernels whose vector-memory waits the compiler manages.
+template <int TM, int TN>
+__device__ __forceinline__ void acc_init_bias_vec(const IgemmParams& p, const int z, const int n0, const int lg,
+                                                  intx16 (&acc)[TM][TN]) {
+  if (p.bias == nullptr) return;
+  const int* bias = reinterpret_cast<const int*>(p.bias) + (int64_t)z * p.bias_bs;
+  const int last = p.Kout - 1;  // channels past the end are computed but never stored
+  const bool al = (reinterpret_cast<uintptr_t>(bias) & 15u) == 0;
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int c = n0 + j * 32 + q * 8 + lg * 4;
+      intx4 b;
+      if (al && c + 3 <= last) {
+        b = *reinterpret_cast<const intx4*>(bias + c);
+      } else {
+        b.x = bias[c < last ? c : last];
+        b.y = bias[c + 1 < last ? c + 1 : last];
+        b.z = bias[c + 2 < last ? c + 2 : last];
+        b.w = bias[c + 3 < last ? c + 3 : last];
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        acc[i][j][q * 4 + 0] = b.x;
+        acc[i][j][q * 4 + 1] = b.y;
+        acc[i][j][q * 4 + 2] = b.z;
+        acc[i][j][q * 4 + 3] = b.w;
+      }
+    }
+}
+
 // Requantisation of four consecutive channels of one pixel (one dword of the
 // 8-bit result):  q = sat8(max(fma(float(acc), m, add), lo)), where `add` is the
 // result's zero point or, with a residual, fma(float(r), r_mul, r_add) per
 // channel.  v_cvt_pk_u8_f32 rounds to nearest even and saturates to [0, 255];
 // stored bytes are level - 128, i.e. level ^ 0x80.
+template <bool kRes>
 __device__ __forceinline__ unsigned requant4(const int a0, const int a1, const int a2, const int a3, const floatx4 m,
-                                             const bool has_res, const unsigned res_stored, const IgemmParams& p) {
+                                             const unsigned res_stored, const IgemmParams& p) {
   float add0 = p.q_add, add1 = p.q_add, add2 = p.q_add, add3 = p.q_add;
-  if (has_res) {
+  if constexpr (kRes) {
     const unsigned r = res_stored ^ 0x80808080u;  // stored -> levels
     add0 = __builtin_fmaf((float)(r & 0xffu), p.r_mul, p.r_add);
     add1 = __builtin_fmaf((float)((r >> 8) & 0xffu), p.r_mul, p.r_add);
@@ -408,18 +442,25 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
     wave_fence();
     if (has_res && i + 1 < TM) rfetch(i + 1);
     // requantise in the accumulator layout: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
+    // (the residual case is a wavefront-uniform branch around the whole block: as a
+    // per-element condition it costs a select per value)
+    auto requant_block = [&](auto with_res) {
+      constexpr bool kRes = decltype(with_res)::value;
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int ch = j * 32 + q * 8 + lg * 4;
-        const int off = (l32 * PITCH + ch) ^ q8_swz(l32);
-        const floatx4 m = *reinterpret_cast<const floatx4*>(mtile + ch);
-        const unsigned rs = has_res ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
-        const unsigned w = requant4(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3],
-                                    m, has_res, rs, p);
-        *reinterpret_cast<unsigned*>(otile + off) = w;
-      }
+        for (int q = 0; q < 4; ++q) {
+          const int ch = j * 32 + q * 8 + lg * 4;
+          const int off = (l32 * PITCH + ch) ^ q8_swz(l32);
+          const floatx4 m = *reinterpret_cast<const floatx4*>(mtile + ch);
+          const unsigned rs = kRes ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
+          const unsigned w = requant4<kRes>(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                                            acc[i][j][q * 4 + 3], m, rs, p);
+          *reinterpret_cast<unsigned*>(otile + off) = w;
+        }
+    };
+    if (has_res) requant_block(std::true_type{});
+    else requant_block(std::false_type{});
     wave_fence();
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {
