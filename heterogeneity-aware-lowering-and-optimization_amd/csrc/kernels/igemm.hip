@@ -85,25 +85,23 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
     __builtin_amdgcn_sched_barrier(0);
   };
   lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
-  auto slice = [&](auto slice_no) __attribute__((always_inline)) {
+  // (with or without a residual: two straight-line copies of the slice chosen by one
+  // workgroup-uniform branch; as a condition inside, every value pays a move or a select)
+  auto slice = [&](auto slice_no, auto with_res) __attribute__((always_inline)) {
     constexpr int i = decltype(slice_no)::value;
+    constexpr bool kRes = decltype(with_res)::value;
     unsigned char* otile = smem + (i & 1) * (2 * TILE);
     unsigned char* rtile = otile + TILE;
-    if (has_res) {
+    if constexpr (kRes) {
       *reinterpret_cast<uintx4*>(rtile + rp * PITCH + c16) = q8_swz_chunk(rall[i], rp);
       lds_barrier();
     }
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int off = (l32 * PITCH + wave * 32 + q * 8 + lg * 4) ^ q8_swz(l32);
-      unsigned w;
-      if (has_res)   // wavefront-uniform
-        w = requant4<true>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q],
-                           *reinterpret_cast<const unsigned*>(rtile + off), p);
-      else
-        w = requant4<false>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q],
-                            0u, p);
-      *reinterpret_cast<unsigned*>(otile + off) = w;
+      const unsigned rs = kRes ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
+      *reinterpret_cast<unsigned*>(otile + off) =
+          requant4<kRes>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q], rs, p);
     }
     // Nobody passes this barrier before every wavefront has written slice i; a wavefront
     // writes slice i+1 into the other tile pair, and slice i+2 into this one only after
@@ -113,10 +111,17 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
     const uintx4 v = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + rp * PITCH + c16), rp);
     if (m < M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
   };
-  slice(std::integral_constant<int, 0>{});
-  slice(std::integral_constant<int, 1>{});
-  slice(std::integral_constant<int, 2>{});
-  slice(std::integral_constant<int, 3>{});
+  if (has_res) {
+    slice(std::integral_constant<int, 0>{}, std::true_type{});
+    slice(std::integral_constant<int, 1>{}, std::true_type{});
+    slice(std::integral_constant<int, 2>{}, std::true_type{});
+    slice(std::integral_constant<int, 3>{}, std::true_type{});
+  } else {
+    slice(std::integral_constant<int, 0>{}, std::false_type{});
+    slice(std::integral_constant<int, 1>{}, std::false_type{});
+    slice(std::integral_constant<int, 2>{}, std::false_type{});
+    slice(std::integral_constant<int, 3>{}, std::false_type{});
+  }
 }
 
 // ---------------------------------------------------------------------------
