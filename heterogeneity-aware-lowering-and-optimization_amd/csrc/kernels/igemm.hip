@@ -687,29 +687,11 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   if constexpr (EpiTraits<Epi>::quant) {
     // 8-bit layers: the int32 bias starts in the accumulators (element q*4 + r of
     // a lane is channel wave*32 + q*8 + (lane/32)*4 + r), which takes its addition
-    // out of the requantising epilogue, the busiest part of these layers.  The
-    // addresses are wavefront-uniform so that these are scalar loads: a vector
-    // load here would be one more operation in flight than the hand-counted
-    // waits of the K loop allow for.
-    if (p.bias != nullptr) {
-      const int* bias = reinterpret_cast<const int*>(p.bias) + (int64_t)z * p.bias_bs;
-      const int last = p.Kout - 1;  // channels past the end are computed but never stored
+    // out of the requantising epilogue, the busiest part of these layers.  Eight
+    // 16-byte loads per slice, consumed right here: they are older than every
+    // request the K loop counts, so its waits stay valid.
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        const int nb = (tile_n * NJ + j) * 128 + wave_u * 32;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int c0 = nb + q * 8 + r, c1 = c0 + 4;
-            const int b0 = bias[c0 < last ? c0 : last], b1 = bias[c1 < last ? c1 : last];
-            const int b = lg ? b1 : b0;
-#pragma unroll
-            for (int i = 0; i < TM; ++i) acc[j][i][0][q * 4 + r] = b;
-          }
-        }
-      }
-    }
+    for (int j = 0; j < NJ; ++j) acc_init_bias_vec<TM, 1>(p, z, (tile_n * NJ + j) * 128 + wave_u * 32, lg, acc[j]);
   }
 
   // fragment read offsets: row l32 (+32*i), chunk 2*kk + lg, swizzled
