@@ -44,8 +44,8 @@ METRIC = "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW
 MEASURED_TRAFFIC = {
     # 8.81 GB fetched + 5.76 GB written per step over its 54 conv/gemm launches
     "resnet50_fp16": 269.8e6,
-    # 4.16 GB fetched + 2.99 GB written per step over its 54 conv/gemm launches
-    "resnet50_int8": 132.5e6,
+    # 4.17 GB fetched + 2.99 GB written per step over its 54 conv/gemm launches
+    "resnet50_int8": 132.6e6,
 }
 
 
