@@ -4,6 +4,7 @@
 #define ODLA_HIP_DEVICE_UTILS_H_
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
@@ -78,6 +79,28 @@ template <typename T> struct Vec16 {
     Store<T>::st(e + i, v);
   }
 };
+
+// Eight fp32 values to eight 2-byte values, round to nearest even.  bf16 goes
+// through v_cvt_pk_bf16_f32 (the integer formulation of the same rounding costs
+// five to six instructions per value, a quarter of a bf16 GEMM epilogue).
+template <typename T>
+__device__ __forceinline__ uintx4 pack8_rne(const float (&v)[8]) {
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    uintx4 o;
+    o.x = __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2){v[0], v[1]}, bf16x2));
+    o.y = __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2){v[2], v[3]}, bf16x2));
+    o.z = __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2){v[4], v[5]}, bf16x2));
+    o.w = __builtin_bit_cast(unsigned, __builtin_convertvector((floatx2){v[6], v[7]}, bf16x2));
+    return o;
+  } else {
+    Vec16<T> o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o.set(e, v[e]);
+    return o.raw;
+  }
+}
 
 __device__ __forceinline__ float gelu_erf(float x) {
   return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));

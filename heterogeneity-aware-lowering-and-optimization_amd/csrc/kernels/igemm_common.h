@@ -165,8 +165,7 @@ struct EpiFloat {
         *reinterpret_cast<floatx4*>(y + 4) = (floatx4){v[4], v[5], v[6], v[7]};
       } else {
         Vec16<TOut> o;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o.set(e, v[e]);
+        o.raw = pack8_rne<TOut>(v);
         // (not in the instantiations with the wider activation set: they have no registers to spare)
         if (!kRich && p.stream_out) {
           // The pointer passes through an empty asm so that the optimizer cannot

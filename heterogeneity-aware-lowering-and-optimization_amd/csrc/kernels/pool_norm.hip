@@ -538,7 +538,12 @@ __device__ __forceinline__ float group_sum(float v) {
 
 template <typename TO, int V>
 __device__ __forceinline__ void store_row_vec(TO* dst, const float* v) {
-  if constexpr (sizeof(TO) * V == 16) {
+  if constexpr (sizeof(TO) == 2 && V == 8) {
+    Vec16<TO> o;
+    const float (&v8)[8] = *reinterpret_cast<const float (*)[8]>(v);
+    o.raw = pack8_rne<TO>(v8);
+    o.store(dst);
+  } else if constexpr (sizeof(TO) * V == 16) {
     Vec16<TO> o;
 #pragma unroll
     for (int e = 0; e < V; ++e) o.set(e, v[e]);
