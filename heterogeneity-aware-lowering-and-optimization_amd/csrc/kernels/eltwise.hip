@@ -444,32 +444,50 @@ bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 // consecutive points of its walk at once (register q, point e at
 // regs[(q * E + e) * kThreads + thread]): the E loads of an instruction are in
 // flight together and the decoding of the instruction is shared.
-template <typename T, int E>
+// Activation inside a group.  With 16-bit storage the result keeps 8 or 11
+// significant bits, so the hardware exponential and reciprocal (1 ulp each)
+// stand in for the library's exp and the IEEE division.
+template <typename T>
+__device__ __forceinline__ float fused_act(const float v, const ActKind act, const float a, const float b) {
+  if constexpr (sizeof(T) == 2) {
+    if (act == ACT_SIGMOID) return __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    if (act == ACT_EXP) return __expf(v);
+  }
+  return apply_act(v, act, a, b);
+}
+
+// I is the type of the index arithmetic: 32-bit when the walk and every view fit
+// (integer division and multiplication in 64 bits cost several times as much).
+template <typename T, int E, typename I>
 __global__ void __launch_bounds__(kThreads) fused_eltwise_kernel(const FusedParams p) {
   extern __shared__ float fused_regs[];
   float* r = fused_regs + threadIdx.x;
-  const int64_t d1 = p.dims[1], d2 = p.dims[2], d3 = p.dims[3];
-  const int64_t walk = p.walk > 0 ? p.walk : d2;
-  const int64_t pieces = (d2 + walk - 1) / walk;
-  const int64_t total = p.dims[0] * d1 * pieces * d3;
-  for (int64_t t = blockIdx.x * (int64_t)kThreads + threadIdx.x; t < total; t += (int64_t)gridDim.x * kThreads) {
-    const int64_t i3 = t % d3;
-    int64_t q = t / d3;
-    const int64_t piece = q % pieces;
-    q /= pieces;
-    const int64_t i1 = q % d1, i0 = q / d1;
-    const int64_t i2_end = piece * walk + walk < d2 ? piece * walk + walk : d2;
-    for (int64_t i2 = piece * walk; i2 < i2_end; i2 += E) {
-      const int live = i2_end - i2 < E ? (int)(i2_end - i2) : E;
+  const I d1 = (I)p.dims[1], d2 = (I)p.dims[2], d3 = (I)p.dims[3];
+  const I walk = p.walk > 0 ? (I)p.walk : d2;
+  const I pieces = (d2 + walk - 1) / walk;
+  const int64_t total = p.dims[0] * p.dims[1] * (int64_t)pieces * p.dims[3];
+  for (int64_t t64 = blockIdx.x * (int64_t)kThreads + threadIdx.x; t64 < total; t64 += (int64_t)gridDim.x * kThreads) {
+    const I t = (I)t64;
+    I q = t / d3;
+    const I i3 = t - q * d3;
+    const I q1 = q / pieces;
+    const I piece = q - q1 * pieces;
+    const I i0 = q1 / d1;
+    const I i1 = q1 - i0 * d1;
+    const I i2_end = piece * walk + walk < d2 ? piece * walk + walk : d2;
+    for (I i2 = piece * walk; i2 < i2_end; i2 += E) {
+      const int live = i2_end - i2 < (I)E ? (int)(i2_end - i2) : E;
       for (int k = 0; k < p.n_instr; ++k) {
         const FusedInstr& in = p.prog[k];
         switch (in.op) {
           case FOP_LOAD: {
             const FusedView& v = p.view[in.a];
-            const T* src = reinterpret_cast<const T*>(v.base) + v.off + i0 * v.st[0] + i1 * v.st[1] + i2 * v.st[2] + i3 * v.st[3];
+            const I st2 = (I)v.st[2];
+            const T* src = reinterpret_cast<const T*>(v.base) +
+                           (I)((I)v.off + i0 * (I)v.st[0] + i1 * (I)v.st[1] + i2 * st2 + i3 * (I)v.st[3]);
             float val[E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) val[e] = e < live ? Store<T>::ld(src + e * v.st[2]) : 0.f;
+            for (int e = 0; e < E; ++e) val[e] = e < live ? Store<T>::ld(src + (I)e * st2) : 0.f;
 #pragma unroll
             for (int e = 0; e < E; ++e) r[(in.dst * E + e) * kThreads] = val[e];
             break;
@@ -477,7 +495,7 @@ __global__ void __launch_bounds__(kThreads) fused_eltwise_kernel(const FusedPara
           case FOP_UNARY:
 #pragma unroll
             for (int e = 0; e < E; ++e)
-              r[(in.dst * E + e) * kThreads] = apply_act(r[(in.a * E + e) * kThreads], (ActKind)in.kind, in.fa, in.fb);
+              r[(in.dst * E + e) * kThreads] = fused_act<T>(r[(in.a * E + e) * kThreads], (ActKind)in.kind, in.fa, in.fb);
             break;
           case FOP_BINARY:   // a negative register number selects the immediate
 #pragma unroll
@@ -489,10 +507,12 @@ __global__ void __launch_bounds__(kThreads) fused_eltwise_kernel(const FusedPara
             break;
           default: {
             const FusedView& v = p.view[in.dst];
-            T* dst = const_cast<T*>(reinterpret_cast<const T*>(v.base)) + v.off + i0 * v.st[0] + i1 * v.st[1] + i2 * v.st[2] + i3 * v.st[3];
+            const I st2 = (I)v.st[2];
+            T* dst = const_cast<T*>(reinterpret_cast<const T*>(v.base)) +
+                     (I)((I)v.off + i0 * (I)v.st[0] + i1 * (I)v.st[1] + i2 * st2 + i3 * (I)v.st[3]);
 #pragma unroll
             for (int e = 0; e < E; ++e)
-              if (e < live) Store<T>::st(dst + e * v.st[2], r[(in.a * E + e) * kThreads]);
+              if (e < live) Store<T>::st(dst + (I)e * st2, r[(in.a * E + e) * kThreads]);
             break;
           }
         }
@@ -751,9 +771,27 @@ hipError_t launch_fused_eltwise(const FusedParams& p, hipStream_t stream) {
   const int e = (walk >= 4 && n_regs * 4 <= 32) ? 4 : ((walk >= 2 && n_regs * 2 <= 32) ? 2 : 1);
   const size_t lds = (size_t)n_regs * e * kThreads * sizeof(float);
   const int grid = grid_for(threads, kThreads);
-  if (e == 4) { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, 4>), dim3(grid), dim3(kThreads), lds, stream, p)); }
-  else if (e == 2) { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, 2>), dim3(grid), dim3(kThreads), lds, stream, p)); }
-  else { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, 1>), dim3(grid), dim3(kThreads), lds, stream, p)); }
+  // 32-bit index arithmetic when the thread count and every view's furthest element fit
+  bool small = threads < ((int64_t)1 << 31);
+  for (int v = 0; v < kFusedMaxViews && small; ++v) {
+    if (p.view[v].base == nullptr) continue;
+    int64_t far = p.view[v].off;
+    if (far < 0) small = false;
+    for (int q = 0; q < 4 && small; ++q) {
+      if (p.view[v].st[q] < 0) small = false;
+      else far += (p.dims[q] - 1 + (q == 2 ? e : 0)) * p.view[v].st[q];
+    }
+    if (far >= ((int64_t)1 << 31)) small = false;
+  }
+#define FUSED_LAUNCH(E_)                                                                                                  \
+  do {                                                                                                                    \
+    if (small) { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, E_, uint32_t>), dim3(grid), dim3(kThreads), lds, stream, p)); } \
+    else { FLOAT_DISPATCH(p.dt, hipLaunchKernelGGL((fused_eltwise_kernel<T, E_, int64_t>), dim3(grid), dim3(kThreads), lds, stream, p)); }        \
+  } while (0)
+  if (e == 4) FUSED_LAUNCH(4);
+  else if (e == 2) FUSED_LAUNCH(2);
+  else FUSED_LAUNCH(1);
+#undef FUSED_LAUNCH
   return hipGetLastError();
 }
 

@@ -414,7 +414,8 @@ hipError_t launch_rownorm(const void* x, void* y, DType dt, int64_t rows, int64_
 // out int32 [N][max_out][3] = {image, class, box}, -1 padded.
 // workspace: at least nms_workspace_bytes(N, B) bytes of device memory.
 size_t nms_workspace_bytes(int N, int B);
-hipError_t launch_nms(const float* boxes, const float* scores, int N, int C, int B,
+// boxes / scores are read in their storage type (DT_F32, DT_F16 or DT_BF16).
+hipError_t launch_nms(const void* boxes, DType boxes_dt, const void* scores, DType scores_dt, int N, int C, int B,
                       int max_out, float iou_thr, float score_thr, int32_t* out,
                       void* workspace, hipStream_t stream);
 

@@ -144,25 +144,72 @@ __global__ void __launch_bounds__(kThreads) nhwc_to_nchw_tiled(LayoutParams p) {
 }
 
 // Generic strided copy of `ES`-byte elements; the innermost dim is walked by
-// consecutive threads.
-template <typename E>
+// consecutive threads.  I is the type the flat index is decomposed in: 32-bit
+// division costs a fifth of the 64-bit one.
+template <typename E, typename I>
 __global__ void __launch_bounds__(kThreads) strided_copy_kernel(StridedCopyParams p, int64_t n) {
   const E* x = reinterpret_cast<const E*>(p.x) + p.x_off;
   E* y = reinterpret_cast<E*>(p.y) + p.y_off;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * blockDim.x) {
-    int64_t rem = i, ox = 0, oy = 0;
+    I rem = (I)i;
+    int64_t ox = 0, oy = 0;
 #pragma unroll
     for (int d = 7; d >= 0; --d) {
       if (d < p.rank) {
-        const int64_t q = rem / p.dims[d];
-        const int64_t idx = rem - q * p.dims[d];
+        const I dim = (I)p.dims[d];
+        const I q = rem / dim;
+        const int64_t idx = (int64_t)(rem - q * dim);
         rem = q;
         ox += idx * p.sx[d];
         oy += idx * p.sy[d];
       }
     }
     y[oy] = x[ox];
+  }
+}
+
+// Strided copy whose source is contiguous along one dim (`a`) and whose
+// destination is contiguous along another (`b`): 64 x 64 tiles of the (a, b)
+// plane go through LDS, so that both sides move whole runs.  The remaining
+// dims index the tiles' origins.
+struct TileCopyParams {
+  const void* x; void* y;
+  int64_t x_off, y_off;
+  int Da, Db;          // extents of the two dims
+  int64_t sxb, sya;    // source stride along b, destination stride along a
+  int n_outer;
+  int64_t odims[6], osx[6], osy[6];
+};
+
+template <typename E>
+__global__ void __launch_bounds__(kThreads) strided_tile_copy_kernel(TileCopyParams p, int64_t ntiles) {
+  constexpr int TS = 64;
+  __shared__ E tile[TS][TS + 2];
+  const E* x = reinterpret_cast<const E*>(p.x) + p.x_off;
+  E* y = reinterpret_cast<E*>(p.y) + p.y_off;
+  const int ta_n = (p.Da + TS - 1) / TS, tb_n = (p.Db + TS - 1) / TS;
+  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int a0 = (int)(t % ta_n) * TS;
+    const int b0 = (int)((t / ta_n) % tb_n) * TS;
+    int64_t o = t / ((int64_t)ta_n * tb_n), ox = 0, oy = 0;
+    for (int d = p.n_outer - 1; d >= 0; --d) {
+      const int64_t q = o / p.odims[d], idx = o - q * p.odims[d];
+      o = q;
+      ox += idx * p.osx[d];
+      oy += idx * p.osy[d];
+    }
+    for (int rr = ty; rr < TS; rr += kThreads / TS) {
+      const int b = b0 + rr, a = a0 + tx;
+      if (b < p.Db && a < p.Da) tile[rr][tx] = x[ox + b * p.sxb + a];
+    }
+    __syncthreads();
+    for (int cc = ty; cc < TS; cc += kThreads / TS) {
+      const int a = a0 + cc, b = b0 + tx;
+      if (a < p.Da && b < p.Db) y[oy + a * p.sya + b] = tile[tx][cc];
+    }
+    __syncthreads();
   }
 }
 
@@ -420,22 +467,80 @@ hipError_t launch_nhwc_to_nchw(const LayoutParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_strided_copy(const StridedCopyParams& p, hipStream_t stream) {
-  if (!p.x || !p.y || p.rank < 1 || p.rank > 8) return hipErrorInvalidValue;
+hipError_t launch_strided_copy(const StridedCopyParams& p_in, hipStream_t stream) {
+  if (!p_in.x || !p_in.y || p_in.rank < 1 || p_in.rank > 8) return hipErrorInvalidValue;
   int64_t n = 1;
-  for (int d = 0; d < p.rank; ++d) {
-    if (p.dims[d] <= 0) return hipErrorInvalidValue;
-    n *= p.dims[d];
+  for (int d = 0; d < p_in.rank; ++d) {
+    if (p_in.dims[d] <= 0) return hipErrorInvalidValue;
+    n *= p_in.dims[d];
   }
+  // Drop dims of extent 1 and merge neighbours that both sides walk as one run.
+  StridedCopyParams p = p_in;
+  int r = 0;
+  for (int d = 0; d < p_in.rank; ++d) {
+    if (p_in.dims[d] == 1) continue;
+    if (r > 0 && p.sx[r - 1] == p_in.sx[d] * p_in.dims[d] && p.sy[r - 1] == p_in.sy[d] * p_in.dims[d]) {
+      p.dims[r - 1] *= p_in.dims[d];
+      p.sx[r - 1] = p_in.sx[d];
+      p.sy[r - 1] = p_in.sy[d];
+    } else {
+      p.dims[r] = p_in.dims[d]; p.sx[r] = p_in.sx[d]; p.sy[r] = p_in.sy[d];
+      ++r;
+    }
+  }
+  if (r == 0) { p.dims[0] = 1; p.sx[0] = p.sy[0] = 0; r = 1; }
+  for (int d = r; d < 8; ++d) { p.dims[d] = 1; p.sx[d] = p.sy[d] = 0; }
+  p.rank = r;
+
+  // A dim the source runs along and another the destination runs along: tiles.
+  int a = -1, b = -1;
+  for (int d = 0; d < r; ++d) {
+    if (p.sx[d] == 1 && (a < 0 || p.dims[d] > p.dims[a])) a = d;
+    if (p.sy[d] == 1 && (b < 0 || p.dims[d] > p.dims[b])) b = d;
+  }
+  const bool tiles = a >= 0 && b >= 0 && a != b && p.sy[a] != 1 && p.sx[b] != 1 && p.dims[a] >= 16 &&
+                     p.dims[b] >= 16 && p.dims[a] < (1 << 30) && p.dims[b] < (1 << 30) && r <= 8 &&
+                     p.elem_size <= 8;
+  if (tiles) {
+    TileCopyParams tp;
+    tp.x = p.x; tp.y = p.y; tp.x_off = p.x_off; tp.y_off = p.y_off;
+    tp.Da = (int)p.dims[a]; tp.Db = (int)p.dims[b];
+    tp.sxb = p.sx[b]; tp.sya = p.sy[a];
+    tp.n_outer = 0;
+    int64_t outer = 1;
+    for (int d = 0; d < r; ++d) {
+      if (d == a || d == b) continue;
+      tp.odims[tp.n_outer] = p.dims[d]; tp.osx[tp.n_outer] = p.sx[d]; tp.osy[tp.n_outer] = p.sy[d];
+      ++tp.n_outer;
+      outer *= p.dims[d];
+    }
+    for (int d = tp.n_outer; d < 6; ++d) { tp.odims[d] = 1; tp.osx[d] = tp.osy[d] = 0; }
+    const int64_t ntiles = outer * ((tp.Da + 63) / 64) * ((tp.Db + 63) / 64);
+    const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
+    switch (p.elem_size) {
+      case 1: hipLaunchKernelGGL(strided_tile_copy_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, tp, ntiles); break;
+      case 2: hipLaunchKernelGGL(strided_tile_copy_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, tp, ntiles); break;
+      case 4: hipLaunchKernelGGL(strided_tile_copy_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, tp, ntiles); break;
+      case 8: hipLaunchKernelGGL(strided_tile_copy_kernel<uint64_t>, dim3(grid), dim3(kThreads), 0, stream, tp, ntiles); break;
+      default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+  }
+
   const int grid = grid_for(n, kThreads * 2);
+#define SC(E) do { \
+    if (n < (int64_t)1 << 31) hipLaunchKernelGGL((strided_copy_kernel<E, uint32_t>), dim3(grid), dim3(kThreads), 0, stream, p, n); \
+    else hipLaunchKernelGGL((strided_copy_kernel<E, int64_t>), dim3(grid), dim3(kThreads), 0, stream, p, n); \
+  } while (0)
   switch (p.elem_size) {
-    case 1: hipLaunchKernelGGL(strided_copy_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
-    case 2: hipLaunchKernelGGL(strided_copy_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
-    case 4: hipLaunchKernelGGL(strided_copy_kernel<uint32_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
-    case 8: hipLaunchKernelGGL(strided_copy_kernel<uint64_t>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
-    case 16: hipLaunchKernelGGL(strided_copy_kernel<b16>, dim3(grid), dim3(kThreads), 0, stream, p, n); break;
+    case 1: SC(uint8_t); break;
+    case 2: SC(uint16_t); break;
+    case 4: SC(uint32_t); break;
+    case 8: SC(uint64_t); break;
+    case 16: SC(b16); break;
     default: return hipErrorInvalidValue;
   }
+#undef SC
   return hipGetLastError();
 }
 

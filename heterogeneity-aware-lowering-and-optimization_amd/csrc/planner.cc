@@ -2080,6 +2080,8 @@ bool Planner::fuse_slice_seed(int ni) const {
 
 // `seed`: the operator the group grows from; `from` <= seed: the node being
 // lowered, where the group's launch is emitted.
+static constexpr int64_t kTransposeSinkMax = 1 << 22;
+
 bool Planner::lower_fused_group(int seed, int from) {
   const int n_nodes = (int)comp_->nodes.size();
   if (no_fuse_.empty()) no_fuse_.assign((size_t)n_nodes, 0);
@@ -2264,7 +2266,11 @@ bool Planner::lower_fused_group(int seed, int from) {
           continue;
         }
       }
-      if (cn.op == OP_TRANSPOSE && !cn.absorbed && full && storage_dtype(cn.out) == dt && (int)cn.iv.size() == R) {
+      // A Transpose that moves the innermost dim turns the group's stores into single
+      // elements a row apart; beyond a few million elements the tiled copy
+      // behind a plain store is several times faster than that.
+      if (cn.op == OP_TRANSPOSE && !cn.absorbed && full && storage_dtype(cn.out) == dt && (int)cn.iv.size() == R &&
+          (cn.iv[R - 1] == R - 1 || S.numel() <= kTransposeSinkMax)) {
         if (std::find(sink_nodes.begin(), sink_nodes.end(), c) == sink_nodes.end()) {
           sink_nodes.push_back(c);
           sinks.push_back({c, v, 2, 0});
@@ -2399,6 +2405,10 @@ bool Planner::lower_fused_group(int seed, int from) {
     }
     if (mi != nullptr && mi->st[d3] != 1)
       for (int i = 0; i < R; ++i) if (i != d3 && S.d[i] > 1 && mi->st[i] == 1) d2 = i;
+    // no such dim: with points to spare, a thread still takes four per decoded instruction,
+    // along the longest other dim
+    if (d2 < 0 && S.numel() >= (int64_t)4 * 256 * 2048)
+      for (int i = 0; i < R; ++i) if (i != d3 && S.d[i] >= 4 && (d2 < 0 || S.d[i] > S.d[d2])) d2 = i;
   }
   int order[4] = {-1, -1, d2, d3};
   {
@@ -2412,7 +2422,7 @@ bool Planner::lower_fused_group(int seed, int from) {
     const int64_t base = fp.dims[0] * fp.dims[1] * fp.dims[3];
     const int64_t want = 256 * 2048 * 2;
     int64_t w = fp.dims[2] * base / want;
-    fp.walk = std::min<int64_t>(fp.dims[2], std::max<int64_t>(4, w));
+    fp.walk = std::min<int64_t>(fp.dims[2], std::max<int64_t>(4, w / 4 * 4));   // whole groups of four points
   }
   for (size_t k = 0; k < views.size(); ++k) {
     fp.view[k].off = views[k].off;
@@ -3091,9 +3101,10 @@ void Planner::lower_nms(int ni) {
   Node& n = comp_->nodes[ni];
   const _odla_value* boxes = n.in[0];
   const _odla_value* scores = n.in[1];
-  auto as_f32 = [&](const _odla_value* v) -> int {
+  // fp32 / fp16 / bf16 are read as they are stored; anything else is converted first
+  auto as_float = [&](const _odla_value* v) -> int {
     int t = get(v, L_ROWMAJOR, FORM_FLOAT);
-    if (T(t).dt == DT_F32) return t;
+    if (T(t).dt == DT_F32 || T(t).dt == DT_F16 || T(t).dt == DT_BF16) return t;
     const int d = new_tensor(DT_F32, L_ROWMAJOR, v->shape, 0, SP_ARENA);
     const int64_t ne = v->shape.numel();
     const DType sdt = T(t).dt;
@@ -3101,7 +3112,8 @@ void Planner::lower_nms(int ni) {
     emit("nms.cast:" + v->name, {t}, {d}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), DT_F32, ne, st); });
     return d;
   };
-  const int tb = as_f32(boxes), ts = as_f32(scores);
+  const int tb = as_float(boxes), ts = as_float(scores);
+  const DType bdt = T(tb).dt, sdt = T(ts).dt;
   const int N = (int)boxes->shape.d[0], B = (int)boxes->shape.d[1], C = (int)scores->shape.d[1];
   const int max_out = (int)n.i[0];
   const float iou = n.f[0], thr = n.f[1];
@@ -3110,7 +3122,7 @@ void Planner::lower_nms(int ni) {
   const int ty = new_tensor(DT_I32, L_ROWMAJOR, o32, 0, SP_ARENA);
   const Ref rb = ref(tb), rs = ref(ts), rw = ref(tw), ry = ref(ty);
   emit("nms:" + n.out->name, {tb, ts, tw}, {ty, tw}, [=](const ExecEnv& e, hipStream_t st) {
-    return launch_nms((const float*)rb(e), (const float*)rs(e), N, C, B, max_out, iou, thr, (int32_t*)ry(e), rw(e), st);
+    return launch_nms(rb(e), bdt, rs(e), sdt, N, C, B, max_out, iou, thr, (int32_t*)ry(e), rw(e), st);
   });
   if (dtype_from_odla(n.out->etype) == DT_I64) {
     const int t64 = new_tensor(DT_I64, L_ROWMAJOR, o32, 0, SP_ARENA);
