@@ -174,12 +174,63 @@ namespace {
 void drop_graph(_odla_context* ctx) {
   if (ctx->graph_exec) { (void)hipGraphExecDestroy(ctx->graph_exec); ctx->graph_exec = nullptr; }
   if (ctx->graph) { (void)hipGraphDestroy(ctx->graph); ctx->graph = nullptr; }
+  ctx->graph_ext.clear();
+  for (_odla_context::ParkedGraph& g : ctx->parked_graphs) {
+    if (g.exec) (void)hipGraphExecDestroy(g.exec);
+    if (g.graph) (void)hipGraphDestroy(g.graph);
+  }
+  ctx->parked_graphs.clear();
 }
 
-odla_status run_steps(_odla_context* ctx, const Plan& plan, char* arena) {
+constexpr size_t kMaxParkedGraphs = 3;
+
+// The captured launches hold the argument buffers they read in place.  When the
+// caller has bound other buffers, the current graph is set aside and one captured
+// for these buffers comes back, if there is one; otherwise graph_exec stays null and
+// the caller captures.
+void select_graph(_odla_context* ctx, const std::vector<const char*>& ext) {
+  if (ctx->graph_exec == nullptr || ctx->graph_ext == ext) return;
+  ctx->parked_graphs.push_back({ctx->graph_ext, ctx->graph, ctx->graph_exec});
+  ctx->graph = nullptr;
+  ctx->graph_exec = nullptr;
+  for (size_t i = 0; i < ctx->parked_graphs.size(); ++i) {
+    if (ctx->parked_graphs[i].ext != ext) continue;
+    ctx->graph = ctx->parked_graphs[i].graph;
+    ctx->graph_exec = ctx->parked_graphs[i].exec;
+    ctx->graph_ext = ext;
+    ctx->parked_graphs.erase(ctx->parked_graphs.begin() + (long)i);
+    return;
+  }
+  if (ctx->parked_graphs.size() > kMaxParkedGraphs) {
+    (void)hipGraphExecDestroy(ctx->parked_graphs.front().exec);
+    (void)hipGraphDestroy(ctx->parked_graphs.front().graph);
+    ctx->parked_graphs.erase(ctx->parked_graphs.begin());
+  }
+}
+
+// ODLA_HIP_IN_PLACE_ARGS=0 copies every argument into the arena, as for host buffers.
+bool in_place_args_enabled() {
+  static const bool on = [] {
+    const char* e = getenv("ODLA_HIP_IN_PLACE_ARGS");
+    return e == nullptr || strcmp(e, "0") != 0;
+  }();
+  return on;
+}
+
+bool is_device_memory(const void* p) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();   // ordinary host memory is reported as an error
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice;
+}
+
+odla_status run_steps(_odla_context* ctx, const Plan& plan, char* arena, const std::vector<const char*>* ext = nullptr) {
   ExecEnv env;
   env.base[SP_ARENA] = arena;
   env.base[SP_CONST] = plan.const_pool;
+  env.ext = ext != nullptr && !ext->empty() ? ext->data() : nullptr;
   for (const Step& s : plan.steps) {
     hipError_t e = s.fn(env, ctx->stream);
     if (e != hipSuccess) {
@@ -190,12 +241,22 @@ odla_status run_steps(_odla_context* ctx, const Plan& plan, char* arena) {
   return ODLA_SUCCESS;
 }
 
-odla_status stage_inputs(_odla_context* ctx, const Plan& plan, char* arena) {
-  for (const Plan::IO& io : plan.inputs) {
+// Copies the bound arguments into their staging tensors.  With `ext`, an argument
+// that lives in device memory and that the plan can read in place is not copied:
+// its buffer is entered in (*ext)[k] instead (nullptr for the copied ones).
+odla_status stage_inputs(_odla_context* ctx, const Plan& plan, char* arena, std::vector<const char*>* ext = nullptr) {
+  if (ext != nullptr) ext->assign(plan.inputs.size() + plan.outputs.size(), nullptr);
+  for (size_t k = 0; k < plan.inputs.size(); ++k) {
+    const Plan::IO& io = plan.inputs[k];
     auto it = ctx->bound_in.find(io.v);
     if (it == ctx->bound_in.end()) {
       OHIP_ERR("argument '%s' is not bound", io.v->name.c_str());
       return ODLA_INVALID_PARAM;
+    }
+    if (ext != nullptr && io.in_place_ok && in_place_args_enabled() && is_device_memory(it->second)) {
+      (*ext)[k] = static_cast<const char*>(it->second);
+      OHIP_DEBUG("argument '%s' is read in place", io.v->name.c_str());
+      continue;
     }
     char* dst = arena + plan.tensors[io.tensor].offset;
     if (hipMemcpyAsync(dst, it->second, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
@@ -206,11 +267,40 @@ odla_status stage_inputs(_odla_context* ctx, const Plan& plan, char* arena) {
   return ODLA_SUCCESS;
 }
 
+// Results bound to device memory that the final conversion can write directly: their
+// buffers are entered behind the arguments in *ext (filled by stage_inputs).  A buffer
+// that overlaps an argument read in place keeps its copy.
+void place_outputs(_odla_context* ctx, const Plan& plan, std::vector<const char*>* ext) {
+  if (!in_place_args_enabled()) return;
+  const size_t n_in = plan.inputs.size();
+  for (size_t k = 0; k < plan.outputs.size(); ++k) {
+    const Plan::IO& io = plan.outputs[k];
+    if (!io.in_place_ok) continue;
+    auto it = ctx->bound_out.find(io.v);
+    if (it == ctx->bound_out.end() || it->second == nullptr) continue;
+    const char* p = static_cast<const char*>(it->second);
+    if ((reinterpret_cast<uintptr_t>(p) & 15u) != 0 || !is_device_memory(p)) continue;
+    bool clash = false;
+    for (size_t j = 0; j < n_in + k && !clash; ++j) {
+      const char* q = (*ext)[j];
+      if (q == nullptr) continue;
+      const size_t qb = j < n_in ? plan.inputs[j].bytes : plan.outputs[j - n_in].bytes;
+      clash = p < q + qb && q < p + io.bytes;
+    }
+    if (clash) continue;
+    (*ext)[n_in + k] = p;
+    OHIP_DEBUG("result '%s' is written in place", io.v->name.c_str());
+  }
+}
+
 // Copies the bound results out of `arena` (or the constant pool) and waits for the stream.
-odla_status fetch_outputs(_odla_context* ctx, const Plan& plan, const char* arena) {
-  for (const Plan::IO& io : plan.outputs) {
+odla_status fetch_outputs(_odla_context* ctx, const Plan& plan, const char* arena,
+                          const std::vector<const char*>* ext = nullptr) {
+  for (size_t k = 0; k < plan.outputs.size(); ++k) {
+    const Plan::IO& io = plan.outputs[k];
     auto it = ctx->bound_out.find(io.v);
     if (it == ctx->bound_out.end()) continue;
+    if (ext != nullptr && !ext->empty() && (*ext)[plan.inputs.size() + k] != nullptr) continue;   // already there
     const PTensor& t = plan.tensors[io.tensor];
     const char* src = (t.space == SP_CONST ? plan.const_pool : arena) + t.offset + io.offset;
     if (hipMemcpyAsync(it->second, src, io.bytes, hipMemcpyDefault, ctx->stream) != hipSuccess) {
@@ -586,20 +676,24 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
   if (!c->plan) return ODLA_FAILURE;
   const Plan& plan = *c->plan;
 
-  // 1. stage arguments (host -> device across PCIe, or device -> device)
+  // 1. stage arguments (host -> device across PCIe, or device -> device; device buffers
+  //    that the first steps can read where they are stay there)
+  std::vector<const char*> ext;
   {
-    odla_status st = stage_inputs(ctx, plan, ctx->arena);
+    odla_status st = stage_inputs(ctx, plan, ctx->arena, &ext);
     if (st != ODLA_SUCCESS) return st;
+    place_outputs(ctx, plan, &ext);
   }
 
   // 2. launch sequence: captured once into a hipGraph, replayed afterwards
   if (ctx->use_graph && !plan.steps.empty()) {
+    select_graph(ctx, ext);
     if (ctx->graph_exec == nullptr) {
       if (hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
         OHIP_ERR("odla_ExecuteComputation: hipStreamBeginCapture failed");
         return ODLA_FAILURE;
       }
-      odla_status st = run_steps(ctx, plan, ctx->arena);
+      odla_status st = run_steps(ctx, plan, ctx->arena, &ext);
       hipGraph_t g = nullptr;
       hipError_t e = hipStreamEndCapture(ctx->stream, &g);
       if (st != ODLA_SUCCESS || e != hipSuccess || g == nullptr) {
@@ -608,6 +702,7 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
         return ODLA_FAILURE;
       }
       ctx->graph = g;
+      ctx->graph_ext = ext;
       if (hipGraphInstantiate(&ctx->graph_exec, g, nullptr, nullptr, 0) != hipSuccess) {
         drop_graph(ctx);
         OHIP_ERR("odla_ExecuteComputation: hipGraphInstantiate failed");
@@ -619,13 +714,14 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
       return ODLA_FAILURE;
     }
   } else {
-    odla_status st = run_steps(ctx, plan, ctx->arena);
+    odla_status st = run_steps(ctx, plan, ctx->arena, &ext);
     if (st != ODLA_SUCCESS) return st;
   }
 
   // 3. results
-  odla_status st = fetch_outputs(ctx, plan, ctx->arena);
+  odla_status st = fetch_outputs(ctx, plan, ctx->arena, &ext);
   if (st != ODLA_SUCCESS) return st;
+  ctx->last_ext = ext;
   ctx->executed = true;
   if (!plan.stat_recs.empty()) return profiler_collect(plan, ctx->arena);
   return ODLA_SUCCESS;
@@ -903,10 +999,13 @@ odla_status odla_GetValueData(const odla_value value, odla_void* data_ptr, odla_
   }
   if (!ctx->executed || !ctx->comp->plan) return ODLA_FAILURE;
   const Plan& plan = *ctx->comp->plan;
-  for (const Plan::IO& io : plan.outputs) {
+  for (size_t k = 0; k < plan.outputs.size(); ++k) {
+    const Plan::IO& io = plan.outputs[k];
     if (io.v != value) continue;
     const PTensor& t = plan.tensors[io.tensor];
     const char* src = (t.space == SP_CONST ? plan.const_pool : ctx->arena) + t.offset + io.offset;
+    const size_t slot = plan.inputs.size() + k;
+    if (slot < ctx->last_ext.size() && ctx->last_ext[slot] != nullptr) src = ctx->last_ext[slot];   // written in place
     if (hipMemcpy(data_ptr, src, io.bytes, hipMemcpyDefault) != hipSuccess) return ODLA_FAILURE;
     return ODLA_SUCCESS;
   }

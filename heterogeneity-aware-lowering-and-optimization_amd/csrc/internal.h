@@ -129,6 +129,7 @@ struct PTensor {
   size_t alias_off = 0;  // byte offset of an alias inside the root tensor's storage
   int def_step = -1, last_step = -1;
   bool pinned = false;   // lives for the whole execution (inputs being staged, outputs)
+  int ext_slot = -1;     // argument staging tensor that steps may read in the caller's buffer instead (ExecEnv::ext)
   bool quant = false;    // 8-bit affine levels stored as q-128
   float qscale = 1.f;
   int qzp = 0;
@@ -140,6 +141,10 @@ struct PTensor {
 
 struct ExecEnv {
   char* base[3] = {nullptr, nullptr, nullptr};  // indexed by Space
+  // Per argument (Plan::inputs order), then per result (Plan::outputs order): the caller's
+  // device buffer when the steps read / write it in place, nullptr when the data goes
+  // through the staging tensor in the arena.
+  const char* const* ext = nullptr;
 };
 
 struct Step {
@@ -167,6 +172,11 @@ struct Plan {
     int tensor = -1;  // staging tensor in the arena: row-major, declared element type
     size_t offset = 0;  // byte offset inside that tensor (results that are slices of a merged launch)
     size_t bytes = 0;
+    // arguments: every step that touches the staging tensor reads exactly its elements and
+    // checks alignment itself, and nothing writes it: a device buffer can be read in place;
+    // results: only the final conversion to the declared type touches the tensor, and it
+    // writes exactly its elements: a device buffer can be written in place
+    bool in_place_ok = false;
   };
   std::vector<IO> inputs, outputs;
   std::unordered_map<const _odla_value*, int> final_tensor;  // for odla_GetValueData
@@ -248,6 +258,12 @@ struct _odla_context {
   bool use_graph = true;
   hipGraph_t graph = nullptr;
   hipGraphExec_t graph_exec = nullptr;
+  std::vector<const char*> graph_ext;   // the caller's buffers the captured launches read / write in place
+  std::vector<const char*> last_ext;    // those of the last execution (odla_GetValueData finds results there)
+  // Graphs captured for other sets of argument buffers (a caller that alternates between a
+  // few device buffers replays instead of capturing again); bounded, oldest dropped first.
+  struct ParkedGraph { std::vector<const char*> ext; hipGraph_t graph; hipGraphExec_t exec; };
+  std::vector<ParkedGraph> parked_graphs;
   std::unordered_map<const _odla_value*, const void*> bound_in;
   std::unordered_map<const _odla_value*, void*> bound_out;
   bool executed = false;

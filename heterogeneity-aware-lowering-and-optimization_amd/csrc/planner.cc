@@ -17,6 +17,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <unordered_set>
 
 #include "internal.h"
 
@@ -146,6 +147,7 @@ class Planner {
     plan_->tensors.push_back(t);
     return (int)plan_->tensors.size() - 1;
   }
+  std::unordered_set<int> arena_only_;   // root tensors that some step writes, or reads relying on the arena
   int root(int t) const {
     while (plan_->tensors[t].alias_of >= 0) t = plan_->tensors[t].alias_of;
     return t;
@@ -160,6 +162,8 @@ class Planner {
       int r = t;
       while (plan->tensors[r].alias_of >= 0) r = plan->tensors[r].alias_of;
       const PTensor& pt = plan->tensors[r];
+      if (pt.ext_slot >= 0 && env.ext != nullptr && env.ext[pt.ext_slot] != nullptr)
+        return const_cast<char*>(env.ext[pt.ext_slot]) + plan->tensors[t].alias_off;
       return env.base[pt.space] + pt.offset + plan->tensors[t].alias_off;  // (alias offsets are relative to the root)
     }
   };
@@ -185,6 +189,11 @@ class Planner {
     };
     for (int t : reads) touch(t);
     for (int t : writes) touch(t);
+    // Layout conversions read exactly the elements of their source and test its alignment
+    // at launch; any other reader may rely on the arena (256-byte bases, slack behind a tensor).
+    const bool exact_reader = name.compare(0, 8, "to_nhwc:") == 0 || name.compare(0, 7, "to_s2d:") == 0;
+    for (int t : reads) if (t >= 0 && !exact_reader) arena_only_.insert(root(t));
+    for (int t : writes) if (t >= 0) arena_only_.insert(root(t));
     plan_->steps.push_back({name, std::move(fn)});
   }
 
@@ -675,6 +684,7 @@ void Planner::run() {
   for (_odla_value* ov : comp_->outputs) {
     const DType want = dtype_from_odla(ov->etype);
     int t = get(ov, L_ROWMAJOR, FORM_FLOAT);
+    bool converted = false;
     if (T(t).dt != want) {
       const int dst = new_tensor(want, L_ROWMAJOR, ov->shape, 0, SP_ARENA);
       const int64_t n = ov->shape.numel();
@@ -682,6 +692,7 @@ void Planner::run() {
       const Ref a = ref(t), b = ref(dst);
       emit("out.cast:" + ov->name, {t}, {dst}, [=](const ExecEnv& e, hipStream_t st) { return launch_cast(a(e), sdt, b(e), want, n, st); });
       t = dst;
+      converted = true;
     }
     PTensor& p = T(root(t));
     if (p.space == SP_ARENA) { p.pinned = true; p.last_step = 1 << 30; }
@@ -690,7 +701,26 @@ void Planner::run() {
     io.tensor = root(t);
     io.offset = T(t).alias_off;
     io.bytes = (size_t)ov->shape.numel() * dtype_size(want);
+    // The conversion to the declared type is the only step that touches its result, and it
+    // writes exactly the result's elements: it can write the caller's device buffer directly.
+    if (converted && !calib_ && io.tensor == t && io.offset == 0) {
+      io.in_place_ok = true;
+      T(t).ext_slot = (int)(plan_->inputs.size() + plan_->outputs.size());
+    }
     plan_->outputs.push_back(io);
+  }
+  // Arguments whose staging tensor only layout conversions read: the conversion can read the
+  // caller's device buffer, and the copy into the arena is skipped.
+  for (size_t k = 0; k < plan_->inputs.size(); ++k) {
+    Plan::IO& io = plan_->inputs[k];
+    const int r = root(io.tensor);
+    bool ok = !calib_ && r == io.tensor && T(r).space == SP_ARENA && T(r).last_step >= 0 && !arena_only_.count(r);
+    for (const Plan::IO& o : plan_->outputs) ok = ok && root(o.tensor) != r;
+    for (const auto& ft : plan_->final_tensor) ok = ok && root(ft.second) != r;
+    if (ok) {
+      io.in_place_ok = true;
+      T(r).ext_slot = (int)k;
+    }
   }
   assign_arena();
 }
