@@ -253,7 +253,7 @@ odla_status stage_inputs(_odla_context* ctx, const Plan& plan, char* arena, std:
       OHIP_ERR("argument '%s' is not bound", io.v->name.c_str());
       return ODLA_INVALID_PARAM;
     }
-    if (ext != nullptr && io.in_place_ok && in_place_args_enabled() && is_device_memory(it->second)) {
+    if (ext != nullptr && io.in_place_ok && !ctx->in_place_off && in_place_args_enabled() && is_device_memory(it->second)) {
       (*ext)[k] = static_cast<const char*>(it->second);
       OHIP_DEBUG("argument '%s' is read in place", io.v->name.c_str());
       continue;
@@ -271,7 +271,7 @@ odla_status stage_inputs(_odla_context* ctx, const Plan& plan, char* arena, std:
 // buffers are entered behind the arguments in *ext (filled by stage_inputs).  A buffer
 // that overlaps an argument read in place keeps its copy.
 void place_outputs(_odla_context* ctx, const Plan& plan, std::vector<const char*>* ext) {
-  if (!in_place_args_enabled()) return;
+  if (!in_place_args_enabled() || ctx->in_place_off) return;
   const size_t n_in = plan.inputs.size();
   for (size_t k = 0; k < plan.outputs.size(); ++k) {
     const Plan::IO& io = plan.outputs[k];
@@ -688,6 +688,22 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
   // 2. launch sequence: captured once into a hipGraph, replayed afterwards
   if (ctx->use_graph && !plan.steps.empty()) {
     select_graph(ctx, ext);
+    // A caller that brings new buffers every time would capture every time: after a few
+    // captures in a row this context goes back to staging copies and one graph.
+    constexpr int kCaptureStreakLimit = 8;
+    if (ctx->graph_exec != nullptr) {
+      ctx->capture_streak = 0;
+    } else if (++ctx->capture_streak > kCaptureStreakLimit && !ctx->in_place_off) {
+      bool any = false;
+      for (const char* p : ext) any = any || p != nullptr;
+      if (any) {
+        OHIP_INFO("odla_ExecuteComputation: %d executions in a row with new device buffers; arguments and results are copied from now on", ctx->capture_streak);
+        ctx->in_place_off = true;
+        drop_graph(ctx);
+        odla_status st2 = stage_inputs(ctx, plan, ctx->arena, &ext);
+        if (st2 != ODLA_SUCCESS) return st2;
+      }
+    }
     if (ctx->graph_exec == nullptr) {
       if (hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
         OHIP_ERR("odla_ExecuteComputation: hipStreamBeginCapture failed");

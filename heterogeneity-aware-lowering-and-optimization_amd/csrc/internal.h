@@ -260,6 +260,8 @@ struct _odla_context {
   hipGraphExec_t graph_exec = nullptr;
   std::vector<const char*> graph_ext;   // the caller's buffers the captured launches read / write in place
   std::vector<const char*> last_ext;    // those of the last execution (odla_GetValueData finds results there)
+  int capture_streak = 0;               // executions in a row that had to capture for new buffers
+  bool in_place_off = false;            // the caller binds new buffers every time: copy instead
   // Graphs captured for other sets of argument buffers (a caller that alternates between a
   // few device buffers replays instead of capturing again); bounded, oldest dropped first.
   struct ParkedGraph { std::vector<const char*> ext; hipGraph_t graph; hipGraphExec_t exec; };

@@ -196,3 +196,38 @@ def test_device_results_are_written_in_place():
         L.odla_SetLogger(None)
         bufs.free()
         hb.destroy()
+
+
+def test_new_buffer_every_call_goes_back_to_copies():
+    """Twelve executions, each with another device buffer: after eight captures in a
+    row the context stages the argument again and replays one graph."""
+    announce("device arguments, a new buffer every call")
+    pkg = entry.load()
+    odla = pkg.odla
+    L = odla.load_library()
+    N = 2
+    r = np.random.default_rng(20)
+    hb = odla.HipBuilder()
+    bufs = DeviceBuffers(odla, L)
+    seen = []
+    cb = capture_log(L, seen)
+    try:
+        small_net(hb, N, True)
+        s = hb.session(True)
+        oh, oshape, odt = hb.outs["y"]
+        out = np.empty(oshape, odt)
+        assert L.odla_BindToOutput(oh, out.ctypes.data_as(ctypes.c_void_p), s.ctx) == 0
+        for k in range(12):
+            x = r.standard_normal((N, 3, 20, 20)).astype(np.float32)
+            want = run_ref(lambda b: small_net(b, N, True), {"x": x})["y"]
+            assert L.odla_BindToArgument(hb.args["x"][0], bufs.put(x), s.ctx) == 0
+            s.execute()
+            assert float(np.max(np.abs(out - want))) <= 1e-4 * max(1.0, float(np.max(np.abs(want)))), k
+        assert any("copied from now on" in m for m in seen)
+        assert sum("read in place" in m for m in seen) <= 9
+        s.close()
+    finally:
+        L.odla_SetLogLevel(2)
+        L.odla_SetLogger(None)
+        bufs.free()
+        hb.destroy()
