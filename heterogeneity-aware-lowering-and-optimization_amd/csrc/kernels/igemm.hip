@@ -876,6 +876,146 @@ igemm_lean_kernel(const IgemmParams p, const int epi_vec, const int tiles_per_wg
   }
 }
 
+// ---------------------------------------------------------------------------
+// Variant for filters over one or two 16-byte vectors of channels per tap
+// (network stems: three input channels padded to a vector, or their
+// space-to-depth form).  K is R*S short taps and the layer is pure streaming
+// like the 1x1 case above; the 16 bytes a lane supplies to a matrix
+// instruction are exactly one vector of one tap of its pixel, so they come
+// straight from global memory into the operand register (the overlap between
+// the windows of neighbouring pixels is served by the caches), nothing is
+// staged and nothing is shared.  Every wavefront owns 32 pixels x 64 channels
+// and keeps the fragment-ordered weights of all K steps in registers for the
+// pixel tiles it walks; the pixels of the next tile are requested between the
+// matrix instructions of the current one and its epilogue.  A tap's position
+// is tested against the image only for pixel blocks that touch the border.
+// NKK = 32-byte K steps (R*S*VPT 16-byte units, rounded up to a pair);
+// VPT = 16-byte vectors per tap (xcs * sizeof(TIn) / 16).
+template <typename TIn, typename Epi, int NKK, int VPT, int NJ>
+__global__ void __launch_bounds__(256, 2)
+igemm_taps_kernel(const IgemmParams p, const int epi_vec, const int tiles_per_wg) {
+  // NJ = 2: four wavefronts on four 32-pixel blocks, 64 channels each; NJ = 1 (K rows too
+  // long to keep 64 channels of weights in registers): two blocks, two channel halves
+  constexpr int BM = NJ == 2 ? 128 : 64, BN = 64, WN = 32 * NJ;
+  using Acc = typename Mma<TIn>::Acc;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * 32 * (64 + 4) * 4];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, lg = lane >> 5;
+  const int wm = wave % (BM / 32), wn = wave / (BM / 32);
+  const int M = p.N * p.Ho * p.Wo;
+  const int tiles_m = (M + BM - 1) / BM;
+  const int tiles_n = (p.Kout + BN - 1) / BN;
+  int bid = blockIdx.x;
+  {
+    const int per = gridDim.x >> 3;
+    if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int tile_n = bid % tiles_n;
+  const int tm0 = (bid / tiles_n) * tiles_per_wg;
+  const int tm1 = tm0 + tiles_per_wg < tiles_m ? tm0 + tiles_per_wg : tiles_m;
+
+  const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag) + lane;
+  uintx4 w[NJ][NKK];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    int wtile = tile_n * 2 + wn * NJ + j;
+    wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;  // a surplus slice computes channels that are never stored
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) w[j][kk] = wf[((int64_t)wtile * p.wf_chunks + kk) * 64];
+  }
+
+  // The accumulators start at the bias (held for every pixel tile this wavefront walks),
+  // and the multipliers of an 8-bit layer are parked once: the epilogues then begin with
+  // no vector-memory wait, behind which the next tile's pixels would have to queue.
+  Acc acc0[1][NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc0[0][j][e] = 0;
+  IgemmParams pe = p;   // the epilogue's view: no bias left to add
+  if constexpr (EpiTraits<Epi>::quant) {
+    acc_init_bias_vec<1, NJ>(p, 0, tile_n * BN + wn * WN, lg, acc0);
+    constexpr int TILE = 32 * (WN + 16);
+    float* mtile = reinterpret_cast<float*>(smem + wave * (2 * TILE + WN * 4) + 2 * TILE);
+    if (lane < WN / 4) *reinterpret_cast<floatx4*>(mtile + lane * 4) = load_qmul4(p.qmul, tile_n * BN + wn * WN + lane * 4, p.Kout);
+  } else {
+    if (p.bias != nullptr) {
+      const float* bias = reinterpret_cast<const float*>(p.bias);
+      const int last = p.Kout - 1;   // channels past the end are computed but never stored
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int c = tile_n * BN + wn * WN + j * 32 + q * 8 + lg * 4 + r;
+            acc0[0][j][q * 4 + r] = p.alpha == 1.0f ? bias[c < last ? c : last] : 0.f;
+          }
+      if (p.alpha == 1.0f) pe.bias = nullptr;   // (a scaled accumulator keeps its bias in the epilogue)
+    }
+  }
+
+  // unit u = 2 kk + lg of the K row is vector (u % VPT) of tap (u / VPT) = (tr, tc), tr = tap / S
+  // through a multiplication (taps < 64, S <= 8: exact).  Taps outside the image and units
+  // past the last tap (their weights are zero) are read at a clamped position and replaced
+  // by the fill value before use: the requests themselves are unconditional.
+  const int units = p.R * p.S * VPT;
+  const unsigned s_inv = (65536u + (unsigned)p.S - 1u) / (unsigned)p.S;
+  const unsigned fill_w = (unsigned)(p.a_fill & 0xff) * 0x01010101u;
+  const uintx4 fillv = {fill_w, fill_w, fill_w, fill_w};
+  const uintx4* x16 = reinterpret_cast<const uintx4*>(p.x);
+  const int HoWo = p.Ho * p.Wo;
+
+  uintx4 a[NKK];
+  unsigned okmask = 0;   // bit kk: this lane's unit of K step kk is real data
+  auto load_a = [&](const int tile_m) {
+    int m = tile_m * BM + wm * 32 + l32;
+    m = m < M ? m : M - 1;
+    const int n_img = fast_div(m, p.howo_magic, p.howo_shift);
+    const int rem = m - n_img * HoWo;
+    const int ho = fast_div(rem, p.wo_magic, p.wo_shift);
+    const int wo = rem - ho * p.Wo;
+    const int hi0 = ho * p.sh - p.ph, wi0 = wo * p.sw - p.pw;
+    const int img = n_img * p.H;   // (the whole source has fewer than 2^31 16-byte units)
+    okmask = 0;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      const int u = 2 * kk + lg;
+      const int tap = u / VPT;
+      const int tr = (int)(((unsigned)tap * s_inv) >> 16), tc = tap - tr * p.S;
+      const int hi = hi0 + tr, wi = wi0 + tc;
+      const bool ok = u < units && (unsigned)hi < (unsigned)p.H && (unsigned)wi < (unsigned)p.W;
+      const int hc = hi < 0 ? 0 : (hi < p.H ? hi : p.H - 1), wc = wi < 0 ? 0 : (wi < p.W ? wi : p.W - 1);
+      a[kk] = x16[(unsigned)(((img + hc) * p.W + wc) * VPT + u % VPT)];
+      okmask |= ok ? 1u << kk : 0u;
+    }
+  };
+
+  load_a(tm0);
+  for (int tile_m = tm0; tile_m < tm1; ++tile_m) {
+    if (__builtin_amdgcn_ballot_w64(okmask != (1u << NKK) - 1u) != 0) {   // a border block
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) a[kk] = (okmask >> kk) & 1u ? a[kk] : fillv;
+    }
+    Acc acc[1][NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) acc[0][j] = Mma<TIn>::run(w[j][0], a[0], acc0[0][j]);
+#pragma unroll
+    for (int kk = 1; kk < NKK; ++kk)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) acc[0][j] = Mma<TIn>::run(w[j][kk], a[kk], acc[0][j]);
+    // the operand registers are free again: the next tile's pixels travel during the epilogue
+    if (tile_m + 1 < tm1) load_a(tile_m + 1);
+    igemm_epilogue<TIn, Epi, BM, BN, 32, WN, false, true>(pe, epi_vec, acc, smem, tile_m, tile_n, 0, M, wave, lane, 0);
+    // the same wavefront parks into its slice again next: order it behind the read-back
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
 // Rearranges packed weight rows ([batch][rows][row_bytes], zero padded) into
 // MFMA fragment order, followed by kWfragTailBytes of the fill byte: 16-byte unit ((b * tiles + t) * chunks + q) * 64 + lane
 // holds bytes [q*32 + (lane/32)*16, +16) of row t*32 + lane%32.
@@ -1030,6 +1170,55 @@ hipError_t launch_lean(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Filters over one or two 16-byte vectors of channels per tap, at most 64 (128)
+// output channels: the short-tap streaming variant.  Returns its K steps and
+// vectors per tap, or {0, 0}.
+struct TapsShape { int nkk, vpt; };
+TapsShape taps_shape(const IgemmParams& p) {
+  if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid
+    if (strcmp(force, "taps") != 0 && force[0] != 0) return {0, 0};
+  }
+  const int es = dtype_size(p.in_dt);
+  if (p.in_dt != DT_F16 && p.in_dt != DT_BF16 && p.in_dt != DT_I8) return {0, 0};
+  if (p.out_dt != p.in_dt || p.batch != 1 || p.dh != 1 || p.dw != 1 || p.C != p.xcs) return {0, 0};
+  if (p.y_rdiv > 0 || p.y_zdiv > 0) return {0, 0};
+  if (p.act != ACT_NONE && p.act != ACT_RELU && p.act != ACT_LEAKY && p.act != ACT_CLAMP) return {0, 0};
+  const int pix_bytes = p.xcs * es;
+  if (pix_bytes != 16 && pix_bytes != 32) return {0, 0};
+  const int vpt = pix_bytes / 16;
+  if (p.R * p.S < 2 || p.S > 8 || p.Kout > 128) return {0, 0};
+  const int nkk = (p.R * p.S * vpt + 1) / 2;
+  // the indices of the 16-byte units of the whole source fit 31 bits
+  if ((int64_t)p.N * p.H * p.W * vpt >= (1ll << 31)) return {0, 0};
+  // Built and selected where it was measured faster than the two-operand kernel: 16 taps of
+  // one 8-bit vector (the space-to-depth form of a 7x7 stride-2 stem; ResNet-50 at batch
+  // 256: 159 -> 122 us).  The 2-byte forms of the same layers request twice the bytes per
+  // pixel from the vector-memory pipeline, which then bounds them (215 -> 288 us), and stay
+  // on the two-operand kernel.
+  const bool built = vpt == 1 && nkk == 8 && es == 1;
+  return built ? TapsShape{nkk, vpt} : TapsShape{0, 0};
+}
+
+template <typename TIn, typename Epi>
+hipError_t launch_taps(const IgemmParams& p, int epi_vec, hipStream_t stream) {
+  const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+  const TapsShape ts = taps_shape(p);
+  if (ts.nkk != 8) return hipErrorInvalidValue;
+  const int64_t tiles_m = (M + 127) / 128, tiles_n = (p.Kout + 63) / 64;
+  // several pixel tiles per workgroup (the weights are fetched once for all of them),
+  // as long as the chip keeps eight workgroups per compute unit
+  int tpw = 1;
+  while (tpw < 16 && tiles_m * tiles_n / (tpw * 2) >= 2048) tpw *= 2;
+  if (const char* force = getenv("ODLA_HIP_LEAN_TILES")) {  // test aid: pixel tiles per workgroup
+    const int v = atoi(force);
+    if (v >= 1 && v <= 64) tpw = v;
+  }
+  const int64_t wgs = ((tiles_m + tpw - 1) / tpw) * tiles_n;
+  if (wgs <= 0 || wgs > 0x7fffffff) return hipErrorInvalidValue;
+  hipLaunchKernelGGL((igemm_taps_kernel<TIn, Epi, 8, 1, 2>), dim3((unsigned)wgs), dim3(256), 0, stream, p, epi_vec, tpw);
+  return hipGetLastError();
+}
+
 // The weights-in-registers kernel pays off once a layer has enough output
 // channels to give each of the four wavefronts its own 32-channel slice.
 bool wreg_shape(const IgemmParams& p) {
@@ -1050,13 +1239,17 @@ hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
   if constexpr (std::is_same<TIn, f16_t>::value || std::is_same<TIn, bf16_t>::value) {
     if (p.w_frag != nullptr && lean_steps(p) > 0) return launch_lean<TIn, Epi>(p, epi_vec, s);
   }
+  // (the short-tap kernel is built for 8-bit layers with 8-bit results)
+  if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
+    if (p.w_frag != nullptr && taps_shape(p).nkk > 0) return launch_taps<TIn, Epi>(p, epi_vec, s);
+  }
   if (p.w_frag != nullptr && wreg_shape(p)) return launch_wreg<TIn, Epi>(p, epi_vec, s);
   return dispatch_tiles<TIn, Epi>(p, epi_vec, s);
 }
 
 }  // namespace
 
-bool igemm_wants_wfrag(const IgemmParams& p) { return wreg_shape(p) || lean_steps(p) > 0; }
+bool igemm_wants_wfrag(const IgemmParams& p) { return wreg_shape(p) || lean_steps(p) > 0 || taps_shape(p).nkk > 0; }
 
 hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
   if (p.src == nullptr || p.dst == nullptr || p.rows <= 0 || p.row_bytes <= 0 || p.row_bytes % 16 != 0 ||
@@ -1076,6 +1269,7 @@ const char* igemm_variant_name(const IgemmParams& p) {
     default: break;
   }
   if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
+  if (p.w_frag != nullptr && taps_shape(p).nkk > 0) return "128x64t";
   if (p.w_frag != nullptr && wreg_shape(p)) return "128x128w";
   return choose_variant(p).name;
 }

@@ -374,7 +374,10 @@ __device__ __forceinline__ uintx4 q8_swz_chunk(const uintx4 v, const int row) {
 // the lane's four channels.
 // LDS per wavefront: two [32 pixels][WN + 16] byte tiles (result, residual; dwords
 // swizzled by q8_swz) and the WN multipliers of its channels.
-template <int BM, int BN, int WM, int WN, bool kEnterBarrier = true>
+// kMulReady: the caller has parked the wavefront's multipliers already (a kernel that
+// runs the epilogue for many pixel tiles of the same channels does that once, and
+// keeps a vector-memory wait out of every epilogue).
+template <int BM, int BN, int WM, int WN, bool kEnterBarrier = true, bool kMulReady = false>
 __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[WM / 32][WN / 32],
                                                   unsigned char* smem, const int tile_m, const int tile_n, const int z,
                                                   const int M, const int wave, const int lane, const int n_off = 0) {
@@ -420,7 +423,9 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
   if (has_res) rfetch(0);
   // the multipliers of the wavefront's channels, four per lane, parked in LDS below
   floatx4 mload = {0.f, 0.f, 0.f, 0.f};
-  if (lane < WN / 4) mload = load_qmul4(p.qmul, n0 + lane * 4, p.Kout);
+  if constexpr (!kMulReady) {
+    if (lane < WN / 4) mload = load_qmul4(p.qmul, n0 + lane * 4, p.Kout);
+  }
 
   auto wave_fence = [&]() {
     // each wavefront only touches its own tiles and its LDS operations complete in issue order
@@ -430,7 +435,9 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
   };
 
   if constexpr (kEnterBarrier) __syncthreads();  // the K loop's LDS traffic is done; the buffer becomes the staging area
-  if (lane < WN / 4) *reinterpret_cast<floatx4*>(mtile + lane * 4) = mload;
+  if constexpr (!kMulReady) {
+    if (lane < WN / 4) *reinterpret_cast<floatx4*>(mtile + lane * 4) = mload;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     if (has_res) {
@@ -481,14 +488,14 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
 // kEnterBarrier = false: the caller's wavefronts never shared `smem` before
 // (each only ever touches its own staging slice); n_off shifts the channels
 // this call covers within the tile.
-template <typename TIn, typename Epi, int BM, int BN, int WM, int WN, bool kEnterBarrier = true>
+template <typename TIn, typename Epi, int BM, int BN, int WM, int WN, bool kEnterBarrier = true, bool kMulReady = false>
 __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int epi_vec,
                                                typename Mma<TIn>::Acc (&acc)[WM / 32][WN / 32],
                                                unsigned char* smem, const int tile_m, const int tile_n,
                                                const int z, const int M, const int wave, const int lane,
                                                const int n_off = 0) {
   if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
-    igemm_epilogue_q8<BM, BN, WM, WN, kEnterBarrier>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane, n_off);
+    igemm_epilogue_q8<BM, BN, WM, WN, kEnterBarrier, kMulReady>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane, n_off);
     return;
   }
   constexpr int TM = WM / 32, TN = WN / 32;
