@@ -123,7 +123,10 @@ __global__ void __launch_bounds__(kThreads) pool2d_scalar_kernel(PoolParams p) {
 
 // 8-bit levels stored as q-128.  Max keeps levels; average requantises:
 // q = clamp(rne(((sum - cnt*zp_in) / cnt) * q_mul) + zp_out, 0, 255).
-template <bool IS_MAX>
+// KH, KW > 0 (maximum only): a window of that size with all its loads in flight at once.
+// A tap outside the image is read at the nearest position inside, which belongs to the
+// same window (every window overlaps the image), so the maximum is unchanged.
+template <bool IS_MAX, int KH = 0, int KW = 0>
 __global__ void __launch_bounds__(kThreads) pool2d_q8_kernel(PoolParams p) {
   const int cv = p.C / 16;
   const int8_t* x = reinterpret_cast<const int8_t*>(p.x);
@@ -138,32 +141,53 @@ __global__ void __launch_bounds__(kThreads) pool2d_q8_kernel(PoolParams p) {
   for (int n = blockIdx.y; n < p.N; n += gridDim.y) {
     const int h0 = ho * p.sh - p.ph, w0 = wo * p.sw - p.pw;
     if constexpr (IS_MAX) {
-      // Levels as unsigned bytes (stored ^ 0x80); even and odd bytes of a dword are two
-      // 16-bit lanes each, so one packed 16-bit maximum handles two levels.
-      typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
-      unsigned ev[4] = {0u, 0u, 0u, 0u}, od[4] = {0u, 0u, 0u, 0u};
-      for (int r = 0; r < p.kh; ++r) {
-        const int hi = h0 + r;
-        if ((unsigned)hi >= (unsigned)p.H) continue;
-        for (int s = 0; s < p.kw; ++s) {
-          const int wi = w0 + s;
-          if ((unsigned)wi >= (unsigned)p.W) continue;
-          const uintx4 v = *reinterpret_cast<const uintx4*>(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c);
-          const unsigned w[4] = {v.x ^ 0x80808080u, v.y ^ 0x80808080u, v.z ^ 0x80808080u, v.w ^ 0x80808080u};
+      // Stored bytes are signed (level - 128) and keep their order as the high byte of a signed
+      // 16-bit lane: the even bytes of a dword move there with one byte permute, the odd ones
+      // with one mask, and one packed 16-bit maximum handles two of them.
+      typedef short shortx2 __attribute__((ext_vector_type(2)));
+      unsigned ev[4] = {0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+      unsigned od[4] = {0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+      auto take = [&](const uintx4 v) {
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const ushortx2 a0 = __builtin_bit_cast(ushortx2, ev[k]), b0 = __builtin_bit_cast(ushortx2, w[k] & 0x00ff00ffu);
-            const ushortx2 a1 = __builtin_bit_cast(ushortx2, od[k]), b1 = __builtin_bit_cast(ushortx2, (w[k] >> 8) & 0x00ff00ffu);
-            ev[k] = __builtin_bit_cast(unsigned, __builtin_elementwise_max(a0, b0));
-            od[k] = __builtin_bit_cast(unsigned, __builtin_elementwise_max(a1, b1));
+        for (int k = 0; k < 4; ++k) {
+          const shortx2 a0 = __builtin_bit_cast(shortx2, ev[k]);
+          const shortx2 b0 = __builtin_bit_cast(shortx2, __builtin_amdgcn_perm(0u, w[k], 0x020c000cu));   // [b2, 0, b0, 0]
+          const shortx2 a1 = __builtin_bit_cast(shortx2, od[k]), b1 = __builtin_bit_cast(shortx2, w[k] & 0xff00ff00u);
+          ev[k] = __builtin_bit_cast(unsigned, __builtin_elementwise_max(a0, b0));
+          od[k] = __builtin_bit_cast(unsigned, __builtin_elementwise_max(a1, b1));
+        }
+      };
+      if constexpr (KH > 0) {
+        uintx4 v[KH * KW];
+#pragma unroll
+        for (int r = 0; r < KH; ++r) {
+          const int hi = h0 + r, hc = hi < 0 ? 0 : (hi < p.H ? hi : p.H - 1);
+#pragma unroll
+          for (int s = 0; s < KW; ++s) {
+            const int wi = w0 + s, wc = wi < 0 ? 0 : (wi < p.W ? wi : p.W - 1);
+            // (read by at most a few neighbouring windows, all of them close in time)
+            v[r * KW + s] = *reinterpret_cast<const uintx4*>(x + (((int64_t)n * p.H + hc) * p.W + wc) * p.cs + c);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < KH * KW; ++t) take(v[t]);
+      } else {
+        for (int r = 0; r < p.kh; ++r) {
+          const int hi = h0 + r;
+          if ((unsigned)hi >= (unsigned)p.H) continue;
+          for (int s = 0; s < p.kw; ++s) {
+            const int wi = w0 + s;
+            if ((unsigned)wi >= (unsigned)p.W) continue;
+            take(*reinterpret_cast<const uintx4*>(x + (((int64_t)n * p.H + hi) * p.W + wi) * p.cs + c));
           }
         }
       }
       uintx4 o;
-      o.x = (ev[0] | (od[0] << 8)) ^ 0x80808080u;
-      o.y = (ev[1] | (od[1] << 8)) ^ 0x80808080u;
-      o.z = (ev[2] | (od[2] << 8)) ^ 0x80808080u;
-      o.w = (ev[3] | (od[3] << 8)) ^ 0x80808080u;
+      o.x = (ev[0] >> 8) | od[0];   // (the low byte of every lane stayed 0)
+      o.y = (ev[1] >> 8) | od[1];
+      o.z = (ev[2] >> 8) | od[2];
+      o.w = (ev[3] >> 8) | od[3];
       // (a window without a valid tap cannot occur: the planner derives Ho, Wo from the padding)
       *reinterpret_cast<uintx4*>(y + (((int64_t)n * p.Ho + ho) * p.Wo + wo) * p.ycs + c) = o;
     } else {
@@ -813,7 +837,12 @@ hipError_t launch_pool2d(const PoolParams& p_in, hipStream_t stream) {
     div_magic(cv, &p.cv_magic, &p.cv_shift);
     const dim3 grid((unsigned)((per_image + kThreads - 1) / kThreads), (unsigned)(p.N < 65535 ? p.N : 65535));
     if (p.dt == DT_I8) {
-      if (p.is_max) hipLaunchKernelGGL(pool2d_q8_kernel<true>, grid, dim3(kThreads), 0, stream, p);
+      // (the clamped taps of the unrolled windows need every window to overlap the image)
+      const bool overlap = p.ph < p.kh && p.pw < p.kw && (int64_t)(p.Ho - 1) * p.sh - p.ph < p.H &&
+                           (int64_t)(p.Wo - 1) * p.sw - p.pw < p.W;
+      if (p.is_max && p.kh == 3 && p.kw == 3 && overlap) hipLaunchKernelGGL((pool2d_q8_kernel<true, 3, 3>), grid, dim3(kThreads), 0, stream, p);
+      else if (p.is_max && p.kh == 2 && p.kw == 2 && overlap) hipLaunchKernelGGL((pool2d_q8_kernel<true, 2, 2>), grid, dim3(kThreads), 0, stream, p);
+      else if (p.is_max) hipLaunchKernelGGL(pool2d_q8_kernel<true>, grid, dim3(kThreads), 0, stream, p);
       else hipLaunchKernelGGL(pool2d_q8_kernel<false>, grid, dim3(kThreads), 0, stream, p);
       return hipGetLastError();
     }
