@@ -1170,9 +1170,8 @@ hipError_t launch_lean(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// Filters over one or two 16-byte vectors of channels per tap, at most 64 (128)
-// output channels: the short-tap streaming variant.  Returns its K steps and
-// vectors per tap, or {0, 0}.
+// The layers that run on the short-tap streaming variant.  Returns its K steps
+// and vectors per tap, or {0, 0}.
 struct TapsShape { int nkk, vpt; };
 TapsShape taps_shape(const IgemmParams& p) {
   if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid
@@ -1184,6 +1183,11 @@ TapsShape taps_shape(const IgemmParams& p) {
   if (p.y_rdiv > 0 || p.y_zdiv > 0) return {0, 0};
   if (p.act != ACT_NONE && p.act != ACT_RELU && p.act != ACT_LEAKY && p.act != ACT_CLAMP) return {0, 0};
   const int pix_bytes = p.xcs * es;
+  // (8-bit 1x1 filters over 64 channels into at most 64: one "tap" of four vectors; ResNet-50's
+  // first bottleneck at batch 256: 35 -> 27 us.  With more output channels, or longer pixel
+  // rows, the same layers were measured slower here than on the other kernels.)
+  if (es == 1 && p.R * p.S == 1 && pix_bytes == 64 && p.Kout <= 64 && (int64_t)p.N * p.H * p.W * 4 < (1ll << 31))
+    return {2, 4};
   if (pix_bytes != 16 && pix_bytes != 32) return {0, 0};
   const int vpt = pix_bytes / 16;
   if (p.R * p.S < 2 || p.S > 8 || p.Kout > 128) return {0, 0};
@@ -1203,7 +1207,6 @@ template <typename TIn, typename Epi>
 hipError_t launch_taps(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
   const TapsShape ts = taps_shape(p);
-  if (ts.nkk != 8) return hipErrorInvalidValue;
   const int64_t tiles_m = (M + 127) / 128, tiles_n = (p.Kout + 63) / 64;
   // several pixel tiles per workgroup (the weights are fetched once for all of them),
   // as long as the chip keeps eight workgroups per compute unit
@@ -1215,7 +1218,9 @@ hipError_t launch_taps(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   }
   const int64_t wgs = ((tiles_m + tpw - 1) / tpw) * tiles_n;
   if (wgs <= 0 || wgs > 0x7fffffff) return hipErrorInvalidValue;
-  hipLaunchKernelGGL((igemm_taps_kernel<TIn, Epi, 8, 1, 2>), dim3((unsigned)wgs), dim3(256), 0, stream, p, epi_vec, tpw);
+  const dim3 grid((unsigned)wgs), block(256);
+  if (ts.vpt == 1) hipLaunchKernelGGL((igemm_taps_kernel<TIn, Epi, 8, 1, 2>), grid, block, 0, stream, p, epi_vec, tpw);
+  else hipLaunchKernelGGL((igemm_taps_kernel<TIn, Epi, 2, 4, 2>), grid, block, 0, stream, p, epi_vec, tpw);
   return hipGetLastError();
 }
 
