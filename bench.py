@@ -44,8 +44,8 @@ METRIC = "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW
 MEASURED_TRAFFIC = {
     # 8.81 GB fetched + 5.76 GB written per step over its 54 conv/gemm launches
     "resnet50_fp16": 269.8e6,
-    # 4.17 GB fetched + 2.99 GB written per step over its 54 conv/gemm launches
-    "resnet50_int8": 132.6e6,
+    # 4.17 GB fetched + 2.97 GB written per step over its 54 conv/gemm launches
+    "resnet50_int8": 132.1e6,
 }
 
 
@@ -350,7 +350,7 @@ def profile_roofline(L, sess, wl, dump_path=None):
     roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
             "unit": "TOP/s" if wl.mode == "int8" else "TFLOP/s",
             "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(wl.name),
-            "kernel": "igemm_wreg_kernel / igemm_kernel / igemm_lean_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
+            "kernel": "igemm_wreg_kernel / igemm_kernel / igemm_lean_kernel / igemm_taps_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
                       "avg %.2f GFLOP per launch)" % (launches, 1e3 * mm_ms / max(launches, 1),
                                                      wl.flop / 1e9 / max(launches, 1)),
             "mm_ms_per_step": round(mm_ms, 4), "all_kernels_ms_per_step": round(total_ms, 4),
