@@ -37,9 +37,12 @@ namespace ohip {
 // covers the 32 x 128 tile with full 128-byte rows.  The residual tile takes the
 // same road in the other direction.  Two tile pairs alternate, so that a slice
 // needs one barrier between its phases and one before its tiles are reused.
+// mtile: the tile's 128 multipliers in LDS (parked there by the caller ahead of its K
+// loop: the epilogue then starts without a round trip to memory), or nullptr.
 __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[4][1],
                                                           unsigned char* smem, const int tile_m, const int tile_n,
-                                                          const int z, const int M, const int wave, const int lane) {
+                                                          const int z, const int M, const int wave, const int lane,
+                                                          const float* mtile = nullptr) {
   constexpr int BM = 128, BN = 128, TM = 4;
   constexpr int PITCH = BN + 16;  // bytes per staged pixel row
   constexpr int TILE = 32 * PITCH;
@@ -59,7 +62,9 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
 
   floatx4 mq[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) mq[q] = load_qmul4(p.qmul, n0 + wave * 32 + q * 8 + lg * 4, p.Kout);
+  for (int q = 0; q < 4; ++q)
+    mq[q] = mtile != nullptr ? *reinterpret_cast<const floatx4*>(mtile + wave * 32 + q * 8 + lg * 4)
+                             : load_qmul4(p.qmul, n0 + wave * 32 + q * 8 + lg * 4, p.Kout);
 
   // The residual rows of all four slices are requested ahead of the first barrier:
   // one memory round trip per tile.
@@ -136,9 +141,9 @@ template <typename TIn, typename Epi>
 __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, const int epi_vec,
                                                        typename Mma<TIn>::Acc (&acc)[4][1], unsigned char* smem,
                                                        const int tile_m, const int tile_n, const int z, const int M,
-                                                       const int wave, const int lane) {
+                                                       const int wave, const int lane, const float* mtile = nullptr) {
   if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
-    igemm_epilogue_rows128_q8(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane);
+    igemm_epilogue_rows128_q8(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane, mtile);
     return;
   }
   constexpr int BM = 128, BN = 128, TM = 4;
@@ -523,7 +528,9 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   // vmcnt(0), and vmcnt(2 * NWF + 4) = 12 / 20 for the wait at the top of a stage
   constexpr int kWaitVm0 = 0x0f70, kWaitVmStage = NJ == 1 ? 0x0f7c : 0x4f74;
 
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[NBUF * BUF_BYTES];
+  // (8-bit results: the multipliers of the tile's channels wait behind the pixel ring)
+  constexpr bool kMulLds = std::is_same<Epi, EpiQuant<0>>::value;
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[NBUF * BUF_BYTES + (kMulLds ? NJ * 512 : 0)];
 
   const int tid = threadIdx.x;
   const int M = p.N * p.Ho * p.Wo;
@@ -693,6 +700,19 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) acc_init_bias_vec<TM, 1>(p, z, (tile_n * NJ + j) * 128 + wave_u * 32, lg, acc[j]);
   }
+  if constexpr (kMulLds) {
+    // The multipliers of this wavefront's channels, into LDS behind the ring (requested
+    // and consumed here, like the bias; read back by the same wavefront in the epilogue,
+    // which then begins without a round trip to memory).
+    float* mt = reinterpret_cast<float*>(smem + NBUF * BUF_BYTES);
+    const int last = p.Kout - 1;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int c = (tile_n * NJ + j) * 128 + wave_u * 32 + l32;
+      const float v = p.qmul[c < last ? c : last];
+      if (lg == 0) mt[j * 128 + wave_u * 32 + l32] = v;
+    }
+  }
 
   // fragment read offsets: row l32 (+32*i), chunk 2*kk + lg, swizzled
   const int sw = (l32 >> 1) & 7;
@@ -786,7 +806,8 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
 #undef IGEMM_WDRAIN8
 #pragma unroll
   for (int j = 0; j < NJ; ++j)
-    igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc[j], smem, tile_m, tile_n * NJ + j, z, M, wave, lane);
+    igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc[j], smem, tile_m, tile_n * NJ + j, z, M, wave, lane,
+                                     kMulLds ? reinterpret_cast<const float*>(smem + NBUF * BUF_BYTES) + j * 128 : nullptr);
 }
 
 // ---------------------------------------------------------------------------
