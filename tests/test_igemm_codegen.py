@@ -8,7 +8,11 @@ speed rely on and that a compiler change could silently break:
     flight: each fragment keeps one register quad, and between the pipeline
     fill and the wait that follows the K loop only the MFMAs and those requests
     themselves may name these registers, on any path (a compiler-inserted copy
-    or reuse there would read or clobber data that has not landed yet).
+    or reuse there would read or clobber data that has not landed yet);
+  * those requests take their address from a scalar register pair, which a
+    vector-memory instruction must not read within five wait states of a VECTOR
+    instruction writing it (v_readfirstlane, v_cmp); the compiler does not look
+    into the inline assembly for that, so the distance is checked here.
 """
 import os
 import re
@@ -62,7 +66,8 @@ def kernel_bodies(asm, prefix):
 
 def test_weight_fragment_registers_untouched_in_flight(compiled):
     asm, _ = compiled
-    req = re.compile(r"global_load_dwordx4 v\[(\d+):(\d+)\], v\[\d+:\d+\], off offset:(0|1024|2048|3072)$")
+    # (the lane's 32-bit offset in a vector register, the fragment's wavefront-uniform address in scalar ones)
+    req = re.compile(r"global_load_dwordx4 v\[(\d+):(\d+)\], (?:v\d+, s\[\d+:\d+\]|v\[\d+:\d+\], off) offset:(0|1024|2048|3072)$")
     checked = 0
     for name, body in kernel_bodies(asm, "_ZN4ohip17igemm_wreg_kernel"):
         quads = {(int(m.group(1)), int(m.group(2))) for m in map(req.match, body) if m}
@@ -100,3 +105,25 @@ def test_weight_fragment_registers_untouched_in_flight(compiled):
             assert not hit, (name, i, l)
         checked += 1
     assert checked >= 12
+
+
+def test_scalar_addresses_of_fragment_requests_are_settled(compiled):
+    asm, _ = compiled
+    req = re.compile(r"global_load_dwordx4 v\[\d+:\d+\], v\d+, s\[(\d+):(\d+)\]")
+    vwrite = re.compile(r"(v_readfirstlane_b32|v_readlane_b32|v_cmp\w*)\s+s\[?(\d+)(?::(\d+))?")
+    loads = 0
+    for name, body in kernel_bodies(asm, "_ZN4ohip17igemm_wreg_kernel"):
+        real = [l for l in body if not l.startswith(".LBB")]
+        for i, l in enumerate(real):
+            m = req.match(l)
+            if not m:
+                continue
+            loads += 1
+            lo, hi = int(m.group(1)), int(m.group(2))
+            for back in real[max(0, i - 8):i]:
+                w = vwrite.match(back)
+                if w:
+                    a = int(w.group(2))
+                    b = int(w.group(3)) if w.group(3) else a
+                    assert b < lo or a > hi, (name, back, l)
+    assert loads >= 200
