@@ -42,10 +42,10 @@ METRIC = "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW
 # summaries the figures come from are the traffic_* files under profiles/.
 # null = not measured.
 MEASURED_TRAFFIC = {
-    # 8.81 GB fetched + 5.76 GB written per step over its 54 conv/gemm launches
-    "resnet50_fp16": 269.8e6,
-    # 4.17 GB fetched + 2.97 GB written per step over its 54 conv/gemm launches
-    "resnet50_int8": 132.1e6,
+    # 8.79 GB fetched + 5.76 GB written per step over its 54 conv/gemm launches
+    "resnet50_fp16": 269.4e6,
+    # 4.16 GB fetched + 2.97 GB written per step over its 54 conv/gemm launches
+    "resnet50_int8": 132.0e6,
 }
 
 
