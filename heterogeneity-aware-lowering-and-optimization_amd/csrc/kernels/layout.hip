@@ -213,6 +213,84 @@ __global__ void __launch_bounds__(kThreads) strided_tile_copy_kernel(TileCopyPar
   }
 }
 
+// The same for 2-byte elements, moving eight of them per request on the side(s) whose
+// strides and base keep 16-byte alignment (VL: the source runs, VS: the destination runs);
+// the other side moves single elements as above.  Tile [b][a], 66 elements per row.
+template <bool VL, bool VS>
+__global__ void __launch_bounds__(kThreads) strided_tile_copy16_kernel(TileCopyParams p, int64_t ntiles) {
+  constexpr int TS = 64, PITCH = 66;
+  __shared__ __attribute__((aligned(16))) uint16_t tile[TS * PITCH];
+  const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x) + p.x_off;
+  uint16_t* y = reinterpret_cast<uint16_t*>(p.y) + p.y_off;
+  const int ta_n = (p.Da + TS - 1) / TS, tb_n = (p.Db + TS - 1) / TS;
+  const int tid = threadIdx.x;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int a0 = (int)(t % ta_n) * TS;
+    const int b0 = (int)((t / ta_n) % tb_n) * TS;
+    int64_t o = t / ((int64_t)ta_n * tb_n), ox = 0, oy = 0;
+    for (int d = p.n_outer - 1; d >= 0; --d) {
+      const int64_t q = o / p.odims[d], idx = o - q * p.odims[d];
+      o = q;
+      ox += idx * p.osx[d];
+      oy += idx * p.osy[d];
+    }
+    if constexpr (VL) {
+      const int v = tid & 7;
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+        const int bb = (tid >> 3) + pass * 32;
+        const int a = a0 + v * 8, b = b0 + bb;
+        if (b < p.Db && a < p.Da) {
+          const uint16_t* src = x + ox + (int64_t)b * p.sxb + a;
+          uint16_t* dst = tile + bb * PITCH + v * 8;
+          if (a + 8 <= p.Da) {
+            const uintx4 q = *reinterpret_cast<const uintx4*>(src);
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);   // (PITCH and 8 v are even)
+            d32[0] = q.x; d32[1] = q.y; d32[2] = q.z; d32[3] = q.w;
+          } else {
+            for (int e = 0; a + e < p.Da; ++e) dst[e] = src[e];
+          }
+        }
+      }
+    } else {
+      const int tx = tid % TS, ty = tid / TS;
+      for (int rr = ty; rr < TS; rr += kThreads / TS) {
+        const int b = b0 + rr, a = a0 + tx;
+        if (b < p.Db && a < p.Da) tile[rr * PITCH + tx] = x[ox + (int64_t)b * p.sxb + a];
+      }
+    }
+    __syncthreads();
+    if constexpr (VS) {
+      const int v = tid & 7;
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass) {
+        const int aa = (tid >> 3) + pass * 32;
+        const int a = a0 + aa, b = b0 + v * 8;
+        if (a < p.Da && b < p.Db) {
+          uint16_t* dst = y + oy + (int64_t)a * p.sya + b;
+          const uint16_t* src = tile + (v * 8) * PITCH + aa;
+          if (b + 8 <= p.Db) {
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              w[e] = (uint32_t)src[(2 * e) * PITCH] | ((uint32_t)src[(2 * e + 1) * PITCH] << 16);
+            *reinterpret_cast<uintx4*>(dst) = uintx4{w[0], w[1], w[2], w[3]};
+          } else {
+            for (int e = 0; b + e < p.Db; ++e) dst[e] = src[e * PITCH];
+          }
+        }
+      }
+    } else {
+      const int tx = tid % TS, ty = tid / TS;
+      for (int cc = ty; cc < TS; cc += kThreads / TS) {
+        const int a = a0 + cc, b = b0 + tx;
+        if (a < p.Da && b < p.Db) y[oy + (int64_t)a * p.sya + b] = tile[tx * PITCH + cc];
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // Batched 2-D transpose through an LDS tile: y[b][c][r] = x[b][r][c]; the
 // destination row pitch may exceed `rows` (zero padding is the caller's job).
 template <typename E>
@@ -517,6 +595,19 @@ hipError_t launch_strided_copy(const StridedCopyParams& p_in, hipStream_t stream
     for (int d = tp.n_outer; d < 6; ++d) { tp.odims[d] = 1; tp.osx[d] = tp.osy[d] = 0; }
     const int64_t ntiles = outer * ((tp.Da + 63) / 64) * ((tp.Db + 63) / 64);
     const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
+    if (p.elem_size == 2) {
+      // eight elements per request on the sides that stay 16-byte aligned
+      bool vl = tp.sxb % 8 == 0 && tp.x_off % 8 == 0 && (reinterpret_cast<uintptr_t>(tp.x) & 15u) == 0;
+      bool vs = tp.sya % 8 == 0 && tp.y_off % 8 == 0 && (reinterpret_cast<uintptr_t>(tp.y) & 15u) == 0;
+      for (int d = 0; d < tp.n_outer; ++d) {
+        vl = vl && tp.osx[d] % 8 == 0;
+        vs = vs && tp.osy[d] % 8 == 0;
+      }
+      if (vl && vs) hipLaunchKernelGGL((strided_tile_copy16_kernel<true, true>), dim3(grid), dim3(kThreads), 0, stream, tp, ntiles);
+      else if (vl) hipLaunchKernelGGL((strided_tile_copy16_kernel<true, false>), dim3(grid), dim3(kThreads), 0, stream, tp, ntiles);
+      else if (vs) hipLaunchKernelGGL((strided_tile_copy16_kernel<false, true>), dim3(grid), dim3(kThreads), 0, stream, tp, ntiles);
+      if (vl || vs) return hipGetLastError();
+    }
     switch (p.elem_size) {
       case 1: hipLaunchKernelGGL(strided_tile_copy_kernel<uint8_t>, dim3(grid), dim3(kThreads), 0, stream, tp, ntiles); break;
       case 2: hipLaunchKernelGGL(strided_tile_copy_kernel<uint16_t>, dim3(grid), dim3(kThreads), 0, stream, tp, ntiles); break;
@@ -547,6 +638,14 @@ hipError_t launch_strided_copy(const StridedCopyParams& p_in, hipStream_t stream
 hipError_t launch_transpose2d(const void* x, void* y, int elem_size, int batch, int rows, int cols,
                               int dst_pitch, hipStream_t stream) {
   if (!x || !y || batch <= 0 || rows <= 0 || cols <= 0 || dst_pitch < rows) return hipErrorInvalidValue;
+  if (elem_size == 2 && rows >= 16 && cols >= 16) {   // (the tiled strided copy has vector requests for this size)
+    StridedCopyParams cp;
+    cp.x = x; cp.y = y; cp.elem_size = 2; cp.rank = 3;
+    cp.dims[0] = batch; cp.dims[1] = cols; cp.dims[2] = rows;
+    cp.sy[0] = (int64_t)cols * dst_pitch; cp.sy[1] = dst_pitch; cp.sy[2] = 1;
+    cp.sx[0] = (int64_t)rows * cols; cp.sx[1] = 1; cp.sx[2] = cols;
+    return launch_strided_copy(cp, stream);
+  }
   const int64_t ntiles = (int64_t)batch * ((rows + 63) / 64) * ((cols + 63) / 64);
   const int grid = (int)(ntiles < 65536 ? ntiles : 65536);
   switch (elem_size) {

@@ -749,17 +749,27 @@ def test_transpose_paths_parity(shape, perm, dtype):
     assert np.array_equal(got["t"], np.transpose(x, perm))
 
 
-def test_transpose_fp16_storage_tiles():
-    """2-byte elements through the tiled route (fp16 storage of an fp32 graph)."""
-    announce("transpose fp16 tiles")
-    x = rng(66).standard_normal((4, 100, 72)).astype(np.float32)
+@pytest.mark.parametrize("shape,perm", [
+    ((4, 100, 72), (0, 2, 1)),        # source rows keep 16-byte alignment, destination rows do not
+    ((3, 64, 80), (0, 2, 1)),         # both sides aligned: eight elements per request each way
+    ((2, 48, 37), (0, 2, 1)),         # only the destination aligned
+    ((2, 50, 37), (0, 2, 1)),         # neither: single elements
+    ((2, 200, 136), (0, 2, 1)),       # several tiles each way, the last ones partly filled
+    ((2, 3, 85, 13, 16), (0, 1, 3, 4, 2)),   # detection head
+    ((2, 16, 3, 72), (3, 1, 2, 0)),   # outer dims on both sides of the tile plane
+])
+def test_transpose_fp16_storage_tiles(shape, perm):
+    """2-byte elements through the tiled route (fp16 storage of an fp32 graph), with and
+    without 16-byte requests on either side."""
+    announce("transpose fp16 tiles %s %s" % (shape, perm))
+    x = rng(66).standard_normal(shape).astype(np.float32)
 
     def build(b):
         a = b.arg("x", x.shape)
-        b.output(b.transpose(a, (0, 2, 1), name="t"), "t")
+        b.output(b.transpose(a, perm, name="t"), "t")
 
     got = run_hip(build, {"x": x}, fp16=True)
-    assert np.array_equal(got["t"], np.transpose(x.astype(np.float16).astype(np.float32), (0, 2, 1)))
+    assert np.array_equal(got["t"], np.transpose(x.astype(np.float16).astype(np.float32), perm))
 
 
 def test_nhwc_chain_then_concat_resize():
