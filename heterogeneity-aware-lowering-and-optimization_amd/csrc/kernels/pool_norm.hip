@@ -628,7 +628,9 @@ softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
     for (int k = 0; k < PER; ++k)
 #pragma unroll
       for (int e = 0; e < V; ++e) {
-        const float ex = expf(v[k][e] - mx);   // exp(-inf) = 0 for the padding slots
+        // exp(-inf) = 0 for the padding slots.  A 16-bit result keeps 8 or 11 significant bits:
+        // the hardware exponential (1 ulp) stands in for the library's.
+        const float ex = sizeof(TO) == 2 ? __expf(v[k][e] - mx) : expf(v[k][e] - mx);
         sum += ex;
         if (!logsm) v[k][e] = ex;
       }
