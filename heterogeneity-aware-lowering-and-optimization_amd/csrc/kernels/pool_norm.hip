@@ -1016,6 +1016,9 @@ hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int
   SM_CASE(DT_BF16, DT_BF16, bf16_t, bf16_t)
   SM_CASE(DT_F16, DT_F32, f16_t, float)
   SM_CASE(DT_BF16, DT_F32, bf16_t, float)
+  // fp32 scores, probabilities in the operand type of the matrix product that reads them
+  SM_CASE(DT_F32, DT_BF16, float, bf16_t)
+  SM_CASE(DT_F32, DT_F16, float, f16_t)
 #undef SM_CASE
   return hipErrorInvalidValue;
 }

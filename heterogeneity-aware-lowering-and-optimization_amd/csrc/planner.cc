@@ -69,10 +69,12 @@ struct PlanError {
   throw PlanError{st, buf};
 }
 
-enum Form { FORM_FLOAT = 0, FORM_QUANT = 1 };
+// FORM_OPERAND: the 16-bit copy a Conv / Gemm reads under BF16_ACCURACY_MODE, where values
+// are stored as fp32; in every other mode it is the same thing as FORM_FLOAT.
+enum Form { FORM_FLOAT = 0, FORM_QUANT = 1, FORM_OPERAND = 2 };
 
 struct VState {
-  int slot[2][2] = {{-1, -1}, {-1, -1}};  // [layout][form] -> tensor id
+  int slot[2][3] = {{-1, -1, -1}, {-1, -1, -1}};  // [layout][form] -> tensor id
   int main = -1;
 };
 
@@ -101,7 +103,12 @@ class Planner {
   std::vector<VState> vs_;
   std::vector<std::vector<int>> consumers_;  // value index -> node indices
   std::unordered_map<std::string, QuantEntry> qmap_;
-  DType cdt_ = DT_F32;
+  DType cdt_ = DT_F32;     // storage type of FLOAT32 graph values
+  DType op_dt_ = DT_F32;   // type in which Conv / Gemm read their operands
+  // BF16_ACCURACY_MODE [ref: ODLA/include/ODLA/odla_compute.h:72-78; odla_dnnl.cc:1024-1026,
+  // 1780-1802]: values stay fp32, only the operands of Conv / Gemm are rounded to bf16.
+  bool acc_mode_ = false;
+  std::vector<signed char> operand_only_;   // per value, memo of operand_only(): -1 unknown
   bool in_init_ = false;
 
   // ---------------------------------------------------------------- tensors
@@ -246,6 +253,49 @@ class Planner {
     if (d == DT_F32) return cdt_;
     return d;
   }
+  // Type of the tensor a Conv / Gemm reads for a FLOAT32 operand.
+  DType mm_dtype(const _odla_value* v) const {
+    const DType d = dtype_from_odla(v->etype);
+    return d == DT_F32 ? op_dt_ : d;
+  }
+  // Every reader of `v` is a Conv / Gemm operand slot (through Reshape / Transpose, which move
+  // bits): storing it in the operand type loses nothing that the readers would keep.
+  bool operand_only(const _odla_value* v) {
+    if (v == nullptr || v->is_output || consumers_[v->index].empty()) return false;
+    signed char& memo = operand_only_[v->index];
+    if (memo >= 0) return memo != 0;
+    bool all = true;
+    for (int ci : consumers_[v->index]) {
+      const Node& c = comp_->nodes[ci];
+      if (c.op == OP_GEMM || c.op == OP_CONV) {
+        const bool as_operand = c.in[0] == v || c.in[1] == v;
+        const bool as_addend = c.in.size() > 2 && c.in[2] == v;
+        all = all && as_operand && !as_addend;
+      } else if (c.op == OP_RESHAPE || c.op == OP_TRANSPOSE) {
+        all = all && operand_only(c.out);
+      } else {
+        all = false;
+      }
+      if (!all) break;
+    }
+    operand_only_[v->index] = all ? 1 : 0;
+    return all;
+  }
+  // Storage type of what a Conv / Gemm / Softmax launch writes for the FLOAT32 value `v`.
+  DType result_dtype(const _odla_value* v) {
+    const DType d = dtype_from_odla(v->etype);
+    if (d != DT_F32) return d;
+    if (acc_mode_) return operand_only(v) ? op_dt_ : DT_F32;
+    return cdt_;
+  }
+  // `v` in the given layout as some float tensor, preferring what exists: data movement
+  // (Reshape, Transpose, Slice, Concat) keeps whatever type its source is stored in.
+  int get_moved(const _odla_value* v, Layout want) {
+    const VState& s = vs_[v->index];
+    const bool narrow = acc_mode_ && dtype_from_odla(v->etype) == DT_F32 && s.main >= 0 && !T(s.main).quant &&
+                        T(s.main).dt == op_dt_ && s.slot[want][FORM_FLOAT] < 0;
+    return get(v, want, narrow ? FORM_OPERAND : FORM_FLOAT);
+  }
   const QuantEntry* qentry(const _odla_value* v) const {
     if (!comp_->opts.int8 || v == nullptr || v->name.empty()) return nullptr;
     if (dtype_from_odla(v->etype) != DT_F32) return nullptr;
@@ -258,6 +308,7 @@ class Planner {
   // (and caching) a conversion step when the value lives in another one.
   // `cvec` > 0 asks for a channels-last pitch that is a multiple of cvec.
   int get(const _odla_value* v, Layout want, Form form = FORM_FLOAT, int cvec = 0) {
+    if (form == FORM_OPERAND && (!acc_mode_ || dtype_from_odla(v->etype) != DT_F32)) form = FORM_FLOAT;
     VState& s = vs_[v->index];
     if (s.main < 0) materialize_source(v);
     if (want == L_NHWC && v->shape.rank != 4) fail(ODLA_INTERNAL_LOGIC_ERR, "channels-last form requested for rank-%d value", v->shape.rank);
@@ -273,7 +324,8 @@ class Planner {
     // prefer same form, then same layout, then main
     if (s.slot[want][form] >= 0) return s.slot[want][form];
     if (s.slot[1 - want][form] >= 0) return s.slot[1 - want][form];
-    if (s.slot[want][1 - form] >= 0) return s.slot[want][1 - form];
+    for (int f = 0; f < 3; ++f)
+      if (f != form && s.slot[want][f] >= 0) return s.slot[want][f];
     return s.main;
   }
 
@@ -281,20 +333,22 @@ class Planner {
     VState& s = vs_[v->index];
     s.main = t;
     const PTensor p = T(t);  // by value: the tensor table may grow below
-    s.slot[p.layout][p.quant ? FORM_QUANT : FORM_FLOAT] = t;
+    const int form = p.quant ? FORM_QUANT
+                             : (acc_mode_ && p.dt == op_dt_ && dtype_from_odla(v->etype) == DT_F32 ? FORM_OPERAND : FORM_FLOAT);
+    s.slot[p.layout][form] = t;
     // a channels-last tensor with one pixel (or one channel) and no padding is
     // also a valid row-major tensor, and vice versa
     if (p.shape.rank == 4) {
       const bool trivial = (p.shape.d[2] * p.shape.d[3] == 1) || (p.shape.d[1] == 1);
       if (trivial && (p.layout == L_ROWMAJOR || p.cs == p.shape.d[1])) {
         const int other = 1 - (int)p.layout;
-        if (s.slot[other][p.quant ? FORM_QUANT : FORM_FLOAT] < 0) {
+        if (s.slot[other][form] < 0) {
           PTensor a = p;
           a.alias_of = root(t);
           a.layout = (Layout)other;
           a.cs = other == L_NHWC ? (int)p.shape.d[1] : 0;
           plan_->tensors.push_back(a);
-          s.slot[other][p.quant ? FORM_QUANT : FORM_FLOAT] = (int)plan_->tensors.size() - 1;
+          s.slot[other][form] = (int)plan_->tensors.size() - 1;
         }
       }
     }
@@ -335,7 +389,7 @@ class Planner {
     if (dst_q && q == nullptr && !src_q) fail(ODLA_INTERNAL_LOGIC_ERR, "quantised form of '%s' requested without a table entry", v->name.c_str());
     const float scale = src_q ? src.qscale : (q ? q->scale : 1.f);
     const int zp = src_q ? src.qzp : (q ? q->zp : 0);
-    const DType fdt = dst_q ? DT_I8 : storage_dtype(v);
+    const DType fdt = dst_q ? DT_I8 : (form == FORM_OPERAND ? op_dt_ : storage_dtype(v));
     const Space space = SP_ARENA;
     const Shape& sh = v->shape;
 
@@ -345,7 +399,7 @@ class Planner {
       int from = have;
       if (src.layout == L_NHWC && want == L_NHWC) {
         // repitch: go through row-major
-        from = get(v, L_ROWMAJOR, src_q ? FORM_QUANT : FORM_FLOAT);
+        from = get(v, L_ROWMAJOR, src_q ? FORM_QUANT : (form == FORM_OPERAND ? FORM_OPERAND : FORM_FLOAT));
       }
       const PTensor s2 = T(from);
       LayoutParams lp;
@@ -617,10 +671,13 @@ void Planner::run() {
   plan_->calibrated = calib_;
   if (calib_) cdt_ = DT_F32;
   else if (o.fp16) cdt_ = DT_F16;
-  else if (o.bf16 != BF16_DISABLE) cdt_ = DT_BF16;
+  else if (o.bf16 == BF16_ACCURACY_MODE && !o.int8) acc_mode_ = true;   // values fp32, Conv / Gemm operands bf16
+  else if (o.bf16 != BF16_DISABLE) cdt_ = DT_BF16;                      // (performance and auto modes)
+  op_dt_ = acc_mode_ ? DT_BF16 : cdt_;
   if (!calib_) parse_quant_table();
 
   vs_.assign(comp_->values.size(), VState());
+  operand_only_.assign(comp_->values.size(), (signed char)-1);
   consumers_.assign(comp_->values.size(), {});
   for (size_t ni = 0; ni < comp_->nodes.size(); ++ni)
     for (_odla_value* v : comp_->nodes[ni].in)
@@ -914,9 +971,10 @@ void Planner::collect_epilogue(int ni, int64_t channels, int ch_axis, Epilogue* 
       const ActKind a = (ActKind)nx.i[0];
       // the 8-bit epilogue clamps only; the float ones also have a variant with
       // the transcendental activations (GELU behind a feed-forward GEMM)
-      const bool fusable = q8 ? (a == ACT_RELU)
-                              : (a == ACT_RELU || a == ACT_LEAKY || a == ACT_CLAMP || a == ACT_GELU_ERF ||
-                                 a == ACT_GELU_TANH || a == ACT_SIGMOID || a == ACT_TANH);
+      const bool rich = a == ACT_GELU_ERF || a == ACT_GELU_TANH || a == ACT_SIGMOID || a == ACT_TANH;
+      // (the epilogues with the transcendental functions exist for results of the operand type only)
+      const bool rich_ok = rich && ep->residual == nullptr && result_dtype(nx.out) == mm_dtype(nx.out);
+      const bool fusable = q8 ? (a == ACT_RELU) : (a == ACT_RELU || a == ACT_LEAKY || a == ACT_CLAMP || rich_ok);
       if (fusable) {
         ep->act = a;
         ep->act_a = nx.f[0];
@@ -1105,7 +1163,7 @@ void Planner::finish_igemm(const std::string& name, IgemmParams ip, int tx, int 
   if (ep.residual != nullptr) {
     const PTensor yo = T(ty);
     tr = get(ep.residual, yo.layout, FORM_FLOAT);
-    if (T(tr).dt != yo.dt) fail(ODLA_INTERNAL_LOGIC_ERR, "residual type mismatch");
+    if (T(tr).dt != yo.dt) fail(ODLA_INTERNAL_LOGIC_ERR, "residual type mismatch ('%s')", name.c_str());
     ip.rcs = yo.layout == L_NHWC ? T(tr).cs : ip.ycs;
   }
   ip.act = ep.act;
@@ -1225,7 +1283,7 @@ void Planner::lower_conv(int ni) {
       so = (int64_t)C2 * R2 * S2; si = (int64_t)R2 * S2; sr = S2; ss = 1;
 
       // converted input: [N][ceil(H/2)][ceil(W/2)][C2 padded to one vector]
-      const DType fdt = q8 ? DT_I8 : storage_dtype(x);
+      const DType fdt = q8 ? DT_I8 : mm_dtype(x);
       const int vec = 16 / dtype_size(fdt);
       const int cs = round_up_i(C2, vec);
       const int64_t H2 = (H + 1) / 2, W2 = (W + 1) / 2;
@@ -1369,16 +1427,18 @@ void Planner::lower_conv(int ni) {
   }
 
   // ---- floating-point path ----
-  const DType dt = storage_dtype(x);
+  const DType dt = mm_dtype(x);
   if (!dtype_is_float(dt)) fail(ODLA_UNSUPPORTED_DATATYPE, "odla_Conv on element type %d", (int)x->etype);
+  // a result with a residual takes the residual's (storage) type
+  const DType odt = ep.residual != nullptr ? storage_dtype(outv) : result_dtype(outv);
   const int vec = 16 / dtype_size(dt);
   int tx;
   int xcs;
   if (cl) {
-    tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+    tx = get(x, L_ROWMAJOR, FORM_OPERAND);
     xcs = (int)C;
   } else {
-    tx = tx_s2d >= 0 ? tx_s2d : get(x, L_NHWC, FORM_FLOAT, vec);
+    tx = tx_s2d >= 0 ? tx_s2d : get(x, L_NHWC, FORM_OPERAND, vec);
     xcs = T(tx).cs;
   }
   if (T(tx).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "conv input storage type mismatch");
@@ -1405,15 +1465,15 @@ void Planner::lower_conv(int ni) {
   ip.R = (int)R; ip.S = (int)S; ip.sh = str_h; ip.sw = str_w;
   ip.dh = dil_h; ip.dw = dil_w; ip.ph = pad_t; ip.pw = pad_l;
   ip.w_rows = Oge; ip.w_cols = w_rs; ip.w_rs = w_rs;
-  ip.in_dt = dt; ip.out_dt = dt;
+  ip.in_dt = dt; ip.out_dt = odt;
   ip.batch = Ge;
   ip.alpha = ep.scalar;
   if (Ge > 1) { ip.x_bs = Cg; ip.w_bs = (int64_t)Og * w_rs; ip.y_bs = Og; ip.r_bs = Og; ip.bias_bs = Og; }
   ip.ycs = (int)O;
 
   int ty;
-  if (cl) ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
-  else ty = new_tensor(dt, L_NHWC, outv->shape, (int)O, SP_ARENA);
+  if (cl) ty = new_tensor(odt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
+  else ty = new_tensor(odt, L_NHWC, outv->shape, (int)O, SP_ARENA);
 
   if (runtime_bias) {
     // bias supplied at run time: read it as fp32 from its staging tensor
@@ -1502,7 +1562,7 @@ void Planner::lower_gemm(int ni) {
   int64_t lead = 1;
   for (int i = 0; i < as.rank - 2; ++i) lead *= as.d[i];
   const bool shared_b = bs.rank == 2;
-  const DType dt = storage_dtype(A);
+  const DType dt = mm_dtype(A);
   if (!dtype_is_float(dt)) fail(ODLA_UNSUPPORTED_DATATYPE, "odla_Gemm on element type %d", (int)A->etype);
   const int vec = 16 / dtype_size(dt);
 
@@ -1515,6 +1575,8 @@ void Planner::lower_gemm(int ni) {
     else plain_c = gemm_epilogue(ni, &ep);
   }
   _odla_value* outv = ep.final_value;
+  // a result with a residual takes the residual's (storage) type
+  const DType odt = ep.residual != nullptr ? storage_dtype(outv) : result_dtype(outv);
 
   // ---- sibling GEMMs: the same left operand against several constant matrices
   // of one shape (the query / key / value projections of an attention block),
@@ -1529,7 +1591,7 @@ void Planner::lower_gemm(int ni) {
     const int64_t tiles = ((rows + 127) / 128) * ((Nn + 127) / 128);
     auto simple = [&](const Epilogue& e) {
       return e.residual == nullptr && e.row_scale.empty() && e.final_value != nullptr &&
-             storage_dtype(e.final_value) == dt && !e.final_value->is_output;
+             result_dtype(e.final_value) == odt && !e.final_value->is_output;
     };
     if (!calib_ && plain_c && B->kind == _odla_value::CONSTANT && shared_b && !tA && K % vec == 0 && Nn % 32 == 0 &&
         A->kind != _odla_value::CONSTANT && tiles <= 512 && (int64_t)K * es0 >= 256 && simple(ep)) {
@@ -1556,7 +1618,7 @@ void Planner::lower_gemm(int ni) {
   }
 
   // ---- A operand: row-major [lead][M][K], K padded to the vector width ----
-  int ta = get(A, L_ROWMAJOR, FORM_FLOAT);
+  int ta = get(A, L_ROWMAJOR, FORM_OPERAND);
   if (T(ta).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "gemm input storage type mismatch");
   int Kp = round_up_i((int)K, vec);
   if (tA || Kp != K) {
@@ -1584,7 +1646,7 @@ void Planner::lower_gemm(int ni) {
   ip.H = 1; ip.W = 1; ip.Ho = 1; ip.Wo = 1;
   ip.C = Kp; ip.xcs = Kp;
   ip.Kout = (int)Nn;
-  ip.in_dt = dt; ip.out_dt = dt;
+  ip.in_dt = dt; ip.out_dt = odt;
   ip.alpha = alpha * ep.scalar;
   ip.ycs = (int)Nn;
   int tw;
@@ -1622,7 +1684,7 @@ void Planner::lower_gemm(int ni) {
     Shape all;
     all.rank = 3;
     all.d[0] = G; all.d[1] = lead * M; all.d[2] = Nn;
-    const int tall = new_tensor(dt, L_ROWMAJOR, all, 0, SP_ARENA);
+    const int tall = new_tensor(odt, L_ROWMAJOR, all, 0, SP_ARENA);
     Epilogue eall = ep;
     eall.has_bias = any_bias;
     eall.bias = bias_all;
@@ -1640,7 +1702,7 @@ void Planner::lower_gemm(int ni) {
     }
     finish_igemm("gemm.x" + std::to_string(G) + ":" + outv->name, ip, ta, twc, tall, eall, (int64_t)G * Nn);
     if (gemm_merged_.size() < comp_->nodes.size()) gemm_merged_.resize(comp_->nodes.size(), 0);
-    const size_t slice_bytes = (size_t)(lead * M * Nn) * dtype_size(dt);
+    const size_t slice_bytes = (size_t)(lead * M * Nn) * dtype_size(odt);
     for (int g = 0; g < G; ++g) {
       if (split) {
         set_main(hs[g].out, view_tensor(tall, hs[g].out->shape, (size_t)g * slice_bytes));
@@ -1700,11 +1762,11 @@ void Planner::lower_gemm(int ni) {
           p.bias = hb ? rb(e) : nullptr;
           return launch_igemm(p, st);
         });
-        const int ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
+        const int ty = new_tensor(odt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
         const Ref ry = ref(ty);
         const int64_t inner = rows * Nn;
         emit("gemm.sum:" + outv->name, {tp}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
-          return launch_reduce(rp(e), ry(e), DT_F32, dt, 1, splits, inner, RED_SUM, st);
+          return launch_reduce(rp(e), ry(e), DT_F32, odt, 1, splits, inner, RED_SUM, st);
         });
         set_main(outv, ty);
         return;
@@ -1712,7 +1774,7 @@ void Planner::lower_gemm(int ni) {
     }
   } else {
     if (!ep.row_scale.empty()) fail(ODLA_UNSUPPORTED_OP, "odla_Gemm: scale folding into a run-time operand");
-    int tb = get(B, L_ROWMAJOR, FORM_FLOAT);
+    int tb = get(B, L_ROWMAJOR, FORM_OPERAND);
     if (T(tb).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "gemm operand storage type mismatch");
     const int64_t blead = shared_b ? 1 : lead;
     if (!tB || Kp != K) {
@@ -1758,7 +1820,8 @@ void Planner::lower_gemm(int ni) {
       // [B*S, heads*d] stored as [B, heads, S, d]: the Reshape -> Transpose behind it costs nothing
       ip.y_rdiv = (int)hs.S; ip.y_rlo = hs.d; ip.y_rhi = hs.heads * hs.S * hs.d;
       ip.y_cdiv = (int)hs.d; ip.y_chi = hs.S * hs.d;
-      const int ty = new_tensor(dt, L_ROWMAJOR, hs.out->shape, 0, SP_ARENA);
+      ip.out_dt = result_dtype(hs.out);
+      const int ty = new_tensor(ip.out_dt, L_ROWMAJOR, hs.out->shape, 0, SP_ARENA);
       finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
       set_main(hs.out, ty);
       comp_->nodes[hs.reshape].absorbed = true;
@@ -1772,14 +1835,15 @@ void Planner::lower_gemm(int ni) {
       Node& t = comp_->nodes[ti];
       const int64_t heads = os.d[1], S = os.d[2], d = os.d[3];
       ip.y_zdiv = (int)heads; ip.y_bs_hi = S * heads * d; ip.y_bs = d; ip.ycs = (int)(heads * d);
-      const int ty = new_tensor(dt, L_ROWMAJOR, t.out->shape, 0, SP_ARENA);
+      ip.out_dt = result_dtype(t.out);
+      const int ty = new_tensor(ip.out_dt, L_ROWMAJOR, t.out->shape, 0, SP_ARENA);
       finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
       set_main(t.out, ty);
       t.absorbed = true;
       return;
     }
   }
-  const int ty = new_tensor(dt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
+  const int ty = new_tensor(odt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
   finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
   set_main(outv, ty);
 }
@@ -2773,7 +2837,8 @@ void Planner::lower_softmax(int ni) {
   if (tadd >= 0 && T(tadd).dt != dt) fail(ODLA_INTERNAL_LOGIC_ERR, "softmax mask storage type mismatch");
   // a graph output is written in fp32 directly
   const bool to_f32 = n.out->is_output && dtype_from_odla(n.out->etype) == DT_F32 && consumers_[n.out->index].empty();
-  const DType odt = to_f32 ? DT_F32 : dt;
+  // (accuracy mode: probabilities that only feed a matrix product are stored in its operand type)
+  const DType odt = to_f32 ? DT_F32 : (acc_mode_ && dt == DT_F32 && operand_only(n.out) ? op_dt_ : dt);
   const int ty = new_tensor(odt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
   const bool logsm = n.i[1] != 0;
   const Ref a = ref(tx), b = ref(ty), m = ref(tadd >= 0 ? tadd : tx);
@@ -2894,7 +2959,7 @@ void Planner::lower_reshape(int ni) {
   if (s.main >= 0 && T(s.main).quant && s.slot[L_ROWMAJOR][FORM_QUANT] >= 0 && qentry(n.out) != nullptr)
     tx = s.slot[L_ROWMAJOR][FORM_QUANT];
   else
-    tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+    tx = get_moved(x, L_ROWMAJOR);
   const int ty = alias_tensor(tx, n.out->shape);
   set_main(n.out, ty);
 }
@@ -3073,7 +3138,7 @@ void Planner::lower_transpose(int ni) {
     set_main(n.out, alias_tensor(s.main, os));
     return;
   }
-  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const int tx = get_moved(x, L_ROWMAJOR);
   const DType dt = T(tx).dt;
   const int ty = new_tensor(dt, L_ROWMAJOR, os, 0, SP_ARENA);
   int64_t xstr[ODLA_MAX_DIMENSION];
@@ -3230,6 +3295,7 @@ odla_status plan_summary(_odla_computation* comp, int* launches, int* init_launc
   }
   for (Node& n : comp->nodes) n.absorbed = false;
   if (st != ODLA_SUCCESS) return st;
+  for (const Step& sp : plan->steps) OHIP_DEBUG("step %s", sp.name.c_str());
   *launches = (int)plan->steps.size();
   *init_launches = (int)plan->init_steps.size();
   *arena_bytes = plan->arena_bytes;

@@ -329,7 +329,9 @@ class HipBuilder:
             b = ctypes.c_bool(True)
             _check(self.L.odla_SetComputationItem(self.comp, ODLA_FP16_MODE, ctypes.byref(b)), "FP16_MODE")
         if bf16:
-            m = ctypes.c_int32(BF16_PERFORMACE_MODE)
+            # True / "performance": every FLOAT32 value is stored as bf16; "accuracy": values stay fp32 and
+            # only the operands of Conv / Gemm are rounded to bf16 (the reference's two bf16 modes)
+            m = ctypes.c_int32(BF16_ACCURACY_MODE if bf16 == "accuracy" else BF16_PERFORMACE_MODE)
             _check(self.L.odla_SetComputationItem(self.comp, ODLA_BF16_MODE, ctypes.byref(m)), "BF16_MODE")
         if quant_table is not None:
             tbl = (QuantInfo * len(quant_table))(*quant_table)

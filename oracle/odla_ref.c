@@ -26,6 +26,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #if defined(_OPENMP)
@@ -118,14 +119,31 @@ void odla_ref_pool2d_f32(const float* x, float* y, int N, int C, int H, int W, i
 void odla_ref_conv2d_q8(const uint8_t* x, int zp_x, const int8_t* w, const int32_t* bias, int32_t* acc,
                         int N, int C, int H, int W, int O, int R, int S, int sh, int sw, int pt, int pl,
                         int Ho, int Wo) {
+  /* (x - zp_x) once, as int16: the loops below then run on plain multiply-adds */
+  const size_t nx = (size_t)N * C * H * W;
+  int16_t* xs = (int16_t*)malloc(nx * sizeof(int16_t) + 64);
+  if (xs == NULL) return;
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < nx; ++i) xs[i] = (int16_t)((int)x[i] - zp_x);
 #pragma omp parallel for collapse(2) schedule(static)
   for (int n = 0; n < N; ++n) {
     for (int o = 0; o < O; ++o) {
       int32_t* yo = acc + ((size_t)n * O + o) * Ho * Wo;
       const int32_t b = bias ? bias[o] : 0;
       for (int i = 0; i < Ho * Wo; ++i) yo[i] = b;
+      if (R == 1 && S == 1 && sh == 1 && sw == 1 && pt == 0 && pl == 0 && Ho == H && Wo == W) {
+        /* 1x1 filters: the whole image is one contiguous run */
+        const int hw = H * W;
+        for (int c = 0; c < C; ++c) {
+          const int16_t* xc = xs + ((size_t)n * C + c) * hw;
+          const int32_t wv = w[(size_t)o * C + c];
+          if (wv == 0) continue;
+          for (int i = 0; i < hw; ++i) yo[i] += wv * (int32_t)xc[i];
+        }
+        continue;
+      }
       for (int c = 0; c < C; ++c) {
-        const uint8_t* xc = x + ((size_t)n * C + c) * H * W;
+        const int16_t* xc = xs + ((size_t)n * C + c) * H * W;
         const int8_t* wc = w + (((size_t)o * C + c) * R) * S;
         for (int r = 0; r < R; ++r) {
           for (int s = 0; s < S; ++s) {
@@ -134,20 +152,25 @@ void odla_ref_conv2d_q8(const uint8_t* x, int zp_x, const int8_t* w, const int32
             for (int ho = 0; ho < Ho; ++ho) {
               const int hi = ho * sh - pt + r;
               if (hi < 0 || hi >= H) continue;
-              const uint8_t* xr = xc + (size_t)hi * W;
+              const int16_t* xr = xc + (size_t)hi * W;
               int32_t* yr = yo + (size_t)ho * Wo;
               const int off = s - pl;
               int wo0 = 0;
               while (wo0 < Wo && wo0 * sw + off < 0) ++wo0;
               int wo1 = Wo;
               while (wo1 > wo0 && (wo1 - 1) * sw + off >= W) --wo1;
-              for (int wo = wo0; wo < wo1; ++wo) yr[wo] += wv * ((int32_t)xr[wo * sw + off] - zp_x);
+              if (sw == 1) {
+                for (int wo = wo0; wo < wo1; ++wo) yr[wo] += wv * (int32_t)xr[wo + off];
+              } else {
+                for (int wo = wo0; wo < wo1; ++wo) yr[wo] += wv * (int32_t)xr[wo * sw + off];
+              }
             }
           }
         }
       }
     }
   }
+  free(xs);
 }
 
 /* Requantisation of the int8 plan, per channel o; acc (int32 accumulator plus

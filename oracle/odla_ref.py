@@ -82,6 +82,22 @@ def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
 
+def round_to_storage(a, storage):
+    """The fp32 array `a` with every element rounded (to nearest, ties to even) to
+    the nearest value of a 16-bit storage type, still held as fp32.  "bf16": the
+    upper 16 bits of the fp32 pattern; "fp16": IEEE binary16 (values beyond its
+    range become infinities, as in a hardware conversion)."""
+    a = _f32(a)
+    if storage == "bf16":
+        u = a.view(np.uint32).astype(np.uint64)
+        r = ((u + 0x7fff + ((u >> 16) & 1)) & 0xffff0000).astype(np.uint32).view(np.float32)
+        return np.where(np.isnan(a), a, r).astype(np.float32).reshape(a.shape)
+    if storage == "fp16":
+        with np.errstate(over="ignore"):
+            return a.astype(np.float16).astype(np.float32)
+    raise ValueError("unknown storage type %r" % (storage,))
+
+
 # --------------------------------------------------------------------------
 # Heavy kernels (C)
 # --------------------------------------------------------------------------
@@ -476,47 +492,153 @@ _erf = np.vectorize(math.erf, otypes=[np.float64])
 
 
 class RefBuilder:
-    """Eager fp32 evaluation of an ODLA graph on the CPU."""
+    """Eager evaluation of an ODLA graph on the CPU.
 
-    def __init__(self, feeds):
+    Default: every operator in fp32 (the arithmetic of the reference CPU backend).
+
+    Reduced-precision emulation, for networks that a device runs with 16-bit
+    tensors: the same fp32 graph with values rounded to `storage` ("bf16" or
+    "fp16") at chosen points, so that a device result can be told apart from
+    what the storage type alone costs.
+      emulate="operands"  only where a matrix unit must round: both operands of
+          every Conv / Gemm (the reference's BF16_ACCURACY_MODE: operands cast,
+          fp32 results, ODLA/platforms/dnnl/odla_dnnl.cc:1024-1026, 1780-1802);
+          everything else stays fp32.
+      emulate="stored"    at every tensor a 16-bit plan stores: arguments and
+          constants when an operator reads them, every operator's result -
+          except inside the chains one launch computes in fp32: Conv / Gemm with
+          a per-channel constant Add / Sub / Mul / Div, one same-shape residual
+          Add and one activation behind it (an Add behind the activation too),
+          an Add whose only reader is a Softmax, a Softmax that is a graph
+          output.  Parameters that stay fp32 on the device (Conv / Gemm bias,
+          LayerNorm and BatchNorm parameters) are not rounded.
+    """
+
+    _ACTS = ("relu", "leaky_relu", "clamp", "gelu", "sigmoid", "tanh")
+
+    def __init__(self, feeds, emulate=None, storage=None):
+        assert emulate in (None, "operands", "stored")
+        assert (emulate is None) == (storage is None)
         self.feeds = feeds
         self.outputs = {}
         self.values = {}
+        self.emulate, self.storage = emulate, storage
+        self._open = {}      # id -> (array, stage): computed in fp32, not yet rounded to storage
+        self._consts = {}    # id -> array handed out by const()
+        self._rounded_const = {}
+        if emulate == "stored":
+            special = {"arg", "const", "output", "conv", "gemm", "batch_matmul", "add", "sub", "mul", "div",
+                       "softmax", "layernorm", "batchnorm"} | set(self._ACTS)
+            for attr in dir(type(self)):
+                if attr.startswith("_") or attr in special or not callable(getattr(type(self), attr)):
+                    continue
+                setattr(self, attr, self._stored_op(getattr(self, attr)))
 
     def _name(self, name, v):
         if name:
             self.values[name] = v
         return v
 
+    # reduced-precision emulation -------------------------------------------
+    def _rs(self, a):
+        return round_to_storage(a, self.storage)
+
+    def _is_f32(self, v):
+        return isinstance(v, np.ndarray) and v.dtype == np.float32
+
+    def _closed(self, v):
+        """`v` as an operator that reads stored tensors sees it."""
+        if self.emulate != "stored" or not self._is_f32(v):
+            return v
+        ent = self._open.pop(id(v), None)
+        if ent is not None:          # first reader outside its launch: the tensor is stored now
+            v[...] = self._rs(v)
+            return v
+        if id(v) in self._consts:    # constants are converted to the storage type when uploaded
+            r = self._rounded_const.get(id(v))
+            if r is None:
+                r = self._rounded_const[id(v)] = self._rs(v)
+            return r
+        return v
+
+    def _store(self, v):
+        """Result of an operator that writes a stored tensor."""
+        if self.emulate == "stored" and self._is_f32(v) and v.flags.writeable:
+            v[...] = self._rs(v)
+        return v
+
+    def _mark_open(self, v, stage):
+        if self.emulate == "stored" and self._is_f32(v):
+            self._open[id(v)] = (v, stage)
+        return v
+
+    def _stage(self, v):
+        ent = self._open.get(id(v)) if isinstance(v, np.ndarray) else None
+        return None if ent is None else ent[1]
+
+    def _stored_op(self, f):
+        def close(a):
+            if isinstance(a, np.ndarray):
+                return self._closed(a)
+            if isinstance(a, (list, tuple)) and any(isinstance(e, np.ndarray) for e in a):
+                return type(a)(close(e) for e in a)
+            return a
+
+        def run(*args, **kw):
+            out = f(*[close(a) for a in args], **{k: close(a) for k, a in kw.items()})
+            if isinstance(out, tuple):
+                return tuple(self._store(o) for o in out)
+            return self._store(out)
+        return run
+
+    def _operand(self, v):
+        """A Conv / Gemm operand: rounded to the storage type in both emulations."""
+        if self.emulate == "operands":
+            return self._rs(v) if self._is_f32(np.asarray(v)) else v
+        return self._closed(v)
+
     # graph inputs -----------------------------------------------------------
     def arg(self, name, shape, dtype=np.float32):
         v = np.ascontiguousarray(self.feeds[name], dtype=dtype)
         assert tuple(v.shape) == tuple(shape), (name, v.shape, shape)
+        if self.emulate == "stored" and v.dtype == np.float32:
+            v = self._rs(v)          # converted on its way into the plan
         return self._name(name, v)
 
     def const(self, name, array):
-        return self._name(name, np.ascontiguousarray(array))
+        v = np.ascontiguousarray(array)
+        self._consts[id(v)] = v
+        return self._name(name, v)
 
     def output(self, v, name):
-        self.outputs[name] = v
+        st = self._stage(v)
+        if st is not None and st[0] == "softmax":
+            self._open.pop(id(v))    # written in fp32 by the Softmax launch itself
+        self.outputs[name] = self._closed(v)
 
     # heavy operators --------------------------------------------------------
     def conv(self, x, w, bias=None, stride=(1, 1), pad=(0, 0, 0, 0), dilation=(1, 1), group=1, name=None):
-        return self._name(name, conv2d(x, w, bias, stride, pad, dilation, group))
+        y = conv2d(self._operand(x), self._operand(w), bias, stride, pad, dilation, group)
+        return self._name(name, self._mark_open(y, ("acc", 1)))
 
     def gemm(self, a, b, c=None, ta=False, tb=False, alpha=1.0, beta=1.0, name=None):
         """alpha * op(A) op(B) + beta * C; leading dims of A are batch dims.
         [ref: odla_dnnl.cc:1730-1866]"""
-        a, b = _f32(a), _f32(b)
+        a, b = _f32(self._operand(a)), _f32(self._operand(b))
         if ta:
             a = np.swapaxes(a, -1, -2)
         if tb:
             b = np.swapaxes(b, -1, -2)
         y = np.matmul(a.astype(np.float64), b.astype(np.float64))
         y = y * float(alpha)
+        stage = "acc"
         if c is not None and beta != 0:
+            if id(c) not in self._consts:   # a run-time matrix rides as the launch's residual operand
+                c = self._closed(c)
+                stage = "res"
             y = y + float(beta) * _f32(c).astype(np.float64)
-        return self._name(name, y.astype(np.float32))
+        y = y.astype(np.float32)
+        return self._name(name, self._mark_open(y, (stage, y.ndim - 1)))
 
     def batch_matmul(self, a, b, ta=False, tb=False, name=None):
         """op(A) op(B) over matching leading batch dims [ref: ops/odla_ops_math.h:337-339;
@@ -531,7 +653,8 @@ class RefBuilder:
 
     # element-wise -----------------------------------------------------------
     def _bin(self, f, a, b, name):
-        a, b = np.asarray(a), np.asarray(b)
+        a, b = (v if isinstance(v, np.ndarray) else np.asarray(v) for v in (a, b))
+        ra, rb = a, b   # as given: identity matters for the emulation's bookkeeping
         if a.ndim != b.ndim:
             if a.ndim < b.ndim:
                 a = a.reshape(align_like_reference(a.shape, b.shape))
@@ -539,7 +662,41 @@ class RefBuilder:
                 b = b.reshape(align_like_reference(b.shape, a.shape))
         if a.dtype.kind in "iu" and a.dtype == b.dtype:  # integer arithmetic [ref: odla_dnnl.cc:567-610]
             return self._name(name, f(a, b).astype(a.dtype))
-        return self._name(name, f(a.astype(np.float32), b.astype(np.float32)).astype(np.float32))
+        if self.emulate != "stored":
+            return self._name(name, f(a.astype(np.float32), b.astype(np.float32)).astype(np.float32))
+        # ---- 16-bit storage: what joins the launch of an open Conv / Gemm stays fp32
+        out_shape = np.broadcast_shapes(a.shape, b.shape)
+        for cur, other, c_al, o_al, lhs in ((ra, rb, a, b, True), (rb, ra, b, a, False)):
+            st = self._stage(cur)
+            if st is None or st[0] not in ("acc", "act") or tuple(c_al.shape) != tuple(out_shape):
+                continue
+            stage, ch = st
+            is_const = id(other) in self._consts
+            per_channel = o_al.size == 1 or (o_al.size == out_shape[ch] and o_al.shape[ch] == o_al.size)
+            res = None
+            if stage == "acc" and is_const and per_channel and (
+                    f is np.add or f is np.multiply or (f is np.subtract and lhs) or (f is np.divide and lhs and o_al.size == 1)):
+                res, nxt = (f(c_al, o_al.astype(np.float32)) if lhs else f(o_al.astype(np.float32), c_al)), ("acc", ch)
+            elif f is np.add and not is_const and tuple(o_al.shape) == tuple(out_shape):
+                o_cl = self._closed(other).reshape(o_al.shape)
+                res, nxt = c_al + o_cl, (("res", ch) if stage == "acc" else ("done", ch))
+            if res is not None:
+                self._open.pop(id(cur), None)
+                return self._name(name, self._mark_open(res.astype(np.float32), nxt))
+        a = self._closed(ra).reshape(a.shape).astype(np.float32)
+        b = self._closed(rb).reshape(b.shape).astype(np.float32)
+        y = f(a, b).astype(np.float32)
+        if f is np.add:   # an attention mask in front of a Softmax is added inside the Softmax launch
+            return self._name(name, self._mark_open(y, ("bin", y.ndim - 1)))
+        return self._name(name, self._store(y))
+
+    def _act(self, f, x, name):
+        """Activation: joins the launch of an open Conv / Gemm, else reads and writes stored tensors."""
+        st = self._stage(x)
+        if st is not None and st[0] in ("acc", "res"):
+            self._open.pop(id(x))
+            return self._name(name, self._mark_open(f(x), ("act" if st[0] == "acc" else "done", st[1])))
+        return self._name(name, self._store(f(_f32(self._closed(x)))))
 
     def add(self, a, b, name=None): return self._bin(np.add, a, b, name)
     def sub(self, a, b, name=None): return self._bin(np.subtract, a, b, name)
@@ -548,17 +705,19 @@ class RefBuilder:
     def max(self, a, b, name=None): return self._bin(np.maximum, a, b, name)
     def min(self, a, b, name=None): return self._bin(np.minimum, a, b, name)
 
-    def relu(self, x, name=None): return self._name(name, np.maximum(_f32(x), np.float32(0)))
+    def relu(self, x, name=None): return self._act(lambda v: np.maximum(_f32(v), np.float32(0)), x, name)
 
     def leaky_relu(self, x, alpha, name=None):
-        x = _f32(x)
-        return self._name(name, np.where(x > 0, x, np.float32(alpha) * x).astype(np.float32))
+        return self._act(lambda v: np.where(_f32(v) > 0, _f32(v), np.float32(alpha) * _f32(v)).astype(np.float32), x, name)
 
     def _unary64(self, f, x, name):
         return self._name(name, f(_f32(x).astype(np.float64)).astype(np.float32))
 
-    def sigmoid(self, x, name=None): return self._unary64(lambda v: 1.0 / (1.0 + np.exp(-v)), x, name)
-    def tanh(self, x, name=None): return self._unary64(np.tanh, x, name)
+    def _act64(self, f, x, name):
+        return self._act(lambda v: f(_f32(v).astype(np.float64)).astype(np.float32), x, name)
+
+    def sigmoid(self, x, name=None): return self._act64(lambda v: 1.0 / (1.0 + np.exp(-v)), x, name)
+    def tanh(self, x, name=None): return self._act64(np.tanh, x, name)
     def exp(self, x, name=None): return self._unary64(np.exp, x, name)
     def log(self, x, name=None): return self._unary64(np.log, x, name)
     def sqrt(self, x, name=None): return self._unary64(np.sqrt, x, name)
@@ -569,7 +728,7 @@ class RefBuilder:
     def round(self, x, name=None): return self._name(name, np.rint(_f32(x)))
 
     def clamp(self, x, lo, hi, name=None):
-        return self._name(name, np.clip(_f32(x), np.float32(lo), np.float32(hi)))
+        return self._act(lambda v: np.clip(_f32(v), np.float32(lo), np.float32(hi)), x, name)
 
     def gelu(self, x, approx=False, name=None):
         """[ref: odla_dnnl.cc:1868-1876]"""
@@ -577,26 +736,32 @@ class RefBuilder:
             f = lambda v: 0.5 * v * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (v + 0.044715 * v ** 3)))
         else:
             f = lambda v: 0.5 * v * (1.0 + _erf(v / math.sqrt(2.0)))
-        return self._unary64(f, x, name)
+        return self._act64(f, x, name)
 
     # normalisation ----------------------------------------------------------
     def batchnorm(self, x, mean, var, eps, scale=None, offset=None, scalar_scale=1.0, scalar_offset=0.0,
                   name=None):
         """y = scale * (x - mean) / sqrt(var + eps) + offset over channel axis 1.
         [ref: odla_dnnl.cc:1448-1524]"""
+        st = self._stage(x)
+        folded = st is not None and st[0] == "acc" and st[1] == 1   # folded into the Conv in front of it
+        if folded:
+            self._open.pop(id(x))
+        else:
+            x = self._closed(x)
         x = _f32(x)
         C = x.shape[1]
         sh = (1, C) + (1,) * (x.ndim - 2)
         g = np.full(C, scalar_scale, np.float64) if scale is None else _f32(scale).astype(np.float64)
         b = np.full(C, scalar_offset, np.float64) if offset is None else _f32(offset).astype(np.float64)
         m = g / np.sqrt(_f32(var).astype(np.float64) + float(np.float32(eps)))
-        y = x.astype(np.float64) * m.reshape(sh) + (b - _f32(mean).astype(np.float64) * m).reshape(sh)
-        return self._name(name, y.astype(np.float32))
+        y = (x.astype(np.float64) * m.reshape(sh) + (b - _f32(mean).astype(np.float64) * m).reshape(sh)).astype(np.float32)
+        return self._name(name, self._mark_open(y, ("acc", 1)) if folded else self._store(y))
 
     def layernorm(self, x, n_axes, eps, scale=None, offset=None, name=None):
         """Biased variance over the trailing n_axes axes, eps inside the root.
         [ref: lib/transforms/fusion.cc:296-313]"""
-        x64 = _f32(x).astype(np.float64)
+        x64 = _f32(self._closed(x)).astype(np.float64)
         ax = tuple(range(x64.ndim - n_axes, x64.ndim))
         mu = x64.mean(axis=ax, keepdims=True)
         var = ((x64 - mu) ** 2).mean(axis=ax, keepdims=True)
@@ -605,18 +770,23 @@ class RefBuilder:
             y = y * _f32(scale).astype(np.float64).reshape(x64.shape[-n_axes:])
         if offset is not None:
             y = y + _f32(offset).astype(np.float64).reshape(x64.shape[-n_axes:])
-        return self._name(name, y.astype(np.float32))
+        return self._name(name, self._store(y.astype(np.float32)))
 
     def softmax(self, x, axis=-1, log=False, name=None):
         """[ref: odla_dnnl.cc:1628-1669]; every negative axis means the last one."""
+        st = self._stage(x)
+        if st is not None and st[0] == "bin" and axis in (-1, np.ndim(x) - 1):
+            self._open.pop(id(x))    # the Add in front ran inside this launch
+        else:
+            x = self._closed(x)
         x64 = _f32(x).astype(np.float64)
         if axis < 0:
             axis = x64.ndim - 1
         z = x64 - x64.max(axis=axis, keepdims=True)
         e = np.exp(z)
         s = e.sum(axis=axis, keepdims=True)
-        y = z - np.log(s) if log else e / s
-        return self._name(name, y.astype(np.float32))
+        y = (z - np.log(s) if log else e / s).astype(np.float32)
+        return self._name(name, self._mark_open(y, ("softmax", axis)))
 
     def reduce_mean(self, x, axes, keep_dims=True, name=None):
         """[ref: odla_dnnl_statistics.cc:20-46,111-117]"""

@@ -83,16 +83,38 @@ def run_ref(build_fn, feeds):
     return rb.outputs
 
 
+def run_ref_emulated(build_fn, feeds, emulate, storage):
+    """The oracle with values rounded to a 16-bit storage type: emulate = "operands"
+    (Conv / Gemm operands only) or "stored" (every tensor a 16-bit plan stores)."""
+    ref = entry.load_oracle()
+    rb = ref.RefBuilder(feeds, emulate=emulate, storage=storage)
+    build_fn(rb)
+    return rb.outputs
+
+
+def err_stats(got, want):
+    """(max, 99.9th percentile, mean) of |got - want|."""
+    d = np.abs(np.asarray(got, np.float64) - np.asarray(want, np.float64))
+    return float(d.max()), float(np.quantile(d, 0.999)), float(d.mean())
+
+
 def run_both(build_fn, feeds, **kw):
     return run_hip(build_fn, feeds, **kw), run_ref(build_fn, feeds)
 
 
-def max_rel_err(got, want):
-    """Largest |got-want| relative to the largest magnitude of the expected tensor."""
+REL_ERR_FLOOR = 0.05
+
+
+def max_rel_err(got, want, floor=REL_ERR_FLOOR):
+    """Largest element-wise relative error  |got - want| / max(|want|, floor * max|want|).
+    Elements smaller than `floor` x the tensor's largest magnitude are measured against that
+    magnitude instead of their own: they are sums that cancel, and a sum that cancels has no
+    relative accuracy of its own in any summation order (its absolute error is that of its
+    terms, which are of the tensor's scale)."""
     got = np.asarray(got, np.float64)
     want = np.asarray(want, np.float64)
-    scale = max(float(np.max(np.abs(want))), 1e-30)
-    return float(np.max(np.abs(got - want))) / scale
+    scale = max(float(np.max(np.abs(want))) if want.size else 0.0, 1e-30)
+    return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), floor * scale))) if want.size else 0.0
 
 
 def announce(msg):
