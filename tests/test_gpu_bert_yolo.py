@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import __graft_entry__ as entry
-from util import announce, max_rel_err, run_hip, run_ref
+from util import announce, max_rel_err, run_hip, run_ref, run_ref_emulated
 
 pytestmark = pytest.mark.gpu
 
@@ -27,6 +27,23 @@ def test_small_bert_encoder(mode):
     else:
         # bf16 storage (8 significant bits) of O(1) LayerNorm outputs
         assert np.max(np.abs(got - want)) <= 2e-2 * max(1.0, float(np.max(np.abs(want))))
+
+
+def test_small_bert_encoder_bf16_accuracy_mode():
+    """BF16_ACCURACY_MODE against the oracle that rounds only the Gemm operands; a padded sequence
+    exercises the mask, which stays fp32 in this mode."""
+    announce("small bert bf16, accuracy mode")
+    mb = entry.load().models_bert
+    w = mb.bert_weights(SMALL_BERT, seed=3)
+    feeds = mb.bert_input(4, 32, SMALL_BERT, seed=4)
+    feeds["attention_mask"][1, 0, 0, 20:] = 0.0
+    build = lambda b: mb.build_bert(b, w, 4, 32, SMALL_BERT)
+    got = run_hip(build, feeds, bf16="accuracy")["hidden"]
+    want = run_ref(build, feeds)["hidden"]
+    emu = run_ref_emulated(build, feeds, "operands", "bf16")["hidden"]
+    floor, e, d = (float(np.max(np.abs(a - b))) for a, b in ((emu, want), (got, want), (got, emu)))
+    announce("small bert bf16 accuracy mode: operands floor %.3e, GPU vs fp32 %.3e, GPU vs emulated %.3e" % (floor, e, d))
+    assert e <= 2e-2 and e <= 1.5 * floor and d <= floor
 
 
 def test_small_yolov3_heads_and_detections():

@@ -6,7 +6,7 @@ choices, aliasing and the arena - rather than at any one kernel."""
 import numpy as np
 import pytest
 
-from util import announce, max_rel_err, run_hip, run_hip_stored, run_ref
+from util import announce, max_rel_err, run_hip, run_hip_stored, run_ref, run_ref_emulated
 
 pytestmark = pytest.mark.gpu
 
@@ -142,19 +142,26 @@ class Chain:
             b.output(vals[k], "v%d" % k)
 
 
-@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+def _mode_kwargs(mode):
+    return {"fp32": {}, "fp16": {"fp16": True}, "bf16acc": {"bf16": "accuracy"}}[mode]
+
+
+@pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16acc"])
 def test_random_chains(mode, tmp_path):
+    """bf16acc: BF16_ACCURACY_MODE (values fp32, Conv operands bf16) against the oracle that
+    rounds exactly those operands - what is left are roundings that fell the other way."""
+    kw = _mode_kwargs(mode)
     for seed in range(200):
         ch = Chain(SEED0 + seed)
         if not ch.steps:
             continue
         announce("chain %s seed %d: %s -> outputs %s" % (mode, seed, [s[0] for s in ch.steps], ch.outputs))
         feeds = {"x": ch.x}
-        want = run_ref(ch.build, feeds)
-        got = run_hip(ch.build, feeds, fp16=(mode == "fp16"), repeats=2)
+        want = run_ref_emulated(ch.build, feeds, "operands", "bf16") if mode == "bf16acc" else run_ref(ch.build, feeds)
+        got = run_hip(ch.build, feeds, repeats=2, **kw)
         if seed % 4 == 0:
             # the same program stored to a file and loaded back computes the same bits
-            again = run_hip_stored(ch.build, feeds, str(tmp_path / ("chain%d.odla" % seed)), fp16=(mode == "fp16"))
+            again = run_hip_stored(ch.build, feeds, str(tmp_path / ("chain%d.odla" % seed)), **kw)
             for k in got:
                 assert np.array_equal(again[k], got[k]), (seed, k, "stored")
         for k, w in want.items():
@@ -163,7 +170,8 @@ def test_random_chains(mode, tmp_path):
                 assert max_rel_err(got[k], w) <= 5e-4, (seed, k, [s[0] for s in ch.steps])
             else:
                 scale = max(1.0, float(np.max(np.abs(w))))
-                assert float(np.max(np.abs(got[k] - w))) <= 6e-2 * scale, (seed, k, [s[0] for s in ch.steps])
+                tol = 6e-2 if mode == "fp16" else 1e-2
+                assert float(np.max(np.abs(got[k] - w))) <= tol * scale, (seed, k, [s[0] for s in ch.steps])
 
 
 @pytest.mark.parametrize("mode", ["fp32", "fp16"])

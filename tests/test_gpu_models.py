@@ -6,7 +6,7 @@ network is covered by test_gpu_resnet50_full.py).
 import numpy as np
 import pytest
 
-from util import announce, max_rel_err, run_hip, run_ref
+from util import run_ref_emulated, announce, max_rel_err, run_hip, run_ref
 
 pytestmark = pytest.mark.gpu
 
@@ -69,6 +69,26 @@ def test_small_resnet_reduced_precision(models, mode):
     assert np.max(np.abs(got["logits"] - want["logits"])) <= tol
     if mode == "fp16":
         assert np.array_equal(np.argmax(got["logits"], 1), np.argmax(want["logits"], 1))
+
+
+def test_small_resnet_bf16_accuracy_mode(models):
+    """BF16_ACCURACY_MODE: values stay fp32, only Conv / Gemm operands are bf16.  Against the oracle
+    that rounds exactly those operands the logits agree to a small fraction of what the operand
+    rounding itself costs; against fp32 they are several times closer than with bf16 storage."""
+    announce("small resnet bf16, accuracy mode")
+    w = models.resnet50_weights(seed=3, num_classes=100, stages=SMALL_STAGES, stem=16)
+    feeds = models.resnet50_input(4, 64, seed=4)
+    build = lambda b: models.build_resnet50(b, w, 4, 64, SMALL_STAGES, 16, 100)
+    got = run_hip(build, feeds, bf16="accuracy")["logits"]
+    perf = run_hip(build, feeds, bf16="performance")["logits"]
+    want = run_ref(build, feeds)["logits"]
+    emu = run_ref_emulated(build, feeds, "operands", "bf16")["logits"]
+    floor = float(np.max(np.abs(emu - want)))
+    e_acc, e_perf, d = (float(np.max(np.abs(a - b))) for a, b in ((got, want), (perf, want), (got, emu)))
+    announce("small resnet bf16: operands floor %.3e, accuracy mode vs fp32 %.3e, vs emulated %.3e; performance mode vs fp32 %.3e"
+             % (floor, e_acc, d, e_perf))
+    assert e_acc <= 1.5 * floor and d <= floor
+    assert np.array_equal(np.argmax(got, 1), np.argmax(emu, 1))
 
 
 def test_graph_replay_equals_eager(models):
