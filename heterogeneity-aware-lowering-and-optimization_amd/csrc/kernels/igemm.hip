@@ -92,9 +92,10 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
   lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
   // (with or without a residual: two straight-line copies of the slice chosen by one
   // workgroup-uniform branch; as a condition inside, every value pays a move or a select)
-  auto slice = [&](auto slice_no, auto with_res) __attribute__((always_inline)) {
+  auto slice = [&](auto slice_no, auto with_res, auto with_clamp) __attribute__((always_inline)) {
     constexpr int i = decltype(slice_no)::value;
     constexpr bool kRes = decltype(with_res)::value;
+    constexpr bool kClamp = decltype(with_clamp)::value;
     unsigned char* otile = smem + (i & 1) * (2 * TILE);
     unsigned char* rtile = otile + TILE;
     if constexpr (kRes) {
@@ -106,7 +107,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
       const int off = (l32 * PITCH + wave * 32 + q * 8 + lg * 4) ^ q8_swz(l32);
       const unsigned rs = kRes ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
       *reinterpret_cast<unsigned*>(otile + off) =
-          requant4<kRes>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q], rs, p);
+          requant4<kRes, kClamp>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q], rs, p);
     }
     // Nobody passes this barrier before every wavefront has written slice i; a wavefront
     // writes slice i+1 into the other tile pair, and slice i+2 into this one only after
@@ -116,17 +117,15 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
     const uintx4 v = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + rp * PITCH + c16), rp);
     if (m < M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
   };
-  if (has_res) {
-    slice(std::integral_constant<int, 0>{}, std::true_type{});
-    slice(std::integral_constant<int, 1>{}, std::true_type{});
-    slice(std::integral_constant<int, 2>{}, std::true_type{});
-    slice(std::integral_constant<int, 3>{}, std::true_type{});
-  } else {
-    slice(std::integral_constant<int, 0>{}, std::false_type{});
-    slice(std::integral_constant<int, 1>{}, std::false_type{});
-    slice(std::integral_constant<int, 2>{}, std::false_type{});
-    slice(std::integral_constant<int, 3>{}, std::false_type{});
-  }
+  auto slices = [&](auto with_res, auto with_clamp) __attribute__((always_inline)) {
+    slice(std::integral_constant<int, 0>{}, with_res, with_clamp);
+    slice(std::integral_constant<int, 1>{}, with_res, with_clamp);
+    slice(std::integral_constant<int, 2>{}, with_res, with_clamp);
+    slice(std::integral_constant<int, 3>{}, with_res, with_clamp);
+  };
+  const bool clamp = p.q_lo > 0.f;   // (a lower bound of 0 is what the saturating conversion applies anyway)
+  if (has_res) { if (clamp) slices(std::true_type{}, std::true_type{}); else slices(std::true_type{}, std::false_type{}); }
+  else { if (clamp) slices(std::false_type{}, std::true_type{}); else slices(std::false_type{}, std::false_type{}); }
 }
 
 // ---------------------------------------------------------------------------
@@ -1288,8 +1287,9 @@ hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
   if constexpr (std::is_same<TIn, f16_t>::value || std::is_same<TIn, bf16_t>::value) {
     if (p.w_frag != nullptr && lean_steps(p) > 0) return launch_lean<TIn, Epi>(p, epi_vec, s);
   }
-  // (the short-tap kernel is built for 8-bit layers with 8-bit results)
+  // (the streaming 1x1 kernel and the short-tap kernel are built for 8-bit layers with 8-bit results)
   if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
+    if (p.w_frag != nullptr && (epi_vec & 2) && igemm_stream_q8_geometry(p)) return launch_igemm_stream_q8(p, s);
     if (p.w_frag != nullptr && taps_shape(p).nkk > 0) return launch_taps<TIn, Epi>(p, epi_vec, s);
   }
   if (p.w_frag != nullptr && wreg_shape(p)) return launch_wreg<TIn, Epi>(p, epi_vec, s);
@@ -1298,7 +1298,9 @@ hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
 
 }  // namespace
 
-bool igemm_wants_wfrag(const IgemmParams& p) { return wreg_shape(p) || lean_steps(p) > 0 || taps_shape(p).nkk > 0; }
+bool igemm_wants_wfrag(const IgemmParams& p) {
+  return wreg_shape(p) || lean_steps(p) > 0 || taps_shape(p).nkk > 0 || igemm_stream_q8_geometry(p);
+}
 
 hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
   if (p.src == nullptr || p.dst == nullptr || p.rows <= 0 || p.row_bytes <= 0 || p.row_bytes % 16 != 0 ||
@@ -1317,6 +1319,7 @@ const char* igemm_variant_name(const IgemmParams& p) {
     case 3: return "128x256";
     default: break;
   }
+  if (p.w_frag != nullptr && igemm_stream_q8_geometry(p)) return "stream";
   if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
   if (p.w_frag != nullptr && taps_shape(p).nkk > 0) return "128x64t";
   if (p.w_frag != nullptr && wreg_shape(p)) return "128x128w";

@@ -293,7 +293,9 @@ __device__ __forceinline__ void acc_init_bias_vec(const IgemmParams& p, const in
 // result's zero point or, with a residual, fma(float(r), r_mul, r_add) per
 // channel.  v_cvt_pk_u8_f32 rounds to nearest even and saturates to [0, 255];
 // stored bytes are level - 128, i.e. level ^ 0x80.
-template <bool kRes>
+// kClamp = false: the lower bound is 0 (no ReLU, or a ReLU whose result has zero point 0, the
+// usual case), which the saturating conversion applies by itself - same bits, one operation less.
+template <bool kRes, bool kClamp = true>
 __device__ __forceinline__ unsigned requant4(const int a0, const int a1, const int a2, const int a3, const floatx4 m,
                                              const unsigned res_stored, const IgemmParams& p) {
   float add0 = p.q_add, add1 = p.q_add, add2 = p.q_add, add3 = p.q_add;
@@ -304,10 +306,13 @@ __device__ __forceinline__ unsigned requant4(const int a0, const int a1, const i
     add2 = __builtin_fmaf((float)((r >> 16) & 0xffu), p.r_mul, p.r_add);
     add3 = __builtin_fmaf((float)(r >> 24), p.r_mul, p.r_add);
   }
-  const float f0 = fmaxf(__builtin_fmaf((float)a0, m.x, add0), p.q_lo);
-  const float f1 = fmaxf(__builtin_fmaf((float)a1, m.y, add1), p.q_lo);
-  const float f2 = fmaxf(__builtin_fmaf((float)a2, m.z, add2), p.q_lo);
-  const float f3 = fmaxf(__builtin_fmaf((float)a3, m.w, add3), p.q_lo);
+  float f0 = __builtin_fmaf((float)a0, m.x, add0);
+  float f1 = __builtin_fmaf((float)a1, m.y, add1);
+  float f2 = __builtin_fmaf((float)a2, m.z, add2);
+  float f3 = __builtin_fmaf((float)a3, m.w, add3);
+  if constexpr (kClamp) {
+    f0 = fmaxf(f0, p.q_lo); f1 = fmaxf(f1, p.q_lo); f2 = fmaxf(f2, p.q_lo); f3 = fmaxf(f3, p.q_lo);
+  }
   unsigned w = 0u;
   w = __builtin_amdgcn_cvt_pk_u8_f32(f0, 0, w);
   w = __builtin_amdgcn_cvt_pk_u8_f32(f1, 1, w);
@@ -450,8 +455,9 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
     // requantise in the accumulator layout: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
     // (the residual case is a wavefront-uniform branch around the whole block: as a
     // per-element condition it costs a select per value)
-    auto requant_block = [&](auto with_res) {
+    auto requant_block = [&](auto with_res, auto with_clamp) {
       constexpr bool kRes = decltype(with_res)::value;
+      constexpr bool kClamp = decltype(with_clamp)::value;
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -460,13 +466,14 @@ __device__ __forceinline__ void igemm_epilogue_q8(const IgemmParams& p, const in
           const int off = (l32 * PITCH + ch) ^ q8_swz(l32);
           const floatx4 m = *reinterpret_cast<const floatx4*>(mtile + ch);
           const unsigned rs = kRes ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
-          const unsigned w = requant4<kRes>(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+          const unsigned w = requant4<kRes, kClamp>(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
                                             acc[i][j][q * 4 + 3], m, rs, p);
           *reinterpret_cast<unsigned*>(otile + off) = w;
         }
     };
-    if (has_res) requant_block(std::true_type{});
-    else requant_block(std::false_type{});
+    const bool clamp = p.q_lo > 0.f;   // (wavefront-uniform, like has_res)
+    if (has_res) { if (clamp) requant_block(std::true_type{}, std::true_type{}); else requant_block(std::true_type{}, std::false_type{}); }
+    else { if (clamp) requant_block(std::false_type{}, std::true_type{}); else requant_block(std::false_type{}, std::false_type{}); }
     wave_fence();
 #pragma unroll
     for (int ps = 0; ps < NPASS; ++ps) {

@@ -1,0 +1,279 @@
+// Streaming kernel for 8-bit 1x1 convolutions over short pixel rows (gfx950).
+//
+// The 1x1 layers of a network's first stages move far more bytes than they
+// compute: 64 -> 256 channels at 56 x 56 and batch 256 reads 51 MB (+ 205 MB of
+// residual) and writes 205 MB for 26 GOP.  A tiled GEMM with a K loop, operand
+// staging and workgroup barriers turns such a layer into a chain of latencies
+// per tile.  Here nothing is staged per tile and nothing is shared but the
+// weights:
+//   * a workgroup keeps ALL weights of the layer (Kout x K bytes <= 64 KiB, in
+//     MFMA fragment order), the int32 bias and the multipliers in LDS for its
+//     whole life and walks pixel groups with a grid stride;
+//   * a wavefront owns 32 pixels x all output channels: the 16 bytes a lane
+//     feeds to v_mfma_i32_32x32x32_i8 are one contiguous piece of its pixel's
+//     row, so the pixel operand goes straight from global memory into the
+//     operand registers, once per tile;
+//   * per 32-channel slice: the weight fragments come from LDS, the
+//     accumulators start at the bias, the requantisation runs in the accumulator
+//     layout (four consecutive channels of one pixel per dword), and the 16-byte
+//     row vectors of the result - and of the residual, in the other direction -
+//     are formed by exchanging dwords between lanes l and l + 32
+//     (v_permlane32_swap): no LDS round trip, no barrier, no wave-level fence.
+// The arithmetic of the result is that of igemm_epilogue_q8 (requant4).
+#include "igemm_common.h"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace ohip {
+
+namespace {
+
+// X' = [X.lo | Y.lo], Y' = [X.hi | Y.hi] over the two 32-lane halves (its own inverse).
+__device__ __forceinline__ void swap32(unsigned& x, unsigned& y) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uintx2 r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+  x = r.x;
+  y = r.y;
+#endif
+}
+
+// Accumulator layout of one 32 x 32 block: lane (l32, lg) holds, for pixel l32,
+// the dwords of channel groups q*8 + lg*4 (q = 0..3).  Row layout: lane (l32, lg)
+// holds the 16 consecutive channels lg*16 .. lg*16 + 15 of pixel l32.
+// For lg = 0 the row vector holds the groups (q0,0) (q0,1) (q1,0) (q1,1), for lg = 1
+// (q2,0) (q2,1) (q3,0) (q3,1), where group (q, s) = channels q*8 + s*4 .. + 3.
+// rows -> accumulator dwords d[q]
+__device__ __forceinline__ void rows_to_acc(const uintx4 v, unsigned (&d)[4]) {
+  unsigned a = v.x, b = v.y, c = v.z, e = v.w;
+  swap32(a, b);   // a' = [(q0,0) | (q0,1)]: group q0 at every lane's own lg;  b' = [(q2,0) | (q2,1)]
+  swap32(c, e);   // c' = [(q1,0) | (q1,1)],  e' = [(q3,0) | (q3,1)]
+  d[0] = a; d[2] = b; d[1] = c; d[3] = e;
+}
+// accumulator dwords d[q] -> rows
+__device__ __forceinline__ uintx4 acc_to_rows(const unsigned (&d)[4]) {
+  unsigned a = d[0], b = d[2], c = d[1], e = d[3];
+  swap32(a, b);   // a' = [(q0,0) | (q2,0)], b' = [(q0,1) | (q2,1)]
+  swap32(c, e);   // c' = [(q1,0) | (q3,0)], e' = [(q1,1) | (q3,1)]
+  return uintx4{a, b, c, e};
+}
+
+constexpr int kStreamMaxLds = 64 * 1024 + 8 * 1024;
+
+template <int NKK, int NS, int NW>
+__global__ void __launch_bounds__(NW * 64, 2)
+igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
+  // NKK: 32-byte K steps per pixel row; NS: 32-channel slices (Kout / 32); NW: wavefronts
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, lg = lane >> 5;
+  const int M = p.N * p.Ho * p.Wo;
+  constexpr int KOUT = NS * 32;
+
+  uintx4* wl = reinterpret_cast<uintx4*>(smem);                              // [NS][NKK][64] fragments
+  int* bl = reinterpret_cast<int*>(smem + (size_t)NS * NKK * 1024);          // [Kout] bias
+  float* ml = reinterpret_cast<float*>(bl + KOUT);                           // [Kout] multipliers
+  {
+    const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag);
+    constexpr int per_slice = NKK * 64;
+    for (int u = tid; u < NS * per_slice; u += NW * 64) {
+      const int t = u / per_slice, rem = u - t * per_slice;
+      wl[u] = wf[(int64_t)t * p.wf_chunks * 64 + rem];
+    }
+    const int* bias = reinterpret_cast<const int*>(p.bias);
+    for (int c = tid; c < KOUT; c += NW * 64) {
+      bl[c] = bias != nullptr ? bias[c] : 0;
+      ml[c] = p.qmul[c];
+    }
+  }
+  __syncthreads();
+
+  const int8_t* x = reinterpret_cast<const int8_t*>(p.x);
+  int8_t* y = reinterpret_cast<int8_t*>(p.y);
+  const int8_t* res = reinterpret_cast<const int8_t*>(p.residual);
+  const bool has_res = res != nullptr;
+  const bool clamp = p.q_lo > 0.f;   // (a lower bound of 0 is what the saturating conversion applies anyway)
+  const int HoWo = p.Ho * p.Wo;
+  const bool plain = p.sh == 1 && p.sw == 1 && p.Ho == p.H && p.Wo == p.W;   // output pixel m reads input pixel m
+
+  // this lane's piece of the pixel operand of group g: bytes [32 kk + 16 lg, +16) of its pixel's row
+  auto load_b = [&](const int g, uintx4 (&b)[NKK]) {
+    int m = (g * NW + wave) * 32 + l32;
+    m = m < M ? m : M - 1;
+    int64_t xin = m;
+    if (!plain) {
+      const int n_img = fast_div(m, p.howo_magic, p.howo_shift);
+      const int rem = m - n_img * HoWo;
+      const int ho = fast_div(rem, p.wo_magic, p.wo_shift);
+      const int wo = rem - ho * p.Wo;
+      xin = ((int64_t)n_img * p.H + ho * p.sh) * p.W + wo * p.sw;
+    }
+    const uintx4* xrow = reinterpret_cast<const uintx4*>(x + xin * p.xcs) + lg;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) b[kk] = xrow[2 * kk];
+  };
+
+  uintx4 b[NKK], bnext[NKK];
+  if ((int)blockIdx.x < groups) load_b(blockIdx.x, b);
+  for (int g = blockIdx.x; g < groups; g += gridDim.x) {
+    const int m = (g * NW + wave) * 32 + l32;
+    const bool live = m < M;
+    const int mc = live ? m : M - 1;
+    int8_t* yrow = y + (int64_t)mc * p.ycs + lg * 16;
+    // the residual rows travel up to PRE slices ahead of their use: PRE KiB per wavefront in flight
+    constexpr int PRE = NS < 8 ? NS : 8;
+    uintx4 rr[NS];
+    const int8_t* rrow = has_res ? res + (int64_t)mc * p.rcs + lg * 16 : nullptr;
+    if (has_res) {
+#pragma unroll
+      for (int j = 0; j < PRE; ++j) rr[j] = *reinterpret_cast<const uintx4*>(rrow + j * 32);
+    }
+    // ... and so is the pixel operand of this wavefront's next tile
+    const int gn = g + (int)gridDim.x;
+    if (gn < groups) load_b(gn, bnext);
+
+#pragma unroll
+    for (int j = 0; j < NS; j += 2) {
+      // (unrolled for the static indices of rr[]; the scheduler must not pull the LDS reads of
+      //  every later pair up here, which would cost more registers than the chip has)
+      __builtin_amdgcn_sched_barrier(0);
+      if (has_res && j + PRE < NS) {
+        rr[j + PRE] = *reinterpret_cast<const uintx4*>(rrow + (j + PRE) * 32);
+        rr[j + PRE + 1] = *reinterpret_cast<const uintx4*>(rrow + (j + PRE + 1) * 32);
+      }
+      intx16 acc[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int* bj = bl + (j + h) * 32 + lg * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const intx4 bv = *reinterpret_cast<const intx4*>(bj + q * 8);
+          acc[h][q * 4 + 0] = bv.x; acc[h][q * 4 + 1] = bv.y; acc[h][q * 4 + 2] = bv.z; acc[h][q * 4 + 3] = bv.w;
+        }
+      }
+      const uintx4* wj = wl + (size_t)j * NKK * 64 + lane;
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        const uintx4 w0 = wj[kk * 64], w1 = wj[(NKK + kk) * 64];
+        acc[0] = Mma<int8_t>::run(w0, b[kk], acc[0]);
+        acc[1] = Mma<int8_t>::run(w1, b[kk], acc[1]);
+      }
+      auto finish = [&](auto with_res, auto with_clamp) __attribute__((always_inline)) {
+        constexpr bool kRes = decltype(with_res)::value;
+        constexpr bool kClamp = decltype(with_clamp)::value;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const float* mj = ml + (j + h) * 32 + lg * 4;
+          unsigned out[4], rd[4] = {0u, 0u, 0u, 0u};
+          if constexpr (kRes) rows_to_acc(rr[j + h], rd);
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            out[q] = requant4<kRes, kClamp>(acc[h][q * 4 + 0], acc[h][q * 4 + 1], acc[h][q * 4 + 2], acc[h][q * 4 + 3],
+                                            *reinterpret_cast<const floatx4*>(mj + q * 8), rd[q], p);
+          const uintx4 v = acc_to_rows(out);
+          // (plain stores: a row leaves in 32-byte pieces, which only the cache assembles into lines;
+          //  written around the cache such pieces cost several times the traffic)
+          if (live) *reinterpret_cast<uintx4*>(yrow + (j + h) * 32) = v;
+        }
+      };
+      // (wavefront-uniform choices)
+      if (has_res) { if (clamp) finish(std::true_type{}, std::true_type{}); else finish(std::true_type{}, std::false_type{}); }
+      else { if (clamp) finish(std::false_type{}, std::true_type{}); else finish(std::false_type{}, std::false_type{}); }
+    }
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) b[kk] = bnext[kk];
+  }
+}
+
+}  // namespace
+
+// Layers the streaming kernel serves: 8-bit 1x1 filters without padding, 8-bit
+// result, K = 64 .. 512 bytes per pixel, a multiple of 64 output channels, all
+// weights within 64 KiB, 16-byte aligned rows.
+bool igemm_stream_q8_geometry(const IgemmParams& p) {
+  if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid
+    if (strcmp(force, "stream") != 0 && force[0] != 0) return false;
+  }
+  if (const char* off = getenv("ODLA_HIP_STREAM_Q8")) {     // tuning aid: "0" turns the kernel off
+    if (off[0] == '0') return false;
+  }
+  if (p.in_dt != DT_I8 || p.out_dt != DT_I8) return false;
+  if (p.R != 1 || p.S != 1 || p.ph != 0 || p.pw != 0 || p.batch != 1) return false;
+  if (p.C != 64 && p.C != 128 && p.C != 256 && p.C != 512) return false;
+  if (p.xcs < p.C || p.xcs % 16 != 0) return false;
+  if (p.Kout % 64 != 0 || p.Kout < 64 || (int64_t)p.Kout * p.C > 64 * 1024) return false;
+  {  // the instantiations that exist (K bytes per pixel / output channels)
+    const int k = p.C, n = p.Kout;
+    const bool built = (k == 64 && (n == 64 || n == 256)) || (k == 128 && (n == 128 || n == 512)) ||
+                       (k == 256 && (n == 64 || n == 128 || n == 256)) || (k == 512 && n == 128);
+    if (!built) return false;
+    // Longer pixel rows are built (and parity-clean) but selected only on request
+    // (ODLA_HIP_STREAM_Q8=all): a lane's 16-byte piece of its pixel is then one of 8 - 32 pieces
+    // of the row, every load touches 32 cache lines, and the same layers are faster on the
+    // kernels that stage whole rows through LDS (ResNet-50 at batch 256: 256 -> 64 at 56 x 56
+    // 55 -> 64 us, 512 -> 128 at 28 x 28 33 -> 37 us).
+    if (k > 128) {
+      const char* sel = getenv("ODLA_HIP_STREAM_Q8");
+      if (sel == nullptr || strcmp(sel, "all") != 0) return false;
+    }
+  }
+  if ((int64_t)(p.Ho - 1) * p.sh >= p.H || (int64_t)(p.Wo - 1) * p.sw >= p.W) return false;
+  if (p.ycs % 16 != 0 || (p.residual != nullptr && p.rcs % 16 != 0)) return false;
+  if (p.y_rdiv > 0 || p.y_zdiv > 0) return false;
+  return true;
+}
+
+static bool stream_q8_ready(const IgemmParams& p) {
+  auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+  return igemm_stream_q8_geometry(p) && p.w_frag != nullptr && p.qmul != nullptr && p.wf_chunks >= p.C / 32 &&
+         al16(p.x) && al16(p.y) && al16(p.residual) && al16(p.w_frag);
+}
+
+hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream) {
+  if (!stream_q8_ready(p)) return hipErrorInvalidValue;
+  const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+  const int nkk = p.C / 32, ns = p.Kout / 32;
+  // wavefronts per workgroup as instantiated below (four where registers or LDS hold the
+  // compute unit to fewer wavefronts: more, smaller workgroups then fill it better)
+  const int nw = ((nkk == 4 && ns == 16) || (nkk == 8 && ns >= 4) || nkk == 16) ? 4 : 8;
+  const int64_t groups = (M + nw * 32 - 1) / (nw * 32);
+  const size_t lds = (size_t)ns * nkk * 1024 + (size_t)p.Kout * 8;
+  if (lds > (size_t)kStreamMaxLds || groups > 0x7fffffff) return hipErrorInvalidValue;
+  // resident workgroups walk the pixel groups with a grid stride
+  int per_cu = (int)((160 * 1024) / (lds + 512));
+  const int by_waves = 16 / nw;   // up to four wavefronts per SIMD
+  if (per_cu > by_waves) per_cu = by_waves;
+  if (per_cu < 1) per_cu = 1;
+  if (const char* e = getenv("ODLA_HIP_STREAM_WGS")) {  // tuning aid: workgroups per compute unit
+    const int v = atoi(e);
+    if (v >= 1 && v <= 8) per_cu = v;
+  }
+  int64_t grid = 256 * per_cu;
+  if (grid > groups) grid = groups;
+#define STREAM_CASE(NKK_, NS_, NW_)                                                                                 \
+  if (nkk == NKK_ && p.Kout == NS_ * 32) {                                                                          \
+    static bool attr_set = false;                                                                                   \
+    if (!attr_set) {                                                                                                \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_kernel<NKK_, NS_, NW_>),   \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, kStreamMaxLds);               \
+      if (e != hipSuccess) return e;                                                                                \
+      attr_set = true;                                                                                              \
+    }                                                                                                               \
+    hipLaunchKernelGGL((igemm_stream_q8_kernel<NKK_, NS_, NW_>), dim3((unsigned)grid), dim3(NW_ * 64), lds, stream, \
+                       p, (int)groups);                                                                             \
+    return hipGetLastError();                                                                                       \
+  }
+  STREAM_CASE(2, 2, 8)
+  STREAM_CASE(2, 8, 8)
+  STREAM_CASE(4, 4, 8)
+  STREAM_CASE(4, 16, 4)
+  STREAM_CASE(8, 2, 8)
+  STREAM_CASE(8, 4, 4)
+  STREAM_CASE(8, 8, 4)
+  STREAM_CASE(16, 4, 4)
+#undef STREAM_CASE
+  return hipErrorInvalidValue;
+}
+
+}  // namespace ohip

@@ -150,6 +150,12 @@ const char* igemm_variant_name(const IgemmParams& p);
 int igemm_big_variant(const IgemmParams& p);
 hipError_t launch_igemm_big(const IgemmParams& p, int epi_vec, int variant, hipStream_t stream);
 
+// Streaming kernel for 8-bit 1x1 filters over short pixel rows (igemm_stream.hip):
+// whether the layer's geometry qualifies (no pointer is looked at), and the launch
+// (p.w_frag, p.qmul and the division magics must be set; launch_igemm does that).
+bool igemm_stream_q8_geometry(const IgemmParams& p);
+hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream);
+
 // True when launch_igemm would use a fragment-ordered weight copy for this shape.
 bool igemm_wants_wfrag(const IgemmParams& p);
 // [batch][rows][row_bytes] packed weight rows -> fragment order: the 16-byte
