@@ -7,9 +7,12 @@
 Workloads: resnet50 (default: the configuration the headline metric is quoted
 on, "ResNet-50 int8 & fp16 at batch 256" - the int8 plan is timed first and is
 the top level of the line, the fp16 plan is timed next in the same process and
-nested under "fp16" with its own roofline block), resnet50_int8, resnet50_fp16,
-resnet50_bf16, resnet50_fp32, yolov3_fp16, bert_bf16, mnist_fp32,
-streaming_fp16.
+nested under "fp16" with its own roofline block; the other benchmark
+configurations follow, each nested under its name with its own value,
+ms_per_step and roofline: "bert_bf16" (performance mode, with the accuracy mode
+under "bert_bf16acc"), "yolov3_fp16", "mnist_fp32"; --headline-only leaves them
+out), resnet50_int8, resnet50_fp16, resnet50_bf16, resnet50_fp32, yolov3_fp16,
+bert_bf16, bert_bf16acc, mnist_fp32, streaming_fp16.
 
 A step is one odla_ExecuteComputation of the whole graph on one batch of
 synthetic input that is already resident in device memory (arguments and
@@ -17,7 +20,10 @@ outputs are bound to buffers from odla_AllocateDeviceMemory).  Prints ONE JSON
 line with the throughput, the roofline of the dominant kernel class (the
 implicit-GEMM convolution / GEMM launches, timed live with HIP events around
 un-captured launches on the library's own stream) and the CPU oracle timed on a
-bounded sample of the same workload.
+bounded sample of the same workload.  Beside that device-resident figure the
+line carries an "end_to_end" block: the same step with HOST buffers bound, so
+that the copies of the arguments to the device and of the results back are
+inside the timed region (what a caller of the reference's harness pays).
 """
 import argparse
 import ctypes
@@ -30,23 +36,26 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
-PEAK = {"fp16": 2500.0, "bf16": 2500.0, "int8": 5000.0, "fp32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
-DTYPE = {"fp16": "f16", "bf16": "bf16", "fp32": "f32", "int8": "i8"}
+PEAK = {"fp16": 2500.0, "bf16": 2500.0, "bf16acc": 2500.0, "int8": 5000.0, "fp32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
+DTYPE = {"fp16": "f16", "bf16": "bf16", "bf16acc": "bf16", "fp32": "f32", "int8": "i8"}
 METRIC = "images/sec at batch 256, ResNet-50 int8 & fp16; % MFMA peak / % HBM BW"
 
 
-# HBM bytes per conv/gemm launch (average over the launches of one step) read
-# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by
-# what the same counters read for a plain elementwise kernel of known size (the
-# ReLU launch of --workload streaming_fp16: 411 MB in, 411 MB out); the
-# summaries the figures come from are the traffic_* files under profiles/.
-# null = not measured.
-MEASURED_TRAFFIC = {
-    # 8.79 GB fetched + 5.76 GB written per step over its 54 conv/gemm launches
-    "resnet50_fp16": 269.4e6,
-    # 4.16 GB fetched + 2.97 GB written per step over its 54 conv/gemm launches
-    "resnet50_int8": 132.0e6,
-}
+def measured_traffic(name):
+    """HBM bytes per conv/gemm launch (average over the launches of one step) from the
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries: the table rows
+    `| workload | bytes per launch | ...` of profiles/traffic_per_launch.md.  None when
+    the workload has no row (not measured)."""
+    path = os.path.join(ROOT, "profiles", "traffic_per_launch.md")
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 2 and cells[0] == name:
+                    return float(cells[1])
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 class Workload:
@@ -113,7 +122,8 @@ def make_workload(name, batch, pkg):
             mb.build_bert(rb, w, n, seq)
         return Workload(name, "sequences/s", batch, mb.bert_gflop_per_sequence(seq) * 1e9 * batch,
                         "BERT-base encoder %s, batch %d x seq %d, 12 layers, hidden 768, 12 heads, FFN 3072"
-                        % (mode, batch, seq),
+                        % ({"bf16": "bf16 (BF16_PERFORMACE_MODE: every tensor bf16)",
+                            "bf16acc": "bf16 (BF16_ACCURACY_MODE: fp32 tensors, bf16 Gemm operands)"}.get(mode, mode), batch, seq),
                         lambda b: mb.build_bert(b, w, batch, seq), feeds, ref_run, mode)
     if family == "mnist":
         batch = batch or 64
@@ -177,6 +187,10 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=-1,
                     help="units (images / sequences) timed on the CPU oracle; 0 = skip, -1 = per-workload default")
     ap.add_argument("--dump-steps", default=None, help="write the per-launch timing table to this file")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="default workload: time the ResNet-50 int8 / fp16 plans only, not the other configurations")
+    ap.add_argument("--e2e-steps", type=int, default=5,
+                    help="executions timed with host buffers bound (the end_to_end block); 0 = skip")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this build has a single MI355X and the path "
@@ -191,8 +205,13 @@ def main():
     if args.workload == "resnet50":
         # the headline metric names both precisions: int8 (the optimisation target) on top, fp16 nested
         line = run_workload(pkg, L, "resnet50_int8", args, with_cpu=True)
+        nested = ("value", "unit", "ms_per_step", "dtype", "config", "roofline", "end_to_end")
         fp16 = run_workload(pkg, L, "resnet50_fp16", args, with_cpu=False)
-        line["fp16"] = {k: fp16[k] for k in ("value", "unit", "ms_per_step", "dtype", "config", "roofline")}
+        line["fp16"] = {k: fp16[k] for k in nested}
+        if not args.headline_only:
+            for name in ("bert_bf16", "bert_bf16acc", "yolov3_fp16", "mnist_fp32"):
+                sub = run_workload(pkg, L, name, args, with_cpu=False)
+                line[name] = {k: sub[k] for k in nested}
     else:
         line = run_workload(pkg, L, args.workload, args, with_cpu=True)
     print(json.dumps(line))
@@ -205,7 +224,8 @@ def run_workload(pkg, L, name, args, with_cpu):
     wl = make_workload(name, args.batch, pkg)
     mode = wl.mode
 
-    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16=(mode == "bf16"), quant_table=wl.table)
+    hb = odla.HipBuilder(fp16=(mode == "fp16"), bf16={"bf16": "performance", "bf16acc": "accuracy"}.get(mode, False),
+                         quant_table=wl.table)
     wl.build(hb)
     sess = hb.session(use_graph=True)
     sess.bind_device_io(wl.feeds)
@@ -220,6 +240,8 @@ def run_workload(pkg, L, name, args, with_cpu):
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     per_s = wl.batch / (ms_per_step * 1e-3)
+
+    e2e = end_to_end(hb, wl, args.e2e_steps) if args.e2e_steps > 0 else None
 
     dump = args.dump_steps
     if dump and args.workload == "resnet50":   # two plans in one run: one table each
@@ -240,11 +262,33 @@ def run_workload(pkg, L, name, args, with_cpu):
         "scaling": "weak", "vs_baseline": None, "dtype": DTYPE[mode], "data": "synthetic",
         "config": {"workload": wl.desc, "batch": wl.batch,
                    "executor": "hipGraph replay through odla_ExecuteComputation"},
-        "roofline": roof, "cpu_baseline": cpu,
+        "roofline": roof, "cpu_baseline": cpu, "end_to_end": e2e,
     }
     sess.close()
     hb.destroy()
     return line
+
+
+def end_to_end(hb, wl, steps):
+    """The same step with HOST buffers bound: odla_ExecuteComputation copies the arguments to the
+    device, runs the graph and copies the results back before it returns
+    [ref: python/halo/odla.py:172-175 times exactly that call].  Timed twice: with ordinary
+    (pageable) numpy arrays, as the reference harness passes them, and with page-locked buffers
+    from odla_AllocateHostMemory."""
+    out = {"steps": steps, "unit": wl.unit,
+           "host_bytes_per_step": int(sum(v.nbytes for v in wl.feeds.values()))}
+    for kind, pinned in (("pageable", False), ("pinned", True)):
+        sess = hb.session(use_graph=True)
+        outs = sess.bind_host_io(wl.feeds, pinned=pinned)
+        out["host_bytes_per_step"] = int(sum(v.nbytes for v in wl.feeds.values()) + sum(o.nbytes for o in outs.values()))
+        sess.execute()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            sess.execute()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out[kind] = {"value": round(wl.batch / (ms * 1e-3), 1), "ms_per_step": round(ms, 4)}
+        sess.close()
+    return out
 
 
 class StepTime(ctypes.Structure):
@@ -349,7 +393,7 @@ def profile_roofline(L, sess, wl, dump_path=None):
     peak = PEAK[wl.mode]
     roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
             "unit": "TOP/s" if wl.mode == "int8" else "TFLOP/s",
-            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(wl.name),
+            "frac": round(achieved / peak, 4), "traffic": measured_traffic(wl.name),
             "kernel": "igemm_wreg_kernel / igemm_kernel / igemm_lean_kernel / igemm_taps_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
                       "avg %.2f GFLOP per launch)" % (launches, 1e3 * mm_ms / max(launches, 1),
                                                      wl.flop / 1e9 / max(launches, 1)),
@@ -359,7 +403,7 @@ def profile_roofline(L, sess, wl, dump_path=None):
         # The same launches priced against both rooflines: per launch the bound is
         # max(FLOPs / MFMA peak, algorithmic bytes / 8 TB/s); most 1x1 layers of
         # this network at batch 256 sit on the HBM side.
-        es = {"fp32": 4, "fp16": 2, "bf16": 2, "int8": 1}[wl.mode]
+        es = {"fp32": 4, "fp16": 2, "bf16": 2, "bf16acc": 2, "int8": 1}[wl.mode]
         t_by = {}
         for i in range(n.value):
             name = buf[i].name.decode()

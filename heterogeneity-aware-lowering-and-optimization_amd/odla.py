@@ -720,6 +720,38 @@ class Session:
             self.dev_out[name] = (p, shape, dt)
             _check(self.L.odla_BindToOutput(h, p, self.ctx), "odla_BindToOutput")
 
+    def bind_host_io(self, feeds, pinned=False):
+        """Bind HOST buffers for every argument and output, so that execute() copies the
+        arguments to the device and the results back, as a caller of the reference's
+        harness pays it (python/halo/odla.py:172-175 times odla_ExecuteComputation on host
+        arrays).  pinned=False: ordinary (pageable) numpy arrays; True: page-locked
+        buffers from odla_AllocateHostMemory.  Returns name -> numpy view of each output."""
+        self._host_keep = []
+        self._host_pinned = getattr(self, "_host_pinned", [])
+
+        def buffer(nbytes, dt, shape):
+            if not pinned:
+                return np.empty(shape, dt)
+            p = ctypes.c_void_p()
+            _check(self.L.odla_AllocateHostMemory(ctypes.byref(p), max(nbytes, 1)), "odla_AllocateHostMemory")
+            self._host_pinned.append(p)
+            raw = (ctypes.c_uint8 * max(nbytes, 1)).from_address(p.value)
+            return np.frombuffer(raw, dtype=dt, count=int(np.prod(shape))).reshape(shape)
+
+        for name, (h, shape, dt) in self.b.args.items():
+            src = np.ascontiguousarray(feeds[name], dtype=dt)
+            a = buffer(src.nbytes, dt, src.shape)
+            a[...] = src
+            self._host_keep.append(a)
+            _check(self.L.odla_BindToArgument(h, a.ctypes.data_as(ctypes.c_void_p), self.ctx), "odla_BindToArgument")
+        outs = {}
+        for name, (h, shape, dt) in self.b.outs.items():
+            o = buffer(int(np.prod(shape)) * dt.itemsize, dt, tuple(shape))
+            outs[name] = o
+            self._host_keep.append(o)
+            _check(self.L.odla_BindToOutput(h, o.ctypes.data_as(ctypes.c_void_p), self.ctx), "odla_BindToOutput")
+        return outs
+
     def execute(self):
         _check(self.L.odla_ExecuteComputation(self.b.comp, self.ctx, ODLA_COMPUTE_INFERENCE, None), "odla_ExecuteComputation")
 
@@ -740,6 +772,10 @@ class Session:
         for p in self._dev:
             self.L.odla_FreeDeviceMemory(p)
         self._dev = []
+        for p in getattr(self, "_host_pinned", []):
+            self.L.odla_FreeHostMemory(p)
+        self._host_pinned = []
+        self._host_keep = []
         if self.ctx:
             self.L.odla_DestroyContext(self.ctx)
             self.ctx = None
