@@ -176,12 +176,16 @@ class Planner {
   };
   Ref ref(int t) const { return Ref{plan_, t}; }
 
+  // exact_reader: the launch reads exactly the elements of its sources and tests their alignment
+  // itself (the layout conversions launch_nchw_to_nhwc / launch_nchw_to_s2d do), so a source that
+  // is an argument's staging tensor may be the caller's own device buffer.  Every other reader
+  // may rely on the arena (256-byte bases, slack behind a tensor) and pins its sources to it.
   void emit(const std::string& name, std::initializer_list<int> reads, std::initializer_list<int> writes,
-            std::function<hipError_t(const ExecEnv&, hipStream_t)> fn) {
-    emit_lists(name, std::vector<int>(reads), std::vector<int>(writes), std::move(fn));
+            std::function<hipError_t(const ExecEnv&, hipStream_t)> fn, bool exact_reader = false) {
+    emit_lists(name, std::vector<int>(reads), std::vector<int>(writes), std::move(fn), exact_reader);
   }
   void emit_lists(const std::string& name, const std::vector<int>& reads, const std::vector<int>& writes,
-                  std::function<hipError_t(const ExecEnv&, hipStream_t)> fn) {
+                  std::function<hipError_t(const ExecEnv&, hipStream_t)> fn, bool exact_reader = false) {
     if (in_init_) {
       plan_->init_steps.push_back({name, std::move(fn)});
       return;
@@ -196,9 +200,6 @@ class Planner {
     };
     for (int t : reads) touch(t);
     for (int t : writes) touch(t);
-    // Layout conversions read exactly the elements of their source and test its alignment
-    // at launch; any other reader may rely on the arena (256-byte bases, slack behind a tensor).
-    const bool exact_reader = name.compare(0, 8, "to_nhwc:") == 0 || name.compare(0, 7, "to_s2d:") == 0;
     for (int t : reads) if (t >= 0 && !exact_reader) arena_only_.insert(root(t));
     for (int t : writes) if (t >= 0) arena_only_.insert(root(t));
     plan_->steps.push_back({name, std::move(fn)});
@@ -421,7 +422,7 @@ class Planner {
         emit("to_nhwc:" + v->name, {from}, {dst}, [=](const ExecEnv& e, hipStream_t st) {
           LayoutParams p = lp; p.src = a(e); p.dst = b(e);
           return launch_nchw_to_nhwc(p, st);
-        });
+        }, /*exact_reader=*/true);
         return dst;
       } else {
         lp.cs = s2.cs;
@@ -1305,7 +1306,7 @@ void Planner::lower_conv(int ni) {
       emit("to_s2d:" + x->name, {from}, {tx_s2d}, [=](const ExecEnv& e, hipStream_t st) {
         S2dParams p = sp; p.src = a(e); p.dst = b(e);
         return launch_nchw_to_s2d(p, st);
-      });
+      }, /*exact_reader=*/true);
       C = C2; Cg = C2; H = H2; W = W2; R = R2; S = S2;
       str_h = str_w = 1;
       pad_t = -dy0; pad_l = -dx0;
@@ -1364,6 +1365,10 @@ void Planner::lower_conv(int ni) {
     const QuantEntry* qf = qentry(outv);
     std::vector<float> mul((size_t)O);
     int ty;
+    if (qf != nullptr && ep.pre_residual_value != nullptr && ep.pre_residual_value != outv &&
+        qentry(ep.pre_residual_value) != nullptr)
+      OHIP_INFO("int8 plan: the quant-table entry of '%s' is not used - the residual Add behind it is fused and the "
+                "convolution requantises once, to the entry of '%s'", ep.pre_residual_value->name.c_str(), outv->name.c_str());
     if (qf != nullptr) {
       // One requantisation per convolution, whatever is fused behind it: the result
       // (after the residual add and the ReLU, if any) takes the scale and zero point

@@ -196,7 +196,10 @@ odla_status validate_loaded(const _odla_computation* c) {
     for (int i = 0; i < nin; ++i) {
       const _odla_value* v = n.in[(size_t)i];
       if (v == nullptr) {
-        LOADED_REQUIRE(i >= 32 || !((r.required >> i) & 1u), "%s node %lld lacks operand %d", name, (long long)k, i);
+        // (an operator that requires every slot says so with all bits set: that covers slots
+        //  beyond the 32 the mask has a bit for - a Concat may have up to ODLA_MAX_OUTPUTS)
+        const bool must = r.required == ~0u || (i < 32 && ((r.required >> i) & 1u));
+        LOADED_REQUIRE(!must, "%s node %lld lacks operand %d", name, (long long)k, i);
         continue;
       }
       // operands are defined before their use

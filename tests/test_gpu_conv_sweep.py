@@ -128,8 +128,10 @@ def test_random_convolutions_int8():
     odla = entry.load().odla
     models = entry.load().models
     ref = entry.load_oracle()
-    done = 0
-    for i, c in enumerate(cases(SEED0 + 777, 140)):
+    done, wanted = 0, 30
+    for i, c in enumerate(cases(SEED0 + 777, 1000)):
+        if done == wanted:
+            break
         if c["group"] != 1 or c["dh"] != 1 or c["dw"] != 1:
             continue        # the 8-bit plan covers dense, undilated convolutions; the rest stays in float
         if c["pad"][0] != c["pad"][2] or c["pad"][1] != c["pad"][3] or c["kh"] != c["kw"] or c["sh"] != c["sw"]:
@@ -157,4 +159,5 @@ def test_random_convolutions_int8():
         want = ref.dequantize_act(q_want, *y_qp)
         assert np.array_equal(got, want), (i, c)
         done += 1
-    assert done >= 20   # (the share of eligible shapes varies with the seed)
+    announce("sweep int8: %d eligible shapes ran (seed %d)" % (done, SEED0 + 777))
+    assert done == wanted   # shapes are drawn until that many eligible ones have run

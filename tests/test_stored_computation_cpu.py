@@ -226,3 +226,33 @@ def test_well_hashed_files_with_malformed_records_are_refused(odla, tmp_path):
     # an operand count that no longer matches the bytes that follow
     assert load(st.patched(conv["nin_at"], 2)) == odla.ODLA_INVALID_PARAM
     assert load(st.patched(tr["niv_at"], 1)) == odla.ODLA_INVALID_PARAM
+
+
+def test_concat_with_a_missing_operand_beyond_slot_32_is_refused(odla, tmp_path):
+    """A Concat may have up to 64 operands; every slot is required, also those beyond the 32
+    the per-operator mask has a bit for (a well-hashed file with slot 32 empty used to pass
+    validation and crash in the shape checks)."""
+    L = odla.load_library()
+    hb = odla.HipBuilder()
+    x = hb.arg("x", (1, 2, 4))
+    parts = [hb.relu(x, name="r%d" % i) for i in range(33)]
+    hb.output(hb.concat(parts, 1, name="cat"), "cat")
+    p = str(tmp_path / "cat.odla")
+    loc, keep = odla.path_location(p)
+    assert L.odla_StoreComputation(loc, hb.comp) == 0
+    hb.destroy()
+    st = _Stored(open(p, "rb").read())
+    OP_CONCAT = 10
+    cat = st.node(OP_CONCAT)
+
+    def load(data):
+        comp = ctypes.c_void_p()
+        mloc, mk = odla.memory_location(data)
+        rc = L.odla_LoadComputation(mloc, ctypes.byref(comp))
+        if rc == 0:
+            L.odla_DestroyComputation(comp)
+        return rc
+
+    assert load(st.patched(8, 1)) == 0
+    assert load(st.patched(cat["in_at"] + 8 * 32, -1)) == odla.ODLA_INVALID_PARAM
+    assert load(st.patched(cat["in_at"] + 8 * 5, -1)) == odla.ODLA_INVALID_PARAM
