@@ -190,6 +190,31 @@ struct PackWeightsParams {
 hipError_t launch_pack_weights(const PackWeightsParams& p, hipStream_t stream);
 
 // ---------------------------------------------------------------------------
+// One-launch attention (attention.hip):
+//   out[b, h] = softmax(scale * q[b, h] . k[b, h]^T + mask[b]) . v[b, h]
+// q, k, v: [S][d] matrices of 16-bit elements per (batch, head), rows of d = 64
+// contiguous values; S = 32, 64, 96 or 128.  mask: one row of S values per batch
+// (added to every query's scores), of the operands' type or fp32, or null.
+// All strides in elements.
+struct AttentionParams {
+  const void* q = nullptr; const void* k = nullptr; const void* v = nullptr;
+  void* out = nullptr;
+  const void* mask = nullptr;
+  DType dt = DT_BF16;        // q, k, v, out
+  DType mask_dt = DT_BF16;
+  int B = 0, heads = 0, S = 0, d = 0;
+  float scale = 1.f;
+  int64_t q_bs = 0, q_hs = 0, q_rs = 0;   // batch / head / row strides
+  int64_t k_bs = 0, k_hs = 0, k_rs = 0;
+  int64_t v_bs = 0, v_hs = 0, v_rs = 0;
+  int64_t o_bs = 0, o_hs = 0, o_rs = 0;
+  int64_t mask_bs = 0;                    // between batches (0: one row for all)
+};
+// Shapes / types the kernel serves (no pointer is looked at).
+bool attention_supported(const AttentionParams& p);
+hipError_t launch_attention(const AttentionParams& p, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
 // Layout conversion between row-major N,C,HW (any float type) and
 // channels-last N,HW,cs with optional channel padding (pad lanes get `fill`).
 struct LayoutParams {

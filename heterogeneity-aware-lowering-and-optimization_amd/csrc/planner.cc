@@ -554,6 +554,7 @@ class Planner {
   bool fuse_slice_seed(int ni) const;
   bool fuse_candidate(int ni) const;
   bool gemm_epilogue(int ni, Epilogue* ep);
+  bool try_fused_attention(int ni);
   std::unordered_map<int, Epilogue> gemm_ep_ahead_;  // epilogues collected while looking for sibling GEMMs
   std::vector<char> gemm_merged_;                    // nodes already lowered inside a sibling's launch
   std::vector<char> no_fuse_;                        // nodes of an element-wise group that was given up
@@ -1553,8 +1554,125 @@ int Planner::head_merge_behind(const _odla_value* v) const {
   return ti;
 }
 
+// q . k^T -> [scalar Mul / Div] -> [+ mask] -> Softmax -> . v (-> head merge): the attention block
+// of an encoder layer as ONE launch [ref: the reference's compiler matches the same block,
+// lib/transforms/fusion.cc:315-348].  `ni` is the q . k^T product; on success every node of the
+// block is marked as done and the block's result exists.
+bool Planner::try_fused_attention(int ni) {
+  if (calib_ || comp_->opts.int8) return false;
+  Node& n = comp_->nodes[ni];
+  const _odla_value* Q = n.in[0];
+  const _odla_value* K = n.in[1];
+  if (Q == nullptr || K == nullptr || (n.in.size() > 2 && n.in[2] != nullptr)) return false;
+  if (n.i[0] != 0 || n.i[1] == 0) return false;   // q . k^T
+  const Shape& qs = Q->shape;
+  if (qs.rank != 4 || !(K->shape == qs) || Q->kind == _odla_value::CONSTANT || K->kind == _odla_value::CONSTANT) return false;
+  const int64_t B = qs.d[0], heads = qs.d[1], S = qs.d[2], d = qs.d[3];
+  const DType dt = mm_dtype(Q);
+  if (mm_dtype(K) != dt || !available(Q) || !available(K)) return false;
+  auto sole_reader = [&](const _odla_value* v) -> int {
+    if (v->is_output || consumers_[v->index].size() != 1) return -1;
+    const int c = consumers_[v->index][0];
+    return comp_->nodes[c].absorbed ? -1 : c;
+  };
+  std::vector<int> block;   // nodes behind `ni` that the launch covers
+  float scale = n.f[0];
+  const _odla_value* cur = n.out;
+  int ci = sole_reader(cur);
+  if (ci < 0) return false;
+  // a scalar factor (scores / sqrt(d))
+  if (comp_->nodes[ci].op == OP_BINARY && (comp_->nodes[ci].i[0] == BIN_MUL || comp_->nodes[ci].i[0] == BIN_DIV)) {
+    const Node& m = comp_->nodes[ci];
+    const bool lhs = m.in[0] == cur;
+    const _odla_value* other = lhs ? m.in[1] : m.in[0];
+    if (other == cur || other->kind != _odla_value::CONSTANT || other->shape.numel() != 1 || !(m.out->shape == cur->shape)) return false;
+    const float c = const_as_float(other)[0];
+    if (m.i[0] == BIN_DIV) {
+      if (!lhs || c == 0.f) return false;
+      scale *= 1.0f / c;
+    } else {
+      scale *= c;
+    }
+    block.push_back(ci);
+    cur = m.out;
+    if ((ci = sole_reader(cur)) < 0) return false;
+  }
+  // an additive mask: one row of S values per batch entry (or one for all)
+  const _odla_value* mask = nullptr;
+  int64_t mask_bs = 0;
+  if (comp_->nodes[ci].op == OP_BINARY && comp_->nodes[ci].i[0] == BIN_ADD) {
+    const Node& a = comp_->nodes[ci];
+    const bool lhs = a.in[0] == cur;
+    const _odla_value* other = lhs ? a.in[1] : a.in[0];
+    const int r = (int)a.iv[0];
+    if (other == cur || r != 4 || !(a.out->shape == cur->shape) || !available(other)) return false;
+    int64_t al[4];
+    for (int i = 0; i < 4; ++i) al[i] = a.iv[1 + (lhs ? r : 0) + i];
+    if ((al[0] != B && al[0] != 1) || al[1] != 1 || al[2] != 1 || al[3] != S) return false;
+    const DType mdt = storage_dtype(other);
+    if (mdt != dt && mdt != DT_F32) return false;
+    mask = other;
+    mask_bs = al[0] == 1 ? 0 : S;
+    block.push_back(ci);
+    cur = a.out;
+    if ((ci = sole_reader(cur)) < 0) return false;
+  }
+  {
+    const Node& sm = comp_->nodes[ci];
+    if (sm.op != OP_SOFTMAX || (int)sm.i[0] != 3 || sm.i[1] != 0) return false;
+    block.push_back(ci);
+    cur = sm.out;
+    if ((ci = sole_reader(cur)) < 0) return false;
+  }
+  const Node& g2 = comp_->nodes[ci];
+  if (g2.op != OP_GEMM || g2.in[0] != cur || g2.i[0] != 0 || g2.i[1] != 0 || g2.f[0] != 1.f ||
+      (g2.in.size() > 2 && g2.in[2] != nullptr))
+    return false;
+  const _odla_value* V = g2.in[1];
+  if (V == nullptr || !(V->shape == qs) || V->kind == _odla_value::CONSTANT || mm_dtype(V) != dt || !available(V)) return false;
+  if (gemm_ep_ahead_.count(ci) || (ci < (int)gemm_merged_.size() && gemm_merged_[ci])) return false;
+  block.push_back(ci);
+  _odla_value* fv = g2.out;
+  const int ti = head_merge_behind(fv);   // [B, heads, S, d] -> [B, S, heads, d] behind it: stored that way
+  if (ti >= 0) fv = comp_->nodes[ti].out;
+  if (result_dtype(fv) != dt) return false;
+
+  AttentionParams ap;
+  ap.dt = dt;
+  ap.mask_dt = mask != nullptr ? storage_dtype(mask) : dt;
+  ap.B = (int)B; ap.heads = (int)heads; ap.S = (int)S; ap.d = (int)d;
+  ap.scale = scale;
+  ap.q_bs = ap.k_bs = ap.v_bs = heads * S * d;
+  ap.q_hs = ap.k_hs = ap.v_hs = S * d;
+  ap.q_rs = ap.k_rs = ap.v_rs = d;
+  if (ti >= 0) { ap.o_bs = S * heads * d; ap.o_hs = d; ap.o_rs = heads * d; }
+  else { ap.o_bs = heads * S * d; ap.o_hs = S * d; ap.o_rs = d; }
+  ap.mask_bs = mask_bs;
+  if (B * heads > 0x7fffffff || !attention_supported(ap)) return false;
+
+  // ---- from here on the plan changes
+  const int tq = get(Q, L_ROWMAJOR, FORM_OPERAND), tk = get(K, L_ROWMAJOR, FORM_OPERAND), tv = get(V, L_ROWMAJOR, FORM_OPERAND);
+  const int tm = mask != nullptr ? get(mask, L_ROWMAJOR, FORM_FLOAT) : -1;
+  if (T(tq).dt != dt || T(tk).dt != dt || T(tv).dt != dt || (tm >= 0 && T(tm).dt != ap.mask_dt))
+    fail(ODLA_INTERNAL_LOGIC_ERR, "attention operand storage type mismatch ('%s')", fv->name.c_str());
+  const int ty = new_tensor(dt, L_ROWMAJOR, fv->shape, 0, SP_ARENA);
+  const Ref rq = ref(tq), rk = ref(tk), rv = ref(tv), ry = ref(ty), rm = ref(tm >= 0 ? tm : tq);
+  const bool hm = tm >= 0;
+  emit("attention:" + fv->name, {tq, tk, tv, tm}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+    AttentionParams p = ap;
+    p.q = rq(e); p.k = rk(e); p.v = rv(e); p.out = ry(e);
+    p.mask = hm ? rm(e) : nullptr;
+    return launch_attention(p, st);
+  });
+  for (int j : block) comp_->nodes[j].absorbed = true;
+  if (ti >= 0) comp_->nodes[ti].absorbed = true;
+  set_main(fv, ty);
+  return true;
+}
+
 void Planner::lower_gemm(int ni) {
   if (ni < (int)gemm_merged_.size() && gemm_merged_[ni]) return;  // computed by an earlier sibling's launch
+  if (try_fused_attention(ni)) return;
   Node& n = comp_->nodes[ni];
   const _odla_value* A = n.in[0];
   const _odla_value* B = n.in[1];

@@ -510,7 +510,9 @@ class RefBuilder:
           a per-channel constant Add / Sub / Mul / Div, one same-shape residual
           Add and one activation behind it (an Add behind the activation too),
           an Add whose only reader is a Softmax, a Softmax that is a graph
-          output.  Parameters that stay fp32 on the device (Conv / Gemm bias,
+          output; the scores of an attention block with head size 64 and at most
+          128 keys (q . k^T, scale and mask stay fp32 up to the Softmax, whose
+          probabilities are stored).  Parameters that stay fp32 on the device (Conv / Gemm bias,
           LayerNorm and BatchNorm parameters) are not rounded.
     """
 
@@ -638,7 +640,11 @@ class RefBuilder:
                 stage = "res"
             y = y + float(beta) * _f32(c).astype(np.float64)
         y = y.astype(np.float32)
-        return self._name(name, self._mark_open(y, (stage, y.ndim - 1)))
+        # q . k^T of an attention block that a 16-bit plan runs as one launch (head size 64, up to
+        # 128 keys in blocks of 32): the scores then never leave the launch, see _bin
+        attn = (y.ndim == 4 and tb and not ta and c is None and a.shape[-1] == 64 and y.shape[-1] == y.shape[-2]
+                and y.shape[-1] % 32 == 0 and y.shape[-1] <= 128)
+        return self._name(name, self._mark_open(y, (stage, y.ndim - 1, attn)))
 
     def batch_matmul(self, a, b, ta=False, tb=False, name=None):
         """op(A) op(B) over matching leading batch dims [ref: ops/odla_ops_math.h:337-339;
@@ -670,16 +676,22 @@ class RefBuilder:
             st = self._stage(cur)
             if st is None or st[0] not in ("acc", "act") or tuple(c_al.shape) != tuple(out_shape):
                 continue
-            stage, ch = st
+            stage, ch = st[0], st[1]
+            attn = len(st) > 2 and st[2]
             is_const = id(other) in self._consts
             per_channel = o_al.size == 1 or (o_al.size == out_shape[ch] and o_al.shape[ch] == o_al.size)
             res = None
             if stage == "acc" and is_const and per_channel and (
                     f is np.add or f is np.multiply or (f is np.subtract and lhs) or (f is np.divide and lhs and o_al.size == 1)):
-                res, nxt = (f(c_al, o_al.astype(np.float32)) if lhs else f(o_al.astype(np.float32), c_al)), ("acc", ch)
+                res, nxt = (f(c_al, o_al.astype(np.float32)) if lhs else f(o_al.astype(np.float32), c_al)), ("acc", ch, attn)
             elif f is np.add and not is_const and tuple(o_al.shape) == tuple(out_shape):
                 o_cl = self._closed(other).reshape(o_al.shape)
                 res, nxt = c_al + o_cl, (("res", ch) if stage == "acc" else ("done", ch))
+            elif (f is np.add and not is_const and attn and stage == "acc" and o_al.ndim == 4
+                  and o_al.shape[1] == 1 and o_al.shape[2] == 1 and o_al.shape[3] == out_shape[3]):
+                # the mask of an attention block: added to fp32 scores inside the one launch
+                o_cl = self._closed(other).reshape(o_al.shape)
+                res, nxt = (c_al + o_cl).astype(np.float32), ("bin", ch)
             if res is not None:
                 self._open.pop(id(cur), None)
                 return self._name(name, self._mark_open(res.astype(np.float32), nxt))
@@ -775,8 +787,9 @@ class RefBuilder:
     def softmax(self, x, axis=-1, log=False, name=None):
         """[ref: odla_dnnl.cc:1628-1669]; every negative axis means the last one."""
         st = self._stage(x)
-        if st is not None and st[0] == "bin" and axis in (-1, np.ndim(x) - 1):
-            self._open.pop(id(x))    # the Add in front ran inside this launch
+        last = axis in (-1, np.ndim(x) - 1)
+        if st is not None and last and (st[0] == "bin" or (st[0] == "acc" and len(st) > 2 and st[2])):
+            self._open.pop(id(x))    # the Add in front ran inside this launch / the scores of an attention block
         else:
             x = self._closed(x)
         x64 = _f32(x).astype(np.float64)

@@ -118,6 +118,31 @@ def test_stored_emulation_attention_rules(ref):
     assert not np.array_equal(_rs(ref, sm0, st), sm0)
 
 
+def test_stored_emulation_attention_block_keeps_scores_fp32(ref):
+    """Head size 64 and a multiple of 32 keys (at most 128): the block is one launch in a 16-bit
+    plan, so scale, mask and Softmax see fp32 scores; the probabilities are stored."""
+    st = "bf16"
+    rng = np.random.default_rng(10)
+    q = rng.standard_normal((2, 2, 32, 64)).astype(np.float32)
+    k = rng.standard_normal((2, 2, 32, 64)).astype(np.float32)
+    v = rng.standard_normal((2, 2, 32, 64)).astype(np.float32)
+    mask = np.where(rng.random((2, 1, 1, 32)) < 0.3, -10000.0, 0.0).astype(np.float32)
+    rb = ref.RefBuilder({"q": q, "k": k, "v": v, "m": mask}, emulate="stored", storage=st)
+    qv, kv, vv, mv = (rb.arg(n, a.shape) for n, a in (("q", q), ("k", k), ("v", v), ("m", mask)))
+    s = rb.div(rb.gemm(qv, kv, None, False, True, 1.0, 0.0), rb.const("scale", np.full((1,), 8.0, np.float32)))
+    ctx = rb.gemm(rb.softmax(rb.add(s, mv), -1), vv, None, False, False, 1.0, 0.0)
+    rb.output(ctx, "ctx")
+    qr, kr, vr, mr = (_rs(ref, a, st) for a in (q, k, v, mask))
+    s0 = (qr.astype(np.float64) @ np.swapaxes(kr, -1, -2).astype(np.float64)).astype(np.float32) / np.float32(8.0)
+    plain = ref.RefBuilder({})
+    p0 = _rs(ref, plain.softmax(s0 + mr, -1), st)
+    ctx0 = _rs(ref, (p0.astype(np.float64) @ vr.astype(np.float64)).astype(np.float32), st)
+    assert np.array_equal(rb.outputs["ctx"], ctx0)
+    # with stored (rounded) scores the result differs: the rule matters
+    p1 = _rs(ref, plain.softmax(_rs(ref, s0, st) + mr, -1), st)
+    assert not np.array_equal(p1, p0)
+
+
 def test_stored_emulation_keeps_normalisation_parameters_fp32(ref):
     st = "bf16"
     rng = np.random.default_rng(11)
