@@ -69,7 +69,8 @@ igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
   const int wave = tid >> 6, lane = tid & 63;
   const int l32 = lane & 31, lg = lane >> 5;
   const int M = p.N * p.Ho * p.Wo;
-  constexpr int KOUT = NS * 32;
+  constexpr int KOUT = NS * 32;            // channels of this workgroup: [n0, n0 + KOUT)
+  const int n0 = blockIdx.y * KOUT;
 
   uintx4* wl = reinterpret_cast<uintx4*>(smem);                              // [NS][NKK][64] fragments
   int* bl = reinterpret_cast<int*>(smem + (size_t)NS * NKK * 1024);          // [Kout] bias
@@ -79,12 +80,12 @@ igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
     constexpr int per_slice = NKK * 64;
     for (int u = tid; u < NS * per_slice; u += NW * 64) {
       const int t = u / per_slice, rem = u - t * per_slice;
-      wl[u] = wf[(int64_t)t * p.wf_chunks * 64 + rem];
+      wl[u] = wf[(int64_t)(n0 / 32 + t) * p.wf_chunks * 64 + rem];
     }
     const int* bias = reinterpret_cast<const int*>(p.bias);
     for (int c = tid; c < KOUT; c += NW * 64) {
-      bl[c] = bias != nullptr ? bias[c] : 0;
-      ml[c] = p.qmul[c];
+      bl[c] = bias != nullptr ? bias[n0 + c] : 0;
+      ml[c] = p.qmul[n0 + c];
     }
   }
   __syncthreads();
@@ -120,11 +121,11 @@ igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
     const int m = (g * NW + wave) * 32 + l32;
     const bool live = m < M;
     const int mc = live ? m : M - 1;
-    int8_t* yrow = y + (int64_t)mc * p.ycs + lg * 16;
+    int8_t* yrow = y + (int64_t)mc * p.ycs + n0 + lg * 16;
     // the residual rows travel up to PRE slices ahead of their use: PRE KiB per wavefront in flight
     constexpr int PRE = NS < 8 ? NS : 8;
     uintx4 rr[NS];
-    const int8_t* rrow = has_res ? res + (int64_t)mc * p.rcs + lg * 16 : nullptr;
+    const int8_t* rrow = has_res ? res + (int64_t)mc * p.rcs + n0 + lg * 16 : nullptr;
     if (has_res) {
 #pragma unroll
       for (int j = 0; j < PRE; ++j) rr[j] = *reinterpret_cast<const uintx4*>(rrow + j * 32);
@@ -191,6 +192,18 @@ igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
 // Layers the streaming kernel serves: 8-bit 1x1 filters without padding, 8-bit
 // result, K = 64 .. 512 bytes per pixel, a multiple of 64 output channels, all
 // weights within 64 KiB, 16-byte aligned rows.
+// Output channels a workgroup keeps the weights of (at most 64 KiB): all of them, or an
+// equal share when the layer has more.
+static int stream_q8_channels_per_wg(const IgemmParams& p) {
+  if (p.C <= 0 || p.Kout <= 0) return 0;
+  const int cap = (64 * 1024 / p.C) / 64 * 64;
+  if (cap <= 0) return 0;
+  if (p.Kout <= cap) return p.Kout;
+  int n = cap;
+  while (n >= 64 && p.Kout % n != 0) n -= 64;
+  return n >= 64 ? n : 0;
+}
+
 bool igemm_stream_q8_geometry(const IgemmParams& p) {
   if (const char* force = getenv("ODLA_HIP_IGEMM_TILE")) {  // tuning aid
     if (strcmp(force, "stream") != 0 && force[0] != 0) return false;
@@ -202,17 +215,18 @@ bool igemm_stream_q8_geometry(const IgemmParams& p) {
   if (p.R != 1 || p.S != 1 || p.ph != 0 || p.pw != 0 || p.batch != 1) return false;
   if (p.C != 64 && p.C != 128 && p.C != 256 && p.C != 512) return false;
   if (p.xcs < p.C || p.xcs % 16 != 0) return false;
-  if (p.Kout % 64 != 0 || p.Kout < 64 || (int64_t)p.Kout * p.C > 64 * 1024) return false;
-  {  // the instantiations that exist (K bytes per pixel / output channels)
-    const int k = p.C, n = p.Kout;
+  if (p.Kout % 64 != 0 || p.Kout < 64) return false;
+  {  // the instantiations that exist: K bytes per pixel / output channels per workgroup
+    const int k = p.C, n = stream_q8_channels_per_wg(p);
     const bool built = (k == 64 && (n == 64 || n == 256)) || (k == 128 && (n == 128 || n == 512)) ||
                        (k == 256 && (n == 64 || n == 128 || n == 256)) || (k == 512 && n == 128);
-    if (!built) return false;
+    if (!built || p.Kout % n != 0) return false;
     // Longer pixel rows are built (and parity-clean) but selected only on request
     // (ODLA_HIP_STREAM_Q8=all): a lane's 16-byte piece of its pixel is then one of 8 - 32 pieces
-    // of the row, every load touches 32 cache lines, and the same layers are faster on the
-    // kernels that stage whole rows through LDS (ResNet-50 at batch 256: 256 -> 64 at 56 x 56
-    // 55 -> 64 us, 512 -> 128 at 28 x 28 33 -> 37 us).
+    // of the row and every load touches 32 cache lines.  Measured on ResNet-50 at batch 256
+    // against the kernels that stage whole rows through LDS: reductions 256 -> 64 at 56 x 56
+    // 55 -> 64 us, 512 -> 128 at 28 x 28 33 -> 37 us; expansions with a channel share per
+    // workgroup 256 -> 1024 at 14 x 14 41.5 -> 43 .. 49 us, 512 -> 2048 at 7 x 7 32 -> 40 us.
     if (k > 128) {
       const char* sel = getenv("ODLA_HIP_STREAM_Q8");
       if (sel == nullptr || strcmp(sel, "all") != 0) return false;
@@ -233,12 +247,13 @@ static bool stream_q8_ready(const IgemmParams& p) {
 hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream) {
   if (!stream_q8_ready(p)) return hipErrorInvalidValue;
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
-  const int nkk = p.C / 32, ns = p.Kout / 32;
+  const int kout_wg = stream_q8_channels_per_wg(p);
+  const int nkk = p.C / 32, ns = kout_wg / 32, nsplit = p.Kout / kout_wg;
   // wavefronts per workgroup as instantiated below (four where registers or LDS hold the
   // compute unit to fewer wavefronts: more, smaller workgroups then fill it better)
   const int nw = ((nkk == 4 && ns == 16) || (nkk == 8 && ns >= 4) || nkk == 16) ? 4 : 8;
   const int64_t groups = (M + nw * 32 - 1) / (nw * 32);
-  const size_t lds = (size_t)ns * nkk * 1024 + (size_t)p.Kout * 8;
+  const size_t lds = (size_t)ns * nkk * 1024 + (size_t)kout_wg * 8;
   if (lds > (size_t)kStreamMaxLds || groups > 0x7fffffff) return hipErrorInvalidValue;
   // resident workgroups walk the pixel groups with a grid stride
   int per_cu = (int)((160 * 1024) / (lds + 512));
@@ -249,10 +264,10 @@ hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream) {
     const int v = atoi(e);
     if (v >= 1 && v <= 8) per_cu = v;
   }
-  int64_t grid = 256 * per_cu;
+  int64_t grid = (256 * per_cu + nsplit - 1) / nsplit;   // per channel share
   if (grid > groups) grid = groups;
 #define STREAM_CASE(NKK_, NS_, NW_)                                                                                 \
-  if (nkk == NKK_ && p.Kout == NS_ * 32) {                                                                          \
+  if (nkk == NKK_ && ns == NS_) {                                                                          \
     static bool attr_set = false;                                                                                   \
     if (!attr_set) {                                                                                                \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_kernel<NKK_, NS_, NW_>),   \
@@ -260,7 +275,7 @@ hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream) {
       if (e != hipSuccess) return e;                                                                                \
       attr_set = true;                                                                                              \
     }                                                                                                               \
-    hipLaunchKernelGGL((igemm_stream_q8_kernel<NKK_, NS_, NW_>), dim3((unsigned)grid), dim3(NW_ * 64), lds, stream, \
+    hipLaunchKernelGGL((igemm_stream_q8_kernel<NKK_, NS_, NW_>), dim3((unsigned)grid, (unsigned)nsplit), dim3(NW_ * 64), lds, stream, \
                        p, (int)groups);                                                                             \
     return hipGetLastError();                                                                                       \
   }
