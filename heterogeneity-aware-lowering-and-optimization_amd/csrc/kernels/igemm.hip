@@ -29,266 +29,6 @@
 namespace ohip {
 
 // ---------------------------------------------------------------------------
-// The 8-bit form of the epilogue below (four wavefronts, each with all 128 pixels
-// of the tile and a 32-channel slice): every wavefront requantises its slice in
-// the accumulator layout and writes the dwords of its 32 channels into one
-// [32 pixels][128 channels] BYTE tile, side by side with the others; then each
-// of the 256 threads moves 16 consecutive channels of one pixel, i.e. one pass
-// covers the 32 x 128 tile with full 128-byte rows.  The residual tile takes the
-// same road in the other direction.  Two tile pairs alternate, so that a slice
-// needs one barrier between its phases and one before its tiles are reused.
-// mtile: the tile's 128 multipliers in LDS (parked there by the caller ahead of its K
-// loop: the epilogue then starts without a round trip to memory), or nullptr.
-__device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[4][1],
-                                                          unsigned char* smem, const int tile_m, const int tile_n,
-                                                          const int z, const int M, const int wave, const int lane,
-                                                          const float* mtile = nullptr) {
-  constexpr int BM = 128, BN = 128, TM = 4;
-  constexpr int PITCH = BN + 16;  // bytes per staged pixel row
-  constexpr int TILE = 32 * PITCH;
-  const int tid = wave * 64 + lane;
-  const int l32 = lane & 31, lg = lane >> 5;
-  const int n0 = tile_n * BN;
-
-  int8_t* ybase = reinterpret_cast<int8_t*>(p.y) + (int64_t)z * p.y_bs;
-  const int8_t* rbase = p.residual ? reinterpret_cast<const int8_t*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
-  const bool has_res = rbase != nullptr;
-
-  const int rp = tid >> 3;         // pixel of the slice this thread moves
-  const int c16 = (tid & 7) * 16;  // ... and its 16 channels
-  int nvalid = p.Kout - (n0 + c16);
-  nvalid = nvalid < 0 ? 0 : (nvalid > 16 ? 16 : nvalid);
-  const bool vec = (epi_vec & 2) && nvalid == 16;
-
-  floatx4 mq[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q)
-    mq[q] = mtile != nullptr ? *reinterpret_cast<const floatx4*>(mtile + wave * 32 + q * 8 + lg * 4)
-                             : load_qmul4(p.qmul, n0 + wave * 32 + q * 8 + lg * 4, p.Kout);
-
-  // The residual rows of all four slices are requested ahead of the first barrier:
-  // one memory round trip per tile.
-  uintx4 rall[TM];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    rall[i] = uintx4{0u, 0u, 0u, 0u};
-    if (has_res && nvalid > 0) {
-      const int m = tile_m * BM + i * 32 + rp;
-      const int mc = m < M ? m : M - 1;
-      rall[i] = load_row16(rbase + (int64_t)mc * p.rcs + n0 + c16, vec, nvalid);
-    }
-  }
-
-  // Workgroup barrier for LDS traffic only: the fence of __syncthreads would
-  // also wait for the global stores of the slices before.
-  auto lds_barrier = [&]() {
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0), other counters at their maxima
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
-  // (with or without a residual: two straight-line copies of the slice chosen by one
-  // workgroup-uniform branch; as a condition inside, every value pays a move or a select)
-  auto slice = [&](auto slice_no, auto with_res, auto with_clamp) __attribute__((always_inline)) {
-    constexpr int i = decltype(slice_no)::value;
-    constexpr bool kRes = decltype(with_res)::value;
-    constexpr bool kClamp = decltype(with_clamp)::value;
-    unsigned char* otile = smem + (i & 1) * (2 * TILE);
-    unsigned char* rtile = otile + TILE;
-    if constexpr (kRes) {
-      *reinterpret_cast<uintx4*>(rtile + rp * PITCH + c16) = q8_swz_chunk(rall[i], rp);
-      lds_barrier();
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int off = (l32 * PITCH + wave * 32 + q * 8 + lg * 4) ^ q8_swz(l32);
-      const unsigned rs = kRes ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
-      *reinterpret_cast<unsigned*>(otile + off) =
-          requant4<kRes, kClamp>(acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3], mq[q], rs, p);
-    }
-    // Nobody passes this barrier before every wavefront has written slice i; a wavefront
-    // writes slice i+1 into the other tile pair, and slice i+2 into this one only after
-    // the barrier(s) of slice i+1, which every wavefront reaches after its reads here.
-    lds_barrier();
-    const int m = tile_m * BM + i * 32 + rp;
-    const uintx4 v = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + rp * PITCH + c16), rp);
-    if (m < M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
-  };
-  auto slices = [&](auto with_res, auto with_clamp) __attribute__((always_inline)) {
-    slice(std::integral_constant<int, 0>{}, with_res, with_clamp);
-    slice(std::integral_constant<int, 1>{}, with_res, with_clamp);
-    slice(std::integral_constant<int, 2>{}, with_res, with_clamp);
-    slice(std::integral_constant<int, 3>{}, with_res, with_clamp);
-  };
-  const bool clamp = p.q_lo > 0.f;   // (a lower bound of 0 is what the saturating conversion applies anyway)
-  if (has_res) { if (clamp) slices(std::true_type{}, std::true_type{}); else slices(std::true_type{}, std::false_type{}); }
-  else { if (clamp) slices(std::false_type{}, std::true_type{}); else slices(std::false_type{}, std::false_type{}); }
-}
-
-// ---------------------------------------------------------------------------
-// Epilogue for workgroups whose four wavefronts each own all 128 pixels of the
-// tile and a 32-channel slice: per 32-pixel slice the four wavefronts park
-// their channels side by side in one [32 pixels][128 channels] LDS tile (two
-// tiles, alternating, one workgroup barrier per slice), and every thread then
-// handles eight consecutive channels of one pixel, so that 16 consecutive lanes
-// write one full 128-channel output row and no cache line is written in halves
-// by different wavefronts.
-template <typename TIn, typename Epi>
-__device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, const int epi_vec,
-                                                       typename Mma<TIn>::Acc (&acc)[4][1], unsigned char* smem,
-                                                       const int tile_m, const int tile_n, const int z, const int M,
-                                                       const int wave, const int lane, const float* mtile = nullptr) {
-  if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
-    igemm_epilogue_rows128_q8(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane, mtile);
-    return;
-  }
-  constexpr int BM = 128, BN = 128, TM = 4;
-  constexpr int PITCH = BN + 4;  // 4-byte words per staged pixel row
-  constexpr int TILE_WORDS = 32 * PITCH;
-  using AccE = typename Epi::AccE;
-  using TOut = typename EpiTraits<Epi>::TOut;
-  const int tid = wave * 64 + lane;
-  const int l32 = lane & 31, lg = lane >> 5;
-
-  TOut* ybase = reinterpret_cast<TOut*>(p.y) + y_batch_off(p, z);
-  const TOut* rbase = p.residual ? reinterpret_cast<const TOut*>(p.residual) + (int64_t)z * p.r_bs : nullptr;
-  const AccE* bias = p.bias ? reinterpret_cast<const AccE*>(p.bias) + (int64_t)z * p.bias_bs : nullptr;
-
-  const int rp = tid >> 4;          // pixel within a pass of 16
-  const int c8 = (tid & 15) * 8;    // this thread's eight channels
-  const int n = tile_n * BN + c8;
-  int nvalid = p.Kout - n;
-  nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);
-  const bool vec = (epi_vec & 1) && nvalid == 8;
-
-  AccE b8[8];
-  float m8[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) { b8[e] = 0; m8[e] = 0.f; }
-  if (nvalid > 0) {
-    // (8-bit layers carry their bias in the accumulators already)
-    if (bias != nullptr && !EpiTraits<Epi>::quant) {
-      if (vec) {
-        const intx4 t0 = *reinterpret_cast<const intx4*>(bias + n);
-        const intx4 t1 = *reinterpret_cast<const intx4*>(bias + n + 4);
-        __builtin_memcpy(&b8[0], &t0, 16);
-        __builtin_memcpy(&b8[4], &t1, 16);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) b8[e] = bias[n + e];
-      }
-    }
-    if constexpr (EpiTraits<Epi>::quant) {
-      if (p.qmul != nullptr) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (e < nvalid) m8[e] = p.qmul[n + e];
-      }
-    }
-  }
-
-  TOut* const ythr = ybase + y_col_off(p, n);  // + the row's offset
-  const TOut* const rthr = rbase ? rbase + (int64_t)(tile_m * BM + rp) * p.rcs + n : nullptr;
-
-  using RVec = typename Epi::RVec;
-  const bool have_rpre = Epi::kPrefetchResidual && vec && rbase != nullptr;
-  auto rfetch = [&](const int i, RVec (&dst)[2]) {
-#pragma unroll
-    for (int ps = 0; ps < 2; ++ps) {
-      const int m = tile_m * BM + i * 32 + ps * 16 + rp;
-      const int mc = m < M ? m : M - 1;
-      // read once by the whole launch: a non-temporal load leaves the cache lines to the operands that are re-read
-      dst[ps] = __builtin_nontemporal_load(reinterpret_cast<const RVec*>(rbase + (int64_t)mc * p.rcs + n));
-    }
-  };
-  // The residual vectors of all four slices are requested here, ahead of the
-  // parking and the barriers of the first slice: one memory round trip per tile.
-  // (Fetched a slice ahead instead, each slice would wait for its own request:
-  // behind the stores of the slice before, the compiler waits for every
-  // vector-memory operation in flight.)
-  RVec rall[TM][2];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int ps = 0; ps < 2; ++ps) rall[i][ps] = RVec{};
-  if constexpr (Epi::kPrefetchResidual) {
-    if (have_rpre) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i) rfetch(i, rall[i]);
-    }
-  }
-
-  // Workgroup barrier for LDS traffic only: the fence of __syncthreads would
-  // also wait for the global stores of the slices before, one store round trip
-  // per slice.
-  auto lds_barrier = [&]() {
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0), other counters at their maxima
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
-  // One call per 32-pixel slice with the slice number as a constant: a loop the
-  // optimizer declines to unroll would index the accumulators dynamically and
-  // move them to scratch memory.
-  auto slice = [&](auto slice_no) __attribute__((always_inline)) {
-    constexpr int i = decltype(slice_no)::value;
-    AccE* tile = reinterpret_cast<AccE*>(smem) + (i & 1) * TILE_WORDS;
-    // park: lane holds, for pixel l32, channels wave*32 + q*8 + lg*4 + (0..3)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      AccE* dst = tile + l32 * PITCH + wave * 32 + q * 8 + lg * 4;
-      if constexpr (sizeof(AccE) == 4 && !EpiTraits<Epi>::quant) {
-        *reinterpret_cast<floatx4*>(dst) =
-            (floatx4){acc[i][0][q * 4 + 0], acc[i][0][q * 4 + 1], acc[i][0][q * 4 + 2], acc[i][0][q * 4 + 3]};
-      } else {
-        *reinterpret_cast<intx4*>(dst) =
-            (intx4){(int)acc[i][0][q * 4 + 0], (int)acc[i][0][q * 4 + 1], (int)acc[i][0][q * 4 + 2], (int)acc[i][0][q * 4 + 3]};
-      }
-    }
-    // One barrier per slice is enough: a wavefront parks slice i+1 into the
-    // other tile only after its own read-back of slice i, and nobody passes
-    // this barrier before every wavefront has finished reading slice i-1.
-    lds_barrier();
-#pragma unroll
-    for (int ps = 0; ps < 2; ++ps) {
-      const int pix = ps * 16 + rp;
-      const int m = tile_m * BM + i * 32 + pix;
-      AccE a8[8];
-      const AccE* src = tile + pix * PITCH + c8;
-      if constexpr (!EpiTraits<Epi>::quant) {
-        const floatx4 v0 = *reinterpret_cast<const floatx4*>(src);
-        const floatx4 v1 = *reinterpret_cast<const floatx4*>(src + 4);
-        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-      } else {
-        const intx4 v0 = *reinterpret_cast<const intx4*>(src);
-        const intx4 v1 = *reinterpret_cast<const intx4*>(src + 4);
-        a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w;
-        a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
-      }
-      if (m < M && nvalid > 0) {
-        // thread row pointer + a wavefront-uniform offset
-        TOut* yrow = ythr + y_row_off(p, m);
-        const TOut* rrow = rbase ? rthr + (int64_t)(i * 32 + ps * 16) * p.rcs : nullptr;
-        Epi::store8(p, a8, nvalid, vec, b8, m8, yrow, rrow, have_rpre, rall[i][ps]);
-      }
-    }
-  };
-  static_assert(TM == 4, "one call per slice below");
-  slice(std::integral_constant<int, 0>{});
-  slice(std::integral_constant<int, 1>{});
-  slice(std::integral_constant<int, 2>{});
-  slice(std::integral_constant<int, 3>{});
-}
-
-// ---------------------------------------------------------------------------
 // Main kernel.
 //
 // K pipeline: per stage the workgroup holds 128 bytes of K per row for both
@@ -1299,7 +1039,7 @@ hipError_t dispatch(const IgemmParams& p, int epi_vec, hipStream_t s) {
 }  // namespace
 
 bool igemm_wants_wfrag(const IgemmParams& p) {
-  return wreg_shape(p) || lean_steps(p) > 0 || taps_shape(p).nkk > 0 || igemm_stream_q8_geometry(p);
+  return wreg_shape(p) || lean_steps(p) > 0 || taps_shape(p).nkk > 0 || igemm_stream_q8_geometry(p) || igemm_c3_geometry(p);
 }
 
 hipError_t launch_wfrag_pack(const WfragPackParams& p, hipStream_t stream) {
@@ -1319,6 +1059,7 @@ const char* igemm_variant_name(const IgemmParams& p) {
     case 3: return "128x256";
     default: break;
   }
+  if (p.w_frag != nullptr && igemm_c3_geometry(p)) return "patch3x3";
   if (p.w_frag != nullptr && igemm_stream_q8_geometry(p)) return "stream";
   if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
   if (p.w_frag != nullptr && taps_shape(p).nkk > 0) return "128x64t";
@@ -1396,6 +1137,7 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
   }
 
   if (const int big = igemm_big_variant(p)) return launch_igemm_big(p, epi_vec, big, stream);
+  if (p.w_frag != nullptr && igemm_c3_geometry(p)) return launch_igemm_c3(p, epi_vec, stream);
 
   switch (p.in_dt) {
     case DT_F32:

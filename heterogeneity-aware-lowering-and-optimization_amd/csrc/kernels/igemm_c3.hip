@@ -1,0 +1,309 @@
+// 3x3 convolutions with stride 1 and padding 1 (NHWC, constant weights) whose
+// input patch lives in LDS: a workgroup of WS wavefronts computes a tile of 4 pixel
+// blocks (BR rows x BC columns each, stacked vertically, BR * BC <= 32) of ONE image
+// for 32 * WS output channels; every wavefront owns a 32-channel slice and all four
+// blocks, so that a weight fragment feeds four MFMAs.  Per chunk of NKK * 32 bytes of input channels it
+// stages the (4 BR + 2) x (BC + 2) patch of input pixels around the tile once and
+// runs all nine taps on it: nine K stages of MFMAs per patch, where the gathering
+// kernels fetch 128 pixel rows per stage (the same input bytes nine times).
+//
+// LDS layout of a patch chunk: one plane of 4 KiB per 16-byte piece of the chunk,
+// plane[c][patch pixel] - the 32 pixels a fragment read covers are consecutive or
+// nearly consecutive 16-byte slots of one plane (no bank conflicts, no swizzle),
+// and a tap is a constant offset from the lane's base address: (r * PW + s) * 16.
+// Patch pixels outside the image hold the byte that represents 0.
+//
+// Weights come fragment-ordered from the packed copy (p.w_frag), one K stage
+// (tap x chunk) ahead, straight into registers.  Two patch buffers alternate: the
+// next chunk's patch is requested at the start of a chunk, parked in registers
+// during its nine stages and written to the other buffer at its end; one
+// workgroup barrier per chunk.
+//
+// The epilogues are the shared ones, told through a table in LDS which output
+// pixel each of the tile's 128 positions is (-1: none - rows past the image,
+// lanes past BR * BC).
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+#include <type_traits>
+
+#include "igemm_common.h"
+
+namespace ohip {
+namespace {
+
+struct C3Geom {
+  int br = 0, bc = 0;            // pixel block
+  int pw = 0, npp = 0;           // patch width (bc + 2) and pixels ((4 br + 2) * pw)
+  int tiles_x = 0, tiles_y = 0;  // tiles per image
+  int tiles_n = 0;               // channel tiles
+  int nck = 0;                   // channel chunks
+  int cpt = 0;                   // 32-byte K chunks per tap (C * element size / 32)
+  int nkk = 0, ws = 0;           // template choice
+  float eff = 0.f;               // share of the MFMA columns that are output pixels
+};
+
+// LDS ahead of the pixel table: the patch buffers (two; one for the two-wavefront form, which
+// serves single-chunk layers only), or the epilogue's staging tiles if those are larger
+constexpr int c3_main_bytes(const int nkk, const int ws) {
+  const int bufs = (ws == 4 ? 2 : 1) * nkk * 2 * 4096;
+  const int epi = ws == 4 ? 2 * 32 * (128 + 4) * 4 : 2 * 32 * (32 + 4) * 4;
+  return bufs > epi ? bufs : epi;
+}
+
+template <typename TIn, typename Epi, int NKK, int WS>
+__global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams p, const int epi_vec, const C3Geom g) {
+  constexpr int NCH = NKK * 2;   // 16-byte planes of a chunk
+  constexpr int CKB = NKK * 32;  // bytes of a chunk
+  constexpr int PLANE = 4096;    // 256 patch pixels x 16 bytes
+  constexpr int BUF = NCH * PLANE;
+  constexpr int NB = 4;          // pixel blocks of the tile, all of them in every wavefront
+  constexpr int NT = WS * 64;    // threads
+  constexpr int PR = 256 / NT;   // patch pixels per thread
+  constexpr int MAIN = c3_main_bytes(NKK, WS);
+  using Acc = typename Mma<TIn>::Acc;
+  static_assert(WS == 4 || WS == 2, "four slices of 32 channels, or two");
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // MAIN + 512 bytes
+  int* mtab = reinterpret_cast<int*>(smem + MAIN);
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, lg = lane >> 5;
+  const int M = p.N * p.H * p.W;
+
+  int bid = blockIdx.x;
+  {
+    // neighbouring tiles (which share weights and patch borders) on one XCD's L2
+    const int per = gridDim.x >> 3;
+    if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int tile_n = bid % g.tiles_n;
+  int t = bid / g.tiles_n;
+  const int tx = t % g.tiles_x;
+  t /= g.tiles_x;
+  const int ty = t % g.tiles_y;
+  const int n_img = t / g.tiles_y;
+  const int y0 = ty * 4 * g.br, x0 = tx * g.bc;
+
+  // which output pixel each position of the tile is
+  if (tid < 128) {
+    const int blk = tid >> 5, l = tid & 31;
+    const int br = l / g.bc, bc = l - br * g.bc;
+    const int yy = y0 + blk * g.br + br, xx = x0 + bc;
+    mtab[tid] = (l < g.br * g.bc && yy < p.H) ? (n_img * p.H + yy) * p.W + xx : -1;
+  }
+
+  // this thread's patch pixels: tid, tid + NT, ..
+  const unsigned fill_w = (unsigned)(p.a_fill & 0xff) * 0x01010101u;
+  const uintx4 fill = {fill_w, fill_w, fill_w, fill_w};
+  const unsigned char* src[PR];
+  bool inside[PR];
+#pragma unroll
+  for (int r = 0; r < PR; ++r) {
+    const int pp = tid + r * NT;
+    const int py = pp / g.pw, px = pp - py * g.pw;
+    const int gy = y0 - 1 + py, gx = x0 - 1 + px;
+    inside[r] = pp < g.npp && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
+    src[r] = reinterpret_cast<const unsigned char*>(p.x) +
+             ((int64_t)(n_img * p.H + (inside[r] ? gy : 0)) * p.W + (inside[r] ? gx : 0)) * p.xcs * (int64_t)sizeof(TIn);
+  }
+
+  uintx4 pr[PR][NCH];
+  auto patch_load = [&](const int ck) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < PR; ++r) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) pr[r][c] = fill;
+      if (inside[r]) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) pr[r][c] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + c * 16);
+      }
+    }
+  };
+  auto patch_store = [&](const int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < PR; ++r) {
+      const int pp = tid + r * NT;
+      if (pp < g.npp) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) *reinterpret_cast<uintx4*>(smem + buf * BUF + c * PLANE + pp * 16) = pr[r][c];
+      }
+    }
+  };
+
+  // this wavefront's channel slice and pixel blocks
+  const int slice = wave;
+  int wtile = tile_n * WS + slice;
+  wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;
+  const unsigned char* wfp = reinterpret_cast<const unsigned char*>(p.w_frag) + (int64_t)wtile * p.wf_chunks * 1024 + lane * 16;
+  auto wload = [&](uintx4 (&dst)[NKK], const int ck, const int tap) __attribute__((always_inline)) {
+    const unsigned char* b = wfp + (int64_t)(tap * g.cpt + ck * NKK) * 1024;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) dst[kk] = *reinterpret_cast<const uintx4*>(b + kk * 1024);
+  };
+
+  // LDS address of the window's top left pixel, per block: lanes past the block read its first pixel
+  unsigned base[NB];
+  {
+    const bool live = l32 < g.br * g.bc;
+    const int br = live ? l32 / g.bc : 0;
+    const int bc = live ? l32 - br * g.bc : 0;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) base[i] = (unsigned)(((i * g.br + br) * g.pw + bc) * 16 + lg * PLANE);
+  }
+
+  // Weight fragments of three K stages: the one in use and the two behind it (requested two
+  // stages, about 2 x 16 MFMAs, ahead of their use).  Nine stages per chunk keep stage
+  // st of every chunk in set st % 3.
+  uintx4 w[3][NKK];
+  patch_load(0);
+  wload(w[0], 0, 0);
+  wload(w[1], 0, 1);
+
+  Acc acc[NB][1];
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][0][e] = 0;
+  if constexpr (EpiTraits<Epi>::quant) acc_init_bias_vec<NB, 1>(p, 0, (tile_n * WS + slice) * 32, lg, acc);
+
+  patch_store(0);
+  __syncthreads();
+
+  // pixel fragments of the step in flight and of the next one
+  uintx4 b[2][NB];
+  auto bread = [&](uintx4 (&dst)[NB], const unsigned char* buf, const int tap, const int kk) __attribute__((always_inline)) {
+    const unsigned off = (unsigned)(((tap / 3) * g.pw + (tap % 3)) * 16) + kk * 2 * PLANE;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) dst[i] = *reinterpret_cast<const uintx4*>(buf + base[i] + off);
+  };
+
+  constexpr int STEPS = 9 * NKK;
+  for (int ck = 0; ck < g.nck; ++ck) {
+    const unsigned char* buf = smem + (WS == 4 ? (ck & 1) * BUF : 0);
+    const bool more = WS == 4 && ck + 1 < g.nck;
+    if (more) patch_load(ck + 1);
+    bread(b[0], buf, 0, 0);
+    // The scheduling barriers keep the requests where they are written - ahead of the MFMAs
+    // of the step before their use; left alone, the compiler moves every request down to
+    // its use and waits for it there.
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+      const int tap = st / NKK, kk = st % NKK;
+      if (kk == 0) {
+        if (tap + 2 < 9) wload(w[(tap + 2) % 3], ck, tap + 2);
+        else if (more) wload(w[(tap + 2) % 3], ck + 1, tap + 2 - 9);
+      }
+      if (st + 1 < STEPS) bread(b[(st + 1) & 1], buf, (st + 1) / NKK, (st + 1) % NKK);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NB; ++i) acc[i][0] = Mma<TIn>::run(w[tap % 3][kk], b[st & 1][i], acc[i][0]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // Nobody reads the other buffer any more: every wavefront has passed the barrier that
+    // ended the chunk before, i.e. has finished that chunk's reads.
+    if (more) patch_store((ck + 1) & 1);
+    __syncthreads();
+  }
+
+  if constexpr (WS == 4) {
+    igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc, smem, 0, tile_n, 0, M, wave, lane, nullptr, mtab);
+  } else {
+    igemm_epilogue<TIn, Epi, 128, 64, 128, 32>(p, epi_vec, acc, smem, 0, tile_n, 0, M, wave, lane, 0, mtab);
+  }
+}
+
+bool c3_geometry(const IgemmParams& p, C3Geom* out) {
+  if (const char* e = getenv("ODLA_HIP_C3")) {  // tuning aid: 0 keeps these layers on the gathering kernels
+    if (e[0] == '0') return false;
+  }
+  const int es = dtype_size(p.in_dt);
+  if (p.in_dt != DT_F16 && p.in_dt != DT_BF16 && p.in_dt != DT_I8) return false;
+  if (p.out_dt != p.in_dt || p.batch != 1) return false;
+  if (p.R != 3 || p.S != 3 || p.sh != 1 || p.sw != 1 || p.dh != 1 || p.dw != 1 || p.ph != 1 || p.pw != 1) return false;
+  if (p.Ho != p.H || p.Wo != p.W) return false;
+  if (p.y_rdiv > 0 || p.y_zdiv > 0) return false;
+  if (p.act != ACT_NONE && p.act != ACT_RELU && p.act != ACT_LEAKY && p.act != ACT_CLAMP) return false;
+  C3Geom g;
+  const int cb = p.C * es;
+  if (cb % 128 == 0) g.nkk = 4;
+  else if (cb == 64) g.nkk = 2;
+  else return false;
+  g.nck = cb / (g.nkk * 32);
+  g.cpt = cb / 32;
+  if (p.Kout % 128 == 0) g.ws = 4;
+  else if (p.Kout == 64 && g.nck == 1) g.ws = 2;   // (two wavefronts, one patch buffer)
+  else return false;
+  g.tiles_n = p.Kout / (32 * g.ws);
+  // the block shape that wastes the fewest MFMA columns (lanes past the block, rows past the
+  // image); among equals the one with the smallest patch per output pixel
+  float best_halo = 0.f;
+  for (int bc = 32; bc >= 4; --bc) {
+    if (p.W % bc != 0) continue;
+    int br = 32 / bc;
+    if (br > p.H) br = p.H;
+    const int th = 4 * br, ty = (p.H + th - 1) / th;
+    const float eff = (float)(br * bc) / 32.f * (float)p.H / (float)(ty * th);
+    const int npp = (th + 2) * (bc + 2);
+    if (npp > 256) continue;
+    const float halo = (float)npp / (float)(th * bc);
+    if (eff > g.eff + 1e-6f || (eff > g.eff - 1e-6f && halo < best_halo)) {
+      g.eff = eff; best_halo = halo;
+      g.br = br; g.bc = bc; g.pw = bc + 2; g.npp = npp;
+      g.tiles_x = p.W / bc; g.tiles_y = ty;
+    }
+  }
+  float min_eff = 0.7f;
+  if (const char* e = getenv("ODLA_HIP_C3_MIN_FILL")) min_eff = (float)atof(e);  // tuning aid
+  if (g.bc == 0 || g.eff < min_eff) return false;
+  const int64_t wgs = (int64_t)p.N * g.tiles_y * g.tiles_x * g.tiles_n;
+  if (wgs <= 0 || wgs > 0x7fffffff) return false;
+  if ((int64_t)p.N * p.H * p.W * p.xcs * es >= (1ll << 40)) return false;
+  if (out) *out = g;
+  return true;
+}
+
+template <typename TIn, typename Epi>
+hipError_t launch_c3(const IgemmParams& p, const int epi_vec, const C3Geom& g, hipStream_t stream) {
+  const dim3 grid((unsigned)((int64_t)p.N * g.tiles_y * g.tiles_x * g.tiles_n)), block(g.ws * 64);
+  // (more than the 64 KiB a kernel may use without asking)
+#define C3_CASE(NKK, WS)                                                                                            \
+  if (g.nkk == NKK && g.ws == WS) {                                                                                 \
+    constexpr int lds = c3_main_bytes(NKK, WS) + 512;                                                                  \
+    static bool ready = false; /* (repeating the call is harmless: no lock) */                                      \
+    if (!ready) {                                                                                                   \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_c3_kernel<TIn, Epi, NKK, WS>), \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds);                    \
+      if (e != hipSuccess) return e;                                                                                \
+      ready = true;                                                                                                 \
+    }                                                                                                               \
+    hipLaunchKernelGGL((igemm_c3_kernel<TIn, Epi, NKK, WS>), grid, block, lds, stream, p, epi_vec, g);             \
+    return hipGetLastError();                                                                                       \
+  }
+  C3_CASE(4, 4)
+  C3_CASE(4, 2)
+  C3_CASE(2, 4)
+  C3_CASE(2, 2)
+#undef C3_CASE
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+bool igemm_c3_geometry(const IgemmParams& p) { return c3_geometry(p, nullptr); }
+
+hipError_t launch_igemm_c3(const IgemmParams& p, const int epi_vec, hipStream_t stream) {
+  C3Geom g;
+  if (p.w_frag == nullptr || !c3_geometry(p, &g)) return hipErrorInvalidValue;
+  switch (p.in_dt) {
+    case DT_F16: return launch_c3<f16_t, EpiFloat<f16_t>>(p, epi_vec, g, stream);
+    case DT_BF16: return launch_c3<bf16_t, EpiFloat<bf16_t>>(p, epi_vec, g, stream);
+    case DT_I8:
+      if (p.qmul == nullptr) return hipErrorInvalidValue;
+      return launch_c3<int8_t, EpiQuant<0>>(p, epi_vec, g, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace ohip

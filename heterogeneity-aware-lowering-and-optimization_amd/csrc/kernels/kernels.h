@@ -155,6 +155,10 @@ hipError_t launch_igemm_big(const IgemmParams& p, int epi_vec, int variant, hipS
 // (p.w_frag, p.qmul and the division magics must be set; launch_igemm does that).
 bool igemm_stream_q8_geometry(const IgemmParams& p);
 hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream);
+// 3x3, stride 1, padding 1 with the input patch of a tile held in LDS (igemm_c3.hip): whether
+// the layer is one of its shapes, and its launch (called by launch_igemm with its epi_vec).
+bool igemm_c3_geometry(const IgemmParams& p);
+hipError_t launch_igemm_c3(const IgemmParams& p, int epi_vec, hipStream_t stream);
 
 // True when launch_igemm would use a fragment-ordered weight copy for this shape.
 bool igemm_wants_wfrag(const IgemmParams& p);
