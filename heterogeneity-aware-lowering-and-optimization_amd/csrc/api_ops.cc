@@ -26,6 +26,7 @@
 //   TOPK       i0 K, i1 largest, i2 axis; out = values, out2 = indices
 //   LRN        i0 layout, i1 window; f0 alpha, f1 beta, f2 bias
 //   ROWNORM    i0 layout; f0 eps, f1 scalar scale, f2 scalar offset; in = {x, scale?, offset?}
+#include <climits>
 #include <cmath>
 #include <cstring>
 
@@ -803,6 +804,134 @@ odla_value odla_Gather(odla_value input, odla_value indices, odla_int32 axis, od
   if (n == nullptr) return ADD_NODE_FAILED;
   n->i[0] = axis;
   return n->out;
+}
+
+// ---------------------------------------------------------------------------
+// Operators along one axis (OP_AXISOP): i[0] = AxisOp, i[1] = axis (resolved, >= 0).
+// CumSum: i[2] = exclusive, i[3] = reverse.  Compress: i[2] = conditions used,
+// i[3] = 1 when the operand is taken as one flat axis.
+
+// [ref: ops/odla_ops_process.h:187-201; dnnl odla_dnnl.cc:509-567]
+odla_value odla_GatherElements(odla_value input, odla_value indices, odla_int32 axis, odla_value_shape,
+                               const odla_value_id id) {
+  REQUIRE(input && indices, "odla_GatherElements: null operand");
+  _odla_computation* c = comp_of(input, indices);
+  REQUIRE(c, "odla_GatherElements: no current computation");
+  REQUIRE(indices->etype == ODLA_INT32 || indices->etype == ODLA_INT64, "odla_GatherElements: indices must be int32/int64");
+  const int r = input->shape.rank;
+  REQUIRE(indices->shape.rank == r, "odla_GatherElements: indices %s and input %s differ in rank", indices->shape.str().c_str(),
+          input->shape.str().c_str());
+  if (axis < 0) axis += r;
+  REQUIRE(axis >= 0 && axis < r, "odla_GatherElements: axis out of range");
+  // The operands are walked as [i][j][k] with j the axis (like the reference): the leading and
+  // trailing extents of the indices may be smaller than the input's only where that keeps
+  // the flattened walk meaningful - a smaller extent in the first of the merged dims.
+  for (int i = 0; i < r; ++i) {
+    if (i == axis) continue;
+    REQUIRE(indices->shape.d[i] <= input->shape.d[i], "odla_GatherElements: indices %s exceed the input %s",
+            indices->shape.str().c_str(), input->shape.str().c_str());
+    const bool first_of_group = i == 0 || i == axis + 1;
+    REQUIRE(indices->shape.d[i] == input->shape.d[i] || first_of_group,
+            "odla_GatherElements: indices %s may only be smaller than the input %s along the axis, dim 0 or the dim behind the axis",
+            indices->shape.str().c_str(), input->shape.str().c_str());
+  }
+  Node* n = add_node(c, OP_AXISOP, {input, indices}, input->etype, indices->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
+  n->i[0] = AX_GATHER_ELEMENTS;
+  n->i[1] = axis;
+  return n->out;
+}
+
+// The axis is a constant scalar (INT32 or INT64); the reference reads it when the
+// computation runs, here it is read when the node is recorded.
+// [ref: ops/odla_ops_math.h:239-241; dnnl odla_dnnl_statistics.cc:147-200]
+odla_value odla_CumSum(odla_value input, odla_value axis, odla_bool exclusion, odla_bool reverse, const odla_value_id id) {
+  REQUIRE(input && axis, "odla_CumSum: null operand");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_CumSum: no current computation");
+  REQUIRE(is_float_type(input->etype), "odla_CumSum: operand must be a float type");
+  REQUIRE(axis->kind == _odla_value::CONSTANT && axis->host_data != nullptr && axis->shape.numel() >= 1 &&
+              (axis->etype == ODLA_INT32 || axis->etype == ODLA_INT64),
+          "odla_CumSum: the axis must be a constant INT32 / INT64 scalar");
+  int64_t ax = axis->etype == ODLA_INT32 ? (int64_t) * static_cast<const int32_t*>(axis->host_data)
+                                         : *static_cast<const int64_t*>(axis->host_data);
+  const int r = input->shape.rank;
+  if (ax < 0) ax += r;
+  REQUIRE(ax >= 0 && ax < r, "odla_CumSum: axis out of range for %s", input->shape.str().c_str());
+  Node* n = add_node(c, OP_AXISOP, {input}, input->etype, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
+  n->i[0] = AX_CUMSUM;
+  n->i[1] = ax;
+  n->i[2] = exclusion != 0;
+  n->i[3] = reverse != 0;
+  return n->out;
+}
+
+// One-hot of the first largest element along the axis (a negative axis counts from the
+// end; the reference takes every negative axis as the last one in its second half).
+// [ref: ops/odla_ops_nn.h:114-126; dnnl odla_dnnl.cc:1688-1727]
+odla_value odla_Hardmax(odla_value input, odla_int32 axis, const odla_value_id id) {
+  REQUIRE(input, "odla_Hardmax: null operand");
+  _odla_computation* c = comp_of(input);
+  REQUIRE(c, "odla_Hardmax: no current computation");
+  REQUIRE(is_float_type(input->etype), "odla_Hardmax: operand must be a float type");
+  const int r = input->shape.rank;
+  if (axis < 0) axis += r;
+  REQUIRE(axis >= 0 && axis < r, "odla_Hardmax: axis out of range for %s", input->shape.str().c_str());
+  Node* n = add_node(c, OP_AXISOP, {input}, input->etype, input->shape, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
+  n->i[0] = AX_HARDMAX;
+  n->i[1] = axis;
+  return n->out;
+}
+
+// The result has the declared maximum shape; the selected slices fill it densely from the
+// start ([outer][selected][inner]) and the rest is zero (undefined in the reference).
+// axis == INT_MAX: the operand is taken as one flat axis.
+// [ref: ops/odla_ops_process.h:83-98; dnnl odla_dnnl.cc:1280-1328]
+odla_value odla_Compress(odla_value input, odla_value condition, odla_int32 axis, odla_value_shape max_output_shape,
+                         const odla_value_id id) {
+  REQUIRE(input && condition, "odla_Compress: null operand");
+  _odla_computation* c = comp_of(input, condition);
+  REQUIRE(c, "odla_Compress: no current computation");
+  REQUIRE(condition->etype == ODLA_BOOL && condition->shape.rank == 1, "odla_Compress: the condition must be a boolean vector");
+  REQUIRE(shape_valid(max_output_shape) && max_output_shape.size >= 1, "odla_Compress: the maximum result shape is required");
+  const Shape o = shape_from(max_output_shape);
+  const int r = input->shape.rank;
+  const bool flat = axis == INT_MAX;
+  int64_t used = condition->shape.d[0];
+  if (flat) {
+    axis = 0;
+    used = std::min(used, std::min(o.numel(), input->shape.numel()));
+  } else {
+    if (axis < 0) axis += r;
+    REQUIRE(axis >= 0 && axis < r, "odla_Compress: axis out of range for %s", input->shape.str().c_str());
+    used = std::min(used, input->shape.d[axis]);
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; ++i) outer *= input->shape.d[i];
+    for (int i = axis + 1; i < r; ++i) inner *= input->shape.d[i];
+    REQUIRE(outer * used * inner <= o.numel(), "odla_Compress: the maximum result shape %s cannot hold %lld slices",
+            o.str().c_str(), (long long)used);
+  }
+  REQUIRE(used < (1ll << 31), "odla_Compress: too many conditions");
+  Node* n = add_node(c, OP_AXISOP, {input, condition}, input->etype, o, id);
+  if (n == nullptr) return ADD_NODE_FAILED;
+  n->i[0] = AX_COMPRESS;
+  n->i[1] = axis;
+  n->i[2] = used;
+  n->i[3] = flat;
+  return n->out;
+}
+
+// Logical shifts of unsigned integers (UINT8, UINT32, UINT64; no 16-bit integer storage
+// here); a shift by the width of the type or more gives 0 (undefined in the reference).
+// [ref: ops/odla_ops_math.h:863-876; dnnl odla_dnnl.cc:947-1010]
+odla_value odla_Shift(odla_value input, odla_value shift_amount, odla_bool is_left_shift, const odla_value_id id) {
+  REQUIRE(input && shift_amount, "odla_Shift: null operand");
+  REQUIRE(input->etype == ODLA_UINT8 || input->etype == ODLA_UINT32 || input->etype == ODLA_UINT64,
+          "odla_Shift: operand must be UINT8, UINT32 or UINT64");
+  REQUIRE(input->etype == shift_amount->etype, "odla_Shift: operand and shift amount differ in element type");
+  return ewise(is_left_shift ? EW_SHL : EW_SHR, {input, shift_amount}, input->etype, "odla_Shift", id);
 }
 
 odla_value odla_Reshape(odla_value input, odla_value_shape output_dims, const odla_value_id id) {

@@ -46,9 +46,9 @@ const char* op_name(OpKind k) {
   static const char* names[] = {"Conv", "Gemm", "Binary", "Unary", "BatchNorm", "LayerNorm", "Pool",
                                 "Reduce", "Softmax", "Cast", "Concat", "Gather", "Reshape", "Resize",
                                 "Slice", "Transpose", "Quantize", "Dequantize", "NMS", "Elementwise", "ArgExtreme",
-                                "CopyND", "TopK", "LRN", "RowNorm", "PostProcess"};
-  static_assert(sizeof(names) / sizeof(names[0]) == (size_t)OP_POSTPROCESS + 1, "one name per OpKind");
-  if ((int)k < 0 || (int)k > (int)OP_POSTPROCESS) return "?";
+                                "CopyND", "TopK", "LRN", "RowNorm", "PostProcess", "AxisOp"};
+  static_assert(sizeof(names) / sizeof(names[0]) == (size_t)OP_AXISOP + 1, "one name per OpKind");
+  if ((int)k < 0 || (int)k > (int)OP_AXISOP) return "?";
   return names[(int)k];
 }
 

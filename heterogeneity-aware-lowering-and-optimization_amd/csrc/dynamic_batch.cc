@@ -154,6 +154,11 @@ std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, i
       case OP_POSTPROCESS:
         rs.reject(n, "works on one image");
         break;
+      case OP_AXISOP:
+        if (n.i[1] == 0 || (n.i[0] == AX_COMPRESS && n.i[3] != 0)) rs.reject(n, "runs along the batch");
+        else if (n.i[0] == AX_GATHER_ELEMENTS && !rs.carry(n.in[1])) rs.reject(n, "has indices that do not depend on the batch");
+        else if (n.i[0] == AX_COMPRESS) rs.reject(n, "has a result of a declared maximum shape");
+        break;
       case OP_QUANTIZE: case OP_DEQUANTIZE:
         for (size_t k = 1; k < n.in.size(); ++k)
           if (rs.carry(n.in[k])) rs.reject(n, "has a scale that depends on the batch");

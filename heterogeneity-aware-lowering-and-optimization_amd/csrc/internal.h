@@ -36,8 +36,10 @@ enum OpKind : int {
   OP_CONV, OP_GEMM, OP_BINARY, OP_UNARY, OP_BATCHNORM, OP_LAYERNORM, OP_POOL, OP_REDUCE,
   OP_SOFTMAX, OP_CAST, OP_CONCAT, OP_GATHER, OP_RESHAPE, OP_RESIZE, OP_SLICE, OP_TRANSPOSE,
   OP_QUANTIZE, OP_DEQUANTIZE, OP_NMS, OP_EWISE, OP_ARGEXT, OP_COPYND, OP_TOPK, OP_LRN, OP_ROWNORM,
-  OP_POSTPROCESS
+  OP_POSTPROCESS, OP_AXISOP
 };
+// sub-kinds of OP_AXISOP (Node::i[0])
+enum AxisOp : int { AX_GATHER_ELEMENTS = 0, AX_CUMSUM, AX_HARDMAX, AX_COMPRESS };
 const char* op_name(OpKind k);
 
 struct Shape {

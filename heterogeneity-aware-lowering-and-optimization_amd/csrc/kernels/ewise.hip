@@ -204,6 +204,21 @@ __global__ void __launch_bounds__(kThreads) ewise_select_kernel(EwiseParams p, i
   }
 }
 
+// y = a << b or a >> b on unsigned words of ES bytes
+template <int ES>
+__global__ void __launch_bounds__(kThreads) ewise_shift_kernel(EwiseParams p, int64_t n, bool left) {
+  using W = typename BytesOf<ES>::type;
+  const W* a = reinterpret_cast<const W*>(p.a);
+  const W* b = reinterpret_cast<const W*>(p.b);
+  W* y = reinterpret_cast<W*>(p.y);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) {
+    const Offsets o = decompose(p, i);
+    const W v = a[o.a], s = b[o.b];
+    y[i] = s >= (W)(ES * 8) ? (W)0 : (left ? (W)(v << s) : (W)(v >> s));
+  }
+}
+
 #define EWISE_TYPE_DISPATCH(dt, EXPR)                                 \
   switch (dt) {                                                       \
     case DT_F32: { using T = float; EXPR; break; }                    \
@@ -225,7 +240,8 @@ hipError_t launch_ewise(const EwiseParams& p, hipStream_t stream) {
     if (p.dims[d] <= 0) return hipErrorInvalidValue;
     n *= p.dims[d];
   }
-  const bool unary = p.op == EW_NOT || p.op >= EW_ISNAN;
+  const bool shift = p.op == EW_SHL || p.op == EW_SHR;
+  const bool unary = p.op == EW_NOT || (p.op >= EW_ISNAN && !shift);
   EwiseParams q = p;
   if (unary) { q.b = p.a; for (int d = 0; d < 6; ++d) q.sb[d] = p.sa[d]; }
   if (!q.b) return hipErrorInvalidValue;
@@ -238,6 +254,16 @@ hipError_t launch_ewise(const EwiseParams& p, hipStream_t stream) {
       case 4: hipLaunchKernelGGL(ewise_select_kernel<4>, dim3(grid), dim3(kThreads), 0, stream, q, n); break;
       case 8: hipLaunchKernelGGL(ewise_select_kernel<8>, dim3(grid), dim3(kThreads), 0, stream, q, n); break;
       default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+  }
+  if (shift) {
+    if (p.dt != DT_U8 && p.dt != DT_I32 && p.dt != DT_I64) return hipErrorInvalidValue;
+    const bool left = p.op == EW_SHL;
+    switch (dtype_size(p.dt)) {
+      case 1: hipLaunchKernelGGL(ewise_shift_kernel<1>, dim3(grid), dim3(kThreads), 0, stream, q, n, left); break;
+      case 4: hipLaunchKernelGGL(ewise_shift_kernel<4>, dim3(grid), dim3(kThreads), 0, stream, q, n, left); break;
+      default: hipLaunchKernelGGL(ewise_shift_kernel<8>, dim3(grid), dim3(kThreads), 0, stream, q, n, left); break;
     }
     return hipGetLastError();
   }

@@ -337,7 +337,8 @@ enum EwiseOp : int {
   EW_SELECT,
   EW_EQ, EW_NE, EW_LT, EW_LE, EW_GT, EW_GE,
   EW_AND, EW_OR, EW_XOR, EW_NOT,
-  EW_ISNAN, EW_ISINF, EW_ISINF_POS, EW_ISINF_NEG
+  EW_ISNAN, EW_ISINF, EW_ISINF_POS, EW_ISINF_NEG,
+  EW_SHL, EW_SHR   // bit shifts of unsigned integers (logical; a shift by the width or more gives 0)
 };
 struct EwiseParams {
   const void* a = nullptr; const void* b = nullptr; const void* c = nullptr; void* y = nullptr;
@@ -420,6 +421,25 @@ hipError_t launch_resize_linear_nhwc(const void* x, void* y, DType dt, int N, in
 hipError_t launch_gather_rows(const void* x, const void* idx, DType idx_dt, void* y,
                               int64_t outer, int64_t n_src_rows, int64_t n_idx,
                               int64_t row_bytes, hipStream_t stream);
+// Operators along one axis of a row-major tensor [outer][len][inner] (axis_ops.hip).
+// GatherElements: y[i][j][k] = x[i][idx[i][j][k]][k] with idx [ii][ij][ik] (INT32 / INT64) and
+// x [di][dj][dk], ii <= di, ik <= dk; a negative index counts from the end, one outside
+// the axis is clamped into it.
+hipError_t launch_gather_elements(const void* x, const void* idx, DType idx_dt, void* y, int elem_size, int64_t ii,
+                                  int64_t ij, int64_t ik, int64_t di, int64_t dj, int64_t dk, hipStream_t stream);
+// Running sum along the axis (fp32 accumulation; exclusive: the element itself is left out;
+// reverse: from the end of the axis).
+hipError_t launch_cumsum(const void* x, void* y, DType dt, int64_t outer, int64_t len, int64_t inner, bool exclusive,
+                         bool reverse, hipStream_t stream);
+// y[o][i][in] = 1 where i == amax[o][in], else 0 (the second half of Hardmax).
+hipError_t launch_onehot_axis(const void* amax, DType idx_dt, void* y, DType dt, int64_t outer, int64_t len, int64_t inner,
+                              hipStream_t stream);
+// Compress: the slices x[o][j][:] with cond[j] != 0 (j < n_cond <= len), dense from the start of
+// y as [outer][selected][inner]; the rest of y's n_out elements is zero.  sel: n_cond + 1 int32
+// of scratch memory.
+hipError_t launch_compress(const void* x, const void* cond, int n_cond, int32_t* sel, void* y, int elem_size,
+                           int64_t outer, int64_t len, int64_t inner, int64_t n_out, hipStream_t stream);
+
 hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t stream);
 // Fills `bytes` (a multiple of 4) with a repeated 32-bit pattern.
 hipError_t launch_fill_bytes(void* p, size_t bytes, uint32_t pattern, hipStream_t stream);

@@ -550,6 +550,7 @@ class Planner {
   void lower_lrn(int ni);
   void lower_rownorm(int ni);
   void lower_postprocess(int ni);
+  void lower_axisop(int ni);
   bool lower_fused_group(int seed, int from);
   bool fuse_slice_seed(int ni) const;
   bool fuse_candidate(int ni) const;
@@ -850,6 +851,7 @@ void Planner::lower(int ni) {
     case OP_LRN: lower_lrn(ni); break;
     case OP_ROWNORM: lower_rownorm(ni); break;
     case OP_POSTPROCESS: lower_postprocess(ni); break;
+    case OP_AXISOP: lower_axisop(ni); break;
   }
 }
 
@@ -3069,6 +3071,79 @@ void Planner::lower_gather(int ni) {
   emit("gather:" + n.out->name, {tx, ti}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
     return launch_gather_rows(a(e), ri(e), idt, b(e), outer, n_src, n_idx, row_bytes, st);
   });
+  set_main(n.out, ty);
+}
+
+// ------------------------------- GatherElements, CumSum, Hardmax, Compress ----
+void Planner::lower_axisop(int ni) {
+  Node& n = comp_->nodes[ni];
+  const _odla_value* x = n.in[0];
+  const Shape& xs = x->shape;
+  const AxisOp op = (AxisOp)n.i[0];
+  const int axis = (int)n.i[1];
+  const int tx = get(x, L_ROWMAJOR, FORM_FLOAT);
+  const DType dt = T(tx).dt;
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= xs.d[i];
+  for (int i = axis + 1; i < xs.rank; ++i) inner *= xs.d[i];
+  const int64_t len = xs.d[axis];
+  const int ty = new_tensor(dt, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  const Ref a = ref(tx), b = ref(ty);
+  switch (op) {
+    case AX_GATHER_ELEMENTS: {
+      const _odla_value* idx = n.in[1];
+      const int ti = get(idx, L_ROWMAJOR, FORM_FLOAT);
+      const DType idt = T(ti).dt;
+      int64_t ii = 1, ik = 1;
+      for (int i = 0; i < axis; ++i) ii *= idx->shape.d[i];
+      for (int i = axis + 1; i < xs.rank; ++i) ik *= idx->shape.d[i];
+      const int64_t ij = idx->shape.d[axis];
+      const int es = dtype_size(dt);
+      const Ref ri = ref(ti);
+      emit("gather_elements:" + n.out->name, {tx, ti}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_gather_elements(a(e), ri(e), idt, b(e), es, ii, ij, ik, outer, len, inner, st);
+      });
+      break;
+    }
+    case AX_CUMSUM: {
+      const bool exclusive = n.i[2] != 0, reverse = n.i[3] != 0;
+      emit("cumsum:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_cumsum(a(e), b(e), dt, outer, len, inner, exclusive, reverse, st);
+      });
+      break;
+    }
+    case AX_HARDMAX: {
+      // the index of the first largest element, then its one-hot form (the reference's two steps)
+      Shape is;
+      is.rank = 1;
+      is.d[0] = outer * inner;
+      const int tm = new_tensor(DT_I32, L_ROWMAJOR, is, 0, SP_ARENA);
+      const Ref m = ref(tm);
+      emit("hardmax.argmax:" + n.out->name, {tx}, {tm}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_arg_extreme(a(e), m(e), dt, DT_I32, outer, len, inner, true, false, st);
+      });
+      emit("hardmax:" + n.out->name, {tm}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_onehot_axis(m(e), DT_I32, b(e), dt, outer, len, inner, st);
+      });
+      break;
+    }
+    case AX_COMPRESS: {
+      const int tc = get(n.in[1], L_ROWMAJOR, FORM_FLOAT);
+      const int n_cond = (int)n.i[2];
+      const bool flat = n.i[3] != 0;
+      const int64_t o2 = flat ? 1 : outer, l2 = flat ? xs.numel() : len, i2 = flat ? 1 : inner;
+      const int64_t n_out = n.out->shape.numel();
+      const int es = dtype_size(dt);
+      const int tsel = raw_buffer(((size_t)n_cond + 1) * sizeof(int32_t), SP_ARENA);
+      const Ref rc = ref(tc), rs = ref(tsel);
+      emit("compress:" + n.out->name, {tx, tc}, {ty, tsel}, [=](const ExecEnv& e, hipStream_t st) {
+        return launch_compress(a(e), rc(e), n_cond, reinterpret_cast<int32_t*>(rs(e)), b(e), es, o2, l2, i2, n_out, st);
+      });
+      break;
+    }
+    default:
+      fail(ODLA_INTERNAL_LOGIC_ERR, "unknown axis operator %d", (int)op);
+  }
   set_main(n.out, ty);
 }
 

@@ -156,6 +156,14 @@ const char* api_op_name(const Node& n) {
     case OP_LRN: return "odla_LRN";
     case OP_ROWNORM: return "odla_InstanceNormalization";
     case OP_POSTPROCESS: return "odla_PostProcess";
+    case OP_AXISOP:
+      switch ((AxisOp)n.i[0]) {
+        case AX_GATHER_ELEMENTS: return "odla_GatherElements";
+        case AX_CUMSUM: return "odla_CumSum";
+        case AX_HARDMAX: return "odla_Hardmax";
+        case AX_COMPRESS: return "odla_Compress";
+      }
+      return "?";
   }
   return "odla_Op";
 }

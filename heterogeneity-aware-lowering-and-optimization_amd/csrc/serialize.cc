@@ -156,6 +156,7 @@ bool op_rule(OpKind op, OpRule* r) {
     case OP_LRN: *r = {1, 1, 0x1, false}; return true;
     case OP_ROWNORM: *r = {3, 3, 0x1, false}; return true;
     case OP_POSTPROCESS: *r = {5, 5, 0x1f, true}; return true;
+    case OP_AXISOP: *r = {1, 2, ~0u, false}; return true;
   }
   return false;
 }
@@ -308,6 +309,33 @@ odla_status validate_loaded(const _odla_computation* c) {
         LOADED_REQUIRE(xmax < x->shape.numel() && ymax < n.out->shape.numel(), "CopyND node %lld reaches outside its tensors", (long long)k);
         break;
       }
+      case OP_AXISOP: {
+        LOADED_REQUIRE(n.i[0] >= AX_GATHER_ELEMENTS && n.i[0] <= AX_COMPRESS, "AxisOp node %lld: kind %lld", (long long)k, (long long)n.i[0]);
+        LOADED_REQUIRE(n.i[1] >= 0 && n.i[1] < xr, "AxisOp node %lld: axis out of range", (long long)k);
+        const bool two = n.i[0] == AX_GATHER_ELEMENTS || n.i[0] == AX_COMPRESS;
+        LOADED_REQUIRE(n.in.size() == (two ? 2u : 1u), "AxisOp node %lld: %zu operands", (long long)k, n.in.size());
+        if (n.i[0] == AX_GATHER_ELEMENTS) {
+          const Shape& is = n.in[1]->shape;
+          LOADED_REQUIRE(is.rank == xr && n.out->shape == is, "GatherElements node %lld: malformed indices", (long long)k);
+          for (int i = 0; i < xr; ++i)
+            LOADED_REQUIRE(i == n.i[1] || is.d[i] == x->shape.d[i] || ((i == 0 || i == n.i[1] + 1) && is.d[i] <= x->shape.d[i]),
+                           "GatherElements node %lld: indices exceed the operand", (long long)k);
+        } else if (n.i[0] == AX_COMPRESS) {
+          const int64_t lim = n.i[3] ? std::min(x->shape.numel(), n.out->shape.numel()) : x->shape.d[n.i[1]];
+          LOADED_REQUIRE(n.in[1]->shape.rank == 1 && n.i[2] >= 0 && n.i[2] <= n.in[1]->shape.d[0] && n.i[2] <= lim,
+                         "Compress node %lld: malformed condition", (long long)k);
+          if (!n.i[3]) {
+            int64_t rest = 1;
+            for (int i = 0; i < xr; ++i) if (i != n.i[1]) rest *= x->shape.d[i];
+            LOADED_REQUIRE(rest * n.i[2] <= n.out->shape.numel(), "Compress node %lld: result too small", (long long)k);
+          } else {
+            LOADED_REQUIRE(n.i[1] == 0, "Compress node %lld: flat form with an axis", (long long)k);
+          }
+        } else {
+          LOADED_REQUIRE(n.out->shape == x->shape, "AxisOp node %lld: result shape differs from the operand's", (long long)k);
+        }
+        break;
+      }
       case OP_TOPK:
         LOADED_REQUIRE(n.i[2] >= 0 && n.i[2] < xr && n.i[0] >= 1 && n.i[0] <= x->shape.d[n.i[2]], "TopK node %lld: bad axis or K", (long long)k);
         break;
@@ -399,7 +427,7 @@ odla_status deserialize(const uint8_t* data, size_t size, _odla_computation* c) 
   for (int64_t k = 0; k < nn; ++k) {
     Node n;
     const int64_t op = r.i64();
-    if (op < 0 || op > (int64_t)OP_POSTPROCESS) return ODLA_INVALID_PARAM;
+    if (op < 0 || op > (int64_t)OP_AXISOP) return ODLA_INVALID_PARAM;
     n.op = (OpKind)op;
     const int64_t nin = r.i64();
     if (!r.ok || nin < 0 || nin > ODLA_MAX_OUTPUTS) return ODLA_INVALID_PARAM;

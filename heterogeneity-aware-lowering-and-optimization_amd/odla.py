@@ -48,7 +48,7 @@ _NP_TO_ODLA = {
     np.dtype(np.float32): ODLA_FLOAT32, np.dtype(np.float16): ODLA_FLOAT16,
     np.dtype(np.int32): ODLA_INT32, np.dtype(np.int64): ODLA_INT64,
     np.dtype(np.int8): ODLA_INT8, np.dtype(np.uint8): ODLA_UINT8, np.dtype(np.bool_): ODLA_BOOL,
-    np.dtype(np.uint32): ODLA_UINT32,
+    np.dtype(np.uint32): ODLA_UINT32, np.dtype(np.uint64): ODLA_UINT64,
 }
 _ODLA_TO_NP = {v: k for k, v in _NP_TO_ODLA.items()}
 
@@ -250,6 +250,11 @@ def load_library(path=None):
     proto("odla_Mean", vp, [Values, cid])
     proto("odla_IsInf", vp, [vp, u32, u32, cid])
     proto("odla_Select", vp, [vp, vp, vp, S, cid])
+    proto("odla_GatherElements", vp, [vp, vp, i32, S, cid])
+    proto("odla_CumSum", vp, [vp, vp, u32, u32, cid])
+    proto("odla_Hardmax", vp, [vp, i32, cid])
+    proto("odla_Compress", vp, [vp, vp, i32, S, cid])
+    proto("odla_Shift", vp, [vp, vp, u32, cid])
     for n in ("ReduceMin", "ReduceProd", "ReduceSumSquare", "ReduceLogSum", "ReduceLogSumExp"):
         proto("odla_" + n, vp, [vp, sz, pu32, u32, S, cid])
     for n in ("ReduceL1", "ReduceL2"):
@@ -469,6 +474,24 @@ class HipBuilder:
 
     def gather(self, x, idx, axis=0, name=None):
         return self._ret(self.L.odla_Gather(x, idx, axis, undefined_shape(), _cid(name)), "odla_Gather")
+
+    def gather_elements(self, x, idx, axis=0, name=None):
+        return self._ret(self.L.odla_GatherElements(x, idx, axis, undefined_shape(), _cid(name)), "odla_GatherElements")
+
+    def cumsum(self, x, axis, exclusive=False, reverse=False, name=None):
+        ax = self.const((name or "cumsum") + ".axis", np.array([axis], np.int32))
+        return self._ret(self.L.odla_CumSum(x, ax, int(exclusive), int(reverse), _cid(name)), "odla_CumSum")
+
+    def hardmax(self, x, axis=-1, name=None):
+        return self._ret(self.L.odla_Hardmax(x, axis, _cid(name)), "odla_Hardmax")
+
+    def compress(self, x, cond, axis, max_shape, name=None):
+        """axis None: x is taken as one flat axis (the C API's INT_MAX)."""
+        return self._ret(self.L.odla_Compress(x, cond, 2 ** 31 - 1 if axis is None else axis, make_shape(max_shape), _cid(name)),
+                         "odla_Compress")
+
+    def shift(self, x, amount, left=True, name=None):
+        return self._ret(self.L.odla_Shift(x, amount, int(left), _cid(name)), "odla_Shift")
 
     def reshape(self, x, shape, name=None):
         return self._ret(self.L.odla_Reshape(x, make_shape(shape), _cid(name)), "odla_Reshape")

@@ -657,6 +657,39 @@ odla_value odla_Select(odla_value condition, odla_value a, odla_value b,
                        odla_value_shape output_dims,
                        const odla_value_id value_id);
 
+/* out[i][j][k] = input[i][indices[i][j][k]][k] with j the axis: `indices` (INT32 or
+ * INT64) has the rank of `input` and the shape of the result.  A negative index
+ * counts from the end of the axis; an index outside the axis is clamped into it
+ * (the reference reads outside the tensor).
+ * [ref: ops/odla_ops_process.h:187-201; dnnl odla_dnnl.cc:509-567] */
+odla_value odla_GatherElements(odla_value input, odla_value indices,
+                               odla_int32 axis, odla_value_shape output_dims,
+                               const odla_value_id value_id);
+/* Running sum along `axis`, a constant INT32 / INT64 scalar that is read when the
+ * node is recorded (the reference reads it at run time).  exclusion: an element's
+ * own value is left out of its sum; reverse: sums run from the end of the axis.
+ * [ref: ops/odla_ops_math.h:239-241; dnnl odla_dnnl_statistics.cc:147-200] */
+odla_value odla_CumSum(odla_value input, odla_value axis, odla_bool exclusion,
+                       odla_bool reverse, const odla_value_id value_id);
+/* 1 at the first largest element along `axis`, 0 elsewhere.
+ * [ref: ops/odla_ops_nn.h:114-126; dnnl odla_dnnl.cc:1688-1727] */
+odla_value odla_Hardmax(odla_value input, odla_int32 axis,
+                        const odla_value_id value_id);
+/* The slices of `input` along `axis` whose entry of the boolean vector `condition`
+ * is set.  The result has the declared maximum shape; the selected slices are
+ * packed densely from its start ([outer][selected][inner]) and the rest is zero
+ * (undefined in the reference).  axis == INT_MAX: `input` is one flat axis.
+ * [ref: ops/odla_ops_process.h:83-98; dnnl odla_dnnl.cc:1280-1328] */
+odla_value odla_Compress(odla_value input, odla_value condition, odla_int32 axis,
+                         odla_value_shape max_output_shape,
+                         const odla_value_id value_id);
+/* Logical bit shift of UINT8 / UINT32 / UINT64 values by `shift_amount` (same
+ * type, broadcast like the binary operators); a shift by the width of the type
+ * or more gives 0.  UINT16 is not a storage type of this library.
+ * [ref: ops/odla_ops_math.h:863-876; dnnl odla_dnnl.cc:947-1010] */
+odla_value odla_Shift(odla_value input, odla_value shift_amount,
+                      odla_bool is_left_shift, const odla_value_id value_id);
+
 /* More reductions.  L1 = sum|x| + epsilon, L2 = sqrt(sum x^2 + epsilon).
  * [ref: ops/odla_ops_math.h:657-819; dnnl odla_dnnl_statistics.cc:21-160] */
 odla_value odla_ReduceMin(odla_value input, odla_size_t num_of_axes,

@@ -491,6 +491,119 @@ def align_like_reference(src_shape, dst_shape):
 _erf = np.vectorize(math.erf, otypes=[np.float64])
 
 
+# ---------------------------------------------------------------------------
+# Operators along one axis.  Each follows the reference's loop over the tensor seen as
+# [i][j][k] (j = the axis); the pins compare them with the operator examples the
+# reference's own test names point at and with independent numpy formulations.
+
+def _ijk(shape, axis):
+    i = int(np.prod(shape[:axis], dtype=np.int64))
+    k = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return i, int(shape[axis]), k
+
+
+def gather_elements(data, indices, axis):
+    """out[i][j][k] = data[i][indices[i][j][k]][k]
+    [ref: ODLA/platforms/dnnl/odla_dnnl.cc:509-522 do_gather_elements, :525-567].  A negative
+    index counts from the end of the axis (the reference adds the extent BEHIND the axis
+    instead, which is the same for the square operands of its test; the operator's
+    definition is followed here); an index outside the axis is clamped into it (the reference
+    reads outside the tensor)."""
+    data = np.asarray(data)
+    indices = np.asarray(indices)
+    axis = axis % data.ndim
+    di, dj, dk = _ijk(data.shape, axis)
+    ii, ij, ik = _ijk(indices.shape, axis)
+    flat = data.reshape(-1)
+    idx = indices.reshape(ii, ij, ik).astype(np.int64)
+    out = np.empty((ii, ij, ik), data.dtype)
+    for i in range(ii):
+        for j in range(ij):
+            v = idx[i, j]
+            v = np.where(v < 0, v + dj, v)
+            v = np.clip(v, 0, dj - 1)
+            out[i, j] = flat[i * dj * dk + v * dk + np.arange(ik)]
+    return out.reshape(indices.shape)
+
+
+def cumsum(x, axis, exclusive=False, reverse=False):
+    """Running sum along the axis, accumulated in order in fp32
+    [ref: ODLA/platforms/dnnl/odla_dnnl_statistics.cc:147-170 DoCumSum]."""
+    x = np.asarray(x, np.float32)
+    axis = axis % x.ndim
+    ni, nj, nk = _ijk(x.shape, axis)
+    src = x.reshape(ni, nj, nk)
+    out = np.empty_like(src)
+    acc = np.zeros((ni, nk), np.float32)
+    order = range(nj - 1, -1, -1) if reverse else range(nj)
+    for j in order:
+        cur = src[:, j, :]
+        out[:, j, :] = acc if exclusive else acc + cur
+        acc = acc + cur
+    return out.reshape(x.shape)
+
+
+def hardmax(x, axis):
+    """1 at the first largest element along the axis, 0 elsewhere
+    [ref: ODLA/platforms/dnnl/odla_dnnl.cc:1688-1727 (ArgMax without return_last_index, then
+    DoHardmax); odla_dnnl_statistics.cc:203-232 for the comparison: strictly greater replaces]."""
+    x = np.asarray(x, np.float32)
+    axis = axis % x.ndim
+    ni, nj, nk = _ijk(x.shape, axis)
+    src = x.reshape(ni, nj, nk)
+    best = src[:, 0, :].copy()
+    arg = np.zeros((ni, nk), np.int64)
+    for j in range(1, nj):
+        cur = src[:, j, :]
+        take = cur > best
+        best = np.where(take, cur, best)
+        arg = np.where(take, j, arg)
+    out = (np.arange(nj)[None, :, None] == arg[:, None, :]).astype(np.float32)
+    return out.reshape(x.shape)
+
+
+def compress(x, condition, axis, max_shape):
+    """Slices of x along the axis whose condition is set, packed densely from the start of a
+    buffer of the declared maximum shape ([outer][selected][inner], outer after outer); the
+    rest is zero here and undefined in the reference.  axis None: x is taken as one flat axis
+    [ref: ODLA/platforms/dnnl/odla_dnnl.cc:1280-1328]."""
+    x = np.asarray(x)
+    cond = np.asarray(condition).astype(bool).reshape(-1)
+    n_out = int(np.prod(max_shape, dtype=np.int64))
+    if axis is None:
+        src = x.reshape(1, -1, 1)
+        used = min(cond.size, n_out, src.shape[1])
+    else:
+        axis = axis % x.ndim
+        src = x.reshape(_ijk(x.shape, axis))
+        used = min(cond.size, src.shape[1])
+    out = np.zeros(n_out, x.dtype)
+    pos = 0
+    for i in range(src.shape[0]):
+        for j in range(used):
+            if cond[j]:
+                out[pos:pos + src.shape[2]] = src[i, j]
+                pos += src.shape[2]
+    return out.reshape(max_shape)
+
+
+def shift(x, amount, left):
+    """Logical shift of unsigned integers; a shift by the width or more gives 0 (undefined
+    in the reference) [ref: ODLA/platforms/dnnl/odla_dnnl.cc:947-1010]."""
+    x = np.asarray(x)
+    amount = np.asarray(amount)
+    assert x.dtype.kind == "u" and amount.dtype == x.dtype
+    bits = x.dtype.itemsize * 8
+    wide = x.astype(np.uint64)
+    s = np.minimum(amount.astype(np.uint64), np.uint64(63))
+    r = (wide << s) if left else (wide >> s)
+    if bits < 64:
+        r = r & np.uint64((1 << bits) - 1)
+    r = np.where(amount.astype(np.uint64) >= bits, np.uint64(0), r)
+    return r.astype(x.dtype)
+
+
+
 class RefBuilder:
     """Eager evaluation of an ODLA graph on the CPU.
 
@@ -1047,6 +1160,11 @@ class RefBuilder:
     def cast(self, x, dtype, name=None): return self._name(name, cast_like_reference(x, dtype))
     def concat(self, xs, axis, name=None): return self._name(name, np.concatenate(xs, axis=axis))
     def gather(self, x, idx, axis=0, name=None): return self._name(name, np.take(x, np.asarray(idx), axis=axis))
+    def gather_elements(self, x, idx, axis=0, name=None): return self._name(name, gather_elements(x, idx, axis))
+    def cumsum(self, x, axis, exclusive=False, reverse=False, name=None): return self._name(name, cumsum(x, axis, exclusive, reverse))
+    def hardmax(self, x, axis=-1, name=None): return self._name(name, hardmax(x, axis))
+    def compress(self, x, cond, axis, max_shape, name=None): return self._name(name, compress(x, cond, axis, max_shape))
+    def shift(self, x, amount, left=True, name=None): return self._name(name, shift(x, amount, left))
     def reshape(self, x, shape, name=None): return self._name(name, np.reshape(x, shape))
     def transpose(self, x, perm, name=None): return self._name(name, np.ascontiguousarray(np.transpose(x, perm)))
 

@@ -28,6 +28,11 @@ def _record(odla, with_table=False):
     hb.output(hb.gather(hb.transpose(logits, (1, 0), name="lt"), hb.const("idx", idx), 0, name="picked"), "picked")
     v, i = hb.topk(logits, 2, 1, names=("tv", "ti"))
     hb.output(i, "ti")
+    # operators along an axis (recorded, not marked as outputs: the counts above stay)
+    hm = hb.hardmax(logits, -1, name="hm")
+    cs = hb.cumsum(hm, 1, exclusive=True, name="cs")
+    ge = hb.gather_elements(cs, hb.const("gi", np.array([[0, 4, 1], [2, 3, 3]], np.int64)), 1, name="ge")
+    hb.compress(ge, hb.const("cc", np.array([1, 0, 1], np.bool_)), 1, (2, 3), name="cp")
     return hb
 
 
@@ -171,7 +176,8 @@ class _Stored:
         return next(n for n in self.nodes if n["op"] == op)
 
 
-OP_CONV, OP_GEMM, OP_REDUCE, OP_SOFTMAX, OP_GATHER, OP_RESHAPE, OP_TRANSPOSE, OP_TOPK = 0, 1, 7, 8, 11, 12, 15, 22
+OP_CONV, OP_GEMM, OP_REDUCE, OP_SOFTMAX, OP_GATHER, OP_RESHAPE, OP_TRANSPOSE, OP_TOPK, OP_AXISOP = 0, 1, 7, 8, 11, 12, 15, 22, 26
+AX_GATHER_ELEMENTS, AX_CUMSUM, AX_HARDMAX, AX_COMPRESS = range(4)
 
 
 def test_well_hashed_files_with_malformed_records_are_refused(odla, tmp_path):
@@ -194,6 +200,8 @@ def test_well_hashed_files_with_malformed_records_are_refused(odla, tmp_path):
 
     assert load(st.patched(8, 1)) == 0                       # the re-hashed, unchanged payload still loads
     conv, gemm, tr, topk = st.node(OP_CONV), st.node(OP_GEMM), st.node(OP_TRANSPOSE), st.node(OP_TOPK)
+    axis_nodes = {st.struct.unpack_from("<q", st.buf, n["i_at"])[0]: n for n in st.nodes if n["op"] == OP_AXISOP}
+    assert sorted(axis_nodes) == [AX_GATHER_ELEMENTS, AX_CUMSUM, AX_HARDMAX, AX_COMPRESS]
     arg_dims = st.values[0]["dims"]
     bad = {
         "extent 0": st.patched(arg_dims, 0),
@@ -217,6 +225,12 @@ def test_well_hashed_files_with_malformed_records_are_refused(odla, tmp_path):
         "softmax: axis out of range": st.patched(st.node(OP_SOFTMAX)["i_at"], 9),
         "gather: axis out of range": st.patched(st.node(OP_GATHER)["i_at"], -4),
         "reduce: axis out of range": st.patched(st.node(OP_REDUCE)["iv_at"], 4),
+        "axis operator: unknown kind": st.patched(axis_nodes[AX_CUMSUM]["i_at"], 9),
+        "cumsum: axis out of range": st.patched(axis_nodes[AX_CUMSUM]["i_at"] + 8, 2),
+        "hardmax: negative axis": st.patched(axis_nodes[AX_HARDMAX]["i_at"] + 8, -1),
+        "gather elements without indices": st.patched(axis_nodes[AX_GATHER_ELEMENTS]["in_at"] + 8, -1),
+        "compress: more conditions than the axis is long": st.patched(axis_nodes[AX_COMPRESS]["i_at"] + 16, 4),
+        "compress: flat form with an axis": st.patched(axis_nodes[AX_COMPRESS]["i_at"] + 24, 1),
         "reshape changes the element count": st.patched(st.values[
             st.struct.unpack_from("<q", st.buf, st.node(OP_RESHAPE)["out_at"])[0]]["dims"], 3),
     }
