@@ -343,6 +343,16 @@ __device__ __forceinline__ int quant_one(float x, float scale, float zf, bool sg
   return sgn ? (int)fminf(fmaxf(t, -128.f), 127.f) : (int)fminf(fmaxf(t, 0.f), 255.f);
 }
 
+// rne(x / scale) without the division where that is certain: x * (1 / scale) is within 1.5
+// units of the last place of the quotient, so unless it lies that close to a rounding boundary
+// (k + 0.5) both round to the same integer; the rare lanes near a boundary divide.
+__device__ __forceinline__ float rne_quotient(float x, float scale, float inv) {
+  const float m = x * inv;
+  float q = rintf(m);
+  if (fabsf(fabsf(m - q) - 0.5f) <= 4e-7f * fabsf(m) + 1e-30f) q = rintf(x / scale);
+  return q;
+}
+
 template <typename TS>
 __global__ void __launch_bounds__(kThreads)
 quantize_kernel(QuantParams p) {
@@ -350,35 +360,48 @@ quantize_kernel(QuantParams p) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   const int64_t t0 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   int64_t done = 0;
-  if (p.channels == 1 && (reinterpret_cast<uintptr_t>(p.src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(p.dst) & 7u) == 0) {
-    // per-tensor parameters: 8 elements per step, one 8-byte store
+  if (p.channels == 1 && (reinterpret_cast<uintptr_t>(p.src) & 15u) == 0 && (reinterpret_cast<uintptr_t>(p.dst) & 15u) == 0) {
+    // per-tensor parameters: a workgroup takes contiguous tiles of 256 threads x 2 x 16 elements;
+    // a thread's loads are issued back to back and each of its two results is one 16-byte store
     const float sc = p.scale[0], zf = p.zp ? (float)p.zp[0] : 0.f;
-    const int64_t n8 = p.n / 8;
-    for (int64_t i = t0; i < n8; i += stride) {
-      float v[8];
-      if constexpr (sizeof(TS) == 2) {
-        Vec16<TS> t;
-        t.load(x + i * 8);
+    const float inv = 1.0f / sc;
+    constexpr int LV = 16 * (int)sizeof(TS) / 16;   // 16-byte loads per 16 elements
+    constexpr int PER = 16 / LV;                     // elements per load
+    const int64_t tile = (int64_t)kThreads * 32;
+    const int64_t ntiles = p.n / tile;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+      Vec16<TS> in[2][LV];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = t.get(e);
-      } else {
-        Vec16<TS> t0v, t1v;
-        t0v.load(x + i * 8);
-        t1v.load(x + i * 8 + 4);
+      for (int g = 0; g < 2; ++g)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { v[e] = t0v.get(e); v[e + 4] = t1v.get(e); }
+        for (int l = 0; l < LV; ++l) in[g][l].load(x + t * tile + ((int64_t)g * kThreads + threadIdx.x) * 16 + l * PER);
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        uintx4 ov;
+        if (!p.dst_signed) {
+          // unsigned levels: the packing conversion rounds (an integer already) and saturates to [0, 255]
+          unsigned w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int l = 0; l < LV; ++l)
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+              const int k = l * PER + e;
+              w[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(rne_quotient(in[g][l].get(e), sc, inv) + zf, k & 3, w[k >> 2]);
+            }
+          const unsigned flip = p.dst_dt == DT_I8 ? 0x80808080u : 0u;   // stored as level - 128
+          ov = uintx4{w[0] ^ flip, w[1] ^ flip, w[2] ^ flip, w[3] ^ flip};
+        } else {
+          unsigned char o[16];
+#pragma unroll
+          for (int l = 0; l < LV; ++l)
+#pragma unroll
+            for (int e = 0; e < PER; ++e) o[l * PER + e] = (unsigned char)quant_one<TS>(in[g][l].get(e), sc, zf, true);
+          __builtin_memcpy(&ov, o, 16);
+        }
+        *reinterpret_cast<uintx4*>(reinterpret_cast<unsigned char*>(p.dst) + t * tile + ((int64_t)g * kThreads + threadIdx.x) * 16) = ov;
       }
-      unsigned char o[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int q = quant_one<TS>(v[e], sc, zf, p.dst_signed);
-        o[e] = (unsigned char)((!p.dst_signed && p.dst_dt == DT_I8) ? (q - 128) : q);
-      }
-      uintx2 ov;
-      __builtin_memcpy(&ov, o, 8);
-      *reinterpret_cast<uintx2*>(reinterpret_cast<unsigned char*>(p.dst) + i * 8) = ov;
     }
-    done = n8 * 8;
+    done = ntiles * tile;
   }
   for (int64_t i = done + t0; i < p.n; i += stride) {
     const int c = (p.channels > 1) ? (int)((i / p.inner) % p.channels) : 0;

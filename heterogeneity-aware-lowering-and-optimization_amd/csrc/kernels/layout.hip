@@ -337,6 +337,27 @@ resize_nearest_kernel(const E* __restrict__ x, E* __restrict__ y, int N, int H, 
   }
 }
 
+// Nearest resize by whole factors (Ho = fh * H, Wo = fw * W): workgroups walk source rows
+// (grid.x) in pieces of 256 vectors (grid.y); every source vector is read once and written fh * fw times; no division per element
+// but the one by the vectors per pixel.
+template <typename E>
+__global__ void __launch_bounds__(kThreads)
+resize_nearest_whole_kernel(const E* __restrict__ x, E* __restrict__ y, int rows, int H, int W, int cv, int fh, int fw) {
+  const int row_vecs = W * cv;
+  const int Wo = W * fw;
+  for (int row = blockIdx.x; row < rows; row += gridDim.x) {
+    const int n = row / H, hi = row - n * H;
+    const E* src = x + (int64_t)row * row_vecs;
+    E* dst = y + ((int64_t)n * H * fh + (int64_t)hi * fh) * Wo * cv;
+    for (int j = blockIdx.y * kThreads + threadIdx.x; j < row_vecs; j += gridDim.y * kThreads) {
+      const int wi = j / cv, c = j - wi * cv;
+      const E v = src[j];
+      for (int a = 0; a < fh; ++a)
+        for (int b = 0; b < fw; ++b) dst[((int64_t)a * Wo + wi * fw + b) * cv + c] = v;
+    }
+  }
+}
+
 // Bilinear resize, channels-last, pixel centres at half-integers and edge
 // clamping: source coordinate s = (o + 0.5) * in / out - 0.5, neighbours
 // floor(s) and floor(s) + 1 clamped into the image, weights 1 - frac and frac
@@ -662,7 +683,15 @@ hipError_t launch_resize_nearest_nhwc(const void* x, void* y, int elem_size, int
   if (!x || !y || N <= 0 || H <= 0 || W <= 0 || cs <= 0 || Ho <= 0 || Wo <= 0) return hipErrorInvalidValue;
   const int64_t row_bytes = (int64_t)cs * elem_size;
   const bool v16 = row_bytes % 16 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0;
-  if (v16) {
+  if (v16 && Ho % H == 0 && Wo % W == 0 && (int64_t)N * H < (1ll << 31) && (int64_t)W * (row_bytes / 16) < (1ll << 31)) {
+    // (nearest: source index floor(o * in / out) = o / factor)
+    const int cv = (int)(row_bytes / 16);
+    const int64_t rows = (int64_t)N * H;
+    const int64_t pieces = ((int64_t)W * cv + kThreads - 1) / kThreads;   // workgroups per source row
+    hipLaunchKernelGGL(resize_nearest_whole_kernel<b16>,
+                       dim3((unsigned)(rows < 65536 * 16 ? rows : 65536 * 16), (unsigned)(pieces < 64 ? pieces : 64)), dim3(kThreads), 0,
+                       stream, (const b16*)x, (b16*)y, (int)rows, H, W, cv, Ho / H, Wo / W);
+  } else if (v16) {
     const int cv = (int)(row_bytes / 16);
     const int grid = grid_for((int64_t)N * Ho * Wo * cv, kThreads * 2);
     hipLaunchKernelGGL(resize_nearest_kernel<b16>, dim3(grid), dim3(kThreads), 0, stream,

@@ -839,6 +839,39 @@ def test_quantize_parity_per_axis_and_ties():
     assert np.array_equal(got["qs"], want["qs"])
 
 
+@pytest.mark.parametrize("mode", ["fp32", "fp16"])
+@pytest.mark.parametrize("scale", [0.02, 0.037, 1.0 / 3.0, 2.0])
+def test_quantize_per_tensor_large_with_near_ties(mode, scale):
+    """Per-tensor parameters on a tensor large enough for the tiled path, whose rounding avoids
+    the division where x * (1 / scale) is clearly away from a rounding boundary: values placed
+    on and one float step beside every boundary k + 0.5 must give the oracle's levels (the
+    oracle divides), as must values far outside the range, in unsigned, stored-signed and
+    signed form."""
+    announce("quantize per tensor, near ties, %s scale %g" % (mode, scale))
+    r = rng(72)
+    n = 3 * 8192 + 40          # three full tiles and a ragged rest
+    x = (r.standard_normal(n) * 60 * scale).astype(np.float32)
+    k = np.arange(-140, 140, dtype=np.float32)
+    ties = ((k + 0.5) * np.float32(scale)).astype(np.float32)
+    x[:280] = ties
+    x[280:560] = np.nextafter(ties, np.float32(np.inf))
+    x[560:840] = np.nextafter(ties, np.float32(-np.inf))
+    x[840:850] = [1e30, -1e30, 3e4, -3e4, 0.0, -0.0, 1e-30, -1e-30, 255 * scale, 256 * scale]
+    x[9000:9280] = ties * np.float32(1.0000001)
+    if mode == "fp16":
+        x = x.astype(np.float16).astype(np.float32)
+    x = x.reshape(1, -1)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        b.output(b.quantize(a, [scale], [117], name="qu"), "qu")
+        b.output(b.quantize(a, [scale], None, signed=True, name="qs"), "qs")
+
+    got, want = run_both(build, {"x": x}, fp16=mode == "fp16")
+    assert np.array_equal(got["qu"], want["qu"])
+    assert np.array_equal(got["qs"], want["qs"])
+
+
 # --------------------------------------------------------------------------
 # NMS
 # --------------------------------------------------------------------------
