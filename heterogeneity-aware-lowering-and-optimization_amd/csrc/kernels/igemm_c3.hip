@@ -45,21 +45,22 @@ struct C3Geom {
 
 // LDS ahead of the pixel table: the patch buffers (two; one for the two-wavefront form, which
 // serves single-chunk layers only), or the epilogue's staging tiles if those are larger
+constexpr int kC3Plane = 3072;   // bytes of a patch plane: 192 patch pixels x 16 bytes
 constexpr int c3_main_bytes(const int nkk, const int ws) {
-  const int bufs = (ws == 4 ? 2 : 1) * nkk * 2 * 4096;
+  const int bufs = (ws == 4 ? 2 : 1) * nkk * 2 * kC3Plane;
   const int epi = ws == 4 ? 2 * 32 * (128 + 4) * 4 : 2 * 32 * (32 + 4) * 4;
   return bufs > epi ? bufs : epi;
 }
 
 template <typename TIn, typename Epi, int NKK, int WS>
-__global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams p, const int epi_vec, const C3Geom g) {
+__global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams p, const int epi_vec, const C3Geom g) {
   constexpr int NCH = NKK * 2;   // 16-byte planes of a chunk
   constexpr int CKB = NKK * 32;  // bytes of a chunk
-  constexpr int PLANE = 4096;    // 256 patch pixels x 16 bytes
+  constexpr int PLANE = kC3Plane;
   constexpr int BUF = NCH * PLANE;
   constexpr int NB = 4;          // pixel blocks of the tile, all of them in every wavefront
   constexpr int NT = WS * 64;    // threads
-  constexpr int PR = 256 / NT;   // patch pixels per thread
+  constexpr int PR = (kC3Plane / 16 + NT - 1) / NT;   // patch pixels per thread
   constexpr int MAIN = c3_main_bytes(NKK, WS);
   using Acc = typename Mma<TIn>::Acc;
   static_assert(WS == 4 || WS == 2, "four slices of 32 channels, or two");
@@ -109,25 +110,28 @@ __global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams 
              ((int64_t)(n_img * p.H + (inside[r] ? gy : 0)) * p.W + (inside[r] ? gx : 0)) * p.xcs * (int64_t)sizeof(TIn);
   }
 
+  // The patch of the next chunk travels through registers in two halves of NCH / 2 planes
+  // (the whole patch at once for the first chunk, whose registers nothing else needs yet).
+  constexpr int HP = NCH / 2;
   uintx4 pr[PR][NCH];
-  auto patch_load = [&](const int ck) __attribute__((always_inline)) {
+  auto patch_load = [&](const int ck, const int c0, const int c1) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) pr[r][c] = fill;
+      for (int c = c0; c < c1; ++c) pr[r][c - c0] = fill;
       if (inside[r]) {
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) pr[r][c] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + c * 16);
+        for (int c = c0; c < c1; ++c) pr[r][c - c0] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + c * 16);
       }
     }
   };
-  auto patch_store = [&](const int buf) __attribute__((always_inline)) {
+  auto patch_store = [&](const int buf, const int c0, const int c1) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
       const int pp = tid + r * NT;
       if (pp < g.npp) {
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) *reinterpret_cast<uintx4*>(smem + buf * BUF + c * PLANE + pp * 16) = pr[r][c];
+        for (int c = c0; c < c1; ++c) *reinterpret_cast<uintx4*>(smem + buf * BUF + c * PLANE + pp * 16) = pr[r][c - c0];
       }
     }
   };
@@ -137,10 +141,9 @@ __global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams 
   int wtile = tile_n * WS + slice;
   wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;
   const unsigned char* wfp = reinterpret_cast<const unsigned char*>(p.w_frag) + (int64_t)wtile * p.wf_chunks * 1024 + lane * 16;
-  auto wload = [&](uintx4 (&dst)[NKK], const int ck, const int tap) __attribute__((always_inline)) {
-    const unsigned char* b = wfp + (int64_t)(tap * g.cpt + ck * NKK) * 1024;
-#pragma unroll
-    for (int kk = 0; kk < NKK; ++kk) dst[kk] = *reinterpret_cast<const uintx4*>(b + kk * 1024);
+  // fragment of K step st (tap st / NKK, 32-byte piece st % NKK) of chunk ck
+  auto wload = [&](uintx4& dst, const int ck, const int st) __attribute__((always_inline)) {
+    dst = *reinterpret_cast<const uintx4*>(wfp + (int64_t)((st / NKK) * g.cpt + ck * NKK + st % NKK) * 1024);
   };
 
   // LDS address of the window's top left pixel, per block: lanes past the block read its first pixel
@@ -153,13 +156,16 @@ __global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams 
     for (int i = 0; i < NB; ++i) base[i] = (unsigned)(((i * g.br + br) * g.pw + bc) * 16 + lg * PLANE);
   }
 
-  // Weight fragments of three K stages: the one in use and the two behind it (requested two
-  // stages, about 2 x 16 MFMAs, ahead of their use).  Nine stages per chunk keep stage
-  // st of every chunk in set st % 3.
-  uintx4 w[3][NKK];
-  patch_load(0);
-  wload(w[0], 0, 0);
-  wload(w[1], 0, 1);
+  // Weight fragments: a ring of six K steps, requested five steps (20 MFMAs of this wavefront)
+  // ahead of their use.  The steps of a chunk are a multiple of six, so step st of every
+  // chunk sits in slot st % 6.
+  constexpr int STEPS = 9 * NKK;
+  constexpr int RW = 6, AHEAD = 5;
+  static_assert(STEPS % RW == 0, "the ring position of a step must not depend on the chunk");
+  uintx4 w[RW];
+  patch_load(0, 0, NCH);
+#pragma unroll
+  for (int st = 0; st < AHEAD; ++st) wload(w[st], 0, st);
 
   Acc acc[NB][1];
 #pragma unroll
@@ -168,7 +174,7 @@ __global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams 
     for (int e = 0; e < 16; ++e) acc[i][0][e] = 0;
   if constexpr (EpiTraits<Epi>::quant) acc_init_bias_vec<NB, 1>(p, 0, (tile_n * WS + slice) * 32, lg, acc);
 
-  patch_store(0);
+  patch_store(0, 0, NCH);
   __syncthreads();
 
   // pixel fragments of the step in flight and of the next one
@@ -179,31 +185,33 @@ __global__ __launch_bounds__(WS * 64, 2) void igemm_c3_kernel(const IgemmParams 
     for (int i = 0; i < NB; ++i) dst[i] = *reinterpret_cast<const uintx4*>(buf + base[i] + off);
   };
 
-  constexpr int STEPS = 9 * NKK;
   for (int ck = 0; ck < g.nck; ++ck) {
     const unsigned char* buf = smem + (WS == 4 ? (ck & 1) * BUF : 0);
     const bool more = WS == 4 && ck + 1 < g.nck;
-    if (more) patch_load(ck + 1);
+    const int nbuf = (ck + 1) & 1;
     bread(b[0], buf, 0, 0);
     // The scheduling barriers keep the requests where they are written - ahead of the MFMAs
-    // of the step before their use; left alone, the compiler moves every request down to
+    // of the steps before their use; left alone, the compiler moves every request down to
     // its use and waits for it there.
 #pragma unroll
     for (int st = 0; st < STEPS; ++st) {
-      const int tap = st / NKK, kk = st % NKK;
-      if (kk == 0) {
-        if (tap + 2 < 9) wload(w[(tap + 2) % 3], ck, tap + 2);
-        else if (more) wload(w[(tap + 2) % 3], ck + 1, tap + 2 - 9);
+      if (st + AHEAD < STEPS) wload(w[(st + AHEAD) % RW], ck, st + AHEAD);
+      else if (more) wload(w[(st + AHEAD) % RW], ck + 1, st + AHEAD - STEPS);
+      // The next chunk's patch: first half of its planes requested at the start of this chunk and
+      // written a third of the way in, the second half from there to two thirds.  Nobody reads
+      // the other buffer any more: every wavefront has passed the barrier that ended the chunk
+      // before, i.e. has finished that chunk's reads.
+      if (more) {
+        if (st == 0) patch_load(ck + 1, 0, HP);
+        if (st == STEPS / 3) { patch_store(nbuf, 0, HP); patch_load(ck + 1, HP, NCH); }
+        if (st == 2 * STEPS / 3) patch_store(nbuf, HP, NCH);
       }
       if (st + 1 < STEPS) bread(b[(st + 1) & 1], buf, (st + 1) / NKK, (st + 1) % NKK);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < NB; ++i) acc[i][0] = Mma<TIn>::run(w[tap % 3][kk], b[st & 1][i], acc[i][0]);
+      for (int i = 0; i < NB; ++i) acc[i][0] = Mma<TIn>::run(w[st % RW], b[st & 1][i], acc[i][0]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    // Nobody reads the other buffer any more: every wavefront has passed the barrier that
-    // ended the chunk before, i.e. has finished that chunk's reads.
-    if (more) patch_store((ck + 1) & 1);
     __syncthreads();
   }
 
@@ -246,7 +254,7 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
     const int th = 4 * br, ty = (p.H + th - 1) / th;
     const float eff = (float)(br * bc) / 32.f * (float)p.H / (float)(ty * th);
     const int npp = (th + 2) * (bc + 2);
-    if (npp > 256) continue;
+    if (npp > kC3Plane / 16) continue;
     const float halo = (float)npp / (float)(th * bc);
     if (eff > g.eff + 1e-6f || (eff > g.eff - 1e-6f && halo < best_halo)) {
       g.eff = eff; best_halo = halo;
