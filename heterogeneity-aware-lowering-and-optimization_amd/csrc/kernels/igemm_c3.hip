@@ -1,8 +1,8 @@
 // 3x3 convolutions with stride 1 and padding 1 (NHWC, constant weights) whose
 // input patch lives in LDS: a workgroup of WS wavefronts computes a tile of 4 pixel
 // blocks (BR rows x BC columns each, stacked vertically, BR * BC <= 32) of ONE image
-// for 32 * WS output channels; every wavefront owns a 32-channel slice and all four
-// blocks, so that a weight fragment feeds four MFMAs.  Per chunk of NKK * 32 bytes of input channels it
+// for 32 * WS * NJ output channels; every wavefront owns NJ 32-channel slices and all
+// four blocks, so that a weight fragment feeds four MFMAs and a pixel fragment NJ.  Per chunk of NKK * 32 bytes of input channels it
 // stages the (4 BR + 2) x (BC + 2) patch of input pixels around the tile once and
 // runs all nine taps on it: nine K stages of MFMAs per patch, where the gathering
 // kernels fetch 128 pixel rows per stage (the same input bytes nine times).
@@ -36,24 +36,27 @@ struct C3Geom {
   int br = 0, bc = 0;            // pixel block
   int pw = 0, npp = 0;           // patch width (bc + 2) and pixels ((4 br + 2) * pw)
   int tiles_x = 0, tiles_y = 0;  // tiles per image
-  int tiles_n = 0;               // channel tiles
+  int tiles_n = 0;               // channel tiles of 32 * ws * nj channels
   int nck = 0;                   // channel chunks
   int cpt = 0;                   // 32-byte K chunks per tap (C * element size / 32)
-  int nkk = 0, ws = 0;           // template choice
+  int nkk = 0, ws = 0, nj = 0;   // template choice
+  int main_bytes = 0;            // LDS ahead of the pixel table
   float eff = 0.f;               // share of the MFMA columns that are output pixels
 };
 
-// LDS ahead of the pixel table: the patch buffers (two; one for the two-wavefront form, which
-// serves single-chunk layers only), or the epilogue's staging tiles if those are larger
 constexpr int kC3Plane = 3072;   // bytes of a patch plane: 192 patch pixels x 16 bytes
-constexpr int c3_main_bytes(const int nkk, const int ws) {
-  const int bufs = (ws == 4 ? 2 : 1) * nkk * 2 * kC3Plane;
+// LDS ahead of the pixel table: the patch buffers (two; one when the layer has a single chunk),
+// or the epilogue's staging tiles if those are larger
+inline int c3_main_bytes(const int nkk, const int ws, const int nck) {
+  const int bufs = (nck > 1 ? 2 : 1) * nkk * 2 * kC3Plane;
   const int epi = ws == 4 ? 2 * 32 * (128 + 4) * 4 : 2 * 32 * (32 + 4) * 4;
   return bufs > epi ? bufs : epi;
 }
 
-template <typename TIn, typename Epi, int NKK, int WS>
-__global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams p, const int epi_vec, const C3Geom g) {
+// NJ = 2: every wavefront owns two 32-channel slices, i.e. every pixel fragment read from LDS
+// feeds two MFMAs (with one slice the LDS read rate saturates together with the matrix pipes).
+template <typename TIn, typename Epi, int NKK, int WS, int NJ>
+__global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(const IgemmParams p, const int epi_vec, const C3Geom g) {
   constexpr int NCH = NKK * 2;   // 16-byte planes of a chunk
   constexpr int CKB = NKK * 32;  // bytes of a chunk
   constexpr int PLANE = kC3Plane;
@@ -61,12 +64,11 @@ __global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams 
   constexpr int NB = 4;          // pixel blocks of the tile, all of them in every wavefront
   constexpr int NT = WS * 64;    // threads
   constexpr int PR = (kC3Plane / 16 + NT - 1) / NT;   // patch pixels per thread
-  constexpr int MAIN = c3_main_bytes(NKK, WS);
   using Acc = typename Mma<TIn>::Acc;
-  static_assert(WS == 4 || WS == 2, "four slices of 32 channels, or two");
+  static_assert(WS == 4 || WS == 2, "four wavefronts, or two");
 
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // MAIN + 512 bytes
-  int* mtab = reinterpret_cast<int*>(smem + MAIN);
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];  // g.main_bytes + 512
+  int* mtab = reinterpret_cast<int*>(smem + g.main_bytes);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -110,40 +112,48 @@ __global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams 
              ((int64_t)(n_img * p.H + (inside[r] ? gy : 0)) * p.W + (inside[r] ? gx : 0)) * p.xcs * (int64_t)sizeof(TIn);
   }
 
-  // The patch of the next chunk travels through registers in two halves of NCH / 2 planes
-  // (the whole patch at once for the first chunk, whose registers nothing else needs yet).
-  constexpr int HP = NCH / 2;
-  uintx4 pr[PR][NCH];
-  auto patch_load = [&](const int ck, const int c0, const int c1) __attribute__((always_inline)) {
+  // The patch of the next chunk travels through registers in PH pieces of NCH / PH planes, so
+  // that a thread parks 32 bytes at a time (the whole patch at once for the first chunk, whose
+  // registers nothing else needs yet).
+  constexpr int PH = 2 * PR < NCH ? 2 * PR : NCH;   // pieces
+  constexpr int PP = NCH / PH;                      // planes per piece
+  uintx4 pr[PR][PP];
+  auto patch_load = [&](const int ck, const int c0) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
 #pragma unroll
-      for (int c = c0; c < c1; ++c) pr[r][c - c0] = fill;
+      for (int c = 0; c < PP; ++c) pr[r][c] = fill;
       if (inside[r]) {
 #pragma unroll
-        for (int c = c0; c < c1; ++c) pr[r][c - c0] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + c * 16);
+        for (int c = 0; c < PP; ++c) pr[r][c] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + (c0 + c) * 16);
       }
     }
   };
-  auto patch_store = [&](const int buf, const int c0, const int c1) __attribute__((always_inline)) {
+  auto patch_store = [&](const int buf, const int c0) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
       const int pp = tid + r * NT;
       if (pp < g.npp) {
 #pragma unroll
-        for (int c = c0; c < c1; ++c) *reinterpret_cast<uintx4*>(smem + buf * BUF + c * PLANE + pp * 16) = pr[r][c - c0];
+        for (int c = 0; c < PP; ++c) *reinterpret_cast<uintx4*>(smem + buf * BUF + (c0 + c) * PLANE + pp * 16) = pr[r][c];
       }
     }
   };
 
-  // this wavefront's channel slice and pixel blocks
-  const int slice = wave;
-  int wtile = tile_n * WS + slice;
-  wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;
-  const unsigned char* wfp = reinterpret_cast<const unsigned char*>(p.w_frag) + (int64_t)wtile * p.wf_chunks * 1024 + lane * 16;
-  // fragment of K step st (tap st / NKK, 32-byte piece st % NKK) of chunk ck
-  auto wload = [&](uintx4& dst, const int ck, const int st) __attribute__((always_inline)) {
-    dst = *reinterpret_cast<const uintx4*>(wfp + (int64_t)((st / NKK) * g.cpt + ck * NKK + st % NKK) * 1024);
+  // this wavefront's channel slices: slice j is block wave of channel tile tile_n * NJ + j (the
+  // epilogue's view: WS blocks of 32 channels side by side per tile)
+  const unsigned char* wfp[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    int wtile = (tile_n * NJ + j) * WS + wave;
+    wtile = wtile < p.wf_tiles ? wtile : p.wf_tiles - 1;
+    wfp[j] = reinterpret_cast<const unsigned char*>(p.w_frag) + (int64_t)wtile * p.wf_chunks * 1024 + lane * 16;
+  }
+  // fragments of K step st (tap st / NKK, 32-byte piece st % NKK) of chunk ck
+  auto wload = [&](uintx4 (&dst)[NJ], const int ck, const int st) __attribute__((always_inline)) {
+    const int64_t off = (int64_t)((st / NKK) * g.cpt + ck * NKK + st % NKK) * 1024;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) dst[j] = *reinterpret_cast<const uintx4*>(wfp[j] + off);
   };
 
   // LDS address of the window's top left pixel, per block: lanes past the block read its first pixel
@@ -156,25 +166,46 @@ __global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams 
     for (int i = 0; i < NB; ++i) base[i] = (unsigned)(((i * g.br + br) * g.pw + bc) * 16 + lg * PLANE);
   }
 
-  // Weight fragments: a ring of six K steps, requested five steps (20 MFMAs of this wavefront)
-  // ahead of their use.  The steps of a chunk are a multiple of six, so step st of every
-  // chunk sits in slot st % 6.
+  // Weight fragments: a ring of RW K steps, requested RW - 1 steps ahead of their use.  The
+  // steps of a chunk are a multiple of RW, so step st of every chunk sits in slot st % RW.
   constexpr int STEPS = 9 * NKK;
-  constexpr int RW = 6, AHEAD = 5;
+  constexpr int RW = NJ == 1 ? 6 : (STEPS % 4 == 0 ? 4 : 3), AHEAD = RW - 1;
   static_assert(STEPS % RW == 0, "the ring position of a step must not depend on the chunk");
-  uintx4 w[RW];
-  patch_load(0, 0, NCH);
+  uintx4 w[RW][NJ];
+  {
+    // the first patch: every request of a thread in flight at once (its registers are free:
+    // the accumulators are not live yet)
+    uintx4 first[PR][NCH];
+#pragma unroll
+    for (int r = 0; r < PR; ++r) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) first[r][c] = fill;
+      if (inside[r]) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) first[r][c] = *reinterpret_cast<const uintx4*>(src[r] + c * 16);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < PR; ++r) {
+      const int pp = tid + r * NT;
+      if (pp < g.npp) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) *reinterpret_cast<uintx4*>(smem + c * PLANE + pp * 16) = first[r][c];
+      }
+    }
+  }
 #pragma unroll
   for (int st = 0; st < AHEAD; ++st) wload(w[st], 0, st);
 
-  Acc acc[NB][1];
+  Acc acc[NJ][NB][1];
 #pragma unroll
-  for (int i = 0; i < NB; ++i)
+  for (int j = 0; j < NJ; ++j) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][0][e] = 0;
-  if constexpr (EpiTraits<Epi>::quant) acc_init_bias_vec<NB, 1>(p, 0, (tile_n * WS + slice) * 32, lg, acc);
-
-  patch_store(0, 0, NCH);
+    for (int i = 0; i < NB; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[j][i][0][e] = 0;
+    if constexpr (EpiTraits<Epi>::quant) acc_init_bias_vec<NB, 1>(p, 0, ((tile_n * NJ + j) * WS + wave) * 32, lg, acc[j]);
+  }
   __syncthreads();
 
   // pixel fragments of the step in flight and of the next one
@@ -186,8 +217,9 @@ __global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams 
   };
 
   for (int ck = 0; ck < g.nck; ++ck) {
-    const unsigned char* buf = smem + (WS == 4 ? (ck & 1) * BUF : 0);
-    const bool more = WS == 4 && ck + 1 < g.nck;
+    const unsigned char* buf = smem + (ck & 1) * BUF;
+    // (two wavefronts x one slice serve single-chunk layers only: no code for a second patch)
+    const bool more = !(WS == 2 && NJ == 1) && ck + 1 < g.nck;
     const int nbuf = (ck + 1) & 1;
     bread(b[0], buf, 0, 0);
     // The scheduling barriers keep the requests where they are written - ahead of the MFMAs
@@ -197,28 +229,35 @@ __global__ __launch_bounds__(WS * 64, 3) void igemm_c3_kernel(const IgemmParams 
     for (int st = 0; st < STEPS; ++st) {
       if (st + AHEAD < STEPS) wload(w[(st + AHEAD) % RW], ck, st + AHEAD);
       else if (more) wload(w[(st + AHEAD) % RW], ck + 1, st + AHEAD - STEPS);
-      // The next chunk's patch: first half of its planes requested at the start of this chunk and
-      // written a third of the way in, the second half from there to two thirds.  Nobody reads
-      // the other buffer any more: every wavefront has passed the barrier that ended the chunk
-      // before, i.e. has finished that chunk's reads.
+      // The next chunk's patch, piece k requested at step k * STEPS / (PH + 1) and written at the
+      // next of these points.  Nobody reads the other buffer any more: every wavefront has
+      // passed the barrier that ended the chunk before, i.e. has finished that chunk's reads.
       if (more) {
-        if (st == 0) patch_load(ck + 1, 0, HP);
-        if (st == STEPS / 3) { patch_store(nbuf, 0, HP); patch_load(ck + 1, HP, NCH); }
-        if (st == 2 * STEPS / 3) patch_store(nbuf, HP, NCH);
+#pragma unroll
+        for (int k = 0; k <= PH; ++k)
+          if (st == k * STEPS / (PH + 1)) {
+            if (k > 0) patch_store(nbuf, (k - 1) * PP);
+            if (k < PH) patch_load(ck + 1, k * PP);
+          }
       }
       if (st + 1 < STEPS) bread(b[(st + 1) & 1], buf, (st + 1) / NKK, (st + 1) % NKK);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < NB; ++i) acc[i][0] = Mma<TIn>::run(w[st % RW], b[st & 1][i], acc[i][0]);
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int i = 0; i < NB; ++i) acc[j][i][0] = Mma<TIn>::run(w[st % RW][j], b[st & 1][i], acc[j][i][0]);
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
   }
 
-  if constexpr (WS == 4) {
-    igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc, smem, 0, tile_n, 0, M, wave, lane, nullptr, mtab);
-  } else {
-    igemm_epilogue<TIn, Epi, 128, 64, 128, 32>(p, epi_vec, acc, smem, 0, tile_n, 0, M, wave, lane, 0, mtab);
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if constexpr (WS == 4) {
+      igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc[j], smem, 0, tile_n * NJ + j, 0, M, wave, lane, nullptr, mtab);
+    } else {
+      igemm_epilogue<TIn, Epi, 128, 64, 128, 32>(p, epi_vec, acc[j], smem, 0, tile_n * NJ + j, 0, M, wave, lane, 0, mtab);
+    }
   }
 }
 
@@ -240,10 +279,21 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
   else return false;
   g.nck = cb / (g.nkk * 32);
   g.cpt = cb / 32;
-  if (p.Kout % 128 == 0) g.ws = 4;
-  else if (p.Kout == 64 && g.nck == 1) g.ws = 2;   // (two wavefronts, one patch buffer)
+  // Wavefronts x slices per wavefront: 4 x 1 (128 channels per workgroup) or 2 x 1 (64).  Two
+  // slices per wavefront (4 x 2: 256 channels, 2 x 2: 128) halve the LDS reads per MFMA and were
+  // measured no faster (ResNet-50 int8 at batch 256, 3x3 256 -> 256 at 14 x 14: 41.5 against
+  // 40 us; 128 -> 128 at 28 x 28 as 2 x 2: 50 against 41 us): with the K loop removed these
+  // launches still take 13 and 27 us, and in the loop a wavefront waits for weight fragments,
+  // not for LDS.  ODLA_HIP_C3_SLICES=2 selects them for measurement.
+  int nj2 = 0;
+  if (const char* e = getenv("ODLA_HIP_C3_SLICES")) nj2 = atoi(e) == 2 ? 1 : 0;
+  if (p.Kout % 256 == 0 && nj2) { g.ws = 4; g.nj = 2; }
+  else if (p.Kout % 128 == 0 && nj2 && g.nkk == 4) { g.ws = 2; g.nj = 2; }
+  else if (p.Kout % 128 == 0) { g.ws = 4; g.nj = 1; }
+  else if (p.Kout == 64 && g.nck == 1) { g.ws = 2; g.nj = 1; }
   else return false;
-  g.tiles_n = p.Kout / (32 * g.ws);
+  g.tiles_n = p.Kout / (32 * g.ws * g.nj);
+  g.main_bytes = c3_main_bytes(g.nkk, g.ws, g.nck);
   // the block shape that wastes the fewest MFMA columns (lanes past the block, rows past the
   // image); among equals the one with the smallest patch per output pixel
   float best_halo = 0.f;
@@ -276,23 +326,26 @@ template <typename TIn, typename Epi>
 hipError_t launch_c3(const IgemmParams& p, const int epi_vec, const C3Geom& g, hipStream_t stream) {
   const dim3 grid((unsigned)((int64_t)p.N * g.tiles_y * g.tiles_x * g.tiles_n)), block(g.ws * 64);
   // (more than the 64 KiB a kernel may use without asking)
-#define C3_CASE(NKK, WS)                                                                                            \
-  if (g.nkk == NKK && g.ws == WS) {                                                                                 \
-    constexpr int lds = c3_main_bytes(NKK, WS) + 512;                                                                  \
-    static bool ready = false; /* (repeating the call is harmless: no lock) */                                      \
-    if (!ready) {                                                                                                   \
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_c3_kernel<TIn, Epi, NKK, WS>), \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds);                    \
-      if (e != hipSuccess) return e;                                                                                \
-      ready = true;                                                                                                 \
-    }                                                                                                               \
-    hipLaunchKernelGGL((igemm_c3_kernel<TIn, Epi, NKK, WS>), grid, block, lds, stream, p, epi_vec, g);             \
-    return hipGetLastError();                                                                                       \
+#define C3_CASE(NKK, WS, NJ)                                                                                            \
+  if (g.nkk == NKK && g.ws == WS && g.nj == NJ) {                                                                       \
+    static bool ready = false; /* (repeating the call is harmless: no lock) */                                          \
+    if (!ready) {                                                                                                       \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_c3_kernel<TIn, Epi, NKK, WS, NJ>), \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, c3_main_bytes(NKK, WS, 2) + 512); \
+      if (e != hipSuccess) return e;                                                                                    \
+      ready = true;                                                                                                     \
+    }                                                                                                                   \
+    hipLaunchKernelGGL((igemm_c3_kernel<TIn, Epi, NKK, WS, NJ>), grid, block, lds, stream, p, epi_vec, g);             \
+    return hipGetLastError();                                                                                           \
   }
-  C3_CASE(4, 4)
-  C3_CASE(4, 2)
-  C3_CASE(2, 4)
-  C3_CASE(2, 2)
+  const int lds = g.main_bytes + 512;
+  C3_CASE(4, 4, 1)
+  C3_CASE(4, 2, 1)
+  C3_CASE(2, 4, 1)
+  C3_CASE(2, 2, 1)
+  C3_CASE(4, 4, 2)
+  C3_CASE(4, 2, 2)
+  C3_CASE(2, 4, 2)
 #undef C3_CASE
   return hipErrorInvalidValue;
 }

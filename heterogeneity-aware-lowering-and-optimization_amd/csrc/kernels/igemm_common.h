@@ -369,6 +369,17 @@ __device__ __forceinline__ uintx4 q8_swz_chunk(const uintx4 v, const int row) {
   return (row & 16) ? uintx4{t.z, t.w, t.x, t.y} : t;
 }
 
+// f(integral_constant<int, 0>{}) ... f(integral_constant<int, N - 1>{}), in order: a loop whose
+// index is a constant in every iteration (a loop the optimizer declines to unroll would index
+// the accumulators dynamically and move them to scratch memory).
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
 // Output pixel (row of the GEMM) behind pixel `local` of a workgroup's tile: consecutive
 // rows from `first` on, or - for kernels whose tile is a patch of the image rather than a
 // run of rows - the entry of the tile's table in LDS (-1: no such pixel).
@@ -655,11 +666,12 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
 // needs one barrier between its phases and one before its tiles are reused.
 // mtile: the tile's 128 multipliers in LDS (parked there by the caller ahead of its K
 // loop: the epilogue then starts without a round trip to memory), or nullptr.
-__device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[4][1],
+template <int TM = 4>
+__device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, const int epi_vec, intx16 (&acc)[TM][1],
                                                           unsigned char* smem, const int tile_m, const int tile_n,
                                                           const int z, const int M, const int wave, const int lane,
                                                           const float* mtile = nullptr, const int* mtab = nullptr) {
-  constexpr int BM = 128, BN = 128, TM = 4;
+  constexpr int BM = TM * 32, BN = 128;
   constexpr int PITCH = BN + 16;  // bytes per staged pixel row
   constexpr int TILE = 32 * PITCH;
   const int tid = wave * 64 + lane;
@@ -734,10 +746,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
     if ((unsigned)m < (unsigned)M && nvalid > 0) store_row16(ybase + (int64_t)m * p.ycs + n0 + c16, v, vec, nvalid, p.stream_out);
   };
   auto slices = [&](auto with_res, auto with_clamp) __attribute__((always_inline)) {
-    slice(std::integral_constant<int, 0>{}, with_res, with_clamp);
-    slice(std::integral_constant<int, 1>{}, with_res, with_clamp);
-    slice(std::integral_constant<int, 2>{}, with_res, with_clamp);
-    slice(std::integral_constant<int, 3>{}, with_res, with_clamp);
+    static_for<TM>([&](auto slice_no) __attribute__((always_inline)) { slice(slice_no, with_res, with_clamp); });
   };
   const bool clamp = p.q_lo > 0.f;   // (a lower bound of 0 is what the saturating conversion applies anyway)
   if (has_res) { if (clamp) slices(std::true_type{}, std::true_type{}); else slices(std::true_type{}, std::false_type{}); }
@@ -752,17 +761,17 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
 // handles eight consecutive channels of one pixel, so that 16 consecutive lanes
 // write one full 128-channel output row and no cache line is written in halves
 // by different wavefronts.
-template <typename TIn, typename Epi>
+template <typename TIn, typename Epi, int TM = 4>
 __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, const int epi_vec,
-                                                       typename Mma<TIn>::Acc (&acc)[4][1], unsigned char* smem,
+                                                       typename Mma<TIn>::Acc (&acc)[TM][1], unsigned char* smem,
                                                        const int tile_m, const int tile_n, const int z, const int M,
                                                        const int wave, const int lane, const float* mtile = nullptr,
                                                        const int* mtab = nullptr) {
   if constexpr (std::is_same<Epi, EpiQuant<0>>::value) {
-    igemm_epilogue_rows128_q8(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane, mtile, mtab);
+    igemm_epilogue_rows128_q8<TM>(p, epi_vec, acc, smem, tile_m, tile_n, z, M, wave, lane, mtile, mtab);
     return;
   }
-  constexpr int BM = 128, BN = 128, TM = 4;
+  constexpr int BM = TM * 32, BN = 128;
   constexpr int PITCH = BN + 4;  // 4-byte words per staged pixel row
   constexpr int TILE_WORDS = 32 * PITCH;
   using AccE = typename Epi::AccE;
@@ -898,11 +907,7 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
       }
     }
   };
-  static_assert(TM == 4, "one call per slice below");
-  slice(std::integral_constant<int, 0>{});
-  slice(std::integral_constant<int, 1>{});
-  slice(std::integral_constant<int, 2>{});
-  slice(std::integral_constant<int, 3>{});
+  static_for<TM>(slice);
 }
 
 }  // namespace ohip

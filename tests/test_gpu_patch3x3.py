@@ -31,6 +31,8 @@ FLOAT_CASES = [
     case(2, 64, 9, 16, 64, "clamp"),          # 16 x 2, most of the second tile is past the image
     case(1, 128, 5, 4, 128, "relu"),          # an image smaller than one block
     case(1, 64, 40, 104, 64, "add"),          # wide image, 8 x 4 blocks
+    case(1, 128, 16, 16, 384, "add_relu"),    # three channel tiles (of two wavefronts x two slices with ODLA_HIP_C3_SLICES=2)
+    case(2, 64, 12, 28, 512, "leaky"),        # four channel tiles (two of four wavefronts x two slices)
 ]
 
 INT8_CASES = [
@@ -39,12 +41,17 @@ INT8_CASES = [
     case(3, 256, 14, 14, 256, "none"),
     case(2, 64, 13, 13, 128, "relu"),
     case(1, 128, 9, 16, 64, "none"),
+    case(1, 64, 16, 16, 256, "relu"),         # 64-byte rows
+    case(2, 256, 10, 28, 512, "relu"),
 ]
 
 
 @pytest.mark.parametrize("mode", ["fp16", "bf16"])
-def test_patch_kernel_float(mode, monkeypatch):
+@pytest.mark.parametrize("slices", ["", "2"])
+def test_patch_kernel_float(mode, slices, monkeypatch):
     monkeypatch.setenv("ODLA_HIP_C3_MIN_FILL", "0")
+    if slices:
+        monkeypatch.setenv("ODLA_HIP_C3_SLICES", slices)   # two 32-channel slices per wavefront
     kw = {"fp16": mode == "fp16", "bf16": mode == "bf16"}
     for i, c in enumerate(FLOAT_CASES):
         announce("patch3x3 %s #%d %s" % (mode, i, c))
@@ -60,8 +67,11 @@ def test_patch_kernel_float(mode, monkeypatch):
         assert float(np.max(np.abs(got - want))) <= tol * max(1.0, float(np.max(np.abs(want)))), (i, c)
 
 
-def test_patch_kernel_int8(monkeypatch):
+@pytest.mark.parametrize("slices", ["", "2"])
+def test_patch_kernel_int8(slices, monkeypatch):
     monkeypatch.setenv("ODLA_HIP_C3_MIN_FILL", "0")
+    if slices:
+        monkeypatch.setenv("ODLA_HIP_C3_SLICES", slices)
     odla = entry.load().odla
     models = entry.load().models
     ref = entry.load_oracle()
