@@ -394,7 +394,7 @@ def profile_roofline(L, sess, wl, dump_path=None):
     roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
             "unit": "TOP/s" if wl.mode == "int8" else "TFLOP/s",
             "frac": round(achieved / peak, 4), "traffic": measured_traffic(wl.name),
-            "kernel": "igemm_wreg_kernel / igemm_kernel / igemm_lean_kernel / igemm_taps_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
+            "kernel": "igemm_wreg_kernel / igemm_kernel / igemm_lean_kernel / igemm_taps_kernel / igemm_stream_q8_kernel / igemm_c3_kernel (all %d conv/gemm launches of one step, avg %.1f us, "
                       "avg %.2f GFLOP per launch)" % (launches, 1e3 * mm_ms / max(launches, 1),
                                                      wl.flop / 1e9 / max(launches, 1)),
             "mm_ms_per_step": round(mm_ms, 4), "all_kernels_ms_per_step": round(total_ms, 4),
