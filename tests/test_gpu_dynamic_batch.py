@@ -226,6 +226,62 @@ def test_graphs_that_move_the_batch_are_refused_but_run_at_the_recorded_batch():
             hb.destroy()
 
 
+def test_axis_operators_with_a_dynamic_batch():
+    """Hardmax, CumSum and GatherElements along a non-batch axis follow the batch; along the
+    batch (or with indices that do not depend on it) the batch cannot be changed."""
+    odla = entry.load().odla
+    r = np.random.default_rng(19)
+    MAXB = 6
+
+    def build(batch):
+        def f(b):
+            x = b.arg("x", (batch, 7, 9))
+            idx = b.arg("idx", (batch, 4, 9), np.int32)
+            b.output(b.hardmax(x, 2, name="hm"), "hm")
+            b.output(b.cumsum(x, 1, exclusive=True, name="cs"), "cs")
+            b.output(b.gather_elements(x, idx, 1, name="ge"), "ge")
+        return f
+
+    hb = odla.HipBuilder(max_batch=MAXB)
+    try:
+        build(-1)(hb)
+        s = hb.session(True)
+        try:
+            for bs in (MAXB, 2, 5):
+                announce("dynamic batch axis operators, batch %d" % bs)
+                feeds = {"x": np.round(r.standard_normal((bs, 7, 9)) * 3).astype(np.float32),
+                         "idx": r.integers(-7, 7, (bs, 4, 9)).astype(np.int32)}
+                s.set_batch(bs)
+                got = s.run(feeds)
+                want = run_ref(build(bs), feeds)
+                for k in want:
+                    assert got[k].shape == want[k].shape and np.array_equal(got[k], want[k]), (k, bs)
+        finally:
+            s.close()
+    finally:
+        hb.destroy()
+
+    def along_batch(b):
+        b.output(b.cumsum(b.arg("x", (-1, 7, 9)), 0, name="cs"), "cs")
+
+    def constant_indices(b):
+        x = b.arg("x", (-1, 7, 9))
+        b.output(b.gather_elements(x, b.const("i", np.zeros((MAXB, 2, 9), np.int32)), 1, name="ge"), "ge")
+
+    for bld in (along_batch, constant_indices):
+        hb = odla.HipBuilder(max_batch=MAXB)
+        try:
+            bld(hb)
+            s = hb.session(True)
+            try:
+                with pytest.raises(odla.OdlaError):
+                    s.set_batch(3)
+            finally:
+                s.close()
+        finally:
+            hb.destroy()
+
+
 def test_int8_plan_at_a_smaller_batch_is_bit_exact():
     """The quantisation table names values, so the same table drives the plan of every batch."""
     pkg = entry.load()
