@@ -110,17 +110,20 @@ def test_q8_conv_two_channel_slices_per_wavefront(case, odla, ref, monkeypatch):
     test_q8_conv_accumulators_and_requant(case, odla, ref)
 
 
-@pytest.mark.parametrize("tiles_per_wg", [0, 3])
+@pytest.mark.parametrize("tiles_per_wg", [0, 3, -1])
 @pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (3, 128, 7, 7, 200), (4, 64, 21, 19, 256), (2, 128, 30, 30, 512),
-                                  (3, 256, 9, 9, 136)])
+                                  (3, 256, 9, 9, 136), (2, 64, 17, 9, 128), (1, 128, 40, 40, 384)])
 def test_q8_residual_fused_equals_unfused_equals_oracle(dims, tiles_per_wg, odla, ref, monkeypatch):
     """Conv -> Add(residual) -> ReLU: fused into the conv epilogue, and as separate
     quantised kernels (the conv result is also a graph output, which blocks fusion).
-    64 / 128 input channels take the streaming 1x1 kernel (also with several pixel
-    tiles per workgroup), 256 the weights-in-registers kernel."""
+    64 / 128 input channels take the streaming 1x1 kernel (whole groups of 128 output
+    channels in its row-epilogue form, otherwise - and with tiles_per_wg = -1 - in its
+    lane-exchange form), 256 the weights-in-registers kernel."""
     announce("q8 residual %s tiles/wg %d" % (dims, tiles_per_wg))
-    if tiles_per_wg:
+    if tiles_per_wg > 0:
         monkeypatch.setenv("ODLA_HIP_LEAN_TILES", str(tiles_per_wg))
+    if tiles_per_wg < 0:   # the streaming kernel's lane-exchange epilogue instead of its row epilogue
+        monkeypatch.setenv("ODLA_HIP_STREAM_ROWS", "0")
     r = rng(7)
     N, C, H, W, O = dims
     x = r.standard_normal((N, C, H, W)).astype(np.float32)
