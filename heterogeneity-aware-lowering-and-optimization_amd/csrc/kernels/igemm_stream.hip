@@ -311,7 +311,10 @@ bool igemm_stream_q8_geometry(const IgemmParams& p) {
     // against the kernels that stage whole rows through LDS: reductions 256 -> 64 at 56 x 56
     // 55 -> 64 us, 512 -> 128 at 28 x 28 33 -> 37 us; expansions with a channel share per
     // workgroup 256 -> 1024 at 14 x 14 41.5 -> 43 .. 49 us, 512 -> 2048 at 7 x 7 32 -> 40 us.
-    if (k > 128) {
+    // (512-byte rows stay on request; 256-byte rows are selected since the row-epilogue form
+    //  exists: same box, 256 -> 128 at 56 x 56 81 -> 65 us, 256 -> 512 stride 2 72 -> 64 us,
+    //  256 -> 1024 + residual 43.5 -> 41 us, 256 -> 64 57 -> 52 us)
+    if (k > 256) {
       const char* sel = getenv("ODLA_HIP_STREAM_Q8");
       if (sel == nullptr || strcmp(sel, "all") != 0) return false;
     }
@@ -366,6 +369,7 @@ static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream
   ROWS_CASE(2, 2)
   ROWS_CASE(4, 1)
   ROWS_CASE(4, 2)
+  ROWS_CASE(8, 1)
 #undef ROWS_CASE
   return hipErrorInvalidValue;
 }
@@ -377,7 +381,7 @@ hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream) {
   // and the layers that read these results lose the penalty the lane-exchange form's plain
   // residual loads left in the cache (256 -> 64 60 -> 57 us, 512 -> 128 39 -> 34 us, 512 -> 256 55 -> 48 us):
   // 2.68 -> 2.57 ms per step.  ODLA_HIP_STREAM_ROWS=0 keeps the lane-exchange form.
-  if (p.Kout % 128 == 0 && (p.C == 64 || p.C == 128)) {
+  if (p.Kout % 128 == 0 && (p.C == 64 || p.C == 128 || p.C == 256)) {
     const char* e = getenv("ODLA_HIP_STREAM_ROWS");
     if (e == nullptr || e[0] != '0') {
       const hipError_t r = launch_stream_q8_rows(p, stream);
