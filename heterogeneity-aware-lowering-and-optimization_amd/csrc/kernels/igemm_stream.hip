@@ -305,15 +305,13 @@ bool igemm_stream_q8_geometry(const IgemmParams& p) {
     const bool built = (k == 64 && (n == 64 || n == 256)) || (k == 128 && (n == 128 || n == 512)) ||
                        (k == 256 && (n == 64 || n == 128 || n == 256)) || (k == 512 && n == 128);
     if (!built || p.Kout % n != 0) return false;
-    // Longer pixel rows are built (and parity-clean) but selected only on request
-    // (ODLA_HIP_STREAM_Q8=all): a lane's 16-byte piece of its pixel is then one of 8 - 32 pieces
-    // of the row and every load touches 32 cache lines.  Measured on ResNet-50 at batch 256
-    // against the kernels that stage whole rows through LDS: reductions 256 -> 64 at 56 x 56
-    // 55 -> 64 us, 512 -> 128 at 28 x 28 33 -> 37 us; expansions with a channel share per
-    // workgroup 256 -> 1024 at 14 x 14 41.5 -> 43 .. 49 us, 512 -> 2048 at 7 x 7 32 -> 40 us.
-    // (512-byte rows stay on request; 256-byte rows are selected since the row-epilogue form
-    //  exists: same box, 256 -> 128 at 56 x 56 81 -> 65 us, 256 -> 512 stride 2 72 -> 64 us,
-    //  256 -> 1024 + residual 43.5 -> 41 us, 256 -> 64 57 -> 52 us)
+    // 512-byte pixel rows are built (and parity-clean) but selected only on request
+    // (ODLA_HIP_STREAM_Q8=all): a lane's 16-byte piece of its pixel is then one of 32 pieces of
+    // the row and every load touches 32 cache lines.  Measured on ResNet-50 at batch 256 against
+    // the kernels that stage whole rows through LDS: 512 -> 128 at 28 x 28 33 -> 37 us, 512 -> 2048
+    // at 7 x 7 32 -> 40 us.  256-byte rows are selected: with the row-epilogue form, same box,
+    // 256 -> 128 at 56 x 56 81 -> 65 us, 256 -> 512 stride 2 72 -> 64 us, 256 -> 1024 + residual
+    // 43.5 -> 41 us, 256 -> 64 (lane-exchange form) 57 -> 52 us.
     if (k > 256) {
       const char* sel = getenv("ODLA_HIP_STREAM_Q8");
       if (sel == nullptr || strcmp(sel, "all") != 0) return false;
