@@ -254,7 +254,7 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
     if constexpr (WS == 4) {
-      igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc[j], smem, 0, tile_n * NJ + j, 0, M, wave, lane, nullptr, mtab);
+      igemm_epilogue_rows128<TIn, Epi, 4, false>(p, epi_vec, acc[j], smem, 0, tile_n * NJ + j, 0, M, wave, lane, nullptr, mtab);
     } else {
       igemm_epilogue<TIn, Epi, 128, 64, 128, 32>(p, epi_vec, acc[j], smem, 0, tile_n * NJ + j, 0, M, wave, lane, 0, mtab);
     }

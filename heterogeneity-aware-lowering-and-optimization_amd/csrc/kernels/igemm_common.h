@@ -153,8 +153,12 @@ struct EpiFloat {
           v[0] += r0.x; v[1] += r0.y; v[2] += r0.z; v[3] += r0.w;
           v[4] += r1.x; v[5] += r1.y; v[6] += r1.z; v[7] += r1.w;
         } else {
+          // (both callers request the vector ahead whenever this branch is taken: vec, a
+          //  residual and a 2-byte result.  A load here, even on a path never taken, would make
+          //  the compiler wait for every store in flight where the paths join.)
           Vec16<TOut> rv;
-          if (have_rpre) rv.raw = rpre; else rv.load(r);
+          (void)have_rpre;
+          rv.raw = rpre;
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] += rv.get(e);
         }
@@ -378,6 +382,23 @@ __device__ __forceinline__ void static_for(F&& f) {
     f(std::integral_constant<int, I>{});
     static_for<N, I + 1>(f);
   }
+}
+
+// Makes the compiler wait HERE for a value that was requested from memory in conditional code.
+// The epilogues below request bias and residual vectors inside branches (per-lane validity) and
+// consume them in later branches, between which they store results.  For a value whose request
+// or first use sits in a branch the compiler cannot count the operations in flight behind it and
+// waits for all of them at every later use - stores included, which share the counter: one store
+// round trip per pass of an epilogue.  Naming the value as an operand of an (empty) statement in
+// straight-line code settles it once, before the first store; the passes then issue their stores
+// back to back.
+template <typename T>
+__device__ __forceinline__ void epi_settle(T& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(v));
+#else
+  (void)v;
+#endif
 }
 
 // Output pixel (row of the GEMM) behind pixel `local` of a workgroup's tile: consecutive
@@ -619,6 +640,15 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // this slice's operands from memory are complete before its first store (see epi_settle)
+    if (i == 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { epi_settle(b8[e]); epi_settle(m8[e]); }
+    }
+    if constexpr (Epi::kPrefetchResidual) {
+#pragma unroll
+      for (int ps = 0; ps < NPASS; ++ps) epi_settle(rcur[ps]);
+    }
     if constexpr (Epi::kPrefetchResidual && TM > 1) {
       if (have_rpre && i + 1 < TM) rfetch(i + 1, rnxt);
     }
@@ -761,7 +791,9 @@ __device__ __forceinline__ void igemm_epilogue_rows128_q8(const IgemmParams& p, 
 // handles eight consecutive channels of one pixel, so that 16 consecutive lanes
 // write one full 128-channel output row and no cache line is written in halves
 // by different wavefronts.
-template <typename TIn, typename Epi, int TM = 4>
+// kSettleRes = false leaves the residual vectors unsettled (a kernel at its register limit whose
+// layers carry no residual: settling holds all of them in registers at once, zeros included).
+template <typename TIn, typename Epi, int TM = 4, bool kSettleRes = true>
 __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, const int epi_vec,
                                                        typename Mma<TIn>::Acc (&acc)[TM][1], unsigned char* smem,
                                                        const int tile_m, const int tile_n, const int z, const int M,
@@ -860,6 +892,15 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
     __builtin_amdgcn_sched_barrier(0);
   };
   lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
+  // every operand requested from memory above is complete before the first store (see epi_settle)
+#pragma unroll
+  for (int e = 0; e < 8; ++e) { epi_settle(b8[e]); epi_settle(m8[e]); }
+  if constexpr (Epi::kPrefetchResidual && kSettleRes) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int ps = 0; ps < 2; ++ps) epi_settle(rall[i][ps]);
+  }
   // One call per 32-pixel slice with the slice number as a constant: a loop the
   // optimizer declines to unroll would index the accumulators dynamically and
   // move them to scratch memory.
