@@ -118,24 +118,29 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
   constexpr int PH = 2 * PR < NCH ? 2 * PR : NCH;   // pieces
   constexpr int PP = NCH / PH;                      // planes per piece
   uintx4 pr[PR][PP];
+  // Requests are unconditional (a position outside the image or past the patch reads the
+  // image's first pixel and is replaced by the fill value when it is parked): a request inside a
+  // branch is waited for right there, with everything else in flight, because the compiler
+  // copies its result out of the branch.
   auto patch_load = [&](const int ck, const int c0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < PR; ++r) {
+    for (int r = 0; r < PR; ++r)
 #pragma unroll
-      for (int c = 0; c < PP; ++c) pr[r][c] = fill;
-      if (inside[r]) {
-#pragma unroll
-        for (int c = 0; c < PP; ++c) pr[r][c] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + (c0 + c) * 16);
-      }
-    }
+      for (int c = 0; c < PP; ++c) pr[r][c] = *reinterpret_cast<const uintx4*>(src[r] + (int64_t)ck * CKB + (c0 + c) * 16);
   };
   auto patch_store = [&](const int buf, const int c0) __attribute__((always_inline)) {
+    // (the wait for the requests sits here, in straight-line code, not inside the branch below)
+#pragma unroll
+    for (int r = 0; r < PR; ++r)
+#pragma unroll
+      for (int c = 0; c < PP; ++c) epi_settle(pr[r][c]);
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
       const int pp = tid + r * NT;
       if (pp < g.npp) {
 #pragma unroll
-        for (int c = 0; c < PP; ++c) *reinterpret_cast<uintx4*>(smem + buf * BUF + (c0 + c) * PLANE + pp * 16) = pr[r][c];
+        for (int c = 0; c < PP; ++c)
+          *reinterpret_cast<uintx4*>(smem + buf * BUF + (c0 + c) * PLANE + pp * 16) = inside[r] ? pr[r][c] : fill;
       }
     }
   };
@@ -175,6 +180,8 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
   {
     // the first patch: every request of a thread in flight at once (its registers are free:
     // the accumulators are not live yet)
+    // (conditional here: with two wavefronts most threads have no second patch pixel, and
+    //  nothing else is in flight yet that a wait inside the branch could hold up)
     uintx4 first[PR][NCH];
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
@@ -227,8 +234,10 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
     // its use and waits for it there.
 #pragma unroll
     for (int st = 0; st < STEPS; ++st) {
+      // (behind the last chunk the ring re-reads that chunk's first steps: a request that is
+      //  always made keeps the number of operations in flight a constant the compiler can count)
       if (st + AHEAD < STEPS) wload(w[(st + AHEAD) % RW], ck, st + AHEAD);
-      else if (more) wload(w[(st + AHEAD) % RW], ck + 1, st + AHEAD - STEPS);
+      else wload(w[(st + AHEAD) % RW], more ? ck + 1 : ck, st + AHEAD - STEPS);
       // The next chunk's patch, piece k requested at step k * STEPS / (PH + 1) and written at the
       // next of these points.  Nobody reads the other buffer any more: every wavefront has
       // passed the barrier that ended the chunk before, i.e. has finished that chunk's reads.

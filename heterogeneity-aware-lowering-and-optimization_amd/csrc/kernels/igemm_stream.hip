@@ -187,28 +187,36 @@ igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
   }
 }
 
-// The same walk with the shared row epilogue: a wavefront computes 128 channels (four slices)
-// of its 32 pixels at a time and hands them to igemm_epilogue_q8, which requantises in the
-// accumulator layout, turns the bytes into full 128-byte rows through the wavefront's own LDS
-// tile and moves rows (and residual rows) with non-temporal 16-byte accesses - eight lanes per
-// row piece, where the lane-exchange form above moves 32-byte pieces.
+// The same walk with a row epilogue: a wavefront computes 128 channels (four slices) of its 32
+// pixels at a time, requantises them in the accumulator layout (requant4, the arithmetic of
+// igemm_epilogue_q8), turns the bytes into full 128-byte rows through its own LDS tile and moves
+// rows (and residual rows) with non-temporal 16-byte accesses - eight lanes per row, where the
+// lane-exchange form above moves 32-byte pieces.
+//
+// Order of the memory operations.  Loads and stores share one in-order counter, and the stores
+// sit in branches (pixels past the end), so the compiler cannot count them: every wait for a
+// load that comes after a store waits for that store too.  Hence: every request - the pixels of
+// the next group, the residual rows of the NEXT 128-channel step - is made after the stores of
+// the step before and is waited for (epi_settle) right before the stores of the current step.
+// A step's MFMAs and requantisation then cover the latency of its requests, and a store burst
+// has a whole step to drain before anything waits behind it.
 // NG: groups of 128 channels of this workgroup (blockIdx.y selects its share of the layer's).
-template <int NKK, int NG, int NW>
-__global__ void __launch_bounds__(NW * 64, 2)
-igemm_stream_q8_rows_kernel(const IgemmParams p, const int groups, const int epi_vec) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+template <int NKK, int NG, int NW, bool kRes, bool kClamp>
+__device__ __forceinline__ void stream_rows_body(const IgemmParams& p, const int groups, unsigned char* smem) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int l32 = lane & 31, lg = lane >> 5;
   const int M = p.N * p.Ho * p.Wo;
   constexpr int NS = NG * 4;
   constexpr int KOUT = NS * 32;
-  constexpr int STAGE = 2 * 32 * (128 + 16) + 128 * 4;   // igemm_epilogue_q8's LDS per wavefront at 128 channels
+  constexpr int PITCH = 128 + 16, TILE = 32 * PITCH;   // a staged [32 pixels][128 channels] byte tile
   const int n0 = blockIdx.y * KOUT;
 
   uintx4* wl = reinterpret_cast<uintx4*>(smem);                              // [NS][NKK][64] fragments
   int* bl = reinterpret_cast<int*>(smem + (size_t)NS * NKK * 1024);          // [KOUT] bias
-  unsigned char* stage = smem + (size_t)NS * NKK * 1024 + (size_t)KOUT * 4;  // NW staging areas
+  float* ml = reinterpret_cast<float*>(bl + KOUT);                           // [KOUT] multipliers
+  unsigned char* otile = reinterpret_cast<unsigned char*>(ml + KOUT) + wave * (2 * TILE);
+  unsigned char* rtile = otile + TILE;
   {
     const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag);
     constexpr int per_slice = NKK * 64;
@@ -217,11 +225,16 @@ igemm_stream_q8_rows_kernel(const IgemmParams p, const int groups, const int epi
       wl[u] = wf[(int64_t)(n0 / 32 + t) * p.wf_chunks * 64 + rem];
     }
     const int* bias = reinterpret_cast<const int*>(p.bias);
-    for (int c = tid; c < KOUT; c += NW * 64) bl[c] = bias != nullptr ? bias[n0 + c] : 0;
+    for (int c = tid; c < KOUT; c += NW * 64) {
+      bl[c] = bias != nullptr ? bias[n0 + c] : 0;
+      ml[c] = p.qmul[n0 + c];
+    }
   }
   __syncthreads();
 
   const int8_t* x = reinterpret_cast<const int8_t*>(p.x);
+  int8_t* ybase = reinterpret_cast<int8_t*>(p.y);
+  const int8_t* rbase = reinterpret_cast<const int8_t*>(p.residual);
   const int HoWo = p.Ho * p.Wo;
   const bool plain = p.sh == 1 && p.sw == 1 && p.Ho == p.H && p.Wo == p.W;
   auto load_b = [&](const int g, uintx4 (&b)[NKK]) {
@@ -239,35 +252,112 @@ igemm_stream_q8_rows_kernel(const IgemmParams p, const int groups, const int epi
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) b[kk] = xrow[2 * kk];
   };
+  // row passes: lane handles channels c16 .. c16 + 15 of pixel ps * 8 + rp
+  const int rp = lane >> 3, c16 = (lane & 7) * 16;
+  auto rreq = [&](const int g, const int grp, uintx4 (&r)[4]) {
+#pragma unroll
+    for (int ps = 0; ps < 4; ++ps) {
+      int m = (g * NW + wave) * 32 + ps * 8 + rp;
+      m = m < M ? m : M - 1;
+      r[ps] = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(rbase + (int64_t)m * p.rcs + n0 + grp * 128 + c16));
+    }
+  };
+  auto wave_fence = [&]() {
+    // a wavefront only touches its own tiles and its LDS operations complete in issue order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
 
-  uintx4 b[NKK], bnext[NKK];
-  if ((int)blockIdx.x < groups) load_b(blockIdx.x, b);
-  for (int g = blockIdx.x; g < groups; g += gridDim.x) {
-    const int gn = g + (int)gridDim.x;
-    if (gn < groups) load_b(gn, bnext);
-#pragma unroll 1
-    for (int grp = 0; grp < NG; ++grp) {
-      intx16 acc[1][4];
+  uintx4 b[NKK], bnext[NKK], rnx[4];
+#pragma unroll
+  for (int ps = 0; ps < 4; ++ps) rnx[ps] = uintx4{0u, 0u, 0u, 0u};
+  int g = blockIdx.x;   // (the launcher starts no more workgroups than there are pixel groups)
+  load_b(g, b);
+  if constexpr (kRes) rreq(g, 0, rnx);
+  for (; g < groups; g += gridDim.x) {
+    // (behind the last group a workgroup re-reads that group: a request that is always made is
+    //  one the compiler can count)
+    const int gn = g + (int)gridDim.x < groups ? g + (int)gridDim.x : g;
+    load_b(gn, bnext);
+    static_for<NG>([&](auto grp_no) __attribute__((always_inline)) {
+      constexpr int grp = decltype(grp_no)::value;
+      intx16 acc[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int* bj = bl + (grp * 4 + j) * 32 + lg * 4;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const intx4 bv = *reinterpret_cast<const intx4*>(bj + q * 8);
-          acc[0][j][q * 4 + 0] = bv.x; acc[0][j][q * 4 + 1] = bv.y; acc[0][j][q * 4 + 2] = bv.z; acc[0][j][q * 4 + 3] = bv.w;
+          acc[j][q * 4 + 0] = bv.x; acc[j][q * 4 + 1] = bv.y; acc[j][q * 4 + 2] = bv.z; acc[j][q * 4 + 3] = bv.w;
         }
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uintx4* wj = wl + (size_t)(grp * 4 + j) * NKK * 64 + lane;
 #pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) acc[0][j] = Mma<int8_t>::run(wj[kk * 64], b[kk], acc[0][j]);
+        for (int kk = 0; kk < NKK; ++kk) acc[j] = Mma<int8_t>::run(wj[kk * 64], b[kk], acc[j]);
       }
-      // pixels (g * NW + wave) * 32 + ..., channels n0 + grp * 128 + ...
-      igemm_epilogue_q8<NW * 32, 128, 32, 128, false, false>(p, epi_vec, acc, stage, g, 0, 0, M, wave, lane, n0 + grp * 128);
-    }
+      if constexpr (kRes) {
+        // this step's residual rows (settled before the stores of the step before) into LDS
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps)
+          *reinterpret_cast<uintx4*>(rtile + (ps * 8 + rp) * PITCH + c16) = q8_swz_chunk(rnx[ps], ps * 8 + rp);
+        wave_fence();
+        // the next step's: the other channel group of these pixels, or the first of the next pixels
+        if constexpr (grp + 1 < NG) rreq(g, grp + 1, rnx);
+        else rreq(gn, 0, rnx);
+      }
+      // requantise in the accumulator layout: lane holds, for pixel l32, channels j*32 + q*8 + lg*4 + (0..3)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ch = j * 32 + q * 8 + lg * 4;
+          const int off = (l32 * PITCH + ch) ^ q8_swz(l32);
+          const floatx4 m = *reinterpret_cast<const floatx4*>(ml + grp * 128 + ch);
+          const unsigned rs = kRes ? *reinterpret_cast<const unsigned*>(rtile + off) : 0u;
+          *reinterpret_cast<unsigned*>(otile + off) =
+              requant4<kRes, kClamp>(acc[j][q * 4 + 0], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3], m, rs, p);
+        }
+      wave_fence();
+      uintx4 v[4];
+#pragma unroll
+      for (int ps = 0; ps < 4; ++ps) v[ps] = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + (ps * 8 + rp) * PITCH + c16), ps * 8 + rp);
+      // everything requested is complete before the first store
+      if constexpr (kRes) {
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) epi_settle(rnx[ps]);
+      }
+      if constexpr (grp == 0) {
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) epi_settle(bnext[kk]);
+      }
+#pragma unroll
+      for (int ps = 0; ps < 4; ++ps) {
+        const int m = (g * NW + wave) * 32 + ps * 8 + rp;
+        if (m < M) store_row16(ybase + (int64_t)m * p.ycs + n0 + grp * 128 + c16, v[ps], true, 16, p.stream_out);
+      }
+      wave_fence();   // the tiles are written again by the next step
+    });
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) b[kk] = bnext[kk];
+  }
+}
+
+template <int NKK, int NG, int NW>
+__global__ void __launch_bounds__(NW * 64, 2)
+igemm_stream_q8_rows_kernel(const IgemmParams p, const int groups, const int epi_vec) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  (void)epi_vec;   // rows and bases are 16-byte aligned and the channels whole groups of 128 (checked by the launcher)
+  // (workgroup-uniform choices: the body is compiled once per case, so that none of its memory
+  //  requests sits in a branch)
+  if (p.residual != nullptr) {
+    if (p.q_lo > 0.f) stream_rows_body<NKK, NG, NW, true, true>(p, groups, smem);
+    else stream_rows_body<NKK, NG, NW, true, false>(p, groups, smem);
+  } else {
+    if (p.q_lo > 0.f) stream_rows_body<NKK, NG, NW, false, true>(p, groups, smem);
+    else stream_rows_body<NKK, NG, NW, false, false>(p, groups, smem);
   }
 }
 
@@ -339,7 +429,8 @@ static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream
   while (ng > 1 && (ng * 128 * p.C > 32 * 1024 || (ng != 1 && ng != 2))) ng = (ng % 2 == 0) ? ng / 2 : 1;
   const int nsplit = p.Kout / (ng * 128);
   const int64_t groups = (M + nw * 32 - 1) / (nw * 32);
-  const size_t lds = (size_t)ng * 4 * nkk * 1024 + (size_t)ng * 128 * 4 + (size_t)nw * (2 * 32 * 144 + 512);
+  // weights, bias and multipliers of the share, two staged byte tiles per wavefront
+  const size_t lds = (size_t)ng * 4 * nkk * 1024 + (size_t)ng * 128 * 8 + (size_t)nw * (2 * 32 * 144);
   if (groups > 0x7fffffff) return hipErrorInvalidValue;
   int per_cu = (int)((160 * 1024) / (lds + 512));
   per_cu = per_cu > 4 ? 4 : (per_cu < 1 ? 1 : per_cu);
