@@ -247,10 +247,16 @@ igemm_kernel(const IgemmParams p, const int epi_vec) {
 // wave*32 of a 256-channel tile), i.e. twice the MFMA work for the same pixel
 // fragments read from LDS and the same pixel requests; it pays for that with twice
 // the accumulators and weight fragments (two wavefronts per SIMD).
-template <typename TIn, typename Epi, int NJ>
+//
+// KS = 2: eight wavefronts in two groups of four, each group with its own ring and one half
+// of the K stages; the second group's accumulators are added to the first's through LDS
+// before the epilogue, which the first group runs alone.  For layers with fewer tiles than
+// compute units (13 x 13 feature maps at batch 16): their time is the latency chain of the K
+// stages of one workgroup, and two chains of half the length run side by side.
+template <typename TIn, typename Epi, int NJ, int KS = 1>
 // NJ = 1: three wavefronts per SIMD: at most 168 registers (two with the
 // transcendental activations in the epilogue, which need more)
-__global__ void __launch_bounds__(256, (EpiTraits<Epi>::rich || NJ == 2) ? 2 : 3)
+__global__ void __launch_bounds__(256 * KS, (EpiTraits<Epi>::rich || NJ == 2) ? 2 : 3)
 igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   constexpr int BM = 128, BN = 128 * NJ, WM = 128, NW = 4;
   constexpr int NWF = 4 * NJ;  // weight fragments of a wavefront per K stage
@@ -267,9 +273,11 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   // vmcnt(0), and vmcnt(2 * NWF + 4) = 12 / 20 for the wait at the top of a stage
   constexpr int kWaitVm0 = 0x0f70, kWaitVmStage = NJ == 1 ? 0x0f7c : 0x4f74;
 
-  // (8-bit results: the multipliers of the tile's channels wait behind the pixel ring)
+  // (8-bit results: the multipliers of the tile's channels wait behind the pixel rings)
   constexpr bool kMulLds = std::is_same<Epi, EpiQuant<0>>::value;
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[NBUF * BUF_BYTES + (kMulLds ? NJ * 512 : 0)];
+  constexpr int RING_BYTES = KS * NBUF * BUF_BYTES;
+  static_assert(KS == 1 || (KS == 2 && NJ == 1), "two K groups with one slice per wavefront only");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];   // RING_BYTES (+ NJ * 512 for the multipliers)
 
   const int tid = threadIdx.x;
   const int M = p.N * p.Ho * p.Wo;
@@ -282,8 +290,9 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   const int tile_n = bid % tiles_n;
   const int tile_m = bid / tiles_n;
   const int z = blockIdx.z;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = (tid >> 6) & 3, lane = tid & 63;   // wavefront within its K group
   const int l32 = lane & 31, lg = lane >> 5;
+  const int kg_u = KS == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 8);   // K group
 
   const TIn* x = reinterpret_cast<const TIn*>(p.x) + (int64_t)z * p.x_bs;
   // fragment q of a 32-channel slice: 1 KiB at wf[j] + q * 1024, this lane's 16 bytes at lane * 16.
@@ -307,7 +316,13 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   const TIn* fill_ptr = reinterpret_cast<const TIn*>(reinterpret_cast<const unsigned char*>(p.w_frag) +
                                                      (int64_t)p.batch * p.wf_tiles * p.wf_chunks * 1024);
 
-  const int nkt = p.wf_chunks / 4;
+  // (the launcher gives two K groups an even number of stages)
+  const int nkt = p.wf_chunks / 4 / KS;
+  const int kt0 = kg_u * nkt;   // this group's first stage
+  if constexpr (KS > 1) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) wf[j] += (int64_t)kt0 * 4096;
+  }
 
   // Weight fragment requests and their waits are issued by hand: next to the
   // direct-to-LDS loads the compiler would otherwise treat the vector-memory
@@ -384,7 +399,7 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   // and the tap walk is wavefront-uniform (scalar registers).  Per row the
   // thread keeps the address of its chunk at tap (0,0), channel 0 - possibly
   // outside the image - and one validity bit per tap.
-  const int row0 = tid >> 3;
+  const int row0 = (tid & 255) >> 3;
   const int kv = (lane & 7) ^ ((row0 >> 1) & 7);  // the chunk that belongs in this lane's slot
   const int RS = p.R * p.S;
   const TIn* a_row[A_IT];
@@ -421,9 +436,19 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
   unsigned tapbit = 1u;     // 1 << tap, 0 behind the last tap
   const int step_s = p.dw * p.xcs;                              // to the next tap of the row
   const int step_r = p.dh * p.W * p.xcs - (p.S - 1) * step_s;   // from the last tap of a row to the first of the next
+  if constexpr (KS > 1) {
+    // the walk starts at this group's first stage
+    const int e0 = kt0 * BK;          // elements of K before it
+    tap = e0 / p.C;
+    kc0 = e0 - tap * p.C;
+    const int tap_r = tap / p.S;
+    tap_s = tap - tap_r * p.S;
+    toff = (tap_r * p.dh * p.W + tap_s * p.dw) * p.xcs + kc0;
+    tapbit = tap < RS ? 1u << tap : 0u;
+  }
   const uint64_t fill_u = reinterpret_cast<uint64_t>(fill_ptr);
   auto dma = [&](const int buf) {
-    unsigned char* dst = smem + buf * BUF_BYTES + wave_u * 1024;
+    unsigned char* dst = smem + (kg_u * NBUF + buf) * BUF_BYTES + wave_u * 1024;
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) {
       const uint64_t live = reinterpret_cast<uint64_t>(a_row[i] + toff);
@@ -459,14 +484,16 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
     // out of the requantising epilogue, the busiest part of these layers.  Eight
     // 16-byte loads per slice, consumed right here: they are older than every
     // request the K loop counts, so its waits stay valid.
+    if (KS == 1 || kg_u == 0) {   // (once per tile: the second K group starts from zero)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) acc_init_bias_vec<TM, 1>(p, z, (tile_n * NJ + j) * 128 + wave_u * 32, lg, acc[j]);
+      for (int j = 0; j < NJ; ++j) acc_init_bias_vec<TM, 1>(p, z, (tile_n * NJ + j) * 128 + wave_u * 32, lg, acc[j]);
+    }
   }
   if constexpr (kMulLds) {
     // The multipliers of this wavefront's channels, into LDS behind the ring (requested
     // and consumed here, like the bias; read back by the same wavefront in the epilogue,
     // which then begins without a round trip to memory).
-    float* mt = reinterpret_cast<float*>(smem + NBUF * BUF_BYTES);
+    float* mt = reinterpret_cast<float*>(smem + RING_BYTES);
     const int last = p.Kout - 1;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -499,7 +526,7 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
     // every wavefront has also left stage kt-1, whose buffer is (kt+2) % 3
     dma(buf == 0 ? 2 : buf - 1);
     __builtin_amdgcn_sched_barrier(0);
-    const unsigned char* ab = smem + buf * BUF_BYTES + rd_base;
+    const unsigned char* ab = smem + (kg_u * NBUF + buf) * BUF_BYTES + rd_base;
     const int ktn = kt + 2 < nkt ? kt + 2 : nkt - 1;
     const unsigned char* wnext[NJ];
 #pragma unroll
@@ -566,10 +593,47 @@ igemm_wreg_kernel(const IgemmParams p, const int epi_vec) {
 #undef IGEMM_WRELOAD
 #undef IGEMM_WWAIT
 #undef IGEMM_WDRAIN8
+  if constexpr (KS == 2) {
+    // The second group's partial sums join the first's: 16 vectors per lane through the rings
+    // (64 KiB of them), which nobody reads any more once every wavefront has passed the first
+    // barrier.  Barriers for LDS traffic only, as in the epilogue.
+    using V4 = typename std::conditional<std::is_same<TIn, int8_t>::value, intx4, floatx4>::type;
+    auto lds_barrier = [&]() {
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    V4* red = reinterpret_cast<V4*>(smem) + (wave_u * 16) * 64 + lane;
+    lds_barrier();
+    if (kg_u == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          red[(i * 4 + q) * 64] = (V4){acc[0][i][0][q * 4 + 0], acc[0][i][0][q * 4 + 1], acc[0][i][0][q * 4 + 2], acc[0][i][0][q * 4 + 3]};
+    }
+    lds_barrier();
+    if (kg_u == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const V4 v = red[(i * 4 + q) * 64];
+          acc[0][i][0][q * 4 + 0] += v.x; acc[0][i][0][q * 4 + 1] += v.y;
+          acc[0][i][0][q * 4 + 2] += v.z; acc[0][i][0][q * 4 + 3] += v.w;
+        }
+    }
+    lds_barrier();   // the sums are read: the rings become the epilogue's staging area
+    // (a wavefront that has ended no longer counts at the workgroup's barriers)
+    if (kg_u == 1) return;
+  }
 #pragma unroll
   for (int j = 0; j < NJ; ++j)
     igemm_epilogue_rows128<TIn, Epi>(p, epi_vec, acc[j], smem, tile_m, tile_n * NJ + j, z, M, wave, lane,
-                                     kMulLds ? reinterpret_cast<const float*>(smem + NBUF * BUF_BYTES) + j * 128 : nullptr);
+                                     kMulLds ? reinterpret_cast<const float*>(smem + RING_BYTES) + j * 128 : nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -892,6 +956,24 @@ int wreg_slices(const IgemmParams& p) {
   return 1;
 }
 
+// K groups of the weights-in-registers kernel (one slice per wavefront): two where the launch has
+// fewer workgroups than the chip has compute units and the K loop is long enough to be worth
+// splitting (an even number of stages, at least 24: measured on YOLOv3 at batch 16, 72 stages
+// 53 -> 46 us, 16 stages unchanged, 8 stages 14.6 -> 16 .. 21 us).
+int wreg_k_groups(const IgemmParams& p, const int64_t workgroups) {
+  const int64_t stages = (int64_t)p.wf_chunks / 4;
+  const bool legal = stages % 2 == 0 && stages >= 4;
+  if (const char* force = getenv("ODLA_HIP_WREG_KSPLIT")) {  // tuning aid: 0 = never, 2 = wherever legal
+    const int v = atoi(force);
+    if (v == 0) return 1;
+    if (v == 2) return legal ? 2 : 1;
+  }
+  // (fp32 layers keep one summation chain per result: their parity bound is relative to single
+  //  results, which a second chain's rounding can exceed where a sum nearly cancels)
+  if (p.in_dt == DT_F32) return 1;
+  return legal && stages >= 24 && workgroups <= 256 ? 2 : 1;
+}
+
 template <typename TIn, typename Epi>
 hipError_t launch_wreg(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
@@ -901,14 +983,29 @@ hipError_t launch_wreg(const IgemmParams& p, int epi_vec, hipStream_t stream) {
   const int nj = EpiTraits<Epi>::rich ? 1 : wreg_slices(p);
   const int64_t tiles = ((M + 127) / 128) * ((p.Kout + 128 * nj - 1) / (128 * nj));
   if (tiles <= 0 || tiles > 0x7fffffff) return hipErrorInvalidValue;
+  // pixel ring(s) and, for 8-bit results, the tile's multipliers
+  constexpr size_t ring = 3 * 128 * 128;
+  constexpr size_t mul = std::is_same<Epi, EpiQuant<0>>::value ? 512 : 0;
   if constexpr (!EpiTraits<Epi>::rich) {
     if (nj == 2) {
-      hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 2>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0,
-                         stream, p, epi_vec);
+      hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 2>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256),
+                         ring + 2 * mul, stream, p, epi_vec);
+      return hipGetLastError();
+    }
+    if (wreg_k_groups(p, tiles * p.batch) == 2) {
+      static bool ready = false;   // (repeating the call is harmless: no lock)
+      if (!ready) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_wreg_kernel<TIn, Epi, 1, 2>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * ring + mul));
+        if (e != hipSuccess) return e;
+        ready = true;
+      }
+      hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 1, 2>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(512),
+                         2 * ring + mul, stream, p, epi_vec);
       return hipGetLastError();
     }
   }
-  hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 1>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), 0,
+  hipLaunchKernelGGL((igemm_wreg_kernel<TIn, Epi, 1>), dim3((unsigned)tiles, 1, (unsigned)p.batch), dim3(256), ring + mul,
                      stream, p, epi_vec);
   return hipGetLastError();
 }
@@ -1063,7 +1160,14 @@ const char* igemm_variant_name(const IgemmParams& p) {
   if (p.w_frag != nullptr && igemm_stream_q8_geometry(p)) return "stream";
   if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
   if (p.w_frag != nullptr && taps_shape(p).nkk > 0) return "128x64t";
-  if (p.w_frag != nullptr && wreg_shape(p)) return "128x128w";
+  if (p.w_frag != nullptr && wreg_shape(p)) {
+    const bool rich = p.act == ACT_GELU_ERF || p.act == ACT_GELU_TANH || p.act == ACT_SIGMOID || p.act == ACT_TANH;
+    const int nj = rich ? 1 : wreg_slices(p);
+    const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
+    const int64_t tiles = ((M + 127) / 128) * ((p.Kout + 128 * nj - 1) / (128 * nj));
+    if (!rich && nj == 1 && wreg_k_groups(p, tiles * p.batch) == 2) return "128x128w2k";   // two K groups per workgroup
+    return "128x128w";
+  }
   return choose_variant(p).name;
 }
 

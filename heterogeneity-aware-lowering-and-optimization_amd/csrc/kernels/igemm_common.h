@@ -640,12 +640,16 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // this slice's operands from memory are complete before its first store (see epi_settle)
-    if (i == 0) {
+    // this slice's operands from memory are complete before its first store (see epi_settle;
+    // not in the instantiations with the wider activation set, which have no registers to spare)
+    if (i == 0 && !EpiTraits<Epi>::rich) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { epi_settle(b8[e]); epi_settle(m8[e]); }
+      for (int e = 0; e < 8; ++e) {
+        if constexpr (EpiTraits<Epi>::quant) epi_settle(m8[e]);
+        else epi_settle(b8[e]);
+      }
     }
-    if constexpr (Epi::kPrefetchResidual) {
+    if constexpr (Epi::kPrefetchResidual && !EpiTraits<Epi>::rich) {
 #pragma unroll
       for (int ps = 0; ps < NPASS; ++ps) epi_settle(rcur[ps]);
     }
@@ -894,7 +898,10 @@ __device__ __forceinline__ void igemm_epilogue_rows128(const IgemmParams& p, con
   lds_barrier();  // the K loop's LDS reads are done; the ring becomes the staging area
   // every operand requested from memory above is complete before the first store (see epi_settle)
 #pragma unroll
-  for (int e = 0; e < 8; ++e) { epi_settle(b8[e]); epi_settle(m8[e]); }
+  for (int e = 0; e < 8; ++e) {
+    if constexpr (EpiTraits<Epi>::quant) epi_settle(m8[e]);
+    else epi_settle(b8[e]);
+  }
   if constexpr (Epi::kPrefetchResidual && kSettleRes) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)

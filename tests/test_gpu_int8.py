@@ -110,6 +110,14 @@ def test_q8_conv_two_channel_slices_per_wavefront(case, odla, ref, monkeypatch):
     test_q8_conv_accumulators_and_requant(case, odla, ref)
 
 
+@pytest.mark.parametrize("case", [c for c in Q8_CONV_CASES if c[1] % 128 == 0])
+def test_q8_conv_two_k_groups_per_workgroup(case, odla, ref, monkeypatch):
+    """Weights-in-registers kernel with two K groups per workgroup, 8-bit operands: the int32
+    partial sums of the second group join the first's (which carry the bias) through LDS."""
+    monkeypatch.setenv("ODLA_HIP_WREG_KSPLIT", "2")
+    test_q8_conv_accumulators_and_requant(case, odla, ref)
+
+
 @pytest.mark.parametrize("tiles_per_wg", [0, 3, -1])
 @pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (3, 128, 7, 7, 200), (4, 64, 21, 19, 256), (2, 128, 30, 30, 512),
                                   (3, 256, 9, 9, 136), (2, 64, 17, 9, 128), (1, 128, 40, 40, 384)])

@@ -178,6 +178,51 @@ def test_conv_two_channel_slices_per_wavefront(case, mode, monkeypatch):
     test_conv_parity(case, mode)
 
 
+K_GROUP_CASES = [
+    # N, C, H, W, O, k, stride, pad, group, dilation: an even number of 128-byte K stages in
+    # every mode, ragged pixel and channel tiles, a tap boundary inside the second group's half
+    (2, 128, 13, 13, 256, 3, 1, 1, 1, 1),
+    (1, 256, 13, 13, 200, 1, 1, 0, 1, 1),
+    (2, 128, 9, 9, 160, 3, 2, 1, 1, 1),
+    (1, 128, 7, 7, 130, 3, 1, 2, 1, 2),
+    (3, 64, 6, 6, 136, 2, 1, 0, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", K_GROUP_CASES + [c for c in CONV_CASES if c[1] % 64 == 0 and c[8] == 1 and c[4] > 64])
+@pytest.mark.parametrize("mode", ["fp32", "fp16", "bf16"])
+def test_conv_two_k_groups_per_workgroup(case, mode, monkeypatch):
+    """The weights-in-registers kernel with eight wavefronts in two K groups (each half of the
+    K stages, summed through LDS), which the library picks by itself for launches with fewer
+    workgroups than compute units; forced here wherever the stage count is even."""
+    monkeypatch.setenv("ODLA_HIP_WREG_KSPLIT", "2")
+    test_conv_parity(case, mode)
+
+
+def test_small_launch_takes_two_k_groups_by_itself():
+    """A 3x3 layer over a 13 x 13 map at batch 2 (6 workgroups, 36 K stages in fp16) is given
+    the two-group form without being asked, with a fused residual and LeakyReLU."""
+    from test_gpu_taps_kernel import run_logged
+    N, C, H, W, O = 2, 256, 13, 13, 256
+    r = rng(77)
+    w = (r.standard_normal((O, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    bias = r.standard_normal(O).astype(np.float32)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    res = r.standard_normal((N, O, H, W)).astype(np.float32)
+
+    def build(b):
+        v = b.arg("x", (N, C, H, W))
+        sc = b.arg("res", (N, O, H, W))
+        y = b.conv(v, b.const("w", w), b.const("b", bias), (1, 1), (1, 1, 1, 1), (1, 1), 1, name="y")
+        y = b.leaky_relu(y, 0.1, name="act")
+        b.output(b.add(y, sc, name="sum"), "sum")
+
+    announce("conv two K groups by default")
+    (got, want), seen = run_logged(lambda: run_both(build, {"x": x, "res": res}, fp16=True))
+    assert any(m.endswith("kernel 128x128w2k") for m in seen), [m for m in seen if "kernel" in m]
+    assert np.max(np.abs(got["sum"] - want["sum"])) <= 2e-2 * max(1.0, float(np.max(np.abs(want["sum"]))))
+
+
 LEAN_CASES = [
     # 1x1 filters over 64 / 128 bytes of input channels per pixel (the streaming kernel):
     # N, C, H, W, O, stride, residual

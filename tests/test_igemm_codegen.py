@@ -71,11 +71,13 @@ def test_weight_fragment_registers_untouched_in_flight(compiled):
     checked = 0
     for name, body in kernel_bodies(asm, "_ZN4ohip17igemm_wreg_kernel"):
         quads = {(int(m.group(1)), int(m.group(2))) for m in map(req.match, body) if m}
-        # Two sets of four fragments per 32-channel slice (the last template
-        # argument: one or two slices per wavefront), each tied to one register
-        # quad for the whole K loop (also in stages the optimizer peels off the loop).
-        slices = int(re.search(r"Li(\d)EEEvNS_11IgemmParamsEi$", name).group(1))
-        assert slices in (1, 2), name
+        # Two sets of four fragments per 32-channel slice (the last two template
+        # arguments: one or two slices per wavefront, one or two K groups per
+        # workgroup), each tied to one register quad for the whole K loop (also in
+        # stages the optimizer peels off the loop).
+        targs = re.search(r"Li(\d)ELi(\d)EEEvNS_11IgemmParamsEi$", name)
+        slices, k_groups = int(targs.group(1)), int(targs.group(2))
+        assert slices in (1, 2) and k_groups in (1, 2), name
         assert len(quads) == 8 * slices, (name, quads)
         owned = {x for a, b in quads for x in range(a, b + 1)}
         assert len(owned) == 32 * slices, (name, quads)
