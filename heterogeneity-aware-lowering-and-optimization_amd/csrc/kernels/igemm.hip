@@ -699,6 +699,9 @@ igemm_lean_kernel(const IgemmParams p, const int epi_vec, const int tiles_per_wg
   uintx4 a_cur[NKK], a_nxt[NKK];
   load_a(tm0, a_cur);
   for (int tile_m = tm0; tile_m < tm1; ++tile_m) {
+    // (requested only where a next tile exists: a workgroup walks two or three tiles, and re-reading
+    //  the last one instead - which would let the compiler count the requests in flight - costs more
+    //  than the wait it saves: 64 -> 256 + residual at 56 x 56, fp16, 175 -> 186 us)
     if (tile_m + 1 < tm1) load_a(tile_m + 1, a_nxt);
     // 64 channels at a time: half the accumulator registers, half the staging space
 #pragma unroll
@@ -854,7 +857,8 @@ igemm_taps_kernel(const IgemmParams p, const int epi_vec, const int tiles_per_wg
 #pragma unroll
       for (int j = 0; j < NJ; ++j) acc[0][j] = Mma<TIn>::run(w[j][kk], a[kk], acc[0][j]);
     // the operand registers are free again: the next tile's pixels travel during the epilogue
-    if (tile_m + 1 < tm1) load_a(tile_m + 1);
+    // (always requested: the last tile re-reads itself)
+    load_a(tile_m + 1 < tm1 ? tile_m + 1 : tile_m);
     igemm_epilogue<TIn, Epi, BM, BN, 32, WN, false, true>(pe, epi_vec, acc, smem, tile_m, tile_n, 0, M, wave, lane, 0);
     // the same wavefront parks into its slice again next: order it behind the read-back
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
