@@ -230,8 +230,19 @@ def run_workload(pkg, L, name, args, with_cpu):
     sess = hb.session(use_graph=True)
     sess.bind_device_io(wl.feeds)
 
-    for _ in range(args.warmup):
-        sess.execute()
+    # the library says (at INFO level) when it runs a batch as two half-batch copies side by side
+    said = []
+    LOGCB = ctypes.CFUNCTYPE(None, ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p)
+    cb = LOGCB(lambda f, line, fn_, lvl, msg: said.append(msg.decode(errors="replace")))
+    L.odla_SetLogger(ctypes.cast(cb, ctypes.c_void_p))
+    L.odla_SetLogLevel(4)
+    try:
+        for _ in range(args.warmup):
+            sess.execute()
+    finally:
+        L.odla_SetLogLevel(2)
+        L.odla_SetLogger(None)
+    halves = any("two halves side by side" in m for m in said)
     # odla_ExecuteComputation returns after the device is idle, so the wall
     # clock around K executions is the device-synchronised time of K steps.
     t0 = time.perf_counter()
@@ -261,7 +272,8 @@ def run_workload(pkg, L, name, args, with_cpu):
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": DTYPE[mode], "data": "synthetic",
         "config": {"workload": wl.desc, "batch": wl.batch,
-                   "executor": "hipGraph replay through odla_ExecuteComputation"},
+                   "executor": "hipGraph replay through odla_ExecuteComputation"
+                               + (": two half-batch copies of the plan side by side on two streams" if halves else "")},
         "roofline": roof, "cpu_baseline": cpu, "end_to_end": e2e,
     }
     sess.close()

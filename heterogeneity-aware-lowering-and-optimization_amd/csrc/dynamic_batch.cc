@@ -28,10 +28,14 @@ struct Rescaler {
 
   bool carry(const _odla_value* v) const { return v != nullptr && carries[v->index] != 0; }
 
+  bool quiet = false;   // a refusal is not an error: the caller has another way to run the computation
+
   void reject(const Node& n, const char* why) {
-    if (ok)
+    if (ok && !quiet)
       OHIP_ERR("dynamic batch: %s '%s' %s; run this computation at its recorded batch %lld", api_op_name(n),
                n.out ? n.out->name.c_str() : "", why, (long long)from);
+    else if (ok)
+      OHIP_DEBUG("batch halves: %s '%s' %s", api_op_name(n), n.out ? n.out->name.c_str() : "", why);
     ok = false;
   }
   bool scalable(int64_t d) const { return d % from == 0; }
@@ -47,15 +51,16 @@ struct Rescaler {
 
 }  // namespace
 
-std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, int64_t from, int64_t to) {
+std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, int64_t from, int64_t to, bool rows_apart) {
   if (from <= 0 || to <= 0) return nullptr;
   Rescaler rs{c, from, to, std::vector<char>(c.values.size(), 0)};
+  rs.quiet = rows_apart;
 
   bool flagged = false;
   for (const _odla_value* a : c.args) flagged = flagged || a->dyn_batch;
   for (const _odla_value* a : c.args) {
     if (a->eager) {
-      OHIP_ERR("dynamic batch: values made by odla_CreateValue have no batch");
+      if (!rows_apart) OHIP_ERR("dynamic batch: values made by odla_CreateValue have no batch");
       return nullptr;
     }
     // without an explicit -1 every argument's leading extent is the batch, as in the reference
@@ -121,6 +126,8 @@ std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, i
       case OP_CONCAT:
         for (const _odla_value* v : n.in)
           if (!rs.carry(v)) rs.reject(n, "joins the batch with a constant");
+        // (batches laid end to end: the rows of one half of the batch are not one half of the result)
+        if (rows_apart && n.i[0] == 0) rs.reject(n, "joins along the batch");
         break;
       case OP_GATHER:
         if (rs.carry(n.in[0]) && (n.i[0] == 0 || rs.carry(n.in[1]))) rs.reject(n, "gathers along the batch");
@@ -162,9 +169,13 @@ std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, i
       case OP_QUANTIZE: case OP_DEQUANTIZE:
         for (size_t k = 1; k < n.in.size(); ++k)
           if (rs.carry(n.in[k])) rs.reject(n, "has a scale that depends on the batch");
+        if (n.i[0] == 0 && n.in.size() > 1 && n.in[1] != nullptr && n.in[1]->shape.numel() > 1)
+          rs.reject(n, "has one scale per row of the batch");
         break;
       case OP_NMS:
         if (!rs.carry(n.in[0]) || !rs.carry(n.in[1])) rs.reject(n, "has boxes or scores that do not depend on the batch");
+        // (its result lists image numbers, and the images' detections follow each other without gaps)
+        if (rows_apart) rs.reject(n, "numbers the images of the batch in its result");
         break;
       case OP_UNARY: case OP_POOL: case OP_CAST: case OP_RESHAPE: case OP_RESIZE: case OP_LRN:
         break;

@@ -283,6 +283,15 @@ struct _odla_context {
   };
   std::map<int, Variant> variant_ctx;
   uint64_t variant_clock = 0;
+  // Two contexts over ONE copy of the recording at half the batch, executed side by side on
+  // their own streams, each on its half of the caller's buffers (see execute_split).
+  struct Split {
+    bool tried = false, ok = false;
+    std::shared_ptr<_odla_computation> comp;
+    _odla_context* half[2] = {nullptr, nullptr};
+  } split;
+  bool is_half = false;   // this context is one of those halves: it runs as it is
+  bool last_split = false;   // the last execution ran as halves: results live in their arenas / the caller's buffers
 };
 
 struct _odla_device {
@@ -301,7 +310,11 @@ int recorded_batch(const _odla_computation& c);
 // A copy of the recording of `c` in which every value that depends on an
 // argument has its leading extent rescaled from `from` to `to`; nullptr (and a
 // log line) when the graph moves the batch out of the leading position.
-std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, int64_t from, int64_t to);
+// rows_apart: the copy is to run on one part of the batch while another copy runs on the rest, so
+// the graph must also keep the rows of different images apart in every result (refusals are then
+// logged at debug level only).
+std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, int64_t from, int64_t to,
+                                                   bool rows_apart = false);
 }  // namespace ohip
 
 #endif

@@ -110,6 +110,14 @@ def test_q8_conv_two_channel_slices_per_wavefront(case, odla, ref, monkeypatch):
     test_q8_conv_accumulators_and_requant(case, odla, ref)
 
 
+@pytest.mark.parametrize("dims", [(2, 32, 8, 8, 64), (4, 64, 21, 19, 256), (2, 128, 30, 30, 512)])
+def test_q8_two_half_batches_side_by_side(dims, odla, ref, monkeypatch):
+    """The 8-bit residual block executed as two half-batch copies on two streams: bit-equal to
+    the oracle like the whole batch (every image's arithmetic is its own)."""
+    monkeypatch.setenv("ODLA_HIP_BATCH_SPLIT", "2")
+    test_q8_residual_fused_equals_unfused_equals_oracle(dims, 0, odla, ref, monkeypatch)
+
+
 @pytest.mark.parametrize("case", [c for c in Q8_CONV_CASES if c[1] % 128 == 0])
 def test_q8_conv_two_k_groups_per_workgroup(case, odla, ref, monkeypatch):
     """Weights-in-registers kernel with two K groups per workgroup, 8-bit operands: the int32
