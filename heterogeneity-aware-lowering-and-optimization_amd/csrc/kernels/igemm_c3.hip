@@ -94,7 +94,7 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
     const int blk = tid >> 5, l = tid & 31;
     const int br = l / g.bc, bc = l - br * g.bc;
     const int yy = y0 + blk * g.br + br, xx = x0 + bc;
-    mtab[tid] = (l < g.br * g.bc && yy < p.H) ? (n_img * p.H + yy) * p.W + xx : -1;
+    mtab[tid] = (l < g.br * g.bc && yy < p.H && xx < p.W) ? (n_img * p.H + yy) * p.W + xx : -1;
   }
 
   // this thread's patch pixels: tid, tid + NT, ..
@@ -326,11 +326,17 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
   int force_bc = 0;
   if (const char* e = getenv("ODLA_HIP_C3_BC")) force_bc = atoi(e);   // tuning aid: block columns
   for (int bc = 32; bc >= 4; --bc) {
-    if (p.W % bc != 0 || (force_bc > 0 && p.W % force_bc == 0 && bc != force_bc)) continue;
+    // Blocks of 16 or 32 columns may hang over the right edge (a 14-column image as one block
+    // of 16: each half of a wavefront then reads 16 consecutive slots of one patch row - no
+    // second LDS pass - where 2 x 14 blocks wrap two lanes into the next row); other widths
+    // must divide the image's.
+    const bool over = (bc == 16 || bc == 32) && p.W % bc != 0;
+    if ((p.W % bc != 0 && !over) || (force_bc > 0 && (p.W % force_bc == 0 || force_bc == 16 || force_bc == 32) && bc != force_bc)) continue;
     int br = 32 / bc;
     if (br > p.H) br = p.H;
     const int th = 4 * br, ty = (p.H + th - 1) / th;
-    const float eff = (float)(br * bc) / 32.f * (float)p.H / (float)(ty * th);
+    const int tx = (p.W + bc - 1) / bc;
+    const float eff = (float)(br * bc) / 32.f * (float)p.H / (float)(ty * th) * (float)p.W / (float)(tx * bc);
     const int npp = (th + 2) * (bc + 2);
     if (npp > kC3Plane / 16) continue;
     const float halo = (float)npp / (float)(th * bc);
@@ -338,7 +344,7 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
     if (score > best_score + 1e-6f || (score > best_score - 1e-6f && halo < best_halo)) {
       g.eff = eff; best_halo = halo; best_score = score;
       g.br = br; g.bc = bc; g.pw = bc + 2; g.npp = npp;
-      g.tiles_x = p.W / bc; g.tiles_y = ty;
+      g.tiles_x = tx; g.tiles_y = ty;
     }
   }
   float min_eff = 0.7f;

@@ -33,6 +33,8 @@ FLOAT_CASES = [
     case(1, 64, 40, 104, 64, "add"),          # wide image, 8 x 4 blocks
     case(1, 128, 16, 16, 384, "add_relu"),    # three channel tiles (of two wavefronts x two slices with ODLA_HIP_C3_SLICES=2)
     case(2, 64, 12, 28, 512, "leaky"),        # four channel tiles (two of four wavefronts x two slices)
+    case(1, 64, 11, 26, 128, "add_relu"),     # 26 columns in one block of 32 that hangs over the right edge
+    case(2, 128, 6, 30, 128, "leaky_add"),    # 30 of 32
 ]
 
 INT8_CASES = [
@@ -43,6 +45,8 @@ INT8_CASES = [
     case(1, 128, 9, 16, 64, "none"),
     case(1, 64, 16, 16, 256, "relu"),         # 64-byte rows
     case(2, 256, 10, 28, 512, "relu"),
+    case(1, 128, 11, 26, 128, "relu"),        # a block of 32 columns over a 26-column image
+    case(2, 64, 7, 30, 128, "none"),
 ]
 
 
