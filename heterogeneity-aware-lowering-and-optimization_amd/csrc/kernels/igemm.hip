@@ -961,7 +961,7 @@ int wreg_slices(const IgemmParams& p) {
 }
 
 // K groups of the weights-in-registers kernel (one slice per wavefront): two where the launch has
-// fewer workgroups than the chip has compute units and the K loop is long enough to be worth
+// far fewer workgroups than the chip has compute units and the K loop is long enough to be worth
 // splitting (an even number of stages, at least 24: measured on YOLOv3 at batch 16, 72 stages
 // 53 -> 46 us, 16 stages unchanged, 8 stages 14.6 -> 16 .. 21 us).
 int wreg_k_groups(const IgemmParams& p, const int64_t workgroups) {
@@ -975,7 +975,11 @@ int wreg_k_groups(const IgemmParams& p, const int64_t workgroups) {
   // (fp32 layers keep one summation chain per result: their parity bound is relative to single
   //  results, which a second chain's rounding can exceed where a sum nearly cancels)
   if (p.in_dt == DT_F32) return 1;
-  return legal && stages >= 24 && workgroups <= 256 ? 2 : 1;
+  // (at most 180 workgroups: a workgroup of this form takes a compute unit's LDS for itself, and
+  //  when two half-batch copies of a plan run side by side the other copy's launch wants the
+  //  units this one leaves - BERT-base halves of 32 sequences, 192 workgroups of 48 stages,
+  //  2.36 -> 2.43 ms per step with it)
+  return legal && stages >= 24 && workgroups <= 180 ? 2 : 1;
 }
 
 template <typename TIn, typename Epi>
