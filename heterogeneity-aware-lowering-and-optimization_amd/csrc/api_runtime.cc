@@ -2,6 +2,7 @@
 // execution (hipGraph replay), value introspection, device / memory / logging.
 #include <atomic>
 #include <cstdlib>
+#include <chrono>
 #include <cstring>
 
 #include "internal.h"
@@ -231,6 +232,7 @@ odla_status run_steps(_odla_context* ctx, const Plan& plan, char* arena, const s
   env.base[SP_ARENA] = arena;
   env.base[SP_CONST] = plan.const_pool;
   env.ext = ext != nullptr && !ext->empty() ? ext->data() : nullptr;
+  env.image_base = ctx->image_base;
   for (const Step& s : plan.steps) {
     hipError_t e = s.fn(env, ctx->stream);
     if (e != hipSuccess) {
@@ -338,8 +340,8 @@ void destroy_context_tree(_odla_context* ctx) {
   delete ctx;
 }
 
-// Batch from which an execution is split into two halves by default (see split_threshold).
-constexpr int kDefaultSplitBatch = 64;
+// Smallest batch at which a context tries two half-batch copies against the whole batch (see split_threshold).
+constexpr int kMinTrialBatch = 8;
 
 // Batches (other than the recorded one) a context keeps planned at a time.
 int max_batch_variants() {
@@ -657,7 +659,7 @@ odla_status odla_BindToOutputById(const odla_value_id id, odla_void* data_ptr, o
 
 namespace {
 
-odla_status execute_impl(odla_context ctx, odla_compute_mode mode, odla_device device, bool wait);
+odla_status execute_impl(odla_context ctx, odla_compute_mode mode, odla_device device, bool wait, bool whole = false);
 
 // Leading extent shared by every argument of `c` (the batch, as in the reference's runtimes), 0 if
 // there is none.
@@ -671,17 +673,21 @@ int64_t common_batch(const _odla_computation& c) {
   return b;
 }
 
-// From which batch on an execution is split in two halves that run side by side (0: never).
-// A network's launches alternate between bandwidth-bound and MFMA-bound ones and each runs as
-// few rounds of workgroups with a serial head and tail; two half-batch replicas on two streams
-// fill each other's gaps.  Measured on one box, whole batch against two halves: ResNet-50 int8
-// at batch 512 / 256 / 128 / 32: +4.2 / +3.8 / +1.6 / -4.2 %; fp16 at 256 / 128 / 64 / 8: +5.9 /
-// +3.9 / +6.5 / -7.3 %; BERT-base bf16 at 64 / 16 sequences: +8.7 / -8.6 %.  Hence from batch 64
-// on, for plans of at least 16 launches (two graph launches and two waits cost ~10 us).
-// ODLA_HIP_BATCH_SPLIT = 0 turns it off, n > 0 sets the batch it starts at.
-int64_t split_threshold() {
+// An execution as two half-batch copies side by side.  A network's launches alternate between
+// bandwidth-bound and MFMA-bound ones and each runs as few rounds of workgroups with a serial head
+// and tail; two half-batch replicas on two streams fill each other's gaps.  Whether that beats
+// the smaller, less efficient launches of a half batch depends on the work per image.  Measured
+// on one box, whole batch against two halves: ResNet-50 int8 at batch 512 / 256 / 128 / 32: +4.2 /
+// +3.8 / +1.6 / -4.2 %; fp16 at 256 / 128 / 64 / 8: +5.9 / +3.9 / +6.5 / -7.3 %; BERT-base bf16 at
+// 64 / 16 sequences: +8.7 / -8.6 %; YOLOv3 fp16 at 16 images of 416 x 416: +8.8 %.  So a context
+// measures (see _odla_context::Split) unless ODLA_HIP_BATCH_SPLIT decides: 0 = never, n > 0 =
+// always from batch n on.  Plans of fewer than 16 launches and batches below 8 are not tried
+// (two graph launches and two waits cost ~10 us).
+// Returns the threshold (0: never) and whether it came from the environment.
+int64_t split_threshold(bool* forced) {
   const char* e = getenv("ODLA_HIP_BATCH_SPLIT");   // (read per execution: a test switches it)
-  if (e == nullptr || e[0] == 0) return (int64_t)kDefaultSplitBatch;
+  *forced = e != nullptr && e[0] != 0;
+  if (!*forced) return (int64_t)kMinTrialBatch;
   return (int64_t)atoll(e);
 }
 
@@ -700,7 +706,15 @@ odla_status execute_split(_odla_context* ctx, odla_compute_mode mode, odla_devic
   for (const Plan::IO& io : plan.outputs)
     if (ctx->bound_out.find(io.v) == ctx->bound_out.end()) return ODLA_SUCCESS;
   if (!plan.stat_recs.empty()) return ODLA_SUCCESS;   // (value statistics are collected on the whole batch)
-  if (plan.steps.size() < 16 && getenv("ODLA_HIP_BATCH_SPLIT") == nullptr) return ODLA_SUCCESS;   // too short to gain
+  // A result buffer that overlaps an argument buffer: one half could write (in place) what the
+  // other still reads.  The whole batch has its own guard for that case.
+  for (const Plan::IO& in : plan.inputs) {
+    const char* a0 = static_cast<const char*>(ctx->bound_in[in.v]);
+    for (const Plan::IO& out : plan.outputs) {
+      const char* b0 = static_cast<const char*>(ctx->bound_out[out.v]);
+      if (a0 < b0 + out.bytes && b0 < a0 + in.bytes) return ODLA_SUCCESS;
+    }
+  }
   if (!sp.tried) {
     sp.tried = true;
     const int64_t B = common_batch(*c);
@@ -727,11 +741,12 @@ odla_status execute_split(_odla_context* ctx, odla_compute_mode mode, odla_devic
         return ODLA_SUCCESS;
       }
       sub->is_half = true;
+      sub->image_base = ctx->image_base + k * (int)(B / 2);
       sp.half[k] = sub;
     }
     sp.comp = std::move(v);
     sp.ok = true;
-    OHIP_INFO("odla_ExecuteComputation: batch %lld runs as two halves side by side", (long long)B);
+    OHIP_DEBUG("odla_ExecuteComputation: two half-batch copies of batch %lld planned", (long long)B);
   }
   *handled = true;
   const Plan& hp = *sp.comp->plan;
@@ -792,15 +807,70 @@ odla_status odla_ExecuteComputation(const odla_computation comp, const odla_cont
 
 namespace {
 
-odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, odla_device device, const bool wait) {
+// whole: run the batch as it is (no half-batch copies, no measuring)
+odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, odla_device device, const bool wait, const bool whole) {
   (void)device;
   if (mode == ODLA_COMPUTE_TRAINING) return ODLA_UNSUPPORTED_OP;
   _odla_computation* c = ctx->comp;
-  if (!ctx->is_half && split_threshold() > 0 && (ctx->run_batch == 0 || ctx->run_batch == recorded_batch(*c)) &&
-      common_batch(*c) >= split_threshold()) {
-    bool handled = false;
-    const odla_status st = execute_split(ctx, mode, device, &handled);
-    if (handled) return st;
+  if (!whole && !ctx->is_half && (ctx->run_batch == 0 || ctx->run_batch == recorded_batch(*c))) {
+    bool forced = false;
+    const int64_t from = split_threshold(&forced);
+    const int64_t B = from > 0 ? common_batch(*c) : 0;
+    _odla_context::Split& sp = ctx->split;
+    if (from > 0 && B >= from && forced) {
+      // the environment decides: halves wherever they apply
+      bool handled = false;
+      const odla_status st = execute_split(ctx, mode, device, &handled);
+      if (handled) {
+        if (sp.choice != 2) OHIP_INFO("odla_ExecuteComputation: batch %lld runs as two halves side by side", (long long)B);
+        sp.choice = 2;
+        return st;
+      }
+    } else if (from > 0 && B >= from && c->plan && c->plan->steps.size() >= 16 && sp.choice != 1) {
+      if (sp.choice == 2) {
+        bool handled = false;
+        const odla_status st = execute_split(ctx, mode, device, &handled);
+        if (handled) return st;
+      } else if (wait) {
+        // measuring: executions 1-3 whole, 4-6 in halves; the first of each three captures its
+        // graph, the faster of the other two counts
+        const int t = sp.trial;
+        const auto t0 = std::chrono::steady_clock::now();
+        odla_status st = ODLA_SUCCESS;
+        bool handled = true;
+        if (t < 3) {
+          st = execute_impl(ctx, mode, device, wait, /*whole=*/true);
+        } else {
+          st = execute_split(ctx, mode, device, &handled);
+        }
+        if (!handled) {
+          sp.choice = 1;   // does not apply to this graph or these bindings: whole from now on
+        } else {
+          const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+          if (st != ODLA_SUCCESS) return st;
+          if (t == 1) sp.whole_ms = ms;
+          if (t == 2 && ms < sp.whole_ms) sp.whole_ms = ms;
+          if (t == 4) sp.halves_ms = ms;
+          if (t == 5 && ms < sp.halves_ms) sp.halves_ms = ms;
+          sp.trial = t + 1;
+          if (sp.trial == 6) {
+            sp.choice = sp.halves_ms < 0.98 * sp.whole_ms ? 2 : 1;
+            if (sp.choice == 2)
+              OHIP_INFO("odla_ExecuteComputation: batch %lld runs as two halves side by side (%.3f ms against %.3f ms whole)",
+                        (long long)B, sp.halves_ms, sp.whole_ms);
+            else
+              OHIP_INFO("odla_ExecuteComputation: batch %lld stays whole (%.3f ms against %.3f ms in two halves)",
+                        (long long)B, sp.whole_ms, sp.halves_ms);
+            if (sp.choice == 1) {   // the halves' arenas, streams and graphs are not needed again
+              for (_odla_context*& h : sp.half) { if (h) destroy_context_tree(h); h = nullptr; }
+              sp.comp.reset();
+              sp.ok = false;
+            }
+          }
+          return st;
+        }
+      }
+    }
   }
   if (ctx->run_batch > 0 && ctx->run_batch != recorded_batch(*c)) {
     // another batch than the recorded one: the same bindings, on the copy planned for that batch

@@ -174,8 +174,8 @@ std::unique_ptr<_odla_computation> clone_for_batch(const _odla_computation& c, i
         break;
       case OP_NMS:
         if (!rs.carry(n.in[0]) || !rs.carry(n.in[1])) rs.reject(n, "has boxes or scores that do not depend on the batch");
-        // (its result lists image numbers, and the images' detections follow each other without gaps)
-        if (rows_apart) rs.reject(n, "numbers the images of the batch in its result");
+        // (every image owns max_num_outputs rows of the result, and the image numbers written there
+        //  start at the executing context's image_base: a half-batch copy gives the whole batch's rows)
         break;
       case OP_UNARY: case OP_POOL: case OP_CAST: case OP_RESHAPE: case OP_RESIZE: case OP_LRN:
         break;

@@ -147,6 +147,9 @@ struct ExecEnv {
   // device buffer when the steps read / write it in place, nullptr when the data goes
   // through the staging tensor in the arena.
   const char* const* ext = nullptr;
+  // Number, in the caller's batch, of the first image this execution works on (not 0 for the
+  // second of two half-batch copies): operators that write image numbers add it.
+  int image_base = 0;
 };
 
 struct Step {
@@ -289,8 +292,15 @@ struct _odla_context {
     bool tried = false, ok = false;
     std::shared_ptr<_odla_computation> comp;
     _odla_context* half[2] = {nullptr, nullptr};
+    // Without ODLA_HIP_BATCH_SPLIT the context measures: executions 1-3 run whole, 4-6 in
+    // halves (the first of each three captures its graph, the faster of the other two counts),
+    // then the faster way is kept.
+    int trial = 0;            // executions counted so far (stops at 6)
+    double whole_ms = 0, halves_ms = 0;
+    int choice = 0;           // 0 undecided, 1 whole, 2 halves
   } split;
   bool is_half = false;   // this context is one of those halves: it runs as it is
+  int image_base = 0;        // see ExecEnv::image_base
   bool last_split = false;   // the last execution ran as halves: results live in their arenas / the caller's buffers
 };
 

@@ -472,7 +472,7 @@ size_t nms_workspace_bytes(int N, int B);
 // boxes / scores are read in their storage type (DT_F32, DT_F16 or DT_BF16).
 hipError_t launch_nms(const void* boxes, DType boxes_dt, const void* scores, DType scores_dt, int N, int C, int B,
                       int max_out, float iou_thr, float score_thr, int32_t* out,
-                      void* workspace, hipStream_t stream);
+                      void* workspace, hipStream_t stream, int image_base = 0);
 
 // YOLOv3 post-processing of one image: decode of three heads [3*(5+classes)][dim][dim]
 // (fp32, channels first) into `boxes` [total][4] (y min, x min, y max, x max in

@@ -234,7 +234,7 @@ __global__ void __launch_bounds__(kNmsThreads)
 nms_kernel(const TB* __restrict__ boxes, const float* __restrict__ best_ws, int B,
            int max_out, float iou_thr, float score_thr, int32_t* __restrict__ out,
            unsigned long long* keys_ws, const int32_t* cls_ws, unsigned char* sup_ws, int64_t bpad,
-           int lds_slots) {
+           int lds_slots, int image_base) {
   const int n = blockIdx.x;
   const int tid = threadIdx.x;
   const TB* bx = boxes + (int64_t)n * B * 4;
@@ -276,7 +276,7 @@ nms_kernel(const TB* __restrict__ boxes, const float* __restrict__ best_ws, int 
   if (M == 0 || max_out == 0) return;
   const int P = (int)next_pow2(M);
   if (P <= lds_slots && P <= kNmsThreads * kNmsPerThread) {
-    nms_on_cu<TB>(bx, cls, o, lds_keys, n, M, P, max_out, iou_thr);
+    nms_on_cu<TB>(bx, cls, o, lds_keys, image_base + n, M, P, max_out, iou_thr);
     return;
   }
 
@@ -311,7 +311,7 @@ nms_kernel(const TB* __restrict__ boxes, const float* __restrict__ best_ws, int 
     if (kept >= max_out) break;
     const int bi = (int)(keys[i] & 0xffffffffu);
     if (tid == 0) {
-      o[kept * 3 + 0] = n;
+      o[kept * 3 + 0] = image_base + n;   // (the image's number in the caller's batch)
       o[kept * 3 + 1] = cls[bi];
       o[kept * 3 + 2] = bi;
     }
@@ -342,7 +342,7 @@ size_t nms_workspace_bytes(int N, int B) {
 template <typename TB>
 static hipError_t launch_nms_kernel(const void* boxes, const float* best, int N, int B, int max_out, float iou_thr,
                                     float score_thr, int32_t* out, unsigned long long* keys, const int32_t* cls,
-                                    unsigned char* sup, int64_t bpad, hipStream_t stream) {
+                                    unsigned char* sup, int64_t bpad, int image_base, hipStream_t stream) {
   // candidate list on the compute unit - first the keys (two exchange buffers of 8 B per
   // slot), then boxes and flags in their place (16 + 1 B per slot): up to 8192 candidates
   const int lds_slots = (int)(bpad < 8192 ? bpad : 8192);
@@ -355,13 +355,13 @@ static hipError_t launch_nms_kernel(const void* boxes, const float* best, int N,
     lds_limit_raised = true;
   }
   hipLaunchKernelGGL(nms_kernel<TB>, dim3(N), dim3(kNmsThreads), lds_bytes, stream, (const TB*)boxes, best, B, max_out,
-                     iou_thr, score_thr, out, keys, cls, sup, bpad, lds_slots);
+                     iou_thr, score_thr, out, keys, cls, sup, bpad, lds_slots, image_base);
   return hipGetLastError();
 }
 
 hipError_t launch_nms(const void* boxes, DType boxes_dt, const void* scores, DType scores_dt, int N, int C, int B,
                       int max_out, float iou_thr, float score_thr, int32_t* out, void* workspace,
-                      hipStream_t stream) {
+                      hipStream_t stream, int image_base) {
   if (!boxes || !scores || !out || !workspace || N <= 0 || C <= 0 || B <= 0 || max_out < 0)
     return hipErrorInvalidValue;
   if ((reinterpret_cast<uintptr_t>(workspace) & 7u) != 0) return hipErrorInvalidValue;
@@ -380,9 +380,9 @@ hipError_t launch_nms(const void* boxes, DType boxes_dt, const void* scores, DTy
     default: return hipErrorInvalidValue;
   }
   switch (boxes_dt) {
-    case DT_F32: return launch_nms_kernel<float>(boxes, best, N, B, max_out, iou_thr, score_thr, out, keys, cls, sup, bpad, stream);
-    case DT_F16: return launch_nms_kernel<f16_t>(boxes, best, N, B, max_out, iou_thr, score_thr, out, keys, cls, sup, bpad, stream);
-    case DT_BF16: return launch_nms_kernel<bf16_t>(boxes, best, N, B, max_out, iou_thr, score_thr, out, keys, cls, sup, bpad, stream);
+    case DT_F32: return launch_nms_kernel<float>(boxes, best, N, B, max_out, iou_thr, score_thr, out, keys, cls, sup, bpad, image_base, stream);
+    case DT_F16: return launch_nms_kernel<f16_t>(boxes, best, N, B, max_out, iou_thr, score_thr, out, keys, cls, sup, bpad, image_base, stream);
+    case DT_BF16: return launch_nms_kernel<bf16_t>(boxes, best, N, B, max_out, iou_thr, score_thr, out, keys, cls, sup, bpad, image_base, stream);
     default: return hipErrorInvalidValue;
   }
 }

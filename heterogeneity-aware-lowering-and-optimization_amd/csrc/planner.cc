@@ -3415,7 +3415,7 @@ void Planner::lower_nms(int ni) {
   const int ty = new_tensor(DT_I32, L_ROWMAJOR, o32, 0, SP_ARENA);
   const Ref rb = ref(tb), rs = ref(ts), rw = ref(tw), ry = ref(ty);
   emit("nms:" + n.out->name, {tb, ts, tw}, {ty, tw}, [=](const ExecEnv& e, hipStream_t st) {
-    return launch_nms(rb(e), bdt, rs(e), sdt, N, C, B, max_out, iou, thr, (int32_t*)ry(e), rw(e), st);
+    return launch_nms(rb(e), bdt, rs(e), sdt, N, C, B, max_out, iou, thr, (int32_t*)ry(e), rw(e), st, e.image_base);
   });
   if (dtype_from_odla(n.out->etype) == DT_I64) {
     const int t64 = new_tensor(DT_I64, L_ROWMAJOR, o32, 0, SP_ARENA);

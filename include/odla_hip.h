@@ -287,11 +287,12 @@ odla_status odla_BindToOutputById(const odla_value_id value_id,
 
 /* Run the graph once: stage bound arguments, replay the planned launch
  * sequence, write every bound output, and return after the device is idle.
- * From batch 64 on (every argument's leading extent; ODLA_HIP_BATCH_SPLIT in
- * the environment: 0 = never, n = from batch n on) a graph that keeps the
- * images' rows apart in every result runs as two copies at half the batch,
- * side by side on two streams, each on its half of the bound buffers: same
- * buffers, same results, a second pair of arenas in the context.
+ * Where that is faster (a context measures during its first six executions;
+ * ODLA_HIP_BATCH_SPLIT in the environment: 0 = never, n = always from batch n
+ * on) a graph that keeps the images' rows apart in every result runs as two
+ * copies at half the batch (every argument's leading extent), side by side on
+ * two streams, each on its half of the bound buffers: same buffers, same
+ * results, a second pair of arenas in the context.
  * [ref: odla_compute.h:158-170; dnnl odla_dnnl.cc:133-159;
  *  tensorrt odla_tensorrt.cc:866-968] */
 odla_status odla_ExecuteComputation(const odla_computation computation,
