@@ -237,9 +237,9 @@ def run_workload(pkg, L, name, args, with_cpu):
     L.odla_SetLogger(ctypes.cast(cb, ctypes.c_void_p))
     L.odla_SetLogLevel(4)
     try:
-        # set-up, like the graph capture: the context's first six executions measure whether the
-        # batch runs whole or as two half-batch copies (three each way) and say which it keeps
-        for _ in range(6):
+        # set-up, like the graph capture: the context's first fourteen executions measure whether
+        # the batch runs whole (six) or as two half-batch copies (eight) and say which it keeps
+        for _ in range(14):
             sess.execute()
         for _ in range(args.warmup):
             sess.execute()
@@ -247,6 +247,9 @@ def run_workload(pkg, L, name, args, with_cpu):
         L.odla_SetLogLevel(2)
         L.odla_SetLogger(None)
     halves = any("two halves side by side" in m for m in said)
+    for m in said:
+        if "two halves" in m or "stays whole" in m:
+            print("[%s] %s" % (name, m), file=sys.stderr)
     # odla_ExecuteComputation returns after the device is idle, so the wall
     # clock around K executions is the device-synchronised time of K steps.
     t0 = time.perf_counter()
@@ -298,8 +301,8 @@ def end_to_end(hb, wl, steps):
         outs = sess.bind_host_io(wl.feeds, pinned=pinned)
         out["host_bytes_per_step"] = int(sum(v.nbytes for v in wl.feeds.values()) + sum(o.nbytes for o in outs.values()))
         # untimed: the captures, and the executions in which the context measures whether to
-        # run the batch whole or as two half-batch copies (three each way)
-        for _ in range(7):
+        # run the batch whole (six) or as two half-batch copies (eight)
+        for _ in range(15):
             sess.execute()
         t0 = time.perf_counter()
         for _ in range(steps):

@@ -335,6 +335,7 @@ void destroy_context_tree(_odla_context* ctx) {
   ctx->split.comp.reset();
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   drop_graph(ctx);
+  if (ctx->inputs_staged) (void)hipEventDestroy(ctx->inputs_staged);
   if (ctx->arena) (void)hipFree(ctx->arena);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
@@ -744,6 +745,10 @@ odla_status execute_split(_odla_context* ctx, odla_compute_mode mode, odla_devic
       sub->image_base = ctx->image_base + k * (int)(B / 2);
       sp.half[k] = sub;
     }
+    if (hipEventCreateWithFlags(&sp.half[0]->inputs_staged, hipEventDisableTiming) == hipSuccess)
+      sp.half[1]->wait_inputs = sp.half[0]->inputs_staged;
+    else
+      sp.half[0]->inputs_staged = nullptr;
     sp.comp = std::move(v);
     sp.ok = true;
     OHIP_DEBUG("odla_ExecuteComputation: two half-batch copies of batch %lld planned", (long long)B);
@@ -832,13 +837,16 @@ odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, o
         const odla_status st = execute_split(ctx, mode, device, &handled);
         if (handled) return st;
       } else if (wait) {
-        // measuring: executions 1-3 whole, 4-6 in halves; the first of each three captures its
-        // graph, the faster of the other two counts
+        // measuring: six executions whole, then eight in halves, the fastest of the last three
+        // of each counts (a fresh context needs some five replays to reach its steady time -
+        // clocks, caches, the graphs' first launches - and the halves, coming second with two
+        // fresh graphs, a few more)
+        constexpr int kWhole = 6, kHalves = 8, kCount = 3;
         const int t = sp.trial;
         const auto t0 = std::chrono::steady_clock::now();
         odla_status st = ODLA_SUCCESS;
         bool handled = true;
-        if (t < 3) {
+        if (t < kWhole) {
           st = execute_impl(ctx, mode, device, wait, /*whole=*/true);
         } else {
           st = execute_split(ctx, mode, device, &handled);
@@ -848,12 +856,10 @@ odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, o
         } else {
           const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
           if (st != ODLA_SUCCESS) return st;
-          if (t == 1) sp.whole_ms = ms;
-          if (t == 2 && ms < sp.whole_ms) sp.whole_ms = ms;
-          if (t == 4) sp.halves_ms = ms;
-          if (t == 5 && ms < sp.halves_ms) sp.halves_ms = ms;
+          if (t >= kWhole - kCount && t < kWhole && (t == kWhole - kCount || ms < sp.whole_ms)) sp.whole_ms = ms;
+          if (t >= kWhole + kHalves - kCount && (t == kWhole + kHalves - kCount || ms < sp.halves_ms)) sp.halves_ms = ms;
           sp.trial = t + 1;
-          if (sp.trial == 6) {
+          if (sp.trial == kWhole + kHalves) {
             sp.choice = sp.halves_ms < 0.98 * sp.whole_ms ? 2 : 1;
             if (sp.choice == 2)
               OHIP_INFO("odla_ExecuteComputation: batch %lld runs as two halves side by side (%.3f ms against %.3f ms whole)",
@@ -896,8 +902,10 @@ odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, o
   //    that the first steps can read where they are stay there)
   std::vector<const char*> ext;
   {
+    if (ctx->wait_inputs != nullptr) (void)hipStreamWaitEvent(ctx->stream, ctx->wait_inputs, 0);
     odla_status st = stage_inputs(ctx, plan, ctx->arena, &ext);
     if (st != ODLA_SUCCESS) return st;
+    if (ctx->inputs_staged != nullptr) (void)hipEventRecord(ctx->inputs_staged, ctx->stream);
     place_outputs(ctx, plan, &ext);
   }
 

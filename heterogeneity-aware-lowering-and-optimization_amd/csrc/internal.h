@@ -292,15 +292,20 @@ struct _odla_context {
     bool tried = false, ok = false;
     std::shared_ptr<_odla_computation> comp;
     _odla_context* half[2] = {nullptr, nullptr};
-    // Without ODLA_HIP_BATCH_SPLIT the context measures: executions 1-3 run whole, 4-6 in
-    // halves (the first of each three captures its graph, the faster of the other two counts),
-    // then the faster way is kept.
-    int trial = 0;            // executions counted so far (stops at 6)
+    // Without ODLA_HIP_BATCH_SPLIT the context measures: six executions whole, eight in halves,
+    // the fastest of the last three of each counts; then the faster way is kept.
+    int trial = 0;            // executions counted so far (stops at 14)
     double whole_ms = 0, halves_ms = 0;
     int choice = 0;           // 0 undecided, 1 whole, 2 halves
   } split;
   bool is_half = false;   // this context is one of those halves: it runs as it is
   int image_base = 0;        // see ExecEnv::image_base
+  // Halves only: the second half stages its arguments after the first has staged its own
+  // (copies from host memory then follow each other at full PCIe rate, and the first half
+  // computes while the second half's arguments travel).  The first half records
+  // `inputs_staged` behind its copies (it owns the event), the second waits for `wait_inputs`.
+  hipEvent_t inputs_staged = nullptr;
+  hipEvent_t wait_inputs = nullptr;
   bool last_split = false;   // the last execution ran as halves: results live in their arenas / the caller's buffers
 };
 

@@ -46,7 +46,7 @@ def test_cnn_in_two_halves_equals_the_whole_batch(mode, use_graph, monkeypatch):
 
 
 def test_a_context_measures_and_keeps_the_faster_way(monkeypatch):
-    """Without ODLA_HIP_BATCH_SPLIT a context runs three times whole, three times in halves, then says
+    """Without ODLA_HIP_BATCH_SPLIT a context runs six times whole, eight times in halves, then says
     which way it keeps; every one of these executions gives the whole batch's results."""
     odla = entry.load().odla
     B = 8
@@ -71,7 +71,7 @@ def test_a_context_measures_and_keeps_the_faster_way(monkeypatch):
         try:
             def go():
                 outs = []
-                for _ in range(9):
+                for _ in range(16):
                     outs.append(s.run({"x": x}))
                 return outs
             outs, seen = run_logged(go)
