@@ -287,7 +287,7 @@ odla_status odla_BindToOutputById(const odla_value_id value_id,
 
 /* Run the graph once: stage bound arguments, replay the planned launch
  * sequence, write every bound output, and return after the device is idle.
- * Where that is faster (a context measures during its first six executions;
+ * Where that is faster (a context measures during its first fourteen executions;
  * ODLA_HIP_BATCH_SPLIT in the environment: 0 = never, n = always from batch n
  * on) a graph that keeps the images' rows apart in every result runs as two
  * copies at half the batch (every argument's leading extent), side by side on
