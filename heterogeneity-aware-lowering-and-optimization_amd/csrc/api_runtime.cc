@@ -742,6 +742,7 @@ odla_status execute_split(_odla_context* ctx, odla_compute_mode mode, odla_devic
         return ODLA_SUCCESS;
       }
       sub->is_half = true;
+      sub->defer_fetch = true;
       sub->image_base = ctx->image_base + k * (int)(B / 2);
       sp.half[k] = sub;
     }
@@ -786,6 +787,9 @@ odla_status execute_split(_odla_context* ctx, odla_compute_mode mode, odla_devic
   }
   odla_status st = ODLA_SUCCESS;
   for (int k = 0; k < 2 && st == ODLA_SUCCESS; ++k) st = execute_impl(sp.half[k], mode, device, /*wait=*/false);
+  // both halves are queued: now their results' copies
+  for (int k = 0; k < 2 && st == ODLA_SUCCESS; ++k)
+    st = fetch_outputs(sp.half[k], hp, sp.half[k]->arena, &sp.half[k]->last_ext, /*wait=*/false);
   for (int k = 0; k < 2; ++k) {
     const hipError_t e = hipStreamSynchronize(sp.half[k]->stream);
     if (e != hipSuccess) {
@@ -959,6 +963,12 @@ odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, o
   }
 
   // 3. results
+  if (ctx->defer_fetch) {   // (a half: its parent fetches, see execute_split)
+    ctx->last_ext = ext;
+    ctx->executed = true;
+    ctx->last_split = false;
+    return ODLA_SUCCESS;
+  }
   odla_status st = fetch_outputs(ctx, plan, ctx->arena, &ext, wait);
   if (st != ODLA_SUCCESS) return st;
   ctx->last_ext = ext;

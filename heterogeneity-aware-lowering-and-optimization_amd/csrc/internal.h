@@ -306,6 +306,11 @@ struct _odla_context {
   // `inputs_staged` behind its copies (it owns the event), the second waits for `wait_inputs`.
   hipEvent_t inputs_staged = nullptr;
   hipEvent_t wait_inputs = nullptr;
+  // Halves only: the execution returns once the launches are queued; the parent queues the
+  // copies of the results of both halves afterwards (a copy into pageable host memory blocks
+  // the calling thread until the stream has reached it - the second half would not even be
+  // queued before the first has finished).
+  bool defer_fetch = false;
   bool last_split = false;   // the last execution ran as halves: results live in their arenas / the caller's buffers
 };
 
