@@ -107,6 +107,44 @@ __global__ void __launch_bounds__(kThreads) nchw_to_nhwc_smallc(LayoutParams p, 
   }
 }
 
+// The same for results of exactly 16 bytes per pixel (cs * sizeof(TD) == 16) and HW a multiple of
+// 1024: a workgroup takes 1024 consecutive pixels and a thread the four pixels tid, tid + 256,
+// ... of them, so that every store instruction of a wavefront writes 1 KiB of contiguous
+// memory (with four consecutive pixels per thread its lanes are 64 bytes apart and every
+// instruction touches 64 cache lines a quarter each).  The loads are one element per lane per
+// channel plane, 256 contiguous bytes per instruction.
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(kThreads) nchw_to_nhwc_rows16(LayoutParams p, float fill) {
+  const TS* src = reinterpret_cast<const TS*>(p.src);
+  TD* dst = reinterpret_cast<TD*>(p.dst);
+  constexpr int CS = 16 / (int)sizeof(TD);
+  const int64_t blocks_per_image = p.HW / 1024;
+  const int64_t total = (int64_t)p.N * blocks_per_image;
+  for (int64_t b = blockIdx.x; b < total; b += gridDim.x) {
+    const int64_t n = b / blocks_per_image;
+    const int64_t hw0 = (b - n * blocks_per_image) * 1024 + threadIdx.x;
+    float in[CS][4];
+#pragma unroll
+    for (int c = 0; c < CS; ++c) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) in[c][k] = fill;
+      if (c < p.C) {   // (uniform: p.C is a kernel argument)
+        const TS* s = src + (n * p.C + c) * p.HW + hw0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) in[c][k] = ld_as_float<TS>(s + k * 256, p.scale, p.zp);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      TD out[CS];
+#pragma unroll
+      for (int c = 0; c < CS; ++c) st_from_float<TD>(&out[c], in[c][k], p.scale, p.zp);
+      uintx4* o = reinterpret_cast<uintx4*>(dst + (n * p.HW + hw0 + k * 256) * p.cs);
+      __builtin_nontemporal_store(*reinterpret_cast<const uintx4*>(out), o);
+    }
+  }
+}
+
 // src [N][HW][cs] -> dst [N][C][HW]
 template <typename TS, typename TD>
 __global__ void __launch_bounds__(kThreads) nhwc_to_nchw_tiled(LayoutParams p) {
@@ -455,6 +493,15 @@ hipError_t launch_nchw_to_nhwc(const LayoutParams& p, hipStream_t stream) {
   if (!layout_ok(p)) return hipErrorInvalidValue;
   // padding lanes hold the real value 0 (its quantised level for 8-bit data)
   const float fill = 0.f;
+  if (p.cs * dtype_size(p.dst_dt) == 16 && p.HW % 1024 == 0 && (reinterpret_cast<uintptr_t>(p.dst) & 15u) == 0 &&
+      (p.dst_dt == DT_F16 || p.dst_dt == DT_BF16 || p.dst_dt == DT_I8)) {
+    const int64_t blocks = (int64_t)p.N * (p.HW / 1024);
+    const int grid = (int)(blocks < 65536 ? blocks : 65536);
+#define K0(TS, TD, ...) hipLaunchKernelGGL((nchw_to_nhwc_rows16<TS, TD>), dim3(grid), dim3(kThreads), 0, stream, p, fill)
+    LAYOUT_PAIR_DISPATCH(K0, 0);
+#undef K0
+    return hipGetLastError();
+  }
   if (p.cs <= 16) {
     const bool px4 = p.HW % 4 == 0 && (reinterpret_cast<uintptr_t>(p.src) & 15u) == 0 && p.src_dt == DT_F32;
     if (px4) {
