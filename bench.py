@@ -239,7 +239,8 @@ def run_workload(pkg, L, name, args, with_cpu):
     try:
         # set-up, like the graph capture: the context's first fourteen executions measure whether
         # the batch runs whole (six) or as two half-batch copies (eight) and say which it keeps
-        for _ in range(14):
+        # (nothing to measure when ODLA_HIP_BATCH_SPLIT decides)
+        for _ in range(0 if os.environ.get("ODLA_HIP_BATCH_SPLIT") else 14):
             sess.execute()
         for _ in range(args.warmup):
             sess.execute()
@@ -302,7 +303,7 @@ def end_to_end(hb, wl, steps):
         out["host_bytes_per_step"] = int(sum(v.nbytes for v in wl.feeds.values()) + sum(o.nbytes for o in outs.values()))
         # untimed: the captures, and the executions in which the context measures whether to
         # run the batch whole (six) or as two half-batch copies (eight)
-        for _ in range(15):
+        for _ in range(1 if os.environ.get("ODLA_HIP_BATCH_SPLIT") else 15):
             sess.execute()
         t0 = time.perf_counter()
         for _ in range(steps):
