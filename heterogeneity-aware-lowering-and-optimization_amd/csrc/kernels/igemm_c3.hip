@@ -7,10 +7,11 @@
 // runs all nine taps on it: nine K stages of MFMAs per patch, where the gathering
 // kernels fetch 128 pixel rows per stage (the same input bytes nine times).
 //
-// LDS layout of a patch chunk: one plane of 4 KiB per 16-byte piece of the chunk,
-// plane[c][patch pixel] - the 32 pixels a fragment read covers are consecutive or
-// nearly consecutive 16-byte slots of one plane (no bank conflicts, no swizzle),
-// and a tap is a constant offset from the lane's base address: (r * PW + s) * 16.
+// LDS layout of a patch chunk: one plane of 3 KiB per 16-byte piece of the chunk,
+// plane[c][patch pixel] - the 32 pixels a fragment read covers are 16-byte slots of one
+// plane, a tap is a constant offset from the lane's base address: (r * PW + s) * 16, and
+// which MFMA column takes which pixel of a block is chosen such that the sixteen lanes the
+// LDS serves in one pass read sixteen different banks (c3_lane_table).
 // Patch pixels outside the image hold the byte that represents 0.
 //
 // Weights come fragment-ordered from the packed copy (p.w_frag), one K stage
@@ -42,6 +43,10 @@ struct C3Geom {
   int nkk = 0, ws = 0, nj = 0;   // template choice
   int main_bytes = 0;            // LDS ahead of the pixel table
   float eff = 0.f;               // share of the MFMA columns that are output pixels
+  // Which position of a pixel block (row-major, br x bc) MFMA column l takes: byte l of
+  // lane_pos[l / 8]; bit 7 marks a column past the block, which reads the pixel of another
+  // column of its LDS pass and stores nothing.
+  unsigned long long lane_pos[4] = {0, 0, 0, 0};
 };
 
 constexpr int kC3Plane = 3072;   // bytes of a patch plane: 192 patch pixels x 16 bytes
@@ -90,11 +95,15 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
   const int y0 = ty * 4 * g.br, x0 = tx * g.bc;
 
   // which output pixel each position of the tile is
+  auto lane_pos = [&](const int l) __attribute__((always_inline)) {
+    const unsigned long long w = l < 16 ? (l < 8 ? g.lane_pos[0] : g.lane_pos[1]) : (l < 24 ? g.lane_pos[2] : g.lane_pos[3]);
+    return (int)((w >> ((l & 7) * 8)) & 0xff);
+  };
   if (tid < 128) {
-    const int blk = tid >> 5, l = tid & 31;
-    const int br = l / g.bc, bc = l - br * g.bc;
+    const int blk = tid >> 5, q = lane_pos(tid & 31);
+    const int br = (q & 0x7f) / g.bc, bc = (q & 0x7f) - br * g.bc;
     const int yy = y0 + blk * g.br + br, xx = x0 + bc;
-    mtab[tid] = (l < g.br * g.bc && yy < p.H && xx < p.W) ? (n_img * p.H + yy) * p.W + xx : -1;
+    mtab[tid] = (q < 0x80 && yy < p.H && xx < p.W) ? (n_img * p.H + yy) * p.W + xx : -1;
   }
 
   // this thread's patch pixels: tid, tid + NT, ..
@@ -161,12 +170,12 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
     for (int j = 0; j < NJ; ++j) dst[j] = *reinterpret_cast<const uintx4*>(wfp[j] + off);
   };
 
-  // LDS address of the window's top left pixel, per block: lanes past the block read its first pixel
+  // LDS address of the window's top left pixel, per block
   unsigned base[NB];
   {
-    const bool live = l32 < g.br * g.bc;
-    const int br = live ? l32 / g.bc : 0;
-    const int bc = live ? l32 - br * g.bc : 0;
+    const int q = lane_pos(l32) & 0x7f;
+    const int br = q / g.bc;
+    const int bc = q - br * g.bc;
 #pragma unroll
     for (int i = 0; i < NB; ++i) base[i] = (unsigned)(((i * g.br + br) * g.pw + bc) * 16 + lg * PLANE);
   }
@@ -174,6 +183,8 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
   // Weight fragments: a ring of RW K steps, requested RW - 1 steps ahead of their use.  The
   // steps of a chunk are a multiple of RW, so step st of every chunk sits in slot st % RW.
   constexpr int STEPS = 9 * NKK;
+  // (deeper rings were measured slower: 9 and 12 steps against 6, ResNet-50 at batch 256, the
+  //  3x3 layers at 14 x 14: int8 250 -> 259 -> 264 us, fp16 435 -> 465 -> 504 us for the six)
   constexpr int RW = NJ == 1 ? 6 : (STEPS % 4 == 0 ? 4 : 3), AHEAD = RW - 1;
   static_assert(STEPS % RW == 0, "the ring position of a step must not depend on the chunk");
   uintx4 w[RW][NJ];
@@ -270,18 +281,42 @@ __global__ __launch_bounds__(WS * 64, NJ == 1 ? 3 : 2) void igemm_c3_kernel(cons
   }
 }
 
-// LDS passes of a pixel-fragment read: sixteen lanes are served together, and two of them
-// conflict when their 16-byte slots are equal modulo 16 (256 bytes = all banks).  Lane l of a
-// block reads slot (l / bc) * (bc + 2) + l % bc of its plane (plus a common offset).
-int c3_lds_passes(const int br, const int bc) {
-  int worst = 1;
-  for (int g0 = 0; g0 < 32; g0 += 16) {
-    int count[16] = {0};
-    for (int l = g0; l < g0 + 16 && l < br * bc; ++l) {
-      const int c = ++count[((l / bc) * (bc + 2) + l % bc) & 15];
-      worst = c > worst ? c : worst;
-    }
+// LDS passes of a pixel-fragment read.  A 16-byte read of a wavefront is served in four passes
+// of sixteen lanes - within each half of the wavefront lanes {0-3, 12-15, 20-27} and lanes
+// {4-11, 16-19, 28-31} (measured: two lanes that trade their slots cost a pass exactly when
+// they are of different sets) - and two lanes of a pass conflict when their 16-byte slots are
+// equal modulo 16 (256 bytes = all banks).  Position q of a block sits in slot
+// (q / bc) * (bc + 2) + q % bc of its plane (plus a common offset); which MFMA column takes
+// which position is free, so the positions are dealt to the two sets such that a set holds
+// every slot residue once where the block's shape allows that (no residue more than twice).
+// Returns the passes of the worse set and writes the table (C3Geom::lane_pos).
+int c3_lane_table(const int br, const int bc, unsigned long long (*table)[4]) {
+  static const int kSet[2][16] = {{0, 1, 2, 3, 12, 13, 14, 15, 20, 21, 22, 23, 24, 25, 26, 27},
+                                  {4, 5, 6, 7, 8, 9, 10, 11, 16, 17, 18, 19, 28, 29, 30, 31}};
+  int members[2][16], count[2] = {0, 0}, used[2][16] = {{0}, {0}};
+  for (int q = 0; q < br * bc; ++q) {
+    const int r = ((q / bc) * (bc + 2) + q % bc) & 15;
+    int s;
+    if (count[0] >= 16) s = 1;
+    else if (count[1] >= 16) s = 0;
+    else if (used[0][r] != used[1][r]) s = used[0][r] < used[1][r] ? 0 : 1;
+    else s = count[0] <= count[1] ? 0 : 1;
+    members[s][count[s]++] = q;
+    ++used[s][r];
   }
+  int worst = 1;
+  unsigned char pos[32];
+  for (int s = 0; s < 2; ++s) {
+    for (int r = 0; r < 16; ++r) worst = used[s][r] > worst ? used[s][r] : worst;
+    // (a column past the block reads what another column of its pass reads: one address, no conflict)
+    const int spare = count[s] > 0 ? members[s][0] : 0;
+    for (int k = 0; k < 16; ++k) pos[kSet[s][k]] = (unsigned char)(k < count[s] ? members[s][k] : (spare | 0x80));
+  }
+  if (table)
+    for (int w = 0; w < 4; ++w) {
+      (*table)[w] = 0;
+      for (int b = 0; b < 8; ++b) (*table)[w] |= (unsigned long long)pos[w * 8 + b] << (b * 8);
+    }
   return worst;
 }
 
@@ -326,10 +361,8 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
   int force_bc = 0;
   if (const char* e = getenv("ODLA_HIP_C3_BC")) force_bc = atoi(e);   // tuning aid: block columns
   for (int bc = 32; bc >= 4; --bc) {
-    // Blocks of 16 or 32 columns may hang over the right edge (a 14-column image as one block
-    // of 16: each half of a wavefront then reads 16 consecutive slots of one patch row - no
-    // second LDS pass - where 2 x 14 blocks wrap two lanes into the next row); other widths
-    // must divide the image's.
+    // Blocks of 16 or 32 columns may hang over the right edge (a 30-column image as blocks of
+    // 32 x 1); other widths must divide the image's.
     const bool over = (bc == 16 || bc == 32) && p.W % bc != 0;
     if ((p.W % bc != 0 && !over) || (force_bc > 0 && (p.W % force_bc == 0 || force_bc == 16 || force_bc == 32) && bc != force_bc)) continue;
     int br = 32 / bc;
@@ -340,7 +373,7 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
     const int npp = (th + 2) * (bc + 2);
     if (npp > kC3Plane / 16) continue;
     const float halo = (float)npp / (float)(th * bc);
-    const float score = c3_lds_passes(br, bc) == 1 ? eff : 0.85f * eff;
+    const float score = c3_lane_table(br, bc, nullptr) == 1 ? eff : 0.85f * eff;
     if (score > best_score + 1e-6f || (score > best_score - 1e-6f && halo < best_halo)) {
       g.eff = eff; best_halo = halo; best_score = score;
       g.br = br; g.bc = bc; g.pw = bc + 2; g.npp = npp;
@@ -350,6 +383,7 @@ bool c3_geometry(const IgemmParams& p, C3Geom* out) {
   float min_eff = 0.7f;
   if (const char* e = getenv("ODLA_HIP_C3_MIN_FILL")) min_eff = (float)atof(e);  // tuning aid
   if (g.bc == 0 || g.eff < min_eff) return false;
+  c3_lane_table(g.br, g.bc, &g.lane_pos);
   const int64_t wgs = (int64_t)p.N * g.tiles_y * g.tiles_x * g.tiles_n;
   if (wgs <= 0 || wgs > 0x7fffffff) return false;
   if ((int64_t)p.N * p.H * p.W * p.xcs * es >= (1ll << 40)) return false;

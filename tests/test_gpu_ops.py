@@ -550,6 +550,40 @@ def test_unary_parity(mode):
             assert np.max(np.abs(got[k] - want[k])) <= 2e-2 * max(1.0, float(np.max(np.abs(want[k])))), k
 
 
+def test_gelu_against_the_exact_function():
+    """odla_Gelu (erf form) against x * Phi(x) in float64, standalone and in the epilogue of a Gemm:
+    absolute error below 1e-6 everywhere and relative error below 1e-5 wherever the result is
+    above 1e-6 in magnitude - the negative tail included, where the float formula
+    0.5 x (1 + erff(x / sqrt 2)) cancels; 0, -0, large arguments and a NaN."""
+    from scipy.special import erfc
+    announce("gelu exact")
+    r = rng(231)
+    x = np.concatenate([np.linspace(-8.0, 8.0, 64 * 511), r.standard_normal(64 * 512) * 2.0,
+                        [0.0, -0.0, 1e-20, -1e-20, 30.0, -30.0, -5.65, -5.66, -5.67, 5.66, 1e10, -1e10]])
+    x = np.concatenate([x, np.zeros(64 * 1024 - x.size)]).astype(np.float32).reshape(1024, 64)
+    eye = np.eye(64, dtype=np.float32)
+
+    def build(b):
+        a = b.arg("x", x.shape)
+        b.output(b.gelu(a, False, name="alone"), "alone")
+        b.output(b.gelu(b.gemm(a, b.const("eye", eye), name="mm"), False, name="fused"), "fused")
+
+    got = run_hip(build, {"x": x})
+    xd = x.astype(np.float64)
+    want = xd * 0.5 * erfc(-xd / np.sqrt(2.0))
+    for k in ("alone", "fused"):
+        g = got[k].astype(np.float64)
+        err = np.abs(g - want)
+        assert err.max() <= 1e-6, (k, err.max(), x.flat[err.argmax()])
+        big = np.abs(want) > 1e-6
+        rel = err[big] / np.abs(want[big])
+        assert rel.max() <= 1e-5, (k, rel.max())
+
+    nan = np.full((64, 64), np.nan, np.float32)
+    got = run_hip(lambda b: b.output(b.gelu(b.arg("x", nan.shape), False, name="y"), "y"), {"x": nan})
+    assert np.all(np.isnan(got["y"]))
+
+
 def test_round_half_even():
     announce("round")
     x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, 2.4999, 3.5], np.float32)
