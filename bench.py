@@ -248,6 +248,7 @@ def run_workload(pkg, L, name, args, with_cpu):
         L.odla_SetLogLevel(2)
         L.odla_SetLogger(None)
     halves = any("two halves side by side" in m for m in said)
+    uncaptured = any("run uncaptured" in m for m in said)
     for m in said:
         if "two halves" in m or "stays whole" in m:
             print("[%s] %s" % (name, m), file=sys.stderr)
@@ -280,7 +281,8 @@ def run_workload(pkg, L, name, args, with_cpu):
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": DTYPE[mode], "data": "synthetic",
         "config": {"workload": wl.desc, "batch": wl.batch,
-                   "executor": "hipGraph replay through odla_ExecuteComputation"
+                   "executor": ("direct launches through odla_ExecuteComputation (fewer than six per execution: no hipGraph)"
+                                if uncaptured else "hipGraph replay through odla_ExecuteComputation")
                                + (": two half-batch copies of the plan side by side on two streams" if halves else "")},
         "roofline": roof, "cpu_baseline": cpu, "end_to_end": e2e,
     }

@@ -660,6 +660,18 @@ odla_status odla_BindToOutputById(const odla_value_id id, odla_void* data_ptr, o
 
 namespace {
 
+// Launch sequences shorter than this run uncaptured: replaying a hipGraph costs a fixed amount
+// per execution that a few direct launches stay below.  Measured on chains of 1 .. 24 small
+// launches (device-resident buffers, one execution after the other): replay 34.5 us for one
+// launch, 35.8 for five, 37.2 for six, 65.9 for 24; direct launches 17.8, 27.0, 45.0 (the
+// runtime hands over more than five queued launches differently), 92.4.
+// ODLA_HIP_GRAPH_MIN_STEPS overrides (read per execution: tests of the capture path set it to 1).
+size_t min_graph_steps() {
+  const char* e = getenv("ODLA_HIP_GRAPH_MIN_STEPS");
+  const long n = e ? atol(e) : 0;
+  return (size_t)(n > 0 ? n : 6);
+}
+
 odla_status execute_impl(odla_context ctx, odla_compute_mode mode, odla_device device, bool wait, bool whole = false);
 
 // Leading extent shared by every argument of `c` (the batch, as in the reference's runtimes), 0 if
@@ -914,7 +926,7 @@ odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, o
   }
 
   // 2. launch sequence: captured once into a hipGraph, replayed afterwards
-  if (ctx->use_graph && !plan.steps.empty()) {
+  if (ctx->use_graph && plan.steps.size() >= min_graph_steps()) {
     select_graph(ctx, ext);
     // A caller that brings new buffers every time would capture every time: after a few
     // captures in a row this context goes back to staging copies and one graph.
@@ -958,6 +970,10 @@ odla_status execute_impl(const odla_context ctx, const odla_compute_mode mode, o
       return ODLA_FAILURE;
     }
   } else {
+    if (ctx->use_graph && !plan.steps.empty() && !ctx->said_uncaptured) {
+      ctx->said_uncaptured = true;
+      OHIP_INFO("odla_ExecuteComputation: %zu launches per execution run uncaptured (a graph replay costs more than that few)", plan.steps.size());
+    }
     odla_status st = run_steps(ctx, plan, ctx->arena, &ext);
     if (st != ODLA_SUCCESS) return st;
   }

@@ -312,6 +312,7 @@ struct _odla_context {
   // queued before the first has finished).
   bool defer_fetch = false;
   bool last_split = false;   // the last execution ran as halves: results live in their arenas / the caller's buffers
+  bool said_uncaptured = false;   // the note that a short launch sequence runs without a graph has been logged
 };
 
 struct _odla_device {

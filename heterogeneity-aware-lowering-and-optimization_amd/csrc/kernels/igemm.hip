@@ -1164,6 +1164,7 @@ const char* igemm_variant_name(const IgemmParams& p) {
     case 3: return "128x256";
     default: break;
   }
+  if (gemm_rowdot_shape(p)) return "rowdot";
   if (p.w_frag != nullptr && igemm_c3_geometry(p)) return "patch3x3";
   if (p.w_frag != nullptr && igemm_stream_q8_geometry(p)) return "stream";
   if (p.w_frag != nullptr && lean_steps(p) > 0) return "128x128s";
@@ -1248,6 +1249,7 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
     if (ok16) epi_vec |= 2;
   }
 
+  if (gemm_rowdot_shape(p)) return launch_gemm_rowdot(p, stream);
   if (const int big = igemm_big_variant(p)) return launch_igemm_big(p, epi_vec, big, stream);
   if (p.w_frag != nullptr && igemm_c3_geometry(p)) return launch_igemm_c3(p, epi_vec, stream);
 

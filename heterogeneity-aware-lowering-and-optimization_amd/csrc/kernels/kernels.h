@@ -145,6 +145,11 @@ hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream);
 // Name of the kernel variant launch_igemm would pick (for reports).
 const char* igemm_variant_name(const IgemmParams& p);
 
+// Products with at most 16 output columns, a long reduction and few rows (gemm_rowdot.hip): one
+// wavefront per output row.  Whether the shape qualifies, and the launch (launch_igemm uses both).
+bool gemm_rowdot_shape(const IgemmParams& p);
+hipError_t launch_gemm_rowdot(const IgemmParams& p, hipStream_t stream);
+
 // Large-tile kernels (igemm_big.hip) for matrix-core-bound layers: the variant
 // launch_igemm uses for this shape (0: none), and the launch itself.
 int igemm_big_variant(const IgemmParams& p);

@@ -287,6 +287,12 @@ odla_status odla_BindToOutputById(const odla_value_id value_id,
 
 /* Run the graph once: stage bound arguments, replay the planned launch
  * sequence, write every bound output, and return after the device is idle.
+ * The sequence is replayed from a hipGraph captured at the first execution,
+ * except that sequences of fewer than six launches are launched directly (a
+ * replay has a fixed cost that so few launches stay below;
+ * ODLA_HIP_GRAPH_MIN_STEPS in the environment sets another bound, 1 = always
+ * a graph) and that a context whose ODLA_AGGREGATE_OPS item is false never
+ * captures.
  * Where that is faster (a context measures during its first fourteen executions;
  * ODLA_HIP_BATCH_SPLIT in the environment: 0 = never, n = always from batch n
  * on) a graph that keeps the images' rows apart in every result runs as two

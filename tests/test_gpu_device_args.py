@@ -231,3 +231,49 @@ def test_new_buffer_every_call_goes_back_to_copies():
         L.odla_SetLogger(None)
         bufs.free()
         hb.destroy()
+
+
+def test_short_launch_sequences_run_uncaptured(monkeypatch):
+    """Without ODLA_HIP_GRAPH_MIN_STEPS a plan of fewer than six launches is not captured: the
+    library says so once, a new device buffer every call needs no new graph, and the results are
+    those of the oracle; a plan of six launches or more is captured as before."""
+    announce("short launch sequences")
+    monkeypatch.delenv("ODLA_HIP_GRAPH_MIN_STEPS", raising=False)
+    pkg = entry.load()
+    odla = pkg.odla
+    L = odla.load_library()
+    r = np.random.default_rng(21)
+    x0 = r.standard_normal((4, 24)).astype(np.float32)
+
+    def chain(b, n):
+        v = b.arg("x", x0.shape)
+        for i in range(n):
+            v = b.softmax(v, -1, name="s%d" % i)
+        b.output(v, "y")
+
+    for n, captured in ((2, False), (7, True)):
+        hb = odla.HipBuilder()
+        bufs = DeviceBuffers(odla, L)
+        seen = []
+        cb = capture_log(L, seen)
+        try:
+            chain(hb, n)
+            s = hb.session(True)
+            oh, oshape, odt = hb.outs["y"]
+            out = np.empty(oshape, odt)
+            assert L.odla_BindToOutput(oh, out.ctypes.data_as(ctypes.c_void_p), s.ctx) == 0
+            for k in range(3):
+                x = r.standard_normal(x0.shape).astype(np.float32)
+                want = run_ref(lambda b: chain(b, n), {"x": x})["y"]
+                assert L.odla_BindToArgument(hb.args["x"][0], bufs.put(x), s.ctx) == 0
+                s.execute()
+                assert float(np.max(np.abs(out - want))) <= 1e-5, (n, k)
+            assert any("run uncaptured" in m for m in seen) == (not captured), (n, seen[-5:])
+            assert sum("run uncaptured" in m for m in seen) <= 1
+            s.close()
+        finally:
+            L.odla_SetLogLevel(2)
+            L.odla_SetLogger(None)
+            bufs.free()
+            hb.destroy()
+        del cb

@@ -430,6 +430,12 @@ GEMM_CASES = [
     (64, 2048, 100, False, False, 1.0, 1.0, "row", True),
     (256, 2048, 1000, False, True, 0.5, 1.0, "row", True),
     (40, 1536, 130, False, False, 1.0, 0.0, None, True),
+    # at most 16 columns, a long reduction, few rows: one wavefront per output row
+    (64, 784, 10, False, False, 1.0, 1.0, "row", True),
+    (1, 2048, 16, False, True, 1.0, 0.0, None, True),
+    (37, 260, 3, False, False, 0.5, 1.0, "row", True),
+    (1000, 256, 1, False, True, 1.0, 1.0, "scalar", True),
+    (5, 1028, 7, False, False, 1.0, 1.0, "row", False),
 ]
 
 
