@@ -384,6 +384,18 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// Position of a lane in the order in which the LDS serves a 16-byte access of a wavefront:
+// four passes of sixteen lanes, and within each half of the wavefront lanes {0-3, 12-15, 20-27}
+// form one pass and lanes {4-11, 16-19, 28-31} the other (measured: two lanes that trade their
+// 16-byte slots cost an extra pass exactly when they are of different sets).  Two lanes of a
+// pass conflict when their slots are equal modulo 16.  Returns pass * 16 + place in the pass.
+__device__ __forceinline__ int lds_pass_order(const int lane) {
+  const int l = lane & 31;
+  const bool second = (l >= 4 && l < 12) || (l >= 16 && l < 20) || l >= 28;
+  const int k = second ? (l < 12 ? l - 4 : (l < 20 ? l - 8 : l - 16)) : (l < 4 ? l : (l < 16 ? l - 8 : l - 12));
+  return (lane & 32) + (second ? 16 : 0) + k;
+}
+
 // Makes the compiler wait HERE for a value that was requested from memory in conditional code.
 // The epilogues below request bias and residual vectors inside branches (per-lane validity) and
 // consume them in later branches, between which they store results.  For a value whose request
@@ -559,8 +571,19 @@ __device__ __forceinline__ void igemm_epilogue(const IgemmParams& p, const int e
   AccE* stage = reinterpret_cast<AccE*>(smem) + wave * (32 * EPI_PITCH);
   constexpr int LPP = WN / 8;    // lanes per pixel row in the read-back
   constexpr int PPP = 64 / LPP;  // pixels per read-back pass
-  const int rp = lane / LPP;     // pixel within a pass
-  const int c8 = (lane % LPP) * 8;
+  // Which (pixel, eight channels) of a pass a lane moves: any assignment covers the same full
+  // rows per store instruction, so it is chosen for the read-back from LDS - the sixteen lanes
+  // of an LDS pass (lds_pass_order) take pixel rows an odd number of 16-byte slots apart,
+  // consecutive pairs of slots each, i.e. sixteen different banks (lanes in their natural
+  // order put slots of equal bank into one pass: 25 % of the LDS cycles of the streaming 2-byte
+  // kernel were conflicts).
+  const int vl = lds_pass_order(lane), vp = vl >> 4, vw = vl & 15;
+  int rp, c8;                    // pixel within a pass, first channel
+  if constexpr (LPP == 8) { rp = vl >> 3; c8 = (vl & 7) * 8; }
+  else if constexpr (LPP == 16) { rp = (vp >> 1) * 2 + (vw >> 3); c8 = ((vp & 1) * 8 + (vw & 7)) * 8; }
+  else if constexpr (LPP == 4) { rp = (vw >> 3) * 8 + vp * 2 + ((vw >> 2) & 1); c8 = (vw & 3) * 8; }
+  else { rp = lane / LPP; c8 = (lane % LPP) * 8; }
+  (void)vp; (void)vw;
   const int n = tile_n * BN + wn * WN + c8 + n_off;
   int nvalid = p.Kout - n;
   nvalid = nvalid < 0 ? 0 : (nvalid > 8 ? 8 : nvalid);

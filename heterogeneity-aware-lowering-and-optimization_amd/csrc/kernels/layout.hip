@@ -91,17 +91,22 @@ __global__ void __launch_bounds__(kThreads) nchw_to_nhwc_smallc(LayoutParams p, 
     }
 #pragma unroll
     for (int k = 0; k < PX; ++k) {
-      TD out[16];
+      // (every index into `out` below is a constant once the loops are unrolled: an array read
+      //  back through a vector pointer at a run-time index is not split into registers, and the
+      //  compiler then keeps it in LDS)
+      alignas(16) TD out[16];
 #pragma unroll
-      for (int c = 0; c < 16; ++c)
-        if (c < p.cs) st_from_float<TD>(&out[c], c < p.C ? in[c][k] : fill, p.scale, p.zp);
+      for (int c = 0; c < 16; ++c) st_from_float<TD>(&out[c], c < p.C ? in[c][k] : fill, p.scale, p.zp);
       TD* o = dst + (n * p.HW + hw + k) * p.cs;
       if ((p.cs * sizeof(TD)) % 16 == 0) {
-        const int nv = p.cs * (int)sizeof(TD) / 16;
-        for (int v = 0; v < nv; ++v)
-          reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
+        constexpr int NV = 16 * (int)sizeof(TD) / 16;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+          if (v * 16 < p.cs * (int)sizeof(TD)) reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
       } else {
-        for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+#pragma unroll
+        for (int c = 0; c < 16; ++c)
+          if (c < p.cs) o[c] = out[c];
       }
     }
   }
@@ -568,21 +573,58 @@ __global__ void __launch_bounds__(kThreads) nchw_to_s2d_kernel(S2dParams p) {
         }
       }
     }
-    TD out[16];
-#pragma unroll
-    for (int c = 4 * CC; c < 16; ++c) st_from_float<TD>(&out[c], 0.f, p.scale, p.zp);
-#pragma unroll
-    for (int py = 0; py < 2; ++py)
-#pragma unroll
-      for (int px = 0; px < 2; ++px)
-#pragma unroll
-        for (int c = 0; c < CC; ++c) st_from_float<TD>(&out[(py * 2 + px) * CC + c], in[py][c][px], p.scale, p.zp);
     TD* o = dst + i * p.cs;
-    if ((p.cs * sizeof(TD)) % 16 == 0) {
-      const int nv = p.cs * (int)sizeof(TD) / 16;
-      for (int v = 0; v < nv; ++v) reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
+    if constexpr (sizeof(TD) <= 2) {
+      // The pixel's 16 stored values, packed into registers word by word.  (An array of TD read
+      // back through a vector pointer at a run-time index is not split into registers: the
+      // compiler moved it to LDS - two-byte writes, half of its LDS cycles bank conflicts.)
+      constexpr int PW = 4 / (int)sizeof(TD);   // values per 32-bit word
+      unsigned word[16 / PW];
+#pragma unroll
+      for (int w = 0; w < 16 / PW; ++w) {
+        word[w] = 0;
+#pragma unroll
+        for (int e = 0; e < PW; ++e) {
+          const int c = w * PW + e;   // (py * 2 + px) * CC + cc, zeros from 4 * CC on
+          const float val = c < 4 * CC ? in[(c / CC) >> 1][c % CC][(c / CC) & 1] : 0.f;
+          TD t;
+          st_from_float<TD>(&t, val, p.scale, p.zp);
+          unsigned bits;
+          if constexpr (sizeof(TD) == 2) bits = __builtin_bit_cast(unsigned short, t);
+          else bits = __builtin_bit_cast(unsigned char, t);
+          word[w] |= bits << (e * 8 * (int)sizeof(TD));
+        }
+      }
+      if ((p.cs * sizeof(TD)) % 16 == 0) {
+        reinterpret_cast<uintx4*>(o)[0] = (uintx4){word[0], word[1], word[2], word[3]};
+        if constexpr (sizeof(TD) == 2) {
+          if (p.cs == 16) reinterpret_cast<uintx4*>(o)[1] = (uintx4){word[4], word[5], word[6], word[7]};
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 16; ++c)
+          if (c < p.cs) {
+            const unsigned b = word[c / PW] >> ((c % PW) * 8 * (int)sizeof(TD));
+            if constexpr (sizeof(TD) == 2) o[c] = __builtin_bit_cast(TD, (unsigned short)b);
+            else o[c] = __builtin_bit_cast(TD, (unsigned char)b);
+          }
+      }
     } else {
-      for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+      TD out[16];
+#pragma unroll
+      for (int c = 4 * CC; c < 16; ++c) st_from_float<TD>(&out[c], 0.f, p.scale, p.zp);
+#pragma unroll
+      for (int py = 0; py < 2; ++py)
+#pragma unroll
+        for (int px = 0; px < 2; ++px)
+#pragma unroll
+          for (int c = 0; c < CC; ++c) st_from_float<TD>(&out[(py * 2 + px) * CC + c], in[py][c][px], p.scale, p.zp);
+      if ((p.cs * sizeof(TD)) % 16 == 0) {
+        const int nv = p.cs * (int)sizeof(TD) / 16;
+        for (int v = 0; v < nv; ++v) reinterpret_cast<uintx4*>(o)[v] = reinterpret_cast<const uintx4*>(out)[v];
+      } else {
+        for (int c = 0; c < p.cs; ++c) o[c] = out[c];
+      }
     }
   }
 }
