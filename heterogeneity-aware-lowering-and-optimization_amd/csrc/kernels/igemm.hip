@@ -1249,6 +1249,11 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
     if (ok16) epi_vec |= 2;
   }
 
+  if (p.f_y != nullptr) {
+    // a second layer rides in this launch: only the streaming row kernel computes it
+    if (p.in_dt != DT_I8 || p.out_dt != DT_I8 || p.w_frag == nullptr || !(epi_vec & 2)) return hipErrorInvalidValue;
+    return launch_igemm_stream_q8(p, stream);
+  }
   if (gemm_rowdot_shape(p)) return launch_gemm_rowdot(p, stream);
   if (const int big = igemm_big_variant(p)) return launch_igemm_big(p, epi_vec, big, stream);
   if (p.w_frag != nullptr && igemm_c3_geometry(p)) return launch_igemm_c3(p, epi_vec, stream);

@@ -201,7 +201,12 @@ igemm_stream_q8_kernel(const IgemmParams p, const int groups) {
 // A step's MFMAs and requantisation then cover the latency of its requests, and a store burst
 // has a whole step to drain before anything waits behind it.
 // NG: groups of 128 channels of this workgroup (blockIdx.y selects its share of the layer's).
-template <int NKK, int NG, int NW, bool kRes, bool kClamp>
+// NF > 0: a second 1x1 layer of NF * 32 channels over this layer's KOUT (all of them: one channel
+// share) is computed from the staged byte tiles - after each 128-channel step the wavefront
+// multiplies the tile it has just requantised, as it lies in LDS, into NF more accumulators, and
+// after the last step requantises those with the second layer's parameters and writes them as
+// rows of NF * 32 bytes (see IgemmParams::f_y).
+template <int NKK, int NG, int NW, bool kRes, bool kClamp, int NF = 0>
 __device__ __forceinline__ void stream_rows_body(const IgemmParams& p, const int groups, unsigned char* smem) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -215,8 +220,25 @@ __device__ __forceinline__ void stream_rows_body(const IgemmParams& p, const int
   uintx4* wl = reinterpret_cast<uintx4*>(smem);                              // [NS][NKK][64] fragments
   int* bl = reinterpret_cast<int*>(smem + (size_t)NS * NKK * 1024);          // [KOUT] bias
   float* ml = reinterpret_cast<float*>(bl + KOUT);                           // [KOUT] multipliers
-  unsigned char* otile = reinterpret_cast<unsigned char*>(ml + KOUT) + wave * (2 * TILE);
+  // second layer: fragments [NF][KOUT / 32][64], bias and multipliers [NF * 32]
+  uintx4* wl2 = reinterpret_cast<uintx4*>(ml + KOUT);
+  int* bl2 = reinterpret_cast<int*>(wl2 + (size_t)NF * (KOUT / 32) * 64);
+  float* ml2 = reinterpret_cast<float*>(bl2 + NF * 32);
+  unsigned char* otile = reinterpret_cast<unsigned char*>(ml2 + NF * 32) + wave * (2 * TILE);
   unsigned char* rtile = otile + TILE;
+  if constexpr (NF > 0) {
+    const uintx4* wf2 = reinterpret_cast<const uintx4*>(p.f_wfrag);
+    constexpr int per_slice2 = (KOUT / 32) * 64;
+    for (int u = tid; u < NF * per_slice2; u += NW * 64) {
+      const int t = u / per_slice2, rem = u - t * per_slice2;
+      wl2[u] = wf2[(int64_t)t * p.f_wf_chunks * 64 + rem];
+    }
+    const int* bias2 = reinterpret_cast<const int*>(p.f_bias);
+    for (int c = tid; c < NF * 32; c += NW * 64) {
+      bl2[c] = bias2 != nullptr ? bias2[c] : 0;
+      ml2[c] = p.f_qmul[c];
+    }
+  }
   {
     const uintx4* wf = reinterpret_cast<const uintx4*>(p.w_frag);
     constexpr int per_slice = NKK * 64;
@@ -280,6 +302,18 @@ __device__ __forceinline__ void stream_rows_body(const IgemmParams& p, const int
     //  one the compiler can count)
     const int gn = g + (int)gridDim.x < groups ? g + (int)gridDim.x : g;
     load_b(gn, bnext);
+    intx16 acc2[NF > 0 ? NF : 1];
+    if constexpr (NF > 0) {
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        const int* bj = bl2 + f * 32 + lg * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const intx4 bv = *reinterpret_cast<const intx4*>(bj + q * 8);
+          acc2[f][q * 4 + 0] = bv.x; acc2[f][q * 4 + 1] = bv.y; acc2[f][q * 4 + 2] = bv.z; acc2[f][q * 4 + 3] = bv.w;
+        }
+      }
+    }
     static_for<NG>([&](auto grp_no) __attribute__((always_inline)) {
       constexpr int grp = decltype(grp_no)::value;
       intx16 acc[4];
@@ -321,6 +355,17 @@ __device__ __forceinline__ void stream_rows_body(const IgemmParams& p, const int
               requant4<kRes, kClamp>(acc[j][q * 4 + 0], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3], m, rs, p);
         }
       wave_fence();
+      if constexpr (NF > 0) {
+        // the tile as the pixel operand of the second layer: lane (pixel l32, K half lg) takes
+        // 16 stored bytes of each of the step's four 32-channel K steps
+#pragma unroll
+        for (int k2 = 0; k2 < 4; ++k2) {
+          const uintx4 a2 = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + l32 * PITCH + k2 * 32 + lg * 16), l32);
+#pragma unroll
+          for (int f = 0; f < NF; ++f)
+            acc2[f] = Mma<int8_t>::run(wl2[(size_t)(f * (KOUT / 32) + grp * 4 + k2) * 64 + lane], a2, acc2[f]);
+        }
+      }
       uintx4 v[4];
 #pragma unroll
       for (int ps = 0; ps < 4; ++ps) v[ps] = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + (ps * 8 + rp) * PITCH + c16), ps * 8 + rp);
@@ -340,12 +385,43 @@ __device__ __forceinline__ void stream_rows_body(const IgemmParams& p, const int
       }
       wave_fence();   // the tiles are written again by the next step
     });
+    if constexpr (NF > 0) {
+      IgemmParams p2;   // (only the two fields requant4 reads without a residual)
+      p2.q_add = p.f_q_add;
+      p2.q_lo = p.f_q_lo;
+      const bool clamp2 = p.f_q_lo > 0.f;   // (wavefront-uniform)
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ch = f * 32 + q * 8 + lg * 4;
+          const int off = (l32 * PITCH + ch) ^ q8_swz(l32);
+          const floatx4 m = *reinterpret_cast<const floatx4*>(ml2 + ch);
+          *reinterpret_cast<unsigned*>(otile + off) =
+              clamp2 ? requant4<false, true>(acc2[f][q * 4 + 0], acc2[f][q * 4 + 1], acc2[f][q * 4 + 2], acc2[f][q * 4 + 3], m, 0u, p2)
+                     : requant4<false, false>(acc2[f][q * 4 + 0], acc2[f][q * 4 + 1], acc2[f][q * 4 + 2], acc2[f][q * 4 + 3], m, 0u, p2);
+        }
+      wave_fence();
+      // rows of NF * 32 bytes: LR lanes per row, 64 / LR rows per pass (kept in the cache: the
+      // next launch reads them)
+      constexpr int LR = NF * 2, RPP = 64 / LR;
+      const int rp2 = lane / LR, c2 = (lane % LR) * 16;
+      int8_t* y2 = reinterpret_cast<int8_t*>(p.f_y);
+#pragma unroll
+      for (int ps = 0; ps < 32 / RPP; ++ps) {
+        const int row = ps * RPP + rp2;
+        const uintx4 v2 = q8_swz_chunk(*reinterpret_cast<const uintx4*>(otile + row * PITCH + c2), row);
+        const int m = (g * NW + wave) * 32 + row;
+        if (m < M) store_row16(y2 + (int64_t)m * p.f_ycs + c2, v2, true, 16, false);
+      }
+      wave_fence();
+    }
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) b[kk] = bnext[kk];
   }
 }
 
-template <int NKK, int NG, int NW>
+template <int NKK, int NG, int NW, int NF = 0>
 __global__ void __launch_bounds__(NW * 64, 2)
 igemm_stream_q8_rows_kernel(const IgemmParams p, const int groups, const int epi_vec) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -353,11 +429,11 @@ igemm_stream_q8_rows_kernel(const IgemmParams p, const int groups, const int epi
   // (workgroup-uniform choices: the body is compiled once per case, so that none of its memory
   //  requests sits in a branch)
   if (p.residual != nullptr) {
-    if (p.q_lo > 0.f) stream_rows_body<NKK, NG, NW, true, true>(p, groups, smem);
-    else stream_rows_body<NKK, NG, NW, true, false>(p, groups, smem);
+    if (p.q_lo > 0.f) stream_rows_body<NKK, NG, NW, true, true, NF>(p, groups, smem);
+    else stream_rows_body<NKK, NG, NW, true, false, NF>(p, groups, smem);
   } else {
-    if (p.q_lo > 0.f) stream_rows_body<NKK, NG, NW, false, true>(p, groups, smem);
-    else stream_rows_body<NKK, NG, NW, false, false>(p, groups, smem);
+    if (p.q_lo > 0.f) stream_rows_body<NKK, NG, NW, false, true, NF>(p, groups, smem);
+    else stream_rows_body<NKK, NG, NW, false, false, NF>(p, groups, smem);
   }
 }
 
@@ -419,6 +495,24 @@ static bool stream_q8_ready(const IgemmParams& p) {
          al16(p.x) && al16(p.y) && al16(p.residual) && al16(p.w_frag);
 }
 
+// Pairs the row-epilogue form computes in one launch: 64 -> 256 channels (one channel share of two
+// 128-channel groups) followed by a plain 1x1 layer 256 -> 64 over the same pixels.  With more
+// channels on either side the two layers' weights and the staged tiles no longer fit the LDS of a
+// compute unit next to a second workgroup.
+bool igemm_stream_q8_fusable(const IgemmParams& a, const IgemmParams& b) {
+  if (const char* e = getenv("ODLA_HIP_STREAM_FUSE")) {   // tuning aid: 0 keeps the layers apart
+    if (e[0] == '0') return false;
+  }
+  if (const char* e = getenv("ODLA_HIP_STREAM_ROWS")) {
+    if (e[0] == '0') return false;
+  }
+  if (!igemm_stream_q8_geometry(a) || !igemm_stream_q8_geometry(b)) return false;
+  if (a.C != 64 || a.Kout != 256 || a.ycs != 256) return false;
+  if (b.C != 256 || b.xcs != 256 || b.Kout != 64 || b.residual != nullptr || b.ycs % 16 != 0) return false;
+  if (b.sh != 1 || b.sw != 1 || b.H != a.Ho || b.W != a.Wo || b.N != a.N || b.Ho != b.H || b.Wo != b.W) return false;
+  return true;
+}
+
 // The row-epilogue form: 128-channel groups, four wavefronts, the layer's channels split over
 // blockIdx.y so that a share's weights stay within 32 KiB.
 static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream) {
@@ -429,8 +523,16 @@ static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream
   while (ng > 1 && (ng * 128 * p.C > 32 * 1024 || (ng != 1 && ng != 2))) ng = (ng % 2 == 0) ? ng / 2 : 1;
   const int nsplit = p.Kout / (ng * 128);
   const int64_t groups = (M + nw * 32 - 1) / (nw * 32);
-  // weights, bias and multipliers of the share, two staged byte tiles per wavefront
-  const size_t lds = (size_t)ng * 4 * nkk * 1024 + (size_t)ng * 128 * 8 + (size_t)nw * (2 * 32 * 144);
+  const int nf = p.f_y != nullptr ? p.f_kout / 32 : 0;
+  if (nf != 0) {   // (igemm_stream_q8_fusable)
+    auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    if (nsplit != 1 || nkk != 2 || ng != 2 || nf != 2 || p.f_kout != 64 || p.f_wfrag == nullptr || p.f_qmul == nullptr ||
+        p.f_wf_chunks < 8 || p.f_ycs % 16 != 0 || !al16(p.f_y) || !al16(p.f_wfrag))
+      return hipErrorInvalidValue;
+  }
+  // weights, bias and multipliers of the share (and of the second layer), two staged byte tiles per wavefront
+  const size_t lds = (size_t)ng * 4 * nkk * 1024 + (size_t)ng * 128 * 8 + (size_t)nf * (ng * 4) * 1024 + (size_t)nf * 32 * 8 +
+                     (size_t)nw * (2 * 32 * 144);
   if (groups > 0x7fffffff) return hipErrorInvalidValue;
   int per_cu = (int)((160 * 1024) / (lds + 512));
   per_cu = per_cu > 4 ? 4 : (per_cu < 1 ? 1 : per_cu);
@@ -454,6 +556,17 @@ static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream
                        p, (int)groups, epi_vec);                                                                    \
     return hipGetLastError();                                                                                       \
   }
+  if (nf == 2) {
+    static bool attr_set = false;
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_rows_kernel<2, 2, nw, 2>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      if (e != hipSuccess) return e;
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((igemm_stream_q8_rows_kernel<2, 2, nw, 2>), dim3((unsigned)grid, 1u), dim3(nw * 64), lds, stream, p, (int)groups, epi_vec);
+    return hipGetLastError();
+  }
   ROWS_CASE(2, 1)
   ROWS_CASE(2, 2)
   ROWS_CASE(4, 1)
@@ -472,11 +585,12 @@ hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream) {
   // 2.68 -> 2.57 ms per step.  ODLA_HIP_STREAM_ROWS=0 keeps the lane-exchange form.
   if (p.Kout % 128 == 0 && (p.C == 64 || p.C == 128 || p.C == 256)) {
     const char* e = getenv("ODLA_HIP_STREAM_ROWS");
-    if (e == nullptr || e[0] != '0') {
+    if (e == nullptr || e[0] != '0' || p.f_y != nullptr) {
       const hipError_t r = launch_stream_q8_rows(p, stream);
       if (r != hipErrorInvalidValue) return r;
     }
   }
+  if (p.f_y != nullptr) return hipErrorInvalidValue;   // (the lane-exchange form computes no second layer)
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
   const int kout_wg = stream_q8_channels_per_wg(p);
   const int nkk = p.C / 32, ns = kout_wg / 32, nsplit = p.Kout / kout_wg;

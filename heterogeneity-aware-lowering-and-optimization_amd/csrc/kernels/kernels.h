@@ -140,6 +140,16 @@ struct IgemmParams {
   int a_fill = 0;  // stored byte that represents the real value 0 in x
   float q_add = 0.f, q_lo = 0.f;
   float r_mul = 0.f, r_add = 0.f;
+  // A second 8-bit 1x1 layer computed from this layer's result while a pixel tile of it is still
+  // in LDS (f_y != nullptr; igemm_stream_q8_fusable says which pairs): y2 = requant(y . w2 + bias2)
+  // with the second layer's own fragment-ordered weights, int32 bias, multipliers, zero point and
+  // lower bound.  Both results are written; the second layer's read of y from memory is what is saved.
+  const void* f_wfrag = nullptr;
+  const void* f_bias = nullptr;
+  const float* f_qmul = nullptr;
+  void* f_y = nullptr;
+  int f_kout = 0, f_ycs = 0, f_wf_chunks = 0;
+  float f_q_add = 0.f, f_q_lo = 0.f;
 };
 hipError_t launch_igemm(const IgemmParams& p, hipStream_t stream);
 // Name of the kernel variant launch_igemm would pick (for reports).
@@ -159,6 +169,9 @@ hipError_t launch_igemm_big(const IgemmParams& p, int epi_vec, int variant, hipS
 // whether the layer's geometry qualifies (no pointer is looked at), and the launch
 // (p.w_frag, p.qmul and the division magics must be set; launch_igemm does that).
 bool igemm_stream_q8_geometry(const IgemmParams& p);
+// Whether layer b (its x being a's result) can ride in a's launch (see IgemmParams::f_y); no
+// pointer is looked at.
+bool igemm_stream_q8_fusable(const IgemmParams& a, const IgemmParams& b);
 hipError_t launch_igemm_stream_q8(const IgemmParams& p, hipStream_t stream);
 // 3x3, stride 1, padding 1 with the input patch of a tile held in LDS (igemm_c3.hip): whether
 // the layer is one of its shapes, and its launch (called by launch_igemm with its epi_vec).

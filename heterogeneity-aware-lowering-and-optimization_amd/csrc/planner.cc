@@ -155,6 +155,15 @@ class Planner {
     return (int)plan_->tensors.size() - 1;
   }
   std::unordered_set<int> arena_only_;   // root tensors that some step writes, or reads relying on the arena
+  // The last 8-bit convolution step, kept so that a plain 1x1 layer over its result can ride in
+  // its launch (lower_conv; igemm_stream_q8_fusable decides).
+  struct FuseProducer {
+    int step = -1;
+    const _odla_value* out = nullptr;
+    IgemmParams ip;
+    int tx = -1, tw = -1, ty = -1, tb = -1, tm = -1, tr = -1, tf = -1;
+  };
+  FuseProducer fuse_prod_;
   int root(int t) const {
     while (plan_->tensors[t].alias_of >= 0) t = plan_->tensors[t].alias_of;
     return t;
@@ -1410,6 +1419,42 @@ void Planner::lower_conv(int ni) {
     const Ref rf = ref(hf ? tf : tx);
     const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb), rm = ref(tm), rr = ref(tr >= 0 ? tr : tx);
     const bool hr = tr >= 0;
+    if (fuse_prod_.step >= 0 && fuse_prod_.out == x && !in_init_ && hf && !hr && ip.out_dt == DT_I8 && tx == fuse_prod_.ty &&
+        igemm_stream_q8_fusable(fuse_prod_.ip, ip)) {
+      // This layer reads the result of the step before it pixel by pixel: that step computes it
+      // too, from its staged tiles, and writes both results - one launch and one pass over the
+      // wide tensor less.
+      const FuseProducer fp = fuse_prod_;
+      fuse_prod_.step = -1;
+      IgemmParams fa = fp.ip;
+      fa.f_kout = ip.Kout; fa.f_ycs = ip.ycs; fa.f_wf_chunks = ip.wf_chunks;
+      fa.f_q_add = ip.q_add; fa.f_q_lo = ip.q_lo;
+      const Ref ax = ref(fp.tx), aw = ref(fp.tw), ay = ref(fp.ty), ab = ref(fp.tb), am = ref(fp.tm), af = ref(fp.tf);
+      const Ref ar = ref(fp.tr >= 0 ? fp.tr : fp.tx);
+      const bool ahr = fp.tr >= 0;
+      Step& sa = plan_->steps[(size_t)fp.step];
+      OHIP_INFO("int8 plan: '%s' is computed in the launch of '%s' (from its tiles in LDS)", outv->name.c_str(), sa.name.c_str());
+      sa.name += "+" + outv->name;
+      sa.fn = [=](const ExecEnv& e, hipStream_t st) {
+        IgemmParams p = fa;
+        p.x = ax(e); p.w = aw(e); p.y = ay(e); p.bias = ab(e);
+        p.qmul = (const float*)am(e);
+        p.residual = ahr ? ar(e) : nullptr;
+        p.w_frag = af(e);
+        p.f_wfrag = rf(e); p.f_bias = rb(e); p.f_qmul = (const float*)rm(e); p.f_y = ry(e);
+        return launch_igemm(p, st);
+      };
+      {  // the second result is written by that step
+        PTensor& yt = T(root(ty));
+        if (yt.space == SP_ARENA) {
+          if (fp.step < yt.def_step) yt.def_step = fp.step;
+          if (fp.step > yt.last_step) yt.last_step = fp.step;
+        }
+        arena_only_.insert(root(ty));
+      }
+      set_main(outv, ty);
+      return;
+    }
     emit("conv.i8:" + outv->name, {tx, tw, tr}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
       IgemmParams p = ip;
       p.x = rx(e); p.w = rw(e); p.y = ry(e); p.bias = rb(e);
@@ -1418,6 +1463,13 @@ void Planner::lower_conv(int ni) {
       p.w_frag = hf ? rf(e) : nullptr;
       return launch_igemm(p, st);
     });
+    fuse_prod_.step = -1;
+    if (!in_init_ && hf && ip.out_dt == DT_I8 && !calib_) {
+      fuse_prod_.step = (int)plan_->steps.size() - 1;
+      fuse_prod_.out = outv;
+      fuse_prod_.ip = ip;
+      fuse_prod_.tx = tx; fuse_prod_.tw = tw; fuse_prod_.ty = ty; fuse_prod_.tb = tb; fuse_prod_.tm = tm; fuse_prod_.tr = tr; fuse_prod_.tf = tf;
+    }
     if (ip.out_dt == DT_I32) {
       // raw accumulators are exposed through the FLOAT32-typed value as bit patterns
       T(ty).dt = DT_F32;
