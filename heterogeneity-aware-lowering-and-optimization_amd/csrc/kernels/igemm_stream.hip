@@ -496,7 +496,7 @@ static bool stream_q8_ready(const IgemmParams& p) {
 }
 
 // Pairs the row-epilogue form computes in one launch: 64 -> 256 channels (one channel share of two
-// 128-channel groups) followed by a plain 1x1 layer 256 -> 64 over the same pixels.  With more
+// 128-channel groups) followed by a plain 1x1 layer 256 -> 64 or 256 -> 128 over the same pixels.  With more
 // channels on either side the two layers' weights and the staged tiles no longer fit the LDS of a
 // compute unit next to a second workgroup.
 bool igemm_stream_q8_fusable(const IgemmParams& a, const IgemmParams& b) {
@@ -508,7 +508,7 @@ bool igemm_stream_q8_fusable(const IgemmParams& a, const IgemmParams& b) {
   }
   if (!igemm_stream_q8_geometry(a) || !igemm_stream_q8_geometry(b)) return false;
   if (a.C != 64 || a.Kout != 256 || a.ycs != 256) return false;
-  if (b.C != 256 || b.xcs != 256 || b.Kout != 64 || b.residual != nullptr || b.ycs % 16 != 0) return false;
+  if (b.C != 256 || b.xcs != 256 || (b.Kout != 64 && b.Kout != 128) || b.residual != nullptr || b.ycs % 16 != 0) return false;
   if (b.sh != 1 || b.sw != 1 || b.H != a.Ho || b.W != a.Wo || b.N != a.N || b.Ho != b.H || b.Wo != b.W) return false;
   return true;
 }
@@ -518,16 +518,18 @@ bool igemm_stream_q8_fusable(const IgemmParams& a, const IgemmParams& b) {
 static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream) {
   const int64_t M = (int64_t)p.N * p.Ho * p.Wo;
   const int nkk = p.C / 32;
-  constexpr int nw = 4;
   int ng = p.Kout / 128;                          // groups per workgroup
   while (ng > 1 && (ng * 128 * p.C > 32 * 1024 || (ng != 1 && ng != 2))) ng = (ng % 2 == 0) ? ng / 2 : 1;
   const int nsplit = p.Kout / (ng * 128);
-  const int64_t groups = (M + nw * 32 - 1) / (nw * 32);
   const int nf = p.f_y != nullptr ? p.f_kout / 32 : 0;
+  // (a second layer of 128 channels: its weights leave room for one workgroup per compute unit,
+  //  which then has eight wavefronts instead of four)
+  const int nw = nf == 4 ? 8 : 4;
+  const int64_t groups = (M + nw * 32 - 1) / (nw * 32);
   if (nf != 0) {   // (igemm_stream_q8_fusable)
     auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
-    if (nsplit != 1 || nkk != 2 || ng != 2 || nf != 2 || p.f_kout != 64 || p.f_wfrag == nullptr || p.f_qmul == nullptr ||
-        p.f_wf_chunks < 8 || p.f_ycs % 16 != 0 || !al16(p.f_y) || !al16(p.f_wfrag))
+    if (nsplit != 1 || nkk != 2 || ng != 2 || (nf != 2 && nf != 4) || p.f_kout != nf * 32 || p.f_wfrag == nullptr ||
+        p.f_qmul == nullptr || p.f_wf_chunks < 8 || p.f_ycs % 16 != 0 || !al16(p.f_y) || !al16(p.f_wfrag))
       return hipErrorInvalidValue;
   }
   // weights, bias and multipliers of the share (and of the second layer), two staged byte tiles per wavefront
@@ -547,26 +549,31 @@ static hipError_t launch_stream_q8_rows(const IgemmParams& p, hipStream_t stream
   if (nkk == NKK_ && ng == NG_) {                                                                                    \
     static bool attr_set = false;                                                                                   \
     if (!attr_set) {                                                                                                \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_rows_kernel<NKK_, NG_, nw>), \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_rows_kernel<NKK_, NG_, 4>), \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);                    \
       if (e != hipSuccess) return e;                                                                                \
       attr_set = true;                                                                                              \
     }                                                                                                               \
-    hipLaunchKernelGGL((igemm_stream_q8_rows_kernel<NKK_, NG_, nw>), dim3((unsigned)grid, (unsigned)nsplit), dim3(nw * 64), lds, stream, \
+    hipLaunchKernelGGL((igemm_stream_q8_rows_kernel<NKK_, NG_, 4>), dim3((unsigned)grid, (unsigned)nsplit), dim3(4 * 64), lds, stream, \
                        p, (int)groups, epi_vec);                                                                    \
     return hipGetLastError();                                                                                       \
   }
-  if (nf == 2) {
-    static bool attr_set = false;
-    if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_rows_kernel<2, 2, nw, 2>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-      if (e != hipSuccess) return e;
-      attr_set = true;
-    }
-    hipLaunchKernelGGL((igemm_stream_q8_rows_kernel<2, 2, nw, 2>), dim3((unsigned)grid, 1u), dim3(nw * 64), lds, stream, p, (int)groups, epi_vec);
-    return hipGetLastError();
+#define FUSED_CASE(NF_, NW_)                                                                                          \
+  if (nf == NF_) {                                                                                                    \
+    static bool attr_set = false;                                                                                    \
+    if (!attr_set) {                                                                                                 \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&igemm_stream_q8_rows_kernel<2, 2, NW_, NF_>), \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);                    \
+      if (e != hipSuccess) return e;                                                                                 \
+      attr_set = true;                                                                                               \
+    }                                                                                                                \
+    hipLaunchKernelGGL((igemm_stream_q8_rows_kernel<2, 2, NW_, NF_>), dim3((unsigned)grid, 1u), dim3(NW_ * 64), lds, stream, p, \
+                       (int)groups, epi_vec);                                                                        \
+    return hipGetLastError();                                                                                        \
   }
+  FUSED_CASE(2, 4)
+  FUSED_CASE(4, 8)
+#undef FUSED_CASE
   ROWS_CASE(2, 1)
   ROWS_CASE(2, 2)
   ROWS_CASE(4, 1)

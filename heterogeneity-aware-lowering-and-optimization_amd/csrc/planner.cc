@@ -155,7 +155,7 @@ class Planner {
     return (int)plan_->tensors.size() - 1;
   }
   std::unordered_set<int> arena_only_;   // root tensors that some step writes, or reads relying on the arena
-  // The last 8-bit convolution step, kept so that a plain 1x1 layer over its result can ride in
+  // The 8-bit convolution steps, kept so that a plain 1x1 layer over the result of one can ride in
   // its launch (lower_conv; igemm_stream_q8_fusable decides).
   struct FuseProducer {
     int step = -1;
@@ -163,7 +163,7 @@ class Planner {
     IgemmParams ip;
     int tx = -1, tw = -1, ty = -1, tb = -1, tm = -1, tr = -1, tf = -1;
   };
-  FuseProducer fuse_prod_;
+  std::unordered_map<const _odla_value*, FuseProducer> fuse_prods_;   // by result value
   int root(int t) const {
     while (plan_->tensors[t].alias_of >= 0) t = plan_->tensors[t].alias_of;
     return t;
@@ -1419,13 +1419,14 @@ void Planner::lower_conv(int ni) {
     const Ref rf = ref(hf ? tf : tx);
     const Ref rx = ref(tx), rw = ref(tw), ry = ref(ty), rb = ref(tb), rm = ref(tm), rr = ref(tr >= 0 ? tr : tx);
     const bool hr = tr >= 0;
-    if (fuse_prod_.step >= 0 && fuse_prod_.out == x && !in_init_ && hf && !hr && ip.out_dt == DT_I8 && tx == fuse_prod_.ty &&
-        igemm_stream_q8_fusable(fuse_prod_.ip, ip)) {
+    const auto prod = fuse_prods_.find(x);
+    if (prod != fuse_prods_.end() && !in_init_ && hf && !hr && ip.out_dt == DT_I8 && tx == prod->second.ty &&
+        igemm_stream_q8_fusable(prod->second.ip, ip)) {
       // This layer reads the result of the step before it pixel by pixel: that step computes it
       // too, from its staged tiles, and writes both results - one launch and one pass over the
       // wide tensor less.
-      const FuseProducer fp = fuse_prod_;
-      fuse_prod_.step = -1;
+      const FuseProducer fp = prod->second;
+      fuse_prods_.erase(prod);   // (one rider per launch)
       IgemmParams fa = fp.ip;
       fa.f_kout = ip.Kout; fa.f_ycs = ip.ycs; fa.f_wf_chunks = ip.wf_chunks;
       fa.f_q_add = ip.q_add; fa.f_q_lo = ip.q_lo;
@@ -1463,12 +1464,12 @@ void Planner::lower_conv(int ni) {
       p.w_frag = hf ? rf(e) : nullptr;
       return launch_igemm(p, st);
     });
-    fuse_prod_.step = -1;
     if (!in_init_ && hf && ip.out_dt == DT_I8 && !calib_) {
-      fuse_prod_.step = (int)plan_->steps.size() - 1;
-      fuse_prod_.out = outv;
-      fuse_prod_.ip = ip;
-      fuse_prod_.tx = tx; fuse_prod_.tw = tw; fuse_prod_.ty = ty; fuse_prod_.tb = tb; fuse_prod_.tm = tm; fuse_prod_.tr = tr; fuse_prod_.tf = tf;
+      FuseProducer& fp = fuse_prods_[outv];
+      fp.step = (int)plan_->steps.size() - 1;
+      fp.out = outv;
+      fp.ip = ip;
+      fp.tx = tx; fp.tw = tw; fp.ty = ty; fp.tb = tb; fp.tm = tm; fp.tr = tr; fp.tf = tf;
     }
     if (ip.out_dt == DT_I32) {
       // raw accumulators are exposed through the FLOAT32-typed value as bit patterns

@@ -179,6 +179,56 @@ def test_q8_residual_fused_equals_unfused_equals_oracle(dims, tiles_per_wg, odla
     assert np.max(np.abs(fq.astype(np.int32) - oq.astype(np.int32))[inside]) <= 2
 
 
+@pytest.mark.parametrize("dims", [(2, 9, 9, 64), (3, 21, 19, 64), (1, 40, 40, 128), (5, 7, 7, 128), (2, 16, 16, 96)])
+@pytest.mark.parametrize("relu2", [True, False])
+def test_q8_expanding_layer_carries_the_next_reducing_layer(dims, relu2, odla, ref, monkeypatch):
+    """64 -> 256 (+ residual + ReLU) followed by a plain 1x1 layer 256 -> 64 / 128 over its result:
+    the first launch computes both (the second layer from the first's tiles in LDS).  Both results
+    are bit-equal to the oracle, and to the two layers launched one after the other
+    (ODLA_HIP_STREAM_FUSE=0); 96 output channels are not carried and take the ordinary road.
+    Pixel counts that end inside a wavefront's 32-pixel tile and inside a workgroup's group."""
+    announce("q8 carried layer %s relu2=%s" % (dims, relu2))
+    N, H, W, O2 = dims
+    r = rng(31)
+    x = r.standard_normal((N, 64, H, W)).astype(np.float32)
+    res = (r.standard_normal((N, 256, H, W)) * 2).astype(np.float32)
+    w1 = (r.standard_normal((256, 64, 1, 1)) * 0.3).astype(np.float32)
+    b1 = r.standard_normal(256).astype(np.float32)
+    w2 = (r.standard_normal((O2, 256, 1, 1)) * 0.1).astype(np.float32)
+    b2 = r.standard_normal(O2).astype(np.float32)
+    ranges = {"x": (float(x.min()), float(x.max())), "res": (float(res.min()), float(res.max())),
+              "c": (-6.0, 6.0), "out": (0.0, 9.0), "y2": ((0.0, 7.0) if relu2 else (-7.0, 7.0))}
+    # ('c' needs its entry for the residual Add to be fused behind the convolution; the fused
+    #  chain then requantises once, to the entry of 'out')
+    qp = {k: ref.act_qparams(*v) for k, v in ranges.items()}
+
+    def build(b):
+        v = b.arg("x", x.shape)
+        rr = b.arg("res", res.shape)
+        c = b.conv(v, b.const("w1", w1), b.const("b1", b1), name="c")
+        out = b.relu(b.add(c, rr, name="add"), name="out")
+        b.output(out, "out")
+        y2 = b.conv(out, b.const("w2", w2), b.const("b2", b2), name="y2pre" if relu2 else "y2")
+        if relu2:
+            y2 = b.relu(y2, name="y2")
+        b.output(y2, "y2")
+
+    def run():
+        return run_hip(build, {"x": x, "res": res}, quant_table=table_for(odla, ranges, {"w1": w1, "w2": w2}))
+
+    carried = run()
+    monkeypatch.setenv("ODLA_HIP_STREAM_FUSE", "0")
+    apart = run()
+
+    xq = ref.quantize_act(x, *qp["x"])
+    rq = ref.quantize_act(res, *qp["res"])
+    oq, _ = ref.qconv(xq, qp["x"], w1, b1, qp["out"], (1, 1), (0, 0, 0, 0), relu=True, residual=(rq, qp["res"]))
+    yq, _ = ref.qconv(oq, qp["out"], w2, b2, qp["y2"], (1, 1), (0, 0, 0, 0), relu=relu2)
+    for got in (carried, apart):
+        assert np.array_equal(got["out"], ref.dequantize_act(oq, *qp["out"]))
+        assert np.array_equal(got["y2"], ref.dequantize_act(yq, *qp["y2"]))
+
+
 SMALL_STAGES = [(16, 2, 1), (32, 2, 2)]
 
 
