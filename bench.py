@@ -437,9 +437,17 @@ def profile_roofline(L, sess, wl, dump_path=None):
                 t_by[key] = t_by.get(key, 0.0) + buf[i].ms
         bound_ms = meas_ms = nbytes = 0.0
         hbm_bound = 0
-        for key, (fl, act, wt) in wl.conv_elements.items():
-            if key not in t_by:
-                continue
+        # a launch that computes a second layer from the first layer's tiles ("a+b") is priced as
+        # one launch: the operations and bytes of both, less the second layer's read of its input
+        priced = {}
+        for key in t_by:
+            parts = key.split("+")
+            if all(k in wl.conv_elements for k in parts):
+                fl = sum(wl.conv_elements[k][0] for k in parts)
+                act = sum(wl.conv_elements[k][1] for k in parts) - sum(wl.conv_elements[k][3] for k in parts[1:])
+                wt = sum(wl.conv_elements[k][2] for k in parts)
+                priced[key] = (fl, act, wt)
+        for key, (fl, act, wt) in priced.items():
             by = (act + wt) * es
             t_m, t_h = fl / (peak * 1e12) * 1e3, by / 8e12 * 1e3
             hbm_bound += t_h > t_m
@@ -450,7 +458,7 @@ def profile_roofline(L, sess, wl, dump_path=None):
             roof["hbm"] = {"algorithmic_GB_per_step": round(nbytes / 1e9, 3),
                            "achieved_GBps": round(nbytes / (meas_ms * 1e-3) / 1e9, 1), "peak_GBps": 8000.0,
                            "frac": round(nbytes / (meas_ms * 1e-3) / 8e12, 4),
-                           "launches_hbm_bound": int(hbm_bound), "launches_priced": len(t_by)}
+                           "launches_hbm_bound": int(hbm_bound), "launches_priced": len(priced)}
             roof["frac_of_per_launch_roofline"] = round(bound_ms / meas_ms, 4)
     return roof
 

@@ -127,14 +127,16 @@ RESNET50_GFLOP_PER_IMAGE = 2 * (4087136256 + 2048000) / 1e9   # conv + FC multip
 
 def resnet50_conv_elements(batch, hw=224, stages=RESNET50_STAGES, stem=64, cin_stored=8):
     """Algorithmic element traffic of the convolution launches of one step:
-    {name: (flops, activation elements read + written, weight elements)}.
+    {name: (flops, activation elements read + written, weight elements, input elements)}.
     Each launch reads its input once, its residual once (c3 launches: the
     block's shortcut is fused into them) and writes its output once; the stem
     reads the library's channels-last copy of the image, which stores
-    `cin_stored` channels per source pixel."""
+    `cin_stored` channels per source pixel.  (The input elements alone are what a
+    launch saves when the layer before it computes it from its own tiles.)"""
     out = {}
     h = (hw + 2 * 3 - 7) // 2 + 1
-    out["stem"] = (2.0 * batch * h * h * stem * 3 * 49, batch * (hw * hw * cin_stored + h * h * stem), stem * 3 * 49)
+    out["stem"] = (2.0 * batch * h * h * stem * 3 * 49, batch * (hw * hw * cin_stored + h * h * stem), stem * 3 * 49,
+                   batch * hw * hw * cin_stored)
     h = (h + 2 - 3) // 2 + 1
     cin = stem
     for si, (mid, blocks, stride) in enumerate(stages):
@@ -144,10 +146,13 @@ def resnet50_conv_elements(batch, hw=224, stages=RESNET50_STAGES, stem=64, cin_s
             p = "l%db%d" % (si + 1, bi)
             ho = (h - 1) // s + 1
             if bi == 0:
-                out[p + "ds"] = (2.0 * batch * ho * ho * cout * cin, batch * (h * h * cin + ho * ho * cout), cout * cin)
-            out[p + "c1"] = (2.0 * batch * h * h * mid * cin, batch * (h * h * cin + h * h * mid), mid * cin)
-            out[p + "c2"] = (2.0 * batch * ho * ho * mid * mid * 9, batch * (h * h * mid + ho * ho * mid), mid * mid * 9)
-            out[p + "c3"] = (2.0 * batch * ho * ho * cout * mid, batch * (ho * ho * mid + 2 * ho * ho * cout), cout * mid)
+                out[p + "ds"] = (2.0 * batch * ho * ho * cout * cin, batch * (h * h * cin + ho * ho * cout), cout * cin,
+                                 batch * h * h * cin)
+            out[p + "c1"] = (2.0 * batch * h * h * mid * cin, batch * (h * h * cin + h * h * mid), mid * cin, batch * h * h * cin)
+            out[p + "c2"] = (2.0 * batch * ho * ho * mid * mid * 9, batch * (h * h * mid + ho * ho * mid), mid * mid * 9,
+                             batch * h * h * mid)
+            out[p + "c3"] = (2.0 * batch * ho * ho * cout * mid, batch * (ho * ho * mid + 2 * ho * ho * cout), cout * mid,
+                             batch * ho * ho * mid)
             cin, h = cout, ho
     return out
 
