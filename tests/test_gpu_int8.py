@@ -179,22 +179,25 @@ def test_q8_residual_fused_equals_unfused_equals_oracle(dims, tiles_per_wg, odla
     assert np.max(np.abs(fq.astype(np.int32) - oq.astype(np.int32))[inside]) <= 2
 
 
-@pytest.mark.parametrize("dims", [(2, 9, 9, 64), (3, 21, 19, 64), (1, 40, 40, 128), (5, 7, 7, 128), (2, 16, 16, 96)])
+@pytest.mark.parametrize("dims", [(2, 9, 9, 64), (3, 21, 19, 64), (1, 40, 40, 128), (5, 7, 7, 128), (2, 16, 16, 96),
+                                  (2, 9, 9, 128, 128, 512), (3, 21, 19, 128, 128, 512), (1, 28, 28, 128, 128, 512)])
 @pytest.mark.parametrize("relu2", [True, False])
 def test_q8_expanding_layer_carries_the_next_reducing_layer(dims, relu2, odla, ref, monkeypatch):
     """64 -> 256 (+ residual + ReLU) followed by a plain 1x1 layer 256 -> 64 / 128 over its result:
     the first launch computes both (the second layer from the first's tiles in LDS).  Both results
     are bit-equal to the oracle, and to the two layers launched one after the other
-    (ODLA_HIP_STREAM_FUSE=0); 96 output channels are not carried and take the ordinary road.
+    (ODLA_HIP_STREAM_FUSE=0); 96 output channels, and the pair 128 -> 512 -> 128, are not carried and
+    take the ordinary road.
     Pixel counts that end inside a wavefront's 32-pixel tile and inside a workgroup's group."""
     announce("q8 carried layer %s relu2=%s" % (dims, relu2))
-    N, H, W, O2 = dims
+    N, H, W, O2 = dims[:4]
+    C1, O1 = dims[4:] if len(dims) > 4 else (64, 256)
     r = rng(31)
-    x = r.standard_normal((N, 64, H, W)).astype(np.float32)
-    res = (r.standard_normal((N, 256, H, W)) * 2).astype(np.float32)
-    w1 = (r.standard_normal((256, 64, 1, 1)) * 0.3).astype(np.float32)
-    b1 = r.standard_normal(256).astype(np.float32)
-    w2 = (r.standard_normal((O2, 256, 1, 1)) * 0.1).astype(np.float32)
+    x = r.standard_normal((N, C1, H, W)).astype(np.float32)
+    res = (r.standard_normal((N, O1, H, W)) * 2).astype(np.float32)
+    w1 = (r.standard_normal((O1, C1, 1, 1)) * 0.3).astype(np.float32)
+    b1 = r.standard_normal(O1).astype(np.float32)
+    w2 = (r.standard_normal((O2, O1, 1, 1)) * 0.1).astype(np.float32)
     b2 = r.standard_normal(O2).astype(np.float32)
     ranges = {"x": (float(x.min()), float(x.max())), "res": (float(res.min()), float(res.max())),
               "c": (-6.0, 6.0), "out": (0.0, 9.0), "y2": ((0.0, 7.0) if relu2 else (-7.0, 7.0))}
