@@ -237,10 +237,10 @@ def run_workload(pkg, L, name, args, with_cpu):
     L.odla_SetLogger(ctypes.cast(cb, ctypes.c_void_p))
     L.odla_SetLogLevel(4)
     try:
-        # set-up, like the graph capture: the context's first fourteen executions measure whether
-        # the batch runs whole (six) or as two half-batch copies (eight) and say which it keeps
+        # set-up, like the graph capture: the context's first sixteen executions measure whether
+        # the batch runs whole (six) or as two half-batch copies (ten) and say which it keeps
         # (nothing to measure when ODLA_HIP_BATCH_SPLIT decides)
-        for _ in range(0 if os.environ.get("ODLA_HIP_BATCH_SPLIT") else 14):
+        for _ in range(0 if os.environ.get("ODLA_HIP_BATCH_SPLIT") else 16):
             sess.execute()
         for _ in range(args.warmup):
             sess.execute()
@@ -304,8 +304,8 @@ def end_to_end(hb, wl, steps):
         outs = sess.bind_host_io(wl.feeds, pinned=pinned)
         out["host_bytes_per_step"] = int(sum(v.nbytes for v in wl.feeds.values()) + sum(o.nbytes for o in outs.values()))
         # untimed: the captures, and the executions in which the context measures whether to
-        # run the batch whole (six) or as two half-batch copies (eight)
-        for _ in range(1 if os.environ.get("ODLA_HIP_BATCH_SPLIT") else 15):
+        # run the batch whole (six) or as two half-batch copies (ten)
+        for _ in range(1 if os.environ.get("ODLA_HIP_BATCH_SPLIT") else 17):
             sess.execute()
         t0 = time.perf_counter()
         for _ in range(steps):

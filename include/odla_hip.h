@@ -293,7 +293,7 @@ odla_status odla_BindToOutputById(const odla_value_id value_id,
  * ODLA_HIP_GRAPH_MIN_STEPS in the environment sets another bound, 1 = always
  * a graph) and that a context whose ODLA_AGGREGATE_OPS item is false never
  * captures.
- * Where that is faster (a context measures during its first fourteen executions;
+ * Where that is faster (a context measures during its first sixteen executions;
  * ODLA_HIP_BATCH_SPLIT in the environment: 0 = never, n = always from batch n
  * on) a graph that keeps the images' rows apart in every result runs as two
  * copies at half the batch (every argument's leading extent), side by side on

@@ -71,7 +71,7 @@ def test_a_context_measures_and_keeps_the_faster_way(monkeypatch):
         try:
             def go():
                 outs = []
-                for _ in range(16):
+                for _ in range(18):
                     outs.append(s.run({"x": x}))
                 return outs
             outs, seen = run_logged(go)
