@@ -190,6 +190,7 @@ def test_q8_expanding_layer_carries_the_next_reducing_layer(dims, relu2, odla, r
     take the ordinary road.
     Pixel counts that end inside a wavefront's 32-pixel tile and inside a workgroup's group."""
     announce("q8 carried layer %s relu2=%s" % (dims, relu2))
+    monkeypatch.delenv("ODLA_HIP_STREAM_FUSE", raising=False)
     N, H, W, O2 = dims[:4]
     C1, O1 = dims[4:] if len(dims) > 4 else (64, 256)
     r = rng(31)
@@ -230,6 +231,14 @@ def test_q8_expanding_layer_carries_the_next_reducing_layer(dims, relu2, odla, r
     for got in (carried, apart):
         assert np.array_equal(got["out"], ref.dequantize_act(oq, *qp["out"]))
         assert np.array_equal(got["y2"], ref.dequantize_act(yq, *qp["y2"]))
+
+
+def test_q8_carried_layer_in_two_half_batches(odla, ref, monkeypatch):
+    """The pair above executed as two half-batch copies of the plan on two streams (each copy's
+    first launch carries the second layer): both results bit-equal to the oracle."""
+    monkeypatch.setenv("ODLA_HIP_BATCH_SPLIT", "2")
+    test_q8_expanding_layer_carries_the_next_reducing_layer((4, 21, 19, 64), True, odla, ref, monkeypatch)
+    test_q8_expanding_layer_carries_the_next_reducing_layer((6, 9, 9, 128), False, odla, ref, monkeypatch)
 
 
 SMALL_STAGES = [(16, 2, 1), (32, 2, 2)]
