@@ -5,7 +5,8 @@
 // lane l takes the 16-byte pieces l, l + 64, .. of the row and of every weight row, all of
 // a lane's requests are in flight together, and the partial sums meet in a wavefront
 // reduction.  fp32 only (the summation order differs from the tiled kernels': within the
-// fp32 bound, as theirs differ among themselves).
+// fp32 bound, as theirs differ among themselves).  With every column of a row in one wavefront
+// a Softmax / LogSoftmax over the columns is a few more instructions (IgemmParams::row_softmax).
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
@@ -46,12 +47,19 @@ __global__ __launch_bounds__(64) void gemm_rowdot_kernel(const IgemmParams p) {
     const float s = wave_sum(acc[n]);
     mine = lane == n ? s : mine;
   }
-  if (lane < p.Kout) {
-    const float b = p.bias ? reinterpret_cast<const float*>(p.bias)[lane] : 0.f;
-    float v = __builtin_fmaf(mine, p.alpha, b);
-    v = apply_act(v, p.act, p.act_a, p.act_b);
-    reinterpret_cast<float*>(p.y)[(int64_t)m * p.ycs + lane] = v;
+  const bool col = lane < p.Kout;
+  const float b = col && p.bias ? reinterpret_cast<const float*>(p.bias)[lane] : 0.f;
+  float v = __builtin_fmaf(mine, p.alpha, b);
+  v = apply_act(v, p.act, p.act_a, p.act_b);
+  if (p.row_softmax != 0) {
+    // (wavefront-uniform)  the row's columns sit in lanes 0 .. Kout-1: maximum, exponentials and
+    // their sum across the wavefront, the arithmetic of the stand-alone Softmax launch
+    const float mx = wave_max(col ? v : -INFINITY);
+    const float e = col ? expf(v - mx) : 0.f;
+    const float sum = wave_sum(e);
+    v = p.row_softmax == 2 ? (v - mx) - logf(sum) : e * (1.0f / sum);
   }
+  if (col) reinterpret_cast<float*>(p.y)[(int64_t)m * p.ycs + lane] = v;
 }
 
 }  // namespace

@@ -1255,6 +1255,7 @@ hipError_t launch_igemm(const IgemmParams& p_in, hipStream_t stream) {
     return launch_igemm_stream_q8(p, stream);
   }
   if (gemm_rowdot_shape(p)) return launch_gemm_rowdot(p, stream);
+  if (p.row_softmax != 0) return hipErrorInvalidValue;   // (no other kernel finishes with a Softmax)
   if (const int big = igemm_big_variant(p)) return launch_igemm_big(p, epi_vec, big, stream);
   if (p.w_frag != nullptr && igemm_c3_geometry(p)) return launch_igemm_c3(p, epi_vec, stream);
 

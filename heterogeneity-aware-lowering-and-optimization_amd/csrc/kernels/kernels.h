@@ -124,6 +124,9 @@ struct IgemmParams {
   float act_a = 0.0f, act_b = 0.0f;  // leaky slope / clamp lo,hi
   bool res_after_act = false;        // float types: y = act(..) + residual instead of act(.. + residual)
   bool stream_out = false;           // 2-byte results leave with non-temporal stores (results far larger than the last-level cache)
+  // Softmax (1) or LogSoftmax (2) over the Kout columns of every result row, behind bias and
+  // activation: only the one-wavefront-per-row kernel computes it (gemm_rowdot_shape).
+  int row_softmax = 0;
   // int8 only -----------------------------------------------------------
   // acc = int32 accumulator + int32 bias; fma = one fused multiply-add in fp32
   // (a single rounding); sat8 = round to nearest even and saturate to [0, 255].

@@ -2021,6 +2021,25 @@ void Planner::lower_gemm(int ni) {
       return;
     }
   }
+  // A Softmax over the columns of a product with very few of them (a classifier head like
+  // mnist_simple's Gemm -> Add -> Softmax): the one-wavefront-per-row kernel has every column of
+  // its row in registers and finishes with it - one launch for the whole head.
+  if (!calib_ && ep.residual == nullptr && ip.batch == 1 && dt == DT_F32 && odt == DT_F32 && ip.y_rdiv == 0 &&
+      ip.y_zdiv == 0 && !outv->is_output && consumers_[outv->index].size() == 1) {
+    Node& sm = comp_->nodes[consumers_[outv->index][0]];
+    IgemmParams probe = ip;
+    probe.act = ep.act;
+    probe.ycs = ip.ycs > 0 ? ip.ycs : (int)Nn;
+    if (sm.op == OP_SOFTMAX && !sm.absorbed && (int)sm.i[0] == sm.in[0]->shape.rank - 1 && sm.in[0] == outv &&
+        result_dtype(sm.out) == DT_F32 && softmax_add_.find(outv->index) == softmax_add_.end() && gemm_rowdot_shape(probe)) {
+      ip.row_softmax = sm.i[1] != 0 ? 2 : 1;
+      sm.absorbed = true;
+      const int ty = new_tensor(DT_F32, L_ROWMAJOR, sm.out->shape, 0, SP_ARENA);
+      finish_igemm("gemm+softmax:" + sm.out->name, ip, ta, tw, ty, ep, Nn);
+      set_main(sm.out, ty);
+      return;
+    }
+  }
   const int ty = new_tensor(odt, L_ROWMAJOR, outv->shape, 0, SP_ARENA);
   finish_igemm("gemm:" + outv->name, ip, ta, tw, ty, ep, Nn);
   set_main(outv, ty);

@@ -465,6 +465,32 @@ def test_gemm_parity(case):
     assert max_rel_err(got["y"], want["y"]) <= F32_TOL
 
 
+@pytest.mark.parametrize("log", [False, True])
+@pytest.mark.parametrize("dims", [(64, 784, 10), (7, 300, 16), (33, 256, 1), (64, 784, 24)])
+def test_gemm_bias_softmax_head(dims, log, monkeypatch):
+    """Gemm + bias + (Log)Softmax over a handful of columns - the softmax-regression head: one
+    launch where the product has at most 16 columns (the row kernel finishes with the Softmax),
+    two otherwise (24 columns) or with ODLA_HIP_ROWDOT=0; all against the oracle."""
+    M, K, N = dims
+    announce("gemm + softmax head %s log=%s" % (dims, log))
+    r = rng(111)
+    A = r.standard_normal((M, K)).astype(np.float32)
+    B = (r.standard_normal((K, N)) * 0.2).astype(np.float32)
+    C = r.standard_normal((N,)).astype(np.float32)
+
+    def build(b):
+        y = b.gemm(b.arg("A", A.shape), b.const("B", B), b.const("C", C), name="logits")
+        b.output(b.softmax(y, -1, log, name="prob"), "prob")
+
+    got, want = run_both(build, {"A": A})
+    assert max_rel_err(got["prob"], want["prob"]) <= F32_TOL
+    monkeypatch.setenv("ODLA_HIP_ROWDOT", "0")
+    apart = run_hip(build, {"A": A})
+    assert max_rel_err(apart["prob"], want["prob"]) <= F32_TOL
+    if not log:
+        assert np.allclose(got["prob"].sum(-1), 1.0, atol=1e-5)
+
+
 def test_batched_gemm_parity():
     announce("batched gemm")
     r = rng(12)
