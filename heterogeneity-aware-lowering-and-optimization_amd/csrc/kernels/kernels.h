@@ -412,9 +412,12 @@ hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int
                           int64_t len, int64_t inner, bool log_softmax, hipStream_t stream,
                           const void* add = nullptr, int64_t add_div = 1);
 // y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last `len` elements.
+// y2 (optional): a second copy of the result in y2_dt (DT_F16 / DT_BF16), written by the same
+// launch - for fp32 rows that layernorm_dual_ok accepts.
 hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int64_t len,
                             const float* gamma, const float* beta, float eps,
-                            hipStream_t stream);
+                            hipStream_t stream, void* y2 = nullptr, DType y2_dt = DT_F32);
+bool layernorm_dual_ok(DType dt, int64_t len);
 
 // ---------------------------------------------------------------------------
 // Data movement.

@@ -655,7 +655,8 @@ softmax_vec_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t rows, i
 template <typename T, int LPR, int PER>
 __global__ void __launch_bounds__(kThreads)
 layernorm_vec_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, int len,
-                     const float* __restrict__ gamma, const float* __restrict__ beta, float eps) {
+                     const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
+                     void* __restrict__ y2 = nullptr, const int y2_kind = 0) {
   constexpr int V = Vec16<T>::N;
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63;
@@ -712,6 +713,17 @@ layernorm_vec_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t rows, i
 #pragma unroll
           for (int e = 0; e < V; ++e) o[e] = (v[k][e] - mean) * rstd * g[e] + b[e];
           store_row_vec<T, V>(out + vi * V, o);
+          // a second copy of the row in a 2-byte type (y2_kind 1: f16, 2: bf16; fp32 rows only):
+          // the matrix products that read this result take it as their operand, no conversion
+          // launch in between
+          if constexpr (V == 4) {
+            if (y2 != nullptr) {
+              const float o8[8] = {o[0], o[1], o[2], o[3], 0.f, 0.f, 0.f, 0.f};
+              const uintx4 h = y2_kind == 1 ? pack8_rne<f16_t>(o8) : pack8_rne<bf16_t>(o8);
+              typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+              *reinterpret_cast<uintx2*>(reinterpret_cast<unsigned short*>(y2) + r * (int64_t)len + vi * V) = (uintx2){h.x, h.y};
+            }
+          }
         }
       }
     }
@@ -1023,9 +1035,17 @@ hipError_t launch_softmax(const void* x, void* y, DType in_dt, DType out_dt, int
   return hipErrorInvalidValue;
 }
 
+bool layernorm_dual_ok(DType dt, int64_t len) { return dt == DT_F32 && len % 4 == 0 && len / 4 <= 256; }
+
 hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int64_t len,
-                            const float* gamma, const float* beta, float eps, hipStream_t stream) {
+                            const float* gamma, const float* beta, float eps, hipStream_t stream,
+                            void* y2, DType y2_dt) {
   if (!x || !y || rows <= 0 || len <= 0) return hipErrorInvalidValue;
+  const int y2_kind = y2 == nullptr ? 0 : (y2_dt == DT_F16 ? 1 : (y2_dt == DT_BF16 ? 2 : -1));
+  // (the second, 2-byte copy: fp32 rows on the vector path only - layernorm_dual_ok)
+  if (y2_kind < 0 || (y2_kind > 0 && !(layernorm_dual_ok(dt, len) && al16(x) && al16(y) && (reinterpret_cast<uintptr_t>(y2) & 7u) == 0 &&
+                                      (!gamma || al16(gamma)) && (!beta || al16(beta)))))
+    return hipErrorInvalidValue;
   if (len > 256 * 16) {
     const int grid = (int)(rows < 16384 ? rows : 16384);
     FLOAT_DISPATCH(dt, hipLaunchKernelGGL((layernorm_long_kernel<T, 256>), dim3(grid), dim3(256), 0, stream,
@@ -1042,7 +1062,7 @@ hipError_t launch_layernorm(const void* x, void* y, DType dt, int64_t rows, int6
       const int per = (nv + lpr - 1) / lpr;
       const int rpw = 64 / lpr;
       const int grid = grid_for((rows + rpw - 1) / rpw * 64, kThreads);
-#define LNV(LPR_, PER_) FLOAT_DISPATCH(dt, hipLaunchKernelGGL((layernorm_vec_kernel<T, LPR_, PER_>), dim3(grid), dim3(kThreads), 0, stream, (const T*)x, (T*)y, rows, (int)len, gamma, beta, eps))
+#define LNV(LPR_, PER_) FLOAT_DISPATCH(dt, hipLaunchKernelGGL((layernorm_vec_kernel<T, LPR_, PER_>), dim3(grid), dim3(kThreads), 0, stream, (const T*)x, (T*)y, rows, (int)len, gamma, beta, eps, y2, y2_kind))
       if (lpr <= 16) { LNV(16, 1); }
       else if (lpr == 32) { LNV(32, 1); }
       else if (per == 1) { LNV(64, 1); }

@@ -2838,11 +2838,26 @@ void Planner::lower_layernorm(int ni) {
   const Ref a = ref(tx), b = ref(ty), rg = ref(tg >= 0 ? tg : tx), rb = ref(tb >= 0 ? tb : tx);
   const bool hg = tg >= 0, hb = tb >= 0;
   const float eps = n.f[0];
-  emit("layernorm:" + n.out->name, {tx}, {ty}, [=](const ExecEnv& e, hipStream_t st) {
+  // Accuracy mode (fp32 tensors, 2-byte matrix operands): a result that matrix products read as
+  // their operand leaves this launch in both forms - the separate conversion launch per
+  // LayerNorm (25 per BERT-base step) is gone.
+  int t2 = -1;
+  if (acc_mode_ && dt == DT_F32 && dtype_from_odla(n.out->etype) == DT_F32 && layernorm_dual_ok(dt, len)) {
+    for (int ci : consumers_[n.out->index]) {
+      const Node& c = comp_->nodes[ci];
+      if ((c.op == OP_GEMM || c.op == OP_CONV) && (c.in[0] == n.out || c.in[1] == n.out)) t2 = -2;
+    }
+    if (t2 == -2) t2 = new_tensor(op_dt_, L_ROWMAJOR, n.out->shape, 0, SP_ARENA);
+  }
+  const Ref b2 = ref(t2 >= 0 ? t2 : ty);
+  const bool dual = t2 >= 0;
+  const DType dt2 = op_dt_;
+  emit("layernorm:" + n.out->name, {tx}, {ty, t2}, [=](const ExecEnv& e, hipStream_t st) {
     return launch_layernorm(a(e), b(e), dt, rows, len, hg ? (const float*)rg(e) : nullptr,
-                            hb ? (const float*)rb(e) : nullptr, eps, st);
+                            hb ? (const float*)rb(e) : nullptr, eps, st, dual ? b2(e) : nullptr, dt2);
   });
   set_main(n.out, ty);
+  if (dual) vs_[n.out->index].slot[L_ROWMAJOR][FORM_OPERAND] = t2;
 }
 
 // ---------------------------------------------------------------- Pool ----
